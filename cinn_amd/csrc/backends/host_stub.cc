@@ -1,0 +1,209 @@
+#include "backends/host_stub.h"
+
+#include <array>
+#include <mutex>
+#include <utility>
+
+namespace cinn {
+namespace backends {
+
+// ---------------------------------------------------------------------------------------------------
+// extern API registry
+// ---------------------------------------------------------------------------------------------------
+namespace {
+
+int I(const BakedArg& a) { return static_cast<int>(a.i); }
+float F(const BakedArg& a) { return static_cast<float>(a.f); }
+bool B(const BakedArg& a) { return a.i != 0; }
+
+// Argument lists below follow the call the lowering builds: (kernel_args, kernel_args_num, <constants...>,
+// kernel_stream).  Index 0/1 and the last entry are the pass-through arguments.
+void InvokeHipKernel(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
+  cinn_call_hip_kernel(a[0].p, args, n, I(a[3]), I(a[4]), I(a[5]), I(a[6]), I(a[7]), I(a[8]), stream);
+}
+void InvokeCublas(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
+  cinn_call_cublas(args, n, B(a[2]), B(a[3]), B(a[4]), F(a[5]), F(a[6]), I(a[7]), I(a[8]), I(a[9]), I(a[10]), I(a[11]),
+                   I(a[12]), I(a[13]), I(a[14]), stream);
+}
+void InvokeConv2dForward(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
+  cinn_call_cudnn_conv2d_forward(args, n, I(a[2]), F(a[3]), F(a[4]), I(a[5]), I(a[6]), I(a[7]), I(a[8]), I(a[9]),
+                                 I(a[10]), I(a[11]), I(a[12]), I(a[13]), I(a[14]), I(a[15]), I(a[16]), I(a[17]),
+                                 I(a[18]), I(a[19]), I(a[20]), I(a[21]), I(a[22]), I(a[23]), stream);
+}
+void InvokeConv2dBnRelu(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
+  cinn_call_hip_conv2d_bn_relu(args, n, I(a[2]), I(a[3]), I(a[4]), I(a[5]), I(a[6]), I(a[7]), I(a[8]), I(a[9]),
+                               I(a[10]), I(a[11]), I(a[12]), I(a[13]), I(a[14]), I(a[15]), I(a[16]), I(a[17]),
+                               I(a[18]), I(a[19]), I(a[20]), I(a[21]), I(a[22]), stream);
+}
+void InvokePool2dForward(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
+  cinn_call_cudnn_pool2d_forward(args, n, I(a[2]), I(a[3]), F(a[4]), F(a[5]), I(a[6]), I(a[7]), I(a[8]), I(a[9]),
+                                 I(a[10]), I(a[11]), I(a[12]), I(a[13]), I(a[14]), I(a[15]), I(a[16]), I(a[17]),
+                                 I(a[18]), I(a[19]), stream);
+}
+void InvokeSoftmaxForward(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
+  cinn_call_cudnn_softmax_forward(args, n, I(a[2]), I(a[3]), F(a[4]), F(a[5]), I(a[6]), I(a[7]), I(a[8]), I(a[9]),
+                                  I(a[10]), I(a[11]), I(a[12]), I(a[13]), stream);
+}
+void InvokeMemset(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
+  cinn_call_cuda_memset(args, n, I(a[2]), static_cast<size_t>(a[3].i), stream);
+}
+void InvokeMemcpy(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
+  cinn_call_cuda_memcpy(args, n, static_cast<size_t>(a[2].i), stream);
+}
+
+}  // namespace
+
+ExternApiRegistry::ExternApiRegistry() {
+  // kernel launch: (kernel_fn, kernel_args, kernel_args_num, gx, gy, gz, bx, by, bz, kernel_stream)
+  Register("cinn_call_hip_kernel", InvokeHipKernel, 10);
+  Register("cinn_call_cuda_kernel", InvokeHipKernel, 10);
+  Register("cinn_call_cublas", InvokeCublas, 16);
+  Register("cinn_call_cudnn_conv2d_forward", InvokeConv2dForward, 25);
+  Register("cinn_call_hip_conv2d_bn_relu", InvokeConv2dBnRelu, 24);
+  Register("cinn_call_cudnn_pool2d_forward", InvokePool2dForward, 21);
+  Register("cinn_call_cudnn_softmax_forward", InvokeSoftmaxForward, 15);
+  Register("cinn_call_cuda_memset", InvokeMemset, 5);
+  Register("cinn_call_cuda_memcpy", InvokeMemcpy, 4);
+}
+
+ExternApiRegistry& ExternApiRegistry::Global() {
+  static ExternApiRegistry r;
+  return r;
+}
+void ExternApiRegistry::Register(const std::string& name, ApiInvoker invoker, size_t num_call_args) {
+  table_[name] = Entry{invoker, num_call_args};
+}
+ApiInvoker ExternApiRegistry::Find(const std::string& name, size_t* num_call_args) const {
+  auto it = table_.find(name);
+  if (it == table_.end()) return nullptr;
+  if (num_call_args) *num_call_args = it->second.num_call_args;
+  return it->second.invoker;
+}
+std::vector<std::string> ExternApiRegistry::Names() const {
+  std::vector<std::string> out;
+  for (auto& kv : table_) out.push_back(kv.first);
+  return out;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// trampoline pool
+// ---------------------------------------------------------------------------------------------------
+namespace {
+struct PoolState {
+  std::mutex mu;
+  std::array<HostStubPool::Closure, HostStubPool::kSlots> closures;
+  std::array<bool, HostStubPool::kSlots> used{};
+  int in_use{0};
+  int next_hint{0};
+};
+PoolState& State() {
+  static PoolState* s = new PoolState;  // intentionally leaked: stubs may run during static teardown
+  return *s;
+}
+
+template <int Slot>
+void Trampoline(void* args, int32_t num_args, void* stream) {
+  State().closures[Slot](args, num_args, stream);
+}
+template <int... Slots>
+constexpr std::array<lower_func_ptr_g, sizeof...(Slots)> MakeTable(std::integer_sequence<int, Slots...>) {
+  return {{&Trampoline<Slots>...}};
+}
+const std::array<lower_func_ptr_g, HostStubPool::kSlots>& Table() {
+  static const auto table = MakeTable(std::make_integer_sequence<int, HostStubPool::kSlots>{});
+  return table;
+}
+}  // namespace
+
+HostStubPool& HostStubPool::Global() {
+  static HostStubPool pool;
+  return pool;
+}
+
+lower_func_ptr_g HostStubPool::Acquire(Closure closure) {
+  auto& s = State();
+  std::lock_guard<std::mutex> lock(s.mu);
+  CINN_CHECK_LT(s.in_use, kSlots) << "all " << kSlots << " host stub slots are in use; release compiled programs";
+  for (int probe = 0; probe < kSlots; ++probe) {
+    int slot = (s.next_hint + probe) % kSlots;
+    if (!s.used[slot]) {
+      s.used[slot]     = true;
+      s.closures[slot] = std::move(closure);
+      s.next_hint      = slot + 1;
+      ++s.in_use;
+      return Table()[slot];
+    }
+  }
+  CINN_CHECK(false) << "host stub pool is inconsistent";
+  return nullptr;
+}
+
+void HostStubPool::Release(lower_func_ptr_g fn) {
+  auto& s = State();
+  std::lock_guard<std::mutex> lock(s.mu);
+  const auto& table = Table();
+  for (int slot = 0; slot < kSlots; ++slot) {
+    if (table[slot] == fn) {
+      if (s.used[slot]) {
+        s.used[slot]     = false;
+        s.closures[slot] = nullptr;
+        --s.in_use;
+      }
+      return;
+    }
+  }
+}
+
+int HostStubPool::in_use() const {
+  auto& s = State();
+  std::lock_guard<std::mutex> lock(s.mu);
+  return s.in_use;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// host function -> closure
+// ---------------------------------------------------------------------------------------------------
+HostStubPool::Closure LowerHostFunction(const ir::LoweredFunc& func, const std::map<std::string, void*>& kernel_symbols) {
+  CINN_CHECK(!func.is_device) << func.name << " is a device function";
+  auto* call = func.body.As<ir::Call>();
+  CINN_CHECK(call) << "the body of host function " << func.name << " must be one intrinsic call";
+  size_t expected = 0;
+  ApiInvoker invoker = ExternApiRegistry::Global().Find(call->name, &expected);
+  CINN_CHECK(invoker) << "host function " << func.name << " calls unknown runtime intrinsic " << call->name;
+  CINN_CHECK_EQ(call->args.size(), expected) << "wrong number of arguments in the call of " << call->name;
+
+  std::vector<BakedArg> baked;
+  for (auto& a : call->args) {
+    BakedArg b;
+    if (auto* v = a.As<ir::Var>()) {
+      if (v->name == "kernel_args") {
+        b.kind = BakedArg::Kind::kArgs;
+      } else if (v->name == "kernel_args_num") {
+        b.kind = BakedArg::Kind::kNumArgs;
+      } else if (v->name == "kernel_stream") {
+        b.kind = BakedArg::Kind::kStream;
+      } else {
+        auto it = kernel_symbols.find(v->name);
+        CINN_CHECK(it != kernel_symbols.end()) << "unresolved symbol " << v->name << " in host function " << func.name;
+        b.kind = BakedArg::Kind::kHandle;
+        b.p    = it->second;
+      }
+    } else if (auto* i = a.As<ir::IntImm>()) {
+      b.kind = BakedArg::Kind::kInt;
+      b.i    = i->value;
+    } else if (auto* u = a.As<ir::UIntImm>()) {
+      b.kind = u->type.is_bool() ? BakedArg::Kind::kBool : BakedArg::Kind::kInt;
+      b.i    = static_cast<int64_t>(u->value);
+    } else if (auto* f = a.As<ir::FloatImm>()) {
+      b.kind = BakedArg::Kind::kFloat;
+      b.f    = f->value;
+    } else {
+      CINN_CHECK(false) << "argument of " << call->name << " in " << func.name << " is not a constant: " << ir::ToString(a);
+    }
+    baked.push_back(b);
+  }
+  return [invoker, baked](void* args, int32_t num_args, void* stream) { invoker(baked, args, num_args, stream); };
+}
+
+}  // namespace backends
+}  // namespace cinn

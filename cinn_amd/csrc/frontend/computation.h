@@ -1,0 +1,71 @@
+// CinnComputation: build, compile and run a program on the GPU.  Interface of
+// cinn/frontend/computation.h:27-159 (BuildAndCompile / Compile / Execute / GetTensor /
+// SetTensorData / GetTensorData); the compile pipeline is the one of CompileProgram
+// (cinn/frontend/computation.cc:43-95) with the gfx950 GraphCompiler underneath.
+#pragma once
+#include <memory>
+#include <set>
+#include <string>
+#include <vector>
+
+#include "frontend/net_builder.h"
+#include "hlir/graph_compiler.h"
+
+namespace cinn {
+namespace frontend {
+
+class CinnComputation {
+ public:
+  struct CompileOptions : public hlir::framework::GraphCompiler::CompileOptions {
+    // composite ops (softmax, batch_norm) are always decomposed on this backend: its kernels are
+    // generated from primitives only
+    bool use_decomposer{true};
+    bool do_prerun{true};
+    // fold `conv2d -> batch_norm [-> relu]` into one convolution call with a fused epilogue
+    bool fuse_conv_bn_relu{false};
+  };
+  static CompileOptions DefaultCompileOptions() { return CompileOptions(); }
+
+  static std::shared_ptr<CinnComputation> BuildAndCompile(const common::Target& target, NetBuilder& builder,
+                                                          const CompileOptions& options        = DefaultCompileOptions(),
+                                                          const std::vector<Variable>& outputs = {},
+                                                          void* stream                         = nullptr);
+  static std::shared_ptr<CinnComputation> Compile(const common::Target& target, Program& program,
+                                                  const CompileOptions& options        = DefaultCompileOptions(),
+                                                  const std::vector<Variable>& outputs = {}, void* stream = nullptr);
+
+  std::vector<std::string> GetAllTensorNames();
+  hlir::framework::Tensor GetTensor(const std::string& name);
+  std::vector<hlir::framework::Tensor> GetInputTensors();
+  std::vector<hlir::framework::Tensor> GetOutputTensors();
+  void SetTensorData(hlir::framework::Tensor& t, void* data, size_t size);
+  void SetTensorData(const std::string& tname, void* data, size_t size);
+  void GetTensorData(hlir::framework::Tensor& t, void* data, size_t size);
+  void GetTensorData(const std::string& tname, void* data, size_t size);
+
+  // run the compiled program once (synchronises when the computation has no stream)
+  void Execute();
+  // replay through a captured HIP graph; needs a stream
+  void ExecuteGraph();
+
+  const std::string& source_code() const { return source_code_; }
+  std::string group_debug_string() const { return graph_->DebugGroupString(); }
+  size_t num_instructions() const { return program_->size(); }
+  const std::vector<std::string>& output_names() const { return output_names_; }
+  const std::vector<std::string>& input_names() const { return input_names_; }
+  void* stream() const { return stream_; }
+  hlir::framework::Program* program() const { return program_.get(); }
+
+ private:
+  common::Target target_;
+  void* stream_{nullptr};
+  std::shared_ptr<hlir::framework::Graph> graph_;
+  std::shared_ptr<hlir::framework::Scope> scope_;
+  std::unique_ptr<hlir::framework::Program> program_;
+  std::unique_ptr<backends::Compiler> compiler_;
+  std::vector<std::string> input_names_, output_names_;
+  std::string source_code_;
+};
+
+}  // namespace frontend
+}  // namespace cinn

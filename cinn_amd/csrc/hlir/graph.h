@@ -1,0 +1,104 @@
+// Dataflow graph of a front-end Program plus its partition into fusion groups.  Mirrors the role of
+// hlir::framework::Graph / Node / NodeData / Graph::Group (cinn/hlir/framework/graph.h) for the
+// GPU path: one Group becomes one kernel (or one library call).
+#pragma once
+#include <map>
+#include <memory>
+#include <set>
+#include <string>
+#include <vector>
+
+#include "common/target.h"
+#include "frontend/syntax.h"
+#include "hlir/op.h"
+
+namespace cinn {
+namespace hlir {
+namespace framework {
+
+struct Node;
+
+// a tensor value of the graph
+struct NodeData {
+  std::string id;
+  ShapeType shape;
+  common::Type dtype;
+  Node* producer{nullptr};  // nullptr: fed input
+  std::vector<Node*> consumers;
+  bool is_fetch{false};
+  int64_t numel() const { return ShapeNumel(shape); }
+};
+
+struct Node {
+  int index{0};  // position in topological order
+  const Operator* op{nullptr};
+  AttributeMap attrs;
+  std::vector<NodeData*> inputs;
+  std::vector<NodeData*> outputs;
+  int group_id{-1};
+  const std::string& op_type() const { return op->name; }
+};
+
+enum class GroupKind {
+  kElementwise,  // injective chain over one flat iteration space
+  kRowReduce,    // reductions over the trailing (contiguous) axes with fused producers and consumers
+  kGeneralReduce,  // a single reduction over arbitrary axes, serial per output element
+  kLibraryCall   // matmul / conv2d / pool2d and other kNonFusible ops
+};
+
+struct Group {
+  int id{0};
+  GroupKind kind{GroupKind::kElementwise};
+  std::vector<Node*> nodes;           // topological order
+  std::vector<NodeData*> inputs;      // values produced outside the group
+  std::vector<NodeData*> outputs;     // values consumed outside the group or fetched
+  // kRowReduce: rows x cols of the reduction space
+  int64_t rows{0}, cols{0};
+  std::string func_name;
+};
+
+class Graph {
+ public:
+  Graph(const frontend::Program& program, const std::set<std::string>& fetch_ids, const common::Target& target);
+
+  const common::Target& target() const { return target_; }
+  const std::vector<std::unique_ptr<Node>>& nodes() const { return nodes_; }
+  NodeData* FindVar(const std::string& id) const;
+  const std::vector<NodeData*>& inputs() const { return inputs_; }
+  std::vector<NodeData*> AllVars() const;
+
+  // partition into fusion groups (hlir/fusion.cc); fills `groups`
+  void BuildFusionGroups();
+  std::vector<std::unique_ptr<Group>> groups;
+
+  std::string DebugGroupString() const;
+
+ private:
+  NodeData* GetOrCreateVar(const frontend::Variable& v);
+  common::Target target_;
+  std::vector<std::unique_ptr<Node>> nodes_;
+  std::map<std::string, std::unique_ptr<NodeData>> vars_;
+  std::vector<NodeData*> inputs_;
+};
+
+// ---- shape classification shared by the fusion pass and the reduce lowering ------------------------
+// Splits a reduce over `dims` of `shape` into rows x cols when the reduced axes are the trailing
+// ones (size-1 axes are ignored).  Returns false for any other axis set.
+bool TrailingReduceSpace(const ShapeType& shape, const std::vector<int>& dims, int64_t* rows, int64_t* cols);
+std::vector<int> ReduceDimsOf(const Node& node);
+
+// how a value relates to the rows x cols space of a row-reduce group
+enum class RowKind { kElem, kRow, kCol, kScalar, kInvalid };
+// kind of broadcast_to's input given that its output is a kElem value of shape out_shape
+RowKind ClassifyBroadcastInput(const ShapeType& in_shape, const ShapeType& out_shape, const std::vector<int>& axes,
+                               int64_t rows, int64_t cols);
+
+// Assigns a RowKind to every value the nodes (in topological order) touch, for a rows x cols
+// row-reduce group.  Returns false when some node does not fit the pattern (then the nodes cannot
+// share one row-resident kernel).
+bool ClassifyRowReduceGroup(const std::vector<Node*>& nodes, int64_t rows, int64_t cols,
+                            std::map<const NodeData*, RowKind>* kinds);
+
+}  // namespace framework
+}  // namespace hlir
+}  // namespace cinn

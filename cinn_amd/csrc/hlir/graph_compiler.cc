@@ -1,0 +1,203 @@
+#include "hlir/graph_compiler.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstring>
+
+#include "optim/optimize.h"
+
+namespace cinn {
+namespace hlir {
+namespace framework {
+
+#define CINN_HIP_STATUS(expr)                                                                       \
+  do {                                                                                              \
+    int cinn_status__ = (expr);                                                                     \
+    CINN_CHECK_EQ(cinn_status__, 0) << #expr << " failed: " << cinn_hip_error_string(cinn_status__); \
+  } while (0)
+
+// ---- Tensor ---------------------------------------------------------------------------------------
+_Tensor_::_Tensor_() { cinn_hip_buffer_init(&buffer_, nullptr, cinn_type_float, 32, nullptr, 0); }
+_Tensor_::~_Tensor_() { Free(); }
+
+void _Tensor_::Free() {
+  if (buffer_.memory) {
+    cinn_hip_free(buffer_.memory);
+    buffer_.memory = nullptr;
+    allocated_     = 0;
+  }
+}
+
+void _Tensor_::Resize(const ShapeType& shape) {
+  CINN_CHECK_LE(shape.size(), static_cast<size_t>(CINN_BUFFER_MAX_DIMS)) << "tensors have at most 8 dimensions";
+  shape_ = shape;
+}
+
+void _Tensor_::set_type(const common::Type& t) { type_ = t; }
+
+void* _Tensor_::mutable_data(const common::Target& target) {
+  CINN_CHECK(target.arch == common::Target::Arch::AMDGPU) << "device tensors need the AMDGPU target";
+  size_t need = bytes();
+  if (!buffer_.memory || allocated_ < need) {
+    Free();
+    void* p = nullptr;
+    CINN_HIP_STATUS(cinn_hip_malloc(&p, need));
+    allocated_ = need;
+    int code   = type_.is_bfloat16() ? cinn_type_bfloat : static_cast<int>(type_.code);
+    cinn_hip_buffer_init(&buffer_, p, code, type_.is_bool() ? 1 : type_.bits, shape_.data(), static_cast<int>(shape_.size()));
+    buffer_.memory_size = need;
+  }
+  return buffer_.memory;
+}
+
+void _Tensor_::CopyFromHost(const void* src, size_t n, const common::Target& target) {
+  CINN_CHECK_EQ(n, bytes()) << "host data size does not match the tensor";
+  void* dst = mutable_data(target);
+  CINN_HIP_STATUS(cinn_hip_memcpy_h2d(dst, src, n, nullptr));
+}
+void _Tensor_::CopyToHost(void* dst, size_t n) const {
+  CINN_CHECK_EQ(n, bytes()) << "host buffer size does not match the tensor";
+  CINN_CHECK(buffer_.memory) << "tensor has no device memory yet";
+  CINN_HIP_STATUS(cinn_hip_memcpy_d2h(dst, buffer_.memory, n, nullptr));
+}
+
+// ---- Scope ----------------------------------------------------------------------------------------
+Tensor Scope::Var(const std::string& name) {
+  auto it = data_.find(name);
+  if (it != data_.end()) return it->second;
+  auto t      = std::make_shared<_Tensor_>();
+  data_[name] = t;
+  return t;
+}
+Tensor Scope::FindVar(const std::string& name) const {
+  auto it = data_.find(name);
+  return it == data_.end() ? nullptr : it->second;
+}
+Tensor Scope::GetTensor(const std::string& name) const {
+  auto t = FindVar(name);
+  CINN_CHECK(t) << "no variable called '" << name << "' in the scope";
+  return t;
+}
+std::vector<std::string> Scope::var_names() const {
+  std::vector<std::string> names;
+  for (auto& kv : data_) names.push_back(kv.first);
+  return names;
+}
+
+// ---- Instruction ----------------------------------------------------------------------------------
+void Instruction::UpdateArgsCache() {
+  args_cache_.clear();
+  auto add = [&](const std::string& name) {
+    auto t = scope_->GetTensor(name);
+    t->mutable_data(target_);
+    cinn_pod_value_t v;
+    cinn_hip_pod_from_buffer(&v, t->buffer());
+    args_cache_.push_back(v);
+  };
+  for (auto& a : in_args_) add(a);
+  for (auto& a : out_args_) add(a);
+}
+
+void Instruction::Run(void* stream) {
+  CINN_CHECK(fn_) << "instruction " << function_name_ << " has no compiled function";
+  if (args_cache_.empty()) UpdateArgsCache();
+  fn_(args_cache_.data(), static_cast<int32_t>(args_cache_.size()), stream);
+}
+
+// ---- Program --------------------------------------------------------------------------------------
+Program::~Program() {
+  if (graph_exec_) (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec_));
+  if (graph_) (void)hipGraphDestroy(static_cast<hipGraph_t>(graph_));
+}
+
+void Program::PreRun(const common::Target& target) {
+  for (auto& ins : instrs_) {
+    for (auto& a : ins->in_args()) scope_->GetTensor(a)->mutable_data(target);
+    for (auto& a : ins->out_args()) scope_->GetTensor(a)->mutable_data(target);
+  }
+}
+
+void Program::Execute(void* stream) {
+  for (auto& ins : instrs_) ins->Run(stream);
+  if (!stream) CINN_HIP_STATUS(cinn_hip_device_synchronize());
+}
+
+void Program::ExecuteGraph(void* stream) {
+  CINN_CHECK(stream) << "graph replay needs an explicit stream";
+  auto s = static_cast<hipStream_t>(stream);
+  if (!graph_exec_) {
+    hipGraph_t graph = nullptr;
+    CINN_HIP_STATUS(static_cast<int>(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal)));
+    for (auto& ins : instrs_) ins->Run(stream);
+    CINN_HIP_STATUS(static_cast<int>(hipStreamEndCapture(s, &graph)));
+    hipGraphExec_t exec = nullptr;
+    CINN_HIP_STATUS(static_cast<int>(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0)));
+    graph_      = graph;
+    graph_exec_ = exec;
+  }
+  CINN_HIP_STATUS(static_cast<int>(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec_), s)));
+}
+
+// ---- GraphCompiler --------------------------------------------------------------------------------
+std::shared_ptr<Scope> BuildScope(const common::Target& target, const std::shared_ptr<Graph>& graph,
+                                  std::shared_ptr<Scope> scope) {
+  if (!scope) scope = Scope::Create();
+  for (auto* v : graph->AllVars()) {
+    auto t = scope->Var(v->id);
+    t->Resize(v->shape);
+    t->set_type(v->dtype);
+  }
+  (void)target;
+  return scope;
+}
+
+ir::Module GraphCompiler::LowerGraph(const CompileOptions& options) {
+  if (graph_->groups.empty()) graph_->BuildFusionGroups();
+  OpLowerer lowerer(target_, options.lowering);
+  ir::Module module;
+  module.name   = "cinn_hip_module";
+  module.target = target_;
+  for (auto& g : graph_->groups) {
+    auto func = lowerer.Lower(*g);
+    if (func->is_device) optim::OptimizeFuncGPU(func.get());
+    module.functions.push_back(func);
+  }
+  return module;
+}
+
+std::string GraphCompiler::GenSourceCode(const CompileOptions& options) {
+  auto module  = LowerGraph(options);
+  auto comp    = backends::Compiler::Create(target_);
+  source_code_ = comp->GetSourceCode(module);
+  return source_code_;
+}
+
+std::unique_ptr<Program> GraphCompiler::Build(const CompileOptions& options) {
+  auto module = LowerGraph(options);
+  compiler_   = backends::Compiler::Create(target_);
+  compiler_->Build(module);
+  source_code_ = compiler_->source_code();
+
+  std::vector<std::unique_ptr<Instruction>> instrs;
+  for (auto& g : graph_->groups) {
+    std::vector<std::string> ins, outs;
+    for (auto* v : g->inputs) ins.push_back(v->id);
+    for (auto* v : g->outputs) outs.push_back(v->id);
+    auto instr = std::make_unique<Instruction>(target_, scope_.get(), ins, outs, g->func_name);
+    void* fn   = compiler_->Lookup(g->func_name);
+    CINN_CHECK(fn) << "compiled function " << g->func_name << " not found";
+    instr->SetLoweredFunc(fn);
+    instrs.push_back(std::move(instr));
+  }
+  auto program = std::make_unique<Program>(scope_, std::move(instrs));
+  if (options.with_instantiate_variables) {
+    int device_count = 0;
+    cinn_hip_device_count(&device_count);
+    if (device_count > 0) program->PreRun(target_);
+  }
+  return program;
+}
+
+}  // namespace framework
+}  // namespace hlir
+}  // namespace cinn

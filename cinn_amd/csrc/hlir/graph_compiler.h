@@ -1,0 +1,152 @@
+// Scope / Tensor / Instruction / Program / GraphCompiler of the GPU path.  Interfaces follow
+// cinn/hlir/framework/{scope.h,tensor.h,buffer.h,memory.cc,instruction.h,graph_compiler.h}:
+//   * a Tensor owns a cinn_buffer_t whose `memory` is device memory obtained through the runtime's
+//     allocator (role of CudaMemoryMng, memory.cc:43-64);
+//   * an Instruction holds the names of its arguments and a lower_func_ptr_g; Run() packs the
+//     cinn_pod_value_t argument array once and calls the function (instruction.cc:77-138);
+//   * Program::Execute runs the instructions in order on one stream and synchronises when no
+//     stream was given (graph_compiler.cc:212-222);
+//   * GraphCompiler::Build lowers every fusion group, builds one module and creates the
+//     instructions (graph_compiler.cc:745-792).
+#pragma once
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "backends/compiler.h"
+#include "cinn_hip_runtime.h"
+#include "hlir/graph.h"
+#include "hlir/lowering.h"
+
+namespace cinn {
+namespace hlir {
+namespace framework {
+
+class _Tensor_ {
+ public:
+  _Tensor_();
+  ~_Tensor_();
+  _Tensor_(const _Tensor_&) = delete;
+
+  void Resize(const ShapeType& shape);
+  const ShapeType& shape() const { return shape_; }
+  const common::Type& type() const { return type_; }
+  void set_type(const common::Type& t);
+  int64_t numel() const { return ShapeNumel(shape_); }
+  size_t bytes() const { return static_cast<size_t>(numel()) * type_.bytes(); }
+
+  // device pointer; allocates on first use
+  void* mutable_data(const common::Target& target);
+  void* data() const { return buffer_.memory; }
+  cinn_buffer_t* buffer() { return &buffer_; }
+
+  // synchronous copies between host memory and the device buffer
+  void CopyFromHost(const void* src, size_t bytes, const common::Target& target);
+  void CopyToHost(void* dst, size_t bytes) const;
+
+ private:
+  void Free();
+  ShapeType shape_;
+  common::Type type_{common::Float(32)};
+  cinn_buffer_t buffer_;
+  size_t allocated_{0};
+};
+using Tensor = std::shared_ptr<_Tensor_>;
+
+class Scope {
+ public:
+  static std::shared_ptr<Scope> Create() { return std::make_shared<Scope>(); }
+  // creates the tensor when it does not exist
+  Tensor Var(const std::string& name);
+  Tensor FindVar(const std::string& name) const;
+  Tensor GetTensor(const std::string& name) const;
+  std::vector<std::string> var_names() const;
+
+ private:
+  std::map<std::string, Tensor> data_;
+};
+
+class Instruction {
+ public:
+  Instruction(const common::Target& target, Scope* scope, std::vector<std::string> in_args,
+              std::vector<std::string> out_args, std::string function_name)
+      : target_(target), scope_(scope), in_args_(std::move(in_args)), out_args_(std::move(out_args)),
+        function_name_(std::move(function_name)) {}
+
+  void SetLoweredFunc(void* fn) { fn_ = reinterpret_cast<lower_func_ptr_g>(fn); }
+  void Run(void* stream = nullptr);
+  const std::string& function_name() const { return function_name_; }
+  const std::vector<std::string>& in_args() const { return in_args_; }
+  const std::vector<std::string>& out_args() const { return out_args_; }
+
+ private:
+  void UpdateArgsCache();
+  common::Target target_;
+  Scope* scope_;
+  std::vector<std::string> in_args_, out_args_;
+  std::string function_name_;
+  lower_func_ptr_g fn_{nullptr};
+  std::vector<cinn_pod_value_t> args_cache_;
+};
+
+class Program {
+ public:
+  Program(std::shared_ptr<Scope> scope, std::vector<std::unique_ptr<Instruction>> instrs)
+      : scope_(std::move(scope)), instrs_(std::move(instrs)) {}
+  ~Program();
+  // allocate every tensor the instructions touch
+  void PreRun(const common::Target& target);
+  // Runs all instructions on `stream`; with stream == nullptr the null stream is used and the device
+  // is synchronised afterwards.
+  void Execute(void* stream = nullptr);
+  // Same work replayed from a HIP graph captured on first use (removes the per-kernel launch cost
+  // of programs with many small kernels).  Falls back to Execute when capture is not possible.
+  void ExecuteGraph(void* stream);
+  size_t size() const { return instrs_.size(); }
+  const std::vector<std::unique_ptr<Instruction>>& GetRunInstructions() const { return instrs_; }
+  std::shared_ptr<Scope> scope() const { return scope_; }
+
+ private:
+  std::shared_ptr<Scope> scope_;
+  std::vector<std::unique_ptr<Instruction>> instrs_;
+  void* graph_exec_{nullptr};
+  void* graph_{nullptr};
+};
+
+struct GraphCompileOptions {
+  bool with_instantiate_variables{true};
+  LoweringOptions lowering{LoweringOptions::FromEnv()};
+};
+
+class GraphCompiler final {
+ public:
+  using CompileOptions = GraphCompileOptions;
+  GraphCompiler(const common::Target& target, std::shared_ptr<Scope> scope, std::shared_ptr<Graph> graph)
+      : target_(target), scope_(std::move(scope)), graph_(std::move(graph)) {}
+
+  std::unique_ptr<Program> Build(const CompileOptions& options = CompileOptions());
+  // device source of the whole graph without loading anything
+  std::string GenSourceCode(const CompileOptions& options = CompileOptions());
+  const std::string& source_code() const { return source_code_; }
+
+ private:
+  ir::Module LowerGraph(const CompileOptions& options);
+  common::Target target_;
+  std::shared_ptr<Scope> scope_;
+  std::shared_ptr<Graph> graph_;
+  std::unique_ptr<backends::Compiler> compiler_;
+  std::string source_code_;
+
+ public:
+  // the Compiler owns the loaded code objects and host stubs; a Program must not outlive it
+  std::unique_ptr<backends::Compiler> ReleaseCompiler() { return std::move(compiler_); }
+};
+
+// creates scope tensors (shape + dtype) for every variable of the graph
+std::shared_ptr<Scope> BuildScope(const common::Target& target, const std::shared_ptr<Graph>& graph,
+                                  std::shared_ptr<Scope> scope = nullptr);
+
+}  // namespace framework
+}  // namespace hlir
+}  // namespace cinn

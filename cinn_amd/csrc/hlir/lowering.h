@@ -1,0 +1,56 @@
+// Lowering of one fusion group to one LoweredFunc for gfx950.  This is the GPU-schedule side of the
+// backend: it decides the launch shape and the loop structure the reference derives in
+// OpLowerer::IRSchedule (cinn/hlir/framework/op_lowering.cc:516-658) with the schedules of
+// cinn/hlir/pe/ir_schedule_pe.cc and the reduce loop assignment of
+// cinn/hlir/framework/op_lowering_util.cc:485-1177 - re-designed for 64-lane wavefronts:
+//   * element-wise groups: one flat space, 128-bit accesses, 256-thread blocks;
+//   * row-reduce groups (reductions over the trailing axes plus everything fused around them):
+//     one wavefront - or, for long rows, one block - owns a row, keeps it in registers across all
+//     reductions and writes every output once, so the group reads and writes each tensor exactly
+//     once whatever the number of reductions in it;
+//   * other reductions: one thread per output element, serial over the reduced axes;
+//   * kNonFusible ops: a host function holding one call to a runtime intrinsic, as
+//     cinn/hlir/op/custom_call.cc:70-217 builds them.
+#pragma once
+#include <string>
+
+#include "hlir/graph.h"
+#include "ir/ir.h"
+
+namespace cinn {
+namespace hlir {
+namespace framework {
+
+struct LoweringOptions {
+  // longest row (in elements per thread) that is kept in registers by the row-reduce template
+  int max_cached_elems_per_thread{64};
+  // elements per lane above which a row is given to a whole block instead of one wavefront
+  int wave_row_elems_per_lane{64};
+  // threads of an element-wise block
+  int elementwise_block{256};
+  // waves (rows) per block when one wavefront owns a row
+  int rows_per_block{4};
+  static LoweringOptions FromEnv();
+};
+
+class OpLowerer {
+ public:
+  OpLowerer(const common::Target& target, const LoweringOptions& options = LoweringOptions::FromEnv());
+  // One function per group.  Device functions come back scheduled, with loops still carrying their
+  // GPU bindings (optim::OptimizeFuncGPU turns them into a kernel body and launch dimensions).
+  ir::LoweredFuncRef Lower(const Group& group) const;
+  // argument order of the function generated for `group`: inputs, then outputs
+  static std::vector<NodeData*> ArgumentsOf(const Group& group);
+
+ private:
+  ir::LoweredFuncRef LowerElementwise(const Group& group) const;
+  ir::LoweredFuncRef LowerRowReduce(const Group& group) const;
+  ir::LoweredFuncRef LowerGeneralReduce(const Group& group) const;
+  ir::LoweredFuncRef LowerLibraryCall(const Group& group) const;
+  common::Target target_;
+  LoweringOptions options_;
+};
+
+}  // namespace framework
+}  // namespace hlir
+}  // namespace cinn

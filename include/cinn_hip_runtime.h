@@ -1,0 +1,254 @@
+/*
+ * C-ABI of the MI355X (gfx950) runtime for the CINN GPU backend.
+ *
+ * Everything a JIT'd / trampolined host stub of a compiled CINN program calls on the GPU path is
+ * declared here with plain pointers and sizes.  Each entry point names the reference interface it
+ * replaces (paths are relative to the CINN source tree).
+ *
+ * Error convention (same as the reference's CUDA_CALL / CUDA_DRIVER_CALL / CHECK macros,
+ * cinn/backends/cuda_util.h:30-88): the `cinn_call_*` intrinsics return void and abort() the process
+ * with a message on stderr when a HIP call fails or an argument is invalid.  The `cinn_hip_*`
+ * management entry points return 0 on success and a non-zero HIP / hiprtc status otherwise and
+ * never abort, so a binding can turn them into exceptions.
+ *
+ * Threading: entry points may be called from any thread; module loading and the kernel cache are
+ * guarded by a mutex, launches are not serialised (HIP streams order them).
+ */
+#ifndef CINN_HIP_RUNTIME_H_
+#define CINN_HIP_RUNTIME_H_
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------------------------------
+ * ABI structs.  Layout-identical to cinn/runtime/cinn_runtime.h:51-93 (cinn_type_t), :186-292
+ * (cinn_buffer_t, 120 bytes: memory@16, type@32, dimensions@44, dims@48, memory_size@88) and
+ * :390-461 (cinn_value_t / cinn_pod_value_t, 16 bytes) as compiled by a C++11 compiler on x86-64.
+ * ---------------------------------------------------------------------------------------------- */
+
+typedef enum cinn_type_code_t {
+  cinn_type_unk    = -1,
+  cinn_type_int    = 0,
+  cinn_type_uint   = 1,
+  cinn_type_float  = 2,
+  cinn_type_handle = 3,
+  cinn_type_bfloat = 4
+} cinn_type_code_t;
+
+typedef struct cinn_type_t {
+  int32_t code; /* a cinn_type_code_t, stored in 4 bytes */
+  uint8_t bits;
+  uint16_t lanes;
+  uint8_t num_asterisks;
+} cinn_type_t;
+
+typedef int cinn_dimension_t;
+
+typedef enum cinn_device_kind_t {
+  cinn_unk_device    = -1,
+  cinn_x86_device    = 0,
+  cinn_opencl_device = 1,
+  cinn_arm_device    = 2
+} cinn_device_kind_t;
+
+typedef enum cinn_buffer_kind_t { cinn_buffer_on_host = 0, cinn_buffer_on_device = 1 << 1 } cinn_buffer_kind_t;
+
+#define CINN_BUFFER_MAX_DIMS 8
+
+typedef struct cinn_buffer_t {
+  int32_t device; /* a cinn_device_kind_t */
+  const void* device_interface;
+  uint8_t* memory; /* device pointer on the GPU path */
+  uint64_t flag;
+  cinn_type_t type;
+  int32_t dimensions;
+  cinn_dimension_t dims[CINN_BUFFER_MAX_DIMS];
+  char lazy;
+  uint64_t memory_size;
+  uint16_t align;
+  void* external_malloc; /* std::function<int(void*, cinn_buffer_t*)>* in the reference; opaque here */
+  void* external_free;
+} cinn_buffer_t;
+
+typedef union cinn_value_t {
+  int64_t v_int64;
+  double v_float64;
+  void* v_handle;
+  char* v_str;
+} cinn_value_t;
+
+typedef struct cinn_pod_value_t {
+  int type_code_; /* values of cinn_type_code<T>() below */
+  cinn_value_t value_;
+} cinn_pod_value_t;
+
+/* cinn_type_code<T>() table, cinn/runtime/cinn_runtime.h:469-491 */
+enum {
+  CINN_POD_INT32 = 0,
+  CINN_POD_INT64 = 1,
+  CINN_POD_FLOAT = 2,
+  CINN_POD_DOUBLE = 3,
+  CINN_POD_VOID_P = 4,
+  CINN_POD_CHAR_P = 5,
+  CINN_POD_CONST_CHAR_P = 6,
+  CINN_POD_BUFFER_P = 7,
+  CINN_POD_INT8 = 8,
+  CINN_POD_BOOL = 9,
+  CINN_POD_FLOAT16 = 10,
+  CINN_POD_INT16 = 11,
+  CINN_POD_UINT8 = 12,
+  CINN_POD_UINT16 = 13,
+  CINN_POD_UINT32 = 14,
+  CINN_POD_UINT64 = 15,
+  CINN_POD_BFLOAT16 = 16
+};
+
+/* Host-stub type every compiled fused group is exposed as (cinn_runtime.h:498-499). */
+typedef void (*lower_func_ptr_g)(void* pod_args, int32_t num_args, void* stream);
+
+/* Helpers to fill ABI structs from a binding (cinn_runtime.cc buffer_p_to_cinn_pod_value etc.). */
+void cinn_hip_buffer_init(cinn_buffer_t* buf, void* device_ptr, int32_t type_code, int32_t bits, const int32_t* dims,
+                          int32_t ndims);
+void cinn_hip_pod_from_buffer(cinn_pod_value_t* out, cinn_buffer_t* buf);
+void cinn_hip_pod_from_int32(cinn_pod_value_t* out, int32_t v);
+void cinn_hip_pod_from_float(cinn_pod_value_t* out, float v);
+
+/* ------------------------------------------------------------------------------------------------
+ * Runtime intrinsics called by host stubs.
+ * ---------------------------------------------------------------------------------------------- */
+
+/* Launch a kernel of a loaded code object.  Replaces cinn_call_cuda_kernel
+ * (cinn/runtime/cuda/cuda_util.h:75-84, cuda_util.cc:78-119): `kernel_fn` is a hipFunction_t,
+ * `v_args` is cinn_pod_value_t[num_args]; a buffer argument is passed as its device pointer, a
+ * scalar by the address of its value; dynamic LDS is always 0.  `stream` is a hipStream_t
+ * (NULL = the null stream). */
+void cinn_call_hip_kernel(void* kernel_fn, void* v_args, int num_args, int grid_x, int grid_y, int grid_z,
+                          int block_x, int block_y, int block_z, void* stream);
+/* Same function under the name upstream host stubs already reference. */
+void cinn_call_cuda_kernel(void* kernel_fn, void* v_args, int num_args, int grid_x, int grid_y, int grid_z,
+                           int block_x, int block_y, int block_z, void* stream);
+
+/* Row-major C = alpha * op(A) * op(B) + beta * C (optionally C^T when trans_o) on MFMA matrix
+ * cores.  Replaces cinn_call_cublas (cuda_util.h:86-101, cuda_util.cc:121-310).  v_args = {A, B, C}
+ * buffers; a1..a4 / b1..b4 are the operand shapes left-padded to 4-D; leading dims broadcast per
+ * the reference rules.  Element type is taken from A's cinn_type_t (fp32, fp16, bf16, fp64);
+ * 16-bit inputs accumulate in fp32. */
+void cinn_call_cublas(void* v_args, int num_args, bool trans_a, bool trans_b, bool trans_o, float alpha, float beta,
+                      int a1, int a2, int a3, int a4, int b1, int b2, int b3, int b4, void* stream);
+
+/* Replaces cinn_call_batched_cublas (cuda_util.h:103-120, cuda_util.cc:312-437): v_args holds one
+ * shared operand, then (num_args-1)/2 other operands, then as many outputs; opside selects which
+ * side the shared operand is on (0 = left). */
+void cinn_call_batched_cublas(void* v_args, int num_args, int opside, bool trans_a, bool trans_b, bool trans_o,
+                              float alpha, float beta, int a1, int a2, int a3, int a4, int b1, int b2, int b3, int b4,
+                              void* stream);
+
+/* y = alpha * conv2d(x, w) + beta * y, cross-correlation, zero padding, as an implicit GEMM on
+ * MFMA.  Replaces cinn_call_cudnn_conv2d_forward (cuda_util.cc:603-720).  format: 0 = NCHW,
+ * 1 = NHWC (cudnnTensorFormat_t values).  v_args = {x, w, y}. */
+void cinn_call_cudnn_conv2d_forward(void* v_args, int num_args, int format, float alpha, float beta, int input_n,
+                                    int input_c, int input_h, int input_w, int filter_n, int filter_c, int filter_h,
+                                    int filter_w, int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h,
+                                    int dilation_w, int groups, int output_n, int output_c, int output_h,
+                                    int output_w, void* stream);
+
+/* Extension with no counterpart in the reference: the same convolution with a per-output-channel
+ * affine (y = conv * scale[c] + shift[c]) and optional ReLU applied in the kernel epilogue, so an
+ * inference batch_norm + relu that follows a convolution costs no extra pass over HBM.
+ * v_args = {x, w, scale, shift, y}; scale/shift are fp32 [output_c]. */
+void cinn_call_hip_conv2d_bn_relu(void* v_args, int num_args, int format, int relu, int input_n, int input_c,
+                                  int input_h, int input_w, int filter_n, int filter_c, int filter_h, int filter_w,
+                                  int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
+                                  int groups, int output_n, int output_c, int output_h, int output_w, void* stream);
+
+/* Replaces cinn_call_cudnn_pool2d_forward (cuda_util.cc:969-1041).  mode: 0 = max,
+ * 1 = avg counting padding, 2 = avg excluding padding, 3 = max (deterministic) — the
+ * cudnnPoolingMode_t values.  v_args = {x, y}. */
+void cinn_call_cudnn_pool2d_forward(void* v_args, int num_args, int mode, int format, float alpha, float beta,
+                                    int input_n, int input_c, int input_h, int input_w, int kernel_h, int kernel_w,
+                                    int pad_h, int pad_w, int stride_h, int stride_w, int output_n, int output_c,
+                                    int output_h, int output_w, void* stream);
+
+/* Replaces cinn_call_cudnn_softmax_forward (cuda_util.cc:1121-1167), which always runs
+ * CUDNN_SOFTMAX_LOG: y = alpha * log_softmax(x) + beta * y over C (mode 1, per position) or over
+ * C*H*W (mode 0, per instance).  v_args = {x, y}. */
+void cinn_call_cudnn_softmax_forward(void* v_args, int num_args, int mode, int format, float alpha, float beta,
+                                     int input_n, int input_c, int input_h, int input_w, int output_n, int output_c,
+                                     int output_h, int output_w, void* stream);
+
+/* Replace cinn_call_cuda_memset / cinn_call_cuda_memcpy (cuda_util.cc:439-462). */
+void cinn_call_cuda_memset(void* v_args, int num_args, int value, size_t count, void* stream);
+void cinn_call_cuda_memcpy(void* v_args, int num_args, size_t count, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Run-time compilation and code-object loading.
+ * ---------------------------------------------------------------------------------------------- */
+
+/* HIP source -> gfx950 code object through hiprtc.  Replaces nvrtc::Compiler::operator()
+ * (cinn/backends/nvrtc/nvrtc_util.cc:40-152).  The device library is prepended as an in-memory
+ * header when `with_device_lib` is non-zero.  On success *code / *code_size describe a malloc'd
+ * image the caller frees with cinn_hip_free_host; on failure the compile log is left in
+ * *log (malloc'd, may be NULL) and a non-zero status is returned. */
+int cinn_hip_rtc_compile(const char* source, int with_device_lib, const char* extra_options, char** code,
+                         size_t* code_size, char** log);
+void cinn_hip_free_host(void* p);
+/* The device library source text (wave64 reductions, math table, 128-bit access helpers) that
+ * replaces cinn/runtime/cuda/cinn_cuda_runtime_source.cuh. */
+const char* cinn_hip_device_lib_source(void);
+
+/* Code-object handle.  Replaces runtime::cuda::CUDAModule (cinn/runtime/cuda/cuda_module.cc:35-149):
+ * the image is loaded lazily with hipModuleLoadData on first cinn_hip_module_get_function. */
+typedef struct cinn_hip_module* cinn_hip_module_t;
+int cinn_hip_module_create(const void* code, size_t code_size, cinn_hip_module_t* out);
+int cinn_hip_module_get_function(cinn_hip_module_t m, const char* name, void** kernel_fn);
+int cinn_hip_module_destroy(cinn_hip_module_t m);
+
+/* ------------------------------------------------------------------------------------------------
+ * Device memory, streams, events.  Replace CudaMemoryMng (cinn/hlir/framework/memory.cc:43-64)
+ * and the cudaMemcpy / cudaDeviceSynchronize calls of frontend/computation.cc:186-215 and
+ * hlir/framework/graph_compiler.cc:212-222.
+ * ---------------------------------------------------------------------------------------------- */
+int cinn_hip_device_count(int* count);
+int cinn_hip_malloc(void** dptr, size_t bytes);
+int cinn_hip_free(void* dptr);
+int cinn_hip_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream);
+int cinn_hip_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream);
+int cinn_hip_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream);
+int cinn_hip_memset(void* dst, int value, size_t bytes, void* stream);
+int cinn_hip_device_synchronize(void);
+int cinn_hip_stream_create(void** stream);
+int cinn_hip_stream_destroy(void* stream);
+int cinn_hip_stream_synchronize(void* stream);
+int cinn_hip_event_create(void** event);
+int cinn_hip_event_destroy(void* event);
+int cinn_hip_event_record(void* event, void* stream);
+int cinn_hip_event_synchronize(void* event);
+int cinn_hip_event_elapsed_ms(void* start, void* stop, float* ms);
+const char* cinn_hip_error_string(int status);
+
+/* Device descriptor consumed by schedules.  Replaces common::Target's cudaDeviceGetAttribute
+ * queries (cinn/common/target.cc:55-84, 177-221).  Filled from the live device when one is
+ * present, otherwise with the MI355X datasheet values (256 CUs, wave64, 160 KiB LDS per CU). */
+typedef struct cinn_hip_target_info {
+  int wavefront_size;
+  int max_threads_per_block;
+  int multi_processor_count;
+  int max_threads_per_multi_processor;
+  int max_blocks_per_multi_processor;
+  int lds_bytes_per_block;
+  int lds_bytes_per_multi_processor;
+  int num_xcd;
+  int from_device; /* 1 when read from a live GPU */
+  char arch[32];
+} cinn_hip_target_info;
+int cinn_hip_get_target_info(cinn_hip_target_info* info);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CINN_HIP_RUNTIME_H_ */
