@@ -43,7 +43,8 @@ void* _Tensor_::mutable_data(const common::Target& target) {
     void* p = nullptr;
     CINN_HIP_STATUS(cinn_hip_malloc(&p, need));
     allocated_ = need;
-    int code   = type_.is_bfloat16() ? cinn_type_bfloat : static_cast<int>(type_.code);
+    // runtime tag: bool is a 1-bit cinn_type_int there (cinn/runtime/cinn_runtime.cc cinn_bool_t)
+    int code = type_.is_bool() ? cinn_type_int : (type_.is_bfloat16() ? cinn_type_bfloat : static_cast<int>(type_.code));
     cinn_hip_buffer_init(&buffer_, p, code, type_.is_bool() ? 1 : type_.bits, shape_.data(), static_cast<int>(shape_.size()));
     buffer_.memory_size = need;
   }

@@ -617,7 +617,14 @@ class RowReduceEmitter {
       value = ir::MakeLoad(materialized_buf_.at(v), LaneSlot());
     } else {
       Node* n = v->producer;
-      if (n->op->pattern == OpPatternKind::kElementWise) {
+      if (n->op_type() == "divide" && v->dtype.is_floating() && RowDivisor(n->inputs[1]) && !ExactDivision()) {
+        // x / (per-row value) -> x * (1 / per-row value): the reciprocal is taken once per row with a
+        // correctly rounded division, so the result stays within 1 ulp of the quotient while the
+        // per-element cost drops from a division sequence to one multiply
+        Expr rcp = RowReciprocal(RowDivisor(n->inputs[1]));
+        Expr a   = ElemValue(n->inputs[0]);
+        value    = ir::MakeCast(v->dtype, ir::MakeCast(rcp.type(), a) * rcp);
+      } else if (n->op->pattern == OpPatternKind::kElementWise) {
         std::vector<Expr> inputs;
         for (auto* in : n->inputs) {
           RowKind kind = KindOf(in);
@@ -648,6 +655,31 @@ class RowReduceEmitter {
     }
     elem_cache_[v] = value;
     return value;
+  }
+
+  static bool ExactDivision() { return EnvInt("FLAGS_cinn_hip_exact_division", 0) != 0; }
+
+  // the per-row value an element operand replicates, looking through reshape / broadcast_to
+  NodeData* RowDivisor(NodeData* v) const {
+    while (ctx_->produced.count(v)) {
+      Node* n = v->producer;
+      if (n->op_type() != "broadcast_to" && n->op_type() != "reshape") return nullptr;
+      v = n->inputs[0];
+      RowKind kind = KindOf(v);
+      if (kind == RowKind::kRow || kind == RowKind::kScalar) return v;
+      if (kind != RowKind::kElem) return nullptr;
+    }
+    return nullptr;
+  }
+  Expr RowReciprocal(NodeData* row_var) {
+    auto it = row_rcp_.find(row_var);
+    if (it != row_rcp_.end()) return it->second;
+    Expr b      = RowValue(row_var);
+    Type wide   = b.type().bits < 32 ? common::Float(32) : b.type();
+    Expr var    = ctx_->NewVar("rcp", wide);
+    row_stmts_->push_back(ir::MakeLet(var, ir::MakeConst(wide, 1) / ir::MakeCast(wide, b)));
+    row_rcp_[row_var] = var;
+    return var;
   }
 
   struct Accumulator {
@@ -767,6 +799,7 @@ class RowReduceEmitter {
   std::vector<Expr>* lane_stmts_{nullptr};
   int cur_phase_{0};
   std::map<const NodeData*, Expr> row_values_;
+  std::map<const NodeData*, Expr> row_rcp_;
   std::set<const NodeData*> stored_rows_;
   std::map<const NodeData*, Expr> elem_cache_;
   std::map<const NodeData*, Stage> stage_;

@@ -27,7 +27,9 @@ void cinn_hip_buffer_init(cinn_buffer_t* buf, void* device_ptr, int32_t type_cod
   buf->flag              = cinn_buffer_on_device;
   buf->type.code         = type_code;
   buf->type.bits         = static_cast<uint8_t>(bits);
-  buf->type.lanes        = 1;
+  // the reference's cinn_float32_t() & co. leave lanes at 0 (cinn/runtime/cinn_runtime.cc passes
+  // num_asterisks in the lanes slot); buffers made by its Tensor class therefore carry lanes == 0
+  buf->type.lanes        = 0;
   buf->type.num_asterisks = 0;
   buf->dimensions        = ndims > CINN_BUFFER_MAX_DIMS ? CINN_BUFFER_MAX_DIMS : ndims;
   uint64_t n             = 1;

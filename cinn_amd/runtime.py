@@ -32,7 +32,8 @@ class cinn_pod_value_t(ctypes.Structure):
 _TYPE_CODES = {  # dtype name -> (cinn_type_code_t, bits)
     "float16": (2, 16), "float32": (2, 32), "float64": (2, 64), "bfloat16": (4, 16),
     "int8": (0, 8), "int16": (0, 16), "int32": (0, 32), "int64": (0, 64),
-    "uint8": (1, 8), "uint16": (1, 16), "uint32": (1, 32), "uint64": (1, 64), "bool": (1, 1),
+    "uint8": (1, 8), "uint16": (1, 16), "uint32": (1, 32), "uint64": (1, 64),
+    "bool": (0, 1),  # the reference tags bool as a 1-bit signed int (cinn_runtime.cc cinn_bool_t)
 }
 
 

@@ -1,0 +1,177 @@
+"""Host logic that needs no GPU: NetBuilder shape / type inference, broadcasting rules, attribute
+normalisation, the decomposer, fusion grouping and the structure of the generated HIP source (the
+analogue of the reference's golden-source tests in cinn/backends/ir_schedule_test.cc, structural
+because the code generator is new)."""
+import re
+
+import numpy as np
+import pytest
+
+from cinn_amd import _lib
+from cinn_amd.common import Bool, Float, Int
+from cinn_amd.frontend import NetBuilder
+
+from helpers import compile_only
+
+
+def test_unary_binary_shapes_and_types():
+    b = NetBuilder("t")
+    x = b.create_input(Float(32), [4, 8], "x")
+    y = b.create_input(Float(32), [4, 8], "y")
+    assert b.exp(x).shape() == [4, 8]
+    assert b.add(x, y).type() == Float(32)
+    assert b.greater_than(x, y).type() == Bool()
+    assert b.cast(x, "float16").type() == Float(16)
+    assert b.is_nan(x).type() == Bool()
+
+
+def test_binary_broadcast_follows_axis_rule():
+    b = NetBuilder("t")
+    x = b.create_input(Float(32), [2, 3, 4, 5], "x")
+    c = b.create_input(Float(32), [3], "c")
+    # axis=1: the vector lines up with dimension 1 (pe::GetBroadcastShape, hlir/pe/broadcast.cc:34-80)
+    assert b.add(x, c, axis=1).shape() == [2, 3, 4, 5]
+    z = b.create_input(Float(32), [4, 5], "z")
+    assert b.multiply(x, z).shape() == [2, 3, 4, 5]  # numpy alignment for axis=-1
+    o = b.create_input(Float(32), [1, 3, 1, 5], "o")
+    assert b.subtract(o, x).shape() == [2, 3, 4, 5]
+    with pytest.raises(_lib.CinnError):
+        b.add(x, b.create_input(Float(32), [7], "bad"))
+    with pytest.raises(_lib.CinnError):
+        b.add(x, b.create_input(Float(16), [2, 3, 4, 5], "h"))  # operand types must be equal
+
+
+def test_broadcast_to_one_dimension_picks_first_matching_axis():
+    b = NetBuilder("t")
+    v = b.create_input(Float(32), [4], "v")
+    out = b.broadcast_to(v, [4, 3, 4])
+    assert out.shape() == [4, 3, 4]
+    assert "broadcast_axes=[0]" in str(b)
+
+
+def test_reduce_shapes():
+    b = NetBuilder("t")
+    x = b.create_input(Float(32), [2, 3, 4], "x")
+    assert b.reduce_sum(x, [1]).shape() == [2, 4]
+    assert b.reduce_max(x, [1], keep_dim=True).shape() == [2, 1, 4]
+    assert b.reduce_sum(x, [-1]).shape() == [2, 3]
+    assert b.reduce_sum(x).shape() == [1]
+    assert b.argmax(x, axis=1).shape() == [2, 4]
+    assert b.argmax(x, axis=1).type() == Int(32)
+    assert b.argmax(x, axis=2, keep_dim=True).shape() == [2, 3, 1]
+    one = b.create_input(Float(32), [1, 1], "one")
+    assert b.reduce_sum(one, [0]).shape() == [1]  # single element: reshaped, not reduced
+
+
+def test_matmul_conv_pool_shapes():
+    b = NetBuilder("t")
+    a = b.create_input(Float(32), [8, 16], "a")
+    w = b.create_input(Float(32), [16, 4], "w")
+    assert b.matmul(a, w).shape() == [8, 4]
+    assert b.matmul(w, a, trans_x=True, trans_y=True).shape() == [4, 8]
+    ba = b.create_input(Float(32), [3, 8, 16], "ba")
+    assert b.matmul(ba, w).shape() == [3, 8, 4]
+    x = b.create_input(Float(32), [32, 256, 56, 56], "xc")
+    k = b.create_input(Float(32), [512, 256, 1, 1], "kc")
+    assert b.conv2d(x, k, strides=[2, 2]).shape() == [32, 512, 28, 28]
+    x3 = b.create_input(Float(32), [2, 64, 56, 56], "x3")
+    k3 = b.create_input(Float(32), [64, 64, 3, 3], "k3")
+    assert b.conv2d(x3, k3, paddings=[1, 1]).shape() == [2, 64, 56, 56]
+    p = b.create_input(Float(32), [2, 64, 112, 112], "p")
+    assert b.pool2d(p, "max", [3, 3], [2, 2], [1, 1]).shape() == [2, 64, 56, 56]
+    assert b.pool2d(p, "avg", [7, 7], global_pooling=True).shape() == [2, 64, 1, 1]
+    assert b.pool2d(p, "max", [3, 3], [2, 2], [0, 0], ceil_mode=True).shape() == [2, 64, 56, 56]
+    assert b.pool2d(p, "max", [3, 3], [2, 2], [0, 0], padding_algorithm="SAME").shape() == [2, 64, 56, 56]
+    with pytest.raises(_lib.CinnError):
+        b.pool2d(p, "median", [3, 3])
+
+
+def test_softmax_decomposes_and_fuses_into_one_row_kernel():
+    b = NetBuilder("t")
+    x = b.create_input(Float(32), [64, 4096], "x")
+    y = b.softmax(x, axes=[-1])
+    comp = compile_only(b, [y])
+    groups = comp.fusion_groups().strip().splitlines()
+    assert len(groups) == 1 and "row_reduce[64x4096]" in groups[0]
+    # exp appears once: the duplicated exp(x) of the decomposition is merged
+    assert groups[0].count(" exp") == 1
+    src = comp.source_code()
+    assert src.count("__global__") == 1
+    assert "cinn_wave_shuffle_sum_fp32_internal" in src  # 4096 / 64 lanes = 64 elements per lane: one wave per row
+    assert "__syncthreads" not in src
+    assert src.count("cinn_hip_exp_fp32") == 1
+    assert "cinn_hip_copy_vec<float, 4>" in src
+    assert re.search(r"__launch_bounds__\(256\)", src)
+
+
+def test_long_rows_use_a_block_per_row():
+    b = NetBuilder("t")
+    x = b.create_input(Float(32), [8, 32768], "x")
+    comp = compile_only(b, [b.reduce_sum(x, [1])])
+    src = comp.source_code()
+    assert "cinn_block_reduce_sum_fp32_internal" in src
+    assert re.search(r"__launch_bounds__\((512|1024)\)", src)
+
+
+def test_layer_norm_is_one_kernel_with_three_outputs():
+    b = NetBuilder("t")
+    x = b.create_input(Float(16), [64, 1024], "x")
+    g = b.create_input(Float(32), [1024], "g")
+    be = b.create_input(Float(32), [1024], "be")
+    y, mean, var = b.paddle_layer_norm(x, g, be)
+    comp = compile_only(b, [y, mean, var])
+    assert comp.num_instructions() == 1
+    src = comp.source_code()
+    assert src.count("cinn_wave_shuffle_sum_fp32_internal") == 2  # sum(x) and sum(x*x) in the same pass
+    assert "cinn_hip_copy_vec<float16, 8>" in src  # 128-bit accesses on the fp16 tensors
+    fn, args = comp.instruction_info(0)
+    assert args[:3] == ["x", "g", "be"] and len(args) == 6
+
+
+def test_elementwise_chain_is_one_kernel_and_library_ops_split_groups():
+    b = NetBuilder("t")
+    a = b.create_input(Float(32), [64, 64], "a")
+    w = b.create_input(Float(32), [64, 64], "w")
+    h = b.relu(b.matmul(b.exp(a), w))
+    out = b.add(h, a)
+    comp = compile_only(b, [out])
+    kinds = [line.split()[2] for line in comp.fusion_groups().strip().splitlines()]
+    assert kinds == ["elementwise", "library_call", "elementwise"]
+    fn, args = comp.instruction_info(1)
+    assert fn.startswith("fn_matmul")
+
+
+def test_batch_norm_keeps_the_reference_operation_order():
+    b = NetBuilder("t")
+    x = b.create_input(Float(32), [2, 8, 4, 4], "x")
+    params = [b.create_input(Float(32), [8], n) for n in ("scale", "bias", "mean", "var")]
+    y = b.batchnorm(x, params[0], params[1], params[2], params[3])[0]
+    comp = compile_only(b, [b.relu(y)])
+    src = comp.source_code()
+    # (x - mean) * scale / sqrt(var + eps) + bias, then relu: one full-size kernel plus the per-channel sqrt
+    full = [k for k in src.split("extern \"C\"") if "float* __restrict__ x" in k or "x," in k]
+    assert any("cinn_hip_max_generic" in k for k in full)
+    assert src.count("cinn_hip_sqrt_fp32") == 1
+
+
+def test_unknown_operator_and_bad_fetch_are_reported():
+    b = NetBuilder("t")
+    x = b.create_input(Float(32), [4], "x")
+    with pytest.raises(_lib.CinnError) as e:
+        b.custom_instr("no_such_op", [x])
+    assert "no_such_op" in str(e.value)
+    with pytest.raises(_lib.CinnError):
+        b.reshape(x, [3])
+
+
+def test_generated_source_idioms():
+    b = NetBuilder("t")
+    x = b.create_input(Float(32), [1000, 3], "x")  # 3000 elements: not a multiple of 256*4 -> guarded tail
+    y = b.scale(b.sigmoid(x), scale=2.0, bias=0.5)
+    comp = compile_only(b, [y])
+    src = comp.source_code()
+    assert "extern \"C\" __global__" in src
+    assert "const float* __restrict__ x" in src and "float* __restrict__ " in src
+    assert "(int32_t)blockIdx.x" in src and "(int32_t)threadIdx.x" in src
+    assert "2.0f" in src and "0.5f" in src
+    assert re.search(r"if \(.*< 750\)", src)  # 3000 / 4 vectors

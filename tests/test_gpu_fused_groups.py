@@ -1,0 +1,195 @@
+"""GPU parity of the generated fused element-wise and reduce kernels (BASELINE configs 1 and 2) against the
+CPU oracle on identical seeded inputs, at the full config sizes, plus the shapes and edge cases the
+reference's own op tests use (python/tests/ops/test_softmax_op.py, test_reduce_op.py, test_argmax_op.py,
+cinn/hlir/op/reduction_test.cc).  Bars: fp32 1e-5 relative, fp16 1e-2 relative (+ one fp16 subnormal
+quantum), integer / index results bit-exact."""
+import numpy as np
+import pytest
+
+import oracle
+from cinn_amd.common import Bool, Float, Int
+from cinn_amd.frontend import NetBuilder
+
+from helpers import assert_close_fp16, run
+
+pytestmark = pytest.mark.gpu
+
+
+def test_config1_add_relu_full_size(gpu):
+    rng = np.random.default_rng(11)
+    a = rng.uniform(-1, 1, (1, 3, 224, 224)).astype(np.float32)
+    b_ = rng.uniform(-1, 1, (1, 3, 224, 224)).astype(np.float32)
+    b = NetBuilder("c1")
+    A, B = b.create_input(Float(32), a.shape, "A"), b.create_input(Float(32), a.shape, "B")
+    (y,), comp = run(b, {A: a, B: b_}, [b.relu(b.add(A, B))])
+    assert comp.num_instructions() == 1
+    assert np.array_equal(y, oracle.add_relu(a, b_))  # one add, one max: bit-exact
+
+
+@pytest.mark.parametrize("n", [1, 3, 255, 1000, 4099, 150528 + 4])
+def test_elementwise_ragged_sizes(gpu, n):
+    rng = np.random.default_rng(n)
+    a, b_ = rng.uniform(-1, 1, n).astype(np.float32), rng.uniform(-1, 1, n).astype(np.float32)
+    b = NetBuilder("r")
+    A, B = b.create_input(Float(32), [n], "A"), b.create_input(Float(32), [n], "B")
+    (y,), _ = run(b, {A: a, B: b_}, [b.relu(b.add(A, B))])
+    assert np.array_equal(y, oracle.add_relu(a, b_))
+
+
+def test_relu_special_values(gpu):
+    a = np.array([-0.0, 0.0, -1.0, 2.5, np.inf, -np.inf, 1e-45, -1e-45], np.float32)
+    b = NetBuilder("s")
+    A = b.create_input(Float(32), [8], "A")
+    (y,), _ = run(b, {A: a}, [b.relu(A)])
+    assert np.array_equal(y, oracle.add_relu(a, np.zeros(8, np.float32)))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_config2_softmax_full_size(gpu, dtype):
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((4096, 4096)).astype(dtype)
+    b = NetBuilder("sm")
+    X = b.create_input(Float(32) if dtype == "float32" else Float(16), x.shape, "x")
+    (y,), comp = run(b, {X: x}, [b.softmax(X, axes=[-1])])
+    assert comp.num_instructions() == 1
+    want = oracle.softmax(x)
+    if dtype == "float32":
+        np.testing.assert_allclose(y, want, rtol=1e-5, atol=0)
+        np.testing.assert_allclose(y.sum(-1, dtype=np.float64), 1.0, rtol=1e-5)
+    else:
+        assert_close_fp16(y, want)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_config2_layer_norm_full_size(gpu, dtype):
+    rng = np.random.default_rng(22)
+    x = rng.standard_normal((8192, 1024)).astype(dtype)
+    g = rng.uniform(0.5, 1.5, 1024).astype(np.float32)
+    be = rng.uniform(0.5, 1.5, 1024).astype(np.float32)
+    b = NetBuilder("ln")
+    X = b.create_input(Float(32) if dtype == "float32" else Float(16), x.shape, "x")
+    G, Be = b.create_input(Float(32), [1024], "g"), b.create_input(Float(32), [1024], "be")
+    (y, m, v), comp = run(b, {X: x, G: g, Be: be}, b.paddle_layer_norm(X, G, Be, epsilon=1e-5))
+    assert comp.num_instructions() == 1
+    wy, wm, wv = oracle.layer_norm(x, g, be, 1e-5)
+    if dtype == "float32":
+        # (x - mean) loses relative accuracy where x is close to mean: bound the error relative to the scale of
+        # the normalised values (|y| ~ 1) as the reference's own comparison does with rtol 1e-5 + atol
+        np.testing.assert_allclose(y, wy, rtol=1e-5, atol=1e-5)
+    else:
+        # y = v * gamma + beta cancels to values near zero for some elements; there the half rounding of an
+        # fp32 intermediate that differs in its last bit decides the result, so the bound needs an absolute
+        # part at the scale of the operands (|v * gamma|, |beta| ~ 1): one fp16 ulp at 1.0 is 9.8e-4
+        np.testing.assert_allclose(y.astype(np.float64), wy.astype(np.float64), rtol=1e-2, atol=1e-3)
+    np.testing.assert_allclose(m, wm, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(v, wv, rtol=1e-5, atol=1e-6)
+
+
+def test_config2_int32_reduce_sum_and_argmax_full_size(gpu):
+    rng = np.random.default_rng(23)
+    x = rng.integers(-1000, 1000, (16384, 512), endpoint=True).astype(np.int32)
+    b = NetBuilder("ri")
+    X = b.create_input(Int(32), x.shape, "x")
+    (s,), _ = run(b, {X: x}, [b.reduce_sum(X, [1])])
+    assert np.array_equal(s, oracle.reduce_sum_i32(x))
+    b = NetBuilder("am")
+    X = b.create_input(Int(32), x.shape, "x")
+    (am,), _ = run(b, {X: x}, [b.argmax(X, axis=1)])
+    want = oracle.argmax_last(x)
+    assert am.dtype == np.int32 and np.array_equal(am, want)
+    # with 512 draws from 2001 values ties for the maximum are common: make sure the test saw some
+    ties = (x == x.max(1, keepdims=True)).sum(1) > 1
+    assert ties.sum() > 100
+
+
+def test_argmax_ties_and_constant_rows(gpu):
+    x = np.zeros((64, 512), np.int32)
+    x[1, 511] = 5
+    x[2, [100, 300]] = 9
+    x[3, :] = -7
+    x[4, [0, 511]] = 3
+    b = NetBuilder("t")
+    X = b.create_input(Int(32), x.shape, "x")
+    (am, amin), _ = run(b, {X: x}, [b.argmax(X, axis=1), b.argmin(X, axis=1)])
+    assert np.array_equal(am, x.argmax(1).astype(np.int32))
+    assert np.array_equal(amin, x.argmin(1).astype(np.int32))
+
+
+# shapes of python/tests/ops/test_softmax_op.py:55-88 (axis is moved last with a transpose when it is not)
+@pytest.mark.parametrize("shape,axis", [([1], 0), ([1024], -1), ([512, 256], 0), ([128, 64, 32], 1),
+                                        ([16, 8, 4, 2], 2), ([16, 8, 4, 2, 1], 2), ([1, 1, 1, 1, 1], 2),
+                                        ([3, 1000], 1), ([5, 33], -1)])
+def test_softmax_reference_shapes(gpu, shape, axis):
+    rng = np.random.default_rng(5)
+    x = rng.uniform(-1, 1, shape).astype(np.float32)
+    b = NetBuilder("s")
+    X = b.create_input(Float(32), shape, "x")
+    (y,), _ = run(b, {X: x}, [b.softmax(X, axes=[axis])])
+    e = np.exp(x.astype(np.float64))
+    want = e / e.sum(axis, keepdims=True)
+    np.testing.assert_allclose(y, want, rtol=1e-5, atol=1e-7)
+    ax = axis % len(shape)
+    if ax == len(shape) - 1:
+        np.testing.assert_allclose(y, oracle.softmax(x), rtol=1e-5, atol=0)
+
+
+# reduce cases in the spirit of cinn/hlir/op/reduction_test.cc:293-404 and python/tests/ops/test_reduce_op.py
+@pytest.mark.parametrize("shape,dim,keep", [
+    ([32, 64], [1], False), ([32, 64], [0], False), ([16, 16, 32], [0, 2], False), ([8, 16, 16, 8], [2, 3], True),
+    ([4, 8, 16, 32], [1], False), ([128, 1023], [1], False), ([3, 9000], [1], False), ([7, 70000], [1], False),
+    ([2, 3, 5], [], False), ([1, 1], [0], False), ([1, 257], [1], True), ([512, 2], [1], False),
+])
+@pytest.mark.parametrize("op", ["reduce_sum", "reduce_max", "reduce_min", "reduce_prod"])
+def test_reduce_ops(gpu, shape, dim, keep, op):
+    rng = np.random.default_rng(7)
+    if op == "reduce_prod":
+        x = rng.uniform(0.9, 1.1, shape).astype(np.float32)
+    else:
+        x = rng.standard_normal(shape).astype(np.float32)
+    b = NetBuilder("r")
+    X = b.create_input(Float(32), shape, "x")
+    (y,), _ = run(b, {X: x}, [getattr(b, op)(X, dim, keep)])
+    fn = {"reduce_sum": np.sum, "reduce_max": np.max, "reduce_min": np.min, "reduce_prod": np.prod}[op]
+    axes = tuple(dim) if dim else None
+    want = fn(x.astype(np.float64), axis=axes, keepdims=keep)
+    want = np.asarray(want).reshape(y.shape)
+    np.testing.assert_allclose(y, want, rtol=1e-4 if op == "reduce_prod" else 1e-5, atol=1e-4)
+
+
+def test_reduce_all_any_bool(gpu):
+    rng = np.random.default_rng(8)
+    x = rng.uniform(0, 1, (64, 300)) > 0.01
+    x[5, :] = True
+    x[6, :] = False
+    b = NetBuilder("b")
+    X = b.create_input(Bool(), x.shape, "x")
+    (a, o), _ = run(b, {X: x}, [b.reduce_all(X, [1]), b.reduce_any(X, [1])])
+    assert np.array_equal(a, x.all(1)) and np.array_equal(o, x.any(1))
+
+
+@pytest.mark.parametrize("shape,axis", [([4, 3, 28, 28], 1), ([16, 100], 0), ([2, 5, 7], 2), ([2, 5, 7], 0)])
+def test_argmax_any_axis(gpu, shape, axis):
+    rng = np.random.default_rng(9)
+    x = rng.integers(-5, 5, shape).astype(np.float32)  # many ties
+    b = NetBuilder("a")
+    X = b.create_input(Float(32), shape, "x")
+    (y, yk), _ = run(b, {X: x}, [b.argmax(X, axis=axis), b.argmax(X, axis=axis, keep_dim=True)])
+    assert np.array_equal(y, x.argmax(axis).astype(np.int32))
+    assert np.array_equal(yk, np.expand_dims(x.argmax(axis), axis).astype(np.int32))
+
+
+def test_fused_reduce_with_producers_and_consumers(gpu):
+    # x -> exp -> (row max, row sum) -> normalised difference; every value stays in one kernel
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((100, 777)).astype(np.float32)
+    b = NetBuilder("f")
+    X = b.create_input(Float(32), x.shape, "x")
+    e = b.exp(X)
+    mx = b.reduce_max(e, [1], keep_dim=True)
+    sm = b.reduce_sum(e, [1], keep_dim=True)
+    out = b.divide(b.subtract(e, b.broadcast_to(mx, x.shape)), b.broadcast_to(sm, x.shape))
+    (y, s), comp = run(b, {X: x}, [out, sm])
+    assert comp.num_instructions() == 1
+    e64 = np.exp(x.astype(np.float64))
+    np.testing.assert_allclose(y, (e64 - e64.max(1, keepdims=True)) / e64.sum(1, keepdims=True), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(s, e64.sum(1, keepdims=True), rtol=1e-5)
