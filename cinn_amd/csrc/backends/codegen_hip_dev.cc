@@ -111,7 +111,9 @@ void CodeGenHIP_Dev::VisitStore(const Store* op) {
   CINN_CHECK(ld) << "a vector store must copy a vector load";
   auto* lramp = ld->index.As<Ramp>();
   CINN_CHECK(lramp && lramp->lanes == ramp->lanes && lramp->stride == 1 && ramp->stride == 1);
-  os_ << "cinn_hip_copy_vec<" << common::TypeCName(op->buffer->dtype) << ", " << ramp->lanes << ">(&"
+  const char* copy_fn = "cinn_hip_copy_vec";
+  if (op->buffer->memory_type == MemoryType::Global && op->buffer->streaming_store) copy_fn = "cinn_hip_store_stream_vec";
+  os_ << copy_fn << "<" << common::TypeCName(op->buffer->dtype) << ", " << ramp->lanes << ">(&"
       << op->buffer->name << "[";
   Visit(ramp->base);
   os_ << "], &" << ld->buffer->name << "[";

@@ -105,7 +105,7 @@ Program ApplyDecomposer(const Program& program) {
       out.push_back(ins);
     }
   }
-  return Program(std::move(out), program.GetInputs());
+  return Program(std::move(out), program.GetInputs(), program.name());
 }
 
 }  // namespace frontend

@@ -18,7 +18,7 @@ std::string NetBuilder::NewVarId(const std::string& hint) { return hint + "_" + 
 Program NetBuilder::Build(bool in_reverse) {
   std::vector<Instruction> instrs = instrs_;
   if (in_reverse) std::reverse(instrs.begin(), instrs.end());
-  return Program(std::move(instrs), inputs_);
+  return Program(std::move(instrs), inputs_, name_);
 }
 
 Placeholder NetBuilder::CreateInput(const common::Type& type, const ShapeType& shape, const std::string& id_hint) {

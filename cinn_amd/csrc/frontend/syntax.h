@@ -79,8 +79,10 @@ class Instruction {
 class Program {
  public:
   Program() = default;
-  Program(std::vector<Instruction> instrs, std::vector<Variable> inputs)
-      : instrs_(std::move(instrs)), inputs_(std::move(inputs)) {}
+  Program(std::vector<Instruction> instrs, std::vector<Variable> inputs, std::string name = "")
+      : instrs_(std::move(instrs)), inputs_(std::move(inputs)), name_(std::move(name)) {}
+  // name of the builder that made the program; generated kernels carry it in their names
+  const std::string& name() const { return name_; }
   size_t size() const { return instrs_.size(); }
   const Instruction& operator[](size_t i) const { return instrs_[i]; }
   const std::vector<Instruction>& instructions() const { return instrs_; }
@@ -91,6 +93,7 @@ class Program {
  private:
   std::vector<Instruction> instrs_;
   std::vector<Variable> inputs_;
+  std::string name_;
 };
 
 }  // namespace frontend

@@ -286,7 +286,7 @@ void Graph::BuildFusionGroups() {
       }
     }
     std::string base = g->nodes.back()->op_type();
-    g->func_name     = "fn_" + base + "_" + std::to_string(g->id);
+    g->func_name     = "fn_" + (name_.empty() ? std::string() : name_ + "_") + base + "_" + std::to_string(g->id);
     groups.push_back(std::move(g));
   }
 }

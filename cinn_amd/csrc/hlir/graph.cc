@@ -21,6 +21,7 @@ NodeData* Graph::GetOrCreateVar(const frontend::Variable& v) {
 
 Graph::Graph(const frontend::Program& program, const std::set<std::string>& fetch_ids, const common::Target& target)
     : target_(target) {
+  for (char c : program.name()) name_.push_back((isalnum(static_cast<unsigned char>(c)) || c == '_') ? c : '_');
   for (auto& in : program.GetInputs()) inputs_.push_back(GetOrCreateVar(in));
 
   // Common sub-expression elimination while the graph is built: an instruction with the same op,

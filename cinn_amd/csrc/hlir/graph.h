@@ -62,6 +62,7 @@ class Graph {
   Graph(const frontend::Program& program, const std::set<std::string>& fetch_ids, const common::Target& target);
 
   const common::Target& target() const { return target_; }
+  const std::string& name() const { return name_; }
   const std::vector<std::unique_ptr<Node>>& nodes() const { return nodes_; }
   NodeData* FindVar(const std::string& id) const;
   const std::vector<NodeData*>& inputs() const { return inputs_; }
@@ -76,6 +77,7 @@ class Graph {
  private:
   NodeData* GetOrCreateVar(const frontend::Variable& v);
   common::Target target_;
+  std::string name_;
   std::vector<std::unique_ptr<Node>> nodes_;
   std::map<std::string, std::unique_ptr<NodeData>> vars_;
   std::vector<NodeData*> inputs_;

@@ -232,6 +232,9 @@ LoweringOptions LoweringOptions::FromEnv() {
   LoweringOptions o;
   o.max_cached_elems_per_thread = EnvInt("FLAGS_cinn_hip_reduce_cached_elems", o.max_cached_elems_per_thread);
   o.wave_row_elems_per_lane     = EnvInt("FLAGS_cinn_hip_reduce_wave_elems", o.wave_row_elems_per_lane);
+  o.block_row_elems_per_thread  = EnvInt("FLAGS_cinn_hip_reduce_block_elems", o.block_row_elems_per_thread);
+  o.nontemporal_store_bytes     = static_cast<int64_t>(EnvInt("FLAGS_cinn_hip_nontemporal_store_mb", 8)) << 20;
+  o.rows_per_wave               = EnvInt("FLAGS_cinn_hip_reduce_rows_per_wave", o.rows_per_wave);
   o.elementwise_block           = EnvInt("FLAGS_cinn_hip_elementwise_block", o.elementwise_block);
   o.rows_per_block              = EnvInt("FLAGS_cinn_hip_reduce_rows_per_block", o.rows_per_block);
   return o;
@@ -356,8 +359,18 @@ bool UsedAtIdentityOnly(const Group& g, const NodeData* v, int64_t numel) {
 
 }  // namespace
 
+namespace {
+void MarkStreamingOutputs(GroupContext* ctx, int64_t threshold_bytes) {
+  if (threshold_bytes <= 0) return;
+  for (auto* o : ctx->group.outputs) {
+    if (o->numel() * o->dtype.bytes() >= threshold_bytes) ctx->global_bufs.at(o)->streaming_store = true;
+  }
+}
+}  // namespace
+
 ir::LoweredFuncRef OpLowerer::LowerElementwise(const Group& group) const {
   GroupContext ctx(group);
+  MarkStreamingOutputs(&ctx, options_.nontemporal_store_bytes);
   CINN_CHECK(!group.outputs.empty());
   const int64_t numel = group.outputs[0]->numel();
   for (auto* o : group.outputs) CINN_CHECK_EQ(o->numel(), numel) << "outputs of an element-wise group differ in size";
@@ -811,6 +824,7 @@ class RowReduceEmitter {
 
 ir::LoweredFuncRef OpLowerer::LowerRowReduce(const Group& group) const {
   GroupContext ctx(group);
+  MarkStreamingOutputs(&ctx, options_.nontemporal_store_bytes);
   std::map<const NodeData*, RowKind> kinds;
   CINN_CHECK(ClassifyRowReduceGroup(group.nodes, group.rows, group.cols, &kinds))
       << "group " << group.func_name << " is not a row-reduce group";
@@ -840,8 +854,7 @@ ir::LoweredFuncRef OpLowerer::LowerRowReduce(const Group& group) const {
     // whole block per row: the smallest power-of-two block (up to 1024 threads) that keeps the row
     // within the register budget
     int team = 128;
-    while (team < target_.max_num_threads() &&
-           (plan.cols + team - 1) / team > options_.max_cached_elems_per_thread) {
+    while (team < target_.max_num_threads() && (plan.cols + team - 1) / team > options_.block_row_elems_per_thread) {
       team *= 2;
     }
     plan.team           = team;
@@ -855,18 +868,28 @@ ir::LoweredFuncRef OpLowerer::LowerRowReduce(const Group& group) const {
   RowReduceEmitter emitter(&ctx, plan, kinds);
   std::vector<Expr> row_body = emitter.EmitRowBody();
 
+  // short rows: let a wavefront work through several rows so that more loads are in flight per lane
+  int rows_per_wave = 1;
+  if (plan.team == wave) {
+    rows_per_wave = std::max(1, options_.rows_per_wave);
+  }
   Expr bx = ir::MakeVar("bx", common::Int(32));
   Expr ty = ir::MakeVar("ty", common::Int(32));
-  int64_t grid = (plan.rows + plan.rows_per_block - 1) / plan.rows_per_block;
-  Expr row_index = plan.rows_per_block > 1 ? bx * I32(plan.rows_per_block) + ty : bx;
+  Expr rr = ir::MakeVar("rr", common::Int(32));
+  int64_t rows_per_group = static_cast<int64_t>(plan.rows_per_block) * rows_per_wave;
+  int64_t grid           = (plan.rows + rows_per_group - 1) / rows_per_group;
+  Expr wave_index        = plan.rows_per_block > 1 ? bx * I32(plan.rows_per_block) + ty : bx;
+  Expr row_index         = rows_per_wave > 1 ? wave_index * I32(rows_per_wave) + rr : wave_index;
 
-  std::vector<Expr> per_thread;
-  per_thread.push_back(ir::MakeLet(emitter.row(), row_index));
+  std::vector<Expr> per_row;
+  per_row.push_back(ir::MakeLet(emitter.row(), row_index));
   Expr work = ir::MakeBlock(row_body);
-  if (plan.rows % plan.rows_per_block != 0) work = ir::MakeIf(emitter.row() < I32(plan.rows), work);
-  per_thread.push_back(work);
+  if (plan.rows % rows_per_group != 0) work = ir::MakeIf(emitter.row() < I32(plan.rows), work);
+  per_row.push_back(work);
+  Expr per_thread = ir::MakeBlock(per_row);
+  if (rows_per_wave > 1) per_thread = ir::MakeFor(rr, I32(0), I32(rows_per_wave), ForType::Unrolled, per_thread);
 
-  Expr body = ir::MakeFor(emitter.tx(), I32(0), I32(plan.team), ForType::Serial, ir::MakeBlock(per_thread), ThreadAxis(0));
+  Expr body = ir::MakeFor(emitter.tx(), I32(0), I32(plan.team), ForType::Serial, per_thread, ThreadAxis(0));
   if (plan.rows_per_block > 1) body = ir::MakeFor(ty, I32(0), I32(plan.rows_per_block), ForType::Serial, body, ThreadAxis(1));
   ctx.func->body = ir::MakeFor(bx, I32(0), I32(grid), ForType::Serial, body, BlockAxis(0));
   return ctx.func;

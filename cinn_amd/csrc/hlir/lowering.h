@@ -26,10 +26,19 @@ struct LoweringOptions {
   int max_cached_elems_per_thread{64};
   // elements per lane above which a row is given to a whole block instead of one wavefront
   int wave_row_elems_per_lane{64};
+  // elements per thread a block-per-row team aims for (the team is the smallest power of two of at
+  // least 128 threads that gets at or below this)
+  int block_row_elems_per_thread{16};
+  // outputs of at least this many bytes are written with non-temporal stores (0 disables): a large
+  // streamed output would otherwise evict the input rows still to be read from the last-level cache
+  int64_t nontemporal_store_bytes{8 << 20};
   // threads of an element-wise block
   int elementwise_block{256};
   // waves (rows) per block when one wavefront owns a row
   int rows_per_block{4};
+  // rows one wavefront works through (unrolled, so their loads overlap).  Measured on MI355X this does
+  // not pay for the BASELINE shapes (1 is the best setting for every one of them), so it stays a knob.
+  int rows_per_wave{1};
   static LoweringOptions FromEnv();
 };
 

@@ -141,6 +141,9 @@ struct Buffer {
   Type dtype;
   MemoryType memory_type{MemoryType::Global};
   int64_t num_elements{0};
+  // global output that is written once and not re-read by this kernel: vector stores to it carry the
+  // non-temporal hint so that they do not displace the data still being read
+  bool streaming_store{false};
   Buffer(std::string n, Type t, MemoryType m, int64_t size) : name(std::move(n)), dtype(t), memory_type(m), num_elements(size) {}
 };
 using BufferRef = std::shared_ptr<Buffer>;

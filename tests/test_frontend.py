@@ -138,7 +138,7 @@ def test_elementwise_chain_is_one_kernel_and_library_ops_split_groups():
     kinds = [line.split()[2] for line in comp.fusion_groups().strip().splitlines()]
     assert kinds == ["elementwise", "library_call", "elementwise"]
     fn, args = comp.instruction_info(1)
-    assert fn.startswith("fn_matmul")
+    assert fn.startswith("fn_t_matmul")  # fn_<builder name>_<root op>_<group id>
 
 
 def test_batch_norm_keeps_the_reference_operation_order():
