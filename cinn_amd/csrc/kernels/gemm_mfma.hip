@@ -1,0 +1,579 @@
+// Hand-written CDNA4 (gfx950) GEMM kernels behind cinn_call_cublas / cinn_call_batched_cublas.
+//
+//   C[M,N] = alpha * op(A)[M,K] * op(B)[K,N] + beta * C          (row-major, optional batch)
+//
+// Three kernels:
+//   * gemm16_mfma_kernel  - bf16 / fp16 inputs, fp32 accumulation on v_mfma_f32_32x32x16_{bf16,f16}.
+//     256x256 block tile, 64-deep K step, 256 threads = 4 wavefronts in a 2x2 grid, each wavefront owning a
+//     128x128 tile (16 MFMA accumulator tiles = 256 accumulator registers).  Both operand tiles live in LDS
+//     as [row][k] with k contiguous, 128 bytes per row, double buffered (2 x 64 KiB of the 160 KiB per CU);
+//     16-byte chunks are XOR-swizzled so that the ds_read_b128 of MFMA fragments and the transposing stores
+//     are conflict free.  Operands whose contiguous axis is not K (row-major B, transposed A) are transposed
+//     in registers (8x8 blocks of 16-bit values) on their way into LDS.  Requires M%256 == N%256 == K%64 == 0.
+//   * gemm32_mfma_kernel  - fp32 on v_mfma_f32_32x32x2f32, 128x128 tile, for M%128 == N%128 == K%16 == 0.
+//   * gemm_generic_kernel - any shape / transpose / type (fp16, bf16, fp32, fp64): 64x64 LDS tile, FMA units.
+#include <hip/hip_runtime.h>
+
+#include <climits>
+#include <cstdint>
+
+#include "cinn_hip_runtime.h"
+#include "runtime/hip_check.h"
+
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T>
+struct Half16;
+template <>
+struct Half16<__bf16> {
+  typedef bf16x8 vec8;
+  static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct Half16<_Float16> {
+  typedef f16x8 vec8;
+  static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+constexpr int kBM      = 256;
+constexpr int kBN      = 256;
+constexpr int kBK      = 64;
+constexpr int kThreads = 256;
+// one operand tile: 256 rows x 64 halves = 256 x 128 bytes
+constexpr int kTileBytes  = kBM * kBK * 2;
+constexpr int kStageBytes = 2 * kTileBytes;  // A tile + B tile
+
+// byte offset of 16-byte chunk `chunk` (0..7) of row `row` inside an operand tile
+__device__ __forceinline__ int TileOffset(int row, int chunk) {
+  int key = (row ^ (row >> 3)) & 7;
+  return row * 128 + ((chunk ^ key) << 4);
+}
+
+// 8x8 transpose of 16-bit values held as 8 rows of 4 dwords: out[c] = column c of in
+__device__ __forceinline__ void Transpose8x8(const u32x4 (&in)[8], u32x4 (&out)[8]) {
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+    const int d  = c >> 1;  // dword that holds column c
+    const bool hi = c & 1;  // upper half of that dword
+#pragma unroll
+    for (int rp = 0; rp < 4; ++rp) {
+      unsigned a = in[2 * rp][d];
+      unsigned b = in[2 * rp + 1][d];
+      // low half from row 2rp, high half from row 2rp+1
+      out[c][rp] = hi ? __builtin_amdgcn_perm(b, a, 0x07060302u) : __builtin_amdgcn_perm(b, a, 0x05040100u);
+    }
+  }
+}
+
+// Global -> register staging of one 256-row operand tile, two access patterns.
+// K_CONTIG: the operand is [rows][K] in memory (K contiguous): thread t copies chunk (t & 7) of rows
+//           (t >> 3) + 32 i.  Otherwise the operand is [K][rows] (rows contiguous): thread t owns the 8x8
+//           block at k-block (t >> 5), row-block (t & 31) and transposes it.
+template <bool K_CONTIG>
+struct TileLoader {
+  u32x4 regs[8];
+  __device__ __forceinline__ void Load(const uint16_t* __restrict__ base, int64_t ld, int row0, int k0, int tid) {
+    if (K_CONTIG) {
+      const uint16_t* p = base + (int64_t)(row0 + (tid >> 3)) * ld + k0 + (tid & 7) * 8;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) regs[i] = *reinterpret_cast<const u32x4*>(p + (int64_t)(32 * i) * ld);
+    } else {
+      const uint16_t* p = base + (int64_t)(k0 + (tid >> 5) * 8) * ld + row0 + (tid & 31) * 8;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) regs[r] = *reinterpret_cast<const u32x4*>(p + (int64_t)r * ld);
+    }
+  }
+  __device__ __forceinline__ void Store(char* tile, int tid) {
+    if (K_CONTIG) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        *reinterpret_cast<u32x4*>(tile + TileOffset((tid >> 3) + 32 * i, tid & 7)) = regs[i];
+    } else {
+      u32x4 t[8];
+      Transpose8x8(regs, t);
+#pragma unroll
+      for (int c = 0; c < 8; ++c) *reinterpret_cast<u32x4*>(tile + TileOffset((tid & 31) * 8 + c, tid >> 5)) = t[c];
+    }
+  }
+};
+
+// A_KC: A is stored [M][K] (not transposed).  B_KC: B is stored [N][K] (transposed).
+template <typename T, bool A_KC, bool B_KC>
+__global__ void __launch_bounds__(kThreads)
+gemm16_mfma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ C, int M, int N,
+                   int K, int64_t lda, int64_t ldb, int64_t ldc, float alpha, float beta, int64_t stride_a,
+                   int64_t stride_b, int64_t stride_c) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  typedef typename Half16<T>::vec8 vec8;
+
+  const int tid  = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm   = wave >> 1;  // wavefront row in the 2x2 grid
+  const int wn   = wave & 1;
+
+  // XCD-aware tile order: consecutive workgroup ids go to different XCDs (8 of them, each with its own L2), so
+  // give every XCD a contiguous band of tiles that share A row panels
+  const int tiles_n = N / kBN;
+  const int tiles   = (M / kBM) * tiles_n;
+  int bid           = blockIdx.x;
+  if ((tiles & 7) == 0) bid = (bid & 7) * (tiles >> 3) + (bid >> 3);
+  const int m0 = (bid / tiles_n) * kBM;
+  const int n0 = (bid % tiles_n) * kBN;
+
+  A += (int64_t)blockIdx.y * stride_a;
+  B += (int64_t)blockIdx.y * stride_b;
+  C += (int64_t)blockIdx.y * stride_c;
+
+  f32x16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  TileLoader<A_KC> la;
+  TileLoader<B_KC> lb;
+  const int kt_count = K / kBK;
+
+  la.Load(A, lda, m0, 0, tid);
+  lb.Load(B, ldb, n0, 0, tid);
+  la.Store(lds, tid);
+  lb.Store(lds + kTileBytes, tid);
+  __syncthreads();
+
+  const int frag_row = lane & 31;
+  const int frag_kg  = lane >> 5;
+
+  for (int kt = 0; kt < kt_count; ++kt) {
+    char* cur = lds + (kt & 1) * kStageBytes;
+    char* nxt = lds + ((kt + 1) & 1) * kStageBytes;
+    const bool more = kt + 1 < kt_count;
+    if (more) {
+      la.Load(A, lda, m0, (kt + 1) * kBK, tid);
+      lb.Load(B, ldb, n0, (kt + 1) * kBK, tid);
+    }
+    const char* a_tile = cur;
+    const char* b_tile = cur + kTileBytes;
+#pragma unroll
+    for (int kk = 0; kk < kBK / 16; ++kk) {
+      vec8 af[4], bf[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        af[t] = *reinterpret_cast<const vec8*>(a_tile + TileOffset(wm * 128 + t * 32 + frag_row, kk * 2 + frag_kg));
+        bf[t] = *reinterpret_cast<const vec8*>(b_tile + TileOffset(wn * 128 + t * 32 + frag_row, kk * 2 + frag_kg));
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = Half16<T>::mfma(af[i], bf[j], acc[i][j]);
+    }
+    if (more) {
+      la.Store(nxt, tid);
+      lb.Store(nxt + kTileBytes, tid);
+    }
+    __syncthreads();
+  }
+
+  // epilogue: accumulator element r of lane l sits at row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its tile
+  T* Ct = reinterpret_cast<T*>(C);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int col = n0 + wn * 128 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + wm * 128 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        T* dst  = Ct + (int64_t)row * ldc + col;
+        float v = alpha * acc[i][j][r];
+        if (beta != 0.0f) v += beta * (float)*dst;
+        *dst = (T)v;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// fp32 on v_mfma_f32_32x32x2f32: 128x128 tile, K step 16, 4 wavefronts each 64x64 (2x2 MFMA tiles).
+// LDS holds A as [k][m] and B as [k][n] (row stride 128 floats) so that a fragment read is one
+// conflict-free ds_read_b32 per lane.
+// ---------------------------------------------------------------------------------------------------
+constexpr int kF32Tile = 128;
+constexpr int kF32K    = 16;
+
+template <bool TRANS_A, bool TRANS_B>
+__global__ void __launch_bounds__(256)
+gemm32_mfma_kernel(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C, int M, int N, int K,
+                   int64_t lda, int64_t ldb, int64_t ldc, float alpha, float beta, int64_t stride_a, int64_t stride_b,
+                   int64_t stride_c) {
+  __shared__ float As[2][kF32K][kF32Tile + 4];
+  __shared__ float Bs[2][kF32K][kF32Tile + 4];
+  const int tid  = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.y * kF32Tile;
+  const int n0 = blockIdx.x * kF32Tile;
+  A += (int64_t)blockIdx.z * stride_a;
+  B += (int64_t)blockIdx.z * stride_b;
+  C += (int64_t)blockIdx.z * stride_c;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  // each thread stages 8 floats of A and 8 of B per K step (128 x 16 = 2048 per operand)
+  float ra[8], rb[8];
+  auto load_tiles = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int e = tid + 256 * i;
+      if (TRANS_A) {  // A stored [K][M]: m contiguous
+        int k = e >> 7, m = e & 127;
+        ra[i] = A[(int64_t)(k0 + k) * lda + m0 + m];
+      } else {  // A stored [M][K]: k contiguous
+        int m = e >> 4, k = e & 15;
+        ra[i] = A[(int64_t)(m0 + m) * lda + k0 + k];
+      }
+      if (TRANS_B) {  // B stored [N][K]
+        int n = e >> 4, k = e & 15;
+        rb[i] = B[(int64_t)(n0 + n) * ldb + k0 + k];
+      } else {  // B stored [K][N]
+        int k = e >> 7, n = e & 127;
+        rb[i] = B[(int64_t)(k0 + k) * ldb + n0 + n];
+      }
+    }
+  };
+  auto store_tiles = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int e = tid + 256 * i;
+      if (TRANS_A) {
+        As[buf][e >> 7][e & 127] = ra[i];
+      } else {
+        As[buf][e & 15][e >> 4] = ra[i];
+      }
+      if (TRANS_B) {
+        Bs[buf][e & 15][e >> 4] = rb[i];
+      } else {
+        Bs[buf][e >> 7][e & 127] = rb[i];
+      }
+    }
+  };
+
+  const int kt_count = K / kF32K;
+  load_tiles(0);
+  store_tiles(0);
+  __syncthreads();
+  for (int kt = 0; kt < kt_count; ++kt) {
+    const int cur  = kt & 1;
+    const bool more = kt + 1 < kt_count;
+    if (more) load_tiles((kt + 1) * kF32K);
+#pragma unroll
+    for (int kk = 0; kk < kF32K; kk += 2) {
+      const int k = kk + (lane >> 5);
+      float af[2], bf[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        af[t] = As[cur][k][wm * 64 + t * 32 + (lane & 31)];
+        bf[t] = Bs[cur][k][wn * 64 + t * 32 + (lane & 31)];
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
+    }
+    if (more) store_tiles(cur ^ 1);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        float* dst = C + (int64_t)row * ldc + col;
+        float v    = alpha * acc[i][j][r];
+        if (beta != 0.0f) v += beta * *dst;
+        *dst = v;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Generic kernel: any M, N, K, transposes and element type; accumulates in ACC (float, or double for fp64).
+// 64x64 tile, K step 16, 256 threads each computing a 4x4 micro tile.
+// ---------------------------------------------------------------------------------------------------
+template <typename T, typename ACC>
+__global__ void __launch_bounds__(256)
+gemm_generic_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int M, int N, int K, int64_t lda,
+                    int64_t ldb, int64_t ldc, bool trans_a, bool trans_b, float alpha, float beta, int64_t stride_a,
+                    int64_t stride_b, int64_t stride_c) {
+  __shared__ ACC As[16][64 + 1];
+  __shared__ ACC Bs[16][64 + 1];
+  const int tid = threadIdx.x;
+  const int tx = tid & 15, ty = tid >> 4;
+  const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  A += (int64_t)blockIdx.z * stride_a;
+  B += (int64_t)blockIdx.z * stride_b;
+  C += (int64_t)blockIdx.z * stride_c;
+  ACC acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = (ACC)0;
+  for (int k0 = 0; k0 < K; k0 += 16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int e = tid + 256 * i;  // 0..1023 = 16 x 64
+      int k = e >> 6, r = e & 63;
+      ACC av = (ACC)0, bv = (ACC)0;
+      if (k0 + k < K) {
+        if (m0 + r < M) av = (ACC)(trans_a ? A[(int64_t)(k0 + k) * lda + m0 + r] : A[(int64_t)(m0 + r) * lda + k0 + k]);
+        if (n0 + r < N) bv = (ACC)(trans_b ? B[(int64_t)(n0 + r) * ldb + k0 + k] : B[(int64_t)(k0 + k) * ldb + n0 + r]);
+      }
+      As[k][r] = av;
+      Bs[k][r] = bv;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      ACC a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        a[i] = As[k][ty * 4 + i];
+        b[i] = Bs[k][tx * 4 + i];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] += a[i] * b[j];
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int row = m0 + ty * 4 + i;
+    if (row >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int col = n0 + tx * 4 + j;
+      if (col >= N) continue;
+      T* dst = C + (int64_t)row * ldc + col;
+      ACC v  = (ACC)alpha * acc[i][j];
+      if (beta != 0.0f) v += (ACC)beta * (ACC)*dst;
+      *dst = (T)v;
+    }
+  }
+}
+
+enum class GemmType { kF16, kBF16, kF32, kF64 };
+
+struct GemmProblem {
+  GemmType type;
+  const void* a;
+  const void* b;
+  void* c;
+  int m, n, k;
+  bool trans_a, trans_b;  // op(A) is [m,k]: A stored [k,m] when trans_a; op(B) is [k,n]: B stored [n,k] when trans_b
+  float alpha, beta;
+  int batch;
+  int64_t stride_a, stride_b, stride_c;  // in elements; 0 broadcasts the operand over the batch
+};
+
+template <typename T, bool A_KC, bool B_KC>
+void LaunchFast16(const GemmProblem& p, hipStream_t stream) {
+  auto kernel = gemm16_mfma_kernel<T, A_KC, B_KC>;
+  static bool configured = false;  // per instantiation
+  if (!configured) {
+    CINN_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      2 * kStageBytes));
+    configured = true;
+  }
+  int64_t lda = p.trans_a ? p.m : p.k;
+  int64_t ldb = p.trans_b ? p.k : p.n;
+  dim3 grid((p.m / kBM) * (p.n / kBN), p.batch, 1);
+  hipLaunchKernelGGL(kernel, grid, dim3(kThreads), 2 * kStageBytes, stream, static_cast<const uint16_t*>(p.a),
+                     static_cast<const uint16_t*>(p.b), static_cast<uint16_t*>(p.c), p.m, p.n, p.k, lda, ldb,
+                     (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c);
+}
+
+template <typename T>
+void DispatchFast16(const GemmProblem& p, hipStream_t stream) {
+  bool a_kc = !p.trans_a, b_kc = p.trans_b;
+  if (a_kc && b_kc) LaunchFast16<T, true, true>(p, stream);
+  if (a_kc && !b_kc) LaunchFast16<T, true, false>(p, stream);
+  if (!a_kc && b_kc) LaunchFast16<T, false, true>(p, stream);
+  if (!a_kc && !b_kc) LaunchFast16<T, false, false>(p, stream);
+}
+
+template <typename T, typename ACC>
+void LaunchGeneric(const GemmProblem& p, hipStream_t stream) {
+  int64_t lda = p.trans_a ? p.m : p.k;
+  int64_t ldb = p.trans_b ? p.k : p.n;
+  dim3 grid((p.n + 63) / 64, (p.m + 63) / 64, p.batch);
+  hipLaunchKernelGGL((gemm_generic_kernel<T, ACC>), grid, dim3(256), 0, stream, static_cast<const T*>(p.a),
+                     static_cast<const T*>(p.b), static_cast<T*>(p.c), p.m, p.n, p.k, lda, ldb, (int64_t)p.n, p.trans_a,
+                     p.trans_b, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c);
+}
+
+void LaunchFast32(const GemmProblem& p, hipStream_t stream) {
+  int64_t lda = p.trans_a ? p.m : p.k;
+  int64_t ldb = p.trans_b ? p.k : p.n;
+  dim3 grid(p.n / kF32Tile, p.m / kF32Tile, p.batch);
+  const float* a = static_cast<const float*>(p.a);
+  const float* b = static_cast<const float*>(p.b);
+  float* c       = static_cast<float*>(p.c);
+#define CINN_LAUNCH_F32(TA, TB)                                                                                       \
+  hipLaunchKernelGGL((gemm32_mfma_kernel<TA, TB>), grid, dim3(256), 0, stream, a, b, c, p.m, p.n, p.k, lda, ldb,       \
+                     (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c)
+  if (!p.trans_a && !p.trans_b) CINN_LAUNCH_F32(false, false);
+  if (!p.trans_a && p.trans_b) CINN_LAUNCH_F32(false, true);
+  if (p.trans_a && !p.trans_b) CINN_LAUNCH_F32(true, false);
+  if (p.trans_a && p.trans_b) CINN_LAUNCH_F32(true, true);
+#undef CINN_LAUNCH_F32
+}
+
+bool ForceGeneric() {
+  static const bool force = getenv("FLAGS_cinn_hip_gemm_generic") && atoi(getenv("FLAGS_cinn_hip_gemm_generic")) != 0;
+  return force;
+}
+
+void RunGemm(const GemmProblem& p, hipStream_t stream) {
+  CINN_RT_CHECK(p.m > 0 && p.n > 0 && p.k > 0 && p.batch > 0, "gemm: dimensions must be positive, got m=%d n=%d k=%d batch=%d",
+                p.m, p.n, p.k, p.batch);
+  CINN_RT_CHECK(p.a && p.b && p.c, "gemm: null operand");
+  CINN_RT_CHECK(p.batch <= 65535, "gemm: batch %d exceeds the grid limit", p.batch);
+  const bool fast16 = !ForceGeneric() && p.m % kBM == 0 && p.n % kBN == 0 && p.k % kBK == 0;
+  const bool fast32 = !ForceGeneric() && p.m % kF32Tile == 0 && p.n % kF32Tile == 0 && p.k % kF32K == 0;
+  switch (p.type) {
+    case GemmType::kBF16:
+      if (fast16) {
+        DispatchFast16<__bf16>(p, stream);
+      } else {
+        LaunchGeneric<__bf16, float>(p, stream);
+      }
+      break;
+    case GemmType::kF16:
+      if (fast16) {
+        DispatchFast16<_Float16>(p, stream);
+      } else {
+        LaunchGeneric<_Float16, float>(p, stream);
+      }
+      break;
+    case GemmType::kF32:
+      if (fast32) {
+        LaunchFast32(p, stream);
+      } else {
+        LaunchGeneric<float, float>(p, stream);
+      }
+      break;
+    case GemmType::kF64: LaunchGeneric<double, double>(p, stream); break;
+  }
+  CINN_HIP_CALL(hipGetLastError());
+}
+
+GemmType TypeOf(const cinn_buffer_t* buf) {
+  int bytes = buf->type.bits / CHAR_BIT;
+  if (buf->type.code == cinn_type_float && bytes == 2) return GemmType::kF16;
+  if (buf->type.code == cinn_type_float && bytes == 4) return GemmType::kF32;
+  if (buf->type.code == cinn_type_float && bytes == 8) return GemmType::kF64;
+  if (buf->type.code == cinn_type_bfloat) return GemmType::kBF16;
+  fprintf(stderr, "unsupported gemm data type: code %d, bits %d\n", buf->type.code, buf->type.bits);
+  abort();
+}
+
+cinn_buffer_t* BufferArg(void* v_args, int index) {
+  auto* args = static_cast<cinn_pod_value_t*>(v_args);
+  CINN_RT_CHECK(args[index].type_code_ == CINN_POD_BUFFER_P, "gemm: argument %d is not a buffer", index);
+  return static_cast<cinn_buffer_t*>(args[index].value_.v_handle);
+}
+
+}  // namespace
+
+extern "C" {
+
+// Shape algebra of cinn_call_cublas (cinn/runtime/cuda/cuda_util.cc:121-310) restated for a row-major kernel:
+// the result is [a1', a2', M, N] with M = trans_a ? a4 : a3, K = trans_a ? a3 : a4, N = trans_b ? b3 : b4;
+// trans_o stores the transposed product, which is the product of the swapped, re-transposed operands.
+// Leading dimensions broadcast: an operand whose leading dims are 1 is shared by every batch.
+void cinn_call_cublas(void* v_args, int num_args, bool trans_a, bool trans_b, bool trans_o, float alpha, float beta,
+                      int a1, int a2, int a3, int a4, int b1, int b2, int b3, int b4, void* stream) {
+  CINN_RT_CHECK(num_args == 3, "cinn_call_cublas takes A, B and C, got %d arguments", num_args);
+  cinn_buffer_t* A = BufferArg(v_args, 0);
+  cinn_buffer_t* B = BufferArg(v_args, 1);
+  cinn_buffer_t* C = BufferArg(v_args, 2);
+  const int m = trans_a ? a4 : a3;
+  const int k = trans_a ? a3 : a4;
+  const int n = trans_b ? b3 : b4;
+  CINN_RT_CHECK(k == (trans_b ? b4 : b3), "cinn_call_cublas: inner dimensions differ (%d vs %d)", k, trans_b ? b4 : b3);
+  CINN_RT_CHECK((a1 == b1 || a1 == 1 || b1 == 1) && (a2 == b2 || a2 == 1 || b2 == 1),
+                "cinn_call_cublas: batch dims [%d,%d] and [%d,%d] do not broadcast", a1, a2, b1, b2);
+  const int o1 = a1 > b1 ? a1 : b1, o2 = a2 > b2 ? a2 : b2;
+
+  GemmProblem p;
+  p.type  = TypeOf(A);
+  p.alpha = alpha;
+  p.beta  = beta;
+  // one launch per leading index o1; the second batch dim goes to the grid
+  const int64_t a_mat = (int64_t)a3 * a4, b_mat = (int64_t)b3 * b4, c_mat = (int64_t)m * n;
+  const int elem = A->type.bits / CHAR_BIT;
+  for (int i1 = 0; i1 < o1; ++i1) {
+    const char* a_base = reinterpret_cast<const char*>(A->memory) + (a1 == 1 ? 0 : (int64_t)i1 * a2 * a_mat) * elem;
+    const char* b_base = reinterpret_cast<const char*>(B->memory) + (b1 == 1 ? 0 : (int64_t)i1 * b2 * b_mat) * elem;
+    char* c_base       = reinterpret_cast<char*>(C->memory) + (int64_t)i1 * o2 * c_mat * elem;
+    const int64_t sa = a2 == 1 ? 0 : a_mat, sb = b2 == 1 ? 0 : b_mat;
+    if (!trans_o) {
+      p.a = a_base, p.b = b_base, p.c = c_base;
+      p.m = m, p.n = n, p.k = k;
+      p.trans_a = trans_a, p.trans_b = trans_b;
+      p.stride_a = sa, p.stride_b = sb;
+    } else {
+      // C^T[n, m] = op(B)^T[n, k] * op(A)^T[k, m]
+      p.a = b_base, p.b = a_base, p.c = c_base;
+      p.m = n, p.n = m, p.k = k;
+      p.trans_a = !trans_b, p.trans_b = !trans_a;
+      p.stride_a = sb, p.stride_b = sa;
+    }
+    p.batch    = o2;
+    p.stride_c = c_mat;
+    RunGemm(p, static_cast<hipStream_t>(stream));
+  }
+}
+
+// cinn_call_batched_cublas (cuda_util.cc:312-437): v_args = {shared operand, others..., outputs...}; every
+// (other_i, output_i) pair is one cinn_call_cublas-shaped problem with the shared operand on side `opside`.
+void cinn_call_batched_cublas(void* v_args, int num_args, int opside, bool trans_a, bool trans_b, bool trans_o,
+                              float alpha, float beta, int a1, int a2, int a3, int a4, int b1, int b2, int b3, int b4,
+                              void* stream) {
+  CINN_RT_CHECK(num_args >= 3 && (num_args - 1) % 2 == 0, "cinn_call_batched_cublas: %d arguments", num_args);
+  const int pairs = (num_args - 1) / 2;
+  auto* args      = static_cast<cinn_pod_value_t*>(v_args);
+  for (int i = 0; i < pairs; ++i) {
+    cinn_pod_value_t triple[3];
+    triple[opside == 0 ? 0 : 1] = args[0];
+    triple[opside == 0 ? 1 : 0] = args[1 + i];
+    triple[2]                   = args[1 + pairs + i];
+    cinn_call_cublas(triple, 3, trans_a, trans_b, trans_o, alpha, beta, a1, a2, a3, a4, b1, b2, b3, b4, stream);
+  }
+}
+
+}  // extern "C"

@@ -1,0 +1,190 @@
+"""GPU parity of the MFMA GEMM behind cinn_call_cublas (BASELINE config 3), called through the C-ABI exactly as
+a host stub calls it (cinn_pod_value_t[3] of cinn_buffer_t, shapes padded to 4-D), and through NetBuilder.matmul.
+Bars: fp32 vs the oracle's ascending-k fp32 sum within 1e-5 relative of the row scale (checked against a float64
+product), 16-bit inputs with fp32 accumulation within 1e-2."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import oracle
+from cinn_amd import _lib, runtime
+from cinn_amd.common import BFloat16, Float, bfloat16_bits_to_float32, float32_to_bfloat16_bits
+from cinn_amd.frontend import NetBuilder
+
+from helpers import run
+from test_golden import load
+
+pytestmark = pytest.mark.gpu
+
+
+def call_cublas(a, b, c_shape, dtype, trans_a=False, trans_b=False, trans_o=False, alpha=1.0, beta=0.0, c_init=None,
+                a_dims=None, b_dims=None):
+    lib = _lib.load()
+    lib.cinn_call_cublas.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_bool, ctypes.c_bool, ctypes.c_bool,
+                                     ctypes.c_float, ctypes.c_float] + [ctypes.c_int] * 8 + [ctypes.c_void_p]
+    A = runtime.DeviceBuffer.from_numpy(a, dtype)
+    B = runtime.DeviceBuffer.from_numpy(b, dtype)
+    C = runtime.DeviceBuffer(c_shape, dtype)
+    if c_init is not None:
+        C.copy_from(c_init)
+    else:
+        C.copy_from(np.zeros(c_shape, C.np_dtype))
+    a4 = a_dims or ([1] * (4 - a.ndim) + list(a.shape))
+    b4 = b_dims or ([1] * (4 - b.ndim) + list(b.shape))
+    args = runtime.pod_args([A, B, C])
+    lib.cinn_call_cublas(args, 3, trans_a, trans_b, trans_o, alpha, beta, *a4, *b4, None)
+    runtime.synchronize()
+    return C.numpy()
+
+
+def check_fp32(got, a64, b64, k):
+    want = a64 @ b64
+    scale = np.abs(a64) @ np.abs(b64)  # error of a k-term fp32 sum is relative to the sum of magnitudes
+    assert np.all(np.abs(got - want) <= 1e-5 * scale + 1e-30), np.abs(got - want).max()
+
+
+@pytest.mark.parametrize("m,n,k", [(128, 128, 16), (256, 384, 64), (1024, 1024, 1024)])
+def test_fp32_mfma_path(gpu, m, n, k):
+    rng = np.random.default_rng(m + n + k)
+    a = (rng.standard_normal((m, k)) * 0.02).astype(np.float32)
+    b = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+    got = call_cublas(a, b, (m, n), "float32")
+    check_fp32(got, a.astype(np.float64), b.astype(np.float64), k)
+    if m <= 256:
+        np.testing.assert_allclose(got, oracle.matmul(a, b), rtol=1e-4, atol=1e-7)
+
+
+def test_fp32_test02_pattern(gpu):
+    # tests/test02_matmul_case.cc: 1024^3, tolerance 1e-4 absolute
+    a = np.ones((1024, 1024), np.float32)
+    b = np.full((1024, 1024), 2.0, np.float32)
+    got = call_cublas(a, b, (1024, 1024), "float32")
+    assert np.abs(got - 2048.0).max() < 1e-4
+
+
+@pytest.mark.parametrize("ta,tb,to", [(False, False, False), (True, False, False), (False, True, False),
+                                      (True, True, False), (False, False, True), (True, True, True)])
+@pytest.mark.parametrize("shape", [(128, 256, 64), (37, 29, 53)])
+def test_fp32_transposes_alpha_beta(gpu, ta, tb, to, shape):
+    m, n, k = shape
+    rng = np.random.default_rng(17)
+    a = rng.standard_normal((k, m) if ta else (m, k)).astype(np.float32)
+    b = rng.standard_normal((n, k) if tb else (k, n)).astype(np.float32)
+    c0 = rng.standard_normal((n, m) if to else (m, n)).astype(np.float32)
+    got = call_cublas(a, b, c0.shape, "float32", ta, tb, to, alpha=0.5, beta=2.0, c_init=c0)
+    a64 = (a.T if ta else a).astype(np.float64)
+    b64 = (b.T if tb else b).astype(np.float64)
+    prod = a64 @ b64
+    want = 0.5 * (prod.T if to else prod) + 2.0 * c0
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("kind", ["float16", "bfloat16"])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_16bit_mfma_path_all_layouts(gpu, kind, ta, tb):
+    m, n, k = 256, 512, 192
+    rng = np.random.default_rng(29)
+    a = (rng.standard_normal((k, m) if ta else (m, k)) * 0.02).astype(np.float32)
+    b = (rng.standard_normal((n, k) if tb else (k, n)) * 0.02).astype(np.float32)
+    if kind == "float16":
+        ab, bb = a.astype(np.float16), b.astype(np.float16)
+        af, bf = ab.astype(np.float64), bb.astype(np.float64)
+        got = call_cublas(ab, bb, (m, n), kind, ta, tb).astype(np.float64)
+        want = oracle.half_to_float(oracle.matmul(ab.view(np.uint16), bb.view(np.uint16), ta, tb, kind=kind))
+    else:
+        ab, bb = float32_to_bfloat16_bits(a), float32_to_bfloat16_bits(b)
+        af, bf = bfloat16_bits_to_float32(ab).astype(np.float64), bfloat16_bits_to_float32(bb).astype(np.float64)
+        got = bfloat16_bits_to_float32(call_cublas(ab, bb, (m, n), kind, ta, tb)).astype(np.float64)
+        want = oracle.bf16_to_float(oracle.matmul(ab, bb, ta, tb, kind=kind))
+    exact = (af.T if ta else af) @ (bf.T if tb else bf)
+    scale = np.abs(af.T if ta else af) @ np.abs(bf.T if tb else bf)
+    # fp32 accumulation then one rounding: within 1e-2 of the exact product relative to its magnitude scale
+    assert np.all(np.abs(got - exact) <= 1e-2 * np.maximum(np.abs(exact), 1e-3 * scale))
+    # and within one ulp of the oracle (same contract, different summation order)
+    ulp = 2.0 ** -7 if kind == "bfloat16" else 2.0 ** -10
+    # (+ one fp16 subnormal quantum for outputs below 2^-14)
+    assert np.all(np.abs(got - want) <= ulp * np.maximum(np.abs(want), 1e-3 * scale) + 2.0 ** -24)
+
+
+@pytest.mark.parametrize("kind", ["float16", "bfloat16"])
+def test_config3_4096_cubed(gpu, kind):
+    rng = np.random.default_rng(31)
+    n = 4096
+    a = (rng.standard_normal((n, n)) * 0.02).astype(np.float32)
+    b = (rng.standard_normal((n, n)) * 0.02).astype(np.float32)
+    if kind == "float16":
+        ab, bb = a.astype(np.float16), b.astype(np.float16)
+        got = call_cublas(ab, bb, (n, n), kind).astype(np.float32)
+        af, bf = ab.astype(np.float32), bb.astype(np.float32)
+    else:
+        ab, bb = float32_to_bfloat16_bits(a), float32_to_bfloat16_bits(b)
+        got = bfloat16_bits_to_float32(call_cublas(ab, bb, (n, n), kind))
+        af, bf = bfloat16_bits_to_float32(ab), bfloat16_bits_to_float32(bb)
+    # size-independent checks at full size: (1) a sample of rows against a float64 product,
+    rows = rng.choice(n, 32, replace=False)
+    exact = af[rows].astype(np.float64) @ bf.astype(np.float64)
+    scale = np.abs(af[rows]).astype(np.float64) @ np.abs(bf).astype(np.float64)
+    assert np.all(np.abs(got[rows] - exact) <= 1e-2 * np.maximum(np.abs(exact), 1e-3 * scale))
+    # (2) linearity: (A B) v == A (B v) for a random vector, which touches every output element
+    v = rng.standard_normal(n)
+    lhs = got.astype(np.float64) @ v
+    rhs = af.astype(np.float64) @ (bf.astype(np.float64) @ v)
+    assert np.abs(lhs - rhs).max() <= 1e-2 * np.abs(rhs).max()
+
+
+def test_batched_and_broadcast_leading_dims(gpu):
+    rng = np.random.default_rng(37)
+    a = rng.standard_normal((2, 3, 40, 24)).astype(np.float32)
+    b = rng.standard_normal((1, 1, 24, 16)).astype(np.float32)
+    got = call_cublas(a, b, (2, 3, 40, 16), "float32")
+    np.testing.assert_allclose(got, a.astype(np.float64) @ b.astype(np.float64), rtol=1e-4, atol=1e-4)
+    b2 = rng.standard_normal((2, 3, 24, 16)).astype(np.float32)
+    got = call_cublas(a, b2, (2, 3, 40, 16), "float32")
+    np.testing.assert_allclose(got, a.astype(np.float64) @ b2.astype(np.float64), rtol=1e-4, atol=1e-4)
+    b3 = rng.standard_normal((1, 3, 24, 16)).astype(np.float32)
+    got = call_cublas(a, b3, (2, 3, 40, 16), "float32")
+    np.testing.assert_allclose(got, a.astype(np.float64) @ b3.astype(np.float64), rtol=1e-4, atol=1e-4)
+
+
+def test_fp64_generic_path(gpu):
+    rng = np.random.default_rng(41)
+    a, b = rng.standard_normal((33, 47)), rng.standard_normal((47, 21))
+    np.testing.assert_allclose(call_cublas(a, b, (33, 21), "float64"), a @ b, rtol=1e-12, atol=1e-12)
+
+
+def test_golden_fixtures_through_netbuilder(gpu):
+    f = load("cfg3_matmul_f32")
+    b = NetBuilder("mm")
+    A, B = b.create_input(Float(32), f["a"].shape, "a"), b.create_input(Float(32), f["b"].shape, "b")
+    (c,), comp = run(b, {A: f["a"], B: f["b"]}, [b.matmul(A, B)])
+    np.testing.assert_allclose(c, f["c"], rtol=1e-4, atol=1e-7)
+    assert comp.instruction_info(0)[0].startswith("fn_mm_matmul")
+    b = NetBuilder("mmt")
+    A, B = b.create_input(Float(32), f["a"].T.shape, "a"), b.create_input(Float(32), f["b"].T.shape, "b")
+    (c,), _ = run(b, {A: f["a"].T.copy(), B: f["b"].T.copy()}, [b.matmul(A, B, trans_x=True, trans_y=True)])
+    np.testing.assert_allclose(c, f["c_tt"], rtol=1e-4, atol=1e-7)
+    f = load("cfg3_matmul_bf16")
+    b = NetBuilder("mmb")
+    A, B = b.create_input(BFloat16(), f["a"].shape, "a"), b.create_input(BFloat16(), f["b"].shape, "b")
+    (c,), _ = run(b, {A: f["a"], B: f["b"]}, [b.matmul(A, B)])
+    np.testing.assert_allclose(bfloat16_bits_to_float32(c), oracle.bf16_to_float(f["c"]), rtol=1e-2, atol=1e-6)
+    f = load("cfg3_matmul_f16")
+    b = NetBuilder("mmh")
+    A, B = b.create_input(Float(16), f["a"].shape, "a"), b.create_input(Float(16), f["b"].shape, "b")
+    (c,), _ = run(b, {A: f["a"].view(np.float16), B: f["b"].view(np.float16)}, [b.matmul(A, B)])
+    np.testing.assert_allclose(c.astype(np.float32), oracle.half_to_float(f["c"]), rtol=1e-2, atol=1e-6)
+
+
+def test_matmul_fused_with_neighbours(gpu):
+    rng = np.random.default_rng(43)
+    x = rng.standard_normal((64, 128)).astype(np.float32)
+    w = rng.standard_normal((128, 32)).astype(np.float32)
+    bias = rng.standard_normal(32).astype(np.float32)
+    b = NetBuilder("fc")
+    X, W, Bi = b.create_input(Float(32), x.shape, "x"), b.create_input(Float(32), w.shape, "w"), b.create_input(
+        Float(32), [32], "bias")
+    out = b.relu(b.add(b.mul(X, W), Bi))
+    (y,), comp = run(b, {X: x, W: w, Bi: bias}, [out])
+    np.testing.assert_allclose(y, np.maximum(x.astype(np.float64) @ w + bias, 0), rtol=1e-4, atol=1e-4)
+    assert comp.num_instructions() == 2
