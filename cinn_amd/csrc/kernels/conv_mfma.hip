@@ -1,0 +1,357 @@
+// Hand-written CDNA4 (gfx950) convolution behind cinn_call_cudnn_conv2d_forward and its fused
+// batch_norm / relu variant: NCHW cross-correlation with zero padding as an implicit GEMM on MFMA,
+//
+//   out[n, f, y, x] = sum_{c, ry, rx} in[n, c, y*s + ry*d - p, x*s + rx*d - p] * w[f, c, ry, rx]
+//
+// GEMM view per group: M = output channels, N = n * oh * ow output pixels (flattened over the batch so that
+// small images still fill a tile), K = (c / groups) * kh * kw.  The weight matrix is [M][K] as stored.  The
+// im2col matrix is never materialised: every thread owns one output pixel of the tile, and a small
+// per-shape table (one entry per k: input offset, dy, dx) replaces the div / mod of decoding k into
+// (c, ry, rx), so a gathered element costs one table read, two range checks and one load.
+//
+// Block tile 128 (channels) x 128 (pixels), 256 threads = 4 wavefronts in a 2x2 grid, each 64x64 = 2x2 MFMA
+// tiles of 32x32.
+//   fp32          : K step 16, v_mfma_f32_32x32x2f32; LDS tiles [k][row] read with conflict-free ds_read_b32.
+//   fp16 / bf16   : K step 32, v_mfma_f32_32x32x16_{f16,bf16} (fp32 accumulation); LDS tiles [row][k] with
+//                   64-byte rows whose 16-byte chunks are XOR-swizzled for conflict-free ds_read_b128.
+// The epilogue applies alpha / beta, or the per-channel affine (+ relu) of an inference batch_norm.
+#include <hip/hip_runtime.h>
+
+#include <climits>
+#include <cstdint>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "cinn_hip_runtime.h"
+#include "runtime/hip_check.h"
+
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+struct KEntry {
+  int offset;   // c * ih * iw + ry * d * iw + rx * d, relative to the input position of the pixel
+  short dy, dx;  // ry * d, rx * d
+};
+
+struct ConvParams {
+  int n, c, ih, iw;        // input
+  int f, kh, kw;           // filter: f output channels, c / groups input channels each
+  int oh, ow;              // output
+  int ph, pw, sh, sw;      // padding, stride (dilation lives in the table)
+  int groups;
+  int k_total;             // (c / groups) * kh * kw
+  int pixels;              // n * oh * ow
+  float alpha, beta;
+  int epilogue;            // 0: alpha / beta, 1: affine, 2: affine + relu
+};
+
+constexpr int kTileM   = 128;
+constexpr int kTileN   = 128;
+constexpr int kThreads = 256;
+
+template <typename T>
+struct ConvTraits;
+template <>
+struct ConvTraits<float> {
+  static constexpr int kStep = 16;
+  static constexpr bool kHalf = false;
+};
+template <>
+struct ConvTraits<_Float16> {
+  static constexpr int kStep = 32;
+  static constexpr bool kHalf = true;
+  typedef f16x8 vec8;
+  static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct ConvTraits<__bf16> {
+  static constexpr int kStep = 32;
+  static constexpr bool kHalf = true;
+  typedef bf16x8 vec8;
+  static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+// 16-bit tiles: rows of 32 elements = 64 bytes = 4 chunks; chunk position = chunk ^ ((row >> 1) & 3)
+__device__ __forceinline__ int HalfTileOffset(int row, int chunk) { return row * 64 + ((chunk ^ ((row >> 1) & 3)) << 4); }
+
+template <typename T>
+__global__ void __launch_bounds__(kThreads)
+conv2d_igemm_kernel(const T* __restrict__ in, const T* __restrict__ w, T* __restrict__ out,
+                    const KEntry* __restrict__ table, const float* __restrict__ scale, const float* __restrict__ shift,
+                    ConvParams p) {
+  constexpr int BK = ConvTraits<T>::kStep;
+  // fp32: A[BK][128 + 4] and B[BK][128 + 4] floats; 16-bit: A[128][32] and B[128][32] halves (8 KiB each)
+  __shared__ __attribute__((aligned(16))) char lds_a[ConvTraits<T>::kHalf ? kTileM * 64 : BK * (kTileM + 4) * 4];
+  __shared__ __attribute__((aligned(16))) char lds_b[ConvTraits<T>::kHalf ? kTileN * 64 : BK * (kTileN + 4) * 4];
+
+  const int tid  = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int group = blockIdx.z;
+  const int fg    = p.f / p.groups;  // output channels per group
+  const int cg    = p.c / p.groups;  // input channels per group
+  const int f0    = blockIdx.y * kTileM;  // within the group
+  const int p0    = blockIdx.x * kTileN;
+  const int ohw   = p.oh * p.ow;
+  const int K     = p.k_total;
+
+  // the output pixel this thread gathers for
+  const int my_pix   = p0 + (tid & 127);
+  const bool pix_ok  = my_pix < p.pixels;
+  int pn = 0, py = 0, px = 0;
+  if (pix_ok) {
+    pn      = my_pix / ohw;
+    int rem = my_pix - pn * ohw;
+    py      = rem / p.ow;
+    px      = rem - py * p.ow;
+  }
+  const int iy0 = py * p.sh - p.ph;
+  const int ix0 = px * p.sw - p.pw;
+  const T* in_pix = in + ((int64_t)pn * p.c + (int64_t)group * cg) * p.ih * p.iw + (int64_t)iy0 * p.iw + ix0;
+  const T* w_grp  = w + (int64_t)group * fg * K;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  auto gather = [&](int k) -> T {
+    if (!pix_ok || k >= K) return (T)0.0f;
+    KEntry e = table[k];
+    int iy = iy0 + e.dy, ix = ix0 + e.dx;
+    if (iy < 0 || iy >= p.ih || ix < 0 || ix >= p.iw) return (T)0.0f;
+    return in_pix[e.offset];
+  };
+
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    if constexpr (!ConvTraits<T>::kHalf) {
+      float(*As)[kTileM + 4] = reinterpret_cast<float(*)[kTileM + 4]>(lds_a);
+      float(*Bs)[kTileN + 4] = reinterpret_cast<float(*)[kTileN + 4]>(lds_b);
+      float ra[8], rb[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        int e = tid + 256 * i;
+        int k = e & 15, f = e >> 4;
+        ra[i] = (f0 + f < fg && k0 + k < K) ? (float)w_grp[(int64_t)(f0 + f) * K + k0 + k] : 0.0f;
+        rb[i] = (float)gather(k0 + (tid >> 7) + 2 * i);
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        int e = tid + 256 * i;
+        As[e & 15][e >> 4]               = ra[i];
+        Bs[(tid >> 7) + 2 * i][tid & 127] = rb[i];
+      }
+      __syncthreads();
+#pragma unroll
+      for (int kk = 0; kk < BK; kk += 2) {
+        const int k = kk + (lane >> 5);
+        float af[2], bf[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          af[t] = As[k][wm * 64 + t * 32 + (lane & 31)];
+          bf[t] = Bs[k][wn * 64 + t * 32 + (lane & 31)];
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
+      }
+      __syncthreads();
+    } else {
+      typedef typename ConvTraits<T>::vec8 vec8;
+      const bool vec_ok = (K & 7) == 0;  // rows of w start 16-byte aligned
+      vec8 ra[2], rb[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        int q = tid + 256 * i;  // weight chunk: row q / 4, chunk q % 4
+        int f = q >> 2, c = q & 3;
+        int k = k0 + c * 8;
+        if (f0 + f < fg && vec_ok && k + 8 <= K) {
+          ra[i] = *reinterpret_cast<const vec8*>(w_grp + (int64_t)(f0 + f) * K + k);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) ra[i][e] = (f0 + f < fg && k + e < K) ? w_grp[(int64_t)(f0 + f) * K + k + e] : (T)0.0f;
+        }
+        int kg = (tid >> 7) + 2 * i;  // gathered chunk: pixel tid % 128, k group kg
+#pragma unroll
+        for (int e = 0; e < 8; ++e) rb[i][e] = gather(k0 + kg * 8 + e);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        int q = tid + 256 * i;
+        *reinterpret_cast<vec8*>(lds_a + HalfTileOffset(q >> 2, q & 3))               = ra[i];
+        *reinterpret_cast<vec8*>(lds_b + HalfTileOffset(tid & 127, (tid >> 7) + 2 * i)) = rb[i];
+      }
+      __syncthreads();
+#pragma unroll
+      for (int kk = 0; kk < BK / 16; ++kk) {
+        vec8 af[2], bf[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          af[t] = *reinterpret_cast<const vec8*>(lds_a + HalfTileOffset(wm * 64 + t * 32 + (lane & 31), kk * 2 + (lane >> 5)));
+          bf[t] = *reinterpret_cast<const vec8*>(lds_b + HalfTileOffset(wn * 64 + t * 32 + (lane & 31), kk * 2 + (lane >> 5)));
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) acc[i][j] = ConvTraits<T>::mfma(af[i], bf[j], acc[i][j]);
+      }
+      __syncthreads();
+    }
+  }
+
+  // epilogue: element r of lane l is channel 8*(r/4) + 4*(l/32) + r%4, pixel l%32 of its 32x32 tile
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int pix = p0 + wn * 64 + j * 32 + (lane & 31);
+    if (pix >= p.pixels) continue;
+    const int n   = pix / ohw;
+    const int rem = pix - n * ohw;
+    T* out_pix    = out + ((int64_t)n * p.f + (int64_t)group * fg) * ohw + rem;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int f = f0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (f >= fg) continue;
+        T* dst  = out_pix + (int64_t)f * ohw;
+        float v = acc[i][j][r];
+        if (p.epilogue == 0) {
+          v *= p.alpha;
+          if (p.beta != 0.0f) v += p.beta * (float)*dst;
+        } else {
+          v = v * scale[group * fg + f] + shift[group * fg + f];
+          if (p.epilogue == 2) v = v > 0.0f ? v : 0.0f;
+        }
+        *dst = (T)v;
+      }
+    }
+  }
+}
+
+// ---- per-shape k table, cached on the device ---------------------------------------------------------
+std::mutex g_table_mu;
+std::map<std::string, KEntry*> g_tables;
+
+const KEntry* GetTable(const ConvParams& p, int dh, int dw) {
+  char key[160];
+  snprintf(key, sizeof(key), "%d,%d,%d,%d,%d,%d,%d,%d", p.c / p.groups, p.ih, p.iw, p.kh, p.kw, dh, dw, p.k_total);
+  std::lock_guard<std::mutex> lock(g_table_mu);
+  auto it = g_tables.find(key);
+  if (it != g_tables.end()) return it->second;
+  std::vector<KEntry> host(p.k_total);
+  int k = 0;
+  for (int c = 0; c < p.c / p.groups; ++c)
+    for (int ry = 0; ry < p.kh; ++ry)
+      for (int rx = 0; rx < p.kw; ++rx) {
+        host[k].offset = (c * p.ih + ry * dh) * p.iw + rx * dw;
+        host[k].dy     = static_cast<short>(ry * dh);
+        host[k].dx     = static_cast<short>(rx * dw);
+        ++k;
+      }
+  KEntry* dev = nullptr;
+  CINN_HIP_CALL(hipMalloc(&dev, sizeof(KEntry) * host.size()));
+  CINN_HIP_CALL(hipMemcpy(dev, host.data(), sizeof(KEntry) * host.size(), hipMemcpyHostToDevice));
+  g_tables[key] = dev;
+  return dev;
+}
+
+cinn_buffer_t* BufferArg(void* v_args, int index) {
+  auto* args = static_cast<cinn_pod_value_t*>(v_args);
+  CINN_RT_CHECK(args[index].type_code_ == CINN_POD_BUFFER_P, "conv2d: argument %d is not a buffer", index);
+  return static_cast<cinn_buffer_t*>(args[index].value_.v_handle);
+}
+
+void RunConv(cinn_buffer_t* x, cinn_buffer_t* w, cinn_buffer_t* y, const float* scale, const float* shift, int epilogue,
+             int format, float alpha, float beta, int in, int ic, int ih, int iw, int fn, int fc, int fh, int fw, int ph,
+             int pw, int sh, int sw, int dh, int dw, int groups, int on, int oc, int oh, int ow, hipStream_t stream) {
+  CINN_RT_CHECK(format == 0, "conv2d: only NCHW (format 0) is implemented, got format %d", format);
+  CINN_RT_CHECK(groups >= 1 && ic % groups == 0 && fn % groups == 0, "conv2d: bad group count %d", groups);
+  CINN_RT_CHECK(fc == ic / groups, "conv2d: filter has %d input channels, expected %d", fc, ic / groups);
+  CINN_RT_CHECK(on == in && oc == fn, "conv2d: output is [%d,%d,..], expected [%d,%d,..]", on, oc, in, fn);
+  CINN_RT_CHECK(sh > 0 && sw > 0 && dh > 0 && dw > 0, "conv2d: strides and dilations must be positive");
+  const int want_oh = (ih - ((fh - 1) * dh + 1) + 2 * ph) / sh + 1;
+  const int want_ow = (iw - ((fw - 1) * dw + 1) + 2 * pw) / sw + 1;
+  CINN_RT_CHECK(oh == want_oh && ow == want_ow, "conv2d: output is %dx%d, the shapes give %dx%d", oh, ow, want_oh, want_ow);
+  CINN_RT_CHECK((int64_t)in * ic * ih * iw < INT_MAX && (int64_t)on * oc * oh * ow < INT_MAX, "conv2d: tensor too large");
+  CINN_RT_CHECK(fh * dh < 32768 && fw * dw < 32768, "conv2d: filter extent too large");
+
+  ConvParams p;
+  p.n = in, p.c = ic, p.ih = ih, p.iw = iw;
+  p.f = fn, p.kh = fh, p.kw = fw;
+  p.oh = oh, p.ow = ow;
+  p.ph = ph, p.pw = pw, p.sh = sh, p.sw = sw;
+  p.groups   = groups;
+  p.k_total  = fc * fh * fw;
+  p.pixels   = in * oh * ow;
+  p.alpha    = alpha;
+  p.beta     = beta;
+  p.epilogue = epilogue;
+  const KEntry* table = GetTable(p, dh, dw);
+
+  dim3 grid((p.pixels + kTileN - 1) / kTileN, (fn / groups + kTileM - 1) / kTileM, groups);
+  CINN_RT_CHECK(grid.y <= 65535 && grid.z <= 65535, "conv2d: grid too large");
+  const int bytes = x->type.bits / CHAR_BIT;
+  if (x->type.code == cinn_type_float && bytes == 4) {
+    hipLaunchKernelGGL(conv2d_igemm_kernel<float>, grid, dim3(kThreads), 0, stream, reinterpret_cast<const float*>(x->memory),
+                       reinterpret_cast<const float*>(w->memory), reinterpret_cast<float*>(y->memory), table, scale, shift, p);
+  } else if (x->type.code == cinn_type_float && bytes == 2) {
+    hipLaunchKernelGGL(conv2d_igemm_kernel<_Float16>, grid, dim3(kThreads), 0, stream,
+                       reinterpret_cast<const _Float16*>(x->memory), reinterpret_cast<const _Float16*>(w->memory),
+                       reinterpret_cast<_Float16*>(y->memory), table, scale, shift, p);
+  } else if (x->type.code == cinn_type_bfloat) {
+    hipLaunchKernelGGL(conv2d_igemm_kernel<__bf16>, grid, dim3(kThreads), 0, stream,
+                       reinterpret_cast<const __bf16*>(x->memory), reinterpret_cast<const __bf16*>(w->memory),
+                       reinterpret_cast<__bf16*>(y->memory), table, scale, shift, p);
+  } else {
+    fprintf(stderr, "conv2d: unsupported data type code %d bits %d\n", x->type.code, x->type.bits);
+    abort();
+  }
+  CINN_HIP_CALL(hipGetLastError());
+}
+
+}  // namespace
+
+extern "C" {
+
+void cinn_call_cudnn_conv2d_forward(void* v_args, int num_args, int format, float alpha, float beta, int input_n,
+                                    int input_c, int input_h, int input_w, int filter_n, int filter_c, int filter_h,
+                                    int filter_w, int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h,
+                                    int dilation_w, int groups, int output_n, int output_c, int output_h,
+                                    int output_w, void* stream) {
+  CINN_RT_CHECK(num_args == 3, "cinn_call_cudnn_conv2d_forward takes x, w and y, got %d arguments", num_args);
+  RunConv(BufferArg(v_args, 0), BufferArg(v_args, 1), BufferArg(v_args, 2), nullptr, nullptr, 0, format, alpha, beta,
+          input_n, input_c, input_h, input_w, filter_n, filter_c, filter_h, filter_w, pad_h, pad_w, stride_h, stride_w,
+          dilation_h, dilation_w, groups, output_n, output_c, output_h, output_w, static_cast<hipStream_t>(stream));
+}
+
+void cinn_call_hip_conv2d_bn_relu(void* v_args, int num_args, int format, int relu, int input_n, int input_c,
+                                  int input_h, int input_w, int filter_n, int filter_c, int filter_h, int filter_w,
+                                  int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
+                                  int groups, int output_n, int output_c, int output_h, int output_w, void* stream) {
+  CINN_RT_CHECK(num_args == 5, "cinn_call_hip_conv2d_bn_relu takes x, w, scale, shift and y, got %d arguments", num_args);
+  cinn_buffer_t* scale = BufferArg(v_args, 2);
+  cinn_buffer_t* shift = BufferArg(v_args, 3);
+  CINN_RT_CHECK(scale->type.code == cinn_type_float && scale->type.bits == 32 && shift->type.bits == 32,
+                "cinn_call_hip_conv2d_bn_relu: scale / shift must be fp32");
+  RunConv(BufferArg(v_args, 0), BufferArg(v_args, 1), BufferArg(v_args, 4), reinterpret_cast<const float*>(scale->memory),
+          reinterpret_cast<const float*>(shift->memory), relu ? 2 : 1, format, 1.0f, 0.0f, input_n, input_c, input_h,
+          input_w, filter_n, filter_c, filter_h, filter_w, pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w,
+          groups, output_n, output_c, output_h, output_w, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,204 @@
+// Pooling and log-softmax kernels behind cinn_call_cudnn_pool2d_forward / cinn_call_cudnn_softmax_forward.
+// Both are HBM-bound gather / reduce kernels with little reuse: one thread per output element for pooling
+// (consecutive threads on consecutive output columns, so input rows are read with unit stride inside a
+// window row), one block per softmax group.
+//
+// Pooling follows pe::PoolImpl (cinn/hlir/pe/nn.cc:956-1109): max pads with the lowest value of the type;
+// avg divides every element by the divisor BEFORE adding (divisor = window positions inside the input for
+// the exclusive mode, kh*kw otherwise), window rows then columns in ascending order.
+#include <hip/hip_runtime.h>
+
+#include <climits>
+#include <cstdint>
+
+#include "cinn_hip_runtime.h"
+#include "runtime/hip_check.h"
+
+namespace {
+
+struct PoolParams {
+  int n, c, ih, iw, oh, ow, kh, kw, ph, pw, sh, sw;
+  int mode;  // 0 / 3 max, 1 avg counting padding, 2 avg excluding padding
+  float alpha, beta;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) pool2d_nchw_kernel(const T* __restrict__ in, T* __restrict__ out, PoolParams p) {
+  const int64_t total = (int64_t)p.n * p.c * p.oh * p.ow;
+  const int64_t idx   = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int x   = (int)(idx % p.ow);
+  const int y   = (int)((idx / p.ow) % p.oh);
+  const int64_t plane = idx / ((int64_t)p.ow * p.oh);
+  const T* src  = in + plane * p.ih * p.iw;
+  const int ys = y * p.sh - p.ph, xs = x * p.sw - p.pw;
+  float result;
+  if (p.mode == 0 || p.mode == 3) {
+    float m = -3.402823466e+38f;
+    for (int ry = 0; ry < p.kh; ++ry) {
+      const int yy = ys + ry;
+      if (yy < 0 || yy >= p.ih) continue;
+      for (int rx = 0; rx < p.kw; ++rx) {
+        const int xx = xs + rx;
+        if (xx < 0 || xx >= p.iw) continue;
+        const float v = (float)src[yy * p.iw + xx];
+        m             = v > m ? v : m;
+      }
+    }
+    result = m;
+  } else {
+    float factor = (float)(p.kh * p.kw);
+    if (p.mode == 2) {
+      const int y0 = ys > 0 ? ys : 0, x0 = xs > 0 ? xs : 0;
+      const int y1 = ys + p.kh < p.ih ? ys + p.kh : p.ih, x1 = xs + p.kw < p.iw ? xs + p.kw : p.iw;
+      const int count = (y1 - y0) * (x1 - x0);
+      factor          = (float)(count > 1 ? count : 1);
+    }
+    float acc = 0.0f;
+    for (int ry = 0; ry < p.kh; ++ry) {
+      const int yy = ys + ry;
+      for (int rx = 0; rx < p.kw; ++rx) {
+        const int xx = xs + rx;
+        float v      = 0.0f;
+        if (yy >= 0 && yy < p.ih && xx >= 0 && xx < p.iw) v = (float)src[yy * p.iw + xx];
+        acc += v / factor;
+      }
+    }
+    result = acc;
+  }
+  float v = p.alpha * result;
+  if (p.beta != 0.0f) v += p.beta * (float)out[idx];
+  out[idx] = (T)v;
+}
+
+// block-wide reduction helper over 256 threads
+template <typename OP>
+__device__ __forceinline__ float BlockReduce(float v, float* scratch, OP op) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = op(v, __shfl_xor(v, off, 64));
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return op(op(scratch[0], scratch[1]), op(scratch[2], scratch[3]));
+}
+
+// y = alpha * log_softmax(x) + beta * y over `len` elements at stride `stride`, one block per group.
+// group g = (outer, inner): base = outer * len * stride_outer_unit + inner
+template <typename T>
+__global__ void __launch_bounds__(256) log_softmax_kernel(const T* __restrict__ in, T* __restrict__ out, int len, int inner,
+                                                          float alpha, float beta) {
+  __shared__ float scratch[4];
+  const int64_t g     = blockIdx.x;
+  const int64_t outer = g / inner, in_idx = g % inner;
+  const int64_t base  = outer * len * inner + in_idx;
+  float m = -3.402823466e+38f;
+  for (int i = threadIdx.x; i < len; i += 256) {
+    float v = (float)in[base + (int64_t)i * inner];
+    m       = v > m ? v : m;
+  }
+  m = BlockReduce(m, scratch, [](float a, float b) { return a > b ? a : b; });
+  float s = 0.0f;
+  for (int i = threadIdx.x; i < len; i += 256) s += expf((float)in[base + (int64_t)i * inner] - m);
+  s = BlockReduce(s, scratch, [](float a, float b) { return a + b; });
+  const float lse = m + logf(s);
+  for (int i = threadIdx.x; i < len; i += 256) {
+    const int64_t at = base + (int64_t)i * inner;
+    float v          = alpha * ((float)in[at] - lse);
+    if (beta != 0.0f) v += beta * (float)out[at];
+    out[at] = (T)v;
+  }
+}
+
+cinn_buffer_t* BufferArg(void* v_args, int index) {
+  auto* args = static_cast<cinn_pod_value_t*>(v_args);
+  CINN_RT_CHECK(args[index].type_code_ == CINN_POD_BUFFER_P, "argument %d is not a buffer", index);
+  return static_cast<cinn_buffer_t*>(args[index].value_.v_handle);
+}
+
+enum class Elem { kF32, kF16, kBF16 };
+Elem ElemOf(const cinn_buffer_t* b) {
+  const int bytes = b->type.bits / CHAR_BIT;
+  if (b->type.code == cinn_type_float && bytes == 4) return Elem::kF32;
+  if (b->type.code == cinn_type_float && bytes == 2) return Elem::kF16;
+  if (b->type.code == cinn_type_bfloat) return Elem::kBF16;
+  fprintf(stderr, "unsupported data type code %d bits %d\n", b->type.code, b->type.bits);
+  abort();
+}
+
+}  // namespace
+
+extern "C" {
+
+void cinn_call_cudnn_pool2d_forward(void* v_args, int num_args, int mode, int format, float alpha, float beta,
+                                    int input_n, int input_c, int input_h, int input_w, int kernel_h, int kernel_w,
+                                    int pad_h, int pad_w, int stride_h, int stride_w, int output_n, int output_c,
+                                    int output_h, int output_w, void* stream) {
+  CINN_RT_CHECK(num_args == 2, "cinn_call_cudnn_pool2d_forward takes x and y, got %d arguments", num_args);
+  CINN_RT_CHECK(format == 0, "pool2d: only NCHW (format 0) is implemented, got format %d", format);
+  CINN_RT_CHECK(mode >= 0 && mode <= 3, "pool2d: unknown pooling mode %d", mode);
+  CINN_RT_CHECK(output_n == input_n && output_c == input_c, "pool2d: batch / channel mismatch");
+  CINN_RT_CHECK(kernel_h > 0 && kernel_w > 0 && stride_h > 0 && stride_w > 0 && output_h > 0 && output_w > 0,
+                "pool2d: kernel, stride and output sizes must be positive");
+  // the last window must start inside the padded input
+  CINN_RT_CHECK((output_h - 1) * stride_h - pad_h < input_h && (output_w - 1) * stride_w - pad_w < input_w,
+                "pool2d: output %dx%d does not fit input %dx%d", output_h, output_w, input_h, input_w);
+  cinn_buffer_t* x = BufferArg(v_args, 0);
+  cinn_buffer_t* y = BufferArg(v_args, 1);
+  PoolParams p{input_n, input_c, input_h, input_w, output_h, output_w, kernel_h, kernel_w, pad_h, pad_w, stride_h,
+               stride_w, mode,    alpha,   beta};
+  const int64_t total = (int64_t)input_n * input_c * output_h * output_w;
+  CINN_RT_CHECK((int64_t)input_c * input_h * input_w * input_n < INT_MAX && total < INT_MAX, "pool2d: tensor too large");
+  dim3 grid((unsigned)((total + 255) / 256));
+  auto s = static_cast<hipStream_t>(stream);
+  switch (ElemOf(x)) {
+    case Elem::kF32:
+      hipLaunchKernelGGL(pool2d_nchw_kernel<float>, grid, dim3(256), 0, s, reinterpret_cast<const float*>(x->memory),
+                         reinterpret_cast<float*>(y->memory), p);
+      break;
+    case Elem::kF16:
+      hipLaunchKernelGGL(pool2d_nchw_kernel<_Float16>, grid, dim3(256), 0, s, reinterpret_cast<const _Float16*>(x->memory),
+                         reinterpret_cast<_Float16*>(y->memory), p);
+      break;
+    case Elem::kBF16:
+      hipLaunchKernelGGL(pool2d_nchw_kernel<__bf16>, grid, dim3(256), 0, s, reinterpret_cast<const __bf16*>(x->memory),
+                         reinterpret_cast<__bf16*>(y->memory), p);
+      break;
+  }
+  CINN_HIP_CALL(hipGetLastError());
+}
+
+void cinn_call_cudnn_softmax_forward(void* v_args, int num_args, int mode, int format, float alpha, float beta,
+                                     int input_n, int input_c, int input_h, int input_w, int output_n, int output_c,
+                                     int output_h, int output_w, void* stream) {
+  CINN_RT_CHECK(num_args == 2, "cinn_call_cudnn_softmax_forward takes x and y, got %d arguments", num_args);
+  CINN_RT_CHECK(format == 0, "softmax: only NCHW (format 0) is implemented, got format %d", format);
+  CINN_RT_CHECK(mode == 0 || mode == 1, "softmax: unknown mode %d", mode);
+  CINN_RT_CHECK(input_n == output_n && input_c == output_c && input_h == output_h && input_w == output_w,
+                "softmax: input and output shapes differ");
+  cinn_buffer_t* x = BufferArg(v_args, 0);
+  cinn_buffer_t* y = BufferArg(v_args, 1);
+  // mode 1 (per position): groups = n * h * w, length c, stride h*w; mode 0 (per instance): groups = n
+  const int len   = mode == 1 ? input_c : input_c * input_h * input_w;
+  const int inner = mode == 1 ? input_h * input_w : 1;
+  const int64_t groups = (int64_t)input_n * inner;
+  CINN_RT_CHECK(groups > 0 && groups < INT_MAX && len > 0, "softmax: bad extents");
+  dim3 grid((unsigned)groups);
+  auto s = static_cast<hipStream_t>(stream);
+  switch (ElemOf(x)) {
+    case Elem::kF32:
+      hipLaunchKernelGGL(log_softmax_kernel<float>, grid, dim3(256), 0, s, reinterpret_cast<const float*>(x->memory),
+                         reinterpret_cast<float*>(y->memory), len, inner, alpha, beta);
+      break;
+    case Elem::kF16:
+      hipLaunchKernelGGL(log_softmax_kernel<_Float16>, grid, dim3(256), 0, s, reinterpret_cast<const _Float16*>(x->memory),
+                         reinterpret_cast<_Float16*>(y->memory), len, inner, alpha, beta);
+      break;
+    case Elem::kBF16:
+      hipLaunchKernelGGL(log_softmax_kernel<__bf16>, grid, dim3(256), 0, s, reinterpret_cast<const __bf16*>(x->memory),
+                         reinterpret_cast<__bf16*>(y->memory), len, inner, alpha, beta);
+      break;
+  }
+  CINN_HIP_CALL(hipGetLastError());
+}
+
+}  // extern "C"

@@ -1,0 +1,211 @@
+"""GPU parity of the implicit-GEMM MFMA convolution, the fused batch_norm + relu that follows it, and pooling
+(BASELINE config 4 and the pooling layers of config 5), against the CPU oracle (pe::Conv2d_NCHW,
+pe::BatchNorm_NCHW, pe::PoolImpl restated).  Called through the C-ABI intrinsics with the argument lists of
+cinn_call_cudnn_conv2d_forward / cinn_call_cudnn_pool2d_forward, and through NetBuilder.  Bars: fp32 1e-5
+relative to the magnitude scale of the sum, fp16 1e-2."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import oracle
+from cinn_amd import _lib, runtime
+from cinn_amd.common import Float
+from cinn_amd.frontend import NetBuilder
+
+from helpers import run
+from test_golden import load
+
+pytestmark = pytest.mark.gpu
+
+
+def call_conv(x, w, stride, pad, dilation=(1, 1), groups=1, alpha=1.0, beta=0.0, y_init=None):
+    lib = _lib.load()
+    lib.cinn_call_cudnn_conv2d_forward.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_float,
+                                                   ctypes.c_float] + [ctypes.c_int] * 19 + [ctypes.c_void_p]
+    n, ic, ih, iw = x.shape
+    oc, fc, kh, kw = w.shape
+    oh = oracle.conv_out_dim(ih, kh, pad[0], stride[0], dilation[0])
+    ow = oracle.conv_out_dim(iw, kw, pad[1], stride[1], dilation[1])
+    dt = x.dtype.name
+    X, W = runtime.DeviceBuffer.from_numpy(x, dt), runtime.DeviceBuffer.from_numpy(w, dt)
+    Y = runtime.DeviceBuffer((n, oc, oh, ow), dt)
+    Y.copy_from(y_init if y_init is not None else np.zeros((n, oc, oh, ow), x.dtype))
+    args = runtime.pod_args([X, W, Y])
+    lib.cinn_call_cudnn_conv2d_forward(args, 3, 0, alpha, beta, n, ic, ih, iw, oc, fc, kh, kw, pad[0], pad[1], stride[0],
+                                       stride[1], dilation[0], dilation[1], groups, n, oc, oh, ow, None)
+    runtime.synchronize()
+    return Y.numpy()
+
+
+def conv_scale(x, w, stride, pad, dilation=(1, 1), groups=1):
+    """sum of |x|*|w| per output: the magnitude an fp32 summation error is relative to"""
+    return oracle.conv2d_nchw(np.abs(x).astype(np.float32), np.abs(w).astype(np.float32), stride, pad, dilation, groups)
+
+
+CASES = [
+    # (n, ic, hw, oc, k, stride, pad, dilation, groups)
+    (2, 8, 14, 8, 3, 1, 1, 1, 1),
+    (2, 16, 14, 32, 1, 2, 0, 1, 1),
+    (1, 3, 37, 10, 7, 2, 3, 1, 1),       # stem-like: K = 147 is not a multiple of the K step
+    (3, 6, 11, 4, 3, 2, 2, 2, 2),        # dilation and groups
+    (1, 130, 9, 140, 3, 1, 1, 1, 1),     # channel tails on both sides of the 128 tile
+    (5, 4, 5, 3, 5, 1, 0, 1, 1),         # single output pixel per image
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_conv2d_fp32_small_cases(gpu, case):
+    n, ic, hw, oc, k, s, p, d, g = case
+    rng = np.random.default_rng(sum(case))
+    x = rng.standard_normal((n, ic, hw, hw + 1)).astype(np.float32)
+    w = (rng.standard_normal((oc, ic // g, k, k)) * np.sqrt(2.0 / (ic // g * k * k))).astype(np.float32)
+    got = call_conv(x, w, (s, s), (p, p), (d, d), g)
+    want = oracle.conv2d_nchw(x, w, (s, s), (p, p), (d, d), g)
+    assert got.shape == want.shape
+    assert np.all(np.abs(got - want) <= 1e-5 * conv_scale(x, w, (s, s), (p, p), (d, d), g) + 1e-30)
+
+
+@pytest.mark.parametrize("case", CASES[:5])
+def test_conv2d_fp16_small_cases(gpu, case):
+    n, ic, hw, oc, k, s, p, d, g = case
+    rng = np.random.default_rng(sum(case) + 1)
+    x = rng.standard_normal((n, ic, hw, hw + 1)).astype(np.float16)
+    w = (rng.standard_normal((oc, ic // g, k, k)) * np.sqrt(2.0 / (ic // g * k * k))).astype(np.float16)
+    got = call_conv(x, w, (s, s), (p, p), (d, d), g).astype(np.float64)
+    want = oracle.conv2d_nchw(x, w, (s, s), (p, p), (d, d), g).astype(np.float64)
+    scale = conv_scale(x.astype(np.float32), w.astype(np.float32), (s, s), (p, p), (d, d), g)
+    assert np.all(np.abs(got - want) <= 1e-2 * np.maximum(np.abs(want), 1e-3 * scale) + 2.0 ** -24)
+
+
+def test_conv2d_alpha_beta(gpu):
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((1, 4, 6, 6)).astype(np.float32)
+    w = rng.standard_normal((5, 4, 3, 3)).astype(np.float32)
+    y0 = rng.standard_normal((1, 5, 6, 6)).astype(np.float32)
+    got = call_conv(x, w, (1, 1), (1, 1), alpha=0.5, beta=2.0, y_init=y0)
+    np.testing.assert_allclose(got, 0.5 * oracle.conv2d_nchw(x, w, (1, 1), (1, 1)) + 2.0 * y0, rtol=1e-5, atol=1e-5)
+
+
+# BASELINE config 4: ResNet-50 stage shapes at batch 32.  The full outputs are checked against the oracle on a
+# sample of images (the oracle's direct loops take seconds per image at these sizes) and for batch consistency.
+CONFIG4 = [("64->64 3x3 s1 p1 56x56", 64, 64, 3, 1, 1, 56), ("256->512 1x1 s2 56x56", 256, 512, 1, 2, 0, 56),
+           ("512->512 3x3 s1 p1 14x14", 512, 512, 3, 1, 1, 14)]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+@pytest.mark.parametrize("name,ic,oc,k,s,p,hw", CONFIG4)
+def test_config4_conv_bn_relu_batch32(gpu, dtype, name, ic, oc, k, s, p, hw):
+    rng = np.random.default_rng(400 + ic + oc + k)
+    x = rng.standard_normal((32, ic, hw, hw)).astype(dtype)
+    w = (rng.standard_normal((oc, ic, k, k)) * np.sqrt(2.0 / (ic * k * k))).astype(dtype)
+    scale = rng.uniform(0.5, 1.5, oc).astype(dtype)
+    bias = rng.uniform(0.5, 1.5, oc).astype(dtype)
+    mean = (rng.standard_normal(oc) * 0.1).astype(dtype)
+    var = rng.uniform(0.5, 1.5, oc).astype(dtype)
+    b = NetBuilder("cfg4")
+    T = Float(32) if dtype == "float32" else Float(16)
+    X, W = b.create_input(T, x.shape, "x"), b.create_input(T, w.shape, "w")
+    S, Bi, M, V = [b.create_input(T, [oc], nm) for nm in ("scale", "bias", "mean", "var")]
+    conv = b.conv2d(X, W, strides=[s, s], paddings=[p, p])
+    y = b.relu(b.batchnorm(conv, S, Bi, M, V, epsilon=1e-5)[0])
+    (got_conv, got), comp = run(b, {X: x, W: w, S: scale, Bi: bias, M: mean, V: var}, [conv, y])
+    # conv (MFMA) + per-channel sqrt + one fused bn/relu kernel
+    assert comp.num_instructions() == 3, comp.fusion_groups()
+    sample = [0, 17, 31]
+    want_conv = oracle.conv2d_nchw(x[sample], w, (s, s), (p, p))
+    want = oracle.batch_norm_relu_nchw(want_conv, scale, bias, mean, var, 1e-5, relu=True)
+    if dtype == "float32":
+        sc = conv_scale(x[sample], w, (s, s), (p, p))
+        assert np.all(np.abs(got_conv[sample] - want_conv) <= 1e-5 * sc)
+        # bn + relu on the GPU's own conv output must reproduce the oracle formula bit for bit
+        assert np.array_equal(got, oracle.batch_norm_relu_nchw(got_conv, scale, bias, mean, var, 1e-5, relu=True))
+        np.testing.assert_allclose(got[sample], want, rtol=1e-4, atol=1e-4)
+    else:
+        sc = conv_scale(x[sample].astype(np.float32), w.astype(np.float32), (s, s), (p, p))
+        assert np.all(np.abs(got_conv[sample].astype(np.float64) - want_conv.astype(np.float64)) <=
+                      1e-2 * np.maximum(np.abs(want_conv.astype(np.float64)), 1e-3 * sc) + 2.0 ** -24)
+        np.testing.assert_allclose(got[sample].astype(np.float64), want.astype(np.float64), rtol=2e-2, atol=2e-2)
+    # size-independent property: the same image placed at two batch positions gives identical outputs
+    x2 = x.copy()
+    x2[5] = x2[29]
+    b2 = NetBuilder("cfg4b")
+    X2, W2 = b2.create_input(T, x.shape, "x"), b2.create_input(T, w.shape, "w")
+    (c2,), _ = run(b2, {X2: x2, W2: w}, [b2.conv2d(X2, W2, strides=[s, s], paddings=[p, p])])
+    assert np.array_equal(c2[5], c2[29]) and np.array_equal(c2[29], got_conv[29])
+
+
+def test_golden_conv_fixtures(gpu):
+    for name, s, p in (("cfg4_conv_3x3_s1p1", 1, 1), ("cfg4_conv_1x1_s2", 2, 0)):
+        f = load(name)
+        got = call_conv(f["x"], f["w"], (s, s), (p, p))
+        np.testing.assert_allclose(got, f["conv"], rtol=1e-4, atol=1e-5)
+        b = NetBuilder("g")
+        X, W = b.create_input(Float(32), f["x"].shape, "x"), b.create_input(Float(32), f["w"].shape, "w")
+        P = [b.create_input(Float(32), f[k].shape, k) for k in ("scale", "bias", "mean", "var")]
+        y = b.relu(b.batchnorm(b.conv2d(X, W, strides=[s, s], paddings=[p, p]), *P)[0])
+        feeds = {X: f["x"], W: f["w"]}
+        feeds.update({v: f[k] for v, k in zip(P, ("scale", "bias", "mean", "var"))})
+        (out,), _ = run(b, feeds, [y])
+        np.testing.assert_allclose(out, f["y"], rtol=1e-4, atol=1e-4)
+
+
+def call_pool(x, ksize, stride, pad, mode, out_hw):
+    lib = _lib.load()
+    lib.cinn_call_cudnn_pool2d_forward.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                   ctypes.c_float, ctypes.c_float] + [ctypes.c_int] * 14 + [ctypes.c_void_p]
+    n, c, ih, iw = x.shape
+    X = runtime.DeviceBuffer.from_numpy(x, x.dtype.name)
+    Y = runtime.DeviceBuffer((n, c) + tuple(out_hw), x.dtype.name)
+    args = runtime.pod_args([X, Y])
+    lib.cinn_call_cudnn_pool2d_forward(args, 2, mode, 0, 1.0, 0.0, n, c, ih, iw, ksize[0], ksize[1], pad[0], pad[1],
+                                       stride[0], stride[1], n, c, out_hw[0], out_hw[1], None)
+    runtime.synchronize()
+    return Y.numpy()
+
+
+@pytest.mark.parametrize("pool_type,exclusive,mode", [("max", True, 0), ("avg", True, 2), ("avg", False, 1)])
+def test_pool2d_intrinsic(gpu, pool_type, exclusive, mode):
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((2, 5, 13, 12)).astype(np.float32)
+    want = oracle.pool2d_nchw(x, (3, 3), (2, 2), (1, 1, 1, 1), pool_type, exclusive)
+    got = call_pool(x, (3, 3), (2, 2), (1, 1), mode, want.shape[2:])
+    if pool_type == "max":
+        assert np.array_equal(got, want)
+    else:
+        np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-7)
+
+
+def test_pool2d_through_netbuilder_resnet_layers_and_golden(gpu):
+    f = load("pool2d")
+    b = NetBuilder("p")
+    X = b.create_input(Float(32), f["x"].shape, "x")
+    outs = [b.pool2d(X, "max", [3, 3], [2, 2], [1, 1]), b.pool2d(X, "avg", [14, 14], global_pooling=True),
+            b.pool2d(X, "max", [3, 3], [2, 2], [0, 0], ceil_mode=True), b.pool2d(X, "avg", [2, 2], [2, 2], [0, 0])]
+    (mx, gap, cm, av), _ = run(b, {X: f["x"]}, outs)
+    assert np.array_equal(mx, f["max_3x3_s2_p1"])
+    np.testing.assert_allclose(gap, f["avg_global"], rtol=1e-5, atol=1e-6)
+    assert np.array_equal(cm, oracle.pool2d_nchw(f["x"], (3, 3), (2, 2), (0, 0, 0, 0), "max", ceil_mode=True))
+    np.testing.assert_allclose(av, oracle.pool2d_nchw(f["x"], (2, 2), (2, 2), (0, 0, 0, 0), "avg"), rtol=1e-6)
+    rng = np.random.default_rng(8)
+    big = rng.standard_normal((4, 64, 112, 112)).astype(np.float32)
+    b = NetBuilder("p2")
+    X = b.create_input(Float(32), big.shape, "x")
+    (y,), _ = run(b, {X: big}, [b.pool2d(X, "max", [3, 3], [2, 2], [1, 1])])
+    assert np.array_equal(y, oracle.pool2d_nchw(big, (3, 3), (2, 2), (1, 1, 1, 1), "max"))
+
+
+def test_log_softmax_intrinsic(gpu):
+    lib = _lib.load()
+    lib.cinn_call_cudnn_softmax_forward.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                    ctypes.c_float, ctypes.c_float] + [ctypes.c_int] * 8 + [ctypes.c_void_p]
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((3, 10, 4, 5)).astype(np.float32)
+    X, Y = runtime.DeviceBuffer.from_numpy(x, "float32"), runtime.DeviceBuffer(x.shape, "float32")
+    args = runtime.pod_args([X, Y])
+    for mode, axes in ((1, (1,)), (0, (1, 2, 3))):
+        lib.cinn_call_cudnn_softmax_forward(args, 2, mode, 0, 1.0, 0.0, 3, 10, 4, 5, 3, 10, 4, 5, None)
+        runtime.synchronize()
+        x64 = x.astype(np.float64)
+        want = x64 - np.log(np.exp(x64).sum(axes, keepdims=True))
+        np.testing.assert_allclose(Y.numpy(), want, rtol=1e-5, atol=1e-6)
