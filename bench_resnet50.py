@@ -1,0 +1,144 @@
+"""ResNet-50 v1.5 inference (batch 32, 224x224, 1000 classes) built with NetBuilder, the whole-model workload the
+reference builds from its paddle model symbols (cinn/frontend/paddle_model_convertor.h:40-95, conv2d/batch_norm/relu/
+pool2d/mul ops of test/python/test_resnet.py).  `build_resnet50` describes the graph, `random_params` makes
+synthetic weights of that architecture, `measure` times whole forward passes (images/s)."""
+import time
+
+import numpy as np
+
+STAGES = ((3, 64, 1), (4, 128, 2), (6, 256, 2), (3, 512, 2))  # blocks, bottleneck width, stride of the stage
+
+
+def layer_specs():
+    """[(name, out_channels, in_channels, kernel, stride, pad)] of the 53 convolutions, in execution order."""
+    specs = [("conv1", 64, 3, 7, 2, 3)]
+    cin = 64
+    for si, (blocks, mid, stride) in enumerate(STAGES):
+        for bi in range(blocks):
+            s = stride if bi == 0 else 1
+            p = "s%db%d" % (si + 2, bi)
+            specs.append((p + "_a", mid, cin, 1, 1, 0))
+            specs.append((p + "_b", mid, mid, 3, s, 1))  # v1.5: the stride sits on the 3x3
+            specs.append((p + "_c", mid * 4, mid, 1, 1, 0))
+            if bi == 0:
+                specs.append((p + "_sc", mid * 4, cin, 1, s, 0))
+            cin = mid * 4
+    return specs
+
+
+def random_params(seed=0, dtype="float32", num_classes=1000):
+    """He-initialised convolutions and batch-norm statistics near identity; the last batch norm of every block is
+    scaled down so that activations keep their magnitude through the 16 residual additions."""
+    rng = np.random.default_rng(seed)
+    params = {}
+    for name, oc, ic, k, _, _ in layer_specs():
+        params[name + "_w"] = (rng.standard_normal((oc, ic, k, k)) * np.sqrt(2.0 / (ic * k * k))).astype(dtype)
+        gamma = rng.uniform(0.2, 0.4, oc) if name.endswith("_c") else rng.uniform(0.8, 1.2, oc)
+        params[name + "_scale"] = gamma.astype(dtype)
+        params[name + "_bias"] = rng.uniform(-0.1, 0.1, oc).astype(dtype)
+        params[name + "_mean"] = (rng.standard_normal(oc) * 0.1).astype(dtype)
+        params[name + "_var"] = rng.uniform(0.8, 1.2, oc).astype(dtype)
+    params["fc_w"] = (rng.standard_normal((2048, num_classes)) / np.sqrt(2048.0)).astype(dtype)
+    params["fc_b"] = rng.uniform(-0.1, 0.1, num_classes).astype(dtype)
+    return params
+
+
+def build_resnet50(builder, batch, dtype, params, image=224):
+    """Adds the network to `builder`; returns (image variable, {parameter name: variable}, logits variable)."""
+    from cinn_amd.common import Float
+    T = Float(32) if dtype == "float32" else Float(16)
+    specs = {s[0]: s for s in layer_specs()}
+    pv = {k: builder.create_input(T, list(v.shape), k) for k, v in params.items()}
+    x = builder.create_input(T, [batch, 3, image, image], "image")
+
+    def conv_bn(inp, name, relu):
+        _, _, _, _, s, p = specs[name]
+        y = builder.conv2d(inp, pv[name + "_w"], strides=[s, s], paddings=[p, p])
+        y = builder.batchnorm(y, pv[name + "_scale"], pv[name + "_bias"], pv[name + "_mean"], pv[name + "_var"],
+                              epsilon=1e-5)[0]
+        return builder.relu(y) if relu else y
+
+    y = conv_bn(x, "conv1", True)
+    y = builder.pool2d(y, "max", [3, 3], [2, 2], [1, 1])
+    for si, (blocks, _, _) in enumerate(STAGES):
+        for bi in range(blocks):
+            p = "s%db%d" % (si + 2, bi)
+            short = conv_bn(y, p + "_sc", False) if bi == 0 else y
+            z = conv_bn(y, p + "_a", True)
+            z = conv_bn(z, p + "_b", True)
+            z = conv_bn(z, p + "_c", False)
+            y = builder.relu(builder.add(z, short))
+    y = builder.pool2d(y, "avg", [7, 7], global_pooling=True)
+    y = builder.reshape(y, [batch, 2048])
+    logits = builder.add(builder.matmul(y, pv["fc_w"]), pv["fc_b"])
+    return x, pv, logits
+
+
+FLOP_PER_IMAGE = None
+
+
+def flop_per_image(image=224):
+    """2 * multiply-adds of the convolutions and the classifier"""
+    total, hw = 0, image
+    size = {}
+    cur = image
+    flops = 0
+    # spatial sizes: conv1 halves, the max pool halves, stages 3..5 halve at their first 3x3 / shortcut
+    for name, oc, ic, k, s, p in layer_specs():
+        if name == "conv1":
+            out = (cur + 2 * p - k) // s + 1
+            flops += 2 * oc * ic * k * k * out * out
+            cur = (out + 2 - 3) // 2 + 1
+            size["in"] = cur
+            continue
+        inp = size["in"] if not name.endswith("_c") else size["mid"]
+        if name.endswith("_a"):
+            out = inp
+        elif name.endswith("_b"):
+            out = (inp + 2 * p - k) // s + 1
+            size["mid"] = out
+        elif name.endswith("_c"):
+            out = inp
+            if not name.endswith("b0_c"):
+                size["in"] = out
+        else:  # shortcut, comes after _c of block 0
+            out = (size["in"] + 2 * p - k) // s + 1
+            size["in"] = out
+        flops += 2 * oc * ic * k * k * out * out
+    return flops + 2 * 2048 * 1000
+
+
+def measure(batch=32, dtype="float16", steps=20, warmup=3, graph=True, seed=0, **options):
+    from cinn_amd import runtime
+    from cinn_amd.common import DefaultAMDGPUTarget
+    from cinn_amd.frontend import Computation, NetBuilder
+    params = random_params(seed, dtype)
+    b = NetBuilder("resnet50")
+    x, pv, logits = build_resnet50(b, batch, dtype, params)
+    t0 = time.perf_counter()
+    stream = runtime.Stream()
+    comp = Computation.build_and_compile(DefaultAMDGPUTarget(), b, outputs=[logits], stream=stream, **options)
+    compile_s = time.perf_counter() - t0
+    rng = np.random.default_rng(seed + 1)
+    comp.get_tensor(x.id).from_numpy(rng.standard_normal((batch, 3, 224, 224)).astype(dtype))
+    for k, v in params.items():
+        comp.get_tensor(pv[k].id).from_numpy(v)
+    run = comp.execute_graph if graph else comp.execute
+    for _ in range(warmup):
+        run()
+    runtime.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run()
+    runtime.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    return {"workload": "resnet50_v1.5_b%d_%s" % (batch, dtype), "images_per_s": batch / dt, "ms_per_batch": dt * 1e3,
+            "tflops": flop_per_image() * batch / dt / 1e12, "instructions": comp.num_instructions(),
+            "compile_s": compile_s, "hip_graph": bool(graph)}
+
+
+if __name__ == "__main__":
+    import json
+    import sys
+    dtype = sys.argv[1] if len(sys.argv) > 1 else "float16"
+    print(json.dumps(measure(dtype=dtype)))

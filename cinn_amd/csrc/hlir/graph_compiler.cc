@@ -127,6 +127,10 @@ void Program::ExecuteGraph(void* stream) {
   CINN_CHECK(stream) << "graph replay needs an explicit stream";
   auto s = static_cast<hipStream_t>(stream);
   if (!graph_exec_) {
+    // Library-call kernels build per-shape tables and set function attributes on their first launch, which a
+    // capturing stream does not allow: run the program once before recording it.
+    for (auto& ins : instrs_) ins->Run(stream);
+    CINN_HIP_STATUS(static_cast<int>(hipStreamSynchronize(s)));
     hipGraph_t graph = nullptr;
     CINN_HIP_STATUS(static_cast<int>(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal)));
     for (auto& ins : instrs_) ins->Run(stream);
