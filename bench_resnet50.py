@@ -43,12 +43,17 @@ def random_params(seed=0, dtype="float32", num_classes=1000):
     return params
 
 
-def build_resnet50(builder, batch, dtype, params, image=224):
-    """Adds the network to `builder`; returns (image variable, {parameter name: variable}, logits variable)."""
+def build_resnet50(builder, batch, dtype, params, image=224, const_params=True):
+    """Adds the network to `builder`; returns (image variable, {parameter name: variable}, logits variable).
+    const_params marks the weights const, as the reference's model loader does for persistable variables: work that
+    depends on weights only (filter layout changes, sqrt(variance + eps)) then runs once instead of per batch."""
     from cinn_amd.common import Float
     T = Float(32) if dtype == "float32" else Float(16)
     specs = {s[0]: s for s in layer_specs()}
     pv = {k: builder.create_input(T, list(v.shape), k) for k, v in params.items()}
+    if const_params:
+        for v in pv.values():
+            v.set_const(True)
     x = builder.create_input(T, [batch, 3, image, image], "image")
 
     def conv_bn(inp, name, relu):

@@ -255,6 +255,14 @@ int cinn_amd_builder_var_info(cinn_amd_builder_t b, const char* id, int32_t* sha
   });
 }
 
+int cinn_amd_builder_set_const(cinn_amd_builder_t b, const char* id, int32_t is_const) {
+  return Guard([&] {
+    auto it = b->vars.find(id);
+    CINN_CHECK(it != b->vars.end()) << "unknown variable '" << id << "'";
+    it->second->is_const = is_const != 0;
+  });
+}
+
 int cinn_amd_builder_size(cinn_amd_builder_t b, int32_t* num_instructions) {
   return Guard([&] { *num_instructions = static_cast<int32_t>(b->builder->size()); });
 }
@@ -287,6 +295,8 @@ int cinn_amd_computation_build_and_compile(cinn_amd_builder_t b, const char* con
           opts.do_prerun = v != 0;
         } else if (k == "fuse_conv_bn_relu") {
           opts.fuse_conv_bn_relu = v != 0;
+        } else if (k == "conv_layout_nhwc") {
+          opts.conv_layout_nhwc = v != 0;
         } else if (k == "reduce_cached_elems") {
           opts.lowering.max_cached_elems_per_thread = v;
         } else if (k == "reduce_wave_elems") {
@@ -316,6 +326,9 @@ int cinn_amd_computation_execute(cinn_amd_computation_t c) {
 }
 int cinn_amd_computation_execute_graph(cinn_amd_computation_t c) {
   return Guard([&] { c->comp->ExecuteGraph(); });
+}
+int cinn_amd_computation_pre_run(cinn_amd_computation_t c) {
+  return Guard([&] { c->comp->PreRun(); });
 }
 int cinn_amd_computation_num_instructions(cinn_amd_computation_t c, int32_t* n) {
   return Guard([&] { *n = static_cast<int32_t>(c->comp->num_instructions()); });

@@ -1,6 +1,7 @@
 #include "frontend/computation.h"
 
 #include "frontend/decomposer.h"
+#include "frontend/layout_pass.h"
 
 namespace cinn {
 namespace frontend {
@@ -39,7 +40,10 @@ std::shared_ptr<CinnComputation> CinnComputation::Compile(const common::Target& 
   }
   for (auto& in : program.GetInputs()) comp->input_names_.push_back(in->id);
 
-  Program lowered = options.use_decomposer ? ApplyDecomposer(program) : program;
+  Program lowered = program;
+  if (options.conv_layout_nhwc) lowered = ConvertConvLayoutToNHWC(lowered, fetch_ids);
+  if (options.fuse_conv_bn_relu) lowered = FuseConvBatchNorm(lowered, fetch_ids);
+  if (options.use_decomposer) lowered = ApplyDecomposer(lowered);
   comp->graph_    = std::make_shared<Graph>(lowered, fetch_ids, target);
   comp->graph_->BuildFusionGroups();
   comp->scope_ = hlir::framework::BuildScope(target, comp->graph_);
@@ -79,6 +83,7 @@ void CinnComputation::GetTensorData(const std::string& tname, void* data, size_t
 }
 void CinnComputation::Execute() { program_->Execute(stream_); }
 void CinnComputation::ExecuteGraph() { program_->ExecuteGraph(stream_); }
+void CinnComputation::PreRun() { program_->RunPreRunInstructions(stream_); }
 
 }  // namespace frontend
 }  // namespace cinn

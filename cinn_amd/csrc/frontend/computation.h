@@ -23,6 +23,9 @@ class CinnComputation {
     bool do_prerun{true};
     // fold `conv2d -> batch_norm [-> relu]` into one convolution call with a fused epilogue
     bool fuse_conv_bn_relu{false};
+    // move conv2d chains written in NCHW to channels-last tensors, the layout the MFMA convolution kernels read
+    // with 16-byte accesses (frontend/layout_pass.h); off: every conv2d runs in the layout it was written in
+    bool conv_layout_nhwc{true};
   };
   static CompileOptions DefaultCompileOptions() { return CompileOptions(); }
 
@@ -47,6 +50,8 @@ class CinnComputation {
   void Execute();
   // replay through a captured HIP graph; needs a stream
   void ExecuteGraph();
+  // runs the pre-run instructions again (after the data of a const input was replaced)
+  void PreRun();
 
   const std::string& source_code() const { return source_code_; }
   std::string group_debug_string() const { return graph_->DebugGroupString(); }

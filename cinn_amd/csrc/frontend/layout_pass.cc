@@ -1,0 +1,330 @@
+#include "frontend/layout_pass.h"
+
+#include <algorithm>
+#include <map>
+
+#include "hlir/op.h"
+
+namespace cinn {
+namespace frontend {
+
+namespace {
+
+using hlir::framework::GetAttr;
+using hlir::framework::OpPatternKind;
+using hlir::framework::OpRegistry;
+using utils::AttributeMap;
+using utils::ShapeType;
+
+// Builds instructions with inferred output shapes; new variables are named <prefix><n>.
+class Emitter {
+ public:
+  Emitter(std::vector<Instruction>* out, std::string prefix) : out_(out), prefix_(std::move(prefix)) {}
+
+  std::vector<Variable> Emit(const std::string& type, const std::vector<Variable>& inputs, const AttributeMap& attrs) {
+    const auto& op = OpRegistry::Global().Get(type);
+    Instruction instr(type);
+    instr->inputs = inputs;
+    instr->attrs  = attrs;
+    std::vector<ShapeType> shapes;
+    std::vector<common::Type> types;
+    for (auto& in : inputs) {
+      shapes.push_back(in->shape);
+      types.push_back(in->type);
+    }
+    auto out_shapes = op.infer_shape(shapes, attrs);
+    auto out_types  = op.infer_dtype(types, attrs);
+    for (size_t i = 0; i < out_shapes.size(); ++i) {
+      Variable v(prefix_ + std::to_string(counter_++));
+      v->shape = out_shapes[i];
+      v->type  = out_types[i];
+      instr->outputs.push_back(v);
+    }
+    out_->push_back(instr);
+    return instr->outputs;
+  }
+  Variable Emit1(const std::string& type, const std::vector<Variable>& inputs, const AttributeMap& attrs) {
+    return Emit(type, inputs, attrs).front();
+  }
+  // same, but the result is the existing variable `result` (keeps its id for the consumers that follow)
+  void EmitInto(const Variable& result, const std::string& type, const std::vector<Variable>& inputs,
+                const AttributeMap& attrs) {
+    Instruction instr(type);
+    instr->inputs  = inputs;
+    instr->attrs   = attrs;
+    instr->outputs = {result};
+    out_->push_back(instr);
+  }
+
+ private:
+  std::vector<Instruction>* out_;
+  std::string prefix_;
+  int counter_{0};
+};
+
+ShapeType ToNhwc(const ShapeType& s) { return {s[0], s[2], s[3], s[1]}; }
+
+bool MfmaType(const common::Type& t) { return t.is_float(32) || t.is_float(16) || t.is_bfloat16(); }
+
+class LayoutConverter {
+ public:
+  LayoutConverter(const Program& program, const std::set<std::string>& fetch_ids)
+      : program_(program), fetch_ids_(fetch_ids), emit_(&out_, "nhwc_") {}
+
+  Program Run() {
+    for (auto& in : program_.GetInputs()) have_nchw_.insert(in->id);
+    for (auto& ins : program_.instructions()) {
+      for (auto& o : ins->outputs) vars_[o->id] = o;
+      Visit(ins);
+    }
+    for (auto& id : fetch_ids_) {
+      auto it = vars_.find(id);
+      if (it != vars_.end()) EnsureNchw(it->second);
+    }
+    return Program(std::move(out_), program_.GetInputs(), program_.name());
+  }
+
+ private:
+  bool HasTwin(const Variable& v) const { return nhwc_.count(v->id) != 0; }
+
+  // channels-last version of a 4-D NCHW value
+  Variable GetNhwc(const Variable& v) {
+    auto it = nhwc_.find(v->id);
+    if (it != nhwc_.end()) return it->second;
+    Variable t;
+    auto bc = channel_broadcast_.find(v->id);
+    if (bc != channel_broadcast_.end() && !have_nchw_.count(v->id)) {
+      // a per-channel vector replicated over an NCHW tensor: replicate it over the NHWC one instead
+      t = emit_.Emit1("broadcast_to", {bc->second->inputs[0]},
+                      {{"out_shape", ToNhwc(v->shape)}, {"broadcast_axes", ShapeType{3}}});
+    } else {
+      EnsureNchw(v);
+      if (v->shape[1] == 1 || (v->shape[2] == 1 && v->shape[3] == 1)) {
+        t = emit_.Emit1("reshape", {v}, {{"shape", ToNhwc(v->shape)}});
+      } else {
+        t = emit_.Emit1("transpose", {v}, {{"axis", ShapeType{0, 2, 3, 1}}});
+      }
+    }
+    nhwc_[v->id] = t;
+    return t;
+  }
+
+  // makes sure the original (NCHW) variable is defined by an emitted instruction
+  void EnsureNchw(const Variable& v) {
+    if (have_nchw_.count(v->id)) return;
+    auto bc = channel_broadcast_.find(v->id);
+    if (bc != channel_broadcast_.end()) {
+      out_.push_back(bc->second);
+    } else {
+      auto it = nhwc_.find(v->id);
+      CINN_CHECK(it != nhwc_.end()) << "variable " << v->id << " is used before it is defined";
+      if (v->shape[1] == 1 || (v->shape[2] == 1 && v->shape[3] == 1)) {
+        emit_.EmitInto(v, "reshape", {it->second}, {{"shape", v->shape}});
+      } else {
+        emit_.EmitInto(v, "transpose", {it->second}, {{"axis", ShapeType{0, 3, 1, 2}}});
+      }
+    }
+    have_nchw_.insert(v->id);
+  }
+
+  Variable FilterToOhwi(const Variable& w) {
+    auto it = filters_.find(w->id);
+    if (it != filters_.end()) return it->second;
+    EnsureNchw(w);
+    Variable t;
+    if (w->shape[2] == 1 && w->shape[3] == 1) {
+      t = emit_.Emit1("reshape", {w}, {{"shape", ShapeType{w->shape[0], 1, 1, w->shape[1]}}});
+    } else {
+      t = emit_.Emit1("transpose", {w}, {{"axis", ShapeType{0, 2, 3, 1}}});
+    }
+    filters_[w->id] = t;
+    return t;
+  }
+
+  void KeepAsIs(const Instruction& ins) {
+    for (auto& in : ins->inputs) {
+      if (in->shape.size() == 4 || channel_broadcast_.count(in->id)) EnsureNchw(in);
+    }
+    out_.push_back(ins);
+    for (auto& o : ins->outputs) have_nchw_.insert(o->id);
+  }
+
+  void Visit(const Instruction& ins) {
+    const std::string& op = ins->op_type;
+    if (op == "conv2d") {
+      auto x = ins->inputs[0], w = ins->inputs[1];
+      bool nchw    = GetAttr<std::string>(ins->attrs, "data_format", "NCHW") == "NCHW";
+      bool forward = GetAttr<std::string>(ins->attrs, "conv_type", "forward") == "forward";
+      int groups   = GetAttr<int>(ins->attrs, "groups", 1);
+      if (nchw && forward && groups == 1 && x->shape.size() == 4 && MfmaType(x->type)) {
+        AttributeMap attrs   = ins->attrs;
+        attrs["data_format"] = std::string("NHWC");
+        const int chunk      = 16 / x->type.bytes();
+        Variable y;
+        if (HasTwin(x) || x->shape[1] % chunk == 0) {
+          y = emit_.Emit1("conv2d", {GetNhwc(x), FilterToOhwi(w)}, attrs);
+        } else {
+          // few input channels (an image): the kernel reads the NCHW tensor and the [O][I][KH][KW] filter as they are
+          EnsureNchw(x);
+          EnsureNchw(w);
+          attrs["input_layout"] = std::string("NCHW");
+          y                     = emit_.Emit1("conv2d", {x, w}, attrs);
+        }
+        nhwc_[ins->outputs[0]->id] = y;
+        return;
+      }
+    } else if (op == "batch_norm") {
+      auto x = ins->inputs[0];
+      if (GetAttr<std::string>(ins->attrs, "data_layout", "NCHW") == "NCHW" && x->shape.size() == 4 && HasTwin(x)) {
+        AttributeMap attrs   = ins->attrs;
+        attrs["data_layout"] = std::string("NHWC");
+        std::vector<Variable> inputs = ins->inputs;
+        inputs[0]                    = GetNhwc(x);
+        auto outs                    = emit_.Emit("batch_norm", inputs, attrs);
+        nhwc_[ins->outputs[0]->id]   = outs[0];
+        return;
+      }
+    } else if (op == "pool2d") {
+      auto x = ins->inputs[0];
+      if (GetAttr<std::string>(ins->attrs, "data_format", "NCHW") == "NCHW" && x->shape.size() == 4 && HasTwin(x)) {
+        AttributeMap attrs   = ins->attrs;
+        attrs["data_format"] = std::string("NHWC");
+        nhwc_[ins->outputs[0]->id] = emit_.Emit1("pool2d", {GetNhwc(x)}, attrs);
+        return;
+      }
+    } else if (op == "broadcast_to") {
+      auto x    = ins->inputs[0];
+      auto axes = GetAttr<ShapeType>(ins->attrs, "broadcast_axes", {});
+      auto& out = ins->outputs[0];
+      if (out->shape.size() == 4 && x->shape.size() == 1 && axes.size() == 1 && axes[0] == 1 &&
+          x->shape[0] == out->shape[1]) {
+        // decided by the first consumer: emitted as it is, or replicated over the channels-last shape
+        channel_broadcast_[out->id] = ins;
+        return;
+      }
+    } else {
+      const auto* def = OpRegistry::Global().Find(op);
+      if (def && def->pattern == OpPatternKind::kElementWise && ins->outputs.size() == 1 &&
+          ins->outputs[0]->shape.size() == 4 && !ins->inputs.empty()) {
+        bool same_shape = true, any_twin = false;
+        for (auto& in : ins->inputs) {
+          same_shape = same_shape && in->shape == ins->outputs[0]->shape;
+          any_twin   = any_twin || (HasTwin(in) && !have_nchw_.count(in->id));
+        }
+        if (same_shape && any_twin) {
+          std::vector<Variable> inputs;
+          for (auto& in : ins->inputs) inputs.push_back(GetNhwc(in));
+          nhwc_[ins->outputs[0]->id] = emit_.Emit1(op, inputs, ins->attrs);
+          return;
+        }
+      }
+    }
+    KeepAsIs(ins);
+  }
+
+  const Program& program_;
+  const std::set<std::string>& fetch_ids_;
+  std::vector<Instruction> out_;
+  Emitter emit_;
+  std::map<std::string, Variable> vars_;     // every variable an instruction of the program defines
+  std::map<std::string, Variable> nhwc_;     // NCHW variable id -> its channels-last twin
+  std::map<std::string, Variable> filters_;  // filter id -> [O][KH][KW][I] copy
+  std::set<std::string> have_nchw_;          // ids whose NCHW form is defined in the output program
+  std::map<std::string, Instruction> channel_broadcast_;  // deferred per-channel broadcast_to instructions
+};
+
+}  // namespace
+
+Program ConvertConvLayoutToNHWC(const Program& program, const std::set<std::string>& fetch_ids) {
+  bool has_conv = false;
+  for (auto& ins : program.instructions()) has_conv = has_conv || ins->op_type == "conv2d";
+  if (!has_conv) return program;
+  return LayoutConverter(program, fetch_ids).Run();
+}
+
+Program FuseConvBatchNorm(const Program& program, const std::set<std::string>& fetch_ids) {
+  const auto& instrs = program.instructions();
+  // consumers of every variable
+  std::map<std::string, std::vector<size_t>> users;
+  for (size_t i = 0; i < instrs.size(); ++i)
+    for (auto& in : instrs[i]->inputs) users[in->id].push_back(i);
+  auto single_user = [&](const Variable& v) -> int {
+    if (fetch_ids.count(v->id)) return -1;
+    auto it = users.find(v->id);
+    if (it == users.end() || it->second.size() != 1) return -1;
+    return static_cast<int>(it->second[0]);
+  };
+
+  std::vector<bool> dropped(instrs.size(), false);
+  std::map<size_t, std::vector<Instruction>> replacement;  // position of the last instruction of a match
+  int serial = 0;
+  for (size_t i = 0; i < instrs.size(); ++i) {
+    auto& conv = instrs[i];
+    if (conv->op_type != "conv2d" || dropped[i]) continue;
+    if (GetAttr<std::string>(conv->attrs, "data_format", "NCHW") != "NHWC") continue;
+    if (GetAttr<int>(conv->attrs, "groups", 1) != 1) continue;
+    int bn_at = single_user(conv->outputs[0]);
+    if (bn_at < 0 || instrs[bn_at]->op_type != "batch_norm" || !(instrs[bn_at]->inputs[0] == conv->outputs[0])) continue;
+    auto& bn = instrs[bn_at];
+    if (GetAttr<std::string>(bn->attrs, "data_layout", "NCHW") != "NHWC") continue;
+    size_t last     = bn_at;
+    Variable result = bn->outputs[0];
+    Variable residual;
+    bool relu = false;
+    int next  = single_user(result);
+    if (next >= 0 && instrs[next]->op_type == "elementwise_add" && instrs[next]->inputs.size() == 2) {
+      auto& add     = instrs[next];
+      Variable other = add->inputs[0] == result ? add->inputs[1] : add->inputs[0];
+      if (!(other == result) && other->shape == result->shape) {
+        residual = other;
+        dropped[next] = true;
+        last     = next;
+        result   = add->outputs[0];
+        next     = single_user(result);
+      }
+    }
+    if (next >= 0 && instrs[next]->op_type == "relu") {
+      relu          = true;
+      dropped[next] = true;
+      last          = next;
+      result        = instrs[next]->outputs[0];
+    }
+    dropped[i]     = true;
+    dropped[bn_at] = true;
+
+    // s = scale / sqrt(variance + eps), t = bias - mean * s, in fp32
+    std::vector<Instruction> seq;
+    Emitter e(&seq, "cbr" + std::to_string(serial++) + "_");
+    float eps  = GetAttr<float>(bn->attrs, "epsilon", 1e-5f);
+    auto to_f32 = [&](const Variable& v) {
+      if (v->type == common::Float(32)) return v;
+      return e.Emit1("cast", {v}, {{"dtype", std::string("float32")}});
+    };
+    auto scale = to_f32(bn->inputs[1]), bias = to_f32(bn->inputs[2]), mean = to_f32(bn->inputs[3]),
+         var   = to_f32(bn->inputs[4]);
+    auto epsv  = e.Emit1("fill_constant", {},
+                         {{"shape", var->shape}, {"value", static_cast<double>(eps)}, {"dtype", std::string("float32")}, {"force_cpu", false}});
+    auto denom = e.Emit1("sqrt", {e.Emit1("elementwise_add", {var, epsv}, {{"axis", -1}})}, {});
+    auto s     = e.Emit1("divide", {scale, denom}, {{"axis", -1}});
+    auto t     = e.Emit1("subtract", {bias, e.Emit1("elementwise_mul", {mean, s}, {{"axis", -1}})}, {{"axis", -1}});
+    AttributeMap attrs = conv->attrs;
+    attrs["relu"]      = relu;
+    std::vector<Variable> inputs = {conv->inputs[0], conv->inputs[1], s, t};
+    if (residual.defined()) inputs.push_back(residual);
+    e.EmitInto(result, "hip_conv2d_bn_relu", inputs, attrs);
+    replacement[last] = seq;
+  }
+  std::vector<Instruction> out;
+  for (size_t i = 0; i < instrs.size(); ++i) {
+    auto it = replacement.find(i);
+    if (it != replacement.end()) {
+      out.insert(out.end(), it->second.begin(), it->second.end());
+    } else if (!dropped[i]) {
+      out.push_back(instrs[i]);
+    }
+  }
+  return Program(std::move(out), program.GetInputs(), program.name());
+}
+
+}  // namespace frontend
+}  // namespace cinn

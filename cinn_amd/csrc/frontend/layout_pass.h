@@ -1,0 +1,28 @@
+// Program passes that prepare convolutional networks for the gfx950 convolution kernels.
+//
+// ConvertConvLayoutToNHWC: the MFMA convolution kernels want the reduction index (input channel) contiguous in
+// memory, i.e. channels-last activations and [O][KH][KW][I] filters.  Programs are written in NCHW (the layout of
+// the paddle models the reference compiles), so this pass moves every chain
+//     conv2d -> batch_norm / pool2d / element-wise ops -> conv2d ...
+// to NHWC: tensors inside the chain only exist channels-last, transposes appear where a chain starts from or
+// returns to an op that needs NCHW (reshape, matmul, fetched outputs), and filters are transposed once (a
+// pre-run instruction when the filter is marked const).  The reference has the same kind of pass for its x86
+// NCHWc kernels (cinn/hlir/pass/alterlayout.cc).
+//
+// FuseConvBatchNorm: folds `conv2d -> batch_norm [-> + residual] [-> relu]` on channels-last tensors into one
+// hip_conv2d_bn_relu call whose epilogue applies y = conv * s + t with s = scale / sqrt(variance + eps),
+// t = bias - mean * s (computed by ordinary fp32 instructions, pre-run for const statistics).
+#pragma once
+#include <set>
+#include <string>
+
+#include "frontend/syntax.h"
+
+namespace cinn {
+namespace frontend {
+
+Program ConvertConvLayoutToNHWC(const Program& program, const std::set<std::string>& fetch_ids);
+Program FuseConvBatchNorm(const Program& program, const std::set<std::string>& fetch_ids);
+
+}  // namespace frontend
+}  // namespace cinn

@@ -38,6 +38,7 @@ bool IsFusibleOp(const Node& n) {
 struct WorkGroup {
   GroupKind kind;
   std::vector<Node*> nodes;  // kept sorted by node index
+  bool pre_run{false};
   int64_t numel{0};          // kElementwise: size of the flat space
   int64_t rows{0}, cols{0};  // kRowReduce
 };
@@ -139,6 +140,7 @@ void Graph::BuildFusionGroups() {
     Node* n = np.get();
     auto g  = std::make_unique<WorkGroup>();
     g->nodes.push_back(n);
+    g->pre_run = n->pre_run;
     if (n->op->pattern == OpPatternKind::kReduction) {
       int64_t r, c;
       if (TrailingReduceSpace(n->inputs[0]->shape, ReduceDimsOf(*n), &r, &c) && c > 1 &&
@@ -190,6 +192,8 @@ void Graph::BuildFusionGroups() {
   auto merged_shape = [&](WorkGroup* p, WorkGroup* c, WorkGroup* out) -> bool {
     auto fusible_kind = [](GroupKind k) { return k == GroupKind::kElementwise || k == GroupKind::kRowReduce; };
     if (!fusible_kind(p->kind) || !fusible_kind(c->kind)) return false;
+    // pre-run nodes execute once, ahead of everything else: they only fuse among themselves
+    if (p->pre_run != c->pre_run) return false;
     std::vector<Node*> nodes = p->nodes;
     nodes.insert(nodes.end(), c->nodes.begin(), c->nodes.end());
     std::sort(nodes.begin(), nodes.end(), [](Node* a, Node* b) { return a->index < b->index; });
@@ -268,6 +272,7 @@ void Graph::BuildFusionGroups() {
     g->nodes = w->nodes;
     g->rows  = w->rows;
     g->cols  = w->cols;
+    g->pre_run = w->pre_run;
     std::map<NodeData*, bool> produced;
     for (Node* n : g->nodes) {
       n->group_id = g->id;

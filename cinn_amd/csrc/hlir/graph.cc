@@ -14,6 +14,7 @@ NodeData* Graph::GetOrCreateVar(const frontend::Variable& v) {
   data->id    = v->id;
   data->shape = v->shape;
   data->dtype = v->type;
+  data->is_const = v->is_const;
   auto* p     = data.get();
   vars_[v->id] = std::move(data);
   return p;
@@ -78,6 +79,39 @@ Graph::Graph(const frontend::Program& program, const std::set<std::string>& fetc
     CINN_CHECK(v) << "fetch variable " << id << " does not exist in the program";
     v->is_fetch = true;
   }
+  ConstPropagate();
+}
+
+// ConstPropagatePass (cinn/hlir/pass/const_propagate.cc:33-58): a node whose inputs are all const is a pre-run node
+// and its outputs are const.  Only fed inputs start const-ness here; a fill_constant joins the pre-run set when
+// a pre-run node consumes it, otherwise it stays with (and is folded into) its consumers.
+void Graph::ConstPropagate() {
+  for (auto& np : nodes_) {
+    Node* n = np.get();
+    if (n->op_type() == "fill_constant") continue;
+    // replicating a const value is left to the consumer, which reads the small tensor in place: materialising the
+    // replicated tensor once would turn a per-channel vector into a full activation-sized read in every execution
+    if (n->op->pattern == OpPatternKind::kBroadcast) continue;
+    bool all_const = !n->inputs.empty();
+    for (auto* in : n->inputs) {
+      bool literal = in->producer && in->producer->op_type() == "fill_constant";
+      all_const    = all_const && (in->is_const || literal);
+    }
+    // something fed must take part: a chain of literals alone is folded, not pre-run
+    bool any_fed = false;
+    for (auto* in : n->inputs) any_fed = any_fed || in->is_const;
+    if (!all_const || !any_fed) continue;
+    n->pre_run = true;
+    for (auto* o : n->outputs) o->is_const = true;
+  }
+  for (auto& np : nodes_) {
+    Node* n = np.get();
+    if (n->op_type() != "fill_constant" || n->outputs[0]->consumers.empty()) continue;
+    // with consumers on both sides it is computed once up front and read from memory by the others
+    bool any_pre_run = false;
+    for (Node* c : n->outputs[0]->consumers) any_pre_run = any_pre_run || c->pre_run;
+    n->pre_run = any_pre_run;
+  }
 }
 
 NodeData* Graph::FindVar(const std::string& id) const {
@@ -101,6 +135,7 @@ std::string Graph::DebugGroupString() const {
       case GroupKind::kGeneralReduce: os << "general_reduce"; break;
       case GroupKind::kLibraryCall: os << "library_call"; break;
     }
+    if (g->pre_run) os << " pre_run";
     os << " {";
     for (auto* n : g->nodes) os << " " << n->op_type();
     os << " } in:";

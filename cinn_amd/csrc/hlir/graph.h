@@ -26,6 +26,9 @@ struct NodeData {
   Node* producer{nullptr};  // nullptr: fed input
   std::vector<Node*> consumers;
   bool is_fetch{false};
+  // value that does not change between executions: a program input marked const (weights) or the result of an
+  // operator whose inputs are all const (NodeData::is_const of cinn/hlir/framework/node.h)
+  bool is_const{false};
   int64_t numel() const { return ShapeNumel(shape); }
 };
 
@@ -36,6 +39,9 @@ struct Node {
   std::vector<NodeData*> inputs;
   std::vector<NodeData*> outputs;
   int group_id{-1};
+  // all inputs are const: runs once in Program::PreRun instead of in every execution (the "pre_run" attribute of
+  // cinn/hlir/pass/const_propagate.cc:33-58)
+  bool pre_run{false};
   const std::string& op_type() const { return op->name; }
 };
 
@@ -54,6 +60,7 @@ struct Group {
   std::vector<NodeData*> outputs;     // values consumed outside the group or fetched
   // kRowReduce: rows x cols of the reduction space
   int64_t rows{0}, cols{0};
+  bool pre_run{false};  // every node of the group is a pre-run node
   std::string func_name;
 };
 
@@ -76,6 +83,7 @@ class Graph {
 
  private:
   NodeData* GetOrCreateVar(const frontend::Variable& v);
+  void ConstPropagate();
   common::Target target_;
   std::string name_;
   std::vector<std::unique_ptr<Node>> nodes_;

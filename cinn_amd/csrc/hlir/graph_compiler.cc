@@ -106,19 +106,38 @@ void Instruction::Run(void* stream) {
 }
 
 // ---- Program --------------------------------------------------------------------------------------
+Program::Program(std::shared_ptr<Scope> scope, std::vector<std::unique_ptr<Instruction>> instrs)
+    : scope_(std::move(scope)) {
+  for (auto& ins : instrs) {
+    if (ins->pre_run) {
+      prerun_instrs_.push_back(std::move(ins));
+    } else {
+      instrs_.push_back(std::move(ins));
+    }
+  }
+}
+
 Program::~Program() {
   if (graph_exec_) (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec_));
   if (graph_) (void)hipGraphDestroy(static_cast<hipGraph_t>(graph_));
 }
 
 void Program::PreRun(const common::Target& target) {
-  for (auto& ins : instrs_) {
-    for (auto& a : ins->in_args()) scope_->GetTensor(a)->mutable_data(target);
-    for (auto& a : ins->out_args()) scope_->GetTensor(a)->mutable_data(target);
+  for (auto* list : {&prerun_instrs_, &instrs_}) {
+    for (auto& ins : *list) {
+      for (auto& a : ins->in_args()) scope_->GetTensor(a)->mutable_data(target);
+      for (auto& a : ins->out_args()) scope_->GetTensor(a)->mutable_data(target);
+    }
   }
 }
 
+void Program::RunPreRunInstructions(void* stream) {
+  for (auto& ins : prerun_instrs_) ins->Run(stream);
+  prerun_done_ = true;
+}
+
 void Program::Execute(void* stream) {
+  if (!prerun_done_) RunPreRunInstructions(stream);
   for (auto& ins : instrs_) ins->Run(stream);
   if (!stream) CINN_HIP_STATUS(cinn_hip_device_synchronize());
 }
@@ -126,6 +145,7 @@ void Program::Execute(void* stream) {
 void Program::ExecuteGraph(void* stream) {
   CINN_CHECK(stream) << "graph replay needs an explicit stream";
   auto s = static_cast<hipStream_t>(stream);
+  if (!prerun_done_) RunPreRunInstructions(stream);
   if (!graph_exec_) {
     // Library-call kernels build per-shape tables and set function attributes on their first launch, which a
     // capturing stream does not allow: run the program once before recording it.
@@ -192,6 +212,7 @@ std::unique_ptr<Program> GraphCompiler::Build(const CompileOptions& options) {
     void* fn   = compiler_->Lookup(g->func_name);
     CINN_CHECK(fn) << "compiled function " << g->func_name << " not found";
     instr->SetLoweredFunc(fn);
+    instr->pre_run = g->pre_run;
     instrs.push_back(std::move(instr));
   }
   auto program = std::make_unique<Program>(scope_, std::move(instrs));

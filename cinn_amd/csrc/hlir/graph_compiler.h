@@ -79,6 +79,8 @@ class Instruction {
   const std::string& function_name() const { return function_name_; }
   const std::vector<std::string>& in_args() const { return in_args_; }
   const std::vector<std::string>& out_args() const { return out_args_; }
+  // runs once ahead of the first execution instead of in every one (cinn/hlir/framework/instruction.h:129)
+  bool pre_run{false};
 
  private:
   void UpdateArgsCache();
@@ -92,11 +94,15 @@ class Instruction {
 
 class Program {
  public:
-  Program(std::shared_ptr<Scope> scope, std::vector<std::unique_ptr<Instruction>> instrs)
-      : scope_(std::move(scope)), instrs_(std::move(instrs)) {}
+  // splits off the pre-run instructions (cinn/hlir/framework/graph_compiler.cc:66-76)
+  Program(std::shared_ptr<Scope> scope, std::vector<std::unique_ptr<Instruction>> instrs);
   ~Program();
   // allocate every tensor the instructions touch
   void PreRun(const common::Target& target);
+  // Runs the pre-run instructions (those whose inputs are all const, e.g. filter layout changes and folded
+  // batch-norm statistics).  Execute / ExecuteGraph call it once by themselves; call it again after the data of
+  // a const input has been replaced.
+  void RunPreRunInstructions(void* stream = nullptr);
   // Runs all instructions on `stream`; with stream == nullptr the null stream is used and the device
   // is synchronised afterwards.
   void Execute(void* stream = nullptr);
@@ -105,11 +111,14 @@ class Program {
   void ExecuteGraph(void* stream);
   size_t size() const { return instrs_.size(); }
   const std::vector<std::unique_ptr<Instruction>>& GetRunInstructions() const { return instrs_; }
+  const std::vector<std::unique_ptr<Instruction>>& GetPreRunInstructions() const { return prerun_instrs_; }
   std::shared_ptr<Scope> scope() const { return scope_; }
 
  private:
   std::shared_ptr<Scope> scope_;
   std::vector<std::unique_ptr<Instruction>> instrs_;
+  std::vector<std::unique_ptr<Instruction>> prerun_instrs_;
+  bool prerun_done_{false};
   void* graph_exec_{nullptr};
   void* graph_{nullptr};
 };

@@ -1050,23 +1050,28 @@ ir::LoweredFuncRef OpLowerer::LowerLibraryCall(const Group& group) const {
     const auto& x = n->inputs[0]->shape;
     const auto& w = n->inputs[1]->shape;
     const auto& y = n->outputs[0]->shape;
-    bool nchw     = layout == "NCHW";
+    bool nchw       = layout == "NCHW";
+    bool nchw_input = GetAttr<std::string>(n->attrs, "input_layout", layout) == "NCHW";
+    // tensor format of the intrinsic: 0 NCHW, 1 NHWC, 2 NHWC output from an NCHW input and OIHW filter
+    int format = nchw ? 0 : (nchw_input ? 2 : 1);
     if (op == "conv2d") {
       api = "cinn_call_cudnn_conv2d_forward";
-      args.push_back(I32(nchw ? 0 : 1));
+      args.push_back(I32(format));
       args.push_back(Expr(1.0f));
       args.push_back(Expr(0.0f));
     } else {
       api = "cinn_call_hip_conv2d_bn_relu";
-      args.push_back(I32(nchw ? 0 : 1));
+      args.push_back(I32(format));
       args.push_back(I32(GetAttr<bool>(n->attrs, "relu", false) ? 1 : 0));
     }
-    if (nchw) {
+    // extents are always passed in n, c, h, w order
+    if (nchw_input) {
       push_ints({x[0], x[1], x[2], x[3]});
+      push_ints({w[0], w[1], w[2], w[3]});
     } else {
       push_ints({x[0], x[3], x[1], x[2]});
+      push_ints({w[0], w[3], w[1], w[2]});
     }
-    push_ints({w[0], w[1], w[2], w[3]});
     push_ints({padding[0], padding[1], stride[0], stride[1], dilation[0], dilation[1], groups});
     if (nchw) {
       push_ints({y[0], y[1], y[2], y[3]});

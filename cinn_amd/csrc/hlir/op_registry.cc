@@ -484,15 +484,24 @@ OpRegistry::OpRegistry() {
       CINN_CHECK(in[0].size() == 4 && in[1].size() == 4) << "conv2d: 4-D input and filter expected";
       CINN_CHECK(layout == "NCHW" || layout == "NHWC") << "conv2d: unknown data_format " << layout;
       ShapeType out(4);
+      // "input_layout" = "NCHW" on a channels-last convolution: the input (and the [O][I][KH][KW] filter) are still
+      // NCHW, only the output is NHWC (the convolution of a network's image input)
+      bool nchw_input = GetAttr<std::string>(a, "input_layout", layout) == "NCHW";
       if (layout == "NCHW") {
         out[0] = in[0][0];
         out[1] = in[1][0];
         out[2] = ConvOutDim(in[0][2], padding[0], dilation[0], in[1][2], stride[0]);
         out[3] = ConvOutDim(in[0][3], padding[1], dilation[1], in[1][3], stride[1]);
-      } else {
+      } else if (nchw_input) {
         out[0] = in[0][0];
-        out[1] = ConvOutDim(in[0][1], padding[0], dilation[0], in[1][2], stride[0]);
-        out[2] = ConvOutDim(in[0][2], padding[1], dilation[1], in[1][3], stride[1]);
+        out[1] = ConvOutDim(in[0][2], padding[0], dilation[0], in[1][2], stride[0]);
+        out[2] = ConvOutDim(in[0][3], padding[1], dilation[1], in[1][3], stride[1]);
+        out[3] = in[1][0];
+      } else {
+        // channels-last filters are [O][KH][KW][I] (InferShapeForConv2d reads h / w at 1 / 2, cinn/hlir/op/nn.cc:510-527)
+        out[0] = in[0][0];
+        out[1] = ConvOutDim(in[0][1], padding[0], dilation[0], in[1][1], stride[0]);
+        out[2] = ConvOutDim(in[0][2], padding[1], dilation[1], in[1][2], stride[1]);
         out[3] = in[1][0];
       }
       return std::vector<ShapeType>{out};
@@ -500,11 +509,11 @@ OpRegistry::OpRegistry() {
     op.infer_dtype = SameTypeAsFirst;
   }
   {
-    // conv2d followed by a per-channel affine and optional relu, produced by the conv+bn+relu
-    // graph rewrite; inputs x, w, scale, shift
+    // conv2d followed by a per-channel affine, an optional residual addition and an optional relu, produced by
+    // the conv+bn+relu graph rewrite; inputs x, w, scale, shift[, residual]
     auto& op       = r->Register("hip_conv2d_bn_relu");
     op.pattern     = OpPatternKind::kNonFusible;
-    op.num_inputs  = 4;
+    op.num_inputs  = -1;
     const auto* cv = r->Find("conv2d");
     auto conv_shape = cv->infer_shape;
     op.infer_shape = [conv_shape](const std::vector<ShapeType>& in, const AttributeMap& a) {

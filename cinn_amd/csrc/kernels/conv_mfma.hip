@@ -25,6 +25,7 @@
 #include <vector>
 
 #include "cinn_hip_runtime.h"
+#include "kernels/conv_nhwc.h"
 #include "runtime/hip_check.h"
 
 namespace {
@@ -276,10 +277,10 @@ cinn_buffer_t* BufferArg(void* v_args, int index) {
   return static_cast<cinn_buffer_t*>(args[index].value_.v_handle);
 }
 
-void RunConv(cinn_buffer_t* x, cinn_buffer_t* w, cinn_buffer_t* y, const float* scale, const float* shift, int epilogue,
-             int format, float alpha, float beta, int in, int ic, int ih, int iw, int fn, int fc, int fh, int fw, int ph,
+void RunConv(cinn_buffer_t* x, cinn_buffer_t* w, cinn_buffer_t* y, const float* scale, const float* shift,
+             cinn_buffer_t* residual, int epilogue, int format, float alpha, float beta, int in, int ic, int ih, int iw, int fn, int fc, int fh, int fw, int ph,
              int pw, int sh, int sw, int dh, int dw, int groups, int on, int oc, int oh, int ow, hipStream_t stream) {
-  CINN_RT_CHECK(format == 0, "conv2d: only NCHW (format 0) is implemented, got format %d", format);
+  CINN_RT_CHECK(format >= 0 && format <= 2, "conv2d: unknown tensor format %d", format);
   CINN_RT_CHECK(groups >= 1 && ic % groups == 0 && fn % groups == 0, "conv2d: bad group count %d", groups);
   CINN_RT_CHECK(fc == ic / groups, "conv2d: filter has %d input channels, expected %d", fc, ic / groups);
   CINN_RT_CHECK(on == in && oc == fn, "conv2d: output is [%d,%d,..], expected [%d,%d,..]", on, oc, in, fn);
@@ -289,6 +290,26 @@ void RunConv(cinn_buffer_t* x, cinn_buffer_t* w, cinn_buffer_t* y, const float* 
   CINN_RT_CHECK(oh == want_oh && ow == want_ow, "conv2d: output is %dx%d, the shapes give %dx%d", oh, ow, want_oh, want_ow);
   CINN_RT_CHECK((int64_t)in * ic * ih * iw < INT_MAX && (int64_t)on * oc * oh * ow < INT_MAX, "conv2d: tensor too large");
   CINN_RT_CHECK(fh * dh < 32768 && fw * dw < 32768, "conv2d: filter extent too large");
+  if (format != 0) {
+    // channels-last output; format 2 reads an NCHW input and [OC][IC][KH][KW] weights
+    cinn_hip_kernels::ConvNhwcArgs a;
+    a.x = x->memory, a.w = w->memory, a.y = y->memory;
+    a.scale = scale, a.shift = shift;
+    a.residual       = residual ? residual->memory : (epilogue == 0 && beta != 0.0f ? y->memory : nullptr);
+    a.alpha          = epilogue == 0 ? alpha : 1.0f;
+    a.residual_scale = residual ? 1.0f : beta;
+    a.relu           = epilogue == 2;
+    a.nchw_input     = format == 2;
+    a.n = in, a.h = ih, a.w_in = iw, a.c = ic;
+    a.oc = fn, a.kh = fh, a.kw = fw, a.oh = oh, a.ow = ow;
+    a.pad_h = ph, a.pad_w = pw, a.stride_h = sh, a.stride_w = sw, a.dil_h = dh, a.dil_w = dw;
+    a.type = x->type;
+    CINN_RT_CHECK(groups == 1, "conv2d: the channels-last kernels do not support groups (got %d)", groups);
+    CINN_RT_CHECK(cinn_hip_kernels::ConvNhwcSupported(a), "conv2d: channels-last needs the channel count (%d) to be a multiple of 16 bytes", ic);
+    cinn_hip_kernels::RunConvNhwc(a, stream);
+    return;
+  }
+  CINN_RT_CHECK(residual == nullptr, "conv2d: a residual input needs the channels-last format");
 
   ConvParams p;
   p.n = in, p.c = ic, p.ih = ih, p.iw = iw;
@@ -334,7 +355,7 @@ void cinn_call_cudnn_conv2d_forward(void* v_args, int num_args, int format, floa
                                     int dilation_w, int groups, int output_n, int output_c, int output_h,
                                     int output_w, void* stream) {
   CINN_RT_CHECK(num_args == 3, "cinn_call_cudnn_conv2d_forward takes x, w and y, got %d arguments", num_args);
-  RunConv(BufferArg(v_args, 0), BufferArg(v_args, 1), BufferArg(v_args, 2), nullptr, nullptr, 0, format, alpha, beta,
+  RunConv(BufferArg(v_args, 0), BufferArg(v_args, 1), BufferArg(v_args, 2), nullptr, nullptr, nullptr, 0, format, alpha, beta,
           input_n, input_c, input_h, input_w, filter_n, filter_c, filter_h, filter_w, pad_h, pad_w, stride_h, stride_w,
           dilation_h, dilation_w, groups, output_n, output_c, output_h, output_w, static_cast<hipStream_t>(stream));
 }
@@ -343,13 +364,15 @@ void cinn_call_hip_conv2d_bn_relu(void* v_args, int num_args, int format, int re
                                   int input_h, int input_w, int filter_n, int filter_c, int filter_h, int filter_w,
                                   int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
                                   int groups, int output_n, int output_c, int output_h, int output_w, void* stream) {
-  CINN_RT_CHECK(num_args == 5, "cinn_call_hip_conv2d_bn_relu takes x, w, scale, shift and y, got %d arguments", num_args);
+  CINN_RT_CHECK(num_args == 5 || num_args == 6,
+                "cinn_call_hip_conv2d_bn_relu takes x, w, scale, shift, [residual] and y, got %d arguments", num_args);
   cinn_buffer_t* scale = BufferArg(v_args, 2);
   cinn_buffer_t* shift = BufferArg(v_args, 3);
   CINN_RT_CHECK(scale->type.code == cinn_type_float && scale->type.bits == 32 && shift->type.bits == 32,
                 "cinn_call_hip_conv2d_bn_relu: scale / shift must be fp32");
-  RunConv(BufferArg(v_args, 0), BufferArg(v_args, 1), BufferArg(v_args, 4), reinterpret_cast<const float*>(scale->memory),
-          reinterpret_cast<const float*>(shift->memory), relu ? 2 : 1, format, 1.0f, 0.0f, input_n, input_c, input_h,
+  RunConv(BufferArg(v_args, 0), BufferArg(v_args, 1), BufferArg(v_args, num_args - 1),
+          reinterpret_cast<const float*>(scale->memory), reinterpret_cast<const float*>(shift->memory),
+          num_args == 6 ? BufferArg(v_args, 4) : nullptr, relu ? 2 : 1, format, 1.0f, 0.0f, input_n, input_c, input_h,
           input_w, filter_n, filter_c, filter_h, filter_w, pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w,
           groups, output_n, output_c, output_h, output_w, static_cast<hipStream_t>(stream));
 }

@@ -1,0 +1,33 @@
+// Internal interface between the convolution intrinsics (conv_mfma.hip) and the channels-last MFMA kernels
+// (conv_nhwc_mfma.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "cinn_hip_runtime.h"
+
+namespace cinn_hip_kernels {
+
+struct ConvNhwcArgs {
+  const void* x;         // NHWC activations, or NCHW when nchw_input is set
+  const void* w;         // [OC][KH][KW][IC], or [OC][IC][KH][KW] when nchw_input is set
+  void* y;               // NHWC [N][OH][OW][OC]
+  const float* scale;    // per output channel, may be null (then alpha is used)
+  const float* shift;    // per output channel, may be null
+  const void* residual;  // NHWC tensor of y's shape added before the activation, may be null
+  float alpha;           // used when scale is null
+  float residual_scale;  // factor of the residual (beta of the alpha / beta form)
+  bool relu;
+  bool nchw_input;
+  int n, h, w_in, c;  // input extents
+  int oc, kh, kw;
+  int oh, ow;
+  int pad_h, pad_w, stride_h, stride_w, dil_h, dil_w;
+  cinn_type_t type;  // element type of x, w, y and residual
+};
+
+// true when the channels-last kernels can run this convolution (groups are not supported; the general path needs
+// the input channel count to be a multiple of one 16-byte chunk)
+bool ConvNhwcSupported(const ConvNhwcArgs& a);
+void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream);
+
+}  // namespace cinn_hip_kernels

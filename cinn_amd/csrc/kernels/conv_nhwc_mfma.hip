@@ -1,0 +1,452 @@
+// Channels-last implicit-GEMM convolution for CDNA4 (gfx950) on the MFMA units.
+//
+//   y[pixel][oc] = epilogue( sum_k  im2col(x)[pixel][k] * w[oc][k] )        pixel = (n, oh, ow), k = (dy, dx, c)
+//
+// With NHWC activations and [OC][KH][KW][IC] weights both GEMM operands have the reduction index contiguous in
+// memory, so every lane moves 16-byte chunks: a chunk of the im2col operand is 8 (fp16 / bf16) or 4 (fp32)
+// consecutive channels of one input pixel, present or - outside the image - zero.  Nothing is gathered element
+// by element and no im2col buffer exists.
+//
+//   * block tile BM pixels x BN output channels (128x128, 128x64 or 64x64, chosen per shape so that the grid
+//     fills the 256 CUs), 256 threads = 4 wavefronts in a 2x2 grid, K step of 128 bytes per row;
+//   * operand tiles in LDS as [row][128 bytes], 16-byte chunks XOR-swizzled (conflict-free ds_read_b128 of MFMA
+//     fragments), double buffered with the next step's global loads in flight during the MFMAs;
+//   * v_mfma_f32_32x32x16_{f16,bf16} or v_mfma_f32_32x32x2_f32, fp32 accumulation;
+//   * epilogue staged through LDS so that each lane writes 16 contiguous bytes of one pixel: per-channel affine
+//     (folded batch norm), residual addition and relu are applied there on the fp32 accumulators;
+//   * a second loader reads an NCHW input with few channels (the network stem) directly, k = (c, dy, dx) with dx
+//     padded to a chunk, so that the image never has to be transposed or channel-padded in memory.
+#include <hip/hip_runtime.h>
+
+#include <climits>
+#include <cstdint>
+#include <cstdlib>
+#include <cstring>
+
+#include "kernels/conv_nhwc.h"
+#include "runtime/hip_check.h"
+
+namespace cinn_hip_kernels {
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads  = 256;
+constexpr int kRowBytes = 128;  // one tile row per K step
+
+struct Params {
+  int n, h, w, c;
+  int oc, kh, kw;
+  int oh, ow;
+  int pad_h, pad_w, stride_h, stride_w, dil_h, dil_w;
+  int k_total;  // reduction length as the kernel walks it
+  int kwp;      // NCHW-input loader: KW rounded up to one chunk
+  int pixels;   // n * oh * ow
+  int relu;
+  float alpha, residual_scale;
+};
+
+// byte offset of 16-byte chunk `chunk` (0..7) of row `row` inside an operand tile
+__device__ __forceinline__ int TileOffset(int row, int chunk) {
+  int key = (row ^ (row >> 3)) & 7;
+  return row * kRowBytes + ((chunk ^ key) << 4);
+}
+
+// ---- one K step of MFMAs on a wave tile ---------------------------------------------------------------------
+template <typename T, int TM, int TN>
+struct WaveMma;
+
+template <int TM, int TN>
+struct WaveMma<float, TM, TN> {
+  static __device__ __forceinline__ void Step(const char* a_tile, const char* b_tile, int a_row, int b_row, int lane,
+                                              f32x16 (&acc)[TM][TN]) {
+    const int half = lane >> 5;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      // lanes 0-31 take chunk 2q, lanes 32-63 chunk 2q+1: the two k values of v_mfma_f32_32x32x2_f32 are element e
+      // of each, which permutes k identically for both operands
+      f32x4 a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const f32x4*>(a_tile + TileOffset(a_row + 32 * i, 2 * q + half));
+#pragma unroll
+      for (int j = 0; j < TN; ++j) b[j] = *reinterpret_cast<const f32x4*>(b_tile + TileOffset(b_row + 32 * j, 2 * q + half));
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i][e], b[j][e], acc[i][j], 0, 0, 0);
+    }
+  }
+};
+
+template <typename T>
+struct Half16;
+template <>
+struct Half16<__bf16> {
+  typedef bf16x8 vec8;
+  static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct Half16<_Float16> {
+  typedef f16x8 vec8;
+  static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+template <typename T, int TM, int TN>
+struct WaveMma {
+  typedef typename Half16<T>::vec8 vec8;
+  static __device__ __forceinline__ void Step(const char* a_tile, const char* b_tile, int a_row, int b_row, int lane,
+                                              f32x16 (&acc)[TM][TN]) {
+    const int half = lane >> 5;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      vec8 a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) a[i] = *reinterpret_cast<const vec8*>(a_tile + TileOffset(a_row + 32 * i, 2 * kk + half));
+#pragma unroll
+      for (int j = 0; j < TN; ++j) b[j] = *reinterpret_cast<const vec8*>(b_tile + TileOffset(b_row + 32 * j, 2 * kk + half));
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = Half16<T>::mfma(a[i], b[j], acc[i][j]);
+    }
+  }
+};
+
+// ---- the kernel -----------------------------------------------------------------------------------------------
+template <typename T, int BM, int BN, bool NCHW_IN>
+__global__ void __launch_bounds__(kThreads)
+conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, const float* __restrict__ scale,
+                      const float* __restrict__ shift, const T* residual, Params p) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  constexpr int E      = 16 / sizeof(T);  // elements per chunk
+  constexpr int BK     = 8 * E;           // elements per K step
+  constexpr int A_TILE = BM * kRowBytes;
+  constexpr int STAGE  = (BM + BN) * kRowBytes;
+  constexpr int RA     = BM / 32;  // chunks of the pixel operand per thread and step
+  constexpr int RB     = BN / 32;
+  constexpr int TM     = BM / 64;  // 32x32 MFMA tiles per wavefront
+  constexpr int TN     = BN / 64;
+  constexpr int SLD    = BN + 8;  // row pitch (floats) of the epilogue staging tile
+
+  const int tid  = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm   = wave >> 1;
+  const int wn   = wave & 1;
+
+  // Consecutive workgroup ids go round-robin to the 8 XCDs, each with its own L2: hand every XCD a contiguous band
+  // of tiles, channel tiles fastest, so that blocks sharing a pixel panel share an L2.
+  const int tiles_n = (p.oc + BN - 1) / BN;
+  const int tiles   = ((p.pixels + BM - 1) / BM) * tiles_n;
+  int bid           = blockIdx.x;
+  {
+    const int q = tiles >> 3, r = tiles & 7, xcd = bid & 7;
+    bid = xcd * q + (xcd < r ? xcd : r) + (bid >> 3);
+  }
+  const int m0 = (bid / tiles_n) * BM;
+  const int n0 = (bid % tiles_n) * BN;
+
+  const int cc = tid & 7;   // chunk column this thread loads
+  const int lr = tid >> 3;  // first tile row this thread loads
+
+  // per-row state of the pixel operand
+  int base[RA], ih0[RA], iw0[RA];
+#pragma unroll
+  for (int i = 0; i < RA; ++i) {
+    int m = m0 + lr + 32 * i;
+    if (m < p.pixels) {
+      int n   = m / (p.oh * p.ow);
+      int rem = m - n * (p.oh * p.ow);
+      int oh  = rem / p.ow;
+      int ow  = rem - oh * p.ow;
+      base[i] = n * p.h * p.w * p.c;
+      ih0[i]  = oh * p.stride_h - p.pad_h;
+      iw0[i]  = ow * p.stride_w - p.pad_w;
+    } else {
+      base[i] = 0;
+      ih0[i]  = INT_MIN / 2;  // fails every bounds test
+      iw0[i]  = 0;
+    }
+  }
+  // position of this thread's chunk in the reduction: channel offset and filter tap (channels-last loader)
+  int ck = 0, dy = 0, dx = 0;
+  if (!NCHW_IN) {
+    int kc  = cc * E;
+    int tap = kc / p.c;
+    ck      = kc - tap * p.c;
+    dy      = tap / p.kw;
+    dx      = tap - dy * p.kw;
+  }
+
+  u32x4 ra[RA], rb[RB];
+  auto load_step = [&](int step) {
+    if (!NCHW_IN) {
+      const bool tap_ok = dy < p.kh;
+#pragma unroll
+      for (int i = 0; i < RA; ++i) {
+        int ih  = ih0[i] + dy * p.dil_h;
+        int iw  = iw0[i] + dx * p.dil_w;
+        bool ok = tap_ok && (unsigned)ih < (unsigned)p.h && (unsigned)iw < (unsigned)p.w;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (ok) v = *reinterpret_cast<const u32x4*>(x + base[i] + (ih * p.w + iw) * p.c + ck);
+        ra[i] = v;
+      }
+      const int kb = step * BK + cc * E;
+#pragma unroll
+      for (int i = 0; i < RB; ++i) {
+        int oc  = n0 + lr + 32 * i;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (oc < p.oc && kb < p.k_total) v = *reinterpret_cast<const u32x4*>(w + (int64_t)oc * p.k_total + kb);
+        rb[i] = v;
+      }
+      // advance to the next step
+      ck += BK;
+      while (ck >= p.c) {
+        ck -= p.c;
+        if (++dx == p.kw) {
+          dx = 0;
+          ++dy;
+        }
+      }
+    } else {
+      // k = (c, dy, dx) with dx padded to a chunk: one chunk is E neighbouring taps of one input row
+      const int chunks_per_row = p.kwp / E;
+      const int q              = step * 8 + cc;
+      const int row_id         = q / chunks_per_row;
+      const int dx0            = (q - row_id * chunks_per_row) * E;
+      const int c              = row_id / p.kh;
+      const int ky             = row_id - c * p.kh;
+      const bool c_ok          = c < p.c;
+#pragma unroll
+      for (int i = 0; i < RA; ++i) {
+        T tmp[E];
+        int ih       = ih0[i] + ky * p.dil_h;
+        bool row_ok  = c_ok && (unsigned)ih < (unsigned)p.h;
+        const T* src = x + base[i] + (c * p.h + ih) * p.w;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          int iw  = iw0[i] + (dx0 + e) * p.dil_w;
+          bool ok = row_ok && dx0 + e < p.kw && (unsigned)iw < (unsigned)p.w;
+          tmp[e]  = ok ? src[iw] : (T)0.0f;
+        }
+        __builtin_memcpy(&ra[i], tmp, 16);
+      }
+#pragma unroll
+      for (int i = 0; i < RB; ++i) {
+        T tmp[E];
+        int oc       = n0 + lr + 32 * i;
+        bool row_ok  = c_ok && oc < p.oc;
+        const T* src = w + ((int64_t)(oc * p.c + c) * p.kh + ky) * p.kw;
+#pragma unroll
+        for (int e = 0; e < E; ++e) tmp[e] = (row_ok && dx0 + e < p.kw) ? src[dx0 + e] : (T)0.0f;
+        __builtin_memcpy(&rb[i], tmp, 16);
+      }
+    }
+  };
+  auto store_step = [&](char* stage) {
+#pragma unroll
+    for (int i = 0; i < RA; ++i) *reinterpret_cast<u32x4*>(stage + TileOffset(lr + 32 * i, cc)) = ra[i];
+#pragma unroll
+    for (int i = 0; i < RB; ++i) *reinterpret_cast<u32x4*>(stage + A_TILE + TileOffset(lr + 32 * i, cc)) = rb[i];
+  };
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  const int steps = (p.k_total + BK - 1) / BK;
+  load_step(0);
+  store_step(lds);
+  __syncthreads();
+  const int a_row = wm * (BM / 2) + (lane & 31);
+  const int b_row = wn * (BN / 2) + (lane & 31);
+  for (int s = 0; s < steps; ++s) {
+    char* cur = lds + (s & 1) * STAGE;
+    if (s + 1 < steps) load_step(s + 1);
+    WaveMma<T, TM, TN>::Step(cur, cur + A_TILE, a_row, b_row, lane, acc);
+    if (s + 1 < steps) store_step(lds + ((s + 1) & 1) * STAGE);
+    __syncthreads();
+  }
+
+  // ---- epilogue: accumulators -> LDS (fp32) -> 8 channels of one pixel per lane ----------------------------------
+  float* st = reinterpret_cast<float*>(lds);
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        int row = wm * (BM / 2) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        int col = wn * (BN / 2) + j * 32 + (lane & 31);
+        st[row * SLD + col] = acc[i][j][r];
+      }
+  __syncthreads();
+
+  constexpr int CPR  = BN / 8;          // 8-channel groups per tile row
+  constexpr int ROWS = kThreads / CPR;  // rows per pass
+  const int cg       = tid % CPR;
+  const int oc0      = n0 + cg * 8;
+  if (oc0 >= p.oc) return;
+  float sc[8], sh[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    int oc = oc0 + e < p.oc ? oc0 + e : p.oc - 1;
+    sc[e]  = scale ? scale[oc] : p.alpha;
+    sh[e]  = shift ? shift[oc] : 0.0f;
+  }
+  const bool full = (p.oc & 7) == 0;  // then every group is whole and 16-byte aligned
+#pragma unroll 2
+  for (int row = tid / CPR; row < BM; row += ROWS) {
+    int m = m0 + row;
+    if (m >= p.pixels) break;
+    float v[8];
+    *reinterpret_cast<f32x4*>(&v[0]) = *reinterpret_cast<const f32x4*>(&st[row * SLD + cg * 8]);
+    *reinterpret_cast<f32x4*>(&v[4]) = *reinterpret_cast<const f32x4*>(&st[row * SLD + cg * 8 + 4]);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = v[e] * sc[e] + sh[e];
+    const int64_t off = (int64_t)m * p.oc + oc0;
+    if (full) {
+      T out[8];
+      if (residual) {
+        T rv[8];
+        __builtin_memcpy(rv, residual + off, 8 * sizeof(T));
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] += p.residual_scale * (float)rv[e];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) out[e] = (T)(p.relu ? fmaxf(v[e], 0.0f) : v[e]);
+      __builtin_memcpy(y + off, out, 8 * sizeof(T));
+    } else {
+      for (int e = 0; e < 8 && oc0 + e < p.oc; ++e) {
+        float t = v[e];
+        if (residual) t += p.residual_scale * (float)residual[off + e];
+        y[off + e] = (T)(p.relu ? fmaxf(t, 0.0f) : t);
+      }
+    }
+  }
+}
+
+// ---- host side ------------------------------------------------------------------------------------------------
+struct TileChoice {
+  int bm, bn;
+};
+
+int LdsBytes(int bm, int bn) {
+  int stages  = 2 * (bm + bn) * kRowBytes;
+  int staging = bm * (bn + 8) * 4;
+  return stages > staging ? stages : staging;
+}
+
+// Picks the block tile: the largest one that still gives every CU work in (nearly) every round.  Larger tiles reuse
+// each LDS fragment for more MFMAs; smaller ones keep 256 CUs busy when the layer has few pixels.
+TileChoice ChooseTile(int pixels, int oc) {
+  static const int forced = [] {
+    const char* e = getenv("FLAGS_cinn_hip_conv_tile");
+    return e ? atoi(e) : -1;
+  }();
+  const TileChoice options[3] = {{128, 128}, {128, 64}, {64, 64}};
+  if (forced >= 0 && forced < 3) return options[forced];
+  // relative MFMA rate a tile reaches (LDS fragment reads per MFMA grow as the tile shrinks)
+  const double efficiency[3] = {1.0, 0.8, 0.55};
+  double best                = 0;
+  int pick                   = -1;
+  for (int i = 0; i < 3; ++i) {
+    if (options[i].bn > 64 && oc <= 64) continue;
+    int64_t blocks = (int64_t)((pixels + options[i].bm - 1) / options[i].bm) * ((oc + options[i].bn - 1) / options[i].bn);
+    // blocks the busiest CU works through, times the cost of one block
+    double cost = (double)((blocks + 255) / 256) * options[i].bm * options[i].bn / efficiency[i];
+    if (pick < 0 || cost < best) {
+      best = cost;
+      pick = i;
+    }
+  }
+  return options[pick];
+}
+
+template <typename T, int BM, int BN, bool NCHW_IN>
+void Launch(const ConvNhwcArgs& a, const Params& p, hipStream_t stream) {
+  auto kernel     = conv_nhwc_mfma_kernel<T, BM, BN, NCHW_IN>;
+  const int bytes = LdsBytes(BM, BN);
+  static bool configured = false;
+  if (!configured) {
+    CINN_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+    configured = true;
+  }
+  const int tiles = ((p.pixels + BM - 1) / BM) * ((p.oc + BN - 1) / BN);
+  hipLaunchKernelGGL(kernel, dim3(tiles), dim3(kThreads), bytes, stream, static_cast<const T*>(a.x),
+                     static_cast<const T*>(a.w), static_cast<T*>(a.y), a.scale, a.shift, static_cast<const T*>(a.residual), p);
+  CINN_HIP_CALL(hipGetLastError());
+}
+
+template <typename T>
+void Dispatch(const ConvNhwcArgs& a, const Params& p, hipStream_t stream) {
+  TileChoice t = ChooseTile(p.pixels, p.oc);
+  if (a.nchw_input) {
+    if (t.bm == 128 && t.bn == 128) t.bn = 64;
+    if (t.bm == 128)
+      Launch<T, 128, 64, true>(a, p, stream);
+    else
+      Launch<T, 64, 64, true>(a, p, stream);
+    return;
+  }
+  if (t.bm == 128 && t.bn == 128)
+    Launch<T, 128, 128, false>(a, p, stream);
+  else if (t.bm == 128)
+    Launch<T, 128, 64, false>(a, p, stream);
+  else
+    Launch<T, 64, 64, false>(a, p, stream);
+}
+
+int ChunkElems(const cinn_type_t& t) { return 16 / (t.bits / CHAR_BIT); }
+
+}  // namespace
+
+bool ConvNhwcSupported(const ConvNhwcArgs& a) {
+  const bool is_float = a.type.code == cinn_type_float && (a.type.bits == 32 || a.type.bits == 16);
+  const bool is_bf16  = a.type.code == cinn_type_bfloat && a.type.bits == 16;
+  if (!is_float && !is_bf16) return false;
+  if (a.nchw_input) return true;
+  return a.c % ChunkElems(a.type) == 0;
+}
+
+void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream) {
+  CINN_RT_CHECK(ConvNhwcSupported(a), "conv2d (channels-last): unsupported type or channel count %d", a.c);
+  CINN_RT_CHECK((int64_t)a.n * a.h * a.w_in * a.c < INT_MAX && (int64_t)a.n * a.oh * a.ow * a.oc < INT_MAX,
+                "conv2d (channels-last): tensor too large for 32-bit offsets");
+  Params p;
+  p.n = a.n, p.h = a.h, p.w = a.w_in, p.c = a.c;
+  p.oc = a.oc, p.kh = a.kh, p.kw = a.kw;
+  p.oh = a.oh, p.ow = a.ow;
+  p.pad_h = a.pad_h, p.pad_w = a.pad_w, p.stride_h = a.stride_h, p.stride_w = a.stride_w;
+  p.dil_h = a.dil_h, p.dil_w = a.dil_w;
+  const int e = ChunkElems(a.type);
+  p.kwp       = (a.kw + e - 1) / e * e;
+  p.k_total   = a.nchw_input ? a.c * a.kh * p.kwp : a.kh * a.kw * a.c;
+  p.pixels    = a.n * a.oh * a.ow;
+  p.relu      = a.relu ? 1 : 0;
+  p.alpha     = a.alpha;
+  p.residual_scale = a.residual_scale;
+  if (a.type.code == cinn_type_bfloat) {
+    Dispatch<__bf16>(a, p, stream);
+  } else if (a.type.bits == 16) {
+    Dispatch<_Float16>(a, p, stream);
+  } else {
+    Dispatch<float>(a, p, stream);
+  }
+}
+
+}  // namespace cinn_hip_kernels

@@ -71,6 +71,78 @@ __global__ void __launch_bounds__(256) pool2d_nchw_kernel(const T* __restrict__ 
   out[idx] = (T)v;
 }
 
+
+// Channels-last pooling: one thread per output pixel and group of V consecutive channels (V elements = 16 bytes
+// when the channel count allows), so that every access is one contiguous vector and consecutive lanes read
+// consecutive vectors.  Arithmetic and order of operations are those of the NCHW kernel.
+template <typename T, int V>
+__global__ void __launch_bounds__(256) pool2d_nhwc_kernel(const T* __restrict__ in, T* __restrict__ out, PoolParams p) {
+  const int groups    = p.c / V;
+  const int64_t total = (int64_t)p.n * p.oh * p.ow * groups;
+  const int64_t idx   = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int g         = (int)(idx % groups);
+  const int64_t pixel = idx / groups;
+  const int x         = (int)(pixel % p.ow);
+  const int y         = (int)((pixel / p.ow) % p.oh);
+  const int64_t n     = pixel / ((int64_t)p.ow * p.oh);
+  const T* src        = in + n * p.ih * p.iw * p.c + g * V;
+  const int ys = y * p.sh - p.ph, xs = x * p.sw - p.pw;
+  const bool is_max = p.mode == 0 || p.mode == 3;
+  float acc[V];
+  float factor = (float)(p.kh * p.kw);
+  if (p.mode == 2) {
+    const int y0 = ys > 0 ? ys : 0, x0 = xs > 0 ? xs : 0;
+    const int y1 = ys + p.kh < p.ih ? ys + p.kh : p.ih, x1 = xs + p.kw < p.iw ? xs + p.kw : p.iw;
+    const int count = (y1 - y0) * (x1 - x0);
+    factor          = (float)(count > 1 ? count : 1);
+  }
+#pragma unroll
+  for (int e = 0; e < V; ++e) acc[e] = is_max ? -3.402823466e+38f : 0.0f;
+  for (int ry = 0; ry < p.kh; ++ry) {
+    const int yy = ys + ry;
+    if (yy < 0 || yy >= p.ih) continue;
+    for (int rx = 0; rx < p.kw; ++rx) {
+      const int xx = xs + rx;
+      if (xx < 0 || xx >= p.iw) continue;
+      T v[V];
+      __builtin_memcpy(v, src + ((int64_t)yy * p.iw + xx) * p.c, V * sizeof(T));
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const float f = (float)v[e];
+        if (is_max)
+          acc[e] = f > acc[e] ? f : acc[e];
+        else
+          acc[e] += f / factor;
+      }
+    }
+  }
+  T* dst = out + pixel * p.c + g * V;
+  T res[V];
+  if (p.beta != 0.0f) __builtin_memcpy(res, dst, V * sizeof(T));
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    float r = p.alpha * acc[e];
+    if (p.beta != 0.0f) r += p.beta * (float)res[e];
+    res[e] = (T)r;
+  }
+  __builtin_memcpy(dst, res, V * sizeof(T));
+}
+
+template <typename T>
+void LaunchPoolNhwc(const void* x, void* y, const PoolParams& p, hipStream_t s) {
+  constexpr int V = 16 / sizeof(T);
+  if (p.c % V == 0) {
+    const int64_t total = (int64_t)p.n * p.oh * p.ow * (p.c / V);
+    hipLaunchKernelGGL((pool2d_nhwc_kernel<T, V>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+                       static_cast<const T*>(x), static_cast<T*>(y), p);
+  } else {
+    const int64_t total = (int64_t)p.n * p.oh * p.ow * p.c;
+    hipLaunchKernelGGL((pool2d_nhwc_kernel<T, 1>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+                       static_cast<const T*>(x), static_cast<T*>(y), p);
+  }
+}
+
 // block-wide reduction helper over 256 threads
 template <typename OP>
 __device__ __forceinline__ float BlockReduce(float v, float* scratch, OP op) {
@@ -134,7 +206,7 @@ void cinn_call_cudnn_pool2d_forward(void* v_args, int num_args, int mode, int fo
                                     int pad_h, int pad_w, int stride_h, int stride_w, int output_n, int output_c,
                                     int output_h, int output_w, void* stream) {
   CINN_RT_CHECK(num_args == 2, "cinn_call_cudnn_pool2d_forward takes x and y, got %d arguments", num_args);
-  CINN_RT_CHECK(format == 0, "pool2d: only NCHW (format 0) is implemented, got format %d", format);
+  CINN_RT_CHECK(format == 0 || format == 1, "pool2d: unknown tensor format %d", format);
   CINN_RT_CHECK(mode >= 0 && mode <= 3, "pool2d: unknown pooling mode %d", mode);
   CINN_RT_CHECK(output_n == input_n && output_c == input_c, "pool2d: batch / channel mismatch");
   CINN_RT_CHECK(kernel_h > 0 && kernel_w > 0 && stride_h > 0 && stride_w > 0 && output_h > 0 && output_w > 0,
@@ -150,6 +222,15 @@ void cinn_call_cudnn_pool2d_forward(void* v_args, int num_args, int mode, int fo
   CINN_RT_CHECK((int64_t)input_c * input_h * input_w * input_n < INT_MAX && total < INT_MAX, "pool2d: tensor too large");
   dim3 grid((unsigned)((total + 255) / 256));
   auto s = static_cast<hipStream_t>(stream);
+  if (format == 1) {
+    switch (ElemOf(x)) {
+      case Elem::kF32: LaunchPoolNhwc<float>(x->memory, y->memory, p, s); break;
+      case Elem::kF16: LaunchPoolNhwc<_Float16>(x->memory, y->memory, p, s); break;
+      case Elem::kBF16: LaunchPoolNhwc<__bf16>(x->memory, y->memory, p, s); break;
+    }
+    CINN_HIP_CALL(hipGetLastError());
+    return;
+  }
   switch (ElemOf(x)) {
     case Elem::kF32:
       hipLaunchKernelGGL(pool2d_nchw_kernel<float>, grid, dim3(256), 0, s, reinterpret_cast<const float*>(x->memory),

@@ -33,6 +33,12 @@ class Variable(object):
     def __str__(self):
         return self.id
 
+    def set_const(self, is_const=True):
+        """Marks a fed input whose data stays the same between executions (weights): operators that only depend
+        on such inputs run once, before the first execution (cinn/frontend/syntax.h:81-87)."""
+        _lib.check(_lib.load().cinn_amd_builder_set_const(self._builder._handle, self.id.encode(), int(bool(is_const))))
+        return self
+
     def __repr__(self):
         return "Variable(%s, %s, %s)" % (self.id, self._shape, self._dtype)
 
@@ -326,6 +332,11 @@ class Computation(object):
 
     def execute(self):
         _lib.check(_lib.load().cinn_amd_computation_execute(self._handle))
+
+    def pre_run(self):
+        """Runs the pre-run instructions again; needed after the data of a const input was replaced (the first
+        execute runs them by itself)."""
+        _lib.check(_lib.load().cinn_amd_computation_pre_run(self._handle))
 
     def execute_graph(self):
         _lib.check(_lib.load().cinn_amd_computation_execute_graph(self._handle))

@@ -37,6 +37,9 @@ int cinn_amd_builder_call(cinn_amd_builder_t b, const char* method, const char* 
 /* shape / dtype of a variable known to the builder; rank_out receives the rank, shape_out up to 8 dims */
 int cinn_amd_builder_var_info(cinn_amd_builder_t b, const char* id, int32_t* shape_out, int32_t* rank_out,
                               char* dtype_out, size_t dtype_cap);
+/* Variable::set_const (cinn/frontend/syntax.h:81-87): marks an input whose data does not change between executions
+ * (weights).  Operators fed by const values only run once, ahead of the first execution. */
+int cinn_amd_builder_set_const(cinn_amd_builder_t b, const char* id, int32_t is_const);
 int cinn_amd_builder_size(cinn_amd_builder_t b, int32_t* num_instructions);
 /* textual listing of the program built so far */
 int cinn_amd_builder_program_string(cinn_amd_builder_t b, char* out, size_t cap, size_t* needed);
@@ -51,6 +54,9 @@ int cinn_amd_computation_build_and_compile(cinn_amd_builder_t b, const char* con
 int cinn_amd_computation_destroy(cinn_amd_computation_t c);
 int cinn_amd_computation_execute(cinn_amd_computation_t c);
 int cinn_amd_computation_execute_graph(cinn_amd_computation_t c);
+/* Program::PreRun (cinn/hlir/framework/graph_compiler.cc:78-87): runs the pre-run instructions.  The first
+ * execute does it by itself; call it again after replacing the data of a const input. */
+int cinn_amd_computation_pre_run(cinn_amd_computation_t c);
 int cinn_amd_computation_num_instructions(cinn_amd_computation_t c, int32_t* n);
 /* SetTensorData / GetTensorData: synchronous host <-> device copies of exactly the tensor's byte size */
 int cinn_amd_computation_set_tensor(cinn_amd_computation_t c, const char* name, const void* data, size_t bytes);

@@ -93,9 +93,10 @@ CONFIG4 = [("64->64 3x3 s1 p1 56x56", 64, 64, 3, 1, 1, 56), ("256->512 1x1 s2 56
            ("512->512 3x3 s1 p1 14x14", 512, 512, 3, 1, 1, 14)]
 
 
+@pytest.mark.parametrize("nhwc", [True, False])
 @pytest.mark.parametrize("dtype", ["float32", "float16"])
 @pytest.mark.parametrize("name,ic,oc,k,s,p,hw", CONFIG4)
-def test_config4_conv_bn_relu_batch32(gpu, dtype, name, ic, oc, k, s, p, hw):
+def test_config4_conv_bn_relu_batch32(gpu, dtype, name, ic, oc, k, s, p, hw, nhwc):
     rng = np.random.default_rng(400 + ic + oc + k)
     x = rng.standard_normal((32, ic, hw, hw)).astype(dtype)
     w = (rng.standard_normal((oc, ic, k, k)) * np.sqrt(2.0 / (ic * k * k))).astype(dtype)
@@ -109,9 +110,10 @@ def test_config4_conv_bn_relu_batch32(gpu, dtype, name, ic, oc, k, s, p, hw):
     S, Bi, M, V = [b.create_input(T, [oc], nm) for nm in ("scale", "bias", "mean", "var")]
     conv = b.conv2d(X, W, strides=[s, s], paddings=[p, p])
     y = b.relu(b.batchnorm(conv, S, Bi, M, V, epsilon=1e-5)[0])
-    (got_conv, got), comp = run(b, {X: x, W: w, S: scale, Bi: bias, M: mean, V: var}, [conv, y])
-    # conv (MFMA) + per-channel sqrt + one fused bn/relu kernel
-    assert comp.num_instructions() == 3, comp.fusion_groups()
+    (got_conv, got), comp = run(b, {X: x, W: w, S: scale, Bi: bias, M: mean, V: var}, [conv, y], conv_layout_nhwc=nhwc)
+    # conv (MFMA) + per-channel sqrt + one fused bn/relu kernel; the channels-last form adds the transposes of x and
+    # w and one back to NCHW for the fetched convolution output (the one of y is fused into the bn/relu kernel)
+    assert comp.num_instructions() == (6 if nhwc else 3), comp.fusion_groups()
     sample = [0, 17, 31]
     want_conv = oracle.conv2d_nchw(x[sample], w, (s, s), (p, p))
     want = oracle.batch_norm_relu_nchw(want_conv, scale, bias, mean, var, 1e-5, relu=True)
@@ -131,7 +133,7 @@ def test_config4_conv_bn_relu_batch32(gpu, dtype, name, ic, oc, k, s, p, hw):
     x2[5] = x2[29]
     b2 = NetBuilder("cfg4b")
     X2, W2 = b2.create_input(T, x.shape, "x"), b2.create_input(T, w.shape, "w")
-    (c2,), _ = run(b2, {X2: x2, W2: w}, [b2.conv2d(X2, W2, strides=[s, s], paddings=[p, p])])
+    (c2,), _ = run(b2, {X2: x2, W2: w}, [b2.conv2d(X2, W2, strides=[s, s], paddings=[p, p])], conv_layout_nhwc=nhwc)
     assert np.array_equal(c2[5], c2[29]) and np.array_equal(c2[29], got_conv[29])
 
 

@@ -39,9 +39,9 @@ def oracle_forward(params, x):
     return (logits + params["fc_b"]).astype(dt)
 
 
-def gpu_forward(params, x, **options):
+def gpu_forward(params, x, const_params=True, **options):
     b = NetBuilder("resnet50")
-    X, pv, logits = rn.build_resnet50(b, x.shape[0], x.dtype.name, params)
+    X, pv, logits = rn.build_resnet50(b, x.shape[0], x.dtype.name, params, const_params=const_params)
     feeds = {X: x}
     feeds.update({pv[k]: v for k, v in params.items()})
     (out,), comp = run(b, feeds, [logits], **options)
@@ -58,6 +58,10 @@ def test_resnet50_fp32_batch2_matches_oracle(gpu):
     scale = np.abs(want).max()
     assert np.abs(got - want).max() <= 1e-4 * scale, (np.abs(got - want).max(), scale)
     assert np.array_equal(np.argsort(got, 1)[:, -5:], np.argsort(want, 1)[:, -5:])
+    # the same network in the layout it was written in (NCHW kernels), and with nothing marked const
+    for options in ({"conv_layout_nhwc": False}, {"const_params": False}):
+        other, _ = gpu_forward(params, x, **options)
+        assert np.abs(other - want).max() <= 1e-4 * scale, options
 
 
 def test_resnet50_fp16_batch2_matches_oracle(gpu):
@@ -125,3 +129,35 @@ def test_resnet50_hip_graph_replay_matches_eager(gpu):
         comp.execute_graph()
         stream.synchronize()
         assert np.array_equal(comp.get_tensor(comp.output_names()[0]).numpy(), eager)
+
+
+def test_const_weights_are_prepared_once_and_pre_run_refreshes_them(gpu):
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((2, 16, 12, 12)).astype(np.float32)
+    w1 = rng.standard_normal((24, 16, 3, 3)).astype(np.float32)
+    w2 = rng.standard_normal((24, 16, 3, 3)).astype(np.float32)
+    var = rng.uniform(0.5, 1.5, 24).astype(np.float32)
+    ones, zeros = np.ones(24, np.float32), np.zeros(24, np.float32)
+    b = NetBuilder("prerun")
+    from cinn_amd.common import Float
+    X = b.create_input(Float(32), x.shape, "x")
+    W = b.create_input(Float(32), w1.shape, "w").set_const()
+    P = [b.create_input(Float(32), [24], n).set_const() for n in ("scale", "bias", "mean", "var")]
+    y = b.relu(b.batchnorm(b.conv2d(X, W, strides=[1, 1], paddings=[1, 1]), *P)[0])
+    (got,), comp = run(b, {X: x, W: w1, P[0]: ones, P[1]: zeros, P[2]: zeros, P[3]: var}, [y])
+    groups = comp.fusion_groups()
+    assert "pre_run { transpose }" in groups and "pre_run { fill_constant elementwise_add sqrt }" in groups
+    # input to channels-last, convolution, batch norm + relu fused with the transpose back to NCHW
+    assert comp.num_instructions() == 3, groups
+
+    def want(w):
+        return oracle.batch_norm_relu_nchw(oracle.conv2d_nchw(x, w, (1, 1), (1, 1)), ones, zeros, zeros, var, 1e-5, relu=True)
+
+    np.testing.assert_allclose(got, want(w1), rtol=1e-4, atol=1e-4)
+    # new filter data is only picked up once the pre-run instructions have run again
+    comp.get_tensor("w").from_numpy(w2)
+    comp.execute()
+    np.testing.assert_allclose(comp.get_tensor(y.id).numpy(), want(w1), rtol=1e-4, atol=1e-4)
+    comp.pre_run()
+    comp.execute()
+    np.testing.assert_allclose(comp.get_tensor(y.id).numpy(), want(w2), rtol=1e-4, atol=1e-4)
