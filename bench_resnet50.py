@@ -146,4 +146,5 @@ if __name__ == "__main__":
     import json
     import sys
     dtype = sys.argv[1] if len(sys.argv) > 1 else "float16"
-    print(json.dumps(measure(dtype=dtype)))
+    options = dict(kv.split("=") for kv in sys.argv[2:])
+    print(json.dumps(measure(dtype=dtype, **{k: int(v) for k, v in options.items()})))

@@ -40,7 +40,7 @@ std::shared_ptr<CinnComputation> CinnComputation::Compile(const common::Target& 
   }
   for (auto& in : program.GetInputs()) comp->input_names_.push_back(in->id);
 
-  Program lowered = program;
+  Program lowered = PretransposeConstMatmulWeights(program);
   if (options.conv_layout_nhwc) lowered = ConvertConvLayoutToNHWC(lowered, fetch_ids);
   if (options.fuse_conv_bn_relu) lowered = FuseConvBatchNorm(lowered, fetch_ids);
   if (options.use_decomposer) lowered = ApplyDecomposer(lowered);

@@ -242,12 +242,40 @@ Program ConvertConvLayoutToNHWC(const Program& program, const std::set<std::stri
   return LayoutConverter(program, fetch_ids).Run();
 }
 
+Program PretransposeConstMatmulWeights(const Program& program) {
+  std::vector<Instruction> out;
+  Emitter emit(&out, "wt_");
+  std::map<std::string, Variable> transposed;
+  for (auto& ins : program.instructions()) {
+    if (ins->op_type == "matmul" && ins->inputs.size() == 2 && ins->inputs[1]->is_const &&
+        ins->inputs[1]->shape.size() == 2 && !GetAttr<bool>(ins->attrs, "trans_b", false)) {
+      auto w  = ins->inputs[1];
+      auto it = transposed.find(w->id);
+      if (it == transposed.end())
+        it = transposed.emplace(w->id, emit.Emit1("transpose", {w}, {{"axis", ShapeType{1, 0}}})).first;
+      AttributeMap attrs = ins->attrs;
+      attrs["trans_b"]   = true;
+      Instruction m("matmul");
+      m->inputs  = {ins->inputs[0], it->second};
+      m->attrs   = attrs;
+      m->outputs = ins->outputs;
+      out.push_back(m);
+    } else {
+      out.push_back(ins);
+    }
+  }
+  return Program(std::move(out), program.GetInputs(), program.name());
+}
+
 Program FuseConvBatchNorm(const Program& program, const std::set<std::string>& fetch_ids) {
   const auto& instrs = program.instructions();
   // consumers of every variable
   std::map<std::string, std::vector<size_t>> users;
   for (size_t i = 0; i < instrs.size(); ++i)
     for (auto& in : instrs[i]->inputs) users[in->id].push_back(i);
+  std::map<std::string, size_t> defined_at;
+  for (size_t i = 0; i < instrs.size(); ++i)
+    for (auto& o : instrs[i]->outputs) defined_at[o->id] = i;
   auto single_user = [&](const Variable& v) -> int {
     if (fetch_ids.count(v->id)) return -1;
     auto it = users.find(v->id);
@@ -272,10 +300,14 @@ Program FuseConvBatchNorm(const Program& program, const std::set<std::string>& f
     Variable residual;
     bool relu = false;
     int next  = single_user(result);
-    if (next >= 0 && instrs[next]->op_type == "elementwise_add" && instrs[next]->inputs.size() == 2) {
+    if (next >= 0 && !dropped[next] && instrs[next]->op_type == "elementwise_add" && instrs[next]->inputs.size() == 2) {
       auto& add     = instrs[next];
       Variable other = add->inputs[0] == result ? add->inputs[1] : add->inputs[0];
-      if (!(other == result) && other->shape == result->shape) {
+      // the other operand must exist when this convolution's inputs do: of two convolution branches meeting in an
+      // addition, the later one takes the addition
+      auto def          = defined_at.find(other->id);
+      bool other_earlier = def == defined_at.end() || def->second < i;
+      if (!(other == result) && other->shape == result->shape && other_earlier) {
         residual = other;
         dropped[next] = true;
         last     = next;
@@ -283,7 +315,7 @@ Program FuseConvBatchNorm(const Program& program, const std::set<std::string>& f
         next     = single_user(result);
       }
     }
-    if (next >= 0 && instrs[next]->op_type == "relu") {
+    if (next >= 0 && !dropped[next] && instrs[next]->op_type == "relu") {
       relu          = true;
       dropped[next] = true;
       last          = next;

@@ -23,6 +23,9 @@ namespace frontend {
 
 Program ConvertConvLayoutToNHWC(const Program& program, const std::set<std::string>& fetch_ids);
 Program FuseConvBatchNorm(const Program& program, const std::set<std::string>& fetch_ids);
+// matmul(x, W) with a const 2-D W stored [K][N]: multiply by a pre-run transposed copy instead (trans_b), so that
+// both operands of the GEMM kernel have K contiguous whatever the sizes of x
+Program PretransposeConstMatmulWeights(const Program& program);
 
 }  // namespace frontend
 }  // namespace cinn

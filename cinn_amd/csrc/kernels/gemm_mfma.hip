@@ -18,6 +18,7 @@
 #include <cstdint>
 
 #include "cinn_hip_runtime.h"
+#include "kernels/conv_nhwc.h"
 #include "runtime/hip_check.h"
 
 namespace {
@@ -464,6 +465,34 @@ void RunGemm(const GemmProblem& p, hipStream_t stream) {
   CINN_RT_CHECK(p.batch <= 65535, "gemm: batch %d exceeds the grid limit", p.batch);
   const bool fast16 = !ForceGeneric() && p.m % kBM == 0 && p.n % kBN == 0 && p.k % kBK == 0;
   const bool fast32 = !ForceGeneric() && p.m % kF32Tile == 0 && p.n % kF32Tile == 0 && p.k % kF32K == 0;
+  // Ragged shapes whose operands are both K-contiguous (A [m,k], B stored [n,k]) go to the channels-last
+  // convolution kernels: a 1x1 convolution over m "pixels" is this GEMM, and those kernels bound-check every tile
+  // edge and pick a tile that fills the chip for small m or n.
+  const int elem_bytes = p.type == GemmType::kF32 ? 4 : (p.type == GemmType::kF64 ? 8 : 2);
+  const bool tile_fit  = p.type == GemmType::kF32 ? fast32 : fast16;
+  if (!ForceGeneric() && !tile_fit && p.type != GemmType::kF64 && !p.trans_a && p.trans_b && p.k % (16 / elem_bytes) == 0) {
+    for (int b = 0; b < p.batch; ++b) {
+      cinn_hip_kernels::ConvNhwcArgs a;
+      a.x = static_cast<const char*>(p.a) + (int64_t)b * p.stride_a * elem_bytes;
+      a.w = static_cast<const char*>(p.b) + (int64_t)b * p.stride_b * elem_bytes;
+      a.y = static_cast<char*>(p.c) + (int64_t)b * p.stride_c * elem_bytes;
+      a.scale = a.shift = nullptr;
+      a.residual        = p.beta != 0.0f ? a.y : nullptr;
+      a.alpha           = p.alpha;
+      a.residual_scale  = p.beta;
+      a.relu            = false;
+      a.nchw_input      = false;
+      a.n = 1, a.h = 1, a.w_in = p.m, a.c = p.k;
+      a.oc = p.n, a.kh = 1, a.kw = 1, a.oh = 1, a.ow = p.m;
+      a.pad_h = a.pad_w = 0;
+      a.stride_h = a.stride_w = a.dil_h = a.dil_w = 1;
+      a.type.code  = p.type == GemmType::kBF16 ? cinn_type_bfloat : cinn_type_float;
+      a.type.bits  = static_cast<uint8_t>(elem_bytes * CHAR_BIT);
+      a.type.lanes = 1;
+      cinn_hip_kernels::RunConvNhwc(a, stream);
+    }
+    return;
+  }
   switch (p.type) {
     case GemmType::kBF16:
       if (fast16) {

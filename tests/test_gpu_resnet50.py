@@ -59,7 +59,7 @@ def test_resnet50_fp32_batch2_matches_oracle(gpu):
     assert np.abs(got - want).max() <= 1e-4 * scale, (np.abs(got - want).max(), scale)
     assert np.array_equal(np.argsort(got, 1)[:, -5:], np.argsort(want, 1)[:, -5:])
     # the same network in the layout it was written in (NCHW kernels), and with nothing marked const
-    for options in ({"conv_layout_nhwc": False}, {"const_params": False}):
+    for options in ({"conv_layout_nhwc": False}, {"const_params": False}, {"fuse_conv_bn_relu": True}):
         other, _ = gpu_forward(params, x, **options)
         assert np.abs(other - want).max() <= 1e-4 * scale, options
 
@@ -73,6 +73,10 @@ def test_resnet50_fp16_batch2_matches_oracle(gpu):
     scale = np.abs(want).max()
     # 53 half-precision layers: 1e-2 of the logit scale
     assert np.abs(got.astype(np.float64) - want).max() <= 1e-2 * scale, (np.abs(got - want).max(), scale)
+    fused, comp = gpu_forward(params, x, fuse_conv_bn_relu=True)
+    # every batch norm, residual addition and relu now lives in a convolution epilogue
+    assert comp.num_instructions() == 53 + 2 + 3, comp.fusion_groups()
+    assert np.abs(fused.astype(np.float64) - want).max() <= 1e-2 * scale
 
 
 def torch_forward(params, x):
