@@ -16,8 +16,8 @@ One JSON line is printed; besides the contract fields it carries
   cpu_baseline - the CPU oracle (a port of the reference's compute definitions, OpenMP) timed on this
                  box's host cores on the same workload
   kernels      - per-kernel event timings of the step
-  extra        - configs[0] (relu(add)) latency, the scaled element-wise streaming rate and, when the
-                 MFMA GEMM is built, configs[2] TFLOP/s
+  extra        - configs[0] (relu(add)) latency, the scaled element-wise streaming rate, configs[2] GEMM TFLOP/s and
+                 configs[4] ResNet-50 images/s
 """
 import argparse
 import json
@@ -166,11 +166,12 @@ def extra_measurements(stream, runtime):
     comp.get_tensor("x").from_numpy(np.ones(n, np.float32))
     ms = time_comp(comp, 20)
     out["copy_256MiB"] = dict(us=round(ms * 1e3, 2), GBps=round(2 * 4 * n / ms / 1e6, 1), bytes=2 * 4 * n)
-    try:
-        import bench_gemm  # optional: configs[2], present once the MFMA GEMM is built
-        out.update(bench_gemm.measure(stream, runtime))
-    except ImportError:
-        pass
+    import bench_gemm  # configs[2]
+    out.update(bench_gemm.measure(stream, runtime))
+    import bench_resnet50  # configs[4]: whole-network images/s, HIP-graph replay of the compiled program
+    for dtype in ("float16", "float32"):
+        r = bench_resnet50.measure(batch=32, dtype=dtype, steps=20, warmup=3, fuse_conv_bn_relu=True)
+        out[r.pop("workload")] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in r.items()}
     return out
 
 

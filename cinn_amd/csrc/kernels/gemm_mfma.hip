@@ -2,8 +2,10 @@
 //
 //   C[M,N] = alpha * op(A)[M,K] * op(B)[K,N] + beta * C          (row-major, optional batch)
 //
-// Three kernels:
-//   * gemm16_mfma_kernel  - bf16 / fp16 inputs, fp32 accumulation on v_mfma_f32_32x32x16_{bf16,f16}.
+// Four kernels:
+//   * gemm16_dma_kernel   - bf16 / fp16 with A stored [M][K] (the common case): 256x256x64 tile, 512 threads, direct
+//     global -> LDS loads, transposing LDS reads for row-major B; see the comment at the kernel.
+//   * gemm16_mfma_kernel  - bf16 / fp16 inputs, any operand layout (used for transposed A), fp32 accumulation on v_mfma_f32_32x32x16_{bf16,f16}.
 //     256x256 block tile, 64-deep K step, 256 threads = 4 wavefronts in a 2x2 grid, each wavefront owning a
 //     128x128 tile (16 MFMA accumulator tiles = 256 accumulator registers).  Both operand tiles live in LDS
 //     as [row][k] with k contiguous, 128 bytes per row, double buffered (2 x 64 KiB of the 160 KiB per CU);
@@ -203,6 +205,176 @@ gemm16_mfma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ 
       }
     }
   }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// bf16 / fp16 with A stored [M][K]: direct global -> LDS loads (global_load_lds_dwordx4), 8 wavefronts.
+// 256x256x64 block tile, 512 threads in a 2 (M) x 4 (N) wavefront grid, each wavefront a 128x64 tile (8 MFMA
+// accumulators), two wavefronts per SIMD so that one runs MFMAs while the other waits for LDS or the barrier.
+// A lane of a load instruction writes its 16 bytes at LDS base + 16 * lane, so the swizzle that makes the fragment
+// reads conflict free is applied on the global side: each lane fetches the chunk that belongs at its LDS slot.
+// B stored [K][N] (the plain row-major matmul) is kept as [k][n] in LDS and read with ds_read_b64_tr_b16, which
+// hands every lane four consecutive k of one column - no transposition in registers.  Two LDS stages of 64 KiB in
+// two separate arrays: the loads of step k+1 are in flight during the MFMAs of step k, and the compiler can tell
+// that they do not alias the stage being read.  Fragment reads are issued one MFMA group ahead.
+// Measured on MI355X the direct-to-LDS path sustains about 27 bytes per clock and CU - close to the 32 a 256x256
+// tile needs at the full MFMA rate - which is what bounds this kernel (about 1.0 PFLOP/s at 4096^3).
+// ---------------------------------------------------------------------------------------------------
+constexpr int kDmaThreads = 512;
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ void AsyncCopy16(const void* src, char* lds_base_uniform) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                   (__attribute__((address_space(3))) void*)lds_base_uniform, 16, 0, 0);
+}
+
+template <typename T, bool B_KC>
+__global__ void __launch_bounds__(kDmaThreads)
+gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ C, int M, int N,
+                  int K, int64_t lda, int64_t ldb, int64_t ldc, float alpha, float beta, int64_t stride_a,
+                  int64_t stride_b, int64_t stride_c) {
+  __shared__ __attribute__((aligned(1024))) char s0[kStageBytes];
+  __shared__ __attribute__((aligned(1024))) char s1[kStageBytes];
+  typedef typename Half16<T>::vec8 vec8;
+  const int tid  = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm   = wave >> 2;
+  const int wn   = wave & 3;
+
+  const int tiles_n = N / kBN;
+  const int tiles   = (M / kBM) * tiles_n;
+  int bid           = blockIdx.x;
+  if ((tiles & 7) == 0) bid = (bid & 7) * (tiles >> 3) + (bid >> 3);
+  const int m0 = (bid / tiles_n) * kBM;
+  const int n0 = (bid % tiles_n) * kBN;
+  A += (int64_t)blockIdx.y * stride_a;
+  B += (int64_t)blockIdx.y * stride_b;
+  C += (int64_t)blockIdx.y * stride_c;
+
+  // Each wavefront issues 4 loads per operand and step; load q = 4 wave + t fills LDS bytes [1024 q, 1024 q + 1024)
+  // of the operand tile: 8 rows of a [row][64 halves] tile, or 2 k-rows of a [k][256 halves] tile.
+  const uint16_t* a_src[4];
+  const uint16_t* b_src[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int q   = wave * 4 + t;
+    const int row = 8 * q + (lane >> 3);
+    const int key = (row ^ (row >> 3)) & 7;
+    a_src[t]      = A + (int64_t)(m0 + row) * lda + (((lane & 7) ^ key) << 3);
+    if (B_KC) {
+      b_src[t] = B + (int64_t)(n0 + row) * ldb + (((lane & 7) ^ key) << 3);
+    } else {
+      const int krow  = 2 * q + (lane >> 5);
+      const int chunk = (lane & 31) ^ (2 * (krow & 3));
+      b_src[t]        = B + (int64_t)krow * ldb + n0 + (chunk << 3);
+    }
+  }
+  const int64_t b_step = B_KC ? kBK : (int64_t)kBK * ldb;
+  auto issue = [&](char* stage, int kt) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) AsyncCopy16(a_src[t] + (int64_t)kt * kBK, stage + (wave * 4 + t) * 1024);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) AsyncCopy16(b_src[t] + kt * b_step, stage + kTileBytes + (wave * 4 + t) * 1024);
+  };
+
+  f32x16 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  const int frag_row = lane & 31;
+  const int frag_kg  = lane >> 5;
+  auto load_frags = [&](const char* cur, int kk, vec8 (&af)[4], vec8 (&bf)[2]) {
+    const char* a_tile = cur;
+    const char* b_tile = cur + kTileBytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      af[i] = *reinterpret_cast<const vec8*>(a_tile + TileOffset(wm * 128 + i * 32 + frag_row, kk * 2 + frag_kg));
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      if (B_KC) {
+        bf[j] = *reinterpret_cast<const vec8*>(b_tile + TileOffset(wn * 64 + j * 32 + frag_row, kk * 2 + frag_kg));
+      } else {
+        // one transposing read returns k = kb .. kb+3 of column n to the lane that owns n: lane j of each group of
+        // 16 supplies the address of row kb + j/4, columns nb + 4 (j%4) .. +3
+        s16x4 part[2];
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+          const int k   = kk * 16 + 4 * (2 * frag_kg + r) + ((lane & 15) >> 2);
+          const int n   = wn * 64 + j * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+          const int off = k * 512 + (((n >> 3) ^ (2 * (k & 3))) << 4) + (n & 7) * 2;
+          part[r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(b_tile + off));
+        }
+        s16x8 both = __builtin_shufflevector(part[0], part[1], 0, 1, 2, 3, 4, 5, 6, 7);
+        bf[j]      = __builtin_bit_cast(vec8, both);
+      }
+    }
+  };
+  auto mma = [&](vec8 (&af)[4], vec8 (&bf)[2]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = Half16<T>::mfma(af[i], bf[j], acc[i][j]);
+  };
+  // fragments of the next 16-deep slice are requested before the MFMAs of the current one are issued; the scheduling
+  // barriers keep the compiler from sinking the reads back to their uses
+  auto compute = [&](const char* cur) {
+    vec8 a0[4], b0[2], a1[4], b1[2];
+    load_frags(cur, 0, a0, b0);
+    __builtin_amdgcn_sched_barrier(0);
+    load_frags(cur, 1, a1, b1);
+    __builtin_amdgcn_sched_barrier(0);
+    mma(a0, b0);
+    __builtin_amdgcn_sched_barrier(0);
+    load_frags(cur, 2, a0, b0);
+    __builtin_amdgcn_sched_barrier(0);
+    mma(a1, b1);
+    __builtin_amdgcn_sched_barrier(0);
+    load_frags(cur, 3, a1, b1);
+    __builtin_amdgcn_sched_barrier(0);
+    mma(a0, b0);
+    __builtin_amdgcn_sched_barrier(0);
+    mma(a1, b1);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  const int nk = K / kBK;
+  issue(s0, 0);
+  for (int kt = 0; kt < nk; kt += 2) {
+    // every load of this wavefront has landed; after the barrier so have everybody's, and nobody still reads the
+    // other stage
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+    if (kt + 1 < nk) issue(s1, kt + 1);
+    compute(s0);
+    if (kt + 1 < nk) {
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      __syncthreads();
+      if (kt + 2 < nk) issue(s0, kt + 2);
+      compute(s1);
+    }
+  }
+
+  T* Ct = reinterpret_cast<T*>(C);
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + wm * 128 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        T* dst  = Ct + (int64_t)row * ldc + col;
+        float v = alpha * acc[i][j][r];
+        if (beta != 0.0f) v += beta * (float)*dst;
+        *dst = (T)v;
+      }
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -417,9 +589,31 @@ void LaunchFast16(const GemmProblem& p, hipStream_t stream) {
                      (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c);
 }
 
+template <typename T, bool B_KC>
+void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
+  int64_t ldb = p.trans_b ? p.k : p.n;
+  dim3 grid((p.m / kBM) * (p.n / kBN), p.batch, 1);
+  hipLaunchKernelGGL((gemm16_dma_kernel<T, B_KC>), grid, dim3(kDmaThreads), 0, stream, static_cast<const uint16_t*>(p.a),
+                     static_cast<const uint16_t*>(p.b), static_cast<uint16_t*>(p.c), p.m, p.n, p.k, (int64_t)p.k, ldb,
+                     (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c);
+}
+
+bool UseRegisterStaging() {
+  static const bool on = getenv("FLAGS_cinn_hip_gemm_register_staging") && atoi(getenv("FLAGS_cinn_hip_gemm_register_staging")) != 0;
+  return on;
+}
+
 template <typename T>
 void DispatchFast16(const GemmProblem& p, hipStream_t stream) {
   bool a_kc = !p.trans_a, b_kc = p.trans_b;
+  if (a_kc && !UseRegisterStaging()) {
+    if (b_kc) {
+      LaunchDma16<T, true>(p, stream);
+    } else {
+      LaunchDma16<T, false>(p, stream);
+    }
+    return;
+  }
   if (a_kc && b_kc) LaunchFast16<T, true, true>(p, stream);
   if (a_kc && !b_kc) LaunchFast16<T, true, false>(p, stream);
   if (!a_kc && b_kc) LaunchFast16<T, false, true>(p, stream);
