@@ -12,7 +12,8 @@
 //     16-byte chunks are XOR-swizzled so that the ds_read_b128 of MFMA fragments and the transposing stores
 //     are conflict free.  Operands whose contiguous axis is not K (row-major B, transposed A) are transposed
 //     in registers (8x8 blocks of 16-bit values) on their way into LDS.  Requires M%256 == N%256 == K%64 == 0.
-//   * gemm32_mfma_kernel  - fp32 on v_mfma_f32_32x32x2f32, 128x128 tile, for M%128 == N%128 == K%16 == 0.
+//   * gemm32_mfma_kernel  - fp32 on v_mfma_f32_32x32x2f32, 128x128 tile (64x64 when that is what fills the chip),
+//     for M%128 == N%128 == K%16 == 0.
 //   * gemm_generic_kernel - any shape / transpose / type (fp16, bf16, fp32, fp64): 64x64 LDS tile, FMA units.
 #include <hip/hip_runtime.h>
 
@@ -385,39 +386,42 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 constexpr int kF32Tile = 128;
 constexpr int kF32K    = 16;
 
-template <bool TRANS_A, bool TRANS_B>
+template <int TILE, bool TRANS_A, bool TRANS_B>
 __global__ void __launch_bounds__(256)
 gemm32_mfma_kernel(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C, int M, int N, int K,
                    int64_t lda, int64_t ldb, int64_t ldc, float alpha, float beta, int64_t stride_a, int64_t stride_b,
                    int64_t stride_c) {
-  __shared__ float As[2][kF32K][kF32Tile + 4];
-  __shared__ float Bs[2][kF32K][kF32Tile + 4];
+  __shared__ float As[2][kF32K][TILE + 4];
+  __shared__ float Bs[2][kF32K][TILE + 4];
+  constexpr int TT = TILE / 64;   // 32x32 MFMA tiles per wavefront and dimension
+  constexpr int EL = TILE / 16;   // elements of each operand a thread stages per K step
+  constexpr int SH = TILE == 128 ? 7 : 6;
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int m0 = blockIdx.y * kF32Tile;
-  const int n0 = blockIdx.x * kF32Tile;
+  const int m0 = blockIdx.y * TILE;
+  const int n0 = blockIdx.x * TILE;
   A += (int64_t)blockIdx.z * stride_a;
   B += (int64_t)blockIdx.z * stride_b;
   C += (int64_t)blockIdx.z * stride_c;
 
-  f32x16 acc[2][2];
+  f32x16 acc[TT][TT];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TT; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TT; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
   // each thread stages 8 floats of A and 8 of B per K step (128 x 16 = 2048 per operand)
-  float ra[8], rb[8];
+  float ra[EL], rb[EL];
   auto load_tiles = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < EL; ++i) {
       int e = tid + 256 * i;
       if (TRANS_A) {  // A stored [K][M]: m contiguous
-        int k = e >> 7, m = e & 127;
+        int k = e >> SH, m = e & (TILE - 1);
         ra[i] = A[(int64_t)(k0 + k) * lda + m0 + m];
       } else {  // A stored [M][K]: k contiguous
         int m = e >> 4, k = e & 15;
@@ -427,24 +431,24 @@ gemm32_mfma_kernel(const float* __restrict__ A, const float* __restrict__ B, flo
         int n = e >> 4, k = e & 15;
         rb[i] = B[(int64_t)(n0 + n) * ldb + k0 + k];
       } else {  // B stored [K][N]
-        int k = e >> 7, n = e & 127;
+        int k = e >> SH, n = e & (TILE - 1);
         rb[i] = B[(int64_t)(k0 + k) * ldb + n0 + n];
       }
     }
   };
   auto store_tiles = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < EL; ++i) {
       int e = tid + 256 * i;
       if (TRANS_A) {
-        As[buf][e >> 7][e & 127] = ra[i];
+        As[buf][e >> SH][e & (TILE - 1)] = ra[i];
       } else {
         As[buf][e & 15][e >> 4] = ra[i];
       }
       if (TRANS_B) {
         Bs[buf][e & 15][e >> 4] = rb[i];
       } else {
-        Bs[buf][e >> 7][e & 127] = rb[i];
+        Bs[buf][e >> SH][e & (TILE - 1)] = rb[i];
       }
     }
   };
@@ -460,28 +464,28 @@ gemm32_mfma_kernel(const float* __restrict__ A, const float* __restrict__ B, flo
 #pragma unroll
     for (int kk = 0; kk < kF32K; kk += 2) {
       const int k = kk + (lane >> 5);
-      float af[2], bf[2];
+      float af[TT], bf[TT];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        af[t] = As[cur][k][wm * 64 + t * 32 + (lane & 31)];
-        bf[t] = Bs[cur][k][wn * 64 + t * 32 + (lane & 31)];
+      for (int t = 0; t < TT; ++t) {
+        af[t] = As[cur][k][wm * (TILE / 2) + t * 32 + (lane & 31)];
+        bf[t] = Bs[cur][k][wn * (TILE / 2) + t * 32 + (lane & 31)];
       }
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < TT; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < TT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
     }
     if (more) store_tiles(cur ^ 1);
     __syncthreads();
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < TT; ++i) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+    for (int j = 0; j < TT; ++j) {
+      const int col = n0 + wn * (TILE / 2) + j * 32 + (lane & 31);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int row = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        const int row = m0 + wm * (TILE / 2) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         float* dst = C + (int64_t)row * ldc + col;
         float v    = alpha * acc[i][j][r];
         if (beta != 0.0f) v += beta * *dst;
@@ -633,13 +637,21 @@ void LaunchGeneric(const GemmProblem& p, hipStream_t stream) {
 void LaunchFast32(const GemmProblem& p, hipStream_t stream) {
   int64_t lda = p.trans_a ? p.m : p.k;
   int64_t ldb = p.trans_b ? p.k : p.n;
-  dim3 grid(p.n / kF32Tile, p.m / kF32Tile, p.batch);
+  // 128x128 tiles unless they leave most of the 256 CUs idle; then 64x64 tiles, four times as many blocks
+  const bool small = (int64_t)(p.n / kF32Tile) * (p.m / kF32Tile) * p.batch < 256;
+  const int tile   = small ? 64 : kF32Tile;
+  dim3 grid(p.n / tile, p.m / tile, p.batch);
   const float* a = static_cast<const float*>(p.a);
   const float* b = static_cast<const float*>(p.b);
   float* c       = static_cast<float*>(p.c);
 #define CINN_LAUNCH_F32(TA, TB)                                                                                       \
-  hipLaunchKernelGGL((gemm32_mfma_kernel<TA, TB>), grid, dim3(256), 0, stream, a, b, c, p.m, p.n, p.k, lda, ldb,       \
-                     (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c)
+  if (small) {                                                                                                        \
+    hipLaunchKernelGGL((gemm32_mfma_kernel<64, TA, TB>), grid, dim3(256), 0, stream, a, b, c, p.m, p.n, p.k, lda, ldb, \
+                       (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c);                            \
+  } else {                                                                                                            \
+    hipLaunchKernelGGL((gemm32_mfma_kernel<128, TA, TB>), grid, dim3(256), 0, stream, a, b, c, p.m, p.n, p.k, lda,     \
+                       ldb, (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c);                       \
+  }
   if (!p.trans_a && !p.trans_b) CINN_LAUNCH_F32(false, false);
   if (!p.trans_a && p.trans_b) CINN_LAUNCH_F32(false, true);
   if (p.trans_a && !p.trans_b) CINN_LAUNCH_F32(true, false);
