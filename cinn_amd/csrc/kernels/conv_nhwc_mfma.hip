@@ -48,6 +48,9 @@ struct Params {
   int pixels;   // n * oh * ow
   int relu;
   float alpha, residual_scale;
+  int steps_per_split;  // K steps each blockIdx.y handles; with more than one split the kernel writes raw fp32 partial
+                        // sums to the workspace and SplitReduceKernel applies the epilogue
+  int splits;
 };
 
 // byte offset of 16-byte chunk `chunk` (0..7) of row `row` inside an operand tile
@@ -126,7 +129,7 @@ struct WaveMma {
 template <typename T, int BM, int BN, bool NCHW_IN>
 __global__ void __launch_bounds__(kThreads)
 conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, const float* __restrict__ scale,
-                      const float* __restrict__ shift, const T* residual, Params p) {
+                      const float* __restrict__ shift, const T* residual, float* __restrict__ workspace, Params p) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   constexpr int E      = 16 / sizeof(T);  // elements per chunk
   constexpr int BK     = 8 * E;           // elements per K step
@@ -179,9 +182,12 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
     }
   }
   // position of this thread's chunk in the reduction: channel offset and filter tap (channels-last loader)
+  const int total_steps = (p.k_total + BK - 1) / BK;
+  const int step0       = blockIdx.y * p.steps_per_split;
+  const int step1       = step0 + p.steps_per_split < total_steps ? step0 + p.steps_per_split : total_steps;
   int ck = 0, dy = 0, dx = 0;
   if (!NCHW_IN) {
-    int kc  = cc * E;
+    int kc  = step0 * BK + cc * E;
     int tap = kc / p.c;
     ck      = kc - tap * p.c;
     dy      = tap / p.kw;
@@ -268,15 +274,15 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  const int steps = (p.k_total + BK - 1) / BK;
-  load_step(0);
+  const int steps = step1 - step0;
+  load_step(step0);
   store_step(lds);
   __syncthreads();
   const int a_row = wm * (BM / 2) + (lane & 31);
   const int b_row = wn * (BN / 2) + (lane & 31);
   for (int s = 0; s < steps; ++s) {
     char* cur = lds + (s & 1) * STAGE;
-    if (s + 1 < steps) load_step(s + 1);
+    if (s + 1 < steps) load_step(step0 + s + 1);
     WaveMma<T, TM, TN>::Step(cur, cur + A_TILE, a_row, b_row, lane, acc);
     if (s + 1 < steps) store_step(lds + ((s + 1) & 1) * STAGE);
     __syncthreads();
@@ -301,6 +307,22 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   const int cg       = tid % CPR;
   const int oc0      = n0 + cg * 8;
   if (oc0 >= p.oc) return;
+  if (p.splits > 1) {
+    // partial sums of this K range, fp32, [split][pixel][oc]
+    float* ws = workspace + (int64_t)blockIdx.y * p.pixels * p.oc;
+    for (int row = tid / CPR; row < BM; row += ROWS) {
+      int m = m0 + row;
+      if (m >= p.pixels) break;
+      const int64_t off = (int64_t)m * p.oc + oc0;
+      if ((p.oc & 7) == 0) {
+        *reinterpret_cast<f32x4*>(ws + off)     = *reinterpret_cast<const f32x4*>(&st[row * SLD + cg * 8]);
+        *reinterpret_cast<f32x4*>(ws + off + 4) = *reinterpret_cast<const f32x4*>(&st[row * SLD + cg * 8 + 4]);
+      } else {
+        for (int e = 0; e < 8 && oc0 + e < p.oc; ++e) ws[off + e] = st[row * SLD + cg * 8 + e];
+      }
+    }
+    return;
+  }
   float sc[8], sh[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
@@ -340,6 +362,37 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   }
 }
 
+// Sums the partial results of a split-K convolution and applies the epilogue: one thread per output element group of
+// 4 channels (oc % 4 == 0) or per element.
+template <typename T, int V>
+__global__ void __launch_bounds__(256)
+SplitReduceKernel(const float* __restrict__ workspace, T* y, const float* __restrict__ scale, const float* __restrict__ shift,
+                  const T* residual, Params p) {
+  const int64_t total = (int64_t)p.pixels * p.oc / V;
+  const int64_t idx   = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int64_t off = idx * V;
+  const int oc0     = (int)(off % p.oc);
+  float v[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) v[e] = 0.0f;
+  for (int sp = 0; sp < p.splits; ++sp) {
+    float part[V];
+    __builtin_memcpy(part, workspace + (int64_t)sp * p.pixels * p.oc + off, V * sizeof(float));
+#pragma unroll
+    for (int e = 0; e < V; ++e) v[e] += part[e];
+  }
+  T rv[V], out[V];
+  if (residual) __builtin_memcpy(rv, residual + off, V * sizeof(T));
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    float t = v[e] * (scale ? scale[oc0 + e] : p.alpha) + (shift ? shift[oc0 + e] : 0.0f);
+    if (residual) t += p.residual_scale * (float)rv[e];
+    out[e] = (T)(p.relu ? fmaxf(t, 0.0f) : t);
+  }
+  __builtin_memcpy(y + off, out, V * sizeof(T));
+}
+
 // ---- host side ------------------------------------------------------------------------------------------------
 struct TileChoice {
   int bm, bn;
@@ -351,8 +404,10 @@ int LdsBytes(int bm, int bn) {
   return stages > staging ? stages : staging;
 }
 
-// Picks the block tile: the largest one that still gives every CU work in (nearly) every round.  Larger tiles reuse
-// each LDS fragment for more MFMAs; smaller ones keep 256 CUs busy when the layer has few pixels.
+// Block tile.  Measured over the ResNet-50 layer shapes at batch 32, the 64x64 tile is the fastest or within a few per
+// cent of the fastest everywhere: the kernel prefetches one K step ahead, so what hides the load latency is the number
+// of blocks resident on a CU, and the small tile (32 KiB of LDS) allows five.  The larger tiles stay selectable for
+// experiments (FLAGS_cinn_hip_conv_tile = 0: 128x128, 1: 128x64, 2: 64x64).
 TileChoice ChooseTile(int pixels, int oc) {
   static const int forced = [] {
     const char* e = getenv("FLAGS_cinn_hip_conv_tile");
@@ -360,25 +415,44 @@ TileChoice ChooseTile(int pixels, int oc) {
   }();
   const TileChoice options[3] = {{128, 128}, {128, 64}, {64, 64}};
   if (forced >= 0 && forced < 3) return options[forced];
-  // relative MFMA rate a tile reaches (LDS fragment reads per MFMA grow as the tile shrinks)
-  const double efficiency[3] = {1.0, 0.8, 0.55};
-  double best                = 0;
-  int pick                   = -1;
-  for (int i = 0; i < 3; ++i) {
-    if (options[i].bn > 64 && oc <= 64) continue;
-    int64_t blocks = (int64_t)((pixels + options[i].bm - 1) / options[i].bm) * ((oc + options[i].bn - 1) / options[i].bn);
-    // blocks the busiest CU works through, times the cost of one block
-    double cost = (double)((blocks + 255) / 256) * options[i].bm * options[i].bn / efficiency[i];
-    if (pick < 0 || cost < best) {
-      best = cost;
-      pick = i;
+  (void)pixels;
+  (void)oc;
+  return options[2];
+}
+
+// fp32 scratch for split-K partial sums; grown on demand and kept (the first, eager execution of a program sizes it, so
+// graph capture never sees an allocation)
+float* Workspace(size_t bytes) {
+  static float* buffer   = nullptr;
+  static size_t capacity = 0;
+  if (bytes > capacity) {
+    if (buffer) {
+      CINN_HIP_CALL(hipDeviceSynchronize());
+      CINN_HIP_CALL(hipFree(buffer));
     }
+    CINN_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&buffer), bytes));
+    capacity = bytes;
   }
-  return options[pick];
+  return buffer;
+}
+
+// K splits: layers whose tile grid cannot fill the 256 CUs spend their time waiting for one block's serial chain of
+// loads; splitting the reduction puts several blocks of the same tile on different CUs
+int ChooseSplits(int tiles, int steps) {
+  static const int forced = [] {
+    const char* e = getenv("FLAGS_cinn_hip_conv_splits");
+    return e ? atoi(e) : 0;
+  }();
+  if (forced > 0) return forced < steps ? forced : steps;
+  // only grids that leave CUs without a single block are split, and every part keeps at least 8 K steps
+  int splits = 1;
+  if (tiles >= 256) return 1;
+  while (tiles * splits < 640 && steps / (splits * 2) >= 8 && splits < 8) splits *= 2;
+  return splits;
 }
 
 template <typename T, int BM, int BN, bool NCHW_IN>
-void Launch(const ConvNhwcArgs& a, const Params& p, hipStream_t stream) {
+void Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream) {
   auto kernel     = conv_nhwc_mfma_kernel<T, BM, BN, NCHW_IN>;
   const int bytes = LdsBytes(BM, BN);
   static bool configured = false;
@@ -386,10 +460,31 @@ void Launch(const ConvNhwcArgs& a, const Params& p, hipStream_t stream) {
     CINN_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
     configured = true;
   }
-  const int tiles = ((p.pixels + BM - 1) / BM) * ((p.oc + BN - 1) / BN);
-  hipLaunchKernelGGL(kernel, dim3(tiles), dim3(kThreads), bytes, stream, static_cast<const T*>(a.x),
-                     static_cast<const T*>(a.w), static_cast<T*>(a.y), a.scale, a.shift, static_cast<const T*>(a.residual), p);
+  Params p              = p_in;
+  constexpr int BK      = 128 / sizeof(T);
+  const int tiles       = ((p.pixels + BM - 1) / BM) * ((p.oc + BN - 1) / BN);
+  const int steps       = (p.k_total + BK - 1) / BK;
+  p.splits              = ChooseSplits(tiles, steps);
+  p.steps_per_split     = (steps + p.splits - 1) / p.splits;
+  p.splits              = (steps + p.steps_per_split - 1) / p.steps_per_split;
+  float* workspace      = nullptr;
+  if (p.splits > 1) workspace = Workspace((size_t)p.splits * p.pixels * p.oc * sizeof(float));
+  hipLaunchKernelGGL(kernel, dim3(tiles, p.splits), dim3(kThreads), bytes, stream, static_cast<const T*>(a.x),
+                     static_cast<const T*>(a.w), static_cast<T*>(a.y), a.scale, a.shift, static_cast<const T*>(a.residual),
+                     workspace, p);
   CINN_HIP_CALL(hipGetLastError());
+  if (p.splits > 1) {
+    if (p.oc % 4 == 0) {
+      const int64_t total = (int64_t)p.pixels * p.oc / 4;
+      hipLaunchKernelGGL((SplitReduceKernel<T, 4>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, workspace,
+                         static_cast<T*>(a.y), a.scale, a.shift, static_cast<const T*>(a.residual), p);
+    } else {
+      const int64_t total = (int64_t)p.pixels * p.oc;
+      hipLaunchKernelGGL((SplitReduceKernel<T, 1>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, workspace,
+                         static_cast<T*>(a.y), a.scale, a.shift, static_cast<const T*>(a.residual), p);
+    }
+    CINN_HIP_CALL(hipGetLastError());
+  }
 }
 
 template <typename T>

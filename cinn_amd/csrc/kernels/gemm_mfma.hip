@@ -564,6 +564,72 @@ gemm_generic_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restr
 
 enum class GemmType { kF16, kBF16, kF32, kF64 };
 
+// ---------------------------------------------------------------------------------------------------
+// Skinny GEMM: C[m][n] = alpha * sum_k A[m][k] * Bt[n][k] + beta * C for a handful of rows m (a classifier layer on
+// one batch).  The work is reading Bt once, so there is no tile to fill: one wavefront owns NC output columns, its
+// lanes split K in 16-byte chunks, products accumulate in fp32 and a butterfly over the wavefront finishes each sum.
+// ---------------------------------------------------------------------------------------------------
+template <typename T, int MT, int NC>
+__global__ void __launch_bounds__(256)
+skinny_gemm_kernel(const T* __restrict__ A, const T* __restrict__ Bt, T* C, int M, int N, int K, float alpha, float beta) {
+  constexpr int E = 16 / sizeof(T);
+  const int lane  = threadIdx.x & 63;
+  const int n0    = (blockIdx.x * 4 + (threadIdx.x >> 6)) * NC;
+  if (n0 >= N) return;
+  for (int mb = 0; mb < M; mb += MT) {
+    float acc[MT][NC];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int c = 0; c < NC; ++c) acc[m][c] = 0.0f;
+    for (int k = lane * E; k < K; k += 64 * E) {
+      T b[NC][E];
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        if (n0 + c < N) {
+          __builtin_memcpy(b[c], Bt + (int64_t)(n0 + c) * K + k, 16);
+        } else {
+#pragma unroll
+          for (int e = 0; e < E; ++e) b[c][e] = (T)0.0f;
+        }
+      }
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        if (mb + m < M) {
+          T a[E];
+          __builtin_memcpy(a, A + (int64_t)(mb + m) * K + k, 16);
+#pragma unroll
+          for (int c = 0; c < NC; ++c)
+#pragma unroll
+            for (int e = 0; e < E; ++e) acc[m][c] += (float)a[e] * (float)b[c][e];
+        }
+      }
+    }
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        float v = acc[m][c];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+        if (lane == 0 && mb + m < M && n0 + c < N) {
+          T* dst  = C + (int64_t)(mb + m) * N + n0 + c;
+          float r = alpha * v;
+          if (beta != 0.0f) r += beta * (float)*dst;
+          *dst = (T)r;
+        }
+      }
+  }
+}
+
+template <typename T>
+void LaunchSkinny(const void* a, const void* b, void* c, int m, int n, int k, float alpha, float beta, hipStream_t stream) {
+  constexpr int NC = 2;
+  const int waves  = (n + NC - 1) / NC;
+  hipLaunchKernelGGL((skinny_gemm_kernel<T, 16, NC>), dim3((waves + 3) / 4), dim3(256), 0, stream, static_cast<const T*>(a),
+                     static_cast<const T*>(b), static_cast<T*>(c), m, n, k, alpha, beta);
+}
+
 struct GemmProblem {
   GemmType type;
   const void* a;
@@ -676,7 +742,22 @@ void RunGemm(const GemmProblem& p, hipStream_t stream) {
   // edge and pick a tile that fills the chip for small m or n.
   const int elem_bytes = p.type == GemmType::kF32 ? 4 : (p.type == GemmType::kF64 ? 8 : 2);
   const bool tile_fit  = p.type == GemmType::kF32 ? fast32 : fast16;
-  if (!ForceGeneric() && !tile_fit && p.type != GemmType::kF64 && !p.trans_a && p.trans_b && p.k % (16 / elem_bytes) == 0) {
+  const bool k_contig  = !ForceGeneric() && p.type != GemmType::kF64 && !p.trans_a && p.trans_b && p.k % (16 / elem_bytes) == 0;
+  if (k_contig && p.m <= 64) {
+    for (int b = 0; b < p.batch; ++b) {
+      const char* a = static_cast<const char*>(p.a) + (int64_t)b * p.stride_a * elem_bytes;
+      const char* w = static_cast<const char*>(p.b) + (int64_t)b * p.stride_b * elem_bytes;
+      char* c       = static_cast<char*>(p.c) + (int64_t)b * p.stride_c * elem_bytes;
+      switch (p.type) {
+        case GemmType::kBF16: LaunchSkinny<__bf16>(a, w, c, p.m, p.n, p.k, p.alpha, p.beta, stream); break;
+        case GemmType::kF16: LaunchSkinny<_Float16>(a, w, c, p.m, p.n, p.k, p.alpha, p.beta, stream); break;
+        default: LaunchSkinny<float>(a, w, c, p.m, p.n, p.k, p.alpha, p.beta, stream); break;
+      }
+    }
+    CINN_HIP_CALL(hipGetLastError());
+    return;
+  }
+  if (k_contig && !tile_fit) {
     for (int b = 0; b < p.batch; ++b) {
       cinn_hip_kernels::ConvNhwcArgs a;
       a.x = static_cast<const char*>(p.a) + (int64_t)b * p.stride_a * elem_bytes;

@@ -129,9 +129,71 @@ __global__ void __launch_bounds__(256) pool2d_nhwc_kernel(const T* __restrict__ 
   __builtin_memcpy(dst, res, V * sizeof(T));
 }
 
+
+// Channels-last pooling whose window is the whole image (global average / max pooling): the generic kernel would give
+// each thread the entire image of its channels to walk through.  Here a block of 256 threads takes one image and 64
+// channels: 8 channel groups of 8 x 32 pixel slices, partial results combined through LDS.  The average still divides
+// every element before adding; only the order of the additions differs from the generic kernel.
+template <typename T, int V>
+__global__ void __launch_bounds__(256) global_pool_nhwc_kernel(const T* __restrict__ in, T* __restrict__ out, PoolParams p) {
+  constexpr int GROUPS = 8;   // channel groups per block
+  constexpr int SLICES = 32;  // pixel slices
+  __shared__ float partial[SLICES][GROUPS * V + 1];
+  const int groups_per_image = (p.c / V + GROUPS - 1) / GROUPS;
+  const int n     = blockIdx.x / groups_per_image;
+  const int g     = (blockIdx.x % groups_per_image) * GROUPS + (threadIdx.x % GROUPS);
+  const int slice = threadIdx.x / GROUPS;
+  const bool is_max = p.mode == 0 || p.mode == 3;
+  const int pixels  = p.ih * p.iw;
+  const float factor = (float)pixels;
+  float acc[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) acc[e] = is_max ? -3.402823466e+38f : 0.0f;
+  if (g * V < p.c) {
+    const T* src = in + (int64_t)n * pixels * p.c + g * V;
+    for (int px = slice; px < pixels; px += SLICES) {
+      T v[V];
+      __builtin_memcpy(v, src + (int64_t)px * p.c, V * sizeof(T));
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const float f = (float)v[e];
+        if (is_max)
+          acc[e] = f > acc[e] ? f : acc[e];
+        else
+          acc[e] += f / factor;
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < V; ++e) partial[slice][(threadIdx.x % GROUPS) * V + e] = acc[e];
+  __syncthreads();
+  // thread t < GROUPS * V finishes channel t of the block
+  if (threadIdx.x < GROUPS * V) {
+    const int c = (blockIdx.x % groups_per_image) * GROUPS * V + threadIdx.x;
+    if (c < p.c) {
+      float r = is_max ? -3.402823466e+38f : 0.0f;
+      for (int s2 = 0; s2 < SLICES; ++s2) {
+        const float f = partial[s2][threadIdx.x];
+        r             = is_max ? (f > r ? f : r) : r + f;
+      }
+      T* dst = out + (int64_t)n * p.c + c;
+      r      = p.alpha * r;
+      if (p.beta != 0.0f) r += p.beta * (float)*dst;
+      *dst = (T)r;
+    }
+  }
+}
+
 template <typename T>
 void LaunchPoolNhwc(const void* x, void* y, const PoolParams& p, hipStream_t s) {
   constexpr int V = 16 / sizeof(T);
+  const bool global = p.oh == 1 && p.ow == 1 && p.kh == p.ih && p.kw == p.iw && p.ph == 0 && p.pw == 0;
+  if (global && p.c % V == 0 && p.ih * p.iw >= 16) {
+    const int groups_per_image = (p.c / V + 7) / 8;
+    hipLaunchKernelGGL((global_pool_nhwc_kernel<T, V>), dim3((unsigned)(p.n * groups_per_image)), dim3(256), 0, s,
+                       static_cast<const T*>(x), static_cast<T*>(y), p);
+    return;
+  }
   if (p.c % V == 0) {
     const int64_t total = (int64_t)p.n * p.oh * p.ow * (p.c / V);
     hipLaunchKernelGGL((pool2d_nhwc_kernel<T, V>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
