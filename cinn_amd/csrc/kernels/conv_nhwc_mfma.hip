@@ -48,10 +48,16 @@ struct Params {
   int pixels;   // n * oh * ow
   int relu;
   float alpha, residual_scale;
+  // exact division of values below 2^31 by oh*ow, ow, c and kw: q = (n * magic) >> shift (64-bit product)
+  unsigned magic_plane, shift_plane, magic_ow, shift_ow, magic_c, shift_c, magic_kw, shift_kw;
   int steps_per_split;  // K steps each blockIdx.y handles; with more than one split the kernel writes raw fp32 partial
                         // sums to the workspace and SplitReduceKernel applies the epilogue
   int splits;
 };
+
+__device__ __forceinline__ int FastDiv(int n, unsigned magic, unsigned shift) {
+  return (int)(((unsigned long long)(unsigned)n * magic) >> shift);
+}
 
 // byte offset of 16-byte chunk `chunk` (0..7) of row `row` inside an operand tile
 __device__ __forceinline__ int TileOffset(int row, int chunk) {
@@ -126,10 +132,11 @@ struct WaveMma {
 };
 
 // ---- the kernel -----------------------------------------------------------------------------------------------
-template <typename T, int BM, int BN, bool NCHW_IN>
+template <typename T, int BM, int BN, bool NCHW_IN, int PF>
 __global__ void __launch_bounds__(kThreads)
 conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, const float* __restrict__ scale,
-                      const float* __restrict__ shift, const T* residual, float* __restrict__ workspace, Params p) {
+                      const float* __restrict__ shift, const T* residual, float* __restrict__ workspace,
+                      const void* __restrict__ zero_page, Params p) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   constexpr int E      = 16 / sizeof(T);  // elements per chunk
   constexpr int BK     = 8 * E;           // elements per K step
@@ -163,18 +170,20 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   const int lr = tid >> 3;  // first tile row this thread loads
 
   // per-row state of the pixel operand
+  // base: element offset of the image (NCHW loader) or of the window origin (ih0, iw0) of the row, which may lie
+  // before the tensor (channels-last loader: a chunk is at base + tap offset)
   int base[RA], ih0[RA], iw0[RA];
 #pragma unroll
   for (int i = 0; i < RA; ++i) {
     int m = m0 + lr + 32 * i;
     if (m < p.pixels) {
-      int n   = m / (p.oh * p.ow);
+      int n   = FastDiv(m, p.magic_plane, p.shift_plane);
       int rem = m - n * (p.oh * p.ow);
-      int oh  = rem / p.ow;
+      int oh  = FastDiv(rem, p.magic_ow, p.shift_ow);
       int ow  = rem - oh * p.ow;
-      base[i] = n * p.h * p.w * p.c;
       ih0[i]  = oh * p.stride_h - p.pad_h;
       iw0[i]  = ow * p.stride_w - p.pad_w;
+      base[i] = NCHW_IN ? n * p.h * p.w * p.c : ((n * p.h + ih0[i]) * p.w + iw0[i]) * p.c;
     } else {
       base[i] = 0;
       ih0[i]  = INT_MIN / 2;  // fails every bounds test
@@ -188,32 +197,45 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   int ck = 0, dy = 0, dx = 0;
   if (!NCHW_IN) {
     int kc  = step0 * BK + cc * E;
-    int tap = kc / p.c;
+    int tap = FastDiv(kc, p.magic_c, p.shift_c);
     ck      = kc - tap * p.c;
-    dy      = tap / p.kw;
+    dy      = FastDiv(tap, p.magic_kw, p.shift_kw);
     dx      = tap - dy * p.kw;
   }
+  // rows of the filter operand this thread loads
+  int wrow[RB];
+#pragma unroll
+  for (int i = 0; i < RB; ++i) {
+    int oc  = n0 + lr + 32 * i;
+    wrow[i] = oc < p.oc ? oc * p.k_total : -1;  // checked on the host: oc * k_total < 2^31
+  }
 
-  u32x4 ra[RA], rb[RB];
-  auto load_step = [&](int step) {
+  // Register slots for the K steps in flight: the loads of step s + PF are issued while step s is computed, so a
+  // block keeps PF steps of global-memory latency covered by itself (slot of step t: t % PF).
+  u32x4 ra_slots[PF][RA], rb_slots[PF][RB];
+  // Loads are unconditional: a chunk that lies outside the image, beyond K or beyond this block's K range is read from
+  // a page of zeros instead.  Straight-line code lets the compiler count exactly how many loads may still be in flight
+  // when a slot is consumed (s_waitcnt vmcnt(N)); a branch per chunk would make it wait for all of them.
+  const T* zeros = static_cast<const T*>(zero_page);
+  auto load_step = [&](int step, u32x4 (&ra)[RA], u32x4 (&rb)[RB]) {
+    const bool live = step < step1;
     if (!NCHW_IN) {
-      const bool tap_ok = dy < p.kh;
+      const bool tap_ok = live && dy < p.kh;
+      const int dyo = dy * p.dil_h, dxo = dx * p.dil_w;
+      const int tap_offset = (dyo * p.w + dxo) * p.c + ck;  // the same for every row of this thread
 #pragma unroll
       for (int i = 0; i < RA; ++i) {
-        int ih  = ih0[i] + dy * p.dil_h;
-        int iw  = iw0[i] + dx * p.dil_w;
-        bool ok = tap_ok && (unsigned)ih < (unsigned)p.h && (unsigned)iw < (unsigned)p.w;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (ok) v = *reinterpret_cast<const u32x4*>(x + base[i] + (ih * p.w + iw) * p.c + ck);
-        ra[i] = v;
+        bool ok      = tap_ok && (unsigned)(ih0[i] + dyo) < (unsigned)p.h && (unsigned)(iw0[i] + dxo) < (unsigned)p.w;
+        const T* src = ok ? x + (base[i] + tap_offset) : zeros;
+        ra[i]        = *reinterpret_cast<const u32x4*>(src);
       }
-      const int kb = step * BK + cc * E;
+      const int kb     = step * BK + cc * E;
+      const bool kb_ok = live && kb < p.k_total;
 #pragma unroll
       for (int i = 0; i < RB; ++i) {
-        int oc  = n0 + lr + 32 * i;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (oc < p.oc && kb < p.k_total) v = *reinterpret_cast<const u32x4*>(w + (int64_t)oc * p.k_total + kb);
-        rb[i] = v;
+        bool ok      = kb_ok && wrow[i] >= 0;
+        const T* src = ok ? w + (wrow[i] + kb) : zeros;
+        rb[i]        = *reinterpret_cast<const u32x4*>(src);
       }
       // advance to the next step
       ck += BK;
@@ -232,7 +254,7 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
       const int dx0            = (q - row_id * chunks_per_row) * E;
       const int c              = row_id / p.kh;
       const int ky             = row_id - c * p.kh;
-      const bool c_ok          = c < p.c;
+      const bool c_ok          = live && c < p.c;
 #pragma unroll
       for (int i = 0; i < RA; ++i) {
         T tmp[E];
@@ -259,7 +281,7 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
       }
     }
   };
-  auto store_step = [&](char* stage) {
+  auto store_step = [&](char* stage, const u32x4 (&ra)[RA], const u32x4 (&rb)[RB]) {
 #pragma unroll
     for (int i = 0; i < RA; ++i) *reinterpret_cast<u32x4*>(stage + TileOffset(lr + 32 * i, cc)) = ra[i];
 #pragma unroll
@@ -274,18 +296,37 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
+  static_assert(PF % 2 == 0, "the LDS stage of a step must be a compile-time function of its slot");
   const int steps = step1 - step0;
-  load_step(step0);
-  store_step(lds);
+#pragma unroll
+  for (int i = 0; i < PF; ++i)
+    if (i == 0 || i < steps) load_step(step0 + i, ra_slots[i], rb_slots[i]);
+  store_step(lds, ra_slots[0], rb_slots[0]);
+  if (PF < steps) load_step(step0 + PF, ra_slots[0], rb_slots[0]);
   __syncthreads();
   const int a_row = wm * (BM / 2) + (lane & 31);
   const int b_row = wn * (BN / 2) + (lane & 31);
-  for (int s = 0; s < steps; ++s) {
-    char* cur = lds + (s & 1) * STAGE;
-    if (s + 1 < steps) load_step(step0 + s + 1);
-    WaveMma<T, TM, TN>::Step(cur, cur + A_TILE, a_row, b_row, lane, acc);
-    if (s + 1 < steps) store_step(lds + ((s + 1) & 1) * STAGE);
-    __syncthreads();
+  int s = 0;
+  // whole groups of PF steps: branch-free, every sub-step refills the slot it has just emptied
+  for (; s + PF <= steps; s += PF) {
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      char* cur = lds + (i & 1) * STAGE;  // s is a multiple of PF, PF is even
+      WaveMma<T, TM, TN>::Step(cur, cur + A_TILE, a_row, b_row, lane, acc);
+      store_step(lds + ((i + 1) & 1) * STAGE, ra_slots[(i + 1) % PF], rb_slots[(i + 1) % PF]);
+      load_step(step0 + s + i + 1 + PF, ra_slots[(i + 1) % PF], rb_slots[(i + 1) % PF]);
+      __syncthreads();
+    }
+  }
+  // the last steps < PF; their data is already in the slots
+#pragma unroll
+  for (int i = 0; i < PF - 1; ++i) {
+    if (s + i < steps) {
+      char* cur = lds + (i & 1) * STAGE;
+      WaveMma<T, TM, TN>::Step(cur, cur + A_TILE, a_row, b_row, lane, acc);
+      store_step(lds + ((i + 1) & 1) * STAGE, ra_slots[(i + 1) % PF], rb_slots[(i + 1) % PF]);
+      __syncthreads();
+    }
   }
 
   // ---- epilogue: accumulators -> LDS (fp32) -> 8 channels of one pixel per lane ----------------------------------
@@ -323,14 +364,19 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
     }
     return;
   }
-  float sc[8], sh[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    int oc = oc0 + e < p.oc ? oc0 + e : p.oc - 1;
-    sc[e]  = scale ? scale[oc] : p.alpha;
-    sh[e]  = shift ? shift[oc] : 0.0f;
-  }
   const bool full = (p.oc & 7) == 0;  // then every group is whole and 16-byte aligned
+  float sc[8], sh[8];
+  if (full && scale && shift) {
+    __builtin_memcpy(sc, scale + oc0, 32);
+    __builtin_memcpy(sh, shift + oc0, 32);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      int oc = oc0 + e < p.oc ? oc0 + e : p.oc - 1;
+      sc[e]  = scale ? scale[oc] : p.alpha;
+      sh[e]  = shift ? shift[oc] : 0.0f;
+    }
+  }
 #pragma unroll 2
   for (int row = tid / CPR; row < BM; row += ROWS) {
     int m = m0 + row;
@@ -420,6 +466,17 @@ TileChoice ChooseTile(int pixels, int oc) {
   return options[2];
 }
 
+// 256 bytes of zeros that masked-out chunks are read from
+const void* ZeroPage() {
+  static void* page = nullptr;
+  if (!page) {
+    CINN_HIP_CALL(hipMalloc(&page, 256));
+    CINN_HIP_CALL(hipMemset(page, 0, 256));
+    CINN_HIP_CALL(hipDeviceSynchronize());
+  }
+  return page;
+}
+
 // fp32 scratch for split-K partial sums; grown on demand and kept (the first, eager execution of a program sizes it, so
 // graph capture never sees an allocation)
 float* Workspace(size_t bytes) {
@@ -453,7 +510,9 @@ int ChooseSplits(int tiles, int steps) {
 
 template <typename T, int BM, int BN, bool NCHW_IN>
 void Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream) {
-  auto kernel     = conv_nhwc_mfma_kernel<T, BM, BN, NCHW_IN>;
+  // steps in flight per block: what the register budget of the tile allows
+  constexpr int PF = 2;
+  auto kernel      = conv_nhwc_mfma_kernel<T, BM, BN, NCHW_IN, PF>;
   const int bytes = LdsBytes(BM, BN);
   static bool configured = false;
   if (!configured) {
@@ -471,7 +530,7 @@ void Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream) {
   if (p.splits > 1) workspace = Workspace((size_t)p.splits * p.pixels * p.oc * sizeof(float));
   hipLaunchKernelGGL(kernel, dim3(tiles, p.splits), dim3(kThreads), bytes, stream, static_cast<const T*>(a.x),
                      static_cast<const T*>(a.w), static_cast<T*>(a.y), a.scale, a.shift, static_cast<const T*>(a.residual),
-                     workspace, p);
+                     workspace, ZeroPage(), p);
   CINN_HIP_CALL(hipGetLastError());
   if (p.splits > 1) {
     if (p.oc % 4 == 0) {
@@ -508,6 +567,18 @@ void Dispatch(const ConvNhwcArgs& a, const Params& p, hipStream_t stream) {
 
 int ChunkElems(const cinn_type_t& t) { return 16 / (t.bits / CHAR_BIT); }
 
+// q = (n * magic) >> shift == n / d for 0 <= n < 2^31 (Granlund-Montgomery with a 64-bit product)
+void MagicFor(int d, unsigned* magic, unsigned* shift) {
+  int l = 0;
+  while ((1ll << l) < d) ++l;
+  *shift = 31 + l;
+  *magic = (unsigned)(((1ull << *shift) / (unsigned)d) + 1);
+  if (d == 1) {  // 2^31 + 1 would round n = 2^31 - 1 up; d == 1 needs no rounding at all
+    *shift = 0;
+    *magic = 1;
+  }
+}
+
 }  // namespace
 
 bool ConvNhwcSupported(const ConvNhwcArgs& a) {
@@ -535,6 +606,11 @@ void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream) {
   p.relu      = a.relu ? 1 : 0;
   p.alpha     = a.alpha;
   p.residual_scale = a.residual_scale;
+  MagicFor(a.oh * a.ow, &p.magic_plane, &p.shift_plane);
+  MagicFor(a.ow, &p.magic_ow, &p.shift_ow);
+  MagicFor(a.c, &p.magic_c, &p.shift_c);
+  MagicFor(a.kw, &p.magic_kw, &p.shift_kw);
+  CINN_RT_CHECK((int64_t)a.oc * p.k_total < INT_MAX, "conv2d (channels-last): filter too large for 32-bit offsets");
   if (a.type.code == cinn_type_bfloat) {
     Dispatch<__bf16>(a, p, stream);
   } else if (a.type.bits == 16) {
