@@ -35,7 +35,6 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kThreads  = 256;
 constexpr int kRowBytes = 128;  // one tile row per K step
 
 struct Params {
@@ -132,8 +131,8 @@ struct WaveMma {
 };
 
 // ---- the kernel -----------------------------------------------------------------------------------------------
-template <typename T, int BM, int BN, bool NCHW_IN, int PF>
-__global__ void __launch_bounds__(kThreads)
+template <typename T, int BM, int BN, int WM, int WN, bool NCHW_IN, int PF>
+__global__ void __launch_bounds__(64 * WM * WN)
 conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, const float* __restrict__ scale,
                       const float* __restrict__ shift, const T* residual, float* __restrict__ workspace,
                       const void* __restrict__ zero_page, Params p) {
@@ -142,17 +141,20 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   constexpr int BK     = 8 * E;           // elements per K step
   constexpr int A_TILE = BM * kRowBytes;
   constexpr int STAGE  = (BM + BN) * kRowBytes;
-  constexpr int RA     = BM / 32;  // chunks of the pixel operand per thread and step
-  constexpr int RB     = BN / 32;
-  constexpr int TM     = BM / 64;  // 32x32 MFMA tiles per wavefront
-  constexpr int TN     = BN / 64;
+  constexpr int THREADS = 64 * WM * WN;  // WM x WN wavefronts, each a (BM / WM) x (BN / WN) tile
+  constexpr int RP     = THREADS / 8;    // tile rows one pass of the loaders covers (8 chunks per row)
+  constexpr int RA     = BM / RP;        // chunks of the pixel operand per thread and step
+  constexpr int RB     = BN / RP;
+  constexpr int TM     = BM / (32 * WM);  // 32x32 MFMA tiles per wavefront
+  constexpr int TN     = BN / (32 * WN);
   constexpr int SLD    = BN + 8;  // row pitch (floats) of the epilogue staging tile
+  static_assert(RA >= 1 && RB >= 1 && TM >= 1 && TN >= 1, "tile too small for the wavefront grid");
 
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm   = wave >> 1;
-  const int wn   = wave & 1;
+  const int wm   = wave / WN;
+  const int wn   = wave % WN;
 
   // Consecutive workgroup ids go round-robin to the 8 XCDs, each with its own L2: hand every XCD a contiguous band
   // of tiles, channel tiles fastest, so that blocks sharing a pixel panel share an L2.
@@ -175,7 +177,7 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   int base[RA], ih0[RA], iw0[RA];
 #pragma unroll
   for (int i = 0; i < RA; ++i) {
-    int m = m0 + lr + 32 * i;
+    int m = m0 + lr + RP * i;
     if (m < p.pixels) {
       int n   = FastDiv(m, p.magic_plane, p.shift_plane);
       int rem = m - n * (p.oh * p.ow);
@@ -206,7 +208,7 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   int wrow[RB];
 #pragma unroll
   for (int i = 0; i < RB; ++i) {
-    int oc  = n0 + lr + 32 * i;
+    int oc  = n0 + lr + RP * i;
     wrow[i] = oc < p.oc ? oc * p.k_total : -1;  // checked on the host: oc * k_total < 2^31
   }
 
@@ -272,7 +274,7 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
 #pragma unroll
       for (int i = 0; i < RB; ++i) {
         T tmp[E];
-        int oc       = n0 + lr + 32 * i;
+        int oc       = n0 + lr + RP * i;
         bool row_ok  = c_ok && oc < p.oc;
         const T* src = w + ((int64_t)(oc * p.c + c) * p.kh + ky) * p.kw;
 #pragma unroll
@@ -283,9 +285,9 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   };
   auto store_step = [&](char* stage, const u32x4 (&ra)[RA], const u32x4 (&rb)[RB]) {
 #pragma unroll
-    for (int i = 0; i < RA; ++i) *reinterpret_cast<u32x4*>(stage + TileOffset(lr + 32 * i, cc)) = ra[i];
+    for (int i = 0; i < RA; ++i) *reinterpret_cast<u32x4*>(stage + TileOffset(lr + RP * i, cc)) = ra[i];
 #pragma unroll
-    for (int i = 0; i < RB; ++i) *reinterpret_cast<u32x4*>(stage + A_TILE + TileOffset(lr + 32 * i, cc)) = rb[i];
+    for (int i = 0; i < RB; ++i) *reinterpret_cast<u32x4*>(stage + A_TILE + TileOffset(lr + RP * i, cc)) = rb[i];
   };
 
   f32x16 acc[TM][TN];
@@ -304,8 +306,8 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   store_step(lds, ra_slots[0], rb_slots[0]);
   if (PF < steps) load_step(step0 + PF, ra_slots[0], rb_slots[0]);
   __syncthreads();
-  const int a_row = wm * (BM / 2) + (lane & 31);
-  const int b_row = wn * (BN / 2) + (lane & 31);
+  const int a_row = wm * (BM / WM) + (lane & 31);
+  const int b_row = wn * (BN / WN) + (lane & 31);
   int s = 0;
   // whole groups of PF steps: branch-free, every sub-step refills the slot it has just emptied
   for (; s + PF <= steps; s += PF) {
@@ -330,79 +332,85 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   }
 
   // ---- epilogue: accumulators -> LDS (fp32) -> 8 channels of one pixel per lane ----------------------------------
-  float* st = reinterpret_cast<float*>(lds);
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        int row = wm * (BM / 2) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        int col = wn * (BN / 2) + j * 32 + (lane & 31);
-        st[row * SLD + col] = acc[i][j][r];
-      }
-  __syncthreads();
-
-  constexpr int CPR  = BN / 8;          // 8-channel groups per tile row
-  constexpr int ROWS = kThreads / CPR;  // rows per pass
-  const int cg       = tid % CPR;
-  const int oc0      = n0 + cg * 8;
-  if (oc0 >= p.oc) return;
-  if (p.splits > 1) {
-    // partial sums of this K range, fp32, [split][pixel][oc]
-    float* ws = workspace + (int64_t)blockIdx.y * p.pixels * p.oc;
-    for (int row = tid / CPR; row < BM; row += ROWS) {
-      int m = m0 + row;
-      if (m >= p.pixels) break;
-      const int64_t off = (int64_t)m * p.oc + oc0;
-      if ((p.oc & 7) == 0) {
-        *reinterpret_cast<f32x4*>(ws + off)     = *reinterpret_cast<const f32x4*>(&st[row * SLD + cg * 8]);
-        *reinterpret_cast<f32x4*>(ws + off + 4) = *reinterpret_cast<const f32x4*>(&st[row * SLD + cg * 8 + 4]);
-      } else {
-        for (int e = 0; e < 8 && oc0 + e < p.oc; ++e) ws[off + e] = st[row * SLD + cg * 8 + e];
-      }
-    }
-    return;
-  }
-  const bool full = (p.oc & 7) == 0;  // then every group is whole and 16-byte aligned
+  // When the whole fp32 tile does not fit the LDS of the two stages it is staged one wavefront row at a time.
+  constexpr bool ONE_PASS = BM * SLD * 4 <= 2 * STAGE;
+  constexpr int PASSES    = ONE_PASS ? 1 : WM;
+  constexpr int PROWS     = BM / PASSES;      // tile rows staged per pass
+  constexpr int CPR       = BN / 8;           // 8-channel groups per tile row
+  constexpr int ROWS      = THREADS / CPR;    // rows the block stores per sweep
+  float* st               = reinterpret_cast<float*>(lds);
+  const int cg            = tid % CPR;
+  const int oc0           = n0 + cg * 8;
+  const bool active       = oc0 < p.oc;
+  const bool full         = (p.oc & 7) == 0;  // then every group is whole and 16-byte aligned
   float sc[8], sh[8];
-  if (full && scale && shift) {
-    __builtin_memcpy(sc, scale + oc0, 32);
-    __builtin_memcpy(sh, shift + oc0, 32);
-  } else {
+  if (active && p.splits == 1) {
+    if (full && scale && shift) {
+      __builtin_memcpy(sc, scale + oc0, 32);
+      __builtin_memcpy(sh, shift + oc0, 32);
+    } else {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      int oc = oc0 + e < p.oc ? oc0 + e : p.oc - 1;
-      sc[e]  = scale ? scale[oc] : p.alpha;
-      sh[e]  = shift ? shift[oc] : 0.0f;
+      for (int e = 0; e < 8; ++e) {
+        int oc = oc0 + e < p.oc ? oc0 + e : p.oc - 1;
+        sc[e]  = scale ? scale[oc] : p.alpha;
+        sh[e]  = shift ? shift[oc] : 0.0f;
+      }
     }
   }
-#pragma unroll 2
-  for (int row = tid / CPR; row < BM; row += ROWS) {
-    int m = m0 + row;
-    if (m >= p.pixels) break;
-    float v[8];
-    *reinterpret_cast<f32x4*>(&v[0]) = *reinterpret_cast<const f32x4*>(&st[row * SLD + cg * 8]);
-    *reinterpret_cast<f32x4*>(&v[4]) = *reinterpret_cast<const f32x4*>(&st[row * SLD + cg * 8 + 4]);
+  float* ws = workspace + (int64_t)blockIdx.y * p.pixels * p.oc;  // split-K: fp32 partial sums [split][pixel][oc]
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = v[e] * sc[e] + sh[e];
-    const int64_t off = (int64_t)m * p.oc + oc0;
-    if (full) {
-      T out[8];
-      if (residual) {
-        T rv[8];
-        __builtin_memcpy(rv, residual + off, 8 * sizeof(T));
+  for (int pass = 0; pass < PASSES; ++pass) {
+    if (pass > 0) __syncthreads();  // the previous pass has been read
+    if (ONE_PASS || wm == pass) {
+      const int row_base = ONE_PASS ? wm * (BM / WM) : 0;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] += p.residual_scale * (float)rv[e];
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            int row = row_base + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            int col = wn * (BN / WN) + j * 32 + (lane & 31);
+            st[row * SLD + col] = acc[i][j][r];
+          }
+    }
+    __syncthreads();
+    if (!active) continue;
+    for (int row = tid / CPR; row < PROWS; row += ROWS) {
+      const int m = m0 + pass * PROWS + row;
+      if (m >= p.pixels) break;
+      float v[8];
+      *reinterpret_cast<f32x4*>(&v[0]) = *reinterpret_cast<const f32x4*>(&st[row * SLD + cg * 8]);
+      *reinterpret_cast<f32x4*>(&v[4]) = *reinterpret_cast<const f32x4*>(&st[row * SLD + cg * 8 + 4]);
+      const int64_t off = (int64_t)m * p.oc + oc0;
+      if (p.splits > 1) {
+        if (full) {
+          *reinterpret_cast<f32x4*>(ws + off)     = *reinterpret_cast<const f32x4*>(&v[0]);
+          *reinterpret_cast<f32x4*>(ws + off + 4) = *reinterpret_cast<const f32x4*>(&v[4]);
+        } else {
+          for (int e = 0; e < 8 && oc0 + e < p.oc; ++e) ws[off + e] = v[e];
+        }
+        continue;
       }
 #pragma unroll
-      for (int e = 0; e < 8; ++e) out[e] = (T)(p.relu ? fmaxf(v[e], 0.0f) : v[e]);
-      __builtin_memcpy(y + off, out, 8 * sizeof(T));
-    } else {
-      for (int e = 0; e < 8 && oc0 + e < p.oc; ++e) {
-        float t = v[e];
-        if (residual) t += p.residual_scale * (float)residual[off + e];
-        y[off + e] = (T)(p.relu ? fmaxf(t, 0.0f) : t);
+      for (int e = 0; e < 8; ++e) v[e] = v[e] * sc[e] + sh[e];
+      if (full) {
+        T out[8];
+        if (residual) {
+          T rv[8];
+          __builtin_memcpy(rv, residual + off, 8 * sizeof(T));
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] += p.residual_scale * (float)rv[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[e] = (T)(p.relu ? fmaxf(v[e], 0.0f) : v[e]);
+        __builtin_memcpy(y + off, out, 8 * sizeof(T));
+      } else {
+        for (int e = 0; e < 8 && oc0 + e < p.oc; ++e) {
+          float t = v[e];
+          if (residual) t += p.residual_scale * (float)residual[off + e];
+          y[off + e] = (T)(p.relu ? fmaxf(t, 0.0f) : t);
+        }
       }
     }
   }
@@ -441,12 +449,16 @@ SplitReduceKernel(const float* __restrict__ workspace, T* y, const float* __rest
 
 // ---- host side ------------------------------------------------------------------------------------------------
 struct TileChoice {
-  int bm, bn;
+  int bm, bn, waves;
 };
 
-int LdsBytes(int bm, int bn) {
+// two operand stages; the epilogue stages the fp32 tile in the same memory, whole if it fits, else one wavefront row
+// (bm / wm rows) at a time
+int LdsBytes(int bm, int bn, int wm) {
   int stages  = 2 * (bm + bn) * kRowBytes;
-  int staging = bm * (bn + 8) * 4;
+  int whole   = bm * (bn + 8) * 4;
+  if (whole <= stages) return stages;
+  int staging = (bm / wm) * (bn + 8) * 4;
   return stages > staging ? stages : staging;
 }
 
@@ -459,8 +471,8 @@ TileChoice ChooseTile(int pixels, int oc) {
     const char* e = getenv("FLAGS_cinn_hip_conv_tile");
     return e ? atoi(e) : -1;
   }();
-  const TileChoice options[3] = {{128, 128}, {128, 64}, {64, 64}};
-  if (forced >= 0 && forced < 3) return options[forced];
+  const TileChoice options[4] = {{128, 128, 4}, {128, 64, 4}, {64, 64, 4}, {128, 128, 8}};
+  if (forced >= 0 && forced < 4) return options[forced];
   (void)pixels;
   (void)oc;
   return options[2];
@@ -508,12 +520,11 @@ int ChooseSplits(int tiles, int steps) {
   return splits;
 }
 
-template <typename T, int BM, int BN, bool NCHW_IN>
+template <typename T, int BM, int BN, int WM, int WN, bool NCHW_IN>
 void Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream) {
-  // steps in flight per block: what the register budget of the tile allows
-  constexpr int PF = 2;
-  auto kernel      = conv_nhwc_mfma_kernel<T, BM, BN, NCHW_IN, PF>;
-  const int bytes = LdsBytes(BM, BN);
+  constexpr int PF = 2;  // K steps in flight per block
+  auto kernel      = conv_nhwc_mfma_kernel<T, BM, BN, WM, WN, NCHW_IN, PF>;
+  const int bytes  = LdsBytes(BM, BN, WM);
   static bool configured = false;
   if (!configured) {
     CINN_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
@@ -528,7 +539,7 @@ void Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream) {
   p.splits              = (steps + p.steps_per_split - 1) / p.steps_per_split;
   float* workspace      = nullptr;
   if (p.splits > 1) workspace = Workspace((size_t)p.splits * p.pixels * p.oc * sizeof(float));
-  hipLaunchKernelGGL(kernel, dim3(tiles, p.splits), dim3(kThreads), bytes, stream, static_cast<const T*>(a.x),
+  hipLaunchKernelGGL(kernel, dim3(tiles, p.splits), dim3(64 * WM * WN), bytes, stream, static_cast<const T*>(a.x),
                      static_cast<const T*>(a.w), static_cast<T*>(a.y), a.scale, a.shift, static_cast<const T*>(a.residual),
                      workspace, ZeroPage(), p);
   CINN_HIP_CALL(hipGetLastError());
@@ -550,19 +561,20 @@ template <typename T>
 void Dispatch(const ConvNhwcArgs& a, const Params& p, hipStream_t stream) {
   TileChoice t = ChooseTile(p.pixels, p.oc);
   if (a.nchw_input) {
-    if (t.bm == 128 && t.bn == 128) t.bn = 64;
     if (t.bm == 128)
-      Launch<T, 128, 64, true>(a, p, stream);
+      Launch<T, 128, 64, 2, 2, true>(a, p, stream);
     else
-      Launch<T, 64, 64, true>(a, p, stream);
+      Launch<T, 64, 64, 2, 2, true>(a, p, stream);
     return;
   }
-  if (t.bm == 128 && t.bn == 128)
-    Launch<T, 128, 128, false>(a, p, stream);
+  if (t.bm == 128 && t.bn == 128 && t.waves == 8)
+    Launch<T, 128, 128, 2, 4, false>(a, p, stream);
+  else if (t.bm == 128 && t.bn == 128)
+    Launch<T, 128, 128, 2, 2, false>(a, p, stream);
   else if (t.bm == 128)
-    Launch<T, 128, 64, false>(a, p, stream);
+    Launch<T, 128, 64, 2, 2, false>(a, p, stream);
   else
-    Launch<T, 64, 64, false>(a, p, stream);
+    Launch<T, 64, 64, 2, 2, false>(a, p, stream);
 }
 
 int ChunkElems(const cinn_type_t& t) { return 16 / (t.bits / CHAR_BIT); }

@@ -3,8 +3,9 @@
 //   C[M,N] = alpha * op(A)[M,K] * op(B)[K,N] + beta * C          (row-major, optional batch)
 //
 // Four kernels:
-//   * gemm16_dma_kernel   - bf16 / fp16 with A stored [M][K] (the common case): 256x256x64 tile, 512 threads, direct
-//     global -> LDS loads, transposing LDS reads for row-major B; see the comment at the kernel.
+//   * gemm16_dma_kernel   - bf16 / fp16 with A stored [M][K] (the common case) and K % 128 == 0: 256x256x32 tile, 512
+//     threads, direct global -> LDS loads into a 4-stage ring, transposing LDS reads for row-major B; see the comment
+//     at the kernel.
 //   * gemm16_mfma_kernel  - bf16 / fp16 inputs, any operand layout (used for transposed A), fp32 accumulation on v_mfma_f32_32x32x16_{bf16,f16}.
 //     256x256 block tile, 64-deep K step, 256 threads = 4 wavefronts in a 2x2 grid, each wavefront owning a
 //     128x128 tile (16 MFMA accumulator tiles = 256 accumulator registers).  Both operand tiles live in LDS
@@ -210,24 +211,42 @@ gemm16_mfma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ 
 
 // ---------------------------------------------------------------------------------------------------
 // bf16 / fp16 with A stored [M][K]: direct global -> LDS loads (global_load_lds_dwordx4), 8 wavefronts.
-// 256x256x64 block tile, 512 threads in a 2 (M) x 4 (N) wavefront grid, each wavefront a 128x64 tile (8 MFMA
+// 256x256 block tile, K step 32, 512 threads in a 2 (M) x 4 (N) wavefront grid, each wavefront a 128x64 tile (8 MFMA
 // accumulators), two wavefronts per SIMD so that one runs MFMAs while the other waits for LDS or the barrier.
-// A lane of a load instruction writes its 16 bytes at LDS base + 16 * lane, so the swizzle that makes the fragment
-// reads conflict free is applied on the global side: each lane fetches the chunk that belongs at its LDS slot.
-// B stored [K][N] (the plain row-major matmul) is kept as [k][n] in LDS and read with ds_read_b64_tr_b16, which
-// hands every lane four consecutive k of one column - no transposition in registers.  Two LDS stages of 64 KiB in
-// two separate arrays: the loads of step k+1 are in flight during the MFMAs of step k, and the compiler can tell
-// that they do not alias the stage being read.  Fragment reads are issued one MFMA group ahead.
-// Measured on MI355X the direct-to-LDS path sustains about 27 bytes per clock and CU - close to the 32 a 256x256
-// tile needs at the full MFMA rate - which is what bounds this kernel (about 1.0 PFLOP/s at 4096^3).
+//   * A lane of a load instruction writes its 16 bytes at LDS base + 16 * lane, so the swizzle that makes the fragment
+//     reads conflict free is applied on the global side: each lane fetches the chunk that belongs at its LDS slot.
+//   * B stored [K][N] (the plain row-major matmul) is kept as [k][n] in LDS and read with ds_read_b64_tr_b16, which
+//     hands every lane four consecutive k of one column - no transposition in registers.
+//   * Four LDS stages of 32 KiB in four separate arrays.  At the barrier of step s every wavefront knows that the
+//     tiles of step s+1 have landed and that nobody reads the tiles of step s-1 any more: the loads of step s+3 go
+//     there.  The loads are issued through inline assembly, one between every four MFMAs: the compiler neither
+//     tracks them (its conservative s_waitcnt vmcnt(0) before LDS reads would serialise the ring - the waits here are
+//     explicit vmcnt(4)) nor lets a wavefront queue all its loads at once, which stalls it behind the address unit
+//     while the MFMA pipe idles.
+//   * The first fragments of step s+1 are fetched while the MFMAs of step s still run, so no LDS read is exposed
+//     after a barrier.
+// Measured on MI355X the direct-to-LDS path sustains about 27 bytes per clock and CU, a 256x256 tile needs 32 at the
+// full MFMA rate: the kernel is bound by that path (about 1.05-1.1 PFLOP/s at 4096^3).
+// Requires M % 256 == N % 256 == K % 128 == 0.
 // ---------------------------------------------------------------------------------------------------
 constexpr int kDmaThreads = 512;
+constexpr int kDmaBK      = 32;
+constexpr int kDmaTile    = kBM * kDmaBK * 2;  // one operand tile of a stage: 16 KiB
+constexpr int kDmaStage   = 2 * kDmaTile;
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 
+// rows of 64 bytes (4 chunks): byte offset of chunk `chunk` of row `row`
+__device__ __forceinline__ int DmaTileOffset(int row, int chunk) {
+  int key = (row >> 2) & 3;
+  return row * 64 + ((chunk ^ key) << 4);
+}
+
+// 16 bytes per lane from global memory straight into LDS at lds_base + 16 * lane
 __device__ __forceinline__ void AsyncCopy16(const void* src, char* lds_base_uniform) {
-  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                   (__attribute__((address_space(3))) void*)lds_base_uniform, 16, 0, 0);
+  unsigned lds_addr =
+      __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) char*)lds_base_uniform);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(src) : "memory");
 }
 
 template <typename T, bool B_KC>
@@ -235,8 +254,10 @@ __global__ void __launch_bounds__(kDmaThreads)
 gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ C, int M, int N,
                   int K, int64_t lda, int64_t ldb, int64_t ldc, float alpha, float beta, int64_t stride_a,
                   int64_t stride_b, int64_t stride_c) {
-  __shared__ __attribute__((aligned(1024))) char s0[kStageBytes];
-  __shared__ __attribute__((aligned(1024))) char s1[kStageBytes];
+  __shared__ __attribute__((aligned(1024))) char s0[kDmaStage];
+  __shared__ __attribute__((aligned(1024))) char s1[kDmaStage];
+  __shared__ __attribute__((aligned(1024))) char s2[kDmaStage];
+  __shared__ __attribute__((aligned(1024))) char s3[kDmaStage];
   typedef typename Half16<T>::vec8 vec8;
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
@@ -254,30 +275,32 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   B += (int64_t)blockIdx.y * stride_b;
   C += (int64_t)blockIdx.y * stride_c;
 
-  // Each wavefront issues 4 loads per operand and step; load q = 4 wave + t fills LDS bytes [1024 q, 1024 q + 1024)
-  // of the operand tile: 8 rows of a [row][64 halves] tile, or 2 k-rows of a [k][256 halves] tile.
-  const uint16_t* a_src[4];
-  const uint16_t* b_src[4];
+  // Each wavefront issues 2 loads per operand and step; load q = 2 wave + t fills LDS bytes [1024 q, 1024 q + 1024)
+  // of the operand tile: 16 rows of a [row][32 halves] tile, or 2 k-rows of a [k][256 halves] tile.
+  const uint16_t* a_src[2];
+  const uint16_t* b_src[2];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    const int q   = wave * 4 + t;
-    const int row = 8 * q + (lane >> 3);
-    const int key = (row ^ (row >> 3)) & 7;
-    a_src[t]      = A + (int64_t)(m0 + row) * lda + (((lane & 7) ^ key) << 3);
+  for (int t = 0; t < 2; ++t) {
+    const int q   = wave * 2 + t;
+    const int row = 16 * q + (lane >> 2);
+    const int key = (row >> 2) & 3;
+    a_src[t]      = A + (int64_t)(m0 + row) * lda + (((lane & 3) ^ key) << 3);
     if (B_KC) {
-      b_src[t] = B + (int64_t)(n0 + row) * ldb + (((lane & 7) ^ key) << 3);
+      b_src[t] = B + (int64_t)(n0 + row) * ldb + (((lane & 3) ^ key) << 3);
     } else {
       const int krow  = 2 * q + (lane >> 5);
       const int chunk = (lane & 31) ^ (2 * (krow & 3));
       b_src[t]        = B + (int64_t)krow * ldb + n0 + (chunk << 3);
     }
   }
-  const int64_t b_step = B_KC ? kBK : (int64_t)kBK * ldb;
-  auto issue = [&](char* stage, int kt) {
-#pragma unroll
-    for (int t = 0; t < 4; ++t) AsyncCopy16(a_src[t] + (int64_t)kt * kBK, stage + (wave * 4 + t) * 1024);
-#pragma unroll
-    for (int t = 0; t < 4; ++t) AsyncCopy16(b_src[t] + kt * b_step, stage + kTileBytes + (wave * 4 + t) * 1024);
+  const int64_t b_step = B_KC ? kDmaBK : (int64_t)kDmaBK * ldb;
+  // load t of step kt: 0, 1 the A tile, 2, 3 the B tile
+  auto issue_one = [&](char* stage, int kt, int t) {
+    if (t < 2) {
+      AsyncCopy16(a_src[t] + (int64_t)kt * kDmaBK, stage + (wave * 2 + t) * 1024);
+    } else {
+      AsyncCopy16(b_src[t - 2] + kt * b_step, stage + kDmaTile + (wave * 2 + t - 2) * 1024);
+    }
   };
 
   f32x16 acc[4][2];
@@ -292,14 +315,14 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   const int frag_kg  = lane >> 5;
   auto load_frags = [&](const char* cur, int kk, vec8 (&af)[4], vec8 (&bf)[2]) {
     const char* a_tile = cur;
-    const char* b_tile = cur + kTileBytes;
+    const char* b_tile = cur + kDmaTile;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      af[i] = *reinterpret_cast<const vec8*>(a_tile + TileOffset(wm * 128 + i * 32 + frag_row, kk * 2 + frag_kg));
+      af[i] = *reinterpret_cast<const vec8*>(a_tile + DmaTileOffset(wm * 128 + i * 32 + frag_row, kk * 2 + frag_kg));
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       if (B_KC) {
-        bf[j] = *reinterpret_cast<const vec8*>(b_tile + TileOffset(wn * 64 + j * 32 + frag_row, kk * 2 + frag_kg));
+        bf[j] = *reinterpret_cast<const vec8*>(b_tile + DmaTileOffset(wn * 64 + j * 32 + frag_row, kk * 2 + frag_kg));
       } else {
         // one transposing read returns k = kb .. kb+3 of column n to the lane that owns n: lane j of each group of
         // 16 supplies the address of row kb + j/4, columns nb + 4 (j%4) .. +3
@@ -316,50 +339,67 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
       }
     }
   };
-  auto mma = [&](vec8 (&af)[4], vec8 (&bf)[2]) {
+  // MFMAs of accumulator rows i0, i0 + 1
+  auto mma_part = [&](vec8 (&af)[4], vec8 (&bf)[2], int i0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = i0; i < i0 + 2; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j) acc[i][j] = Half16<T>::mfma(af[i], bf[j], acc[i][j]);
   };
-  // fragments of the next 16-deep slice are requested before the MFMAs of the current one are issued; the scheduling
-  // barriers keep the compiler from sinking the reads back to their uses
-  auto compute = [&](const char* cur) {
-    vec8 a0[4], b0[2], a1[4], b1[2];
-    load_frags(cur, 0, a0, b0);
-    __builtin_amdgcn_sched_barrier(0);
-    load_frags(cur, 1, a1, b1);
-    __builtin_amdgcn_sched_barrier(0);
-    mma(a0, b0);
-    __builtin_amdgcn_sched_barrier(0);
-    load_frags(cur, 2, a0, b0);
-    __builtin_amdgcn_sched_barrier(0);
-    mma(a1, b1);
-    __builtin_amdgcn_sched_barrier(0);
-    load_frags(cur, 3, a1, b1);
-    __builtin_amdgcn_sched_barrier(0);
-    mma(a0, b0);
-    __builtin_amdgcn_sched_barrier(0);
-    mma(a1, b1);
-    __builtin_amdgcn_sched_barrier(0);
-  };
 
-  const int nk = K / kBK;
-  issue(s0, 0);
-  for (int kt = 0; kt < nk; kt += 2) {
-    // every load of this wavefront has landed; after the barrier so have everybody's, and nobody still reads the
-    // other stage
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    __syncthreads();
-    if (kt + 1 < nk) issue(s1, kt + 1);
-    compute(s0);
-    if (kt + 1 < nk) {
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-      __syncthreads();
-      if (kt + 2 < nk) issue(s0, kt + 2);
-      compute(s1);
-    }
+  const int nk = K / kDmaBK;  // a multiple of 4
+  vec8 a0[4], b0[2], a1[4], b1[2];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) issue_one(s0, 0, t);
+#pragma unroll
+  for (int t = 0; t < 4; ++t) issue_one(s1, 1, t);
+#pragma unroll
+  for (int t = 0; t < 4; ++t) issue_one(s2, 2, t);
+  __builtin_amdgcn_s_waitcnt(0x0F70 | 8);  // vmcnt(8): step 0 has landed
+  __syncthreads();
+  load_frags(s0, 0, a0, b0);
+#define CINN_SB __builtin_amdgcn_sched_barrier(0)
+  // s_waitcnt immediates: vmcnt in bits 3:0 (15:14 zero), expcnt 7 and lgkmcnt 15 = no wait on those
+#define CINN_GEMM_STEP(CUR, NEXT1, FREE, OFF)                                              \
+  {                                                                                        \
+    const int s = kt + OFF;                                                                \
+    if (s + 2 < nk) {                                                                      \
+      __builtin_amdgcn_s_waitcnt(0x0F70 | 4); /* all but the loads of step s+2 are done */ \
+    } else {                                                                               \
+      __builtin_amdgcn_s_waitcnt(0x0F70);                                                  \
+    }                                                                                      \
+    __syncthreads();                                                                       \
+    const bool more = s + 3 < nk;                                                          \
+    CINN_SB;                                                                               \
+    load_frags(CUR, 1, a1, b1);                                                            \
+    CINN_SB;                                                                               \
+    if (more) issue_one(FREE, s + 3, 0);                                                   \
+    CINN_SB;                                                                               \
+    mma_part(a0, b0, 0);                                                                   \
+    CINN_SB;                                                                               \
+    if (more) issue_one(FREE, s + 3, 1);                                                   \
+    CINN_SB;                                                                               \
+    mma_part(a0, b0, 2);                                                                   \
+    CINN_SB;                                                                               \
+    load_frags(NEXT1, 0, a0, b0); /* past the last step: a harmless read of stale data */  \
+    CINN_SB;                                                                               \
+    if (more) issue_one(FREE, s + 3, 2);                                                   \
+    CINN_SB;                                                                               \
+    mma_part(a1, b1, 0);                                                                   \
+    CINN_SB;                                                                               \
+    if (more) issue_one(FREE, s + 3, 3);                                                   \
+    CINN_SB;                                                                               \
+    mma_part(a1, b1, 2);                                                                   \
+    CINN_SB;                                                                               \
   }
+  for (int kt = 0; kt < nk; kt += 4) {
+    CINN_GEMM_STEP(s0, s1, s3, 0)
+    CINN_GEMM_STEP(s1, s2, s0, 1)
+    CINN_GEMM_STEP(s2, s3, s1, 2)
+    CINN_GEMM_STEP(s3, s0, s2, 3)
+  }
+#undef CINN_GEMM_STEP
+#undef CINN_SB
 
   T* Ct = reinterpret_cast<T*>(C);
 #pragma unroll
@@ -564,72 +604,6 @@ gemm_generic_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restr
 
 enum class GemmType { kF16, kBF16, kF32, kF64 };
 
-// ---------------------------------------------------------------------------------------------------
-// Skinny GEMM: C[m][n] = alpha * sum_k A[m][k] * Bt[n][k] + beta * C for a handful of rows m (a classifier layer on
-// one batch).  The work is reading Bt once, so there is no tile to fill: one wavefront owns NC output columns, its
-// lanes split K in 16-byte chunks, products accumulate in fp32 and a butterfly over the wavefront finishes each sum.
-// ---------------------------------------------------------------------------------------------------
-template <typename T, int MT, int NC>
-__global__ void __launch_bounds__(256)
-skinny_gemm_kernel(const T* __restrict__ A, const T* __restrict__ Bt, T* C, int M, int N, int K, float alpha, float beta) {
-  constexpr int E = 16 / sizeof(T);
-  const int lane  = threadIdx.x & 63;
-  const int n0    = (blockIdx.x * 4 + (threadIdx.x >> 6)) * NC;
-  if (n0 >= N) return;
-  for (int mb = 0; mb < M; mb += MT) {
-    float acc[MT][NC];
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-      for (int c = 0; c < NC; ++c) acc[m][c] = 0.0f;
-    for (int k = lane * E; k < K; k += 64 * E) {
-      T b[NC][E];
-#pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        if (n0 + c < N) {
-          __builtin_memcpy(b[c], Bt + (int64_t)(n0 + c) * K + k, 16);
-        } else {
-#pragma unroll
-          for (int e = 0; e < E; ++e) b[c][e] = (T)0.0f;
-        }
-      }
-#pragma unroll
-      for (int m = 0; m < MT; ++m) {
-        if (mb + m < M) {
-          T a[E];
-          __builtin_memcpy(a, A + (int64_t)(mb + m) * K + k, 16);
-#pragma unroll
-          for (int c = 0; c < NC; ++c)
-#pragma unroll
-            for (int e = 0; e < E; ++e) acc[m][c] += (float)a[e] * (float)b[c][e];
-        }
-      }
-    }
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        float v = acc[m][c];
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-        if (lane == 0 && mb + m < M && n0 + c < N) {
-          T* dst  = C + (int64_t)(mb + m) * N + n0 + c;
-          float r = alpha * v;
-          if (beta != 0.0f) r += beta * (float)*dst;
-          *dst = (T)r;
-        }
-      }
-  }
-}
-
-template <typename T>
-void LaunchSkinny(const void* a, const void* b, void* c, int m, int n, int k, float alpha, float beta, hipStream_t stream) {
-  constexpr int NC = 2;
-  const int waves  = (n + NC - 1) / NC;
-  hipLaunchKernelGGL((skinny_gemm_kernel<T, 16, NC>), dim3((waves + 3) / 4), dim3(256), 0, stream, static_cast<const T*>(a),
-                     static_cast<const T*>(b), static_cast<T*>(c), m, n, k, alpha, beta);
-}
-
 struct GemmProblem {
   GemmType type;
   const void* a;
@@ -676,7 +650,7 @@ bool UseRegisterStaging() {
 template <typename T>
 void DispatchFast16(const GemmProblem& p, hipStream_t stream) {
   bool a_kc = !p.trans_a, b_kc = p.trans_b;
-  if (a_kc && !UseRegisterStaging()) {
+  if (a_kc && p.k % 128 == 0 && !UseRegisterStaging()) {
     if (b_kc) {
       LaunchDma16<T, true>(p, stream);
     } else {
@@ -743,20 +717,6 @@ void RunGemm(const GemmProblem& p, hipStream_t stream) {
   const int elem_bytes = p.type == GemmType::kF32 ? 4 : (p.type == GemmType::kF64 ? 8 : 2);
   const bool tile_fit  = p.type == GemmType::kF32 ? fast32 : fast16;
   const bool k_contig  = !ForceGeneric() && p.type != GemmType::kF64 && !p.trans_a && p.trans_b && p.k % (16 / elem_bytes) == 0;
-  if (k_contig && p.m <= 64) {
-    for (int b = 0; b < p.batch; ++b) {
-      const char* a = static_cast<const char*>(p.a) + (int64_t)b * p.stride_a * elem_bytes;
-      const char* w = static_cast<const char*>(p.b) + (int64_t)b * p.stride_b * elem_bytes;
-      char* c       = static_cast<char*>(p.c) + (int64_t)b * p.stride_c * elem_bytes;
-      switch (p.type) {
-        case GemmType::kBF16: LaunchSkinny<__bf16>(a, w, c, p.m, p.n, p.k, p.alpha, p.beta, stream); break;
-        case GemmType::kF16: LaunchSkinny<_Float16>(a, w, c, p.m, p.n, p.k, p.alpha, p.beta, stream); break;
-        default: LaunchSkinny<float>(a, w, c, p.m, p.n, p.k, p.alpha, p.beta, stream); break;
-      }
-    }
-    CINN_HIP_CALL(hipGetLastError());
-    return;
-  }
   if (k_contig && !tile_fit) {
     for (int b = 0; b < p.batch; ++b) {
       cinn_hip_kernels::ConvNhwcArgs a;
