@@ -280,7 +280,10 @@ void Graph::BuildFusionGroups() {
     }
     for (Node* n : g->nodes) {
       for (auto* in : n->inputs) {
-        if (!produced.count(in) && std::find(g->inputs.begin(), g->inputs.end(), in) == g->inputs.end())
+        // a library call takes its operands by position: the same value may be passed twice (a residual that is
+        // also the convolution's input); generated kernels take every value once
+        bool by_position = g->kind == GroupKind::kLibraryCall;
+        if (!produced.count(in) && (by_position || std::find(g->inputs.begin(), g->inputs.end(), in) == g->inputs.end()))
           g->inputs.push_back(in);
       }
       for (auto* o : n->outputs) {

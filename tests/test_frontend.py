@@ -175,3 +175,67 @@ def test_generated_source_idioms():
     assert "(int32_t)blockIdx.x" in src and "(int32_t)threadIdx.x" in src
     assert "2.0f" in src and "0.5f" in src
     assert re.search(r"if \(.*< 750\)", src)  # 3000 / 4 vectors
+
+
+# ---- program passes for convolutional networks (compile only: hiprtc needs no GPU) -------------------------------------
+def _conv_net(const_params, dtype=None):
+    from cinn_amd.common import Float
+    T = dtype or Float(32)
+    b = NetBuilder("convnet")
+    x = b.create_input(T, [2, 16, 12, 12], "x")
+    w1 = b.create_input(T, [32, 16, 3, 3], "w1")
+    w2 = b.create_input(T, [32, 32, 1, 1], "w2")
+    stats = [b.create_input(T, [32], n) for n in ("scale", "bias", "mean", "var")]
+    fc = b.create_input(T, [32, 10], "fc")
+    if const_params:
+        for v in [w1, w2, fc] + stats:
+            v.set_const()
+    y = b.relu(b.batchnorm(b.conv2d(x, w1, strides=[1, 1], paddings=[1, 1]), *stats)[0])
+    z = b.batchnorm(b.conv2d(y, w2), *stats)[0]
+    y = b.relu(b.add(z, y))
+    y = b.pool2d(y, "avg", [12, 12], global_pooling=True)
+    logits = b.matmul(b.reshape(y, [2, 32]), fc)
+    return b, logits
+
+
+def test_conv_chain_moves_to_channels_last_and_back_only_at_the_ends():
+    b, logits = _conv_net(const_params=False)
+    comp = compile_only(b, [logits])
+    groups = comp.fusion_groups()
+    # one transpose of the input, one per 3x3 filter; the 1x1 filter and the pooled [N,C,1,1] tensor are reshapes
+    assert groups.count("transpose") == 2, groups
+    assert "hip_conv2d_bn_relu" not in groups
+    src = comp.source_code()
+    assert "fn_convnet" in src
+    off = compile_only(_conv_net(False)[0], [_conv_net(False)[1]], conv_layout_nhwc=False) if False else None
+    b2, l2 = _conv_net(const_params=False)
+    nchw = compile_only(b2, [l2], conv_layout_nhwc=False)
+    assert "transpose" not in nchw.fusion_groups()
+
+
+def test_const_inputs_make_pre_run_groups_and_broadcasts_stay_in_place():
+    b, logits = _conv_net(const_params=True)
+    comp = compile_only(b, [logits])
+    groups = comp.fusion_groups().splitlines()
+    pre = [g for g in groups if " pre_run " in g]
+    run = [g for g in groups if " pre_run " not in g and g.strip()]
+    # filter layout changes, sqrt(var + eps) and the transposed classifier weight run once
+    assert any("transpose" in g and "w1" in g for g in pre), pre
+    assert any("sqrt" in g for g in pre), pre
+    assert any("transpose" in g and " fc" in g for g in pre), pre
+    # replicating a const vector is never materialised ahead of time
+    assert not any("broadcast_to" in g for g in pre), pre
+    assert comp.num_instructions() == len(run)
+
+
+def test_conv_batch_norm_residual_relu_fold_into_convolution_epilogues():
+    b, logits = _conv_net(const_params=True)
+    comp = compile_only(b, [logits], fuse_conv_bn_relu=True)
+    groups = comp.fusion_groups().splitlines()
+    fused = [g for g in groups if "hip_conv2d_bn_relu" in g]
+    assert len(fused) == 2, groups
+    # the second convolution takes the residual as a fifth input
+    assert len(fused[1].split(" in: ")[1].split(" out: ")[0].split()) == 5, fused[1]
+    assert not any("batch_norm" in g or " relu " in g for g in groups if " pre_run " not in g), groups
+    # scale / shift of the folded batch norm are computed in fp32 ahead of time
+    assert any("pre_run" in g and "divide" in g and "subtract" in g for g in groups), groups

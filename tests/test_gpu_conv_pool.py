@@ -211,3 +211,38 @@ def test_log_softmax_intrinsic(gpu):
         x64 = x.astype(np.float64)
         want = x64 - np.log(np.exp(x64).sum(axes, keepdims=True))
         np.testing.assert_allclose(Y.numpy(), want, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("fuse", [False, True])
+def test_residual_that_is_also_the_convolution_input(gpu, fuse):
+    """y = relu(bn(conv1x1(t)) + t): the fused call receives t twice, as input and as residual."""
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((2, 16, 9, 9)).astype(np.float32)
+    w1 = (rng.standard_normal((32, 16, 3, 3)) * 0.1).astype(np.float32)
+    w2 = (rng.standard_normal((32, 32, 1, 1)) * 0.2).astype(np.float32)
+    stats = [rng.uniform(0.5, 1.5, 32).astype(np.float32), rng.uniform(-0.5, 0.5, 32).astype(np.float32),
+             (rng.standard_normal(32) * 0.1).astype(np.float32), rng.uniform(0.5, 1.5, 32).astype(np.float32)]
+    b = NetBuilder("res")
+    X = b.create_input(Float(32), x.shape, "x")
+    W1, W2 = b.create_input(Float(32), w1.shape, "w1"), b.create_input(Float(32), w2.shape, "w2")
+    P = [b.create_input(Float(32), [32], n) for n in ("scale", "bias", "mean", "var")]
+    t = b.relu(b.batchnorm(b.conv2d(X, W1, strides=[1, 1], paddings=[1, 1]), *P)[0])
+    y = b.relu(b.add(b.batchnorm(b.conv2d(t, W2), *P)[0], t))
+    feeds = {X: x, W1: w1, W2: w2}
+    feeds.update(dict(zip(P, stats)))
+    (got,), comp = run(b, feeds, [y], fuse_conv_bn_relu=fuse)
+    t_ref = oracle.batch_norm_relu_nchw(oracle.conv2d_nchw(x, w1, (1, 1), (1, 1)), *stats, 1e-5, relu=True)
+    z_ref = oracle.batch_norm_relu_nchw(oracle.conv2d_nchw(t_ref, w2, (1, 1), (0, 0)), *stats, 1e-5, relu=False)
+    want = np.maximum(z_ref + t_ref, 0)
+    np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
+    if fuse:
+        assert comp.fusion_groups().count("hip_conv2d_bn_relu") == 2
+
+
+def test_matmul_of_a_matrix_with_itself(gpu):
+    rng = np.random.default_rng(22)
+    a = rng.standard_normal((48, 48)).astype(np.float32)
+    b = NetBuilder("sq")
+    A = b.create_input(Float(32), a.shape, "a")
+    (got,), _ = run(b, {A: a}, [b.matmul(A, A)])
+    np.testing.assert_allclose(got, oracle.matmul(a, a), rtol=1e-5, atol=1e-5)
