@@ -21,8 +21,10 @@ class CinnComputation {
     // generated from primitives only
     bool use_decomposer{true};
     bool do_prerun{true};
-    // fold `conv2d -> batch_norm [-> relu]` into one convolution call with a fused epilogue
-    bool fuse_conv_bn_relu{false};
+    // fold `conv2d -> batch_norm [-> + residual] [-> relu]` on channels-last tensors into one convolution call whose
+    // epilogue applies the folded batch norm in fp32 on the accumulators (frontend/layout_pass.h).  The result
+    // differs from the unfused operation order by rounding only; switch it off to get that order exactly.
+    bool fuse_conv_bn_relu{true};
     // move conv2d chains written in NCHW to channels-last tensors, the layout the MFMA convolution kernels read
     // with 16-byte accesses (frontend/layout_pass.h); off: every conv2d runs in the layout it was written in
     bool conv_layout_nhwc{true};

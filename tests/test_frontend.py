@@ -200,14 +200,13 @@ def _conv_net(const_params, dtype=None):
 
 def test_conv_chain_moves_to_channels_last_and_back_only_at_the_ends():
     b, logits = _conv_net(const_params=False)
-    comp = compile_only(b, [logits])
+    comp = compile_only(b, [logits], fuse_conv_bn_relu=False)
     groups = comp.fusion_groups()
     # one transpose of the input, one per 3x3 filter; the 1x1 filter and the pooled [N,C,1,1] tensor are reshapes
     assert groups.count("transpose") == 2, groups
     assert "hip_conv2d_bn_relu" not in groups
     src = comp.source_code()
     assert "fn_convnet" in src
-    off = compile_only(_conv_net(False)[0], [_conv_net(False)[1]], conv_layout_nhwc=False) if False else None
     b2, l2 = _conv_net(const_params=False)
     nchw = compile_only(b2, [l2], conv_layout_nhwc=False)
     assert "transpose" not in nchw.fusion_groups()
@@ -215,7 +214,7 @@ def test_conv_chain_moves_to_channels_last_and_back_only_at_the_ends():
 
 def test_const_inputs_make_pre_run_groups_and_broadcasts_stay_in_place():
     b, logits = _conv_net(const_params=True)
-    comp = compile_only(b, [logits])
+    comp = compile_only(b, [logits], fuse_conv_bn_relu=False)
     groups = comp.fusion_groups().splitlines()
     pre = [g for g in groups if " pre_run " in g]
     run = [g for g in groups if " pre_run " not in g and g.strip()]
@@ -230,7 +229,7 @@ def test_const_inputs_make_pre_run_groups_and_broadcasts_stay_in_place():
 
 def test_conv_batch_norm_residual_relu_fold_into_convolution_epilogues():
     b, logits = _conv_net(const_params=True)
-    comp = compile_only(b, [logits], fuse_conv_bn_relu=True)
+    comp = compile_only(b, [logits])  # folding is the default
     groups = comp.fusion_groups().splitlines()
     fused = [g for g in groups if "hip_conv2d_bn_relu" in g]
     assert len(fused) == 2, groups

