@@ -171,7 +171,8 @@ def extra_measurements(stream, runtime):
     import bench_resnet50  # configs[4]: whole-network images/s, HIP-graph replay of the compiled program
     for dtype in ("float16", "float32"):
         r = bench_resnet50.measure(batch=32, dtype=dtype, steps=20, warmup=3)
-        out[r.pop("workload")] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in r.items()}
+        name = r.pop("workload")
+        out[name] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in r.items()}
     return out
 
 
