@@ -150,7 +150,9 @@ void cinn_call_batched_cublas(void* v_args, int num_args, int opside, bool trans
 
 /* y = alpha * conv2d(x, w) + beta * y, cross-correlation, zero padding, as an implicit GEMM on
  * MFMA.  Replaces cinn_call_cudnn_conv2d_forward (cuda_util.cc:603-720).  format: 0 = NCHW,
- * 1 = NHWC (cudnnTensorFormat_t values).  v_args = {x, w, y}. */
+ * 1 = NHWC with [O][KH][KW][I] filters (cudnnTensorFormat_t values), 2 = NHWC output from an NCHW
+ * input and [O][I][KH][KW] filter (for inputs with few channels).  Extents are passed in
+ * n, c, h, w order whatever the format.  Groups need format 0.  v_args = {x, w, y}. */
 void cinn_call_cudnn_conv2d_forward(void* v_args, int num_args, int format, float alpha, float beta, int input_n,
                                     int input_c, int input_h, int input_w, int filter_n, int filter_c, int filter_h,
                                     int filter_w, int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h,
@@ -158,9 +160,11 @@ void cinn_call_cudnn_conv2d_forward(void* v_args, int num_args, int format, floa
                                     int output_w, void* stream);
 
 /* Extension with no counterpart in the reference: the same convolution with a per-output-channel
- * affine (y = conv * scale[c] + shift[c]) and optional ReLU applied in the kernel epilogue, so an
- * inference batch_norm + relu that follows a convolution costs no extra pass over HBM.
- * v_args = {x, w, scale, shift, y}; scale/shift are fp32 [output_c]. */
+ * affine (y = conv * scale[c] + shift[c]), an optional residual addition and an optional ReLU
+ * applied in the kernel epilogue on the fp32 accumulators, so an inference batch_norm (+ shortcut
+ * + relu) that follows a convolution costs no extra pass over HBM.
+ * v_args = {x, w, scale, shift, y} or {x, w, scale, shift, residual, y}; scale / shift are fp32
+ * [output_c]; residual has y's shape, type and layout and needs format 1 or 2. */
 void cinn_call_hip_conv2d_bn_relu(void* v_args, int num_args, int format, int relu, int input_n, int input_c,
                                   int input_h, int input_w, int filter_n, int filter_c, int filter_h, int filter_w,
                                   int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
