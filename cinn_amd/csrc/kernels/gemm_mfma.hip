@@ -223,8 +223,9 @@ gemm16_mfma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ 
 //     tracks them (its conservative s_waitcnt vmcnt(0) before LDS reads would serialise the ring - the waits here are
 //     explicit vmcnt(4)) nor lets a wavefront queue all its loads at once, which stalls it behind the address unit
 //     while the MFMA pipe idles.
-//   * The first fragments of step s+1 are fetched while the MFMAs of step s still run, so no LDS read is exposed
-//     after a barrier.
+//   * Every MFMA is followed by exactly one LDS fragment read or one global->LDS load (scheduling barriers pin the
+//     order); fragments are requested 8 MFMAs ahead, those of step s+1 during the MFMAs of step s, so no LDS read is
+//     exposed after a barrier.
 // Measured on MI355X the direct-to-LDS path sustains about 27 bytes per clock and CU, a 256x256 tile needs 32 at the
 // full MFMA rate: the kernel is bound by that path (about 1.05-1.1 PFLOP/s at 4096^3).
 // Requires M % 256 == N % 256 == K % 128 == 0.
@@ -253,7 +254,7 @@ template <typename T, bool B_KC>
 __global__ void __launch_bounds__(kDmaThreads)
 gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ C, int M, int N,
                   int K, int64_t lda, int64_t ldb, int64_t ldc, float alpha, float beta, int64_t stride_a,
-                  int64_t stride_b, int64_t stride_c) {
+                  int64_t stride_b, int64_t stride_c, int xcd_cols, int sub_rows, int sub_cols) {
   __shared__ __attribute__((aligned(1024))) char s0[kDmaStage];
   __shared__ __attribute__((aligned(1024))) char s1[kDmaStage];
   __shared__ __attribute__((aligned(1024))) char s2[kDmaStage];
@@ -265,12 +266,22 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   const int wm   = wave >> 2;
   const int wn   = wave & 3;
 
-  const int tiles_n = N / kBN;
-  const int tiles   = (M / kBM) * tiles_n;
-  int bid           = blockIdx.x;
-  if ((tiles & 7) == 0) bid = (bid & 7) * (tiles >> 3) + (bid >> 3);
-  const int m0 = (bid / tiles_n) * kBM;
-  const int n0 = (bid % tiles_n) * kBN;
+  // Consecutive workgroup ids go round-robin to the 8 XCDs, each with its own L2.  Every XCD gets a compact
+  // sub_rows x sub_cols rectangle of tiles (the XCDs themselves form a (8 / xcd_cols) x xcd_cols grid), so that the
+  // blocks resident on one XCD at a time share as few A and B panels as possible: what misses an L2 crosses the
+  // fabric once per XCD, and that traffic, not the LDS feed, is what bounds this kernel.
+  int tile_row, tile_col;
+  if (sub_rows > 0) {
+    const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+    tile_row = (xcd / xcd_cols) * sub_rows + idx / sub_cols;
+    tile_col = (xcd % xcd_cols) * sub_cols + idx % sub_cols;
+  } else {
+    const int tiles_n = N / kBN;
+    tile_row = blockIdx.x / tiles_n;
+    tile_col = blockIdx.x % tiles_n;
+  }
+  const int m0 = tile_row * kBM;
+  const int n0 = tile_col * kBN;
   A += (int64_t)blockIdx.y * stride_a;
   B += (int64_t)blockIdx.y * stride_b;
   C += (int64_t)blockIdx.y * stride_c;
@@ -313,39 +324,30 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 
   const int frag_row = lane & 31;
   const int frag_kg  = lane >> 5;
-  auto load_frags = [&](const char* cur, int kk, vec8 (&af)[4], vec8 (&bf)[2]) {
-    const char* a_tile = cur;
+  // one A fragment (rows i*32.. of the wavefront tile, 16-deep slice kk) / one B fragment / one MFMA
+  auto read_a = [&](const char* cur, int kk, int i, vec8 (&af)[4]) {
+    af[i] = *reinterpret_cast<const vec8*>(cur + DmaTileOffset(wm * 128 + i * 32 + frag_row, kk * 2 + frag_kg));
+  };
+  auto read_b = [&](const char* cur, int kk, int j, vec8 (&bf)[2]) {
     const char* b_tile = cur + kDmaTile;
+    if (B_KC) {
+      bf[j] = *reinterpret_cast<const vec8*>(b_tile + DmaTileOffset(wn * 64 + j * 32 + frag_row, kk * 2 + frag_kg));
+    } else {
+      // one transposing read returns k = kb .. kb+3 of column n to the lane that owns n: lane j of each group of
+      // 16 supplies the address of row kb + j/4, columns nb + 4 (j%4) .. +3
+      s16x4 part[2];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      af[i] = *reinterpret_cast<const vec8*>(a_tile + DmaTileOffset(wm * 128 + i * 32 + frag_row, kk * 2 + frag_kg));
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      if (B_KC) {
-        bf[j] = *reinterpret_cast<const vec8*>(b_tile + DmaTileOffset(wn * 64 + j * 32 + frag_row, kk * 2 + frag_kg));
-      } else {
-        // one transposing read returns k = kb .. kb+3 of column n to the lane that owns n: lane j of each group of
-        // 16 supplies the address of row kb + j/4, columns nb + 4 (j%4) .. +3
-        s16x4 part[2];
-#pragma unroll
-        for (int r = 0; r < 2; ++r) {
-          const int k   = kk * 16 + 4 * (2 * frag_kg + r) + ((lane & 15) >> 2);
-          const int n   = wn * 64 + j * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-          const int off = k * 512 + (((n >> 3) ^ (2 * (k & 3))) << 4) + (n & 7) * 2;
-          part[r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(b_tile + off));
-        }
-        s16x8 both = __builtin_shufflevector(part[0], part[1], 0, 1, 2, 3, 4, 5, 6, 7);
-        bf[j]      = __builtin_bit_cast(vec8, both);
+      for (int r = 0; r < 2; ++r) {
+        const int k   = kk * 16 + 4 * (2 * frag_kg + r) + ((lane & 15) >> 2);
+        const int n   = wn * 64 + j * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+        const int off = k * 512 + (((n >> 3) ^ (2 * (k & 3))) << 4) + (n & 7) * 2;
+        part[r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(b_tile + off));
       }
+      s16x8 both = __builtin_shufflevector(part[0], part[1], 0, 1, 2, 3, 4, 5, 6, 7);
+      bf[j]      = __builtin_bit_cast(vec8, both);
     }
   };
-  // MFMAs of accumulator rows i0, i0 + 1
-  auto mma_part = [&](vec8 (&af)[4], vec8 (&bf)[2], int i0) {
-#pragma unroll
-    for (int i = i0; i < i0 + 2; ++i)
-#pragma unroll
-      for (int j = 0; j < 2; ++j) acc[i][j] = Half16<T>::mfma(af[i], bf[j], acc[i][j]);
-  };
+  auto mm = [&](vec8 (&af)[4], vec8 (&bf)[2], int i, int j) { acc[i][j] = Half16<T>::mfma(af[i], bf[j], acc[i][j]); };
 
   const int nk = K / kDmaBK;  // a multiple of 4
   vec8 a0[4], b0[2], a1[4], b1[2];
@@ -357,7 +359,10 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   for (int t = 0; t < 4; ++t) issue_one(s2, 2, t);
   __builtin_amdgcn_s_waitcnt(0x0F70 | 8);  // vmcnt(8): step 0 has landed
   __syncthreads();
-  load_frags(s0, 0, a0, b0);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) read_a(s0, 0, i, a0);
+#pragma unroll
+  for (int j = 0; j < 2; ++j) read_b(s0, 0, j, b0);
 #define CINN_SB __builtin_amdgcn_sched_barrier(0)
   // s_waitcnt immediates: vmcnt in bits 3:0 (15:14 zero), expcnt 7 and lgkmcnt 15 = no wait on those
 #define CINN_GEMM_STEP(CUR, NEXT1, FREE, OFF)                                              \
@@ -370,26 +375,26 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     }                                                                                      \
     __syncthreads();                                                                       \
     const bool more = s + 3 < nk;                                                          \
-    CINN_SB;                                                                               \
-    load_frags(CUR, 1, a1, b1);                                                            \
-    CINN_SB;                                                                               \
-    if (more) issue_one(FREE, s + 3, 0);                                                   \
-    CINN_SB;                                                                               \
-    mma_part(a0, b0, 0);                                                                   \
-    CINN_SB;                                                                               \
-    if (more) issue_one(FREE, s + 3, 1);                                                   \
-    CINN_SB;                                                                               \
-    mma_part(a0, b0, 2);                                                                   \
-    CINN_SB;                                                                               \
-    load_frags(NEXT1, 0, a0, b0); /* past the last step: a harmless read of stale data */  \
-    CINN_SB;                                                                               \
-    if (more) issue_one(FREE, s + 3, 2);                                                   \
-    CINN_SB;                                                                               \
-    mma_part(a1, b1, 0);                                                                   \
-    CINN_SB;                                                                               \
-    if (more) issue_one(FREE, s + 3, 3);                                                   \
-    CINN_SB;                                                                               \
-    mma_part(a1, b1, 2);                                                                   \
+    /* every MFMA is followed by one LDS read or one global->LDS load, so that the LDS   */ \
+    /* and address units see an even stream and the wavefront always has MFMAs queued;   */ \
+    /* fragments are requested 8 MFMAs before their use (slice 1 of this step, then       */ \
+    /* slice 0 of the next step, which the barrier above has made visible)                */ \
+    CINN_SB; mm(a0, b0, 0, 0); CINN_SB; read_a(CUR, 1, 0, a1);                             \
+    CINN_SB; mm(a0, b0, 0, 1); CINN_SB; read_b(CUR, 1, 0, b1);                             \
+    CINN_SB; mm(a0, b0, 1, 0); CINN_SB; read_a(CUR, 1, 1, a1);                             \
+    CINN_SB; mm(a0, b0, 1, 1); CINN_SB; read_b(CUR, 1, 1, b1);                             \
+    CINN_SB; mm(a0, b0, 2, 0); CINN_SB; read_a(CUR, 1, 2, a1);                             \
+    CINN_SB; mm(a0, b0, 2, 1); CINN_SB; if (more) issue_one(FREE, s + 3, 0);               \
+    CINN_SB; mm(a0, b0, 3, 0); CINN_SB; read_a(CUR, 1, 3, a1);                             \
+    CINN_SB; mm(a0, b0, 3, 1); CINN_SB; if (more) issue_one(FREE, s + 3, 1);               \
+    CINN_SB; mm(a1, b1, 0, 0); CINN_SB; read_a(NEXT1, 0, 0, a0); /* past the end: stale */ \
+    CINN_SB; mm(a1, b1, 0, 1); CINN_SB; read_b(NEXT1, 0, 0, b0);                           \
+    CINN_SB; mm(a1, b1, 1, 0); CINN_SB; read_a(NEXT1, 0, 1, a0);                           \
+    CINN_SB; mm(a1, b1, 1, 1); CINN_SB; if (more) issue_one(FREE, s + 3, 2);               \
+    CINN_SB; mm(a1, b1, 2, 0); CINN_SB; read_a(NEXT1, 0, 2, a0);                           \
+    CINN_SB; mm(a1, b1, 2, 1); CINN_SB; read_a(NEXT1, 0, 3, a0);                           \
+    CINN_SB; mm(a1, b1, 3, 0); CINN_SB; read_b(NEXT1, 0, 1, b0);                           \
+    CINN_SB; mm(a1, b1, 3, 1); CINN_SB; if (more) issue_one(FREE, s + 3, 3);               \
     CINN_SB;                                                                               \
   }
   for (int kt = 0; kt < nk; kt += 4) {
@@ -636,10 +641,23 @@ void LaunchFast16(const GemmProblem& p, hipStream_t stream) {
 template <typename T, bool B_KC>
 void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
   int64_t ldb = p.trans_b ? p.k : p.n;
-  dim3 grid((p.m / kBM) * (p.n / kBN), p.batch, 1);
+  const int tiles_m = p.m / kBM, tiles_n = p.n / kBN;
+  dim3 grid(tiles_m * tiles_n, p.batch, 1);
+  // split the tile grid over the 8 XCDs as gr x gc rectangles with the smallest half-perimeter
+  int xcd_cols = 0, sub_rows = 0, sub_cols = 0;
+  for (int gc = 1; gc <= 8; gc *= 2) {
+    const int gr = 8 / gc;
+    if (tiles_m % gr != 0 || tiles_n % gc != 0) continue;
+    const int r = tiles_m / gr, c = tiles_n / gc;
+    if (sub_rows == 0 || r + c < sub_rows + sub_cols) {
+      xcd_cols = gc;
+      sub_rows = r;
+      sub_cols = c;
+    }
+  }
   hipLaunchKernelGGL((gemm16_dma_kernel<T, B_KC>), grid, dim3(kDmaThreads), 0, stream, static_cast<const uint16_t*>(p.a),
                      static_cast<const uint16_t*>(p.b), static_cast<uint16_t*>(p.c), p.m, p.n, p.k, (int64_t)p.k, ldb,
-                     (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c);
+                     (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c, xcd_cols, sub_rows, sub_cols);
 }
 
 bool UseRegisterStaging() {
