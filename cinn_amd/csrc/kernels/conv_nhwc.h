@@ -30,4 +30,8 @@ struct ConvNhwcArgs {
 bool ConvNhwcSupported(const ConvNhwcArgs& a);
 void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream);
 
+// NCHW-input convolutions whose filter and input patch fit LDS (conv_stem_mfma.hip): staged instead of gathered
+bool ConvStemSupported(const ConvNhwcArgs& a);
+void RunConvStem(const ConvNhwcArgs& a, hipStream_t stream);
+
 }  // namespace cinn_hip_kernels

@@ -605,6 +605,10 @@ void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream) {
   CINN_RT_CHECK(ConvNhwcSupported(a), "conv2d (channels-last): unsupported type or channel count %d", a.c);
   CINN_RT_CHECK((int64_t)a.n * a.h * a.w_in * a.c < INT_MAX && (int64_t)a.n * a.oh * a.ow * a.oc < INT_MAX,
                 "conv2d (channels-last): tensor too large for 32-bit offsets");
+  if (ConvStemSupported(a)) {
+    RunConvStem(a, stream);
+    return;
+  }
   Params p;
   p.n = a.n, p.h = a.h, p.w = a.w_in, p.c = a.c;
   p.oc = a.oc, p.kh = a.kh, p.kw = a.kw;
