@@ -246,3 +246,98 @@ def test_matmul_of_a_matrix_with_itself(gpu):
     A = b.create_input(Float(32), a.shape, "a")
     (got,), _ = run(b, {A: a}, [b.matmul(A, A)])
     np.testing.assert_allclose(got, oracle.matmul(a, a), rtol=1e-5, atol=1e-5)
+
+
+# ---- the channels-last kernels through the C-ABI (tensor formats 1 and 2 of cinn_call_cudnn_conv2d_forward) --------
+def call_conv_nhwc(x_nchw, w_oihw, stride, pad, fmt, dtype, alpha=1.0, beta=0.0, y_init=None):
+    """x / w are fp32 arrays in NCHW / OIHW; they are converted to `dtype` and to the layout `fmt` asks for.
+    Returns the output as fp32 NCHW."""
+    from cinn_amd.common import bfloat16_bits_to_float32, float32_to_bfloat16_bits
+    lib = _lib.load()
+    lib.cinn_call_cudnn_conv2d_forward.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_float,
+                                                   ctypes.c_float] + [ctypes.c_int] * 19 + [ctypes.c_void_p]
+    n, ic, ih, iw = x_nchw.shape
+    oc, _, kh, kw = w_oihw.shape
+    oh = oracle.conv_out_dim(ih, kh, pad, stride, 1)
+    ow = oracle.conv_out_dim(iw, kw, pad, stride, 1)
+
+    def to_dev(a):
+        a = np.ascontiguousarray(a)
+        if dtype == "bfloat16":
+            return float32_to_bfloat16_bits(a.astype(np.float32))
+        return a.astype(dtype)
+
+    xd = x_nchw.transpose(0, 2, 3, 1) if fmt == 1 else x_nchw
+    wd = w_oihw.transpose(0, 2, 3, 1) if fmt == 1 else w_oihw
+    X, W = runtime.DeviceBuffer.from_numpy(to_dev(xd), dtype), runtime.DeviceBuffer.from_numpy(to_dev(wd), dtype)
+    Y = runtime.DeviceBuffer((n, oh, ow, oc), dtype)
+    y0 = np.zeros((n, oc, oh, ow), np.float32) if y_init is None else y_init
+    Y.copy_from(to_dev(y0.transpose(0, 2, 3, 1)))
+    args = runtime.pod_args([X, W, Y])
+    lib.cinn_call_cudnn_conv2d_forward(args, 3, fmt, alpha, beta, n, ic, ih, iw, oc, ic, kh, kw, pad, pad, stride, stride,
+                                       1, 1, 1, n, oc, oh, ow, None)
+    runtime.synchronize()
+    out = Y.numpy()
+    out = bfloat16_bits_to_float32(out) if dtype == "bfloat16" else out.astype(np.float32)
+    return out.transpose(0, 3, 1, 2)
+
+
+def round_to(a, dtype):
+    from cinn_amd.common import bfloat16_bits_to_float32, float32_to_bfloat16_bits
+    if dtype == "bfloat16":
+        return bfloat16_bits_to_float32(float32_to_bfloat16_bits(a.astype(np.float32)))
+    return a.astype(dtype).astype(np.float32)
+
+
+NHWC_CASES = [
+    # (n, ic, h, w, oc, k, stride, pad)
+    (2, 8, 14, 15, 8, 3, 1, 1),
+    (1, 136, 9, 9, 140, 3, 1, 1),     # channel tails on both operands
+    (3, 16, 11, 7, 20, 1, 2, 0),      # output channels not a multiple of 8: element-wise epilogue
+    (2, 512, 7, 7, 64, 3, 1, 1),      # few pixels, long K: the grid is split along K
+    (2, 64, 5, 5, 1000, 1, 1, 0),     # classifier-like: 50 pixels
+]
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 1e-5), ("float16", 1e-2), ("bfloat16", 2e-2)])
+@pytest.mark.parametrize("case", NHWC_CASES)
+def test_conv2d_channels_last_intrinsic(gpu, case, dtype, tol):
+    n, ic, h, w_, oc, k, s, p = case
+    rng = np.random.default_rng(sum(case))
+    x = round_to(rng.standard_normal((n, ic, h, w_)), dtype)
+    w = round_to(rng.standard_normal((oc, ic, k, k)) * np.sqrt(2.0 / (ic * k * k)), dtype)
+    got = call_conv_nhwc(x, w, s, p, 1, dtype)
+    want = oracle.conv2d_nchw(x, w, (s, s), (p, p))
+    scale = oracle.conv2d_nchw(np.abs(x), np.abs(w), (s, s), (p, p))
+    if dtype == "float32":
+        assert np.all(np.abs(got - want) <= tol * scale + 1e-30)
+    else:
+        assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 1e-5), ("float16", 1e-2), ("bfloat16", 2e-2)])
+@pytest.mark.parametrize("case", [(2, 3, 37, 41, 64, 7, 2, 3), (1, 3, 20, 20, 10, 7, 2, 3), (2, 4, 17, 19, 70, 3, 1, 1),
+                                  (1, 1, 30, 30, 8, 5, 1, 2), (1, 3, 16, 16, 16, 11, 4, 2)])
+def test_conv2d_nchw_input_channels_last_output(gpu, case, dtype, tol):
+    """format 2: the image convolution (staged kernel; the 11x11 filter falls back to the gathering loader)."""
+    n, ic, h, w_, oc, k, s, p = case
+    rng = np.random.default_rng(sum(case) + 7)
+    x = round_to(rng.standard_normal((n, ic, h, w_)), dtype)
+    w = round_to(rng.standard_normal((oc, ic, k, k)) * np.sqrt(2.0 / (ic * k * k)), dtype)
+    got = call_conv_nhwc(x, w, s, p, 2, dtype)
+    want = oracle.conv2d_nchw(x, w, (s, s), (p, p))
+    scale = oracle.conv2d_nchw(np.abs(x), np.abs(w), (s, s), (p, p))
+    if dtype == "float32":
+        assert np.all(np.abs(got - want) <= tol * scale + 1e-30)
+    else:
+        assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+
+
+def test_conv2d_channels_last_alpha_beta(gpu):
+    rng = np.random.default_rng(31)
+    x = rng.standard_normal((2, 16, 6, 6)).astype(np.float32)
+    w = rng.standard_normal((24, 16, 3, 3)).astype(np.float32)
+    y0 = rng.standard_normal((2, 24, 6, 6)).astype(np.float32)
+    for fmt in (1, 2):
+        got = call_conv_nhwc(x, w, 1, 1, fmt, "float32", alpha=0.5, beta=2.0, y_init=y0)
+        np.testing.assert_allclose(got, 0.5 * oracle.conv2d_nchw(x, w, (1, 1), (1, 1)) + 2.0 * y0, rtol=1e-5, atol=1e-4)
