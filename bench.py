@@ -107,7 +107,9 @@ def cpu_baseline(kernels, repeats=3):
                 oracle.argmax_last(f["x"])
         return time.perf_counter() - t0
 
-    one_pass()  # warm-up (page faults, thread pool)
+    warm = one_pass()  # warm-up (page faults, thread pool)
+    # about 10 s of CPU work, between 3 and 200 passes
+    repeats = max(repeats, min(200, int(10.0 / max(warm, 1e-3))))
     times = sorted(one_pass() for _ in range(repeats))
     med = times[len(times) // 2]
     total = sum(k["bytes"] for k in kernels)
