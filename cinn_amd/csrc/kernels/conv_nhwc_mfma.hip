@@ -7,15 +7,17 @@
 // consecutive channels of one input pixel, present or - outside the image - zero.  Nothing is gathered element
 // by element and no im2col buffer exists.
 //
-//   * block tile BM pixels x BN output channels (128x128, 128x64 or 64x64, chosen per shape so that the grid
-//     fills the 256 CUs), 256 threads = 4 wavefronts in a 2x2 grid, K step of 128 bytes per row;
+//   * block tile BM pixels x BN output channels: 64x64 by default (short-K, small-grid layers are bound by load
+//     latency, which the number of resident blocks hides; 128x128 and 128x64 are selectable), 256 threads = 4
+//     wavefronts in a 2x2 grid, K step of 128 bytes per row; grids below one block per CU split K over blockIdx.y;
 //   * operand tiles in LDS as [row][128 bytes], 16-byte chunks XOR-swizzled (conflict-free ds_read_b128 of MFMA
 //     fragments), double buffered with the next step's global loads in flight during the MFMAs;
 //   * v_mfma_f32_32x32x16_{f16,bf16} or v_mfma_f32_32x32x2_f32, fp32 accumulation;
 //   * epilogue staged through LDS so that each lane writes 16 contiguous bytes of one pixel: per-channel affine
 //     (folded batch norm), residual addition and relu are applied there on the fp32 accumulators;
-//   * a second loader reads an NCHW input with few channels (the network stem) directly, k = (c, dy, dx) with dx
-//     padded to a chunk, so that the image never has to be transposed or channel-padded in memory.
+//   * a second loader reads an NCHW input with few channels directly, k = (c, dy, dx) with dx padded to a chunk,
+//     so that the image never has to be transposed or channel-padded in memory; shapes whose filter and input
+//     patch fit LDS (the network's first convolution) go to the staged kernel of conv_stem_mfma.hip instead.
 #include <hip/hip_runtime.h>
 
 #include <climits>
