@@ -3,9 +3,9 @@
 //   C[M,N] = alpha * op(A)[M,K] * op(B)[K,N] + beta * C          (row-major, optional batch)
 //
 // Four kernels:
-//   * gemm16_dma_kernel   - bf16 / fp16 with A stored [M][K] (the common case) and K % 128 == 0: 256x256x32 tile, 512
-//     threads, direct global -> LDS loads into a 4-stage ring, transposing LDS reads for row-major B; see the comment
-//     at the kernel.
+//   * gemm16_dma_kernel   - bf16 / fp16 with A stored [M][K] (the common case) and K % 128 == 0: 256x256x64 tile, 512
+//     threads, direct global -> LDS loads of whole 128-byte lines into two stages, transposing LDS reads for
+//     row-major B; see the comment at the kernel.
 //   * gemm16_mfma_kernel  - bf16 / fp16 inputs, any operand layout (used for transposed A), fp32 accumulation on v_mfma_f32_32x32x16_{bf16,f16}.
 //     256x256 block tile, 64-deep K step, 256 threads = 4 wavefronts in a 2x2 grid, each wavefront owning a
 //     128x128 tile (16 MFMA accumulator tiles = 256 accumulator registers).  Both operand tiles live in LDS
@@ -211,54 +211,55 @@ gemm16_mfma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ 
 
 // ---------------------------------------------------------------------------------------------------
 // bf16 / fp16 with A stored [M][K]: direct global -> LDS loads (global_load_lds_dwordx4), 8 wavefronts.
-// 256x256 block tile, K step 32, 512 threads in a 2 (M) x 4 (N) wavefront grid, each wavefront a 128x64 tile (8 MFMA
-// accumulators), two wavefronts per SIMD so that one runs MFMAs while the other waits for LDS or the barrier.
+// 256x256 block tile, K step 64, 512 threads in a 2 (M) x 4 (N) wavefront grid, each wavefront a 128x64 tile (8 MFMA
+// accumulators), two wavefronts per SIMD.
+//   * Every row of an operand tile is one whole 128-byte line.  With a K step of 32 (64-byte rows) the vector L1
+//     fetches every line twice from L2, one step apart, and that fill traffic bounds the feed: measured 32 bytes per
+//     clock and CU with 64-byte rows against 48-51 with 128-byte rows.
 //   * A lane of a load instruction writes its 16 bytes at LDS base + 16 * lane, so the swizzle that makes the fragment
 //     reads conflict free is applied on the global side: each lane fetches the chunk that belongs at its LDS slot.
-//   * B stored [K][N] (the plain row-major matmul) is kept as [k][n] in LDS and read with ds_read_b64_tr_b16, which
-//     hands every lane four consecutive k of one column - no transposition in registers.
-//   * Four LDS stages of 32 KiB in four separate arrays.  At the barrier of step s every wavefront knows that the
-//     tiles of step s+1 have landed and that nobody reads the tiles of step s-1 any more: the loads of step s+3 go
-//     there.  The loads are issued through inline assembly, one between every four MFMAs: the compiler neither
-//     tracks them (its conservative s_waitcnt vmcnt(0) before LDS reads would serialise the ring - the waits here are
-//     explicit vmcnt(4)) nor lets a wavefront queue all its loads at once, which stalls it behind the address unit
-//     while the MFMA pipe idles.
-//   * Every MFMA is followed by exactly one LDS fragment read or one global->LDS load (scheduling barriers pin the
-//     order); fragments are requested 8 MFMAs ahead, those of step s+1 during the MFMAs of step s, so no LDS read is
-//     exposed after a barrier.
-// Measured on MI355X the direct-to-LDS path sustains about 27 bytes per clock and CU, a 256x256 tile needs 32 at the
-// full MFMA rate: the kernel is bound by that path (about 1.05-1.1 PFLOP/s at 4096^3).
+//     A load instruction covers 8 rows x 128 bytes.
+//   * B stored [K][N] (the plain row-major matmul) is kept as [k][n] in LDS ([64 k][512 B], a load instruction
+//     covers 2 k-rows) and read with ds_read_b64_tr_b16, which hands every lane four consecutive k of one column -
+//     no transposition in registers.
+//   * Two stages of 64 KiB.  One barrier per K step, placed before the MFMAs of the step's last 16-deep slice: at
+//     that point every wavefront has its last fragments of stage s in registers, so stage s's slot is free for the
+//     loads of stage s+2, which are issued right after that barrier and waited for at the barrier of step s+1 - a
+//     whole K step of MFMAs (2048 clocks per SIMD at the full rate) hides their latency.
+//   * After every MFMA one LDS fragment read (requested a slice ahead; scheduling barriers pin the order) and, in the
+//     two slices after the barrier, after every second MFMA one load.
+//   * The result tile goes through LDS (two passes of 128 rows) so that a store instruction covers two whole 512-byte
+//     rows of C.
+// In core clocks the main loop keeps the MFMA pipe 84 % busy (156 k clocks for 131 k of MFMA at 4096^3); what the
+// kernel delivers beyond that is set by the clock the chip sustains under this load (1.2-1.6 GHz measured inside
+// the loop against the 2.4 GHz of the quoted peak).
 // Requires M % 256 == N % 256 == K % 128 == 0.
 // ---------------------------------------------------------------------------------------------------
 constexpr int kDmaThreads = 512;
-constexpr int kDmaBK      = 32;
-constexpr int kDmaTile    = kBM * kDmaBK * 2;  // one operand tile of a stage: 16 KiB
-constexpr int kDmaStage   = 2 * kDmaTile;
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 
-// rows of 64 bytes (4 chunks): byte offset of chunk `chunk` of row `row`
-__device__ __forceinline__ int DmaTileOffset(int row, int chunk) {
-  int key = (row >> 2) & 3;
-  return row * 64 + ((chunk ^ key) << 4);
-}
-
-// 16 bytes per lane from global memory straight into LDS at lds_base + 16 * lane
+// 16 bytes per lane from global memory straight into LDS at lds_base + 16 * lane.  Inline assembly, so that the
+// compiler does not track these loads: tracked, they get a conservative s_waitcnt vmcnt(0) before every LDS read.
 __device__ __forceinline__ void AsyncCopy16(const void* src, char* lds_base_uniform) {
   unsigned lds_addr =
       __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) char*)lds_base_uniform);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(src) : "memory");
 }
 
+constexpr int kD64BK   = 64;
+constexpr int kD64Tile = kBM * kD64BK * 2;  // one operand tile of a stage: 32 KiB
+
 template <typename T, bool B_KC>
 __global__ void __launch_bounds__(kDmaThreads)
 gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ C, int M, int N,
-                  int K, int64_t lda, int64_t ldb, int64_t ldc, float alpha, float beta, int64_t stride_a,
-                  int64_t stride_b, int64_t stride_c, int xcd_cols, int sub_rows, int sub_cols) {
-  __shared__ __attribute__((aligned(1024))) char s0[kDmaStage];
-  __shared__ __attribute__((aligned(1024))) char s1[kDmaStage];
-  __shared__ __attribute__((aligned(1024))) char s2[kDmaStage];
-  __shared__ __attribute__((aligned(1024))) char s3[kDmaStage];
+                    int K, int64_t lda, int64_t ldb, int64_t ldc, float alpha, float beta, int64_t stride_a,
+                    int64_t stride_b, int64_t stride_c, int xcd_cols, int sub_rows, int sub_cols) {
+  __shared__ __attribute__((aligned(1024))) char lds[4 * kD64Tile];
+  char* const sa0 = lds;
+  char* const sb0 = lds + kD64Tile;
+  char* const sa1 = lds + 2 * kD64Tile;
+  char* const sb1 = lds + 3 * kD64Tile;
   typedef typename Half16<T>::vec8 vec8;
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
@@ -266,10 +267,6 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   const int wm   = wave >> 2;
   const int wn   = wave & 3;
 
-  // Consecutive workgroup ids go round-robin to the 8 XCDs, each with its own L2.  Every XCD gets a compact
-  // sub_rows x sub_cols rectangle of tiles (the XCDs themselves form a (8 / xcd_cols) x xcd_cols grid), so that the
-  // blocks resident on one XCD at a time share as few A and B panels as possible: what misses an L2 crosses the
-  // fabric once per XCD, and that traffic, not the LDS feed, is what bounds this kernel.
   int tile_row, tile_col;
   if (sub_rows > 0) {
     const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
@@ -286,31 +283,31 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   B += (int64_t)blockIdx.y * stride_b;
   C += (int64_t)blockIdx.y * stride_c;
 
-  // Each wavefront issues 2 loads per operand and step; load q = 2 wave + t fills LDS bytes [1024 q, 1024 q + 1024)
-  // of the operand tile: 16 rows of a [row][32 halves] tile, or 2 k-rows of a [k][256 halves] tile.
-  const uint16_t* a_src[2];
-  const uint16_t* b_src[2];
+  // Each wavefront issues 4 loads per operand and step; load q = 4 wave + t fills LDS bytes [1024 q, 1024 q + 1024)
+  // of the operand tile: 8 rows of a [row][64 halves] tile, or 2 k-rows of a [k][256 halves] tile.
+  const uint16_t* a_src[4];
+  const uint16_t* b_src[4];
 #pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    const int q   = wave * 2 + t;
-    const int row = 16 * q + (lane >> 2);
-    const int key = (row >> 2) & 3;
-    a_src[t]      = A + (int64_t)(m0 + row) * lda + (((lane & 3) ^ key) << 3);
+  for (int t = 0; t < 4; ++t) {
+    const int q   = wave * 4 + t;
+    const int row = 8 * q + (lane >> 3);
+    const int key = (row ^ (row >> 3)) & 7;
+    a_src[t]      = A + (int64_t)(m0 + row) * lda + (((lane & 7) ^ key) << 3);
     if (B_KC) {
-      b_src[t] = B + (int64_t)(n0 + row) * ldb + (((lane & 3) ^ key) << 3);
+      b_src[t] = B + (int64_t)(n0 + row) * ldb + (((lane & 7) ^ key) << 3);
     } else {
       const int krow  = 2 * q + (lane >> 5);
       const int chunk = (lane & 31) ^ (2 * (krow & 3));
       b_src[t]        = B + (int64_t)krow * ldb + n0 + (chunk << 3);
     }
   }
-  const int64_t b_step = B_KC ? kDmaBK : (int64_t)kDmaBK * ldb;
-  // load t of step kt: 0, 1 the A tile, 2, 3 the B tile
-  auto issue_one = [&](char* stage, int kt, int t) {
-    if (t < 2) {
-      AsyncCopy16(a_src[t] + (int64_t)kt * kDmaBK, stage + (wave * 2 + t) * 1024);
+  const int64_t b_step = B_KC ? kD64BK : (int64_t)kD64BK * ldb;
+  // load t of step kt: 0..3 the A tile, 4..7 the B tile
+  auto issue_one = [&](char* a_tile, char* b_tile, int kt, int t) {
+    if (t < 4) {
+      AsyncCopy16(a_src[t] + (int64_t)kt * kD64BK, a_tile + (wave * 4 + t) * 1024);
     } else {
-      AsyncCopy16(b_src[t - 2] + kt * b_step, stage + kDmaTile + (wave * 2 + t - 2) * 1024);
+      AsyncCopy16(b_src[t - 4] + kt * b_step, b_tile + (wave * 4 + t - 4) * 1024);
     }
   };
 
@@ -324,17 +321,17 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 
   const int frag_row = lane & 31;
   const int frag_kg  = lane >> 5;
-  // one A fragment (rows i*32.. of the wavefront tile, 16-deep slice kk) / one B fragment / one MFMA
-  auto read_a = [&](const char* cur, int kk, int i, vec8 (&af)[4]) {
-    af[i] = *reinterpret_cast<const vec8*>(cur + DmaTileOffset(wm * 128 + i * 32 + frag_row, kk * 2 + frag_kg));
+  struct Frags {
+    vec8 a[4];
+    vec8 b[2];
   };
-  auto read_b = [&](const char* cur, int kk, int j, vec8 (&bf)[2]) {
-    const char* b_tile = cur + kDmaTile;
+  auto read_a = [&](const char* a_tile, int kk, int i, Frags& f) {
+    f.a[i] = *reinterpret_cast<const vec8*>(a_tile + TileOffset(wm * 128 + i * 32 + frag_row, kk * 2 + frag_kg));
+  };
+  auto read_b = [&](const char* b_tile, int kk, int j, Frags& f) {
     if (B_KC) {
-      bf[j] = *reinterpret_cast<const vec8*>(b_tile + DmaTileOffset(wn * 64 + j * 32 + frag_row, kk * 2 + frag_kg));
+      f.b[j] = *reinterpret_cast<const vec8*>(b_tile + TileOffset(wn * 64 + j * 32 + frag_row, kk * 2 + frag_kg));
     } else {
-      // one transposing read returns k = kb .. kb+3 of column n to the lane that owns n: lane j of each group of
-      // 16 supplies the address of row kb + j/4, columns nb + 4 (j%4) .. +3
       s16x4 part[2];
 #pragma unroll
       for (int r = 0; r < 2; ++r) {
@@ -344,69 +341,104 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
         part[r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(b_tile + off));
       }
       s16x8 both = __builtin_shufflevector(part[0], part[1], 0, 1, 2, 3, 4, 5, 6, 7);
-      bf[j]      = __builtin_bit_cast(vec8, both);
+      f.b[j]     = __builtin_bit_cast(vec8, both);
     }
   };
-  auto mm = [&](vec8 (&af)[4], vec8 (&bf)[2], int i, int j) { acc[i][j] = Half16<T>::mfma(af[i], bf[j], acc[i][j]); };
-
-  const int nk = K / kDmaBK;  // a multiple of 4
-  vec8 a0[4], b0[2], a1[4], b1[2];
-#pragma unroll
-  for (int t = 0; t < 4; ++t) issue_one(s0, 0, t);
-#pragma unroll
-  for (int t = 0; t < 4; ++t) issue_one(s1, 1, t);
-#pragma unroll
-  for (int t = 0; t < 4; ++t) issue_one(s2, 2, t);
-  __builtin_amdgcn_s_waitcnt(0x0F70 | 8);  // vmcnt(8): step 0 has landed
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < 4; ++i) read_a(s0, 0, i, a0);
-#pragma unroll
-  for (int j = 0; j < 2; ++j) read_b(s0, 0, j, b0);
 #define CINN_SB __builtin_amdgcn_sched_barrier(0)
-  // s_waitcnt immediates: vmcnt in bits 3:0 (15:14 zero), expcnt 7 and lgkmcnt 15 = no wait on those
-#define CINN_GEMM_STEP(CUR, NEXT1, FREE, OFF)                                              \
-  {                                                                                        \
-    const int s = kt + OFF;                                                                \
-    if (s + 2 < nk) {                                                                      \
-      __builtin_amdgcn_s_waitcnt(0x0F70 | 4); /* all but the loads of step s+2 are done */ \
-    } else {                                                                               \
-      __builtin_amdgcn_s_waitcnt(0x0F70);                                                  \
-    }                                                                                      \
-    __syncthreads();                                                                       \
-    const bool more = s + 3 < nk;                                                          \
-    /* every MFMA is followed by one LDS read or one global->LDS load, so that the LDS   */ \
-    /* and address units see an even stream and the wavefront always has MFMAs queued;   */ \
-    /* fragments are requested 8 MFMAs before their use (slice 1 of this step, then       */ \
-    /* slice 0 of the next step, which the barrier above has made visible)                */ \
-    CINN_SB; mm(a0, b0, 0, 0); CINN_SB; read_a(CUR, 1, 0, a1);                             \
-    CINN_SB; mm(a0, b0, 0, 1); CINN_SB; read_b(CUR, 1, 0, b1);                             \
-    CINN_SB; mm(a0, b0, 1, 0); CINN_SB; read_a(CUR, 1, 1, a1);                             \
-    CINN_SB; mm(a0, b0, 1, 1); CINN_SB; read_b(CUR, 1, 1, b1);                             \
-    CINN_SB; mm(a0, b0, 2, 0); CINN_SB; read_a(CUR, 1, 2, a1);                             \
-    CINN_SB; mm(a0, b0, 2, 1); CINN_SB; if (more) issue_one(FREE, s + 3, 0);               \
-    CINN_SB; mm(a0, b0, 3, 0); CINN_SB; read_a(CUR, 1, 3, a1);                             \
-    CINN_SB; mm(a0, b0, 3, 1); CINN_SB; if (more) issue_one(FREE, s + 3, 1);               \
-    CINN_SB; mm(a1, b1, 0, 0); CINN_SB; read_a(NEXT1, 0, 0, a0); /* past the end: stale */ \
-    CINN_SB; mm(a1, b1, 0, 1); CINN_SB; read_b(NEXT1, 0, 0, b0);                           \
-    CINN_SB; mm(a1, b1, 1, 0); CINN_SB; read_a(NEXT1, 0, 1, a0);                           \
-    CINN_SB; mm(a1, b1, 1, 1); CINN_SB; if (more) issue_one(FREE, s + 3, 2);               \
-    CINN_SB; mm(a1, b1, 2, 0); CINN_SB; read_a(NEXT1, 0, 2, a0);                           \
-    CINN_SB; mm(a1, b1, 2, 1); CINN_SB; read_a(NEXT1, 0, 3, a0);                           \
-    CINN_SB; mm(a1, b1, 3, 0); CINN_SB; read_b(NEXT1, 0, 1, b0);                           \
-    CINN_SB; mm(a1, b1, 3, 1); CINN_SB; if (more) issue_one(FREE, s + 3, 3);               \
-    CINN_SB;                                                                               \
+  // one 16-deep slice: the 8 MFMAs of `cur`, after each of them one fragment read of slice kk_next into `nxt` and,
+  // when n_loads == 4, after every second one a load (first_load ..) of the next stage
+  auto slice = [&](Frags& cur, Frags& nxt, const char* a_rd, const char* b_rd, int kk_next, int first_load, int n_loads,
+                   char* a_wr, char* b_wr, int kt_next, bool more) {
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+      CINN_SB;
+      acc[m >> 1][m & 1] = Half16<T>::mfma(cur.a[m >> 1], cur.b[m & 1], acc[m >> 1][m & 1]);
+      CINN_SB;
+      switch (m) {
+        case 0: read_a(a_rd, kk_next, 0, nxt); break;
+        case 1: read_b(b_rd, kk_next, 0, nxt); break;
+        case 2: read_a(a_rd, kk_next, 1, nxt); break;
+        case 3: read_b(b_rd, kk_next, 1, nxt); break;
+        case 4: read_a(a_rd, kk_next, 2, nxt); break;
+        case 5: read_a(a_rd, kk_next, 3, nxt); break;
+        default: break;
+      }
+      if (n_loads == 4 && (m & 1) == 1) {
+        CINN_SB;
+        if (more) issue_one(a_wr, b_wr, kt_next, first_load + (m >> 1));
+      }
+    }
+    CINN_SB;
+  };
+
+  const int nk = K / kD64BK;  // even
+  Frags f0, f1;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f0.a[i][e] = 0;
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f0.b[j][e] = 0;
+#pragma unroll
+  for (int t = 0; t < 8; ++t) issue_one(sa0, sb0, 0, t);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  __syncthreads();
+  // f0 holds the last slice of the previous stage (zeros before the first)
+#define CINN_GEMM_STEP(ACUR, BCUR, ANXT, BNXT, OFF)                                                          \
+  {                                                                                                          \
+    const int s     = kt + OFF;                                                                              \
+    const bool more = s + 1 < nk;                                                                            \
+    slice(f0, f1, ACUR, BCUR, 0, 0, 4, ANXT, BNXT, s + 1, more);                                             \
+    slice(f1, f0, ACUR, BCUR, 1, 4, 4, ANXT, BNXT, s + 1, more);                                             \
+    slice(f0, f1, ACUR, BCUR, 2, 0, 0, ANXT, BNXT, s + 1, more);                                             \
+    slice(f1, f0, ACUR, BCUR, 3, 0, 0, ANXT, BNXT, s + 1, more);                                             \
+    __builtin_amdgcn_s_waitcnt(0x0070); /* vmcnt(0) lgkmcnt(0): stage s+1 landed, fragments in registers */  \
+    __syncthreads();                                                                                         \
   }
-  for (int kt = 0; kt < nk; kt += 4) {
-    CINN_GEMM_STEP(s0, s1, s3, 0)
-    CINN_GEMM_STEP(s1, s2, s0, 1)
-    CINN_GEMM_STEP(s2, s3, s1, 2)
-    CINN_GEMM_STEP(s3, s0, s2, 3)
+  for (int kt = 0; kt < nk; kt += 2) {
+    CINN_GEMM_STEP(sa0, sb0, sa1, sb1, 0)
+    CINN_GEMM_STEP(sa1, sb1, sa0, sb0, 1)
   }
 #undef CINN_GEMM_STEP
+  // the last slice of the last stage
+#pragma unroll
+  for (int m = 0; m < 8; ++m) acc[m >> 1][m & 1] = Half16<T>::mfma(f0.a[m >> 1], f0.b[m & 1], acc[m >> 1][m & 1]);
 #undef CINN_SB
 
   T* Ct = reinterpret_cast<T*>(C);
+  if (beta == 0.0f) {
+    // Through LDS, half of the tile's rows at a time (the 32-row blocks i = 2 pass, 2 pass + 1 of every wavefront):
+    // accumulators are written as 16-bit values into [128 rows][256 + 8 columns], then every lane moves 16 bytes and
+    // a store instruction covers two whole 512-byte rows of C instead of 64 two-byte pieces.
+    constexpr int kRowBytes = (kBN + 8) * 2;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+      __syncthreads();  // the last stage (or the previous pass) has been read
+#pragma unroll
+      for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int lrow = wm * 64 + ii * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            const int col  = wn * 64 + j * 32 + (lane & 31);
+            *reinterpret_cast<T*>(lds + lrow * kRowBytes + col * 2) = (T)(alpha * acc[2 * pass + ii][j][r]);
+          }
+      __syncthreads();
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int chunk = e * kDmaThreads + tid;  // 128 rows x 32 chunks of 16 bytes
+        const int lrow  = chunk >> 5;
+        const int c16   = chunk & 31;
+        const int row   = m0 + (lrow >> 6) * 128 + pass * 64 + (lrow & 63);
+        const u32x4 v   = *reinterpret_cast<const u32x4*>(lds + lrow * kRowBytes + c16 * 16);
+        *reinterpret_cast<u32x4*>(Ct + (int64_t)row * ldc + n0 + c16 * 8) = v;
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll

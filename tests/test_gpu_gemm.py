@@ -108,6 +108,35 @@ def test_16bit_mfma_path_all_layouts(gpu, kind, ta, tb):
 
 
 @pytest.mark.parametrize("kind", ["float16", "bfloat16"])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (0.5, 2.0)])
+def test_16bit_direct_to_lds_kernel(gpu, kind, tb, alpha, beta):
+    """Shapes the 256x256x64 kernel takes (A stored [M][K], M, N % 256 == 0, K % 128 == 0): both layouts of B, two
+    batches with B broadcast, the staged epilogue (beta == 0) and the read-modify-write one."""
+    batch, m, n, k = 2, 512, 256, 384
+    rng = np.random.default_rng(41)
+    a = (rng.standard_normal((batch, m, k)) * 0.05).astype(np.float32)
+    b = (rng.standard_normal((1, n, k) if tb else (1, k, n)) * 0.05).astype(np.float32)
+    c0 = rng.standard_normal((batch, m, n)).astype(np.float32)
+    if kind == "float16":
+        ab, bb, cb = a.astype(np.float16), b.astype(np.float16), c0.astype(np.float16)
+        af, bf, cf = ab.astype(np.float64), bb.astype(np.float64), cb.astype(np.float64)
+        got = call_cublas(ab, bb, (batch, m, n), kind, False, tb, alpha=alpha, beta=beta, c_init=cb).astype(np.float64)
+        ulp = 2.0 ** -10
+    else:
+        ab, bb, cb = float32_to_bfloat16_bits(a), float32_to_bfloat16_bits(b), float32_to_bfloat16_bits(c0)
+        af, bf, cf = (bfloat16_bits_to_float32(x).astype(np.float64) for x in (ab, bb, cb))
+        got = bfloat16_bits_to_float32(
+            call_cublas(ab, bb, (batch, m, n), kind, False, tb, alpha=alpha, beta=beta, c_init=cb)).astype(np.float64)
+        ulp = 2.0 ** -7
+    bm = np.swapaxes(bf, 1, 2) if tb else bf
+    exact = alpha * (af @ bm) + beta * cf
+    scale = abs(alpha) * (np.abs(af) @ np.abs(bm)) + abs(beta) * np.abs(cf)
+    # fp32 accumulation and epilogue, one rounding to the 16-bit type
+    assert np.all(np.abs(got - exact) <= ulp * np.maximum(np.abs(exact), 1e-3 * scale) + 2.0 ** -24)
+
+
+@pytest.mark.parametrize("kind", ["float16", "bfloat16"])
 def test_config3_4096_cubed(gpu, kind):
     rng = np.random.default_rng(31)
     n = 4096
