@@ -14,7 +14,7 @@
 //     are conflict free.  Operands whose contiguous axis is not K (row-major B, transposed A) are transposed
 //     in registers (8x8 blocks of 16-bit values) on their way into LDS.  Requires M%256 == N%256 == K%64 == 0.
 //   * gemm32_mfma_kernel  - fp32 on v_mfma_f32_32x32x2f32, 128x128 tile (64x64 when that is what fills the chip),
-//     for M%128 == N%128 == K%16 == 0.
+//     for M%128 == N%128 == K%32 == 0.
 //   * gemm_generic_kernel - any shape / transpose / type (fp16, bf16, fp32, fp64): 64x64 LDS tile, FMA units.
 #include <hip/hip_runtime.h>
 
@@ -28,6 +28,7 @@
 namespace {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -456,29 +457,42 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 }
 
 // ---------------------------------------------------------------------------------------------------
-// fp32 on v_mfma_f32_32x32x2f32: 128x128 tile, K step 16, 4 wavefronts each 64x64 (2x2 MFMA tiles).
-// LDS holds A as [k][m] and B as [k][n] (row stride 128 floats) so that a fragment read is one
-// conflict-free ds_read_b32 per lane.
+// fp32 on v_mfma_f32_32x32x2f32: 128x128 (or 64x64) tile, K step KS = 32 or 64, 4 wavefronts each a quarter of the tile.
+// LDS holds A as [k][m] and B as [k][n] (row stride TILE + 4 floats) so that a fragment read is one conflict-free
+// ds_read_b32 per lane; the K step is deep enough (16 MFMAs of 64 clocks per accumulator) to cover the latency of
+// the next step's global loads, which travel as 16 bytes per lane and whole 128-byte lines per row.
 // ---------------------------------------------------------------------------------------------------
 constexpr int kF32Tile = 128;
-constexpr int kF32K    = 16;
+constexpr int kF32K    = 32;
 
-template <int TILE, bool TRANS_A, bool TRANS_B>
-__global__ void __launch_bounds__(256)
+// KSPLIT == 2 (with the 64x64 tile, whose wavefronts own a single accumulator tile): 8 wavefronts, two per 32x32
+// quadrant, each taking every other k pair of a step - a SIMD then holds two independent MFMA chains, which hides
+// the latency between dependent MFMAs and of the LDS reads; the two partial tiles are added through LDS at the end.
+template <int TILE, bool TRANS_A, bool TRANS_B, int KSPLIT, int KS>
+__global__ void __launch_bounds__(256 * KSPLIT)
 gemm32_mfma_kernel(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C, int M, int N, int K,
                    int64_t lda, int64_t ldb, int64_t ldc, float alpha, float beta, int64_t stride_a, int64_t stride_b,
-                   int64_t stride_c) {
-  __shared__ float As[2][kF32K][TILE + 4];
-  __shared__ float Bs[2][kF32K][TILE + 4];
-  constexpr int TT = TILE / 64;   // 32x32 MFMA tiles per wavefront and dimension
-  constexpr int EL = TILE / 16;   // elements of each operand a thread stages per K step
-  constexpr int SH = TILE == 128 ? 7 : 6;
+                   int64_t stride_c, int xcd_cols, int sub_rows, int sub_cols) {
+  __shared__ __attribute__((aligned(16))) float As[2][KS][TILE + 4];
+  __shared__ __attribute__((aligned(16))) float Bs[2][KS][TILE + 4];
+  constexpr int TT      = TILE / 64;  // 32x32 MFMA tiles per wavefront and dimension
+  constexpr int THREADS = 256 * KSPLIT;
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int m0 = blockIdx.y * TILE;
-  const int n0 = blockIdx.x * TILE;
+  const int kgrp = wave >> 2;  // which k pairs of a step this wavefront takes
+  const int wm = (wave >> 1) & 1, wn = wave & 1;
+  // consecutive workgroups go round-robin to the 8 XCDs: give each XCD a compact rectangle of tiles (see
+  // gemm16_dma_kernel), so that its L2 holds few A and B panels
+  int tile_row = blockIdx.y, tile_col = blockIdx.x;
+  if (sub_rows > 0) {
+    const int lin = blockIdx.y * gridDim.x + blockIdx.x;
+    const int xcd = lin & 7, idx = lin >> 3;
+    tile_row = (xcd / xcd_cols) * sub_rows + idx / sub_cols;
+    tile_col = (xcd % xcd_cols) * sub_cols + idx % sub_cols;
+  }
+  const int m0 = tile_row * TILE;
+  const int n0 = tile_col * TILE;
   A += (int64_t)blockIdx.z * stride_a;
   B += (int64_t)blockIdx.z * stride_b;
   C += (int64_t)blockIdx.z * stride_c;
@@ -491,56 +505,57 @@ gemm32_mfma_kernel(const float* __restrict__ A, const float* __restrict__ B, flo
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  // each thread stages 8 floats of A and 8 of B per K step (128 x 16 = 2048 per operand)
-  float ra[EL], rb[EL];
+  // Each thread stages EL4 groups of 4 floats of either operand per K step, 16 bytes per access.  An operand whose
+  // contiguous axis is k is fetched as 8 rows x 128 bytes per wavefront access (whole lines) and scattered into
+  // [k][row]; one whose contiguous axis is the row index is copied as it is.
+  constexpr int EL4 = TILE * KS / 4 / THREADS;
+  f32x4 ra[EL4], rb[EL4];
+  auto load_one = [&](const float* __restrict__ P, int64_t ld, int row0, int k0, bool k_contig, int i) -> f32x4 {
+    const int u = tid + THREADS * i;
+    if (k_contig) {
+      const int r = u / (KS / 4), kc = u % (KS / 4);
+      return *reinterpret_cast<const f32x4*>(P + (int64_t)(row0 + r) * ld + k0 + kc * 4);
+    }
+    const int k = u / (TILE / 4), c = u % (TILE / 4);
+    return *reinterpret_cast<const f32x4*>(P + (int64_t)(k0 + k) * ld + row0 + c * 4);
+  };
+  auto store_one = [&](float (*S)[TILE + 4], bool k_contig, int i, f32x4 v) {
+    const int u = tid + THREADS * i;
+    if (k_contig) {
+      const int r = u / (KS / 4), kc = u % (KS / 4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) S[kc * 4 + j][r] = v[j];
+    } else {
+      const int k = u / (TILE / 4), c = u % (TILE / 4);
+      *reinterpret_cast<f32x4*>(&S[k][c * 4]) = v;
+    }
+  };
   auto load_tiles = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < EL; ++i) {
-      int e = tid + 256 * i;
-      if (TRANS_A) {  // A stored [K][M]: m contiguous
-        int k = e >> SH, m = e & (TILE - 1);
-        ra[i] = A[(int64_t)(k0 + k) * lda + m0 + m];
-      } else {  // A stored [M][K]: k contiguous
-        int m = e >> 4, k = e & 15;
-        ra[i] = A[(int64_t)(m0 + m) * lda + k0 + k];
-      }
-      if (TRANS_B) {  // B stored [N][K]
-        int n = e >> 4, k = e & 15;
-        rb[i] = B[(int64_t)(n0 + n) * ldb + k0 + k];
-      } else {  // B stored [K][N]
-        int k = e >> SH, n = e & (TILE - 1);
-        rb[i] = B[(int64_t)(k0 + k) * ldb + n0 + n];
-      }
+    for (int i = 0; i < EL4; ++i) {
+      ra[i] = load_one(A, lda, m0, k0, !TRANS_A, i);
+      rb[i] = load_one(B, ldb, n0, k0, TRANS_B, i);
     }
   };
   auto store_tiles = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < EL; ++i) {
-      int e = tid + 256 * i;
-      if (TRANS_A) {
-        As[buf][e >> SH][e & (TILE - 1)] = ra[i];
-      } else {
-        As[buf][e & 15][e >> 4] = ra[i];
-      }
-      if (TRANS_B) {
-        Bs[buf][e & 15][e >> 4] = rb[i];
-      } else {
-        Bs[buf][e >> SH][e & (TILE - 1)] = rb[i];
-      }
+    for (int i = 0; i < EL4; ++i) {
+      store_one(As[buf], !TRANS_A, i, ra[i]);
+      store_one(Bs[buf], TRANS_B, i, rb[i]);
     }
   };
 
-  const int kt_count = K / kF32K;
+  const int kt_count = K / KS;
   load_tiles(0);
   store_tiles(0);
   __syncthreads();
   for (int kt = 0; kt < kt_count; ++kt) {
     const int cur  = kt & 1;
     const bool more = kt + 1 < kt_count;
-    if (more) load_tiles((kt + 1) * kF32K);
+    if (more) load_tiles((kt + 1) * KS);
 #pragma unroll
-    for (int kk = 0; kk < kF32K; kk += 2) {
-      const int k = kk + (lane >> 5);
+    for (int kp = 0; kp < KS / 2 / KSPLIT; ++kp) {
+      const int k = 2 * (kp * KSPLIT + kgrp) + (lane >> 5);
       float af[TT], bf[TT];
 #pragma unroll
       for (int t = 0; t < TT; ++t) {
@@ -554,6 +569,19 @@ gemm32_mfma_kernel(const float* __restrict__ A, const float* __restrict__ B, flo
     }
     if (more) store_tiles(cur ^ 1);
     __syncthreads();
+  }
+  if (KSPLIT == 2) {
+    // the last barrier of the loop has passed: the operand tiles are no longer read
+    static_assert(KSPLIT == 1 || TT == 1, "the partial tile exchange assumes one accumulator tile per wavefront");
+    float* part = &As[0][0][0] + ((wave & 3) * 16) * 64 + lane;  // [quadrant][element][lane]
+    if (kgrp == 1) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) part[r * 64] = acc[0][0][r];
+    }
+    __syncthreads();
+    if (kgrp == 1) return;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[0][0][r] += part[r * 64];
   }
 #pragma unroll
   for (int i = 0; i < TT; ++i) {
@@ -670,23 +698,28 @@ void LaunchFast16(const GemmProblem& p, hipStream_t stream) {
                      (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c);
 }
 
+// split a tiles_m x tiles_n grid over the 8 XCDs as gr x gc rectangles with the smallest half-perimeter; sub_rows
+// stays 0 when the grid does not divide
+void XcdRectangles(int tiles_m, int tiles_n, int* xcd_cols, int* sub_rows, int* sub_cols) {
+  for (int gc = 1; gc <= 8; gc *= 2) {
+    const int gr = 8 / gc;
+    if (tiles_m % gr != 0 || tiles_n % gc != 0) continue;
+    const int r = tiles_m / gr, c = tiles_n / gc;
+    if (*sub_rows == 0 || r + c < *sub_rows + *sub_cols) {
+      *xcd_cols = gc;
+      *sub_rows = r;
+      *sub_cols = c;
+    }
+  }
+}
+
 template <typename T, bool B_KC>
 void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
   int64_t ldb = p.trans_b ? p.k : p.n;
   const int tiles_m = p.m / kBM, tiles_n = p.n / kBN;
   dim3 grid(tiles_m * tiles_n, p.batch, 1);
-  // split the tile grid over the 8 XCDs as gr x gc rectangles with the smallest half-perimeter
   int xcd_cols = 0, sub_rows = 0, sub_cols = 0;
-  for (int gc = 1; gc <= 8; gc *= 2) {
-    const int gr = 8 / gc;
-    if (tiles_m % gr != 0 || tiles_n % gc != 0) continue;
-    const int r = tiles_m / gr, c = tiles_n / gc;
-    if (sub_rows == 0 || r + c < sub_rows + sub_cols) {
-      xcd_cols = gc;
-      sub_rows = r;
-      sub_cols = c;
-    }
-  }
+  XcdRectangles(tiles_m, tiles_n, &xcd_cols, &sub_rows, &sub_cols);
   hipLaunchKernelGGL((gemm16_dma_kernel<T, B_KC>), grid, dim3(kDmaThreads), 0, stream, static_cast<const uint16_t*>(p.a),
                      static_cast<const uint16_t*>(p.b), static_cast<uint16_t*>(p.c), p.m, p.n, p.k, (int64_t)p.k, ldb,
                      (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c, xcd_cols, sub_rows, sub_cols);
@@ -734,14 +767,20 @@ void LaunchFast32(const GemmProblem& p, hipStream_t stream) {
   const float* a = static_cast<const float*>(p.a);
   const float* b = static_cast<const float*>(p.b);
   float* c       = static_cast<float*>(p.c);
-#define CINN_LAUNCH_F32(TA, TB)                                                                                       \
-  if (small) {                                                                                                        \
-    hipLaunchKernelGGL((gemm32_mfma_kernel<64, TA, TB>), grid, dim3(256), 0, stream, a, b, c, p.m, p.n, p.k, lda, ldb, \
-                       (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c);                            \
-  } else {                                                                                                            \
-    hipLaunchKernelGGL((gemm32_mfma_kernel<128, TA, TB>), grid, dim3(256), 0, stream, a, b, c, p.m, p.n, p.k, lda,     \
-                       ldb, (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c);                       \
-  }
+  int xcd_cols = 0, sub_rows = 0, sub_cols = 0;
+  XcdRectangles(p.m / tile, p.n / tile, &xcd_cols, &sub_rows, &sub_cols);
+#define CINN_LAUNCH_F32(TA, TB)                                                                                        \
+  do {                                                                                                                 \
+    if (small) {                                                                                                       \
+      hipLaunchKernelGGL((gemm32_mfma_kernel<64, TA, TB, 2, 32>), grid, dim3(512), 0, stream, a, b, c, p.m, p.n, p.k,  \
+                         lda, ldb, (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c, xcd_cols,       \
+                         sub_rows, sub_cols);                                                                          \
+    } else {                                                                                                           \
+      hipLaunchKernelGGL((gemm32_mfma_kernel<128, TA, TB, 1, 32>), grid, dim3(256), 0, stream, a, b, c, p.m, p.n, p.k, \
+                         lda, ldb, (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c, xcd_cols,       \
+                         sub_rows, sub_cols);                                                                          \
+    }                                                                                                                  \
+  } while (0)
   if (!p.trans_a && !p.trans_b) CINN_LAUNCH_F32(false, false);
   if (!p.trans_a && p.trans_b) CINN_LAUNCH_F32(false, true);
   if (p.trans_a && !p.trans_b) CINN_LAUNCH_F32(true, false);
@@ -760,7 +799,9 @@ void RunGemm(const GemmProblem& p, hipStream_t stream) {
   CINN_RT_CHECK(p.a && p.b && p.c, "gemm: null operand");
   CINN_RT_CHECK(p.batch <= 65535, "gemm: batch %d exceeds the grid limit", p.batch);
   const bool fast16 = !ForceGeneric() && p.m % kBM == 0 && p.n % kBN == 0 && p.k % kBK == 0;
-  const bool fast32 = !ForceGeneric() && p.m % kF32Tile == 0 && p.n % kF32Tile == 0 && p.k % kF32K == 0;
+  const bool aligned16 = reinterpret_cast<uintptr_t>(p.a) % 16 == 0 && reinterpret_cast<uintptr_t>(p.b) % 16 == 0 &&
+                         p.stride_a % 4 == 0 && p.stride_b % 4 == 0;
+  const bool fast32 = !ForceGeneric() && p.m % kF32Tile == 0 && p.n % kF32Tile == 0 && p.k % kF32K == 0 && aligned16;
   // Ragged shapes whose operands are both K-contiguous (A [m,k], B stored [n,k]) go to the channels-last
   // convolution kernels: a 1x1 convolution over m "pixels" is this GEMM, and those kernels bound-check every tile
   // edge and pick a tile that fills the chip for small m or n.
