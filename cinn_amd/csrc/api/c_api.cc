@@ -297,6 +297,8 @@ int cinn_amd_computation_build_and_compile(cinn_amd_builder_t b, const char* con
           opts.fuse_conv_bn_relu = v != 0;
         } else if (k == "conv_layout_nhwc") {
           opts.conv_layout_nhwc = v != 0;
+        } else if (k == "split_reductions") {
+          opts.split_reductions = v != 0;
         } else if (k == "reduce_cached_elems") {
           opts.lowering.max_cached_elems_per_thread = v;
         } else if (k == "reduce_wave_elems") {

@@ -2,6 +2,7 @@
 
 #include "frontend/decomposer.h"
 #include "frontend/layout_pass.h"
+#include "frontend/reduce_split_pass.h"
 
 namespace cinn {
 namespace frontend {
@@ -44,6 +45,7 @@ std::shared_ptr<CinnComputation> CinnComputation::Compile(const common::Target& 
   if (options.conv_layout_nhwc) lowered = ConvertConvLayoutToNHWC(lowered, fetch_ids);
   if (options.fuse_conv_bn_relu) lowered = FuseConvBatchNorm(lowered, fetch_ids);
   if (options.use_decomposer) lowered = ApplyDecomposer(lowered);
+  if (options.split_reductions) lowered = SplitReductions(lowered, target.get_multi_processor_count());
   comp->graph_    = std::make_shared<Graph>(lowered, fetch_ids, target);
   comp->graph_->BuildFusionGroups();
   comp->scope_ = hlir::framework::BuildScope(target, comp->graph_);

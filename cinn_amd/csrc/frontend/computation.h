@@ -28,6 +28,9 @@ class CinnComputation {
     // move conv2d chains written in NCHW to channels-last tensors, the layout the MFMA convolution kernels read
     // with 16-byte accesses (frontend/layout_pass.h); off: every conv2d runs in the layout it was written in
     bool conv_layout_nhwc{true};
+    // rewrite reductions over non-trailing axes into chains of per-run (and, for small outputs, two-step) reductions
+    // that fill the chip (frontend/reduce_split_pass.h); off: such a reduction is one kernel whatever its grid size
+    bool split_reductions{true};
   };
   static CompileOptions DefaultCompileOptions() { return CompileOptions(); }
 

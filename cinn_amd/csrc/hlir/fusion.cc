@@ -141,7 +141,9 @@ void Graph::BuildFusionGroups() {
     auto g  = std::make_unique<WorkGroup>();
     g->nodes.push_back(n);
     g->pre_run = n->pre_run;
-    if (n->op->pattern == OpPatternKind::kReduction) {
+    if (n->op->pattern == OpPatternKind::kReduction && IsReduceRun(*n)) {
+      g->kind = GroupKind::kGeneralReduce;
+    } else if (n->op->pattern == OpPatternKind::kReduction) {
       int64_t r, c;
       if (TrailingReduceSpace(n->inputs[0]->shape, ReduceDimsOf(*n), &r, &c) && c > 1 &&
           ClassifyRowReduceGroup(g->nodes, r, c, nullptr)) {

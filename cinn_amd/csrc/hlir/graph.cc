@@ -147,6 +147,8 @@ std::string Graph::DebugGroupString() const {
   return os.str();
 }
 
+bool IsReduceRun(const Node& node) { return node.op_type().rfind("reduce_run_", 0) == 0; }
+
 std::vector<int> ReduceDimsOf(const Node& node) {
   int rank = static_cast<int>(node.inputs[0]->shape.size());
   std::vector<int> dims;

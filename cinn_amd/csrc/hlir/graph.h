@@ -96,6 +96,8 @@ class Graph {
 // ones (size-1 axes are ignored).  Returns false for any other axis set.
 bool TrailingReduceSpace(const ShapeType& shape, const std::vector<int>& dims, int64_t* rows, int64_t* cols);
 std::vector<int> ReduceDimsOf(const Node& node);
+// a reduce_run_<kind> node (reduction of a [a, parts, r / parts, c] view, see the op registry)
+bool IsReduceRun(const Node& node);
 
 // how a value relates to the rows x cols space of a row-reduce group
 enum class RowKind { kElem, kRow, kCol, kScalar, kInvalid };

@@ -237,6 +237,7 @@ LoweringOptions LoweringOptions::FromEnv() {
   o.rows_per_wave               = EnvInt("FLAGS_cinn_hip_reduce_rows_per_wave", o.rows_per_wave);
   o.elementwise_block           = EnvInt("FLAGS_cinn_hip_elementwise_block", o.elementwise_block);
   o.rows_per_block              = EnvInt("FLAGS_cinn_hip_reduce_rows_per_block", o.rows_per_block);
+  o.column_reduce               = EnvInt("FLAGS_cinn_hip_column_reduce", 1) != 0;
   return o;
 }
 
@@ -896,7 +897,141 @@ ir::LoweredFuncRef OpLowerer::LowerRowReduce(const Group& group) const {
 }
 
 // ---------------------------------------------------------------------------------------------------
-// reductions over arbitrary axes: one thread per output element
+// Reduction over one non-trailing run of axes: the input is [a][r][c] with r reduced.  A block is TX x TY
+// threads: x walks the kept, contiguous axis c in vectors of 16 bytes (a wavefront reads whole rows or row
+// segments), y strides over r; every thread keeps one accumulator per vector lane, rows are fetched four at a time
+// so that several loads are in flight, and the TY partial results of a column meet in LDS
+// (cinn_block_column_reduce_*).  Grid: a x ceil(c / (vec * TX)) blocks.  The reference assigns such reductions
+// in LoopAssignReduceWithoutLast (cinn/hlir/framework/op_lowering_util.cc:485-640).
+// ---------------------------------------------------------------------------------------------------
+namespace {
+
+void EmitColumnReduce(GroupContext* ctx, const common::Target& target, NodeData* in, NodeData* out,
+                      const std::string& kind, int64_t a, int64_t r, int64_t c) {
+  const Type acc_type = AccumType(kind, in->dtype);
+  int vec             = std::max(1, std::min(16 / in->dtype.bytes(), 8));
+  while (vec > 1 && c % vec != 0) vec /= 2;
+  CINN_CHECK(vec <= (acc_type.bytes() >= 8 ? 2 : 8)) << "the LDS exchange of the column reduce holds 8 values per thread";
+  const int64_t cv = c / vec;
+  int tx_n         = 1;
+  while (tx_n < 64 && tx_n < cv) tx_n *= 2;
+  int ty_n = 256 / tx_n;
+  while (ty_n > 1 && ty_n / 2 >= r) ty_n /= 2;
+  const int64_t grid_c  = (cv + tx_n - 1) / tx_n;
+  const bool col_guard  = cv % tx_n != 0;
+  const int64_t full    = r / ty_n;  // rows every thread takes without a bound check
+  const int unroll      = full >= 8 ? 4 : 1;
+  const int64_t main_it = full / unroll;
+  CINN_CHECK_LT(a * grid_c, static_cast<int64_t>(std::numeric_limits<int32_t>::max()));
+
+  Expr bid = ir::MakeVar("bid", common::Int(32));
+  Expr tx  = ir::MakeVar("tx", common::Int(32));
+  Expr ty  = ir::MakeVar("ty", common::Int(32));
+  Expr k   = ir::MakeVar("k", common::Int(32));
+  BufferRef src = ctx->global_bufs.at(in);
+  BufferRef dst = ctx->global_bufs.at(out);
+
+  std::vector<Expr> stmts;
+  Expr ai   = ctx->NewVar("a", common::Int(32));
+  Expr cvi  = ctx->NewVar("cv", common::Int(32));
+  Expr base = ctx->NewVar("base", common::Int(32));
+  stmts.push_back(ir::MakeLet(ai, bid / I32(grid_c)));
+  stmts.push_back(ir::MakeLet(cvi, (bid % I32(grid_c)) * I32(tx_n) + tx));
+  stmts.push_back(ir::MakeLet(base, ai * I32(r * c) + cvi * I32(vec)));
+
+  BufferRef acc = ctx->NewLocal("acc", acc_type, vec);
+  {
+    Expr ki = ir::MakeVar("ki", common::Int(32));
+    stmts.push_back(ir::MakeFor(ki, I32(0), I32(vec), ForType::Unrolled,
+                                ir::MakeStore(acc, ir::MakeCast(acc_type, ReduceIdentity(kind, acc_type)), ki)));
+  }
+  // one row: a 16-byte load into registers, then the lane-wise combine
+  auto row = [&](const Expr& row_index, int slot) {
+    BufferRef reg = ctx->NewLocal("x" + std::to_string(slot), in->dtype, vec);
+    Expr kl       = ir::MakeVar("kl", common::Int(32));
+    Expr kc       = ir::MakeVar("kc", common::Int(32));
+    Expr offset   = base + row_index * I32(c);
+    Expr load     = ir::MakeFor(kl, I32(0), I32(vec), ForType::Vectorized,
+                                ir::MakeStore(reg, ir::MakeLoad(src, offset + kl), kl));
+    Expr combine  = ir::MakeFor(
+        kc, I32(0), I32(vec), ForType::Unrolled,
+        ir::MakeStore(acc, Combine(kind, ir::MakeLoad(acc, kc), ir::MakeCast(acc_type, ir::MakeLoad(reg, kc))), kc));
+    return ir::MakeBlock({load, combine});
+  };
+  std::vector<Expr> accumulate;
+  if (main_it > 0) {
+    Expr io = ir::MakeVar("io", common::Int(32));
+    Expr u  = ir::MakeVar("u", common::Int(32));
+    // the loads of the unrolled rows are independent: the compiler issues them together
+    Expr body = row((io * I32(unroll) + u) * I32(ty_n) + ty, 0);
+    accumulate.push_back(ir::MakeFor(io, I32(0), I32(main_it), ForType::Serial,
+                                     ir::MakeFor(u, I32(0), I32(unroll), ForType::Unrolled, body)));
+  }
+  if (full > main_it * unroll) {
+    Expr i = ir::MakeVar("i", common::Int(32));
+    accumulate.push_back(ir::MakeFor(i, I32(main_it * unroll), I32(full - main_it * unroll), ForType::Serial,
+                                     row(i * I32(ty_n) + ty, 1)));
+  }
+  if (r % ty_n != 0) {
+    Expr last = ctx->NewVar("last", common::Int(32));
+    accumulate.push_back(ir::MakeLet(last, I32(full * ty_n) + ty));
+    accumulate.push_back(ir::MakeIf(last < I32(r), row(last, 2)));
+  }
+  Expr accumulate_all = ir::MakeBlock(accumulate);
+  if (col_guard) accumulate_all = ir::MakeIf(cvi < I32(cv), accumulate_all);
+  stmts.push_back(accumulate_all);
+
+  // every thread of the block takes part in the exchange through LDS
+  BufferRef res  = ctx->NewLocal("res", out->dtype, vec);
+  std::string fn = "cinn_block_column_reduce_" + ReduceSuffix(kind, acc_type);
+  {
+    Expr call = ir::MakeCall(Type(), fn, {I32(vec)});
+    const_cast<ir::Call*>(call.As<ir::Call>())->buffer_args.push_back(acc);
+    stmts.push_back(call);
+  }
+  stmts.push_back(ir::MakeFor(k, I32(0), I32(vec), ForType::Unrolled,
+                              ir::MakeStore(res, ir::MakeCast(out->dtype, ir::MakeLoad(acc, k)), k)));
+  Expr ks    = ir::MakeVar("ks", common::Int(32));
+  Expr store = ir::MakeFor(ks, I32(0), I32(vec), ForType::Vectorized,
+                           ir::MakeStore(dst, ir::MakeLoad(res, ks), ai * I32(c) + cvi * I32(vec) + ks));
+  Expr owner = ty == I32(0);
+  if (col_guard) owner = owner && (cvi < I32(cv));
+  stmts.push_back(ir::MakeIf(owner, store));
+
+  Expr threads_x  = ir::MakeFor(tx, I32(0), I32(tx_n), ForType::Serial, ir::MakeBlock(stmts), ThreadAxis(0));
+  Expr threads_y  = ir::MakeFor(ty, I32(0), I32(ty_n), ForType::Serial, threads_x, ThreadAxis(1));
+  ctx->func->body = ir::MakeFor(bid, I32(0), I32(a * grid_c), ForType::Serial, threads_y, BlockAxis(0));
+  (void)target;
+}
+
+// [a][r][c] of a reduction whose reduced axes (sizes > 1) form one run; false otherwise
+bool SingleReduceRun(const ShapeType& shape, const std::vector<int>& dims, int64_t* a, int64_t* r, int64_t* c) {
+  const int rank = static_cast<int>(shape.size());
+  std::vector<bool> reduced(rank, false);
+  for (int d : dims) reduced[d] = true;
+  *a = *r = *c = 1;
+  int state = 0;  // 0: before the run, 1: inside, 2: after
+  for (int i = 0; i < rank; ++i) {
+    if (shape[i] == 1) continue;
+    if (reduced[i]) {
+      if (state == 2) return false;
+      state = 1;
+      *r *= shape[i];
+    } else if (state == 0) {
+      *a *= shape[i];
+    } else {
+      state = 2;
+      *c *= shape[i];
+    }
+  }
+  return true;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------------------
+// reductions over arbitrary axes: a column-reduce kernel when the reduced axes form one run, else one thread per
+// output element
 // ---------------------------------------------------------------------------------------------------
 ir::LoweredFuncRef OpLowerer::LowerGeneralReduce(const Group& group) const {
   CINN_CHECK_EQ(group.nodes.size(), 1u) << "a general reduce group holds exactly one reduction";
@@ -911,6 +1046,19 @@ ir::LoweredFuncRef OpLowerer::LowerGeneralReduce(const Group& group) const {
   for (int d : dims) reduced[d] = true;
   const std::string& kind = n->op->reduce_kind;
   bool is_arg             = kind == "argmax" || kind == "argmin";
+  if (IsReduceRun(*n)) {
+    const int64_t parts = GetAttr<int>(n->attrs, "parts", 1);
+    EmitColumnReduce(&ctx, target_, in, out, kind, static_cast<int64_t>(GetAttr<int>(n->attrs, "a", 1)) * parts,
+                     GetAttr<int>(n->attrs, "r", 1) / parts, GetAttr<int>(n->attrs, "c", 1));
+    return ctx.func;
+  }
+  {
+    int64_t a, r, c;
+    if (!is_arg && options_.column_reduce && SingleReduceRun(shape, dims, &a, &r, &c) && r > 1) {
+      EmitColumnReduce(&ctx, target_, in, out, kind, a, r, c);
+      return ctx.func;
+    }
+  }
 
   ShapeType kept_shape;
   for (int i = 0; i < rank; ++i)

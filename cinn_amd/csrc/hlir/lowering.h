@@ -39,6 +39,8 @@ struct LoweringOptions {
   // rows one wavefront works through (unrolled, so their loads overlap).  Measured on MI355X this does
   // not pay for the BASELINE shapes (1 is the best setting for every one of them), so it stays a knob.
   int rows_per_wave{1};
+  // reductions over one non-trailing run of axes use the column-reduce kernel (off: one thread per output element)
+  bool column_reduce{true};
   static LoweringOptions FromEnv();
 };
 

@@ -122,6 +122,33 @@ void RegisterReduce(OpRegistry* r, const std::string& op_name, const std::string
   op.infer_dtype = SameTypeAsFirst;
 }
 
+// reduce_run_<kind>: the input, viewed as [a, parts, r / parts, c], reduced over its third axis; the result
+// [a, parts, c] is declared with the shape `out_shape` (same element count) and the type `dtype` (the input's when
+// empty).  Internal op: the reduction splitting pass writes reductions over non-trailing axes as chains of these
+// (the reference splits such reductions in cinn/hlir/pass/reduce_split_pass.cc).
+void RegisterReduceRun(OpRegistry* r, const std::string& op_name, const std::string& kind) {
+  auto& op       = r->Register(op_name);
+  op.pattern     = OpPatternKind::kReduction;
+  op.reduce_kind = kind;
+  op.infer_shape = [](const std::vector<ShapeType>& in, const AttributeMap& attrs) {
+    const int64_t a = GetAttr<int>(attrs, "a", 1), rr = GetAttr<int>(attrs, "r", 1), c = GetAttr<int>(attrs, "c", 1);
+    const int64_t parts = GetAttr<int>(attrs, "parts", 1);
+    int64_t numel = 1;
+    for (int d : in[0]) numel *= d;
+    CINN_CHECK_EQ(a * rr * c, numel) << "reduce_run: a * r * c must be the element count of the input";
+    CINN_CHECK(parts >= 1 && rr % parts == 0) << "reduce_run: parts must divide r";
+    ShapeType out = GetAttr<std::vector<int>>(attrs, "out_shape", {});
+    int64_t out_numel = 1;
+    for (int d : out) out_numel *= d;
+    CINN_CHECK_EQ(out_numel, a * parts * c) << "reduce_run: out_shape does not hold a * parts * c elements";
+    return std::vector<ShapeType>{out};
+  };
+  op.infer_dtype = [](const std::vector<Type>& in, const AttributeMap& attrs) {
+    std::string dtype = GetAttr<std::string>(attrs, "dtype", "");
+    return std::vector<Type>{dtype.empty() ? in[0] : common::Str2Type(dtype)};
+  };
+}
+
 void RegisterArgReduce(OpRegistry* r, const std::string& op_name, const std::string& kind) {
   auto& op       = r->Register(op_name);
   op.pattern     = OpPatternKind::kReduction;
@@ -402,6 +429,8 @@ OpRegistry::OpRegistry() {
   RegisterReduce(r, "reduce_min", "min");
   RegisterReduce(r, "reduce_all", "all");
   RegisterReduce(r, "reduce_any", "any");
+  for (const char* kind : {"sum", "prod", "max", "min", "all", "any"})
+    RegisterReduceRun(r, std::string("reduce_run_") + kind, kind);
   RegisterArgReduce(r, "argmax", "argmax");
   RegisterArgReduce(r, "argmin", "argmin");
 

@@ -47,7 +47,7 @@ int cinn_amd_builder_program_string(cinn_amd_builder_t b, char* out, size_t cap,
 /* ---- CinnComputation (cinn/frontend/computation.h) ---- */
 /* CinnComputation::BuildAndCompile for the AMDGPU target.  outputs: ids to fetch (NULL/0: outputs of the
  * last instruction).  stream: hipStream_t or NULL.  options: "key=value;..." (keys: do_prerun,
- * fuse_conv_bn_relu, and the lowering knobs reduce_cached_elems, reduce_wave_elems, elementwise_block,
+ * fuse_conv_bn_relu, conv_layout_nhwc, split_reductions, and the lowering knobs reduce_cached_elems, reduce_wave_elems, elementwise_block,
  * reduce_rows_per_block). */
 int cinn_amd_computation_build_and_compile(cinn_amd_builder_t b, const char* const* outputs, int32_t num_outputs,
                                            void* stream, const char* options, cinn_amd_computation_t* out);

@@ -238,3 +238,36 @@ def test_conv_batch_norm_residual_relu_fold_into_convolution_epilogues():
     assert not any("batch_norm" in g or " relu " in g for g in groups if " pre_run " not in g), groups
     # scale / shift of the folded batch norm are computed in fp32 ahead of time
     assert any("pre_run" in g and "divide" in g and "subtract" in g for g in groups), groups
+
+
+def test_reductions_over_non_trailing_axes_are_split_into_runs_and_steps():
+    # N, H, W of an NCHW tensor: the trailing run (H, W) stays an ordinary reduction (row template), the leading one
+    # becomes a reduce_run over [1][N][C]
+    b = NetBuilder("stat")
+    x = b.create_input(Float(16), [32, 64, 56, 56], "x")
+    comp = compile_only(b, [b.reduce_sum(x, [0, 2, 3], True)])
+    groups = [g for g in comp.fusion_groups().splitlines() if g.strip()]
+    assert len(groups) == 2 and "row_reduce" in groups[0] and "reduce_run_sum" in groups[1], groups
+    # axis 0 of a tall matrix: too few column blocks, so slices of the rows first (fp32 partial sums for fp16 input)
+    b = NetBuilder("tall")
+    x = b.create_input(Float(16), [8192, 1024], "x")
+    comp = compile_only(b, [b.reduce_sum(x, [0], False)])
+    src = comp.source_code()
+    assert src.count("__global__") == 2 and "cinn_block_column_reduce_sum_fp32" in src, src[-2000:]
+    assert "const float16* __restrict__ x, float* __restrict__" in src  # first step writes fp32 partial sums
+    # enough output elements: one step; a full reduction: slices of the single long row
+    b = NetBuilder("wide")
+    x = b.create_input(Float(32), [64, 128, 4096], "x")
+    assert compile_only(b, [b.reduce_max(x, [1], False)]).num_instructions() == 1
+    b = NetBuilder("all")
+    x = b.create_input(Float(32), [1024, 1024], "x")
+    assert compile_only(b, [b.reduce_sum(x, [], False)]).num_instructions() == 2
+    # switched off: a single general reduction, still the column kernel when the axes form one run
+    b = NetBuilder("off")
+    x = b.create_input(Float(32), [8192, 1024], "x")
+    comp = compile_only(b, [b.reduce_sum(x, [0], False)], split_reductions=False)
+    assert comp.num_instructions() == 1 and "cinn_block_column_reduce_sum_fp32" in comp.source_code()
+    # reductions over trailing axes only are left alone (softmax stays one kernel)
+    b = NetBuilder("sm")
+    x = b.create_input(Float(32), [512, 1024], "x")
+    assert compile_only(b, [b.softmax(x, axes=[-1])]).num_instructions() == 1
