@@ -113,6 +113,7 @@ void CodeGenHIP_Dev::VisitStore(const Store* op) {
   CINN_CHECK(lramp && lramp->lanes == ramp->lanes && lramp->stride == 1 && ramp->stride == 1);
   const char* copy_fn = "cinn_hip_copy_vec";
   if (op->buffer->memory_type == MemoryType::Global && op->buffer->streaming_store) copy_fn = "cinn_hip_store_stream_vec";
+  if (ld->buffer->memory_type == MemoryType::Global && ld->buffer->streaming_load) copy_fn = "cinn_hip_load_stream_vec";
   os_ << copy_fn << "<" << common::TypeCName(op->buffer->dtype) << ", " << ramp->lanes << ">(&"
       << op->buffer->name << "[";
   Visit(ramp->base);

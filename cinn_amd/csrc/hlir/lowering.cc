@@ -234,10 +234,12 @@ LoweringOptions LoweringOptions::FromEnv() {
   o.wave_row_elems_per_lane     = EnvInt("FLAGS_cinn_hip_reduce_wave_elems", o.wave_row_elems_per_lane);
   o.block_row_elems_per_thread  = EnvInt("FLAGS_cinn_hip_reduce_block_elems", o.block_row_elems_per_thread);
   o.nontemporal_store_bytes     = static_cast<int64_t>(EnvInt("FLAGS_cinn_hip_nontemporal_store_mb", 8)) << 20;
+  o.nontemporal_load_bytes      = static_cast<int64_t>(EnvInt("FLAGS_cinn_hip_nontemporal_load_mb", 0)) << 20;
   o.rows_per_wave               = EnvInt("FLAGS_cinn_hip_reduce_rows_per_wave", o.rows_per_wave);
   o.elementwise_block           = EnvInt("FLAGS_cinn_hip_elementwise_block", o.elementwise_block);
   o.rows_per_block              = EnvInt("FLAGS_cinn_hip_reduce_rows_per_block", o.rows_per_block);
   o.column_reduce               = EnvInt("FLAGS_cinn_hip_column_reduce", 1) != 0;
+  o.tiled_transpose             = EnvInt("FLAGS_cinn_hip_tiled_transpose", 1) != 0;
   return o;
 }
 
@@ -272,9 +274,13 @@ class ElementwiseEmitter {
 
   // values of group inputs that were staged into registers by a vector load: local buffer + lane
   std::map<const NodeData*, std::pair<BufferRef, Expr>> staged;
+  // values that are already at hand at the identity index (a tile staged through LDS)
+  std::map<const NodeData*, Expr> forced;
 
   Expr ValueAt(NodeData* v, const Index& idx) {
     if (idx.identity) {
+      auto f = forced.find(v);
+      if (f != forced.end()) return f->second;
       auto it = cache_.find(v);
       if (it != cache_.end()) return it->second;
     }
@@ -361,6 +367,12 @@ bool UsedAtIdentityOnly(const Group& g, const NodeData* v, int64_t numel) {
 }  // namespace
 
 namespace {
+void MarkStreamingInputs(GroupContext* ctx, int64_t threshold_bytes) {
+  if (threshold_bytes <= 0) return;
+  for (auto* v : ctx->group.inputs) {
+    if (v->numel() * v->dtype.bytes() >= threshold_bytes) ctx->global_bufs.at(v)->streaming_load = true;
+  }
+}
 void MarkStreamingOutputs(GroupContext* ctx, int64_t threshold_bytes) {
   if (threshold_bytes <= 0) return;
   for (auto* o : ctx->group.outputs) {
@@ -369,9 +381,127 @@ void MarkStreamingOutputs(GroupContext* ctx, int64_t threshold_bytes) {
 }
 }  // namespace
 
+// ---------------------------------------------------------------------------------------------------
+// Element-wise group around one transpose that moves the innermost axis of a group input: the input is staged
+// through LDS in TILE x TILE tiles over (output axis that holds the input's innermost axis, output's innermost
+// axis), so that both the reads of the input and the writes of the outputs walk contiguous memory.  Without it
+// consecutive threads read the input at the stride of the moved axis.  Every other operand of the group is at the
+// group's own index.  Returns false when the group does not have this form.
+// ---------------------------------------------------------------------------------------------------
+namespace {
+bool LowerTiledTranspose(const Group& group, GroupContext* ctx) {
+  Node* t = nullptr;
+  for (Node* n : group.nodes) {
+    if (n->op_type() == "transpose") {
+      if (t) return false;
+      t = n;
+    } else if (n->op->pattern != OpPatternKind::kElementWise) {
+      return false;
+    }
+  }
+  if (!t) return false;
+  NodeData* x = t->inputs[0];
+  if (ctx->produced.count(x)) return false;
+  for (Node* n : group.nodes)
+    for (auto* in : n->inputs)
+      if (in == x && n != t) return false;
+  const ShapeType& shape = t->outputs[0]->shape;
+  const int rank         = static_cast<int>(shape.size());
+  auto axis              = GetAttr<std::vector<int>>(t->attrs, "axis", {});
+  if (rank < 2 || static_cast<int>(axis.size()) != rank) return false;
+  for (auto& a : axis)
+    if (a < 0) a += rank;
+  if (axis[rank - 1] == rank - 1) return false;
+  int q = -1;
+  for (int i = 0; i < rank; ++i)
+    if (axis[i] == rank - 1) q = i;
+  if (q < 0) return false;
+  const int64_t Q = shape[q], N = shape[rank - 1];
+  if (Q < 16 || N < 16) return false;
+  for (auto* o : group.outputs)
+    if (o->shape != shape) return false;
+  for (auto* v : group.inputs)
+    if (v != x && v->shape != shape) return false;
+
+  const int tile   = x->dtype.bytes() >= 4 ? 32 : 64;
+  const int ty_n   = 256 / tile;
+  const int per    = tile / ty_n;
+  const int pitch  = tile + (x->dtype.bytes() >= 4 ? 1 : 2);  // odd number of 4-byte words per row
+  const int64_t gq = (Q + tile - 1) / tile, gn = (N + tile - 1) / tile;
+  ShapeType batch_shape;
+  for (int i = 0; i < rank - 1; ++i)
+    if (i != q) batch_shape.push_back(shape[i]);
+  int64_t batch = 1;
+  for (int d : batch_shape) batch *= d;
+  if (batch * gq * gn >= static_cast<int64_t>(std::numeric_limits<int32_t>::max())) return false;
+  const bool guard = Q % tile != 0 || N % tile != 0;
+
+  Expr bid = ir::MakeVar("bid", common::Int(32));
+  Expr tx  = ir::MakeVar("tx", common::Int(32));
+  Expr ty  = ir::MakeVar("ty", common::Int(32));
+  BufferRef lds = ctx->NewLocal("tile", x->dtype, static_cast<int64_t>(tile) * pitch, MemoryType::GPUShared);
+
+  std::vector<Expr> stmts;
+  Expr q0 = ctx->NewVar("q0", common::Int(32));
+  Expr n0 = ctx->NewVar("n0", common::Int(32));
+  Expr b  = ctx->NewVar("b", common::Int(32));
+  stmts.push_back(ir::MakeLet(n0, (bid % I32(gn)) * I32(tile)));
+  stmts.push_back(ir::MakeLet(q0, ((bid / I32(gn)) % I32(gq)) * I32(tile)));
+  stmts.push_back(ir::MakeLet(b, bid / I32(gn * gq)));
+  auto batch_coords = Decompose(b, batch_shape);
+  auto coords_of    = [&](const Expr& qc, const Expr& nc) {
+    std::vector<Expr> c(rank);
+    for (int i = 0, k = 0; i < rank - 1; ++i)
+      if (i != q) c[i] = batch_coords[k++];
+    c[q]        = qc;
+    c[rank - 1] = nc;
+    return c;
+  };
+  {
+    // phase 1: threads along the input's innermost axis
+    Expr i  = ir::MakeVar("i", common::Int(32));
+    Expr ln = ty + i * I32(ty_n);
+    Index out_idx;
+    out_idx.coords = coords_of(q0 + tx, n0 + ln);
+    Index in_idx   = TransformIndex(*t, 0, out_idx);
+    Expr copy = ir::MakeStore(lds, ir::MakeLoad(ctx->global_bufs.at(x), FlatOf(in_idx, x->shape)), ln * I32(pitch) + tx);
+    if (guard) copy = ir::MakeIf(((q0 + tx) < I32(Q)) && ((n0 + ln) < I32(N)), copy);
+    stmts.push_back(ir::MakeFor(i, I32(0), I32(per), ForType::Unrolled, copy));
+  }
+  stmts.push_back(ir::MakeCall(Type(), "__syncthreads", {}));
+  {
+    // phase 2: threads along the outputs' innermost axis
+    Expr i  = ir::MakeVar("j", common::Int(32));
+    Expr lq = ty + i * I32(ty_n);
+    std::vector<Expr> body;
+    ElementwiseEmitter emitter(ctx, &body);
+    Index idx;
+    idx.coords   = coords_of(q0 + lq, n0 + tx);
+    Expr flat    = ctx->NewVar("o", common::Int(32));
+    body.push_back(ir::MakeLet(flat, Compose(idx.coords, shape)));
+    idx.flat     = flat;
+    idx.identity = true;
+    emitter.forced[t->outputs[0]] = ir::MakeLoad(lds, tx * I32(pitch) + lq);
+    for (auto* o : group.outputs) {
+      Expr value = emitter.ValueAt(o, idx);
+      body.push_back(ir::MakeStore(ctx->global_bufs.at(o), value, flat));
+    }
+    Expr work = ir::MakeBlock(body);
+    if (guard) work = ir::MakeIf(((q0 + lq) < I32(Q)) && ((n0 + tx) < I32(N)), work);
+    stmts.push_back(ir::MakeFor(i, I32(0), I32(per), ForType::Unrolled, work));
+  }
+  Expr threads_x  = ir::MakeFor(tx, I32(0), I32(tile), ForType::Serial, ir::MakeBlock(stmts), ThreadAxis(0));
+  Expr threads_y  = ir::MakeFor(ty, I32(0), I32(ty_n), ForType::Serial, threads_x, ThreadAxis(1));
+  ctx->func->body = ir::MakeFor(bid, I32(0), I32(batch * gq * gn), ForType::Serial, threads_y, BlockAxis(0));
+  return true;
+}
+}  // namespace
+
 ir::LoweredFuncRef OpLowerer::LowerElementwise(const Group& group) const {
   GroupContext ctx(group);
+  if (options_.tiled_transpose && LowerTiledTranspose(group, &ctx)) return ctx.func;
   MarkStreamingOutputs(&ctx, options_.nontemporal_store_bytes);
+  MarkStreamingInputs(&ctx, options_.nontemporal_load_bytes);
   CINN_CHECK(!group.outputs.empty());
   const int64_t numel = group.outputs[0]->numel();
   for (auto* o : group.outputs) CINN_CHECK_EQ(o->numel(), numel) << "outputs of an element-wise group differ in size";
@@ -826,6 +956,7 @@ class RowReduceEmitter {
 ir::LoweredFuncRef OpLowerer::LowerRowReduce(const Group& group) const {
   GroupContext ctx(group);
   MarkStreamingOutputs(&ctx, options_.nontemporal_store_bytes);
+  MarkStreamingInputs(&ctx, options_.nontemporal_load_bytes);
   std::map<const NodeData*, RowKind> kinds;
   CINN_CHECK(ClassifyRowReduceGroup(group.nodes, group.rows, group.cols, &kinds))
       << "group " << group.func_name << " is not a row-reduce group";

@@ -32,6 +32,8 @@ struct LoweringOptions {
   // outputs of at least this many bytes are written with non-temporal stores (0 disables): a large
   // streamed output would otherwise evict the input rows still to be read from the last-level cache
   int64_t nontemporal_store_bytes{8 << 20};
+  // inputs of at least this many bytes are read with non-temporal loads (0 disables)
+  int64_t nontemporal_load_bytes{0};
   // threads of an element-wise block
   int elementwise_block{256};
   // waves (rows) per block when one wavefront owns a row
@@ -41,6 +43,8 @@ struct LoweringOptions {
   int rows_per_wave{1};
   // reductions over one non-trailing run of axes use the column-reduce kernel (off: one thread per output element)
   bool column_reduce{true};
+  // element-wise groups around a transpose that moves the innermost axis stage the input through LDS tiles
+  bool tiled_transpose{true};
   static LoweringOptions FromEnv();
 };
 

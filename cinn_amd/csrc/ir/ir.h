@@ -144,6 +144,7 @@ struct Buffer {
   // global output that is written once and not re-read by this kernel: vector stores to it carry the
   // non-temporal hint so that they do not displace the data still being read
   bool streaming_store{false};
+  bool streaming_load{false};  // read once by the kernel: vector loads bypass the cache allocation policy
   Buffer(std::string n, Type t, MemoryType m, int64_t size) : name(std::move(n)), dtype(t), memory_type(m), num_elements(size) {}
 };
 using BufferRef = std::shared_ptr<Buffer>;

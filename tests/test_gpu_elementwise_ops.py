@@ -135,6 +135,40 @@ def test_injective_ops(gpu):
     assert np.array_equal(sq, x)
 
 
+@pytest.mark.parametrize("shape,axis", [
+    ([4096, 4096], [1, 0]),            # whole tiles
+    ([1000, 37], [1, 0]),              # ragged in both tile directions
+    ([5, 100, 7, 70], [0, 3, 2, 1]),   # innermost axis moved to position 1, two batch axes
+    ([8, 64, 28, 28], [0, 2, 3, 1]),   # NCHW -> NHWC: the last two output axes come from different input axes
+    ([8, 28, 28, 64], [0, 3, 1, 2]),   # NHWC -> NCHW
+    ([3, 17, 33], [2, 0, 1]),
+    ([6, 40, 50], [1, 0, 2]),          # innermost axis stays: plain element-wise template
+])
+@pytest.mark.parametrize("dtype", ["float32", "float16", "int32"])
+def test_transpose_tiles(gpu, shape, axis, dtype):
+    """transpose (alone and with fused element-wise neighbours) is a pure permutation: bit-exact against numpy"""
+    rng = np.random.default_rng(12)
+    if dtype == "int32":
+        x, ty = rng.integers(-1000, 1000, shape).astype(np.int32), Int(32)
+    else:
+        x, ty = rng.standard_normal(shape).astype(dtype), (Float(32) if dtype == "float32" else Float(16))
+    y = rng.integers(-5, 5, [shape[a] for a in axis]).astype(x.dtype)
+    moves_last = axis[-1] != len(shape) - 1 and min(shape[-1], shape[axis[-1]]) >= 16
+    for variant in ("plain", "consumer", "producer"):
+        b = NetBuilder("tp_" + variant)
+        X, Y = b.create_input(ty, shape, "x"), b.create_input(ty, list(y.shape), "y")
+        if variant == "plain":
+            out, want = b.transpose(X, axis), x.transpose(axis)
+        elif variant == "consumer":  # the LDS tile feeds a fused element-wise consumer
+            out, want = b.add(b.transpose(X, axis), Y), x.transpose(axis) + y
+        else:  # a producer ahead of the transpose: the generic element-wise template
+            out, want = b.add(b.transpose(b.identity(X), axis), Y), x.transpose(axis) + y
+        (got,), comp = run(b, {X: x, Y: y}, [out])
+        assert comp.num_instructions() == 1
+        assert ("__shared__" in comp.source_code()) == (moves_last and variant != "producer"), variant
+        assert np.array_equal(got, want), variant  # small integers added to the values: exact in every type here
+
+
 @pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
 def test_sixteen_bit_elementwise(gpu, dtype):
     from cinn_amd.common import BFloat16, bfloat16_bits_to_float32, float32_to_bfloat16_bits
