@@ -240,6 +240,7 @@ LoweringOptions LoweringOptions::FromEnv() {
   o.rows_per_block              = EnvInt("FLAGS_cinn_hip_reduce_rows_per_block", o.rows_per_block);
   o.column_reduce               = EnvInt("FLAGS_cinn_hip_column_reduce", 1) != 0;
   o.tiled_transpose             = EnvInt("FLAGS_cinn_hip_tiled_transpose", 1) != 0;
+  o.sub_wave_rows               = EnvInt("FLAGS_cinn_hip_sub_wave_rows", 1) != 0;
   return o;
 }
 
@@ -583,8 +584,8 @@ namespace {
 
 struct RowReducePlan {
   int64_t rows, cols;
-  int team;            // threads that share a row: 64 (one wavefront) or the whole block
-  int rows_per_block;  // > 1 only when team == 64
+  int team;            // threads that share a row: a power of two up to 32 lanes, 64 (one wavefront) or the whole block
+  int rows_per_block;  // > 1 only when team <= 64
   int vec;             // elements per vector access
   int chunks;          // vectors per thread and row
   bool guard_cols;     // cols is not a multiple of team * vec
@@ -907,14 +908,21 @@ class RowReduceEmitter {
     for (auto& a : accs) {
       NodeData* out = a.node->outputs[0];
       bool wave     = plan_.team == 64;
+      bool sub_wave = plan_.team < 64;  // several rows per wavefront
       Expr result;
       if (a.index) {
-        std::string fn = std::string(wave ? "cinn_wave_" : "cinn_block_") + a.kind;
-        result = ir::MakeCall(common::Int(32), fn, {ir::MakeLoad(a.value, I32(0)), ir::MakeLoad(a.index, I32(0))});
+        std::string fn = std::string(sub_wave ? "cinn_team_" : wave ? "cinn_wave_" : "cinn_block_") + a.kind;
+        std::vector<Expr> args = {ir::MakeLoad(a.value, I32(0)), ir::MakeLoad(a.index, I32(0))};
+        if (sub_wave) args.push_back(I32(plan_.team));
+        result = ir::MakeCall(common::Int(32), fn, args);
       } else {
         std::string suffix = ReduceSuffix(a.kind, a.acc_type);
-        std::string fn     = wave ? "cinn_wave_shuffle_" + suffix + "_internal" : "cinn_block_reduce_" + suffix + "_internal";
-        result = ir::MakeCast(out->dtype, ir::MakeCall(a.acc_type, fn, {ir::MakeLoad(a.value, I32(0))}));
+        std::string fn     = sub_wave ? "cinn_team_shuffle_" + suffix + "_internal"
+                             : wave   ? "cinn_wave_shuffle_" + suffix + "_internal"
+                                      : "cinn_block_reduce_" + suffix + "_internal";
+        std::vector<Expr> args = {ir::MakeLoad(a.value, I32(0))};
+        if (sub_wave) args.push_back(I32(plan_.team));
+        result = ir::MakeCast(out->dtype, ir::MakeCall(a.acc_type, fn, args));
       }
       Expr var = ctx_->NewVar("red", out->dtype);
       row_stmts_->push_back(ir::MakeLet(var, result));
@@ -978,8 +986,15 @@ ir::LoweredFuncRef OpLowerer::LowerRowReduce(const Group& group) const {
 
   const int wave = target_.wavefront_size();
   CINN_CHECK_EQ(wave, 64) << "the row-reduce template is written for 64-lane wavefronts";
-  int64_t per_lane = (plan.cols + wave - 1) / wave;
-  if (per_lane <= options_.wave_row_elems_per_lane) {
+  int64_t per_lane       = (plan.cols + wave - 1) / wave;
+  const int64_t row_vecs = (plan.cols + plan.vec - 1) / plan.vec;
+  if (options_.sub_wave_rows && row_vecs <= wave / 2) {
+    // short rows: a team of the fewest lanes that hold the row with one vector each, 64 / team rows per wavefront
+    int team = 1;
+    while (team < row_vecs) team *= 2;
+    plan.team           = team;
+    plan.rows_per_block = 256 / team;
+  } else if (per_lane <= options_.wave_row_elems_per_lane) {
     plan.team           = wave;
     plan.rows_per_block = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(options_.rows_per_block, plan.rows)));
   } else {

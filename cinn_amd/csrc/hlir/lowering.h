@@ -45,6 +45,8 @@ struct LoweringOptions {
   bool column_reduce{true};
   // element-wise groups around a transpose that moves the innermost axis stage the input through LDS tiles
   bool tiled_transpose{true};
+  // rows of at most 32 vectors are given to teams of 1 .. 32 lanes, several rows per wavefront
+  bool sub_wave_rows{true};
   static LoweringOptions FromEnv();
 };
 

@@ -193,3 +193,37 @@ def test_fused_reduce_with_producers_and_consumers(gpu):
     e64 = np.exp(x.astype(np.float64))
     np.testing.assert_allclose(y, (e64 - e64.max(1, keepdims=True)) / e64.sum(1, keepdims=True), rtol=1e-5, atol=1e-6)
     np.testing.assert_allclose(s, e64.sum(1, keepdims=True), rtol=1e-5)
+
+
+# Short rows are shared out to teams of 1 .. 32 lanes (several rows per wavefront): every team size, rows that do not
+# fill the last block, columns that do not fill the team's vectors.
+@pytest.mark.parametrize("cols", [1, 2, 3, 5, 8, 16, 17, 33, 64, 100, 128, 129])
+def test_short_rows_share_a_wavefront(gpu, cols):
+    rows = 1003
+    rng = np.random.default_rng(cols)
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    xi = rng.integers(-3, 3, (rows, cols)).astype(np.int32)  # many ties for argmax
+    b = NetBuilder("short")
+    X, XI = b.create_input(Float(32), x.shape, "x"), b.create_input(Int(32), xi.shape, "xi")
+    H = b.create_input(Float(16), x.shape, "h")
+    outs = [b.softmax(X, axes=[-1]), b.reduce_sum(XI, [1], False), b.reduce_max(XI, [1], True), b.argmax(XI, axis=1),
+            b.softmax(H, axes=[-1])]
+    (sm, s, m, am, smh), _ = run(b, {X: x, XI: xi, H: x.astype(np.float16)}, outs)
+    np.testing.assert_allclose(sm, oracle.softmax(x), rtol=1e-5, atol=0)
+    assert np.array_equal(s, xi.sum(1)) and np.array_equal(m, xi.max(1, keepdims=True))
+    assert np.array_equal(am, xi.argmax(1).astype(np.int32))  # first maximum
+    assert_close_fp16(smh, oracle.softmax(x.astype(np.float16)))
+
+
+def test_short_row_layer_norm(gpu):
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((4099, 24)).astype(np.float32)
+    g, be = rng.uniform(0.5, 1.5, 24).astype(np.float32), rng.uniform(-1, 1, 24).astype(np.float32)
+    b = NetBuilder("ln_short")
+    X, G, B = b.create_input(Float(32), x.shape, "x"), b.create_input(Float(32), [24], "g"), b.create_input(Float(32), [24], "b")
+    (y, mean, var), comp = run(b, {X: x, G: g, B: be}, b.paddle_layer_norm(X, G, B, epsilon=1e-5))
+    assert comp.num_instructions() == 1
+    wy, wm, wv = oracle.layer_norm(x, g, be, 1e-5)
+    np.testing.assert_allclose(y, wy, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(mean, wm, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(var, wv, rtol=1e-5, atol=1e-6)
