@@ -65,12 +65,15 @@ void CodeGenHIP_Dev::PrintTempBuffers(const LoweredFunc& func) {
   for (auto& buf : func.temp_bufs) {
     Indent();
     CINN_CHECK_GT(buf->num_elements, 0) << "temporary buffer " << buf->name << " has no size";
+    // the alignment specifier leads the declaration: after __shared__ (a GNU attribute) it is rejected by some
+    // front-end configurations ("an attribute list cannot appear here")
+    os_ << "alignas(16) ";
     switch (buf->memory_type) {
       case MemoryType::GPUShared: os_ << "__shared__ "; break;
       case MemoryType::GPULocal: break;
       default: CINN_CHECK(false) << "temporary buffer " << buf->name << " must live in LDS or registers";
     }
-    os_ << "alignas(16) " << common::TypeCName(buf->dtype) << " " << buf->name << "[" << buf->num_elements << "];\n";
+    os_ << common::TypeCName(buf->dtype) << " " << buf->name << "[" << buf->num_elements << "];\n";
   }
 }
 
