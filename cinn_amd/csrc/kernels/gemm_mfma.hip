@@ -2,7 +2,7 @@
 //
 //   C[M,N] = alpha * op(A)[M,K] * op(B)[K,N] + beta * C          (row-major, optional batch)
 //
-// Four kernels:
+// Kernels:
 //   * gemm16_dma_kernel   - bf16 / fp16 with A stored [M][K] (the common case) and K % 128 == 0: 256x256x64 tile, 512
 //     threads, direct global -> LDS loads of whole 128-byte lines into two stages, transposing LDS reads for
 //     row-major B; see the comment at the kernel.
@@ -16,6 +16,9 @@
 //   * gemm32_mfma_kernel  - fp32 on v_mfma_f32_32x32x2f32, 128x128 tile (64x64 when that is what fills the chip),
 //     for M%128 == N%128 == K%32 == 0.
 //   * gemm_generic_kernel - any shape / transpose / type (fp16, bf16, fp32, fp64): 64x64 LDS tile, FMA units.
+// Shapes the tile kernels do not take (ragged, or too few tiles to fill the chip) run on the bounds-checked MFMA
+// kernel of conv_nhwc_mfma.hip as a 1x1 convolution, after transposing copies of the operands that are not
+// K-contiguous (transpose2d_kernel); gemm_generic_kernel is left with K % (16 bytes) != 0 and fp64.
 #include <hip/hip_runtime.h>
 
 #include <climits>
@@ -667,6 +670,60 @@ gemm_generic_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restr
   }
 }
 
+// [rows][cols] -> [cols][rows] through a 32x32 LDS tile (odd pitch), blockIdx.z = batch.  Brings an operand whose
+// contiguous axis is not K into the K-contiguous form the bounds-checked MFMA path wants.
+template <typename T>
+__global__ void __launch_bounds__(256)
+transpose2d_kernel(const T* __restrict__ in, T* __restrict__ out, int rows, int cols, int64_t in_stride, int64_t out_stride) {
+  __shared__ T tile[32][33];
+  in += (int64_t)blockIdx.z * in_stride;
+  out += (int64_t)blockIdx.z * out_stride;
+  const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+  const int tx = threadIdx.x, ty = threadIdx.y;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = r0 + ty + 8 * i, c = c0 + tx;
+    if (r < rows && c < cols) tile[ty + 8 * i][tx] = in[(int64_t)r * cols + c];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = c0 + ty + 8 * i, r = r0 + tx;
+    if (r < rows && c < cols) out[(int64_t)c * rows + r] = tile[tx][ty + 8 * i];
+  }
+}
+
+// scratch for transposed operands; grown on demand and kept.  One buffer per process: GEMMs that take this path on
+// different streams at the same time would share it.
+char* TransposeWorkspace(size_t bytes) {
+  static char* buffer    = nullptr;
+  static size_t capacity = 0;
+  if (bytes > capacity) {
+    if (buffer) {
+      CINN_HIP_CALL(hipDeviceSynchronize());
+      CINN_HIP_CALL(hipFree(buffer));
+    }
+    CINN_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&buffer), bytes));
+    capacity = bytes;
+  }
+  return buffer;
+}
+
+void LaunchTranspose(const void* in, void* out, int rows, int cols, int batch, int64_t in_stride, int elem_bytes,
+                     hipStream_t stream) {
+  dim3 grid((cols + 31) / 32, (rows + 31) / 32, batch);
+  CINN_RT_CHECK(grid.y <= 65535, "gemm: operand with %d rows is too tall for the transposing copy", rows);
+  const int64_t out_stride = (int64_t)rows * cols;
+  if (elem_bytes == 2) {
+    hipLaunchKernelGGL((transpose2d_kernel<uint16_t>), grid, dim3(32, 8), 0, stream, static_cast<const uint16_t*>(in),
+                       static_cast<uint16_t*>(out), rows, cols, in_stride, out_stride);
+  } else {
+    hipLaunchKernelGGL((transpose2d_kernel<uint32_t>), grid, dim3(32, 8), 0, stream, static_cast<const uint32_t*>(in),
+                       static_cast<uint32_t*>(out), rows, cols, in_stride, out_stride);
+  }
+  CINN_HIP_CALL(hipGetLastError());
+}
+
 enum class GemmType { kF16, kBF16, kF32, kF64 };
 
 struct GemmProblem {
@@ -802,17 +859,43 @@ void RunGemm(const GemmProblem& p, hipStream_t stream) {
   const bool aligned16 = reinterpret_cast<uintptr_t>(p.a) % 16 == 0 && reinterpret_cast<uintptr_t>(p.b) % 16 == 0 &&
                          p.stride_a % 4 == 0 && p.stride_b % 4 == 0;
   const bool fast32 = !ForceGeneric() && p.m % kF32Tile == 0 && p.n % kF32Tile == 0 && p.k % kF32K == 0 && aligned16;
-  // Ragged shapes whose operands are both K-contiguous (A [m,k], B stored [n,k]) go to the channels-last
-  // convolution kernels: a 1x1 convolution over m "pixels" is this GEMM, and those kernels bound-check every tile
-  // edge and pick a tile that fills the chip for small m or n.
+  // Shapes the big-tile kernels do not take (ragged, or so few tiles that most CUs would idle) go to the
+  // channels-last convolution kernels: a 1x1 convolution over m "pixels" is this GEMM with both operands
+  // K-contiguous (A [m,k], B stored [n,k]); those kernels bound-check every tile edge, use 64x64 tiles and split K
+  // when the grid is small.  An operand stored the other way round is transposed into scratch first, which costs one
+  // pass over that operand.
   const int elem_bytes = p.type == GemmType::kF32 ? 4 : (p.type == GemmType::kF64 ? 8 : 2);
   const bool tile_fit  = p.type == GemmType::kF32 ? fast32 : fast16;
-  const bool k_contig  = !ForceGeneric() && p.type != GemmType::kF64 && !p.trans_a && p.trans_b && p.k % (16 / elem_bytes) == 0;
-  if (k_contig && !tile_fit) {
+  const int64_t tiles  = p.type == GemmType::kF32 ? (int64_t)(p.m / 64) * (p.n / 64) * p.batch
+                                                  : (int64_t)(p.m / kBM) * (p.n / kBN) * p.batch;
+  const bool few_tiles = tile_fit && tiles < 64;
+  const bool flexible  = !ForceGeneric() && p.type != GemmType::kF64 && p.k % (16 / elem_bytes) == 0 &&
+                         reinterpret_cast<uintptr_t>(p.a) % 16 == 0 && reinterpret_cast<uintptr_t>(p.b) % 16 == 0;
+  if (flexible && (!tile_fit || few_tiles)) {
+    const char* a_base = static_cast<const char*>(p.a);
+    const char* b_base = static_cast<const char*>(p.b);
+    int64_t stride_a = p.stride_a, stride_b = p.stride_b;
+    if (p.trans_a || !p.trans_b) {
+      const int batch_a    = p.trans_a ? (p.stride_a == 0 ? 1 : p.batch) : 0;
+      const int batch_b    = !p.trans_b ? (p.stride_b == 0 ? 1 : p.batch) : 0;
+      const size_t bytes_a = (size_t)batch_a * p.m * p.k * elem_bytes;
+      const size_t bytes_b = (size_t)batch_b * p.k * p.n * elem_bytes;
+      char* scratch        = TransposeWorkspace(bytes_a + bytes_b);
+      if (p.trans_a) {  // stored [k][m]
+        LaunchTranspose(p.a, scratch, p.k, p.m, batch_a, p.stride_a, elem_bytes, stream);
+        a_base   = scratch;
+        stride_a = p.stride_a == 0 ? 0 : (int64_t)p.m * p.k;
+      }
+      if (!p.trans_b) {  // stored [k][n]
+        LaunchTranspose(p.b, scratch + bytes_a, p.k, p.n, batch_b, p.stride_b, elem_bytes, stream);
+        b_base   = scratch + bytes_a;
+        stride_b = p.stride_b == 0 ? 0 : (int64_t)p.k * p.n;
+      }
+    }
     for (int b = 0; b < p.batch; ++b) {
       cinn_hip_kernels::ConvNhwcArgs a;
-      a.x = static_cast<const char*>(p.a) + (int64_t)b * p.stride_a * elem_bytes;
-      a.w = static_cast<const char*>(p.b) + (int64_t)b * p.stride_b * elem_bytes;
+      a.x = a_base + (int64_t)b * stride_a * elem_bytes;
+      a.w = b_base + (int64_t)b * stride_b * elem_bytes;
       a.y = static_cast<char*>(p.c) + (int64_t)b * p.stride_c * elem_bytes;
       a.scale = a.shift = nullptr;
       a.residual        = p.beta != 0.0f ? a.y : nullptr;

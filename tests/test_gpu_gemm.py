@@ -136,6 +136,39 @@ def test_16bit_direct_to_lds_kernel(gpu, kind, tb, alpha, beta):
     assert np.all(np.abs(got - exact) <= ulp * np.maximum(np.abs(exact), 1e-3 * scale) + 2.0 ** -24)
 
 
+@pytest.mark.parametrize("kind", ["float32", "float16", "bfloat16"])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_ragged_shapes_through_transposing_copies(gpu, kind, ta, tb):
+    """Shapes no big-tile kernel takes (K a multiple of one 16-byte chunk): operands that are not K-contiguous are
+    transposed into scratch and the bounds-checked MFMA path runs; two batches with B broadcast, alpha and beta."""
+    batch, m, n, k = 2, 200, 136, 72
+    rng = np.random.default_rng(43)
+    a = (rng.standard_normal((batch, k, m) if ta else (batch, m, k)) * 0.1).astype(np.float32)
+    b = (rng.standard_normal((1, n, k) if tb else (1, k, n)) * 0.1).astype(np.float32)
+    c0 = rng.standard_normal((batch, m, n)).astype(np.float32)
+    if kind == "float32":
+        ab, bb, cb = a, b, c0
+        af, bf, cf = (v.astype(np.float64) for v in (a, b, c0))
+        got = call_cublas(ab, bb, (batch, m, n), kind, ta, tb, alpha=0.5, beta=2.0, c_init=cb).astype(np.float64)
+        tol = 1e-5
+    elif kind == "float16":
+        ab, bb, cb = a.astype(np.float16), b.astype(np.float16), c0.astype(np.float16)
+        af, bf, cf = (v.astype(np.float64) for v in (ab, bb, cb))
+        got = call_cublas(ab, bb, (batch, m, n), kind, ta, tb, alpha=0.5, beta=2.0, c_init=cb).astype(np.float64)
+        tol = 2.0 ** -10
+    else:
+        ab, bb, cb = (float32_to_bfloat16_bits(v) for v in (a, b, c0))
+        af, bf, cf = (bfloat16_bits_to_float32(v).astype(np.float64) for v in (ab, bb, cb))
+        got = bfloat16_bits_to_float32(
+            call_cublas(ab, bb, (batch, m, n), kind, ta, tb, alpha=0.5, beta=2.0, c_init=cb)).astype(np.float64)
+        tol = 2.0 ** -7
+    am = np.swapaxes(af, 1, 2) if ta else af
+    bm = np.swapaxes(bf, 1, 2) if tb else bf
+    exact = 0.5 * (am @ bm) + 2.0 * cf
+    scale = 0.5 * (np.abs(am) @ np.abs(bm)) + 2.0 * np.abs(cf)
+    assert np.all(np.abs(got - exact) <= tol * np.maximum(np.abs(exact), 1e-3 * scale) + 1e-5 * scale * (kind == "float32"))
+
+
 @pytest.mark.parametrize("kind", ["float16", "bfloat16"])
 def test_config3_4096_cubed(gpu, kind):
     rng = np.random.default_rng(31)
