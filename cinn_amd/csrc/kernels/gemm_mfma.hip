@@ -254,22 +254,33 @@ __device__ __forceinline__ void AsyncCopy16(const void* src, char* lds_base_unif
 constexpr int kD64BK   = 64;
 constexpr int kD64Tile = kBM * kD64BK * 2;  // one operand tile of a stage: 32 KiB
 
-template <typename T, bool B_KC>
-__global__ void __launch_bounds__(kDmaThreads)
+// BM x BN block tile on a WAVES_M x WAVES_N grid of wavefronts: 256x256 on 2x4 (8 wavefronts of 128x64) for large
+// problems, 128x128 on 2x2 (4 wavefronts of 64x64, two blocks per CU) when 256x256 tiles would leave CUs idle.
+template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ void __launch_bounds__(64 * WAVES_M * WAVES_N)
 gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ C, int M, int N,
                     int K, int64_t lda, int64_t ldb, int64_t ldc, float alpha, float beta, int64_t stride_a,
                     int64_t stride_b, int64_t stride_c, int xcd_cols, int sub_rows, int sub_cols) {
-  __shared__ __attribute__((aligned(1024))) char lds[4 * kD64Tile];
+  constexpr int NW      = WAVES_M * WAVES_N;
+  constexpr int THREADS = 64 * NW;
+  constexpr int TM      = BM / WAVES_M / 32;  // MFMA tiles per wavefront along M and N
+  constexpr int TN      = BN / WAVES_N / 32;
+  constexpr int A_TILE  = BM * kD64BK * 2;    // bytes of one operand tile of a stage
+  constexpr int B_TILE  = BN * kD64BK * 2;
+  constexpr int LPA     = BM / 8 / NW;        // loads (of 1 KiB per wavefront) per thread, operand and step
+  constexpr int LPB     = BN / 8 / NW;
+  static_assert(LPA >= 1 && LPB >= 1 && TM >= 1 && TN >= 1 && (LPA + LPB) % 2 == 0, "unsupported tile shape");
+  __shared__ __attribute__((aligned(1024))) char lds[2 * (A_TILE + B_TILE)];
   char* const sa0 = lds;
-  char* const sb0 = lds + kD64Tile;
-  char* const sa1 = lds + 2 * kD64Tile;
-  char* const sb1 = lds + 3 * kD64Tile;
+  char* const sb0 = lds + A_TILE;
+  char* const sa1 = lds + A_TILE + B_TILE;
+  char* const sb1 = lds + 2 * A_TILE + B_TILE;
   typedef typename Half16<T>::vec8 vec8;
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm   = wave >> 2;
-  const int wn   = wave & 3;
+  const int wm   = wave / WAVES_N;
+  const int wn   = wave % WAVES_N;
 
   int tile_row, tile_col;
   if (sub_rows > 0) {
@@ -277,71 +288,77 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     tile_row = (xcd / xcd_cols) * sub_rows + idx / sub_cols;
     tile_col = (xcd % xcd_cols) * sub_cols + idx % sub_cols;
   } else {
-    const int tiles_n = N / kBN;
+    const int tiles_n = N / BN;
     tile_row = blockIdx.x / tiles_n;
     tile_col = blockIdx.x % tiles_n;
   }
-  const int m0 = tile_row * kBM;
-  const int n0 = tile_col * kBN;
+  const int m0 = tile_row * BM;
+  const int n0 = tile_col * BN;
   A += (int64_t)blockIdx.y * stride_a;
   B += (int64_t)blockIdx.y * stride_b;
   C += (int64_t)blockIdx.y * stride_c;
 
-  // Each wavefront issues 4 loads per operand and step; load q = 4 wave + t fills LDS bytes [1024 q, 1024 q + 1024)
-  // of the operand tile: 8 rows of a [row][64 halves] tile, or 2 k-rows of a [k][256 halves] tile.
-  const uint16_t* a_src[4];
-  const uint16_t* b_src[4];
+  // Load q = LPA wave + t of an operand fills LDS bytes [1024 q, 1024 q + 1024) of its tile: 8 rows of a
+  // [row][64 halves] tile, or 512 / BN k-rows of a [k][BN halves] tile.
+  const uint16_t* a_src[LPA];
+  const uint16_t* b_src[LPB];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    const int q   = wave * 4 + t;
-    const int row = 8 * q + (lane >> 3);
+  for (int t = 0; t < LPA; ++t) {
+    const int row = 8 * (wave * LPA + t) + (lane >> 3);
     const int key = (row ^ (row >> 3)) & 7;
     a_src[t]      = A + (int64_t)(m0 + row) * lda + (((lane & 7) ^ key) << 3);
+  }
+#pragma unroll
+  for (int t = 0; t < LPB; ++t) {
+    const int q = wave * LPB + t;
     if (B_KC) {
-      b_src[t] = B + (int64_t)(n0 + row) * ldb + (((lane & 7) ^ key) << 3);
+      const int row = 8 * q + (lane >> 3);
+      const int key = (row ^ (row >> 3)) & 7;
+      b_src[t]      = B + (int64_t)(n0 + row) * ldb + (((lane & 7) ^ key) << 3);
     } else {
-      const int krow  = 2 * q + (lane >> 5);
-      const int chunk = (lane & 31) ^ (2 * (krow & 3));
-      b_src[t]        = B + (int64_t)krow * ldb + n0 + (chunk << 3);
+      constexpr int CH = BN / 8;  // 16-byte chunks per k-row
+      const int krow   = q * (64 / CH) + lane / CH;
+      const int chunk  = (lane % CH) ^ (2 * (krow & 3));
+      b_src[t]         = B + (int64_t)krow * ldb + n0 + (chunk << 3);
     }
   }
   const int64_t b_step = B_KC ? kD64BK : (int64_t)kD64BK * ldb;
-  // load t of step kt: 0..3 the A tile, 4..7 the B tile
+  // load t of step kt: first the LPA loads of the A tile, then the LPB loads of the B tile
   auto issue_one = [&](char* a_tile, char* b_tile, int kt, int t) {
-    if (t < 4) {
-      AsyncCopy16(a_src[t] + (int64_t)kt * kD64BK, a_tile + (wave * 4 + t) * 1024);
+    if (t < LPA) {
+      AsyncCopy16(a_src[t] + (int64_t)kt * kD64BK, a_tile + (wave * LPA + t) * 1024);
     } else {
-      AsyncCopy16(b_src[t - 4] + kt * b_step, b_tile + (wave * 4 + t - 4) * 1024);
+      AsyncCopy16(b_src[t - LPA] + kt * b_step, b_tile + (wave * LPB + t - LPA) * 1024);
     }
   };
 
-  f32x16 acc[4][2];
+  f32x16 acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
   const int frag_row = lane & 31;
   const int frag_kg  = lane >> 5;
   struct Frags {
-    vec8 a[4];
-    vec8 b[2];
+    vec8 a[TM];
+    vec8 b[TN];
   };
   auto read_a = [&](const char* a_tile, int kk, int i, Frags& f) {
-    f.a[i] = *reinterpret_cast<const vec8*>(a_tile + TileOffset(wm * 128 + i * 32 + frag_row, kk * 2 + frag_kg));
+    f.a[i] = *reinterpret_cast<const vec8*>(a_tile + TileOffset(wm * (TM * 32) + i * 32 + frag_row, kk * 2 + frag_kg));
   };
   auto read_b = [&](const char* b_tile, int kk, int j, Frags& f) {
     if (B_KC) {
-      f.b[j] = *reinterpret_cast<const vec8*>(b_tile + TileOffset(wn * 64 + j * 32 + frag_row, kk * 2 + frag_kg));
+      f.b[j] = *reinterpret_cast<const vec8*>(b_tile + TileOffset(wn * (TN * 32) + j * 32 + frag_row, kk * 2 + frag_kg));
     } else {
       s16x4 part[2];
 #pragma unroll
       for (int r = 0; r < 2; ++r) {
         const int k   = kk * 16 + 4 * (2 * frag_kg + r) + ((lane & 15) >> 2);
-        const int n   = wn * 64 + j * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-        const int off = k * 512 + (((n >> 3) ^ (2 * (k & 3))) << 4) + (n & 7) * 2;
+        const int n   = wn * (TN * 32) + j * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+        const int off = k * (BN * 2) + (((n >> 3) ^ (2 * (k & 3))) << 4) + (n & 7) * 2;
         part[r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(b_tile + off));
       }
       s16x8 both = __builtin_shufflevector(part[0], part[1], 0, 1, 2, 3, 4, 5, 6, 7);
@@ -349,27 +366,38 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     }
   };
 #define CINN_SB __builtin_amdgcn_sched_barrier(0)
-  // one 16-deep slice: the 8 MFMAs of `cur`, after each of them one fragment read of slice kk_next into `nxt` and,
-  // when n_loads == 4, after every second one a load (first_load ..) of the next stage
-  auto slice = [&](Frags& cur, Frags& nxt, const char* a_rd, const char* b_rd, int kk_next, int first_load, int n_loads,
-                   char* a_wr, char* b_wr, int kt_next, bool more) {
+  constexpr int NM    = TM * TN;            // MFMAs of a slice
+  constexpr int HALF  = (LPA + LPB) / 2;    // loads issued in each of the two slices after the barrier
+  constexpr int EVERY = NM / HALF;          // one load after every EVERY-th MFMA
+  static_assert(NM % HALF == 0 && NM >= TM + TN, "the slice schedule needs a slot per fragment read and load");
+  // one 16-deep slice: the MFMAs of `cur`, after each of them one fragment read of slice kk_next into `nxt`
+  // (a0, b0, a1, b1, ... in the order the next slice uses them) and, when with_loads, after every EVERY-th one a
+  // load (first_load ..) of the next stage
+  auto slice = [&](Frags& cur, Frags& nxt, const char* a_rd, const char* b_rd, int kk_next, int first_load,
+                   bool with_loads, char* a_wr, char* b_wr, int kt_next, bool more) {
 #pragma unroll
-    for (int m = 0; m < 8; ++m) {
+    for (int m = 0; m < NM; ++m) {
       CINN_SB;
-      acc[m >> 1][m & 1] = Half16<T>::mfma(cur.a[m >> 1], cur.b[m & 1], acc[m >> 1][m & 1]);
+      acc[m / TN][m % TN] = Half16<T>::mfma(cur.a[m / TN], cur.b[m % TN], acc[m / TN][m % TN]);
       CINN_SB;
-      switch (m) {
-        case 0: read_a(a_rd, kk_next, 0, nxt); break;
-        case 1: read_b(b_rd, kk_next, 0, nxt); break;
-        case 2: read_a(a_rd, kk_next, 1, nxt); break;
-        case 3: read_b(b_rd, kk_next, 1, nxt); break;
-        case 4: read_a(a_rd, kk_next, 2, nxt); break;
-        case 5: read_a(a_rd, kk_next, 3, nxt); break;
-        default: break;
+      // read m of the list a0, b0, a1, b1, ..., then the rest of the longer operand
+      constexpr int PAIRS = TM < TN ? TM : TN;
+      if (m < 2 * PAIRS) {
+        if (m % 2 == 0) {
+          read_a(a_rd, kk_next, m / 2, nxt);
+        } else {
+          read_b(b_rd, kk_next, m / 2, nxt);
+        }
+      } else if (m < TM + TN) {
+        if (TM > TN) {
+          read_a(a_rd, kk_next, m - PAIRS, nxt);
+        } else {
+          read_b(b_rd, kk_next, m - PAIRS, nxt);
+        }
       }
-      if (n_loads == 4 && (m & 1) == 1) {
+      if (with_loads && m % EVERY == EVERY - 1) {
         CINN_SB;
-        if (more) issue_one(a_wr, b_wr, kt_next, first_load + (m >> 1));
+        if (more) issue_one(a_wr, b_wr, kt_next, first_load + m / EVERY);
       }
     }
     CINN_SB;
@@ -378,15 +406,15 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   const int nk = K / kD64BK;  // even
   Frags f0, f1;
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int e = 0; e < 8; ++e) f0.a[i][e] = 0;
 #pragma unroll
-  for (int j = 0; j < 2; ++j)
+  for (int j = 0; j < TN; ++j)
 #pragma unroll
     for (int e = 0; e < 8; ++e) f0.b[j][e] = 0;
 #pragma unroll
-  for (int t = 0; t < 8; ++t) issue_one(sa0, sb0, 0, t);
+  for (int t = 0; t < LPA + LPB; ++t) issue_one(sa0, sb0, 0, t);
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   __syncthreads();
   // f0 holds the last slice of the previous stage (zeros before the first)
@@ -394,10 +422,10 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   {                                                                                                          \
     const int s     = kt + OFF;                                                                              \
     const bool more = s + 1 < nk;                                                                            \
-    slice(f0, f1, ACUR, BCUR, 0, 0, 4, ANXT, BNXT, s + 1, more);                                             \
-    slice(f1, f0, ACUR, BCUR, 1, 4, 4, ANXT, BNXT, s + 1, more);                                             \
-    slice(f0, f1, ACUR, BCUR, 2, 0, 0, ANXT, BNXT, s + 1, more);                                             \
-    slice(f1, f0, ACUR, BCUR, 3, 0, 0, ANXT, BNXT, s + 1, more);                                             \
+    slice(f0, f1, ACUR, BCUR, 0, 0, true, ANXT, BNXT, s + 1, more);                                          \
+    slice(f1, f0, ACUR, BCUR, 1, HALF, true, ANXT, BNXT, s + 1, more);                                       \
+    slice(f0, f1, ACUR, BCUR, 2, 0, false, ANXT, BNXT, s + 1, more);                                         \
+    slice(f1, f0, ACUR, BCUR, 3, 0, false, ANXT, BNXT, s + 1, more);                                         \
     __builtin_amdgcn_s_waitcnt(0x0070); /* vmcnt(0) lgkmcnt(0): stage s+1 landed, fragments in registers */  \
     __syncthreads();                                                                                         \
   }
@@ -408,35 +436,40 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 #undef CINN_GEMM_STEP
   // the last slice of the last stage
 #pragma unroll
-  for (int m = 0; m < 8; ++m) acc[m >> 1][m & 1] = Half16<T>::mfma(f0.a[m >> 1], f0.b[m & 1], acc[m >> 1][m & 1]);
+  for (int m = 0; m < NM; ++m) acc[m / TN][m % TN] = Half16<T>::mfma(f0.a[m / TN], f0.b[m % TN], acc[m / TN][m % TN]);
 #undef CINN_SB
 
   T* Ct = reinterpret_cast<T*>(C);
   if (beta == 0.0f) {
-    // Through LDS, half of the tile's rows at a time (the 32-row blocks i = 2 pass, 2 pass + 1 of every wavefront):
-    // accumulators are written as 16-bit values into [128 rows][256 + 8 columns], then every lane moves 16 bytes and
-    // a store instruction covers two whole 512-byte rows of C instead of 64 two-byte pieces.
-    constexpr int kRowBytes = (kBN + 8) * 2;
+    // Through LDS, two 32-row blocks of every wavefront at a time (i = 2 pass, 2 pass + 1): accumulators are written
+    // as 16-bit values into [64 WAVES_M rows][BN + 8 columns], then every lane moves 16 bytes and a store
+    // instruction covers whole rows of the C tile instead of 64 two-byte pieces.
+    constexpr int kRowBytes = (BN + 8) * 2;
+    constexpr int IB        = TM < 2 ? TM : 2;        // 32-row blocks per wavefront and pass
+    constexpr int PASS_ROWS = WAVES_M * IB * 32;
+    constexpr int CPR       = BN / 8;                 // 16-byte chunks per row
+    static_assert(PASS_ROWS * kRowBytes <= 2 * (A_TILE + B_TILE), "the staged result does not fit the operand stages");
+    static_assert(PASS_ROWS * CPR % THREADS == 0, "the copy-out loop assumes whole rounds");
 #pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
+    for (int pass = 0; pass < TM / IB; ++pass) {
       __syncthreads();  // the last stage (or the previous pass) has been read
 #pragma unroll
-      for (int ii = 0; ii < 2; ++ii)
+      for (int ii = 0; ii < IB; ++ii)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const int lrow = wm * 64 + ii * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            const int col  = wn * 64 + j * 32 + (lane & 31);
-            *reinterpret_cast<T*>(lds + lrow * kRowBytes + col * 2) = (T)(alpha * acc[2 * pass + ii][j][r]);
+            const int lrow = wm * (IB * 32) + ii * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            const int col  = wn * (TN * 32) + j * 32 + (lane & 31);
+            *reinterpret_cast<T*>(lds + lrow * kRowBytes + col * 2) = (T)(alpha * acc[IB * pass + ii][j][r]);
           }
       __syncthreads();
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int chunk = e * kDmaThreads + tid;  // 128 rows x 32 chunks of 16 bytes
-        const int lrow  = chunk >> 5;
-        const int c16   = chunk & 31;
-        const int row   = m0 + (lrow >> 6) * 128 + pass * 64 + (lrow & 63);
+      for (int e = 0; e < PASS_ROWS * CPR / THREADS; ++e) {
+        const int chunk = e * THREADS + tid;
+        const int lrow  = chunk / CPR;
+        const int c16   = chunk % CPR;
+        const int row   = m0 + (lrow / (IB * 32)) * (TM * 32) + pass * (IB * 32) + lrow % (IB * 32);
         const u32x4 v   = *reinterpret_cast<const u32x4*>(lds + lrow * kRowBytes + c16 * 16);
         *reinterpret_cast<u32x4*>(Ct + (int64_t)row * ldc + n0 + c16 * 8) = v;
       }
@@ -444,13 +477,13 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     return;
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int col = n0 + wn * 64 + j * 32 + (lane & 31);
+    for (int j = 0; j < TN; ++j) {
+      const int col = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int row = m0 + wm * 128 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        const int row = m0 + wm * (TM * 32) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         T* dst  = Ct + (int64_t)row * ldc + col;
         float v = alpha * acc[i][j][r];
         if (beta != 0.0f) v += beta * (float)*dst;
@@ -770,16 +803,54 @@ void XcdRectangles(int tiles_m, int tiles_n, int* xcd_cols, int* sub_rows, int* 
   }
 }
 
-template <typename T, bool B_KC>
+template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N>
 void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
   int64_t ldb = p.trans_b ? p.k : p.n;
-  const int tiles_m = p.m / kBM, tiles_n = p.n / kBN;
+  const int tiles_m = p.m / BM, tiles_n = p.n / BN;
   dim3 grid(tiles_m * tiles_n, p.batch, 1);
   int xcd_cols = 0, sub_rows = 0, sub_cols = 0;
   XcdRectangles(tiles_m, tiles_n, &xcd_cols, &sub_rows, &sub_cols);
-  hipLaunchKernelGGL((gemm16_dma_kernel<T, B_KC>), grid, dim3(kDmaThreads), 0, stream, static_cast<const uint16_t*>(p.a),
-                     static_cast<const uint16_t*>(p.b), static_cast<uint16_t*>(p.c), p.m, p.n, p.k, (int64_t)p.k, ldb,
-                     (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c, xcd_cols, sub_rows, sub_cols);
+  hipLaunchKernelGGL((gemm16_dma_kernel<T, B_KC, BM, BN, WAVES_M, WAVES_N>), grid, dim3(64 * WAVES_M * WAVES_N), 0,
+                     stream, static_cast<const uint16_t*>(p.a), static_cast<const uint16_t*>(p.b),
+                     static_cast<uint16_t*>(p.c), p.m, p.n, p.k, (int64_t)p.k, ldb, (int64_t)p.n, p.alpha, p.beta,
+                     p.stride_a, p.stride_b, p.stride_c, xcd_cols, sub_rows, sub_cols);
+}
+
+// A stored [M][K], K % 128 == 0: 256x256 tiles when they fill the chip, else 128x128 tiles when M and N allow them
+// and there are enough of those; false when neither applies
+template <typename T>
+bool TryDma16(const GemmProblem& p, hipStream_t stream) {
+  if (p.trans_a || p.k % 128 != 0) return false;
+  const bool fit256 = p.m % 256 == 0 && p.n % 256 == 0;
+  const bool fit128 = p.m % 128 == 0 && p.n % 128 == 0;
+  const int64_t tiles256 = fit256 ? (int64_t)(p.m / 256) * (p.n / 256) * p.batch : 0;
+  const int64_t tiles128 = fit128 ? (int64_t)(p.m / 128) * (p.n / 128) * p.batch : 0;
+  static const int forced = getenv("FLAGS_cinn_hip_gemm_tile") ? atoi(getenv("FLAGS_cinn_hip_gemm_tile")) : 0;
+  if (tiles256 >= 192 && forced != 128) {
+    if (p.trans_b) {
+      LaunchDma16<T, true, 256, 256, 2, 4>(p, stream);
+    } else {
+      LaunchDma16<T, false, 256, 256, 2, 4>(p, stream);
+    }
+    return true;
+  }
+  if ((tiles128 >= 128 && forced != 256) || (forced == 128 && tiles128 > 0)) {
+    if (p.trans_b) {
+      LaunchDma16<T, true, 128, 128, 2, 2>(p, stream);
+    } else {
+      LaunchDma16<T, false, 128, 128, 2, 2>(p, stream);
+    }
+    return true;
+  }
+  if (tiles256 >= 64) {
+    if (p.trans_b) {
+      LaunchDma16<T, true, 256, 256, 2, 4>(p, stream);
+    } else {
+      LaunchDma16<T, false, 256, 256, 2, 4>(p, stream);
+    }
+    return true;
+  }
+  return false;
 }
 
 bool UseRegisterStaging() {
@@ -787,17 +858,10 @@ bool UseRegisterStaging() {
   return on;
 }
 
+// 256x256 tiles with register staging: every operand layout (used for A stored [K][M])
 template <typename T>
 void DispatchFast16(const GemmProblem& p, hipStream_t stream) {
   bool a_kc = !p.trans_a, b_kc = p.trans_b;
-  if (a_kc && p.k % 128 == 0 && !UseRegisterStaging()) {
-    if (b_kc) {
-      LaunchDma16<T, true>(p, stream);
-    } else {
-      LaunchDma16<T, false>(p, stream);
-    }
-    return;
-  }
   if (a_kc && b_kc) LaunchFast16<T, true, true>(p, stream);
   if (a_kc && !b_kc) LaunchFast16<T, true, false>(p, stream);
   if (!a_kc && b_kc) LaunchFast16<T, false, true>(p, stream);
@@ -859,6 +923,13 @@ void RunGemm(const GemmProblem& p, hipStream_t stream) {
   const bool aligned16 = reinterpret_cast<uintptr_t>(p.a) % 16 == 0 && reinterpret_cast<uintptr_t>(p.b) % 16 == 0 &&
                          p.stride_a % 4 == 0 && p.stride_b % 4 == 0;
   const bool fast32 = !ForceGeneric() && p.m % kF32Tile == 0 && p.n % kF32Tile == 0 && p.k % kF32K == 0 && aligned16;
+  if (!ForceGeneric() && !UseRegisterStaging() && (p.type == GemmType::kBF16 || p.type == GemmType::kF16)) {
+    const bool taken = p.type == GemmType::kBF16 ? TryDma16<__bf16>(p, stream) : TryDma16<_Float16>(p, stream);
+    if (taken) {
+      CINN_HIP_CALL(hipGetLastError());
+      return;
+    }
+  }
   // Shapes the big-tile kernels do not take (ragged, or so few tiles that most CUs would idle) go to the
   // channels-last convolution kernels: a 1x1 convolution over m "pixels" is this GEMM with both operands
   // K-contiguous (A [m,k], B stored [n,k]); those kernels bound-check every tile edge, use 64x64 tiles and split K

@@ -110,10 +110,12 @@ def test_16bit_mfma_path_all_layouts(gpu, kind, ta, tb):
 @pytest.mark.parametrize("kind", ["float16", "bfloat16"])
 @pytest.mark.parametrize("tb", [False, True])
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (0.5, 2.0)])
-def test_16bit_direct_to_lds_kernel(gpu, kind, tb, alpha, beta):
-    """Shapes the 256x256x64 kernel takes (A stored [M][K], M, N % 256 == 0, K % 128 == 0): both layouts of B, two
-    batches with B broadcast, the staged epilogue (beta == 0) and the read-modify-write one."""
-    batch, m, n, k = 2, 512, 256, 384
+@pytest.mark.parametrize("batch,m,n,k", [(1, 4096, 3072, 128),   # 192 tiles of 256x256: the 8-wavefront kernel
+                                         (1, 1536, 1536, 256),   # 144 tiles of 128x128: the 4-wavefront kernel
+                                         (2, 1024, 1024, 384)])  # the same with two batches and B broadcast
+def test_16bit_direct_to_lds_kernel(gpu, kind, tb, alpha, beta, batch, m, n, k):
+    """Shapes the direct-to-LDS kernels take (A stored [M][K], K % 128 == 0, enough 256x256 or 128x128 tiles): both
+    layouts of B, the staged epilogue (beta == 0) and the read-modify-write one."""
     rng = np.random.default_rng(41)
     a = (rng.standard_normal((batch, m, k)) * 0.05).astype(np.float32)
     b = (rng.standard_normal((1, n, k) if tb else (1, k, n)) * 0.05).astype(np.float32)
