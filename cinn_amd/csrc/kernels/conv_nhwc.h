@@ -30,6 +30,10 @@ struct ConvNhwcArgs {
 bool ConvNhwcSupported(const ConvNhwcArgs& a);
 void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream);
 
+// 1x1, stride 1, unpadded 16-bit convolutions whose shape the direct-to-LDS GEMM kernels take (gemm_mfma.hip): the
+// convolution is the GEMM pixels x channels, with this epilogue; false when the shape does not qualify
+bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream);
+
 // NCHW-input convolutions whose filter and input patch fit LDS (conv_stem_mfma.hip): staged instead of gathered
 bool ConvStemSupported(const ConvNhwcArgs& a);
 void RunConvStem(const ConvNhwcArgs& a, hipStream_t stream);

@@ -611,6 +611,7 @@ void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream) {
     RunConvStem(a, stream);
     return;
   }
+  if (TryPointwiseConvAsGemm(a, stream)) return;
   Params p;
   p.n = a.n, p.h = a.h, p.w = a.w_in, p.c = a.c;
   p.oc = a.oc, p.kh = a.kh, p.kw = a.kw;

@@ -3,7 +3,7 @@
 //   C[M,N] = alpha * op(A)[M,K] * op(B)[K,N] + beta * C          (row-major, optional batch)
 //
 // Kernels:
-//   * gemm16_dma_kernel   - bf16 / fp16 with A stored [M][K] (the common case) and K % 128 == 0: 256x256x64 tile, 512
+//   * gemm16_dma_kernel   - bf16 / fp16 with A stored [M][K] (the common case) and K % 64 == 0: 256x256x64 tile, 512
 //     threads, direct global -> LDS loads of whole 128-byte lines into two stages, transposing LDS reads for
 //     row-major B; see the comment at the kernel.
 //   * gemm16_mfma_kernel  - bf16 / fp16 inputs, any operand layout (used for transposed A), fp32 accumulation on v_mfma_f32_32x32x16_{bf16,f16}.
@@ -237,7 +237,7 @@ gemm16_mfma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ 
 // In core clocks the main loop keeps the MFMA pipe 84 % busy (156 k clocks for 131 k of MFMA at 4096^3); what the
 // kernel delivers beyond that is set by the clock the chip sustains under this load (1.2-1.6 GHz measured inside
 // the loop against the 2.4 GHz of the quoted peak).
-// Requires M % 256 == N % 256 == K % 128 == 0.
+// Requires M % BM == N % BN == K % 64 == 0.
 // ---------------------------------------------------------------------------------------------------
 constexpr int kDmaThreads = 512;
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -254,13 +254,23 @@ __device__ __forceinline__ void AsyncCopy16(const void* src, char* lds_base_unif
 constexpr int kD64BK   = 64;
 constexpr int kD64Tile = kBM * kD64BK * 2;  // one operand tile of a stage: 32 KiB
 
+// epilogue operands of gemm16_dma_kernel: v = acc * (scale[col] or alpha) + shift[col] + residual_scale * R, relu
+struct DmaEpilogue {
+  const float* scale;     // per output column, or null: alpha
+  const float* shift;     // per output column, or null
+  const void* residual;   // [M][N] like C (may be C itself: the beta term of a GEMM), or null
+  float alpha;
+  float residual_scale;
+  int relu;
+};
+
 // BM x BN block tile on a WAVES_M x WAVES_N grid of wavefronts: 256x256 on 2x4 (8 wavefronts of 128x64) for large
 // problems, 128x128 on 2x2 (4 wavefronts of 64x64, two blocks per CU) when 256x256 tiles would leave CUs idle.
 template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N>
 __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N)
-gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ C, int M, int N,
-                    int K, int64_t lda, int64_t ldb, int64_t ldc, float alpha, float beta, int64_t stride_a,
-                    int64_t stride_b, int64_t stride_c, int xcd_cols, int sub_rows, int sub_cols) {
+gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* C, int M, int N, int K,
+                  int64_t lda, int64_t ldb, int64_t ldc, DmaEpilogue epi, int64_t stride_a, int64_t stride_b,
+                  int64_t stride_c, int xcd_cols, int sub_rows, int sub_cols) {
   constexpr int NW      = WAVES_M * WAVES_N;
   constexpr int THREADS = 64 * NW;
   constexpr int TM      = BM / WAVES_M / 32;  // MFMA tiles per wavefront along M and N
@@ -403,7 +413,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     CINN_SB;
   };
 
-  const int nk = K / kD64BK;  // even
+  const int nk = K / kD64BK;
   Frags f0, f1;
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -431,7 +441,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   }
   for (int kt = 0; kt < nk; kt += 2) {
     CINN_GEMM_STEP(sa0, sb0, sa1, sb1, 0)
-    CINN_GEMM_STEP(sa1, sb1, sa0, sb0, 1)
+    if (kt + 1 < nk) CINN_GEMM_STEP(sa1, sb1, sa0, sb0, 1)
   }
 #undef CINN_GEMM_STEP
   // the last slice of the last stage
@@ -439,15 +449,25 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   for (int m = 0; m < NM; ++m) acc[m / TN][m % TN] = Half16<T>::mfma(f0.a[m / TN], f0.b[m % TN], acc[m / TN][m % TN]);
 #undef CINN_SB
 
-  T* Ct = reinterpret_cast<T*>(C);
-  if (beta == 0.0f) {
-    // Through LDS, two 32-row blocks of every wavefront at a time (i = 2 pass, 2 pass + 1): accumulators are written
-    // as 16-bit values into [64 WAVES_M rows][BN + 8 columns], then every lane moves 16 bytes and a store
-    // instruction covers whole rows of the C tile instead of 64 two-byte pieces.
+  // Epilogue on the fp32 accumulators: v = acc * (scale[col] or alpha) + shift[col] + residual_scale * R[row][col],
+  // optional relu, one rounding to T.  The tile goes through LDS so that every lane moves 16 bytes and a store
+  // instruction covers whole rows of the C tile instead of 64 two-byte pieces: as 16-bit values, two 32-row blocks of
+  // every wavefront per pass, or - with a residual, which is added before the rounding - as fp32, one block per pass.
+  T* Ct       = reinterpret_cast<T*>(C);
+  const T* Rt = reinterpret_cast<const T*>(epi.residual);
+  if (Rt) Rt += (int64_t)blockIdx.y * stride_c;
+  float sc[TN], sh[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int col = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
+    sc[j]         = epi.scale ? epi.scale[col] : epi.alpha;
+    sh[j]         = epi.shift ? epi.shift[col] : 0.0f;
+  }
+  constexpr int CPR = BN / 8;  // 8-column chunks per row
+  if (!Rt) {
     constexpr int kRowBytes = (BN + 8) * 2;
-    constexpr int IB        = TM < 2 ? TM : 2;        // 32-row blocks per wavefront and pass
+    constexpr int IB        = TM < 2 ? TM : 2;  // 32-row blocks per wavefront and pass
     constexpr int PASS_ROWS = WAVES_M * IB * 32;
-    constexpr int CPR       = BN / 8;                 // 16-byte chunks per row
     static_assert(PASS_ROWS * kRowBytes <= 2 * (A_TILE + B_TILE), "the staged result does not fit the operand stages");
     static_assert(PASS_ROWS * CPR % THREADS == 0, "the copy-out loop assumes whole rounds");
 #pragma unroll
@@ -461,7 +481,9 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
           for (int r = 0; r < 16; ++r) {
             const int lrow = wm * (IB * 32) + ii * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
             const int col  = wn * (TN * 32) + j * 32 + (lane & 31);
-            *reinterpret_cast<T*>(lds + lrow * kRowBytes + col * 2) = (T)(alpha * acc[IB * pass + ii][j][r]);
+            float v        = acc[IB * pass + ii][j][r] * sc[j] + sh[j];
+            if (epi.relu) v = v > 0.0f ? v : 0.0f;
+            *reinterpret_cast<T*>(lds + lrow * kRowBytes + col * 2) = (T)v;
           }
       __syncthreads();
 #pragma unroll
@@ -476,20 +498,43 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     }
     return;
   }
+  constexpr int kRowFloats = BN + 4;
+  constexpr int PASS_ROWS  = WAVES_M * 32;
+  static_assert(PASS_ROWS * kRowFloats * 4 <= 2 * (A_TILE + B_TILE), "the staged result does not fit the operand stages");
+  static_assert(PASS_ROWS * CPR % THREADS == 0, "the copy-out loop assumes whole rounds");
+  float* stage = reinterpret_cast<float*>(lds);
 #pragma unroll
-  for (int i = 0; i < TM; ++i)
+  for (int pass = 0; pass < TM; ++pass) {
+    __syncthreads();
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int col = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int row = m0 + wm * (TM * 32) + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        T* dst  = Ct + (int64_t)row * ldc + col;
-        float v = alpha * acc[i][j][r];
-        if (beta != 0.0f) v += beta * (float)*dst;
-        *dst = (T)v;
+        const int lrow = wm * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        const int col  = wn * (TN * 32) + j * 32 + (lane & 31);
+        stage[lrow * kRowFloats + col] = acc[pass][j][r] * sc[j] + sh[j];
       }
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < PASS_ROWS * CPR / THREADS; ++e) {
+      const int chunk = e * THREADS + tid;
+      const int lrow  = chunk / CPR;
+      const int c8    = chunk % CPR;
+      const int row   = m0 + (lrow / 32) * (TM * 32) + pass * 32 + lrow % 32;
+      const int64_t o = (int64_t)row * ldc + n0 + c8 * 8;
+      const f32x4 lo  = *reinterpret_cast<const f32x4*>(stage + lrow * kRowFloats + c8 * 8);
+      const f32x4 hi  = *reinterpret_cast<const f32x4*>(stage + lrow * kRowFloats + c8 * 8 + 4);
+      const vec8 res  = *reinterpret_cast<const vec8*>(Rt + o);
+      vec8 out;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        float v = (q < 4 ? lo[q] : hi[q - 4]) + epi.residual_scale * (float)res[q];
+        if (epi.relu) v = v > 0.0f ? v : 0.0f;
+        out[q] = (T)v;
+      }
+      *reinterpret_cast<vec8*>(Ct + o) = out;
     }
+  }
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -769,6 +814,12 @@ struct GemmProblem {
   float alpha, beta;
   int batch;
   int64_t stride_a, stride_b, stride_c;  // in elements; 0 broadcasts the operand over the batch
+  // convolution epilogue (direct-to-LDS kernels only): per-column scale / shift, residual of C's shape, relu
+  const float* scale{nullptr};
+  const float* shift{nullptr};
+  const void* residual{nullptr};
+  float residual_scale{0.0f};
+  bool relu{false};
 };
 
 template <typename T, bool A_KC, bool B_KC>
@@ -810,17 +861,24 @@ void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
   dim3 grid(tiles_m * tiles_n, p.batch, 1);
   int xcd_cols = 0, sub_rows = 0, sub_cols = 0;
   XcdRectangles(tiles_m, tiles_n, &xcd_cols, &sub_rows, &sub_cols);
+  DmaEpilogue epi;
+  epi.scale          = p.scale;
+  epi.shift          = p.shift;
+  epi.alpha          = p.alpha;
+  epi.relu           = p.relu ? 1 : 0;
+  epi.residual       = p.residual ? p.residual : (p.beta != 0.0f ? p.c : nullptr);
+  epi.residual_scale = p.residual ? p.residual_scale : p.beta;
   hipLaunchKernelGGL((gemm16_dma_kernel<T, B_KC, BM, BN, WAVES_M, WAVES_N>), grid, dim3(64 * WAVES_M * WAVES_N), 0,
                      stream, static_cast<const uint16_t*>(p.a), static_cast<const uint16_t*>(p.b),
-                     static_cast<uint16_t*>(p.c), p.m, p.n, p.k, (int64_t)p.k, ldb, (int64_t)p.n, p.alpha, p.beta,
-                     p.stride_a, p.stride_b, p.stride_c, xcd_cols, sub_rows, sub_cols);
+                     static_cast<uint16_t*>(p.c), p.m, p.n, p.k, (int64_t)p.k, ldb, (int64_t)p.n, epi, p.stride_a,
+                     p.stride_b, p.stride_c, xcd_cols, sub_rows, sub_cols);
 }
 
-// A stored [M][K], K % 128 == 0: 256x256 tiles when they fill the chip, else 128x128 tiles when M and N allow them
+// A stored [M][K], K % 64 == 0: 256x256 tiles when they fill the chip, else 128x128 tiles when M and N allow them
 // and there are enough of those; false when neither applies
 template <typename T>
 bool TryDma16(const GemmProblem& p, hipStream_t stream) {
-  if (p.trans_a || p.k % 128 != 0) return false;
+  if (p.trans_a || p.k % 64 != 0) return false;
   const bool fit256 = p.m % 256 == 0 && p.n % 256 == 0;
   const bool fit128 = p.m % 128 == 0 && p.n % 128 == 0;
   const int64_t tiles256 = fit256 ? (int64_t)(p.m / 256) * (p.n / 256) * p.batch : 0;
@@ -1029,6 +1087,50 @@ cinn_buffer_t* BufferArg(void* v_args, int index) {
 }
 
 }  // namespace
+
+namespace cinn_hip_kernels {
+
+bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream) {
+  static const bool enabled = !(getenv("FLAGS_cinn_hip_conv_pointwise_gemm") && atoi(getenv("FLAGS_cinn_hip_conv_pointwise_gemm")) == 0);
+  if (!enabled || ForceGeneric() || UseRegisterStaging()) return false;
+  const bool is_f16  = a.type.code == cinn_type_float && a.type.bits == 16;
+  const bool is_bf16 = a.type.code == cinn_type_bfloat && a.type.bits == 16;
+  if (!is_f16 && !is_bf16) return false;
+  if (a.nchw_input || a.kh != 1 || a.kw != 1 || a.stride_h != 1 || a.stride_w != 1 || a.pad_h != 0 || a.pad_w != 0) return false;
+  if (a.oh != a.h || a.ow != a.w_in) return false;
+  const int64_t pixels = (int64_t)a.n * a.oh * a.ow;
+  if (pixels >= INT_MAX) return false;
+  // measured inside ResNet-50 at batch 32: the GEMM kernels win only with at least one 128x128 tile per CU and a K
+  // loop of two steps or more; smaller grids are better served by the 64x64 tiles and split K of the convolution kernel
+  if (a.c < 128 || (pixels / 128) * (a.oc / 128) < 256) return false;
+  if (reinterpret_cast<uintptr_t>(a.x) % 16 != 0 || reinterpret_cast<uintptr_t>(a.w) % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(a.y) % 16 != 0 || reinterpret_cast<uintptr_t>(a.residual) % 16 != 0)
+    return false;
+  GemmProblem p;
+  p.type    = is_bf16 ? GemmType::kBF16 : GemmType::kF16;
+  p.a       = a.x;  // [pixels][c]
+  p.b       = a.w;  // [oc][c]
+  p.c       = a.y;
+  p.m       = static_cast<int>(pixels);
+  p.n       = a.oc;
+  p.k       = a.c;
+  p.trans_a = false;
+  p.trans_b = true;
+  p.alpha   = a.alpha;
+  p.beta    = 0.0f;
+  p.batch   = 1;
+  p.stride_a = p.stride_b = p.stride_c = 0;
+  p.scale          = a.scale;
+  p.shift          = a.shift;
+  p.residual       = a.residual;
+  p.residual_scale = a.residual_scale;
+  p.relu           = a.relu;
+  const bool taken = is_bf16 ? TryDma16<__bf16>(p, stream) : TryDma16<_Float16>(p, stream);
+  if (taken) CINN_HIP_CALL(hipGetLastError());
+  return taken;
+}
+
+}  // namespace cinn_hip_kernels
 
 extern "C" {
 

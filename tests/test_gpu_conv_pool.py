@@ -341,3 +341,23 @@ def test_conv2d_channels_last_alpha_beta(gpu):
     for fmt in (1, 2):
         got = call_conv_nhwc(x, w, 1, 1, fmt, "float32", alpha=0.5, beta=2.0, y_init=y0)
         np.testing.assert_allclose(got, 0.5 * oracle.conv2d_nchw(x, w, (1, 1), (1, 1)) + 2.0 * y0, rtol=1e-5, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype,tol", [("float16", 2.0 ** -10), ("bfloat16", 2.0 ** -7)])
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (0.5, 2.0)])
+def test_pointwise_convolution_on_the_gemm_kernel(gpu, dtype, tol, alpha, beta):
+    """1x1, stride 1, unpadded, 8192 pixels x 512 channels = 256 tiles of 128x128 and K = 128: the channels-last entry
+    point hands this shape to the direct-to-LDS GEMM kernel (the beta term goes through its fp32-staged epilogue).
+    A 1x1 convolution is a matrix product over the channels, which the oracle confirms on one image."""
+    n, ic, h, w_, oc = 8, 128, 32, 32, 512
+    rng = np.random.default_rng(53)
+    x = round_to(rng.standard_normal((n, ic, h, w_)), dtype)
+    w = round_to(rng.standard_normal((oc, ic, 1, 1)) * np.sqrt(2.0 / ic), dtype)
+    y0 = round_to(rng.standard_normal((n, oc, h, w_)), dtype)
+    got = call_conv_nhwc(x, w, 1, 0, 1, dtype, alpha=alpha, beta=beta, y_init=y0).astype(np.float64)
+    w2 = w[:, :, 0, 0].astype(np.float64)
+    conv = np.einsum("oc,nchw->nohw", w2, x.astype(np.float64))
+    np.testing.assert_allclose(conv[:1], oracle.conv2d_nchw(x[:1], w, (1, 1), (0, 0)), rtol=1e-4, atol=1e-4)
+    want = alpha * conv + beta * y0
+    scale = alpha * np.einsum("oc,nchw->nohw", np.abs(w2), np.abs(x).astype(np.float64)) + beta * np.abs(y0)
+    assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-3 * scale) + 2.0 ** -24)
