@@ -24,6 +24,8 @@
 #include <cstdint>
 #include <cstdlib>
 #include <cstring>
+#include <map>
+#include <mutex>
 
 #include "kernels/conv_nhwc.h"
 #include "runtime/hip_check.h"
@@ -491,20 +493,26 @@ const void* ZeroPage() {
   return page;
 }
 
-// fp32 scratch for split-K partial sums; grown on demand and kept (the first, eager execution of a program sizes it, so
-// graph capture never sees an allocation)
-float* Workspace(size_t bytes) {
-  static float* buffer   = nullptr;
-  static size_t capacity = 0;
-  if (bytes > capacity) {
-    if (buffer) {
+// fp32 scratch for split-K partial sums, one buffer per stream (launches on different streams may overlap); grown on
+// demand and kept (the first, eager execution of a program sizes it, so graph capture never sees an allocation)
+float* Workspace(size_t bytes, hipStream_t stream) {
+  struct Buffer {
+    float* data{nullptr};
+    size_t capacity{0};
+  };
+  static std::mutex mu;
+  static std::map<hipStream_t, Buffer> buffers;
+  std::lock_guard<std::mutex> lock(mu);
+  Buffer& b = buffers[stream];
+  if (bytes > b.capacity) {
+    if (b.data) {
       CINN_HIP_CALL(hipDeviceSynchronize());
-      CINN_HIP_CALL(hipFree(buffer));
+      CINN_HIP_CALL(hipFree(b.data));
     }
-    CINN_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&buffer), bytes));
-    capacity = bytes;
+    CINN_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&b.data), bytes));
+    b.capacity = bytes;
   }
-  return buffer;
+  return b.data;
 }
 
 // K splits: layers whose tile grid cannot fill the 256 CUs spend their time waiting for one block's serial chain of
@@ -540,7 +548,7 @@ void Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream) {
   p.steps_per_split     = (steps + p.splits - 1) / p.splits;
   p.splits              = (steps + p.steps_per_split - 1) / p.steps_per_split;
   float* workspace      = nullptr;
-  if (p.splits > 1) workspace = Workspace((size_t)p.splits * p.pixels * p.oc * sizeof(float));
+  if (p.splits > 1) workspace = Workspace((size_t)p.splits * p.pixels * p.oc * sizeof(float), stream);
   hipLaunchKernelGGL(kernel, dim3(tiles, p.splits), dim3(64 * WM * WN), bytes, stream, static_cast<const T*>(a.x),
                      static_cast<const T*>(a.w), static_cast<T*>(a.y), a.scale, a.shift, static_cast<const T*>(a.residual),
                      workspace, ZeroPage(), p);

@@ -23,6 +23,8 @@
 
 #include <climits>
 #include <cstdint>
+#include <map>
+#include <mutex>
 
 #include "cinn_hip_runtime.h"
 #include "kernels/conv_nhwc.h"
@@ -771,20 +773,25 @@ transpose2d_kernel(const T* __restrict__ in, T* __restrict__ out, int rows, int 
   }
 }
 
-// scratch for transposed operands; grown on demand and kept.  One buffer per process: GEMMs that take this path on
-// different streams at the same time would share it.
-char* TransposeWorkspace(size_t bytes) {
-  static char* buffer    = nullptr;
-  static size_t capacity = 0;
-  if (bytes > capacity) {
-    if (buffer) {
+// scratch for transposed operands, one buffer per stream; grown on demand and kept
+char* TransposeWorkspace(size_t bytes, hipStream_t stream) {
+  struct Buffer {
+    char* data{nullptr};
+    size_t capacity{0};
+  };
+  static std::mutex mu;
+  static std::map<hipStream_t, Buffer> buffers;
+  std::lock_guard<std::mutex> lock(mu);
+  Buffer& b = buffers[stream];
+  if (bytes > b.capacity) {
+    if (b.data) {
       CINN_HIP_CALL(hipDeviceSynchronize());
-      CINN_HIP_CALL(hipFree(buffer));
+      CINN_HIP_CALL(hipFree(b.data));
     }
-    CINN_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&buffer), bytes));
-    capacity = bytes;
+    CINN_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&b.data), bytes));
+    b.capacity = bytes;
   }
-  return buffer;
+  return b.data;
 }
 
 void LaunchTranspose(const void* in, void* out, int rows, int cols, int batch, int64_t in_stride, int elem_bytes,
@@ -1009,7 +1016,7 @@ void RunGemm(const GemmProblem& p, hipStream_t stream) {
       const int batch_b    = !p.trans_b ? (p.stride_b == 0 ? 1 : p.batch) : 0;
       const size_t bytes_a = (size_t)batch_a * p.m * p.k * elem_bytes;
       const size_t bytes_b = (size_t)batch_b * p.k * p.n * elem_bytes;
-      char* scratch        = TransposeWorkspace(bytes_a + bytes_b);
+      char* scratch        = TransposeWorkspace(bytes_a + bytes_b, stream);
       if (p.trans_a) {  // stored [k][m]
         LaunchTranspose(p.a, scratch, p.k, p.m, batch_a, p.stride_a, elem_bytes, stream);
         a_base   = scratch;
