@@ -130,3 +130,16 @@ def test_rtc_compiles_for_gfx950_without_a_gpu():
     assert image[:4] == b"\x7fELF" and len(image) > 1000
     # same source again is served from the cache and is byte-identical
     assert runtime.rtc_compile(src) == image
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """the measured path has no cross-GPU work: bench.py --gpus N > 1 exits with a message instead of a number"""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode != 0
+    assert "ONE GPU" in (r.stdout + r.stderr)
+    assert not any(line.startswith("{") for line in r.stdout.splitlines())
