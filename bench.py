@@ -181,6 +181,9 @@ def extra_measurements(stream, runtime):
     out["copy_256MiB"] = dict(us=round(ms * 1e3, 2), GBps=round(2 * 4 * n / ms / 1e6, 1), bytes=2 * 4 * n)
     import bench_gemm  # configs[2]
     out.update(bench_gemm.measure(stream, runtime))
+    import bench_conv  # configs[3]: conv2d + batch_norm + relu layers at batch 32
+    for dtype in ("float16", "float32"):
+        out.update(bench_conv.measure(stream, runtime, dtype))
     import bench_resnet50  # configs[4]: whole-network images/s, HIP-graph replay of the compiled program
     for dtype in ("float16", "float32"):
         r = bench_resnet50.measure(batch=32, dtype=dtype, steps=20, warmup=3)
