@@ -1,9 +1,13 @@
 #include "hlir/graph_compiler.h"
 
+#include <dlfcn.h>
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
+#include <cstdlib>
 #include <cstring>
 
+#include "hlir/accuracy_checker.h"
 #include "optim/optimize.h"
 
 namespace cinn {
@@ -99,10 +103,72 @@ void Instruction::UpdateArgsCache() {
   for (auto& a : out_args_) add(a);
 }
 
+namespace {
+
+// Debug switches of Instruction::Run, read once from the environment like the reference's flags
+// (cinn/runtime/flags.cc): FLAGS_cinn_sync_run waits for every instruction, FLAGS_cinn_self_check_accuracy also
+// reports its tensors (accuracy_checker.h), FLAGS_cinn_profiler_state != 0 brackets every instruction in a roctx
+// range (the reference's RecordEvent / nvtx ranges, cinn/utils/profiler.cc:58-85) that rocprofv3 --marker-trace
+// shows; the marker library is looked up at run time, a missing one disables the ranges.
+struct RunFlags {
+  bool sync_run{false};
+  bool self_check{false};
+  int (*range_push)(const char*){nullptr};
+  int (*range_pop)(){nullptr};
+  RunFlags() {
+    auto on = [](const char* name) {
+      const char* v = getenv(name);
+      return v && *v && std::strcmp(v, "0") != 0 && std::strcmp(v, "false") != 0;
+    };
+    sync_run   = on("FLAGS_cinn_sync_run");
+    self_check = SelfCheckSink::Get().enabled();
+    if (on("FLAGS_cinn_profiler_state")) {
+      void* lib = nullptr;
+      for (const char* name : {"librocprofiler-sdk-roctx.so", "librocprofiler-sdk-roctx.so.1", "libroctx64.so", "libroctx64.so.4"}) {
+        lib = dlopen(name, RTLD_NOW | RTLD_GLOBAL);
+        if (lib) break;
+      }
+      if (lib) {
+        range_push = reinterpret_cast<int (*)(const char*)>(dlsym(lib, "roctxRangePushA"));
+        range_pop  = reinterpret_cast<int (*)()>(dlsym(lib, "roctxRangePop"));
+        if (!range_push || !range_pop) range_push = nullptr, range_pop = nullptr;
+      }
+    }
+  }
+  bool blocking() const { return sync_run || self_check; }
+};
+const RunFlags& Flags() {
+  static const RunFlags flags;
+  return flags;
+}
+
+}  // namespace
+
+bool InstructionsBlockTheStream() { return Flags().blocking(); }
+
 void Instruction::Run(void* stream) {
   CINN_CHECK(fn_) << "instruction " << function_name_ << " has no compiled function";
   if (args_cache_.empty()) UpdateArgsCache();
+  const RunFlags& flags = Flags();
+  if (flags.range_push) flags.range_push(function_name_.c_str());
   fn_(args_cache_.data(), static_cast<int32_t>(args_cache_.size()), stream);
+  if (flags.blocking()) CINN_HIP_STATUS(static_cast<int>(hipStreamSynchronize(static_cast<hipStream_t>(stream))));
+  if (flags.self_check) CheckResults();
+  if (flags.range_pop) flags.range_pop();
+}
+
+// the report of cinn/hlir/framework/instruction.cc:280-330: inputs and outputs in name order
+void Instruction::CheckResults() {
+  SelfCheckSink& sink = SelfCheckSink::Get();
+  std::string text    = "Instruction {\n  Function " + function_name_ + ":\n";
+  auto describe = [&](std::vector<std::string> names, const char* role) {
+    std::sort(names.begin(), names.end());
+    for (auto& n : names) text += std::string("    ") + role + ": " + DescribeTensor(scope_->GetTensor(n), n, sink.print_num()) + "\n";
+  };
+  describe(in_args_, "input");
+  describe(out_args_, "output");
+  text += "}";
+  sink.Write(text);
 }
 
 // ---- Program --------------------------------------------------------------------------------------
@@ -144,6 +210,11 @@ void Program::Execute(void* stream) {
 
 void Program::ExecuteGraph(void* stream) {
   CINN_CHECK(stream) << "graph replay needs an explicit stream";
+  if (InstructionsBlockTheStream()) {
+    // FLAGS_cinn_sync_run / FLAGS_cinn_self_check_accuracy wait after every instruction, which a capture forbids
+    Execute(stream);
+    return;
+  }
   auto s = static_cast<hipStream_t>(stream);
   if (!prerun_done_) RunPreRunInstructions(stream);
   if (!graph_exec_) {

@@ -84,6 +84,7 @@ class Instruction {
 
  private:
   void UpdateArgsCache();
+  void CheckResults();
   common::Target target_;
   Scope* scope_;
   std::vector<std::string> in_args_, out_args_;
@@ -91,6 +92,9 @@ class Instruction {
   lower_func_ptr_g fn_{nullptr};
   std::vector<cinn_pod_value_t> args_cache_;
 };
+
+// true when a debug flag makes every instruction wait for its kernel (no HIP graph capture then)
+bool InstructionsBlockTheStream();
 
 class Program {
  public:

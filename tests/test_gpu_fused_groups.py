@@ -227,3 +227,35 @@ def test_short_row_layer_norm(gpu):
     np.testing.assert_allclose(y, wy, rtol=1e-5, atol=1e-5)
     np.testing.assert_allclose(mean, wm, rtol=1e-5, atol=1e-6)
     np.testing.assert_allclose(var, wv, rtol=1e-5, atol=1e-6)
+
+
+def test_self_check_reports_and_sync_run(gpu, tmp_path):
+    """FLAGS_cinn_self_check_accuracy (a file name) makes every instruction report its tensors with the reference's
+    verdicts (instruction.cc:280-330); the flags are read once per process, hence the child process."""
+    import os
+    import subprocess
+    import sys
+    report = tmp_path / "check.txt"
+    code = """
+import numpy as np, sys
+sys.path.insert(0, %r); sys.path.insert(0, %r)
+from cinn_amd.common import Float
+from cinn_amd.frontend import NetBuilder
+from helpers import run
+b = NetBuilder("chk")
+X = b.create_input(Float(32), [4, 8], "x")
+Y = b.create_input(Float(32), [4, 8], "y")
+x = np.ones((4, 8), np.float32); y = np.full((4, 8), 2.0, np.float32); y[1, 2] = np.nan
+(d, s), comp = run(b, {X: x, Y: y}, [b.divide(X, Y), b.reduce_sum(b.relu(X), [1], False)])
+comp.execute()
+print("done", float(s[0]))
+""" % (os.path.dirname(os.path.dirname(os.path.abspath(__file__))), os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, FLAGS_cinn_self_check_accuracy=str(report), FLAGS_cinn_self_check_accuracy_num="2",
+               FLAGS_cinn_sync_run="1", FLAGS_cinn_profiler_state="1")
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=300)
+    assert r.returncode == 0 and "done 8.0" in r.stdout, r.stdout + r.stderr
+    text = report.read_text()
+    assert "Instruction {" in text and "Function fn_chk" in text
+    assert "input: name=x, dtype=float32, shape={4, 8}, data=[1, 1, ... , 1, 1], One" in text, text
+    assert any("input: name=y" in line and line.rstrip().endswith("NaN") for line in text.splitlines()), text
+    assert any(line.strip().startswith("output:") and line.rstrip().endswith("NaN") for line in text.splitlines()), text
