@@ -30,9 +30,12 @@ struct ConvNhwcArgs {
 bool ConvNhwcSupported(const ConvNhwcArgs& a);
 void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream);
 
-// 1x1, stride 1, unpadded 16-bit convolutions whose shape the direct-to-LDS GEMM kernels take (gemm_mfma.hip): the
-// convolution is the GEMM pixels x channels, with this epilogue; false when the shape does not qualify
+// 16-bit convolutions whose shape the direct-to-LDS GEMM kernels take (gemm_mfma.hip): a 1x1, stride 1, unpadded
+// convolution is the GEMM pixels x channels; any other one with a multiple of 64 input channels runs as an implicit GEMM
+// (K = kh * kw * c); both with this epilogue.  false when the shape does not qualify.
 bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream);
+// 256 bytes of zeros in device memory (what masked-out chunks are read from)
+const void* ConvZeroPage();
 
 // NCHW-input convolutions whose filter and input patch fit LDS (conv_stem_mfma.hip): staged instead of gathered
 bool ConvStemSupported(const ConvNhwcArgs& a);

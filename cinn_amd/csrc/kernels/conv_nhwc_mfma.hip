@@ -603,6 +603,8 @@ void MagicFor(int d, unsigned* magic, unsigned* shift) {
 
 }  // namespace
 
+const void* ConvZeroPage() { return ZeroPage(); }
+
 bool ConvNhwcSupported(const ConvNhwcArgs& a) {
   const bool is_float = a.type.code == cinn_type_float && (a.type.bits == 32 || a.type.bits == 16);
   const bool is_bf16  = a.type.code == cinn_type_bfloat && a.type.bits == 16;

@@ -266,13 +266,25 @@ struct DmaEpilogue {
   int relu;
 };
 
+// Implicit-GEMM view of a channels-last convolution for gemm16_dma_kernel<.., CONV = true>: row m of A is output pixel
+// m = (n, oy, ox), K runs over (dy, dx, c) with c contiguous; a 64-deep K step lies inside one filter tap (the channel
+// count is a multiple of 64), so a load instruction still fetches whole 128-byte lines: 64 channels of one input pixel,
+// or, outside the image, zeros from `zero_page`.
+struct ConvGeom {
+  int h, w, c;          // input extents (NHWC)
+  int oh_ow, ow;        // output plane
+  int kw;               // filter width (dy = tap / kw)
+  int stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
+  const void* zero_page;  // at least 128 bytes of zeros
+};
+
 // BM x BN block tile on a WAVES_M x WAVES_N grid of wavefronts: 256x256 on 2x4 (8 wavefronts of 128x64) for large
 // problems, 128x128 on 2x2 (4 wavefronts of 64x64, two blocks per CU) when 256x256 tiles would leave CUs idle.
-template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N>
+template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false>
 __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N)
 gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* C, int M, int N, int K,
                   int64_t lda, int64_t ldb, int64_t ldc, DmaEpilogue epi, int64_t stride_a, int64_t stride_b,
-                  int64_t stride_c, int xcd_cols, int sub_rows, int sub_cols) {
+                  int64_t stride_c, int xcd_cols, int sub_rows, int sub_cols, ConvGeom geom) {
   constexpr int NW      = WAVES_M * WAVES_N;
   constexpr int THREADS = 64 * NW;
   constexpr int TM      = BM / WAVES_M / 32;  // MFMA tiles per wavefront along M and N
@@ -314,12 +326,40 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   // [row][64 halves] tile, or 512 / BN k-rows of a [k][BN halves] tile.
   const uint16_t* a_src[LPA];
   const uint16_t* b_src[LPB];
+  // CONV: element offset of image n, top-left input coordinates of the pixel's window, and the lane's chunk
+  int a_img[LPA], a_iy0[LPA], a_ix0[LPA], a_chunk[LPA];
 #pragma unroll
   for (int t = 0; t < LPA; ++t) {
     const int row = 8 * (wave * LPA + t) + (lane >> 3);
     const int key = (row ^ (row >> 3)) & 7;
-    a_src[t]      = A + (int64_t)(m0 + row) * lda + (((lane & 7) ^ key) << 3);
+    if (CONV) {
+      const int pixel = m0 + row;
+      const int n     = pixel / geom.oh_ow;
+      const int rem   = pixel - n * geom.oh_ow;
+      const int oy    = rem / geom.ow;
+      const int ox    = rem - oy * geom.ow;
+      a_img[t]        = n * geom.h * geom.w * geom.c;
+      a_iy0[t]        = oy * geom.stride_h - geom.pad_h;
+      a_ix0[t]        = ox * geom.stride_w - geom.pad_w;
+      a_chunk[t]      = ((lane & 7) ^ key) << 3;
+      a_src[t]        = A;
+    } else {
+      a_src[t] = A + (int64_t)(m0 + row) * lda + (((lane & 7) ^ key) << 3);
+    }
   }
+  // CONV: filter tap and first channel of the K step whose loads are being issued (all loads of one step are issued
+  // between two advances)
+  int tap_dy = 0, tap_dx = 0, tap_c0 = 0;
+  auto advance_tap = [&]() {
+    tap_c0 += kD64BK;
+    if (tap_c0 == geom.c) {
+      tap_c0 = 0;
+      if (++tap_dx == geom.kw) {
+        tap_dx = 0;
+        ++tap_dy;
+      }
+    }
+  };
 #pragma unroll
   for (int t = 0; t < LPB; ++t) {
     const int q = wave * LPB + t;
@@ -338,7 +378,16 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   // load t of step kt: first the LPA loads of the A tile, then the LPB loads of the B tile
   auto issue_one = [&](char* a_tile, char* b_tile, int kt, int t) {
     if (t < LPA) {
-      AsyncCopy16(a_src[t] + (int64_t)kt * kD64BK, a_tile + (wave * LPA + t) * 1024);
+      if (CONV) {
+        const int iy      = a_iy0[t] + tap_dy * geom.dil_h;
+        const int ix      = a_ix0[t] + tap_dx * geom.dil_w;
+        const bool inside = (unsigned)iy < (unsigned)geom.h && (unsigned)ix < (unsigned)geom.w;
+        const uint16_t* src = inside ? A + (a_img[t] + (iy * geom.w + ix) * geom.c + tap_c0 + a_chunk[t])
+                                     : static_cast<const uint16_t*>(geom.zero_page) + a_chunk[t];
+        AsyncCopy16(src, a_tile + (wave * LPA + t) * 1024);
+      } else {
+        AsyncCopy16(a_src[t] + (int64_t)kt * kD64BK, a_tile + (wave * LPA + t) * 1024);
+      }
     } else {
       AsyncCopy16(b_src[t - LPA] + kt * b_step, b_tile + (wave * LPB + t - LPA) * 1024);
     }
@@ -427,6 +476,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     for (int e = 0; e < 8; ++e) f0.b[j][e] = 0;
 #pragma unroll
   for (int t = 0; t < LPA + LPB; ++t) issue_one(sa0, sb0, 0, t);
+  if (CONV) advance_tap();  // the loads issued from now on belong to stage 1
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   __syncthreads();
   // f0 holds the last slice of the previous stage (zeros before the first)
@@ -438,6 +488,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     slice(f1, f0, ACUR, BCUR, 1, HALF, true, ANXT, BNXT, s + 1, more);                                       \
     slice(f0, f1, ACUR, BCUR, 2, 0, false, ANXT, BNXT, s + 1, more);                                         \
     slice(f1, f0, ACUR, BCUR, 3, 0, false, ANXT, BNXT, s + 1, more);                                         \
+    if (CONV) advance_tap(); /* stage s+1 has been requested: the next loads belong to stage s+2 */         \
     __builtin_amdgcn_s_waitcnt(0x0070); /* vmcnt(0) lgkmcnt(0): stage s+1 landed, fragments in registers */  \
     __syncthreads();                                                                                         \
   }
@@ -827,6 +878,8 @@ struct GemmProblem {
   const void* residual{nullptr};
   float residual_scale{0.0f};
   bool relu{false};
+  // A is the input of a channels-last convolution (implicit GEMM), not a matrix
+  const ConvGeom* conv{nullptr};
 };
 
 template <typename T, bool A_KC, bool B_KC>
@@ -861,7 +914,7 @@ void XcdRectangles(int tiles_m, int tiles_n, int* xcd_cols, int* sub_rows, int* 
   }
 }
 
-template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N>
+template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false>
 void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
   int64_t ldb = p.trans_b ? p.k : p.n;
   const int tiles_m = p.m / BM, tiles_n = p.n / BN;
@@ -875,10 +928,12 @@ void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
   epi.relu           = p.relu ? 1 : 0;
   epi.residual       = p.residual ? p.residual : (p.beta != 0.0f ? p.c : nullptr);
   epi.residual_scale = p.residual ? p.residual_scale : p.beta;
-  hipLaunchKernelGGL((gemm16_dma_kernel<T, B_KC, BM, BN, WAVES_M, WAVES_N>), grid, dim3(64 * WAVES_M * WAVES_N), 0,
+  ConvGeom geom{};
+  if (CONV) geom = *p.conv;
+  hipLaunchKernelGGL((gemm16_dma_kernel<T, B_KC, BM, BN, WAVES_M, WAVES_N, CONV>), grid, dim3(64 * WAVES_M * WAVES_N), 0,
                      stream, static_cast<const uint16_t*>(p.a), static_cast<const uint16_t*>(p.b),
                      static_cast<uint16_t*>(p.c), p.m, p.n, p.k, (int64_t)p.k, ldb, (int64_t)p.n, epi, p.stride_a,
-                     p.stride_b, p.stride_c, xcd_cols, sub_rows, sub_cols);
+                     p.stride_b, p.stride_c, xcd_cols, sub_rows, sub_cols, geom);
 }
 
 // A stored [M][K], K % 64 == 0: 256x256 tiles when they fill the chip, else 128x128 tiles when M and N allow them
@@ -891,6 +946,22 @@ bool TryDma16(const GemmProblem& p, hipStream_t stream) {
   const int64_t tiles256 = fit256 ? (int64_t)(p.m / 256) * (p.n / 256) * p.batch : 0;
   const int64_t tiles128 = fit128 ? (int64_t)(p.m / 128) * (p.n / 128) * p.batch : 0;
   static const int forced = getenv("FLAGS_cinn_hip_gemm_tile") ? atoi(getenv("FLAGS_cinn_hip_gemm_tile")) : 0;
+  if (p.conv) {
+    // implicit-GEMM convolution: filters are [OC][K]
+    if (!p.trans_b) return false;
+    if (tiles256 >= 192 && forced != 128) {
+      LaunchDma16<T, true, 256, 256, 2, 4, true>(p, stream);
+      return true;
+    }
+    // measured on ResNet-50 at batch 32 (fp16): with fewer than two 128x128 tiles per CU the 64x64 tiles of the
+    // convolution kernel are faster (19 against 26 us at 196 tiles, K = 1152) unless K is long (68 against 74 us at
+    // 196 tiles, K = 4608)
+    if (tiles128 >= 256 || (tiles128 >= 128 && p.k >= 4096) || (forced == 128 && tiles128 > 0)) {
+      LaunchDma16<T, true, 128, 128, 2, 2, true>(p, stream);
+      return true;
+    }
+    return false;
+  }
   if (tiles256 >= 192 && forced != 128) {
     if (p.trans_b) {
       LaunchDma16<T, true, 256, 256, 2, 4>(p, stream);
@@ -1103,24 +1174,39 @@ bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream) {
   const bool is_f16  = a.type.code == cinn_type_float && a.type.bits == 16;
   const bool is_bf16 = a.type.code == cinn_type_bfloat && a.type.bits == 16;
   if (!is_f16 && !is_bf16) return false;
-  if (a.nchw_input || a.kh != 1 || a.kw != 1 || a.stride_h != 1 || a.stride_w != 1 || a.pad_h != 0 || a.pad_w != 0) return false;
-  if (a.oh != a.h || a.ow != a.w_in) return false;
+  if (a.nchw_input) return false;
   const int64_t pixels = (int64_t)a.n * a.oh * a.ow;
   if (pixels >= INT_MAX) return false;
-  // measured inside ResNet-50 at batch 32: the GEMM kernels win only with at least one 128x128 tile per CU and a K
-  // loop of two steps or more; smaller grids are better served by the 64x64 tiles and split K of the convolution kernel
-  if (a.c < 128 || (pixels / 128) * (a.oc / 128) < 256) return false;
   if (reinterpret_cast<uintptr_t>(a.x) % 16 != 0 || reinterpret_cast<uintptr_t>(a.w) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(a.y) % 16 != 0 || reinterpret_cast<uintptr_t>(a.residual) % 16 != 0)
     return false;
+  const bool pointwise = a.kh == 1 && a.kw == 1 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 0 && a.pad_w == 0 &&
+                         a.oh == a.h && a.ow == a.w_in;
   GemmProblem p;
+  ConvGeom geom{};
+  if (pointwise) {
+    // measured inside ResNet-50 at batch 32: the GEMM kernels win only with at least one 128x128 tile per CU and a K
+    // loop of two steps or more; smaller grids are better served by the 64x64 tiles and split K of the convolution kernel
+    if (a.c < 128 || (pixels / 128) * (a.oc / 128) < 256) return false;
+    p.k = a.c;
+  } else {
+    // any filter, stride, padding, dilation: implicit GEMM, K = kh * kw * c with 64-channel steps inside a tap
+    static const bool conv_enabled = !(getenv("FLAGS_cinn_hip_conv_implicit_gemm") && atoi(getenv("FLAGS_cinn_hip_conv_implicit_gemm")) == 0);
+    if (!conv_enabled || a.c % 64 != 0 || (int64_t)a.n * a.h * a.w_in * a.c >= INT_MAX) return false;
+    geom.h = a.h, geom.w = a.w_in, geom.c = a.c;
+    geom.oh_ow = a.oh * a.ow, geom.ow = a.ow, geom.kw = a.kw;
+    geom.stride_h = a.stride_h, geom.stride_w = a.stride_w, geom.pad_h = a.pad_h, geom.pad_w = a.pad_w;
+    geom.dil_h = a.dil_h, geom.dil_w = a.dil_w;
+    geom.zero_page = ConvZeroPage();
+    p.conv = &geom;
+    p.k    = a.kh * a.kw * a.c;
+  }
   p.type    = is_bf16 ? GemmType::kBF16 : GemmType::kF16;
-  p.a       = a.x;  // [pixels][c]
-  p.b       = a.w;  // [oc][c]
+  p.a       = a.x;  // [pixels][c], or the NHWC input of the implicit GEMM
+  p.b       = a.w;  // [oc][kh * kw * c]
   p.c       = a.y;
   p.m       = static_cast<int>(pixels);
   p.n       = a.oc;
-  p.k       = a.c;
   p.trans_a = false;
   p.trans_b = true;
   p.alpha   = a.alpha;

@@ -343,6 +343,44 @@ def test_conv2d_channels_last_alpha_beta(gpu):
         np.testing.assert_allclose(got, 0.5 * oracle.conv2d_nchw(x, w, (1, 1), (1, 1)) + 2.0 * y0, rtol=1e-5, atol=1e-4)
 
 
+IMPLICIT_GEMM_CASES = [
+    # (n, ic, h, w, oc, k, stride, pad): 64-channel multiples, pixels a multiple of the tile height
+    (8, 64, 32, 32, 512, 3, 1, 1),     # 256 tiles of 128x128, K = 9 steps (odd)
+    (8, 128, 64, 64, 512, 3, 2, 1),    # stride 2: 32x32 outputs, window starts at -1
+    (2, 64, 64, 64, 512, 5, 1, 2),     # 5x5 filter, two rows of padding
+    (32, 64, 32, 32, 512, 3, 1, 1),    # 256 tiles of 256x256
+    (32, 192, 32, 32, 512, 1, 2, 0),   # strided 1x1 (a downsampling shortcut): 3 steps inside the one tap
+]
+
+
+@pytest.mark.parametrize("dtype,tol", [("float16", 1e-2), ("bfloat16", 2e-2)])
+@pytest.mark.parametrize("case", IMPLICIT_GEMM_CASES)
+def test_convolution_as_implicit_gemm(gpu, case, dtype, tol):
+    """Shapes the channels-last entry point runs on the direct-to-LDS GEMM kernel with the filter taps as part of K
+    (64-channel multiples, at least 256 tiles of 128x128); padding, stride and image boundaries inside a tile of 128 / 256 pixels."""
+    n, ic, h, w_, oc, k, s, p = case
+    rng = np.random.default_rng(sum(case) + 11)
+    x = round_to(rng.standard_normal((n, ic, h, w_)), dtype)
+    w = round_to(rng.standard_normal((oc, ic, k, k)) * np.sqrt(2.0 / (ic * k * k)), dtype)
+    got = call_conv_nhwc(x, w, s, p, 1, dtype)
+    want = oracle.conv2d_nchw(x, w, (s, s), (p, p))
+    scale = oracle.conv2d_nchw(np.abs(x), np.abs(w), (s, s), (p, p))
+    assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+
+
+def test_implicit_gemm_convolution_with_residual_epilogue(gpu):
+    """alpha / beta through the fp32-staged epilogue of the GEMM kernel, on a padded 3x3 convolution."""
+    n, ic, h, w_, oc = 8, 64, 32, 32, 512
+    rng = np.random.default_rng(97)
+    x = round_to(rng.standard_normal((n, ic, h, w_)), "float16")
+    w = round_to(rng.standard_normal((oc, ic, 3, 3)) * np.sqrt(2.0 / (ic * 9)), "float16")
+    y0 = round_to(rng.standard_normal((n, oc, h, w_)), "float16")
+    got = call_conv_nhwc(x, w, 1, 1, 1, "float16", alpha=0.5, beta=2.0, y_init=y0).astype(np.float64)
+    want = 0.5 * oracle.conv2d_nchw(x, w, (1, 1), (1, 1)).astype(np.float64) + 2.0 * y0
+    scale = 0.5 * oracle.conv2d_nchw(np.abs(x), np.abs(w), (1, 1), (1, 1)) + 2.0 * np.abs(y0)
+    assert np.all(np.abs(got - want) <= 2.0 ** -10 * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+
+
 @pytest.mark.parametrize("dtype,tol", [("float16", 2.0 ** -10), ("bfloat16", 2.0 ** -7)])
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (0.5, 2.0)])
 def test_pointwise_convolution_on_the_gemm_kernel(gpu, dtype, tol, alpha, beta):
