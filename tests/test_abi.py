@@ -132,6 +132,46 @@ def test_rtc_compiles_for_gfx950_without_a_gpu():
     assert runtime.rtc_compile(src) == image
 
 
+def test_code_objects_are_kept_on_disk_between_processes(tmp_path):
+    """FLAGS_cinn_hip_code_cache_dir: the first process compiles and stores <hash>.hsaco; a later process is served
+    from that file (shown by editing the file's payload: the edited bytes come back); a file whose header does not fit
+    is ignored and replaced."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cache = tmp_path / "code_cache"
+    script = ("import sys; from cinn_amd import runtime; "
+              "src = 'extern \"C\" __global__ void k(float* a) { a[threadIdx.x] += 1.0f; }'; "
+              "sys.stdout.buffer.write(runtime.rtc_compile(src, with_device_lib=False))")
+    env = dict(os.environ, FLAGS_cinn_hip_code_cache_dir=str(cache), PYTHONPATH=root)
+
+    def compile_in_new_process():
+        out = subprocess.run([sys.executable, "-c", script], cwd=root, env=env, capture_output=True, timeout=300)
+        assert out.returncode == 0, out.stderr.decode()
+        return out.stdout
+
+    image = compile_in_new_process()
+    assert image[:4] == b"\x7fELF"
+    files = list(cache.glob("*.hsaco"))
+    assert len(files) == 1 and not list(cache.glob("*.tmp.*"))
+    blob = files[0].read_bytes()
+    assert blob[32:] == image and int.from_bytes(blob[24:32], "little") == len(image)
+    # a payload edited in place comes back from the next process: the file, not hiprtc, served it
+    edited = bytearray(blob)
+    edited[-1] ^= 0xFF
+    files[0].write_bytes(bytes(edited))
+    assert compile_in_new_process() == bytes(edited[32:])
+    # truncated file: size in the header no longer fits -> recompiled and rewritten
+    files[0].write_bytes(blob[:-7])
+    assert compile_in_new_process() == image
+    assert files[0].read_bytes() == blob
+    # a different source gets a file of its own
+    script2 = script.replace("+= 1.0f", "+= 2.0f")
+    out = subprocess.run([sys.executable, "-c", script2], cwd=root, env=env, capture_output=True, timeout=300)
+    assert out.returncode == 0 and len(list(cache.glob("*.hsaco"))) == 2
+
+
 def test_bench_refuses_more_than_one_gpu():
     """the measured path has no cross-GPU work: bench.py --gpus N > 1 exits with a message instead of a number"""
     import os
