@@ -253,6 +253,27 @@ __device__ __forceinline__ void AsyncCopy16(const void* src, char* lds_base_unif
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(src) : "memory");
 }
 
+// The same copy with the address split into a wave-uniform base (scalar registers) and a 32-bit byte offset per lane,
+// so that stepping along K costs scalar additions only.  IMM is added to both the global address and the LDS address:
+// the loads of one operand tile share one m0 (SetLdsBase) and differ in IMM (a multiple of 1 KiB, below 4 KiB).
+__device__ __forceinline__ void SetLdsBase(char* lds_base_uniform) {
+  unsigned lds_addr =
+      __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) char*)lds_base_uniform);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(lds_addr) : "memory");
+}
+template <int IMM>
+__device__ __forceinline__ void AsyncCopy16At(const void* base_uniform, unsigned lane_offset) {
+  asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(lane_offset), "s"(base_uniform), "n"(IMM) : "memory");
+}
+__device__ __forceinline__ void AsyncCopy16Slot(const void* base_uniform, unsigned lane_offset, int slot) {
+  switch (slot) {
+    case 0: AsyncCopy16At<0>(base_uniform, lane_offset); break;
+    case 1: AsyncCopy16At<1024>(base_uniform, lane_offset); break;
+    case 2: AsyncCopy16At<2048>(base_uniform, lane_offset); break;
+    default: AsyncCopy16At<3072>(base_uniform, lane_offset); break;
+  }
+}
+
 constexpr int kD64BK   = 64;
 constexpr int kD64Tile = kBM * kD64BK * 2;  // one operand tile of a stage: 32 KiB
 
@@ -324,8 +345,12 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 
   // Load q = LPA wave + t of an operand fills LDS bytes [1024 q, 1024 q + 1024) of its tile: 8 rows of a
   // [row][64 halves] tile, or 512 / BN k-rows of a [k][BN halves] tile.
-  const uint16_t* a_src[LPA];
-  const uint16_t* b_src[LPB];
+  // GEMM operands: byte offset of the lane's chunk from the tile's first row (A, B stored [N][K]) or from column n0
+  // of row 0 (B stored [K][N]), less the instruction offset 1024 t of load t (which the LDS address needs)
+  static_assert(LPA <= 4 && LPB <= 4, "the instruction offset of a load is below 4 KiB");
+  unsigned a_off[LPA], b_off[LPB];
+  const char* const a_base = reinterpret_cast<const char*>(A + (int64_t)m0 * lda);
+  const char* const b_base = reinterpret_cast<const char*>(B + (B_KC ? (int64_t)n0 * ldb : (int64_t)n0));
   // CONV: element offset of image n, top-left input coordinates of the pixel's window, and the lane's chunk
   int a_img[LPA], a_iy0[LPA], a_ix0[LPA], a_chunk[LPA];
 #pragma unroll
@@ -342,9 +367,9 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
       a_iy0[t]        = oy * geom.stride_h - geom.pad_h;
       a_ix0[t]        = ox * geom.stride_w - geom.pad_w;
       a_chunk[t]      = ((lane & 7) ^ key) << 3;
-      a_src[t]        = A;
+      a_off[t]        = 0;
     } else {
-      a_src[t] = A + (int64_t)(m0 + row) * lda + (((lane & 7) ^ key) << 3);
+      a_off[t] = (unsigned)(((int64_t)row * lda + (((lane & 7) ^ key) << 3)) * 2 - 1024 * t);
     }
   }
   // CONV: filter tap and first channel of the K step whose loads are being issued (all loads of one step are issued
@@ -366,15 +391,15 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     if (B_KC) {
       const int row = 8 * q + (lane >> 3);
       const int key = (row ^ (row >> 3)) & 7;
-      b_src[t]      = B + (int64_t)(n0 + row) * ldb + (((lane & 7) ^ key) << 3);
+      b_off[t]      = (unsigned)(((int64_t)row * ldb + (((lane & 7) ^ key) << 3)) * 2 - 1024 * t);
     } else {
       constexpr int CH = BN / 8;  // 16-byte chunks per k-row
       const int krow   = q * (64 / CH) + lane / CH;
       const int chunk  = (lane % CH) ^ (2 * (krow & 3));
-      b_src[t]         = B + (int64_t)krow * ldb + n0 + (chunk << 3);
+      b_off[t]         = (unsigned)(((int64_t)krow * ldb + (chunk << 3)) * 2 - 1024 * t);
     }
   }
-  const int64_t b_step = B_KC ? kD64BK : (int64_t)kD64BK * ldb;
+  const int64_t b_step = (B_KC ? kD64BK : (int64_t)kD64BK * ldb) * 2;  // bytes per K step
   // load t of step kt: first the LPA loads of the A tile, then the LPB loads of the B tile
   auto issue_one = [&](char* a_tile, char* b_tile, int kt, int t) {
     if (t < LPA) {
@@ -386,10 +411,12 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
                                      : static_cast<const uint16_t*>(geom.zero_page) + a_chunk[t];
         AsyncCopy16(src, a_tile + (wave * LPA + t) * 1024);
       } else {
-        AsyncCopy16(a_src[t] + (int64_t)kt * kD64BK, a_tile + (wave * LPA + t) * 1024);
+        if (t == 0) SetLdsBase(a_tile + wave * LPA * 1024);
+        AsyncCopy16Slot(a_base + (int64_t)kt * (kD64BK * 2), a_off[t], t);
       }
     } else {
-      AsyncCopy16(b_src[t - LPA] + kt * b_step, b_tile + (wave * LPB + t - LPA) * 1024);
+      if (t == LPA) SetLdsBase(b_tile + wave * LPB * 1024);
+      AsyncCopy16Slot(b_base + kt * b_step, b_off[t - LPA], t - LPA);
     }
   };
 
@@ -941,6 +968,8 @@ void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
 template <typename T>
 bool TryDma16(const GemmProblem& p, hipStream_t stream) {
   if (p.trans_a || p.k % 64 != 0) return false;
+  // lanes address a tile with 32-bit byte offsets from its first row: 256 rows of K, or 64 rows of N, 16-bit elements
+  if (p.k >= (1 << 22) || p.n >= (1 << 24)) return false;
   const bool fit256 = p.m % 256 == 0 && p.n % 256 == 0;
   const bool fit128 = p.m % 128 == 0 && p.n % 128 == 0;
   const int64_t tiles256 = fit256 ? (int64_t)(p.m / 256) * (p.n / 256) * p.batch : 0;
