@@ -46,12 +46,18 @@ struct Half16<__bf16> {
   static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
 };
 template <>
 struct Half16<_Float16> {
   typedef f16x8 vec8;
   static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
 };
 
@@ -245,21 +251,18 @@ constexpr int kDmaThreads = 512;
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 
-// 16 bytes per lane from global memory straight into LDS at lds_base + 16 * lane.  Inline assembly, so that the
-// compiler does not track these loads: tracked, they get a conservative s_waitcnt vmcnt(0) before every LDS read.
-__device__ __forceinline__ void AsyncCopy16(const void* src, char* lds_base_uniform) {
-  unsigned lds_addr =
-      __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) char*)lds_base_uniform);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(src) : "memory");
-}
-
-// The same copy with the address split into a wave-uniform base (scalar registers) and a 32-bit byte offset per lane,
+// Direct global -> LDS loads: 16 bytes per lane, written at LDS address m0 + 16 * lane (+ the instruction offset).
+// Inline assembly, so that the compiler does not track these loads: tracked, they get a conservative
+// s_waitcnt vmcnt(0) before every LDS read.
+// The address is split into a wave-uniform base (scalar registers) and a 32-bit byte offset per lane,
 // so that stepping along K costs scalar additions only.  IMM is added to both the global address and the LDS address:
-// the loads of one operand tile share one m0 (SetLdsBase) and differ in IMM (a multiple of 1 KiB, below 4 KiB).
-__device__ __forceinline__ void SetLdsBase(char* lds_base_uniform) {
-  unsigned lds_addr =
-      __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) char*)lds_base_uniform);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(lds_addr) : "memory");
+// the loads of one operand tile use one m0 (SetLdsBase) and differ in IMM (a multiple of 1 KiB, below 4 KiB).
+__device__ __forceinline__ void SetLdsBase(unsigned lds_addr_uniform) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0" : : "s"(lds_addr_uniform) : "memory");
+}
+// the same for a load with a full 64-bit address per lane
+__device__ __forceinline__ void AsyncCopy16To(const void* src, unsigned lds_addr_uniform) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr_uniform), "v"(src) : "memory");
 }
 template <int IMM>
 __device__ __forceinline__ void AsyncCopy16At(const void* base_uniform, unsigned lane_offset) {
@@ -308,14 +311,16 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
                   int64_t stride_c, int xcd_cols, int sub_rows, int sub_cols, ConvGeom geom) {
   constexpr int NW      = WAVES_M * WAVES_N;
   constexpr int THREADS = 64 * NW;
-  constexpr int TM      = BM / WAVES_M / 32;  // MFMA tiles per wavefront along M and N
-  constexpr int TN      = BN / WAVES_N / 32;
+  constexpr int TM      = BM / WAVES_M / 16;  // 16x16 accumulator tiles per wavefront along M and N
+  constexpr int TN      = BN / WAVES_N / 16;
   constexpr int A_TILE  = BM * kD64BK * 2;    // bytes of one operand tile of a stage
   constexpr int B_TILE  = BN * kD64BK * 2;
   constexpr int LPA     = BM / 8 / NW;        // loads (of 1 KiB per wavefront) per thread, operand and step
   constexpr int LPB     = BN / 8 / NW;
-  static_assert(LPA >= 1 && LPB >= 1 && TM >= 1 && TN >= 1 && (LPA + LPB) % 2 == 0, "unsupported tile shape");
+  static_assert(LPA >= 1 && LPB >= 1 && TM % 4 == 0 && TN == 4, "unsupported tile shape");
   __shared__ __attribute__((aligned(1024))) char lds[2 * (A_TILE + B_TILE)];
+  const unsigned lds_addr =
+      __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) char*)lds);
   char* const sa0 = lds;
   char* const sb0 = lds + A_TILE;
   char* const sa1 = lds + A_TILE + B_TILE;
@@ -351,23 +356,23 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   unsigned a_off[LPA], b_off[LPB];
   const char* const a_base = reinterpret_cast<const char*>(A + (int64_t)m0 * lda);
   const char* const b_base = reinterpret_cast<const char*>(B + (B_KC ? (int64_t)n0 * ldb : (int64_t)n0));
-  // CONV: element offset of image n, top-left input coordinates of the pixel's window, and the lane's chunk
-  int a_img[LPA], a_iy0[LPA], a_ix0[LPA], a_chunk[LPA];
+  // CONV: a_off is the byte offset of the lane's chunk at the top-left corner of the pixel's window (it may lie before
+  // the image: the tap's offset is added modulo 2^32), a_yx that corner's coordinates, 16 bits each
+  int a_yx[LPA];
 #pragma unroll
   for (int t = 0; t < LPA; ++t) {
     const int row = 8 * (wave * LPA + t) + (lane >> 3);
-    const int key = (row ^ (row >> 3)) & 7;
+    const int key = (row & 7) ^ ((row >> 3) & 1);  // chunk swizzle of a [row][64 halves] tile, see the fragment reads
     if (CONV) {
       const int pixel = m0 + row;
       const int n     = pixel / geom.oh_ow;
       const int rem   = pixel - n * geom.oh_ow;
       const int oy    = rem / geom.ow;
       const int ox    = rem - oy * geom.ow;
-      a_img[t]        = n * geom.h * geom.w * geom.c;
-      a_iy0[t]        = oy * geom.stride_h - geom.pad_h;
-      a_ix0[t]        = ox * geom.stride_w - geom.pad_w;
-      a_chunk[t]      = ((lane & 7) ^ key) << 3;
-      a_off[t]        = 0;
+      const int iy0   = oy * geom.stride_h - geom.pad_h;
+      const int ix0   = ox * geom.stride_w - geom.pad_w;
+      a_yx[t]         = (iy0 & 0xffff) | (ix0 << 16);
+      a_off[t]        = ((unsigned)((n * geom.h + iy0) * geom.w + ix0) * (unsigned)geom.c + (((lane & 7) ^ key) << 3)) * 2u;
     } else {
       a_off[t] = (unsigned)(((int64_t)row * lda + (((lane & 7) ^ key) << 3)) * 2 - 1024 * t);
     }
@@ -390,12 +395,12 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     const int q = wave * LPB + t;
     if (B_KC) {
       const int row = 8 * q + (lane >> 3);
-      const int key = (row ^ (row >> 3)) & 7;
+      const int key = (row & 7) ^ ((row >> 3) & 1);
       b_off[t]      = (unsigned)(((int64_t)row * ldb + (((lane & 7) ^ key) << 3)) * 2 - 1024 * t);
     } else {
       constexpr int CH = BN / 8;  // 16-byte chunks per k-row
       const int krow   = q * (64 / CH) + lane / CH;
-      const int chunk  = (lane % CH) ^ (2 * (krow & 3));
+      const int chunk  = (lane % CH) ^ (2 * (krow & 3)) ^ (8 * ((krow >> 3) & 1));
       b_off[t]         = (unsigned)(((int64_t)krow * ldb + (chunk << 3)) * 2 - 1024 * t);
     }
   }
@@ -404,129 +409,155 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   auto issue_one = [&](char* a_tile, char* b_tile, int kt, int t) {
     if (t < LPA) {
       if (CONV) {
-        const int iy      = a_iy0[t] + tap_dy * geom.dil_h;
-        const int ix      = a_ix0[t] + tap_dx * geom.dil_w;
+        const int iy      = (short)(a_yx[t] & 0xffff) + tap_dy * geom.dil_h;
+        const int ix      = (a_yx[t] >> 16) + tap_dx * geom.dil_w;
         const bool inside = (unsigned)iy < (unsigned)geom.h && (unsigned)ix < (unsigned)geom.w;
-        const uint16_t* src = inside ? A + (a_img[t] + (iy * geom.w + ix) * geom.c + tap_c0 + a_chunk[t])
-                                     : static_cast<const uint16_t*>(geom.zero_page) + a_chunk[t];
-        AsyncCopy16(src, a_tile + (wave * LPA + t) * 1024);
+        // the tap's offset is uniform: ((dy dil_h) w + dx dil_w) c + c0 elements
+        const unsigned tap_off =
+            ((unsigned)((tap_dy * geom.dil_h) * geom.w + tap_dx * geom.dil_w) * (unsigned)geom.c + tap_c0) * 2u;
+        const char* src = inside ? reinterpret_cast<const char*>(A) + (a_off[t] + tap_off)
+                                 : static_cast<const char*>(geom.zero_page) + ((lane & 7) << 4);
+        AsyncCopy16To(src, lds_addr + (unsigned)(a_tile - lds) + (wave * LPA + t) * 1024);
       } else {
-        if (t == 0) SetLdsBase(a_tile + wave * LPA * 1024);
+        SetLdsBase(lds_addr + (unsigned)(a_tile - lds) + wave * LPA * 1024);
         AsyncCopy16Slot(a_base + (int64_t)kt * (kD64BK * 2), a_off[t], t);
       }
     } else {
-      if (t == LPA) SetLdsBase(b_tile + wave * LPB * 1024);
+      SetLdsBase(lds_addr + (unsigned)(b_tile - lds) + wave * LPB * 1024);
       AsyncCopy16Slot(b_base + kt * b_step, b_off[t - LPA], t - LPA);
     }
   };
 
-  f32x16 acc[TM][TN];
+  f32x4 acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
 
-  const int frag_row = lane & 31;
-  const int frag_kg  = lane >> 5;
-  struct Frags {
-    vec8 a[TM];
-    vec8 b[TN];
+  // v_mfma_f32_16x16x32: lane l holds, of A, row l % 16 and k = 8 (l / 16) .. + 7 of a 32-deep slice (one 16-byte
+  // chunk); of B likewise for column l % 16; of the result, column l % 16 and rows 4 (l / 16) .. + 3.
+  // Which 8 of the 32 k a lane group holds is free as long as A and B agree: groups 0..3 take the k chunks 0, 2, 1, 3,
+  // so that lanes l and l + 32, which the LDS serves together on a 16-byte read, fetch chunks that differ in bit 0
+  // (the row swizzle then puts them in different banks).
+  const int frag_row = lane & 15;
+  const int frag_kg  = ((lane >> 4) & 1) * 2 + (lane >> 5);
+  // [row][64 halves] tiles keep chunk c of row r at chunk position c ^ (r & 7) ^ ((r >> 3) & 1): the eight lanes the
+  // LDS serves together from one k group hit eight different 16-byte bank groups, and the key depends on r % 16 only,
+  // so one address register per slice serves all of a wavefront's tiles (tile i is an immediate offset of 2 KiB i).
+  const int frag_key = (frag_row & 7) ^ (frag_row >> 3);
+  int frag_off[2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) frag_off[kk] = frag_row * 128 + (((kk * 4 + frag_kg) ^ frag_key) << 4);
+  auto read_a = [&](const char* a_tile, int kk, int i) -> vec8 {
+    return *reinterpret_cast<const vec8*>(a_tile + frag_off[kk] + (wm * TM + i) * 2048);
   };
-  auto read_a = [&](const char* a_tile, int kk, int i, Frags& f) {
-    f.a[i] = *reinterpret_cast<const vec8*>(a_tile + TileOffset(wm * (TM * 32) + i * 32 + frag_row, kk * 2 + frag_kg));
-  };
-  auto read_b = [&](const char* b_tile, int kk, int j, Frags& f) {
+  auto read_b = [&](const char* b_tile, int kk, int j) -> vec8 {
     if (B_KC) {
-      f.b[j] = *reinterpret_cast<const vec8*>(b_tile + TileOffset(wn * (TN * 32) + j * 32 + frag_row, kk * 2 + frag_kg));
+      return *reinterpret_cast<const vec8*>(b_tile + frag_off[kk] + (wn * TN + j) * 2048);
     } else {
+      // a transposing read hands lane i of a group of 16 four consecutive k of column i: the group addresses a block
+      // of 4 k-rows x 16 columns, every lane four columns of one k-row
       s16x4 part[2];
 #pragma unroll
       for (int r = 0; r < 2; ++r) {
-        const int k   = kk * 16 + 4 * (2 * frag_kg + r) + ((lane & 15) >> 2);
-        const int n   = wn * (TN * 32) + j * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-        const int off = k * (BN * 2) + (((n >> 3) ^ (2 * (k & 3))) << 4) + (n & 7) * 2;
+        const int k   = kk * 32 + 8 * frag_kg + 4 * r + ((lane & 15) >> 2);
+        const int n   = wn * (TN * 16) + j * 16 + 4 * (lane & 3);
+        const int off = k * (BN * 2) + (((n >> 3) ^ (2 * (k & 3)) ^ (8 * ((k >> 3) & 1))) << 4) + (n & 7) * 2;
         part[r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(b_tile + off));
       }
       s16x8 both = __builtin_shufflevector(part[0], part[1], 0, 1, 2, 3, 4, 5, 6, 7);
-      f.b[j]     = __builtin_bit_cast(vec8, both);
+      return __builtin_bit_cast(vec8, both);
     }
   };
 #define CINN_SB __builtin_amdgcn_sched_barrier(0)
-  constexpr int NM    = TM * TN;            // MFMAs of a slice
-  constexpr int HALF  = (LPA + LPB) / 2;    // loads issued in each of the two slices after the barrier
-  constexpr int EVERY = NM / HALF;          // one load after every EVERY-th MFMA
-  static_assert(NM % HALF == 0 && NM >= TM + TN, "the slice schedule needs a slot per fragment read and load");
-  // one 16-deep slice: the MFMAs of `cur`, after each of them one fragment read of slice kk_next into `nxt`
-  // (a0, b0, a1, b1, ... in the order the next slice uses them) and, when with_loads, after every EVERY-th one a
-  // load (first_load ..) of the next stage
-  auto slice = [&](Frags& cur, Frags& nxt, const char* a_rd, const char* b_rd, int kk_next, int first_load,
-                   bool with_loads, char* a_wr, char* b_wr, int kt_next, bool more) {
-#pragma unroll
-    for (int m = 0; m < NM; ++m) {
-      CINN_SB;
-      acc[m / TN][m % TN] = Half16<T>::mfma(cur.a[m / TN], cur.b[m % TN], acc[m / TN][m % TN]);
-      CINN_SB;
-      // read m of the list a0, b0, a1, b1, ..., then the rest of the longer operand
-      constexpr int PAIRS = TM < TN ? TM : TN;
-      if (m < 2 * PAIRS) {
-        if (m % 2 == 0) {
-          read_a(a_rd, kk_next, m / 2, nxt);
-        } else {
-          read_b(b_rd, kk_next, m / 2, nxt);
-        }
-      } else if (m < TM + TN) {
-        if (TM > TN) {
-          read_a(a_rd, kk_next, m - PAIRS, nxt);
-        } else {
-          read_b(b_rd, kk_next, m - PAIRS, nxt);
-        }
-      }
-      if (with_loads && m % EVERY == EVERY - 1) {
-        CINN_SB;
-        if (more) issue_one(a_wr, b_wr, kt_next, first_load + m / EVERY);
-      }
-    }
-    CINN_SB;
-  };
+  // A K step is ROWS = 2 TM rows of TN MFMAs: row r multiplies the A fragment of tile r % TM, slice r / TM (32 deep),
+  // with the TN B fragments of that slice.  A fragments live in a ring of four (row r + 3 is requested after the first
+  // MFMA of row r), B fragments in two sets (the second slice's are requested early in the first, the next stage's
+  // after the barrier).  The barrier follows row ROWS - 4: by then every fragment of the stage is in registers, so
+  // the three rows after it (12 MFMAs) run while the first fragments of the next stage are fetched, and the stage's
+  // LDS is free for the loads of the stage after next, issued in those same rows.
+  constexpr int ROWS = 2 * TM;
+  constexpr int BAR  = ROWS - 4;
+  // One load per row keeps pace with the 16 clocks per load instruction and CU at which the vector memory path
+  // drains: EARLY loads of stage s + 2 in the three rows after the barrier of step s, the others in the first rows
+  // of step s + 1.
+  constexpr int EARLY = 3;
+  constexpr int LATE  = LPA + LPB - EARLY;
+  static_assert(LATE >= 0 && LATE <= BAR + 1, "the late loads are issued before the barrier that waits for them");
+  vec8 ring[4];
+  vec8 bf[2][TN];
 
   const int nk = K / kD64BK;
-  Frags f0, f1;
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) f0.a[i][e] = 0;
-#pragma unroll
-  for (int j = 0; j < TN; ++j)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) f0.b[j][e] = 0;
 #pragma unroll
   for (int t = 0; t < LPA + LPB; ++t) issue_one(sa0, sb0, 0, t);
-  if (CONV) advance_tap();  // the loads issued from now on belong to stage 1
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-  __syncthreads();
-  // f0 holds the last slice of the previous stage (zeros before the first)
-#define CINN_GEMM_STEP(ACUR, BCUR, ANXT, BNXT, OFF)                                                          \
-  {                                                                                                          \
-    const int s     = kt + OFF;                                                                              \
-    const bool more = s + 1 < nk;                                                                            \
-    slice(f0, f1, ACUR, BCUR, 0, 0, true, ANXT, BNXT, s + 1, more);                                          \
-    slice(f1, f0, ACUR, BCUR, 1, HALF, true, ANXT, BNXT, s + 1, more);                                       \
-    slice(f0, f1, ACUR, BCUR, 2, 0, false, ANXT, BNXT, s + 1, more);                                         \
-    slice(f1, f0, ACUR, BCUR, 3, 0, false, ANXT, BNXT, s + 1, more);                                         \
-    if (CONV) advance_tap(); /* stage s+1 has been requested: the next loads belong to stage s+2 */         \
-    __builtin_amdgcn_s_waitcnt(0x0070); /* vmcnt(0) lgkmcnt(0): stage s+1 landed, fragments in registers */  \
-    __syncthreads();                                                                                         \
+  if (CONV) advance_tap();
+  if (nk > 1) {
+#pragma unroll
+    for (int t = 0; t < EARLY; ++t) issue_one(sa1, sb1, 1, t);
+    __builtin_amdgcn_s_waitcnt(0x0F70 | EARLY);  // vmcnt: stage 0 has landed, the first loads of stage 1 may be in flight
+  } else {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
   }
-  for (int kt = 0; kt < nk; kt += 2) {
-    CINN_GEMM_STEP(sa0, sb0, sa1, sb1, 0)
-    if (kt + 1 < nk) CINN_GEMM_STEP(sa1, sb1, sa0, sb0, 1)
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 3; ++i) ring[i] = read_a(sa0, 0, i);
+#pragma unroll
+  for (int j = 0; j < TN; ++j) bf[0][j] = read_b(sb0, 0, j);
+
+#define CINN_GEMM_STEP(ACUR, BCUR, ANXT, BNXT, OFF, HAS_NEXT, HAS_LOAD)                                      \
+  {                                                                                                          \
+    const int s         = kt + OFF;                                                                          \
+    const bool has_next = HAS_NEXT;                                                                          \
+    const bool has_load = HAS_LOAD;                                                                          \
+    _Pragma("unroll") for (int r = 0; r < ROWS; ++r) {                                                       \
+      _Pragma("unroll") for (int j = 0; j < TN; ++j) {                                                       \
+        CINN_SB;                                                                                             \
+        acc[r % TM][j] = Half16<T>::mfma16(ring[r % 4], bf[r / TM][j], acc[r % TM][j]);                      \
+        CINN_SB;                                                                                             \
+        if (j == 0) {                                                                                        \
+          if (r + 3 < ROWS) {                                                                                \
+            ring[(r + 3) % 4] = read_a(ACUR, (r + 3) / TM, (r + 3) % TM);                                    \
+          } else if (has_next) {                                                                             \
+            ring[(r + 3) % 4] = read_a(ANXT, 0, r + 3 - ROWS);                                               \
+          }                                                                                                  \
+        }                                                                                                    \
+        if ((j == 1 || j == 2) && r >= TM / 2 - 2 && r < TM / 2) {                                           \
+          bf[1][(r - (TM / 2 - 2)) * 2 + j - 1] = read_b(BCUR, 1, (r - (TM / 2 - 2)) * 2 + j - 1);          \
+        }                                                                                                    \
+        if ((j == 1 || j == 2) && r >= ROWS - 3 && r < ROWS - 1 && has_next) {                               \
+          bf[0][(r - (ROWS - 3)) * 2 + j - 1] = read_b(BNXT, 0, (r - (ROWS - 3)) * 2 + j - 1);              \
+        }                                                                                                    \
+        if (j == 3 && r < LATE) {                                                                            \
+          CINN_SB;                                                                                           \
+          if (has_next) issue_one(ANXT, BNXT, s + 1, EARLY + r);                                             \
+          if (CONV && r == LATE - 1) advance_tap(); /* stage s+1 has been requested */                       \
+        }                                                                                                    \
+        if (j == 3 && r >= ROWS - 3) {                                                                       \
+          CINN_SB;                                                                                           \
+          if (has_load) issue_one(ACUR, BCUR, s + 2, r - (ROWS - 3));                                        \
+        }                                                                                                    \
+      }                                                                                                      \
+      if (r == BAR && has_next) {                                                                            \
+        CINN_SB;                                                                                             \
+        __builtin_amdgcn_s_waitcnt(0x0070); /* vmcnt(0) lgkmcnt(0): stage s+1 landed, fragments arrived */   \
+        __syncthreads();                                                                                     \
+      }                                                                                                      \
+    }                                                                                                        \
+  }
+  // pairs of steps that both have a stage after next to request: no branches around the loads; then the last one
+  // to three steps with the conditions evaluated
+  int kt = 0;
+  for (; kt + 3 < nk; kt += 2) {
+    CINN_GEMM_STEP(sa0, sb0, sa1, sb1, 0, true, true)
+    CINN_GEMM_STEP(sa1, sb1, sa0, sb0, 1, true, true)
+  }
+  for (; kt < nk; kt += 2) {
+    CINN_GEMM_STEP(sa0, sb0, sa1, sb1, 0, s + 1 < nk, s + 2 < nk)
+    if (kt + 1 < nk) CINN_GEMM_STEP(sa1, sb1, sa0, sb0, 1, s + 1 < nk, s + 2 < nk)
   }
 #undef CINN_GEMM_STEP
-  // the last slice of the last stage
-#pragma unroll
-  for (int m = 0; m < NM; ++m) acc[m / TN][m % TN] = Half16<T>::mfma(f0.a[m / TN], f0.b[m % TN], acc[m / TN][m % TN]);
 #undef CINN_SB
 
   // Epilogue on the fp32 accumulators: v = acc * (scale[col] or alpha) + shift[col] + residual_scale * R[row][col],
@@ -539,15 +570,15 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   float sc[TN], sh[TN];
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
-    const int col = n0 + wn * (TN * 32) + j * 32 + (lane & 31);
+    const int col = n0 + wn * (TN * 16) + j * 16 + (lane & 15);
     sc[j]         = epi.scale ? epi.scale[col] : epi.alpha;
     sh[j]         = epi.shift ? epi.shift[col] : 0.0f;
   }
   constexpr int CPR = BN / 8;  // 8-column chunks per row
   if (!Rt) {
     constexpr int kRowBytes = (BN + 8) * 2;
-    constexpr int IB        = TM < 2 ? TM : 2;  // 32-row blocks per wavefront and pass
-    constexpr int PASS_ROWS = WAVES_M * IB * 32;
+    constexpr int IB        = 4;  // 16-row blocks per wavefront and pass: 64 rows
+    constexpr int PASS_ROWS = WAVES_M * IB * 16;
     static_assert(PASS_ROWS * kRowBytes <= 2 * (A_TILE + B_TILE), "the staged result does not fit the operand stages");
     static_assert(PASS_ROWS * CPR % THREADS == 0, "the copy-out loop assumes whole rounds");
 #pragma unroll
@@ -558,9 +589,9 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int lrow = wm * (IB * 32) + ii * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            const int col  = wn * (TN * 32) + j * 32 + (lane & 31);
+          for (int r = 0; r < 4; ++r) {
+            const int lrow = wm * (IB * 16) + ii * 16 + 4 * (lane >> 4) + r;
+            const int col  = wn * (TN * 16) + j * 16 + (lane & 15);
             float v        = acc[IB * pass + ii][j][r] * sc[j] + sh[j];
             if (epi.relu) v = v > 0.0f ? v : 0.0f;
             *reinterpret_cast<T*>(lds + lrow * kRowBytes + col * 2) = (T)v;
@@ -571,7 +602,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
         const int chunk = e * THREADS + tid;
         const int lrow  = chunk / CPR;
         const int c16   = chunk % CPR;
-        const int row   = m0 + (lrow / (IB * 32)) * (TM * 32) + pass * (IB * 32) + lrow % (IB * 32);
+        const int row   = m0 + (lrow / (IB * 16)) * (TM * 16) + pass * (IB * 16) + lrow % (IB * 16);
         const u32x4 v   = *reinterpret_cast<const u32x4*>(lds + lrow * kRowBytes + c16 * 16);
         *reinterpret_cast<u32x4*>(Ct + (int64_t)row * ldc + n0 + c16 * 8) = v;
       }
@@ -579,28 +610,31 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     return;
   }
   constexpr int kRowFloats = BN + 4;
-  constexpr int PASS_ROWS  = WAVES_M * 32;
+  constexpr int IB         = 2;  // 16-row blocks per wavefront and pass: 32 rows of fp32
+  constexpr int PASS_ROWS  = WAVES_M * IB * 16;
   static_assert(PASS_ROWS * kRowFloats * 4 <= 2 * (A_TILE + B_TILE), "the staged result does not fit the operand stages");
   static_assert(PASS_ROWS * CPR % THREADS == 0, "the copy-out loop assumes whole rounds");
   float* stage = reinterpret_cast<float*>(lds);
 #pragma unroll
-  for (int pass = 0; pass < TM; ++pass) {
+  for (int pass = 0; pass < TM / IB; ++pass) {
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < TN; ++j)
+    for (int ii = 0; ii < IB; ++ii)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int lrow = wm * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        const int col  = wn * (TN * 32) + j * 32 + (lane & 31);
-        stage[lrow * kRowFloats + col] = acc[pass][j][r] * sc[j] + sh[j];
-      }
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int lrow = wm * (IB * 16) + ii * 16 + 4 * (lane >> 4) + r;
+          const int col  = wn * (TN * 16) + j * 16 + (lane & 15);
+          stage[lrow * kRowFloats + col] = acc[IB * pass + ii][j][r] * sc[j] + sh[j];
+        }
     __syncthreads();
 #pragma unroll
     for (int e = 0; e < PASS_ROWS * CPR / THREADS; ++e) {
       const int chunk = e * THREADS + tid;
       const int lrow  = chunk / CPR;
       const int c8    = chunk % CPR;
-      const int row   = m0 + (lrow / 32) * (TM * 32) + pass * 32 + lrow % 32;
+      const int row   = m0 + (lrow / (IB * 16)) * (TM * 16) + pass * (IB * 16) + lrow % (IB * 16);
       const int64_t o = (int64_t)row * ldc + n0 + c8 * 8;
       const f32x4 lo  = *reinterpret_cast<const f32x4*>(stage + lrow * kRowFloats + c8 * 8);
       const f32x4 hi  = *reinterpret_cast<const f32x4*>(stage + lrow * kRowFloats + c8 * 8 + 4);
@@ -1222,6 +1256,8 @@ bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream) {
     // any filter, stride, padding, dilation: implicit GEMM, K = kh * kw * c with 64-channel steps inside a tap
     static const bool conv_enabled = !(getenv("FLAGS_cinn_hip_conv_implicit_gemm") && atoi(getenv("FLAGS_cinn_hip_conv_implicit_gemm")) == 0);
     if (!conv_enabled || a.c % 64 != 0 || (int64_t)a.n * a.h * a.w_in * a.c >= INT_MAX) return false;
+    // window corners are kept as two signed 16-bit coordinates
+    if (a.h + a.pad_h >= 32768 || a.w_in + a.pad_w >= 32768) return false;
     geom.h = a.h, geom.w = a.w_in, geom.c = a.c;
     geom.oh_ow = a.oh * a.ow, geom.ow = a.ow, geom.kw = a.kw;
     geom.stride_h = a.stride_h, geom.stride_w = a.stride_w, geom.pad_h = a.pad_h, geom.pad_w = a.pad_w;
