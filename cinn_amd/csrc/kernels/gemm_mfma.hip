@@ -400,7 +400,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     } else {
       constexpr int CH = BN / 8;  // 16-byte chunks per k-row
       const int krow   = q * (64 / CH) + lane / CH;
-      const int chunk  = (lane % CH) ^ (2 * (krow & 3)) ^ (8 * ((krow >> 3) & 1));
+      const int chunk  = (lane % CH) ^ (2 * (krow & 3)) ^ (8 * ((krow >> 4) & 1));
       b_off[t]         = (unsigned)(((int64_t)krow * ldb + (chunk << 3)) * 2 - 1024 * t);
     }
   }
@@ -464,7 +464,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
       for (int r = 0; r < 2; ++r) {
         const int k   = kk * 32 + 8 * frag_kg + 4 * r + ((lane & 15) >> 2);
         const int n   = wn * (TN * 16) + j * 16 + 4 * (lane & 3);
-        const int off = k * (BN * 2) + (((n >> 3) ^ (2 * (k & 3)) ^ (8 * ((k >> 3) & 1))) << 4) + (n & 7) * 2;
+        const int off = k * (BN * 2) + (((n >> 3) ^ (2 * (k & 3)) ^ (8 * ((k >> 4) & 1))) << 4) + (n & 7) * 2;
         part[r] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(b_tile + off));
       }
       s16x8 both = __builtin_shufflevector(part[0], part[1], 0, 1, 2, 3, 4, 5, 6, 7);
