@@ -397,14 +397,14 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
         continue;
       }
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = v[e] * sc[e] + sh[e];
+      for (int e = 0; e < 8; ++e) v[e] = __builtin_fmaf(v[e], sc[e], sh[e]);
       if (full) {
         T out[8];
         if (residual) {
           T rv[8];
           __builtin_memcpy(rv, residual + off, 8 * sizeof(T));
 #pragma unroll
-          for (int e = 0; e < 8; ++e) v[e] += p.residual_scale * (float)rv[e];
+          for (int e = 0; e < 8; ++e) v[e] = __builtin_fmaf(p.residual_scale, (float)rv[e], v[e]);
         }
 #pragma unroll
         for (int e = 0; e < 8; ++e) out[e] = (T)(p.relu ? fmaxf(v[e], 0.0f) : v[e]);
@@ -412,7 +412,7 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
       } else {
         for (int e = 0; e < 8 && oc0 + e < p.oc; ++e) {
           float t = v[e];
-          if (residual) t += p.residual_scale * (float)residual[off + e];
+          if (residual) t = __builtin_fmaf(p.residual_scale, (float)residual[off + e], t);
           y[off + e] = (T)(p.relu ? fmaxf(t, 0.0f) : t);
         }
       }

@@ -292,7 +292,7 @@ conv_stem_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, const f
         *reinterpret_cast<f32x4*>(&v[0]) = *reinterpret_cast<const f32x4*>(&stage[pixel * kStagePitch + cg * 8]);
         *reinterpret_cast<f32x4*>(&v[4]) = *reinterpret_cast<const f32x4*>(&stage[pixel * kStagePitch + cg * 8 + 4]);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = v[e] * sc[j][e] + sh[j][e];
+        for (int e = 0; e < 8; ++e) v[e] = __builtin_fmaf(v[e], sc[j][e], sh[j][e]);
         const int64_t off = (((int64_t)n * p.oh + oh) * p.ow + ow) * p.oc + oc0;
         if (full) {
           T out[8];
@@ -300,7 +300,7 @@ conv_stem_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, const f
             T rv[8];
             __builtin_memcpy(rv, residual + off, 8 * sizeof(T));
 #pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] += p.residual_scale * (float)rv[e];
+            for (int e = 0; e < 8; ++e) v[e] = __builtin_fmaf(p.residual_scale, (float)rv[e], v[e]);
           }
 #pragma unroll
           for (int e = 0; e < 8; ++e) out[e] = (T)(p.relu ? fmaxf(v[e], 0.0f) : v[e]);

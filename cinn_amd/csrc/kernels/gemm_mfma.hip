@@ -223,28 +223,36 @@ gemm16_mfma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ 
 
 // ---------------------------------------------------------------------------------------------------
 // bf16 / fp16 with A stored [M][K]: direct global -> LDS loads (global_load_lds_dwordx4), 8 wavefronts.
-// 256x256 block tile, K step 64, 512 threads in a 2 (M) x 4 (N) wavefront grid, each wavefront a 128x64 tile (8 MFMA
-// accumulators), two wavefronts per SIMD.
+// 256x256 block tile, K step 64, 512 threads in a 2 (M) x 4 (N) wavefront grid, each wavefront a 128x64 tile = 8 x 4
+// accumulators of v_mfma_f32_16x16x32 (measured on sustained MFMA-only loops with random operands: 2.14 PFLOP/s
+// with 16x16x32 against 1.92 with 32x32x16 - the chip is power limited and the narrow shape moves less accumulator
+// data per flop), two wavefronts per SIMD.
 //   * Every row of an operand tile is one whole 128-byte line.  With a K step of 32 (64-byte rows) the vector L1
 //     fetches every line twice from L2, one step apart, and that fill traffic bounds the feed: measured 32 bytes per
 //     clock and CU with 64-byte rows against 48-51 with 128-byte rows.
 //   * A lane of a load instruction writes its 16 bytes at LDS base + 16 * lane, so the swizzle that makes the fragment
 //     reads conflict free is applied on the global side: each lane fetches the chunk that belongs at its LDS slot.
-//     A load instruction covers 8 rows x 128 bytes.
+//     A load instruction covers 8 rows x 128 bytes.  Its address is a scalar base (stepped along K with scalar adds)
+//     plus a fixed 32-bit offset per lane.
+//   * 16-byte LDS reads are served eight lanes of each wavefront half at a time (lanes 8p..8p+7 together with
+//     32+8p..32+8p+7; found by counting bank conflicts): the fragment layout gives those sixteen lanes sixteen
+//     different 16-byte bank groups (SQ_LDS_BANK_CONFLICT = 0).
 //   * B stored [K][N] (the plain row-major matmul) is kept as [k][n] in LDS ([64 k][512 B], a load instruction
 //     covers 2 k-rows) and read with ds_read_b64_tr_b16, which hands every lane four consecutive k of one column -
 //     no transposition in registers.
-//   * Two stages of 64 KiB.  One barrier per K step, placed before the MFMAs of the step's last 16-deep slice: at
-//     that point every wavefront has its last fragments of stage s in registers, so stage s's slot is free for the
-//     loads of stage s+2, which are issued right after that barrier and waited for at the barrier of step s+1 - a
-//     whole K step of MFMAs (2048 clocks per SIMD at the full rate) hides their latency.
-//   * After every MFMA one LDS fragment read (requested a slice ahead; scheduling barriers pin the order) and, in the
-//     two slices after the barrier, after every second MFMA one load.
+//   * Two stages of 64 KiB and one barrier per K step, three MFMA rows (12 MFMAs) before the step's end: by then every
+//     fragment of stage s is in registers, so those rows cover the first fragment reads of stage s+1, and stage s's
+//     slot is free for the loads of stage s+2: one load per MFMA row (the rate at which the vector memory path
+//     drains them), three after the barrier and the rest in the first rows of the next step; they are waited for at
+//     the barrier of step s+1.
+//   * A fragments in a ring of four (requested three rows ahead), B fragments in two sets; scheduling barriers pin
+//     the order.  The main loop has no branches: the last one to three steps, which have nothing left to request,
+//     are peeled.
 //   * The result tile goes through LDS (two passes of 128 rows) so that a store instruction covers two whole 512-byte
 //     rows of C.
-// In core clocks the main loop keeps the MFMA pipe 84 % busy (156 k clocks for 131 k of MFMA at 4096^3); what the
-// kernel delivers beyond that is set by the clock the chip sustains under this load (1.2-1.6 GHz measured inside
-// the loop against the 2.4 GHz of the quoted peak).
+// In core clocks a K step takes about 2330 clocks for 2048 of MFMA at 4096^3 (the rest: the slower wavefront of each
+// SIMD waiting for its loads and the barrier, about 190 clocks, and issue gaps); what the kernel delivers beyond that
+// is set by the clock the chip sustains under this load (1.7-1.9 GHz measured against the 2.4 GHz of the quoted peak).
 // Requires M % BM == N % BN == K % 64 == 0.
 // ---------------------------------------------------------------------------------------------------
 constexpr int kDmaThreads = 512;
@@ -483,7 +491,9 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   // One load per row keeps pace with the 16 clocks per load instruction and CU at which the vector memory path
   // drains: EARLY loads of stage s + 2 in the three rows after the barrier of step s, the others in the first rows
   // of step s + 1.
-  constexpr int EARLY = 3;
+  // A wavefront tile of 64 rows has short steps (8 rows): all its loads go into the three rows after the barrier.
+  constexpr int EPR   = TM == 4 ? 3 : 1;  // loads per row after the barrier
+  constexpr int EARLY = 3 * EPR < LPA + LPB ? 3 * EPR : LPA + LPB;
   constexpr int LATE  = LPA + LPB - EARLY;
   static_assert(LATE >= 0 && LATE <= BAR + 1, "the late loads are issued before the barrier that waits for them");
   vec8 ring[4];
@@ -496,6 +506,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   if (nk > 1) {
 #pragma unroll
     for (int t = 0; t < EARLY; ++t) issue_one(sa1, sb1, 1, t);
+    if (CONV && LATE == 0) advance_tap();
     __builtin_amdgcn_s_waitcnt(0x0F70 | EARLY);  // vmcnt: stage 0 has landed, the first loads of stage 1 may be in flight
   } else {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
@@ -534,9 +545,11 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
           if (has_next) issue_one(ANXT, BNXT, s + 1, EARLY + r);                                             \
           if (CONV && r == LATE - 1) advance_tap(); /* stage s+1 has been requested */                       \
         }                                                                                                    \
-        if (j == 3 && r >= ROWS - 3) {                                                                       \
+        if ((j == 3 || (EPR == 3 && j >= 1)) && r >= ROWS - 3 &&                                             \
+            (r - (ROWS - 3)) * EPR + (EPR == 3 ? j - 1 : 0) < EARLY) {                                       \
           CINN_SB;                                                                                           \
-          if (has_load) issue_one(ACUR, BCUR, s + 2, r - (ROWS - 3));                                        \
+          if (has_load) issue_one(ACUR, BCUR, s + 2, (r - (ROWS - 3)) * EPR + (EPR == 3 ? j - 1 : 0));       \
+          if (CONV && LATE == 0 && (r - (ROWS - 3)) * EPR + (EPR == 3 ? j - 1 : 0) == EARLY - 1) advance_tap(); \
         }                                                                                                    \
       }                                                                                                      \
       if (r == BAR && has_next) {                                                                            \
@@ -560,10 +573,13 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 #undef CINN_GEMM_STEP
 #undef CINN_SB
 
-  // Epilogue on the fp32 accumulators: v = acc * (scale[col] or alpha) + shift[col] + residual_scale * R[row][col],
+  // Epilogue on the fp32 accumulators: v = fma(residual_scale, R[row][col], fma(acc, scale[col] or alpha, shift[col]))
+  // (explicit fused multiply-adds rounded to fp32, and an empty asm between them and the conversion to T: left to the
+  // compiler, some accumulators get v_fma_mixlo_f16 - one rounding, straight to fp16 - and others v_fma_f32 plus a
+  // conversion - two roundings - and equal inputs then differ in the last bit depending on their row in the tile),
   // optional relu, one rounding to T.  The tile goes through LDS so that every lane moves 16 bytes and a store
-  // instruction covers whole rows of the C tile instead of 64 two-byte pieces: as 16-bit values, two 32-row blocks of
-  // every wavefront per pass, or - with a residual, which is added before the rounding - as fp32, one block per pass.
+  // instruction covers whole rows of the C tile instead of 64 two-byte pieces: as 16-bit values, 64 rows of every
+  // wavefront per pass, or - with a residual, which is added before the rounding - as fp32, 32 rows per pass.
   T* Ct       = reinterpret_cast<T*>(C);
   const T* Rt = reinterpret_cast<const T*>(epi.residual);
   if (Rt) Rt += (int64_t)blockIdx.y * stride_c;
@@ -592,7 +608,8 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
           for (int r = 0; r < 4; ++r) {
             const int lrow = wm * (IB * 16) + ii * 16 + 4 * (lane >> 4) + r;
             const int col  = wn * (TN * 16) + j * 16 + (lane & 15);
-            float v        = acc[IB * pass + ii][j][r] * sc[j] + sh[j];
+            float v        = __builtin_fmaf(acc[IB * pass + ii][j][r], sc[j], sh[j]);
+            asm volatile("" : "+v"(v));  // keeps the fma and the conversion apart, see above
             if (epi.relu) v = v > 0.0f ? v : 0.0f;
             *reinterpret_cast<T*>(lds + lrow * kRowBytes + col * 2) = (T)v;
           }
@@ -626,7 +643,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
         for (int r = 0; r < 4; ++r) {
           const int lrow = wm * (IB * 16) + ii * 16 + 4 * (lane >> 4) + r;
           const int col  = wn * (TN * 16) + j * 16 + (lane & 15);
-          stage[lrow * kRowFloats + col] = acc[IB * pass + ii][j][r] * sc[j] + sh[j];
+          stage[lrow * kRowFloats + col] = __builtin_fmaf(acc[IB * pass + ii][j][r], sc[j], sh[j]);
         }
     __syncthreads();
 #pragma unroll
@@ -642,7 +659,8 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
       vec8 out;
 #pragma unroll
       for (int q = 0; q < 8; ++q) {
-        float v = (q < 4 ? lo[q] : hi[q - 4]) + epi.residual_scale * (float)res[q];
+        float v = __builtin_fmaf(epi.residual_scale, (float)res[q], q < 4 ? lo[q] : hi[q - 4]);
+        asm volatile("" : "+v"(v));
         if (epi.relu) v = v > 0.0f ? v : 0.0f;
         out[q] = (T)v;
       }
