@@ -242,9 +242,10 @@ gemm16_mfma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ 
 //     no transposition in registers.
 //   * Two stages of 64 KiB and one barrier per K step, three MFMA rows (12 MFMAs) before the step's end: by then every
 //     fragment of stage s is in registers, so those rows cover the first fragment reads of stage s+1, and stage s's
-//     slot is free for the loads of stage s+2: one load per MFMA row (the rate at which the vector memory path
-//     drains them), three after the barrier and the rest in the first rows of the next step; they are waited for at
-//     the barrier of step s+1.
+//     slot is free for the loads of stage s+2, spread over the three rows after the barrier and the first rows of
+//     the next step (about the rate at which the vector memory path drains them); they are waited for at the barrier
+//     of step s+1.  Of the two wavefronts of a SIMD the older one runs ahead and then waits at the barrier: it issues
+//     the loads of both.
 //   * A fragments in a ring of four (requested three rows ahead), B fragments in two sets; scheduling barriers pin
 //     the order.  The main loop has no branches: the last one to three steps, which have nothing left to request,
 //     are peeled.
@@ -323,9 +324,13 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   constexpr int TN      = BN / WAVES_N / 16;
   constexpr int A_TILE  = BM * kD64BK * 2;    // bytes of one operand tile of a stage
   constexpr int B_TILE  = BN * kD64BK * 2;
-  constexpr int LPA     = BM / 8 / NW;        // loads (of 1 KiB per wavefront) per thread, operand and step
-  constexpr int LPB     = BN / 8 / NW;
-  static_assert(LPA >= 1 && LPB >= 1 && TM % 4 == 0 && TN == 4, "unsupported tile shape");
+  // With two wavefronts per SIMD the older one of each pair (wavefronts 0 .. NW/2-1) wins the MFMA arbitration, runs
+  // ahead and then waits at the step's barrier; it issues all the loads (their issue stalls cost it nothing), so the
+  // younger one, which the barrier waits for, has no loads to issue or wait for.
+  constexpr int LW      = (TM == 8 && !CONV) ? NW / 2 : NW;  // wavefronts that issue loads
+  constexpr int LPA     = BM / 8 / LW;                        // loads (of 1 KiB per wavefront) per thread, operand and step
+  constexpr int LPB     = BN / 8 / LW;
+  static_assert(LPA >= 1 && LPB >= 1 && LPA <= 8 && LPB <= 8 && TM % 4 == 0 && TN == 4, "unsupported tile shape");
   __shared__ __attribute__((aligned(1024))) char lds[2 * (A_TILE + B_TILE)];
   const unsigned lds_addr =
       __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) char*)lds);
@@ -360,8 +365,10 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   // [row][64 halves] tile, or 512 / BN k-rows of a [k][BN halves] tile.
   // GEMM operands: byte offset of the lane's chunk from the tile's first row (A, B stored [N][K]) or from column n0
   // of row 0 (B stored [K][N]), less the instruction offset 1024 t of load t (which the LDS address needs)
-  static_assert(LPA <= 4 && LPB <= 4, "the instruction offset of a load is below 4 KiB");
+  // (an instruction offset is below 4 KiB: loads t and t + 4 differ in m0 instead)
   unsigned a_off[LPA], b_off[LPB];
+  const bool loader = LW == NW || wave < LW;
+  const int lwave   = loader ? wave : 0;
   const char* const a_base = reinterpret_cast<const char*>(A + (int64_t)m0 * lda);
   const char* const b_base = reinterpret_cast<const char*>(B + (B_KC ? (int64_t)n0 * ldb : (int64_t)n0));
   // CONV: a_off is the byte offset of the lane's chunk at the top-left corner of the pixel's window (it may lie before
@@ -369,7 +376,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   int a_yx[LPA];
 #pragma unroll
   for (int t = 0; t < LPA; ++t) {
-    const int row = 8 * (wave * LPA + t) + (lane >> 3);
+    const int row = 8 * (lwave * LPA + t) + (lane >> 3);
     const int key = (row & 7) ^ ((row >> 3) & 1);  // chunk swizzle of a [row][64 halves] tile, see the fragment reads
     if (CONV) {
       const int pixel = m0 + row;
@@ -382,7 +389,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
       a_yx[t]         = (iy0 & 0xffff) | (ix0 << 16);
       a_off[t]        = ((unsigned)((n * geom.h + iy0) * geom.w + ix0) * (unsigned)geom.c + (((lane & 7) ^ key) << 3)) * 2u;
     } else {
-      a_off[t] = (unsigned)(((int64_t)row * lda + (((lane & 7) ^ key) << 3)) * 2 - 1024 * t);
+      a_off[t] = (unsigned)(((int64_t)row * lda + (((lane & 7) ^ key) << 3)) * 2 - 1024 * (t & 3));
     }
   }
   // CONV: filter tap and first channel of the K step whose loads are being issued (all loads of one step are issued
@@ -400,16 +407,16 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   };
 #pragma unroll
   for (int t = 0; t < LPB; ++t) {
-    const int q = wave * LPB + t;
+    const int q = lwave * LPB + t;
     if (B_KC) {
       const int row = 8 * q + (lane >> 3);
       const int key = (row & 7) ^ ((row >> 3) & 1);
-      b_off[t]      = (unsigned)(((int64_t)row * ldb + (((lane & 7) ^ key) << 3)) * 2 - 1024 * t);
+      b_off[t]      = (unsigned)(((int64_t)row * ldb + (((lane & 7) ^ key) << 3)) * 2 - 1024 * (t & 3));
     } else {
       constexpr int CH = BN / 8;  // 16-byte chunks per k-row
       const int krow   = q * (64 / CH) + lane / CH;
       const int chunk  = (lane % CH) ^ (2 * (krow & 3)) ^ (8 * ((krow >> 4) & 1));
-      b_off[t]         = (unsigned)(((int64_t)krow * ldb + (chunk << 3)) * 2 - 1024 * t);
+      b_off[t]         = (unsigned)(((int64_t)krow * ldb + (chunk << 3)) * 2 - 1024 * (t & 3));
     }
   }
   const int64_t b_step = (B_KC ? kD64BK : (int64_t)kD64BK * ldb) * 2;  // bytes per K step
@@ -425,14 +432,14 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
             ((unsigned)((tap_dy * geom.dil_h) * geom.w + tap_dx * geom.dil_w) * (unsigned)geom.c + tap_c0) * 2u;
         const char* src = inside ? reinterpret_cast<const char*>(A) + (a_off[t] + tap_off)
                                  : static_cast<const char*>(geom.zero_page) + ((lane & 7) << 4);
-        AsyncCopy16To(src, lds_addr + (unsigned)(a_tile - lds) + (wave * LPA + t) * 1024);
+        AsyncCopy16To(src, lds_addr + (unsigned)(a_tile - lds) + (lwave * LPA + t) * 1024);
       } else {
-        SetLdsBase(lds_addr + (unsigned)(a_tile - lds) + wave * LPA * 1024);
-        AsyncCopy16Slot(a_base + (int64_t)kt * (kD64BK * 2), a_off[t], t);
+        SetLdsBase(lds_addr + (unsigned)(a_tile - lds) + (lwave * LPA + (t & ~3)) * 1024);
+        AsyncCopy16Slot(a_base + (int64_t)kt * (kD64BK * 2), a_off[t], t & 3);
       }
     } else {
-      SetLdsBase(lds_addr + (unsigned)(b_tile - lds) + wave * LPB * 1024);
-      AsyncCopy16Slot(b_base + kt * b_step, b_off[t - LPA], t - LPA);
+      SetLdsBase(lds_addr + (unsigned)(b_tile - lds) + (lwave * LPB + ((t - LPA) & ~3)) * 1024);
+      AsyncCopy16Slot(b_base + kt * b_step, b_off[t - LPA], (t - LPA) & 3);
     }
   };
 
@@ -492,24 +499,30 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   // drains: EARLY loads of stage s + 2 in the three rows after the barrier of step s, the others in the first rows
   // of step s + 1.
   // A wavefront tile of 64 rows has short steps (8 rows): all its loads go into the three rows after the barrier.
-  constexpr int EPR   = TM == 4 ? 3 : 1;  // loads per row after the barrier
+  // Loader wavefronts that carry their partner's loads too issue two per row.
+  constexpr int EPR   = TM == 4 ? 3 : (LW < NW ? 2 : 1);  // loads per row: after the barrier ...
+  constexpr int LPR   = LW < NW ? 2 : 1;                  // ... and in the first rows of the next step
   constexpr int EARLY = 3 * EPR < LPA + LPB ? 3 * EPR : LPA + LPB;
   constexpr int LATE  = LPA + LPB - EARLY;
-  static_assert(LATE >= 0 && LATE <= BAR + 1, "the late loads are issued before the barrier that waits for them");
+  static_assert(LATE >= 0 && (LATE + LPR - 1) / LPR <= BAR + 1, "the late loads are issued before the barrier that waits for them");
+  // slot of a row's per-row loads that follows MFMA j (-1: none)
+#define CINN_LOAD_SLOT(P, j) ((P) == 1 ? ((j) == 3 ? 0 : -1) : (P) == 2 ? ((j) == 1 ? 0 : (j) == 3 ? 1 : -1) : (j) - 1)
   vec8 ring[4];
   vec8 bf[2][TN];
 
   const int nk = K / kD64BK;
+  if (loader) {
 #pragma unroll
-  for (int t = 0; t < LPA + LPB; ++t) issue_one(sa0, sb0, 0, t);
-  if (CONV) advance_tap();
-  if (nk > 1) {
+    for (int t = 0; t < LPA + LPB; ++t) issue_one(sa0, sb0, 0, t);
+    if (CONV) advance_tap();
+    if (nk > 1) {
 #pragma unroll
-    for (int t = 0; t < EARLY; ++t) issue_one(sa1, sb1, 1, t);
-    if (CONV && LATE == 0) advance_tap();
-    __builtin_amdgcn_s_waitcnt(0x0F70 | EARLY);  // vmcnt: stage 0 has landed, the first loads of stage 1 may be in flight
-  } else {
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      for (int t = 0; t < EARLY; ++t) issue_one(sa1, sb1, 1, t);
+      if (CONV && LATE == 0) advance_tap();
+      __builtin_amdgcn_s_waitcnt(0x0F70 | EARLY);  // vmcnt: stage 0 has landed, the first loads of stage 1 may be in flight
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    }
   }
   __syncthreads();
 #pragma unroll
@@ -517,7 +530,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 #pragma unroll
   for (int j = 0; j < TN; ++j) bf[0][j] = read_b(sb0, 0, j);
 
-#define CINN_GEMM_STEP(ACUR, BCUR, ANXT, BNXT, OFF, HAS_NEXT, HAS_LOAD)                                      \
+#define CINN_GEMM_STEP(ACUR, BCUR, ANXT, BNXT, OFF, HAS_NEXT, HAS_LOAD, DO_LOADS)                            \
   {                                                                                                          \
     const int s         = kt + OFF;                                                                          \
     const bool has_next = HAS_NEXT;                                                                          \
@@ -540,16 +553,16 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
         if ((j == 1 || j == 2) && r >= ROWS - 3 && r < ROWS - 1 && has_next) {                               \
           bf[0][(r - (ROWS - 3)) * 2 + j - 1] = read_b(BNXT, 0, (r - (ROWS - 3)) * 2 + j - 1);              \
         }                                                                                                    \
-        if (j == 3 && r < LATE) {                                                                            \
+        if (DO_LOADS && CINN_LOAD_SLOT(LPR, j) >= 0 && r * LPR + CINN_LOAD_SLOT(LPR, j) < LATE) {            \
           CINN_SB;                                                                                           \
-          if (has_next) issue_one(ANXT, BNXT, s + 1, EARLY + r);                                             \
-          if (CONV && r == LATE - 1) advance_tap(); /* stage s+1 has been requested */                       \
+          if (has_next) issue_one(ANXT, BNXT, s + 1, EARLY + r * LPR + CINN_LOAD_SLOT(LPR, j));              \
+          if (CONV && r * LPR + CINN_LOAD_SLOT(LPR, j) == LATE - 1) advance_tap(); /* s+1 requested */       \
         }                                                                                                    \
-        if ((j == 3 || (EPR == 3 && j >= 1)) && r >= ROWS - 3 &&                                             \
-            (r - (ROWS - 3)) * EPR + (EPR == 3 ? j - 1 : 0) < EARLY) {                                       \
+        if (DO_LOADS && r >= ROWS - 3 && CINN_LOAD_SLOT(EPR, j) >= 0 &&                                      \
+            (r - (ROWS - 3)) * EPR + CINN_LOAD_SLOT(EPR, j) < EARLY) {                                       \
           CINN_SB;                                                                                           \
-          if (has_load) issue_one(ACUR, BCUR, s + 2, (r - (ROWS - 3)) * EPR + (EPR == 3 ? j - 1 : 0));       \
-          if (CONV && LATE == 0 && (r - (ROWS - 3)) * EPR + (EPR == 3 ? j - 1 : 0) == EARLY - 1) advance_tap(); \
+          if (has_load) issue_one(ACUR, BCUR, s + 2, (r - (ROWS - 3)) * EPR + CINN_LOAD_SLOT(EPR, j));       \
+          if (CONV && LATE == 0 && (r - (ROWS - 3)) * EPR + CINN_LOAD_SLOT(EPR, j) == EARLY - 1) advance_tap(); \
         }                                                                                                    \
       }                                                                                                      \
       if (r == BAR && has_next) {                                                                            \
@@ -561,15 +574,25 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   }
   // pairs of steps that both have a stage after next to request: no branches around the loads; then the last one
   // to three steps with the conditions evaluated
-  int kt = 0;
-  for (; kt + 3 < nk; kt += 2) {
-    CINN_GEMM_STEP(sa0, sb0, sa1, sb1, 0, true, true)
-    CINN_GEMM_STEP(sa1, sb1, sa0, sb0, 1, true, true)
+#define CINN_GEMM_LOOP(DO_LOADS)                                                         \
+  {                                                                                      \
+    int kt = 0;                                                                          \
+    for (; kt + 3 < nk; kt += 2) {                                                       \
+      CINN_GEMM_STEP(sa0, sb0, sa1, sb1, 0, true, true, DO_LOADS)                        \
+      CINN_GEMM_STEP(sa1, sb1, sa0, sb0, 1, true, true, DO_LOADS)                        \
+    }                                                                                    \
+    for (; kt < nk; kt += 2) {                                                           \
+      CINN_GEMM_STEP(sa0, sb0, sa1, sb1, 0, s + 1 < nk, s + 2 < nk, DO_LOADS)            \
+      if (kt + 1 < nk) CINN_GEMM_STEP(sa1, sb1, sa0, sb0, 1, s + 1 < nk, s + 2 < nk, DO_LOADS) \
+    }                                                                                    \
   }
-  for (; kt < nk; kt += 2) {
-    CINN_GEMM_STEP(sa0, sb0, sa1, sb1, 0, s + 1 < nk, s + 2 < nk)
-    if (kt + 1 < nk) CINN_GEMM_STEP(sa1, sb1, sa0, sb0, 1, s + 1 < nk, s + 2 < nk)
+  if (loader) {
+    CINN_GEMM_LOOP(true)
+  } else {
+    CINN_GEMM_LOOP(false)
   }
+#undef CINN_GEMM_LOOP
+#undef CINN_LOAD_SLOT
 #undef CINN_GEMM_STEP
 #undef CINN_SB
 
