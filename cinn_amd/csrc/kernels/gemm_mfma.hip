@@ -1050,6 +1050,17 @@ bool TryDma16(const GemmProblem& p, hipStream_t stream) {
   const int64_t tiles256 = fit256 ? (int64_t)(p.m / 256) * (p.n / 256) * p.batch : 0;
   const int64_t tiles128 = fit128 ? (int64_t)(p.m / 128) * (p.n / 128) * p.batch : 0;
   static const int forced = getenv("FLAGS_cinn_hip_gemm_tile") ? atoi(getenv("FLAGS_cinn_hip_gemm_tile")) : 0;
+  // narrow outputs with B stored [N][K] (convolutions to 64 channels): 256x64 tiles on 4x1 wavefronts, two blocks per CU
+  const bool narrow = p.trans_b && p.n % 128 != 0 && p.n % 64 == 0 && p.m % 256 == 0 && forced == 0 &&
+                      (int64_t)(p.m / 256) * (p.n / 64) * p.batch >= 256;
+  if (narrow) {
+    if (p.conv) {
+      LaunchDma16<T, true, 256, 64, 4, 1, true>(p, stream);
+    } else {
+      LaunchDma16<T, true, 256, 64, 4, 1>(p, stream);
+    }
+    return true;
+  }
   if (p.conv) {
     // implicit-GEMM convolution: filters are [OC][K]
     if (!p.trans_b) return false;
@@ -1291,7 +1302,8 @@ bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream) {
   if (pointwise) {
     // measured inside ResNet-50 at batch 32: the GEMM kernels win only with at least one 128x128 tile per CU and a K
     // loop of two steps or more; smaller grids are better served by the 64x64 tiles and split K of the convolution kernel
-    if (a.c < 128 || (pixels / 128) * (a.oc / 128) < 256) return false;
+    const bool narrow = a.oc % 128 != 0 && a.oc % 64 == 0 && pixels % 256 == 0 && (pixels / 256) * (a.oc / 64) >= 256;
+    if (a.c < 128 || (!narrow && (pixels / 128) * (a.oc / 128) < 256)) return false;
     p.k = a.c;
   } else {
     // any filter, stride, padding, dilation: implicit GEMM, K = kh * kw * c with 64-channel steps inside a tap

@@ -350,6 +350,8 @@ IMPLICIT_GEMM_CASES = [
     (2, 64, 64, 64, 512, 5, 1, 2),     # 5x5 filter, two rows of padding
     (32, 64, 32, 32, 512, 3, 1, 1),    # 256 tiles of 256x256
     (32, 192, 32, 32, 512, 1, 2, 0),   # strided 1x1 (a downsampling shortcut): 3 steps inside the one tap
+    (16, 64, 64, 64, 64, 3, 1, 1),     # 64 output channels: 256 tiles of 256x64
+    (16, 128, 64, 64, 192, 3, 1, 1),   # 192 output channels: three columns of 256x64 tiles
 ]
 
 
@@ -383,11 +385,13 @@ def test_implicit_gemm_convolution_with_residual_epilogue(gpu):
 
 @pytest.mark.parametrize("dtype,tol", [("float16", 2.0 ** -10), ("bfloat16", 2.0 ** -7)])
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (0.5, 2.0)])
-def test_pointwise_convolution_on_the_gemm_kernel(gpu, dtype, tol, alpha, beta):
-    """1x1, stride 1, unpadded, 8192 pixels x 512 channels = 256 tiles of 128x128 and K = 128: the channels-last entry
-    point hands this shape to the direct-to-LDS GEMM kernel (the beta term goes through its fp32-staged epilogue).
+@pytest.mark.parametrize("shape", [(8, 128, 32, 32, 512), (16, 256, 64, 64, 64)])
+def test_pointwise_convolution_on_the_gemm_kernel(gpu, dtype, tol, alpha, beta, shape):
+    """1x1, stride 1, unpadded, 8192 pixels x 512 channels = 256 tiles of 128x128 and K = 128 (or 65536 pixels x 64
+    channels = 256 tiles of 256x64, K = 256): the channels-last entry point hands these shapes to the direct-to-LDS
+    GEMM kernel (the beta term goes through its fp32-staged epilogue).
     A 1x1 convolution is a matrix product over the channels, which the oracle confirms on one image."""
-    n, ic, h, w_, oc = 8, 128, 32, 32, 512
+    n, ic, h, w_, oc = shape
     rng = np.random.default_rng(53)
     x = round_to(rng.standard_normal((n, ic, h, w_)), dtype)
     w = round_to(rng.standard_normal((oc, ic, 1, 1)) * np.sqrt(2.0 / ic), dtype)
