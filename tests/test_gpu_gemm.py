@@ -114,7 +114,7 @@ def test_16bit_mfma_path_all_layouts(gpu, kind, ta, tb):
                                          (1, 1536, 1536, 256),   # 144 tiles of 128x128: the 4-wavefront kernel
                                          (2, 1024, 1024, 320)])  # the same with two batches, B broadcast, an odd number of K steps
 def test_16bit_direct_to_lds_kernel(gpu, kind, tb, alpha, beta, batch, m, n, k):
-    """Shapes the direct-to-LDS kernels take (A stored [M][K], K % 128 == 0, enough 256x256 or 128x128 tiles): both
+    """Shapes the direct-to-LDS kernels take (A stored [M][K], K % 64 == 0, enough 256x256 or 128x128 tiles): both
     layouts of B, the staged epilogue (beta == 0) and the read-modify-write one."""
     rng = np.random.default_rng(41)
     a = (rng.standard_normal((batch, m, k)) * 0.05).astype(np.float32)
@@ -136,6 +136,23 @@ def test_16bit_direct_to_lds_kernel(gpu, kind, tb, alpha, beta, batch, m, n, k):
     scale = abs(alpha) * (np.abs(af) @ np.abs(bm)) + abs(beta) * np.abs(cf)
     # fp32 accumulation and epilogue, one rounding to the 16-bit type
     assert np.all(np.abs(got - exact) <= ulp * np.maximum(np.abs(exact), 1e-3 * scale) + 2.0 ** -24)
+
+
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("m,n", [(4096, 3072), (1536, 1536)])
+@pytest.mark.parametrize("k", [64, 192, 448])
+def test_direct_to_lds_kernel_short_k_loops(gpu, tb, m, n, k):
+    """One, three and seven K steps on both tile sizes: the prologue alone, and the peeled last steps of the loop
+    (the steady-state part runs pairs of steps that still have a stage to request)."""
+    rng = np.random.default_rng(47 + k)
+    a = (rng.standard_normal((1, m, k)) * 0.05).astype(np.float16)
+    b = (rng.standard_normal((1, n, k) if tb else (1, k, n)) * 0.05).astype(np.float16)
+    got = call_cublas(a, b, (1, m, n), "float16", False, tb).astype(np.float64)
+    af, bf = a.astype(np.float64), b.astype(np.float64)
+    bm = np.swapaxes(bf, 1, 2) if tb else bf
+    exact = af @ bm
+    scale = np.abs(af) @ np.abs(bm)
+    assert np.all(np.abs(got - exact) <= 2.0 ** -10 * np.maximum(np.abs(exact), 1e-3 * scale) + 2.0 ** -24)
 
 
 @pytest.mark.parametrize("kind", ["float32", "float16", "bfloat16"])
