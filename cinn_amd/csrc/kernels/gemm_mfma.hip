@@ -240,7 +240,7 @@ gemm16_mfma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ 
 //   * B stored [K][N] (the plain row-major matmul) is kept as [k][n] in LDS ([64 k][512 B], a load instruction
 //     covers 2 k-rows) and read with ds_read_b64_tr_b16, which hands every lane four consecutive k of one column -
 //     no transposition in registers.
-//   * Two stages of 64 KiB and one barrier per K step, three MFMA rows (12 MFMAs) before the step's end: by then every
+//   * NS stages (two of 64 KiB for the 256x256 tile) and one barrier per K step, three MFMA rows (12 MFMAs) before the step's end: by then every
 //     fragment of stage s is in registers, so those rows cover the first fragment reads of stage s+1, and stage s's
 //     slot is free for the loads of stage s+2, spread over the three rows after the barrier and the first rows of
 //     the next step (about the rate at which the vector memory path drains them); they are waited for at the barrier
@@ -313,7 +313,7 @@ struct ConvGeom {
 
 // BM x BN block tile on a WAVES_M x WAVES_N grid of wavefronts: 256x256 on 2x4 (8 wavefronts of 128x64) for large
 // problems, 128x128 on 2x2 (4 wavefronts of 64x64, two blocks per CU) when 256x256 tiles would leave CUs idle.
-template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false>
+template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false, int NS = 2>
 __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N)
 gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* C, int M, int N, int K,
                   int64_t lda, int64_t ldb, int64_t ldc, DmaEpilogue epi, int64_t stride_a, int64_t stride_b,
@@ -331,13 +331,14 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   constexpr int LPA     = BM / 8 / LW;                        // loads (of 1 KiB per wavefront) per thread, operand and step
   constexpr int LPB     = BN / 8 / LW;
   static_assert(LPA >= 1 && LPB >= 1 && LPA <= 8 && LPB <= 8 && TM % 4 == 0 && TN == 4, "unsupported tile shape");
-  __shared__ __attribute__((aligned(1024))) char lds[2 * (A_TILE + B_TILE)];
+  constexpr int STAGE = A_TILE + B_TILE;
+  static_assert(NS >= 2 && NS * STAGE <= 160 * 1024, "the stages do not fit LDS");
+  __shared__ __attribute__((aligned(1024))) char lds[NS * STAGE];
   const unsigned lds_addr =
       __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) char*)lds);
-  char* const sa0 = lds;
-  char* const sb0 = lds + A_TILE;
-  char* const sa1 = lds + A_TILE + B_TILE;
-  char* const sb1 = lds + 2 * A_TILE + B_TILE;
+  // stage s lives in slot s % NS
+  auto sa = [&](int slot) -> char* { return lds + slot * STAGE; };
+  auto sb = [&](int slot) -> char* { return lds + slot * STAGE + A_TILE; };
   typedef typename Half16<T>::vec8 vec8;
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
@@ -511,29 +512,42 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   vec8 bf[2][TN];
 
   const int nk = K / kD64BK;
+  constexpr int L = LPA + LPB;  // loads of a loader wavefront per stage
+  // vmcnt(n): at most n of the wavefront's loads still in flight; they complete in the order they were issued
+#define CINN_VMCNT(n) ((((n) & 15) | (((n) >> 4) << 14)) | 0x0F70)
   if (loader) {
 #pragma unroll
-    for (int t = 0; t < LPA + LPB; ++t) issue_one(sa0, sb0, 0, t);
-    if (CONV) advance_tap();
-    if (nk > 1) {
+    for (int st = 0; st < NS - 1; ++st) {
+      if (st < nk) {
 #pragma unroll
-      for (int t = 0; t < EARLY; ++t) issue_one(sa1, sb1, 1, t);
+        for (int t = 0; t < L; ++t) issue_one(sa(st), sb(st), st, t);
+        if (CONV) advance_tap();
+      }
+    }
+    if (nk > NS - 1) {
+#pragma unroll
+      for (int t = 0; t < EARLY; ++t) issue_one(sa(NS - 1), sb(NS - 1), NS - 1, t);
       if (CONV && LATE == 0) advance_tap();
-      __builtin_amdgcn_s_waitcnt(0x0F70 | EARLY);  // vmcnt: stage 0 has landed, the first loads of stage 1 may be in flight
+      __builtin_amdgcn_s_waitcnt(CINN_VMCNT((NS - 2) * L + EARLY));  // stage 0 has landed, later ones may be in flight
     } else {
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     }
   }
   __syncthreads();
 #pragma unroll
-  for (int i = 0; i < 3; ++i) ring[i] = read_a(sa0, 0, i);
+  for (int i = 0; i < 3; ++i) ring[i] = read_a(sa(0), 0, i);
 #pragma unroll
-  for (int j = 0; j < TN; ++j) bf[0][j] = read_b(sb0, 0, j);
+  for (int j = 0; j < TN; ++j) bf[0][j] = read_b(sb(0), 0, j);
 
-#define CINN_GEMM_STEP(ACUR, BCUR, ANXT, BNXT, OFF, HAS_NEXT, HAS_LOAD, DO_LOADS)                            \
+  // Step u of a group of NS (slot of its stage: u).  After its barrier the slot is free for stage s + NS: the first
+  // EARLY loads go out in the three rows after the barrier, the others in the first rows of step s + 1 (there: stage
+  // s + NS - 1 into slot u - 1).  WAIT: the s_waitcnt before the barrier; in the steady state the NS - 2 stages
+  // requested after stage s + 1 may stay in flight.
+#define CINN_GEMM_STEP(U, HAS_NEXT, HAS_LATE, HAS_LOAD, DO_LOADS, WAIT)                                       \
   {                                                                                                          \
-    const int s         = kt + OFF;                                                                          \
+    const int s         = kt + U;                                                                            \
     const bool has_next = HAS_NEXT;                                                                          \
+    const bool has_late = HAS_LATE;                                                                          \
     const bool has_load = HAS_LOAD;                                                                          \
     _Pragma("unroll") for (int r = 0; r < ROWS; ++r) {                                                       \
       _Pragma("unroll") for (int j = 0; j < TN; ++j) {                                                       \
@@ -542,49 +556,54 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
         CINN_SB;                                                                                             \
         if (j == 0) {                                                                                        \
           if (r + 3 < ROWS) {                                                                                \
-            ring[(r + 3) % 4] = read_a(ACUR, (r + 3) / TM, (r + 3) % TM);                                    \
+            ring[(r + 3) % 4] = read_a(sa(U), (r + 3) / TM, (r + 3) % TM);                                   \
           } else if (has_next) {                                                                             \
-            ring[(r + 3) % 4] = read_a(ANXT, 0, r + 3 - ROWS);                                               \
+            ring[(r + 3) % 4] = read_a(sa((U + 1) % NS), 0, r + 3 - ROWS);                                   \
           }                                                                                                  \
         }                                                                                                    \
         if ((j == 1 || j == 2) && r >= TM / 2 - 2 && r < TM / 2) {                                           \
-          bf[1][(r - (TM / 2 - 2)) * 2 + j - 1] = read_b(BCUR, 1, (r - (TM / 2 - 2)) * 2 + j - 1);          \
+          bf[1][(r - (TM / 2 - 2)) * 2 + j - 1] = read_b(sb(U), 1, (r - (TM / 2 - 2)) * 2 + j - 1);         \
         }                                                                                                    \
         if ((j == 1 || j == 2) && r >= ROWS - 3 && r < ROWS - 1 && has_next) {                               \
-          bf[0][(r - (ROWS - 3)) * 2 + j - 1] = read_b(BNXT, 0, (r - (ROWS - 3)) * 2 + j - 1);              \
+          bf[0][(r - (ROWS - 3)) * 2 + j - 1] = read_b(sb((U + 1) % NS), 0, (r - (ROWS - 3)) * 2 + j - 1);  \
         }                                                                                                    \
         if (DO_LOADS && CINN_LOAD_SLOT(LPR, j) >= 0 && r * LPR + CINN_LOAD_SLOT(LPR, j) < LATE) {            \
           CINN_SB;                                                                                           \
-          if (has_next) issue_one(ANXT, BNXT, s + 1, EARLY + r * LPR + CINN_LOAD_SLOT(LPR, j));              \
-          if (CONV && r * LPR + CINN_LOAD_SLOT(LPR, j) == LATE - 1) advance_tap(); /* s+1 requested */       \
+          if (has_late)                                                                                      \
+            issue_one(sa((U + NS - 1) % NS), sb((U + NS - 1) % NS), s + NS - 1,                              \
+                      EARLY + r * LPR + CINN_LOAD_SLOT(LPR, j));                                             \
+          if (CONV && r * LPR + CINN_LOAD_SLOT(LPR, j) == LATE - 1) advance_tap(); /* that stage is requested */ \
         }                                                                                                    \
         if (DO_LOADS && r >= ROWS - 3 && CINN_LOAD_SLOT(EPR, j) >= 0 &&                                      \
             (r - (ROWS - 3)) * EPR + CINN_LOAD_SLOT(EPR, j) < EARLY) {                                       \
           CINN_SB;                                                                                           \
-          if (has_load) issue_one(ACUR, BCUR, s + 2, (r - (ROWS - 3)) * EPR + CINN_LOAD_SLOT(EPR, j));       \
+          if (has_load) issue_one(sa(U), sb(U), s + NS, (r - (ROWS - 3)) * EPR + CINN_LOAD_SLOT(EPR, j));    \
           if (CONV && LATE == 0 && (r - (ROWS - 3)) * EPR + CINN_LOAD_SLOT(EPR, j) == EARLY - 1) advance_tap(); \
         }                                                                                                    \
       }                                                                                                      \
       if (r == BAR && has_next) {                                                                            \
         CINN_SB;                                                                                             \
-        __builtin_amdgcn_s_waitcnt(0x0070); /* vmcnt(0) lgkmcnt(0): stage s+1 landed, fragments arrived */   \
+        __builtin_amdgcn_s_waitcnt(WAIT); /* stage s+1 landed (vmcnt), fragments arrived (lgkmcnt(0)) */     \
         __syncthreads();                                                                                     \
       }                                                                                                      \
     }                                                                                                        \
   }
-  // pairs of steps that both have a stage after next to request: no branches around the loads; then the last one
-  // to three steps with the conditions evaluated
-#define CINN_GEMM_LOOP(DO_LOADS)                                                         \
-  {                                                                                      \
-    int kt = 0;                                                                          \
-    for (; kt + 3 < nk; kt += 2) {                                                       \
-      CINN_GEMM_STEP(sa0, sb0, sa1, sb1, 0, true, true, DO_LOADS)                        \
-      CINN_GEMM_STEP(sa1, sb1, sa0, sb0, 1, true, true, DO_LOADS)                        \
-    }                                                                                    \
-    for (; kt < nk; kt += 2) {                                                           \
-      CINN_GEMM_STEP(sa0, sb0, sa1, sb1, 0, s + 1 < nk, s + 2 < nk, DO_LOADS)            \
-      if (kt + 1 < nk) CINN_GEMM_STEP(sa1, sb1, sa0, sb0, 1, s + 1 < nk, s + 2 < nk, DO_LOADS) \
-    }                                                                                    \
+  // groups of NS steps that all have a stage to request: no branches around the loads; then the last steps with
+  // the conditions evaluated and every load waited for
+  constexpr int kSteadyWait = CINN_VMCNT((NS - 2) * L) & ~0x0F00;
+#define CINN_GEMM_LOOP(DO_LOADS)                                                                              \
+  {                                                                                                          \
+    int kt = 0;                                                                                              \
+    for (; kt + 2 * NS - 1 < nk; kt += NS) {                                                                 \
+      _Pragma("unroll") for (int u = 0; u < NS; ++u) {                                                       \
+        CINN_GEMM_STEP(u, true, true, true, DO_LOADS, kSteadyWait)                                           \
+      }                                                                                                      \
+    }                                                                                                        \
+    for (; kt < nk; kt += NS) {                                                                              \
+      _Pragma("unroll") for (int u = 0; u < NS; ++u) {                                                       \
+        if (kt + u < nk) CINN_GEMM_STEP(u, s + 1 < nk, s + NS - 1 < nk, s + NS < nk, DO_LOADS, 0x0070)       \
+      }                                                                                                      \
+    }                                                                                                        \
   }
   if (loader) {
     CINN_GEMM_LOOP(true)
@@ -592,6 +611,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     CINN_GEMM_LOOP(false)
   }
 #undef CINN_GEMM_LOOP
+#undef CINN_VMCNT
 #undef CINN_LOAD_SLOT
 #undef CINN_GEMM_STEP
 #undef CINN_SB
@@ -618,7 +638,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     constexpr int kRowBytes = (BN + 8) * 2;
     constexpr int IB        = 4;  // 16-row blocks per wavefront and pass: 64 rows
     constexpr int PASS_ROWS = WAVES_M * IB * 16;
-    static_assert(PASS_ROWS * kRowBytes <= 2 * (A_TILE + B_TILE), "the staged result does not fit the operand stages");
+    static_assert(PASS_ROWS * kRowBytes <= NS * STAGE, "the staged result does not fit the operand stages");
     static_assert(PASS_ROWS * CPR % THREADS == 0, "the copy-out loop assumes whole rounds");
 #pragma unroll
     for (int pass = 0; pass < TM / IB; ++pass) {
@@ -652,7 +672,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   constexpr int kRowFloats = BN + 4;
   constexpr int IB         = 2;  // 16-row blocks per wavefront and pass: 32 rows of fp32
   constexpr int PASS_ROWS  = WAVES_M * IB * 16;
-  static_assert(PASS_ROWS * kRowFloats * 4 <= 2 * (A_TILE + B_TILE), "the staged result does not fit the operand stages");
+  static_assert(PASS_ROWS * kRowFloats * 4 <= NS * STAGE, "the staged result does not fit the operand stages");
   static_assert(PASS_ROWS * CPR % THREADS == 0, "the copy-out loop assumes whole rounds");
   float* stage = reinterpret_cast<float*>(lds);
 #pragma unroll
@@ -1016,7 +1036,7 @@ void XcdRectangles(int tiles_m, int tiles_n, int* xcd_cols, int* sub_rows, int* 
   }
 }
 
-template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false>
+template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false, int NS = 2>
 void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
   int64_t ldb = p.trans_b ? p.k : p.n;
   const int tiles_m = p.m / BM, tiles_n = p.n / BN;
@@ -1032,7 +1052,7 @@ void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
   epi.residual_scale = p.residual ? p.residual_scale : p.beta;
   ConvGeom geom{};
   if (CONV) geom = *p.conv;
-  hipLaunchKernelGGL((gemm16_dma_kernel<T, B_KC, BM, BN, WAVES_M, WAVES_N, CONV>), grid, dim3(64 * WAVES_M * WAVES_N), 0,
+  hipLaunchKernelGGL((gemm16_dma_kernel<T, B_KC, BM, BN, WAVES_M, WAVES_N, CONV, NS>), grid, dim3(64 * WAVES_M * WAVES_N), 0,
                      stream, static_cast<const uint16_t*>(p.a), static_cast<const uint16_t*>(p.b),
                      static_cast<uint16_t*>(p.c), p.m, p.n, p.k, (int64_t)p.k, ldb, (int64_t)p.n, epi, p.stride_a,
                      p.stride_b, p.stride_c, xcd_cols, sub_rows, sub_cols, geom);
@@ -1053,8 +1073,19 @@ bool TryDma16(const GemmProblem& p, hipStream_t stream) {
   // narrow outputs with B stored [N][K] (convolutions to 64 channels): 256x64 tiles on 4x1 wavefronts, two blocks per CU
   const bool narrow = p.trans_b && p.n % 128 != 0 && p.n % 64 == 0 && p.m % 256 == 0 && forced == 0 &&
                       (int64_t)(p.m / 256) * (p.n / 64) * p.batch >= 256;
+  // 128x128 tiles keep two stages of 32 KiB and two blocks per CU, or - when there is at most one block per CU
+  // anyway - four stages: three K steps of loads in flight instead of one (2048^3: 27.8 -> 21.9 us; with more
+  // blocks than CUs two blocks of two stages are faster).  FLAGS_cinn_hip_gemm_stages = 2 / 4 forces one form.
+  static const int forced_stages = getenv("FLAGS_cinn_hip_gemm_stages") ? atoi(getenv("FLAGS_cinn_hip_gemm_stages")) : 0;
+  const int stages = forced_stages ? forced_stages : (tiles128 > 0 && tiles128 <= 256 ? 4 : 2);
   if (narrow) {
-    if (p.conv) {
+    if (forced_stages == 4) {
+      if (p.conv) {
+        LaunchDma16<T, true, 256, 64, 4, 1, true, 4>(p, stream);
+      } else {
+        LaunchDma16<T, true, 256, 64, 4, 1, false, 4>(p, stream);
+      }
+    } else if (p.conv) {
       LaunchDma16<T, true, 256, 64, 4, 1, true>(p, stream);
     } else {
       LaunchDma16<T, true, 256, 64, 4, 1>(p, stream);
@@ -1072,7 +1103,11 @@ bool TryDma16(const GemmProblem& p, hipStream_t stream) {
     // convolution kernel are faster (19 against 26 us at 196 tiles, K = 1152) unless K is long (68 against 74 us at
     // 196 tiles, K = 4608)
     if (tiles128 >= 256 || (tiles128 >= 128 && p.k >= 4096) || (forced == 128 && tiles128 > 0)) {
-      LaunchDma16<T, true, 128, 128, 2, 2, true>(p, stream);
+      if (stages == 4) {
+        LaunchDma16<T, true, 128, 128, 2, 2, true, 4>(p, stream);
+      } else {
+        LaunchDma16<T, true, 128, 128, 2, 2, true>(p, stream);
+      }
       return true;
     }
     return false;
@@ -1086,7 +1121,13 @@ bool TryDma16(const GemmProblem& p, hipStream_t stream) {
     return true;
   }
   if ((tiles128 >= 128 && forced != 256) || (forced == 128 && tiles128 > 0)) {
-    if (p.trans_b) {
+    if (stages == 4) {
+      if (p.trans_b) {
+        LaunchDma16<T, true, 128, 128, 2, 2, false, 4>(p, stream);
+      } else {
+        LaunchDma16<T, false, 128, 128, 2, 2, false, 4>(p, stream);
+      }
+    } else if (p.trans_b) {
       LaunchDma16<T, true, 128, 128, 2, 2>(p, stream);
     } else {
       LaunchDma16<T, false, 128, 128, 2, 2>(p, stream);

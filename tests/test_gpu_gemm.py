@@ -111,7 +111,8 @@ def test_16bit_mfma_path_all_layouts(gpu, kind, ta, tb):
 @pytest.mark.parametrize("tb", [False, True])
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (0.5, 2.0)])
 @pytest.mark.parametrize("batch,m,n,k", [(1, 4096, 3072, 128),   # 192 tiles of 256x256: the 8-wavefront kernel
-                                         (1, 1536, 1536, 256),   # 144 tiles of 128x128: the 4-wavefront kernel
+                                         (1, 1536, 1536, 256),   # 144 tiles of 128x128: the 4-wavefront kernel, four stages
+                                         (1, 2304, 2304, 192),   # 324 tiles of 128x128: two stages, two blocks per CU
                                          (2, 1024, 1024, 320)])  # the same with two batches, B broadcast, an odd number of K steps
 def test_16bit_direct_to_lds_kernel(gpu, kind, tb, alpha, beta, batch, m, n, k):
     """Shapes the direct-to-LDS kernels take (A stored [M][K], K % 64 == 0, enough 256x256 or 128x128 tiles): both
