@@ -3,9 +3,10 @@
 //   C[M,N] = alpha * op(A)[M,K] * op(B)[K,N] + beta * C          (row-major, optional batch)
 //
 // Kernels:
-//   * gemm16_dma_kernel   - bf16 / fp16 with A stored [M][K] (the common case) and K % 64 == 0: 256x256x64 tile, 512
-//     threads, direct global -> LDS loads of whole 128-byte lines into two stages, transposing LDS reads for
-//     row-major B; see the comment at the kernel.
+//   * gemm16_dma_kernel   - bf16 / fp16 with A stored [M][K] (the common case) and K % 64 == 0, on
+//     v_mfma_f32_16x16x32: 256x256x64 tile, 512 threads, direct global -> LDS loads of whole 128-byte lines into two
+//     stages, transposing LDS reads for row-major B; also as 128x128 tiles (two or four stages) and 256x64 tiles, and
+//     with the A operand gathered from a channels-last image (implicit-GEMM convolution); see the comment at the kernel.
 //   * gemm16_mfma_kernel  - bf16 / fp16 inputs, any operand layout (used for transposed A), fp32 accumulation on v_mfma_f32_32x32x16_{bf16,f16}.
 //     256x256 block tile, 64-deep K step, 256 threads = 4 wavefronts in a 2x2 grid, each wavefront owning a
 //     128x128 tile (16 MFMA accumulator tiles = 256 accumulator registers).  Both operand tiles live in LDS
