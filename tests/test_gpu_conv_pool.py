@@ -249,7 +249,7 @@ def test_matmul_of_a_matrix_with_itself(gpu):
 
 
 # ---- the channels-last kernels through the C-ABI (tensor formats 1 and 2 of cinn_call_cudnn_conv2d_forward) --------
-def call_conv_nhwc(x_nchw, w_oihw, stride, pad, fmt, dtype, alpha=1.0, beta=0.0, y_init=None):
+def call_conv_nhwc(x_nchw, w_oihw, stride, pad, fmt, dtype, alpha=1.0, beta=0.0, y_init=None, dilation=1):
     """x / w are fp32 arrays in NCHW / OIHW; they are converted to `dtype` and to the layout `fmt` asks for.
     Returns the output as fp32 NCHW."""
     from cinn_amd.common import bfloat16_bits_to_float32, float32_to_bfloat16_bits
@@ -258,8 +258,8 @@ def call_conv_nhwc(x_nchw, w_oihw, stride, pad, fmt, dtype, alpha=1.0, beta=0.0,
                                                    ctypes.c_float] + [ctypes.c_int] * 19 + [ctypes.c_void_p]
     n, ic, ih, iw = x_nchw.shape
     oc, _, kh, kw = w_oihw.shape
-    oh = oracle.conv_out_dim(ih, kh, pad, stride, 1)
-    ow = oracle.conv_out_dim(iw, kw, pad, stride, 1)
+    oh = oracle.conv_out_dim(ih, kh, pad, stride, dilation)
+    ow = oracle.conv_out_dim(iw, kw, pad, stride, dilation)
 
     def to_dev(a):
         a = np.ascontiguousarray(a)
@@ -275,7 +275,7 @@ def call_conv_nhwc(x_nchw, w_oihw, stride, pad, fmt, dtype, alpha=1.0, beta=0.0,
     Y.copy_from(to_dev(y0.transpose(0, 2, 3, 1)))
     args = runtime.pod_args([X, W, Y])
     lib.cinn_call_cudnn_conv2d_forward(args, 3, fmt, alpha, beta, n, ic, ih, iw, oc, ic, kh, kw, pad, pad, stride, stride,
-                                       1, 1, 1, n, oc, oh, ow, None)
+                                       dilation, dilation, 1, n, oc, oh, ow, None)
     runtime.synchronize()
     out = Y.numpy()
     out = bfloat16_bits_to_float32(out) if dtype == "bfloat16" else out.astype(np.float32)
@@ -367,6 +367,21 @@ def test_convolution_as_implicit_gemm(gpu, case, dtype, tol):
     got = call_conv_nhwc(x, w, s, p, 1, dtype)
     want = oracle.conv2d_nchw(x, w, (s, s), (p, p))
     scale = oracle.conv2d_nchw(np.abs(x), np.abs(w), (s, s), (p, p))
+    assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+
+
+@pytest.mark.parametrize("dtype,tol", [("float16", 1e-2), ("bfloat16", 2e-2)])
+def test_implicit_gemm_convolution_with_dilation(gpu, dtype, tol):
+    """3x3 filter with dilation 2 and padding 2 (the output keeps the input's extent): taps two pixels apart, windows
+    that start two pixels outside the image."""
+    n, ic, h, w_, oc = 8, 64, 32, 32, 512
+    rng = np.random.default_rng(101)
+    x = round_to(rng.standard_normal((n, ic, h, w_)), dtype)
+    w = round_to(rng.standard_normal((oc, ic, 3, 3)) * np.sqrt(2.0 / (ic * 9)), dtype)
+    got = call_conv_nhwc(x, w, 1, 2, 1, dtype, dilation=2)
+    want = oracle.conv2d_nchw(x, w, (1, 1), (2, 2), (2, 2))
+    scale = oracle.conv2d_nchw(np.abs(x), np.abs(w), (1, 1), (2, 2), (2, 2))
+    assert got.shape == want.shape
     assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
 
 
