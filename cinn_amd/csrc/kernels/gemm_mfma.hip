@@ -765,8 +765,11 @@ gemm32_mfma_kernel(const float* __restrict__ A, const float* __restrict__ B, flo
   // Each thread stages EL4 groups of 4 floats of either operand per K step, 16 bytes per access.  An operand whose
   // contiguous axis is k is fetched as 8 rows x 128 bytes per wavefront access (whole lines) and scattered into
   // [k][row]; one whose contiguous axis is the row index is copied as it is.
+  // The staging registers are a ring of PF steps: the loads of step kt + PF are issued in step kt, so that PF - 1 steps
+  // of MFMAs cover their latency (a 64x64 tile's step is short: 8 MFMAs per wavefront).
   constexpr int EL4 = TILE * KS / 4 / THREADS;
-  f32x4 ra[EL4], rb[EL4];
+  constexpr int PF  = TILE == 64 ? 4 : 2;
+  f32x4 ra[PF][EL4], rb[PF][EL4];
   auto load_one = [&](const float* __restrict__ P, int64_t ld, int row0, int k0, bool k_contig, int i) -> f32x4 {
     const int u = tid + THREADS * i;
     if (k_contig) {
@@ -787,46 +790,62 @@ gemm32_mfma_kernel(const float* __restrict__ A, const float* __restrict__ B, flo
       *reinterpret_cast<f32x4*>(&S[k][c * 4]) = v;
     }
   };
-  auto load_tiles = [&](int k0) {
+  auto load_tiles = [&](int slot, int k0) {
 #pragma unroll
     for (int i = 0; i < EL4; ++i) {
-      ra[i] = load_one(A, lda, m0, k0, !TRANS_A, i);
-      rb[i] = load_one(B, ldb, n0, k0, TRANS_B, i);
+      ra[slot][i] = load_one(A, lda, m0, k0, !TRANS_A, i);
+      rb[slot][i] = load_one(B, ldb, n0, k0, TRANS_B, i);
     }
   };
-  auto store_tiles = [&](int buf) {
+  auto store_tiles = [&](int slot, int buf) {
 #pragma unroll
     for (int i = 0; i < EL4; ++i) {
-      store_one(As[buf], !TRANS_A, i, ra[i]);
-      store_one(Bs[buf], TRANS_B, i, rb[i]);
+      store_one(As[buf], !TRANS_A, i, ra[slot][i]);
+      store_one(Bs[buf], TRANS_B, i, rb[slot][i]);
     }
   };
 
   const int kt_count = K / KS;
-  load_tiles(0);
-  store_tiles(0);
+#pragma unroll
+  for (int d = 0; d < PF; ++d)
+    if (d < kt_count) load_tiles(d, d * KS);
+  store_tiles(0, 0);
   __syncthreads();
-  for (int kt = 0; kt < kt_count; ++kt) {
-    const int cur  = kt & 1;
-    const bool more = kt + 1 < kt_count;
-    if (more) load_tiles((kt + 1) * KS);
-#pragma unroll
-    for (int kp = 0; kp < KS / 2 / KSPLIT; ++kp) {
-      const int k = 2 * (kp * KSPLIT + kgrp) + (lane >> 5);
-      float af[TT], bf[TT];
-#pragma unroll
-      for (int t = 0; t < TT; ++t) {
-        af[t] = As[cur][k][wm * (TILE / 2) + t * 32 + (lane & 31)];
-        bf[t] = Bs[cur][k][wn * (TILE / 2) + t * 32 + (lane & 31)];
-      }
-#pragma unroll
-      for (int i = 0; i < TT; ++i)
-#pragma unroll
-        for (int j = 0; j < TT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
-    }
-    if (more) store_tiles(cur ^ 1);
-    __syncthreads();
+  // one K step: refill ring slot u (it went into LDS at the end of the previous step), all fragment reads of the step,
+  // then its MFMAs, then the next step's registers into the other LDS buffer
+#define CINN_GEMM32_STEP(U, REFILL, NEXT)                                                                   \
+  {                                                                                                         \
+    const int kt  = kt0 + U;                                                                                \
+    const int cur = U & 1; /* PF is even */                                                                 \
+    if (REFILL) load_tiles(U, (kt + PF) * KS);                                                              \
+    constexpr int KP = KS / 2 / KSPLIT;                                                                     \
+    float af[KP][TT], bf[KP][TT];                                                                           \
+    _Pragma("unroll") for (int kp = 0; kp < KP; ++kp) {                                                     \
+      const int k = 2 * (kp * KSPLIT + kgrp) + (lane >> 5);                                                 \
+      _Pragma("unroll") for (int t = 0; t < TT; ++t) {                                                      \
+        af[kp][t] = As[cur][k][wm * (TILE / 2) + t * 32 + (lane & 31)];                                     \
+        bf[kp][t] = Bs[cur][k][wn * (TILE / 2) + t * 32 + (lane & 31)];                                     \
+      }                                                                                                     \
+    }                                                                                                       \
+    _Pragma("unroll") for (int kp = 0; kp < KP; ++kp)                                                       \
+      _Pragma("unroll") for (int i = 0; i < TT; ++i)                                                        \
+        _Pragma("unroll") for (int j = 0; j < TT; ++j)                                                      \
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[kp][i], bf[kp][j], acc[i][j], 0, 0, 0);       \
+    if (NEXT) store_tiles((U + 1) % PF, cur ^ 1);                                                           \
+    __syncthreads();                                                                                        \
   }
+  // groups of PF steps that all have a step to request (no conditions inside), then the last steps
+  int kt0 = 0;
+  for (; kt0 + 2 * PF <= kt_count; kt0 += PF) {
+#pragma unroll
+    for (int u = 0; u < PF; ++u) CINN_GEMM32_STEP(u, true, true)
+  }
+  for (; kt0 < kt_count; kt0 += PF) {
+#pragma unroll
+    for (int u = 0; u < PF; ++u)
+      if (kt0 + u < kt_count) CINN_GEMM32_STEP(u, kt + PF < kt_count, kt + 1 < kt_count)
+  }
+#undef CINN_GEMM32_STEP
   if (KSPLIT == 2) {
     // the last barrier of the loop has passed: the operand tiles are no longer read
     static_assert(KSPLIT == 1 || TT == 1, "the partial tile exchange assumes one accumulator tile per wavefront");
