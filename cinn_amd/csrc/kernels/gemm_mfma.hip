@@ -298,6 +298,7 @@ struct DmaEpilogue {
   float alpha;
   float residual_scale;
   int relu;
+  int streaming;          // store the result with non-temporal stores (large outputs nobody re-reads from L2)
 };
 
 // Implicit-GEMM view of a channels-last convolution for gemm16_dma_kernel<.., CONV = true>: row m of A is output pixel
@@ -665,7 +666,15 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
         const int c16   = chunk % CPR;
         const int row   = m0 + (lrow / (IB * 16)) * (TM * 16) + pass * (IB * 16) + lrow % (IB * 16);
         const u32x4 v   = *reinterpret_cast<const u32x4*>(lds + lrow * kRowBytes + c16 * 16);
-        *reinterpret_cast<u32x4*>(Ct + (int64_t)row * ldc + n0 + c16 * 8) = v;
+        // streaming stores: results that do not sit dirty in L2 shorten the write-back at the end of the kernel
+        // (4096^3 2 %, 8192^3 3.6 % faster); a convolution inside a network keeps its output cached for the next
+        // layer instead (ResNet-50 0.4 % slower with streaming stores)
+        u32x4* dst = reinterpret_cast<u32x4*>(Ct + (int64_t)row * ldc + n0 + c16 * 8);
+        if (epi.streaming) {
+          __builtin_nontemporal_store(v, dst);
+        } else {
+          *dst = v;
+        }
       }
     }
     return;
@@ -708,7 +717,11 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
         if (epi.relu) v = v > 0.0f ? v : 0.0f;
         out[q] = (T)v;
       }
-      *reinterpret_cast<vec8*>(Ct + o) = out;
+      if (epi.streaming) {
+        __builtin_nontemporal_store(out, reinterpret_cast<vec8*>(Ct + o));
+      } else {
+        *reinterpret_cast<vec8*>(Ct + o) = out;
+      }
     }
   }
 }
@@ -1022,6 +1035,8 @@ struct GemmProblem {
   bool relu{false};
   // A is the input of a channels-last convolution (implicit GEMM), not a matrix
   const ConvGeom* conv{nullptr};
+  // the result is a layer's activation: leave it in L2 for the next kernel
+  bool keep_in_cache{false};
 };
 
 template <typename T, bool A_KC, bool B_KC>
@@ -1070,6 +1085,8 @@ void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
   epi.relu           = p.relu ? 1 : 0;
   epi.residual       = p.residual ? p.residual : (p.beta != 0.0f ? p.c : nullptr);
   epi.residual_scale = p.residual ? p.residual_scale : p.beta;
+  // plain GEMMs whose result exceeds half of the L2 capacity (8 x 4 MiB) stream it out
+  epi.streaming = !p.keep_in_cache && (int64_t)p.batch * p.m * p.n * 2 >= (16 << 20);
   ConvGeom geom{};
   if (CONV) geom = *p.conv;
   hipLaunchKernelGGL((gemm16_dma_kernel<T, B_KC, BM, BN, WAVES_M, WAVES_N, CONV, NS>), grid, dim3(64 * WAVES_M * WAVES_N), 0,
@@ -1397,6 +1414,7 @@ bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream) {
   p.residual       = a.residual;
   p.residual_scale = a.residual_scale;
   p.relu           = a.relu;
+  p.keep_in_cache  = true;
   const bool taken = is_bf16 ? TryDma16<__bf16>(p, stream) : TryDma16<_Float16>(p, stream);
   if (taken) CINN_HIP_CALL(hipGetLastError());
   return taken;
