@@ -354,12 +354,13 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     tile_row = (xcd / xcd_cols) * sub_rows + idx / sub_cols;
     tile_col = (xcd % xcd_cols) * sub_cols + idx % sub_cols;
   } else {
-    const int tiles_n = N / BN;
+    const int tiles_n = (N + BN - 1) / BN;
     tile_row = blockIdx.x / tiles_n;
     tile_col = blockIdx.x % tiles_n;
   }
   const int m0 = tile_row * BM;
   const int n0 = tile_col * BN;
+  if (m0 >= M || n0 >= N) return;  // padding of the XCD rectangles (the whole block leaves)
   A += (int64_t)blockIdx.y * stride_a;
   B += (int64_t)blockIdx.y * stride_b;
   C += (int64_t)blockIdx.y * stride_c;
@@ -372,8 +373,14 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   unsigned a_off[LPA], b_off[LPB];
   const bool loader = LW == NW || wave < LW;
   const int lwave   = loader ? wave : 0;
-  const char* const a_base = reinterpret_cast<const char*>(A + (int64_t)m0 * lda);
-  const char* const b_base = reinterpret_cast<const char*>(B + (B_KC ? (int64_t)n0 * ldb : (int64_t)n0));
+  // The last tile row / column may reach beyond M / N: its lanes fetch the last valid row (or 8-column chunk)
+  // instead - what they compute is not stored.  The bases lie kBias bytes below the tile and every lane offset
+  // includes kBias, so that an offset less its instruction offset never wraps below zero.
+  constexpr int kBias = 4096;
+  const char* const a_base = reinterpret_cast<const char*>(A + (int64_t)m0 * lda) - kBias;
+  const char* const b_base = reinterpret_cast<const char*>(B + (B_KC ? (int64_t)n0 * ldb : (int64_t)n0)) - kBias;
+  const int a_last = M - 1 - m0;  // last valid row of this tile (>= 0)
+  const int b_last = N - 1 - n0;
   // CONV: a_off is the byte offset of the lane's chunk at the top-left corner of the pixel's window (it may lie before
   // the image: the tap's offset is added modulo 2^32), a_yx that corner's coordinates, 16 bits each
   int a_yx[LPA];
@@ -389,10 +396,12 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
       const int ox    = rem - oy * geom.ow;
       const int iy0   = oy * geom.stride_h - geom.pad_h;
       const int ix0   = ox * geom.stride_w - geom.pad_w;
-      a_yx[t]         = (iy0 & 0xffff) | (ix0 << 16);
+      // a pixel beyond the last one gets a window that starts far above the image: every tap reads zeros
+      a_yx[t]         = pixel < M ? (iy0 & 0xffff) | (ix0 << 16) : 0x8000;
       a_off[t]        = ((unsigned)((n * geom.h + iy0) * geom.w + ix0) * (unsigned)geom.c + (((lane & 7) ^ key) << 3)) * 2u;
     } else {
-      a_off[t] = (unsigned)(((int64_t)row * lda + (((lane & 7) ^ key) << 3)) * 2 - 1024 * (t & 3));
+      const int row_c = row < a_last ? row : a_last;
+      a_off[t] = (unsigned)(((int64_t)row_c * lda + (((lane & 7) ^ key) << 3)) * 2 + kBias - 1024 * (t & 3));
     }
   }
   // CONV: filter tap and first channel of the K step whose loads are being issued (all loads of one step are issued
@@ -414,12 +423,15 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     if (B_KC) {
       const int row = 8 * q + (lane >> 3);
       const int key = (row & 7) ^ ((row >> 3) & 1);
-      b_off[t]      = (unsigned)(((int64_t)row * ldb + (((lane & 7) ^ key) << 3)) * 2 - 1024 * (t & 3));
+      const int row_c = row < b_last ? row : b_last;
+      b_off[t]      = (unsigned)(((int64_t)row_c * ldb + (((lane & 7) ^ key) << 3)) * 2 + kBias - 1024 * (t & 3));
     } else {
       constexpr int CH = BN / 8;  // 16-byte chunks per k-row
       const int krow   = q * (64 / CH) + lane / CH;
       const int chunk  = (lane % CH) ^ (2 * (krow & 3)) ^ (8 * ((krow >> 4) & 1));
-      b_off[t]         = (unsigned)(((int64_t)krow * ldb + (chunk << 3)) * 2 - 1024 * (t & 3));
+      const int last_c = (b_last + 1) / 8 - 1;  // N % 8 == 0: the last whole chunk of this tile's columns
+      const int chunk_c = chunk < last_c ? chunk : last_c;
+      b_off[t]         = (unsigned)(((int64_t)krow * ldb + (chunk_c << 3)) * 2 + kBias - 1024 * (t & 3));
     }
   }
   const int64_t b_step = (B_KC ? kD64BK : (int64_t)kD64BK * ldb) * 2;  // bytes per K step
@@ -631,9 +643,10 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   float sc[TN], sh[TN];
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
-    const int col = n0 + wn * (TN * 16) + j * 16 + (lane & 15);
-    sc[j]         = epi.scale ? epi.scale[col] : epi.alpha;
-    sh[j]         = epi.shift ? epi.shift[col] : 0.0f;
+    int col = n0 + wn * (TN * 16) + j * 16 + (lane & 15);
+    col     = col < N ? col : N - 1;
+    sc[j]   = epi.scale ? epi.scale[col] : epi.alpha;
+    sh[j]   = epi.shift ? epi.shift[col] : 0.0f;
   }
   constexpr int CPR = BN / 8;  // 8-column chunks per row
   if (!Rt) {
@@ -669,6 +682,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
         // streaming stores: results that do not sit dirty in L2 shorten the write-back at the end of the kernel
         // (4096^3 2 %, 8192^3 3.6 % faster); a convolution inside a network keeps its output cached for the next
         // layer instead (ResNet-50 0.4 % slower with streaming stores)
+        if (row >= M || n0 + c16 * 8 >= N) continue;
         u32x4* dst = reinterpret_cast<u32x4*>(Ct + (int64_t)row * ldc + n0 + c16 * 8);
         if (epi.streaming) {
           __builtin_nontemporal_store(v, dst);
@@ -705,6 +719,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
       const int lrow  = chunk / CPR;
       const int c8    = chunk % CPR;
       const int row   = m0 + (lrow / (IB * 16)) * (TM * 16) + pass * (IB * 16) + lrow % (IB * 16);
+      if (row >= M || n0 + c8 * 8 >= N) continue;
       const int64_t o = (int64_t)row * ldc + n0 + c8 * 8;
       const f32x4 lo  = *reinterpret_cast<const f32x4*>(stage + lrow * kRowFloats + c8 * 8);
       const f32x4 hi  = *reinterpret_cast<const f32x4*>(stage + lrow * kRowFloats + c8 * 8 + 4);
@@ -1071,13 +1086,27 @@ void XcdRectangles(int tiles_m, int tiles_n, int* xcd_cols, int* sub_rows, int* 
   }
 }
 
+// The same for tile counts that do not divide: rectangles of ceil(tiles_m / gr) x ceil(tiles_n / gc) tiles, the grid
+// is 8 * sub_rows * sub_cols blocks and those that fall outside the tile grid return at once.
+void XcdRectanglesPadded(int tiles_m, int tiles_n, int* xcd_cols, int* sub_rows, int* sub_cols) {
+  for (int gc = 1; gc <= 8; gc *= 2) {
+    const int gr = 8 / gc;
+    const int r = (tiles_m + gr - 1) / gr, c = (tiles_n + gc - 1) / gc;
+    if (*sub_rows == 0 || r + c < *sub_rows + *sub_cols) {
+      *xcd_cols = gc;
+      *sub_rows = r;
+      *sub_cols = c;
+    }
+  }
+}
+
 template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false, int NS = 2>
 void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
   int64_t ldb = p.trans_b ? p.k : p.n;
-  const int tiles_m = p.m / BM, tiles_n = p.n / BN;
-  dim3 grid(tiles_m * tiles_n, p.batch, 1);
+  const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
   int xcd_cols = 0, sub_rows = 0, sub_cols = 0;
-  XcdRectangles(tiles_m, tiles_n, &xcd_cols, &sub_rows, &sub_cols);
+  XcdRectanglesPadded(tiles_m, tiles_n, &xcd_cols, &sub_rows, &sub_cols);
+  dim3 grid(8 * sub_rows * sub_cols, p.batch, 1);
   DmaEpilogue epi;
   epi.scale          = p.scale;
   epi.shift          = p.shift;
@@ -1095,26 +1124,30 @@ void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
                      p.stride_b, p.stride_c, xcd_cols, sub_rows, sub_cols, geom);
 }
 
-// A stored [M][K], K % 64 == 0: 256x256 tiles when they fill the chip, else 128x128 tiles when M and N allow them
-// and there are enough of those; false when neither applies
+// A stored [M][K], K % 64 == 0, N % 8 == 0 (whole 16-byte chunks per row of C and of a row-major B): 256x256 tiles
+// when they fill the chip, else 128x128 tiles when there are enough of those; M and N need not be multiples of the
+// tile (the last tile row / column computes some rows / columns that are not stored); false when neither applies
 template <typename T>
 bool TryDma16(const GemmProblem& p, hipStream_t stream) {
-  if (p.trans_a || p.k % 64 != 0) return false;
+  if (p.trans_a || p.k % 64 != 0 || p.n % 8 != 0) return false;
+  // every access moves 16 bytes
+  if (reinterpret_cast<uintptr_t>(p.a) % 16 != 0 || reinterpret_cast<uintptr_t>(p.b) % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(p.c) % 16 != 0 || reinterpret_cast<uintptr_t>(p.residual) % 16 != 0 ||
+      p.stride_a % 8 != 0 || p.stride_b % 8 != 0 || p.stride_c % 8 != 0)
+    return false;
   // lanes address a tile with 32-bit byte offsets from its first row: 256 rows of K, or 64 rows of N, 16-bit elements
   if (p.k >= (1 << 22) || p.n >= (1 << 24)) return false;
-  const bool fit256 = p.m % 256 == 0 && p.n % 256 == 0;
-  const bool fit128 = p.m % 128 == 0 && p.n % 128 == 0;
-  const int64_t tiles256 = fit256 ? (int64_t)(p.m / 256) * (p.n / 256) * p.batch : 0;
-  const int64_t tiles128 = fit128 ? (int64_t)(p.m / 128) * (p.n / 128) * p.batch : 0;
+  const int64_t tiles256 = (int64_t)((p.m + 255) / 256) * ((p.n + 255) / 256) * p.batch;
+  const int64_t tiles128 = (int64_t)((p.m + 127) / 128) * ((p.n + 127) / 128) * p.batch;
   static const int forced = getenv("FLAGS_cinn_hip_gemm_tile") ? atoi(getenv("FLAGS_cinn_hip_gemm_tile")) : 0;
   // narrow outputs with B stored [N][K] (convolutions to 64 channels): 256x64 tiles on 4x1 wavefronts, two blocks per CU
-  const bool narrow = p.trans_b && p.n % 128 != 0 && p.n % 64 == 0 && p.m % 256 == 0 && forced == 0 &&
-                      (int64_t)(p.m / 256) * (p.n / 64) * p.batch >= 256;
+  const bool narrow = p.trans_b && p.n % 128 != 0 && p.n % 64 == 0 && forced == 0 &&
+                      (int64_t)((p.m + 255) / 256) * (p.n / 64) * p.batch >= 256;
   // 128x128 tiles keep two stages of 32 KiB and two blocks per CU, or - when there is at most one block per CU
   // anyway - four stages: three K steps of loads in flight instead of one (2048^3: 27.8 -> 21.9 us; with more
   // blocks than CUs two blocks of two stages are faster).  FLAGS_cinn_hip_gemm_stages = 2 / 4 forces one form.
   static const int forced_stages = getenv("FLAGS_cinn_hip_gemm_stages") ? atoi(getenv("FLAGS_cinn_hip_gemm_stages")) : 0;
-  const int stages = forced_stages ? forced_stages : (tiles128 > 0 && tiles128 <= 256 ? 4 : 2);
+  const int stages = forced_stages ? forced_stages : (tiles128 <= 256 ? 4 : 2);
   if (narrow) {
     if (forced_stages == 4) {
       if (p.conv) {
@@ -1380,8 +1413,8 @@ bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream) {
   if (pointwise) {
     // measured inside ResNet-50 at batch 32: the GEMM kernels win only with at least one 128x128 tile per CU and a K
     // loop of two steps or more; smaller grids are better served by the 64x64 tiles and split K of the convolution kernel
-    const bool narrow = a.oc % 128 != 0 && a.oc % 64 == 0 && pixels % 256 == 0 && (pixels / 256) * (a.oc / 64) >= 256;
-    if (a.c < 128 || (!narrow && (pixels / 128) * (a.oc / 128) < 256)) return false;
+    const bool narrow = a.oc % 128 != 0 && a.oc % 64 == 0 && ((pixels + 255) / 256) * (a.oc / 64) >= 256;
+    if (a.c < 128 || (!narrow && ((pixels + 127) / 128) * ((a.oc + 127) / 128) < 256)) return false;
     p.k = a.c;
   } else {
     // any filter, stride, padding, dilation: implicit GEMM, K = kh * kw * c with 64-channel steps inside a tap

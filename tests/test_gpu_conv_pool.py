@@ -352,6 +352,8 @@ IMPLICIT_GEMM_CASES = [
     (32, 192, 32, 32, 512, 1, 2, 0),   # strided 1x1 (a downsampling shortcut): 3 steps inside the one tap
     (16, 64, 64, 64, 64, 3, 1, 1),     # 64 output channels: 256 tiles of 256x64
     (16, 128, 64, 64, 192, 3, 1, 1),   # 192 output channels: three columns of 256x64 tiles
+    (9, 64, 31, 31, 512, 3, 1, 1),     # 8649 pixels: the last tile row is partly beyond the last pixel
+    (17, 64, 63, 63, 64, 3, 1, 1),     # the same on 256x64 tiles
 ]
 
 
@@ -400,7 +402,7 @@ def test_implicit_gemm_convolution_with_residual_epilogue(gpu):
 
 @pytest.mark.parametrize("dtype,tol", [("float16", 2.0 ** -10), ("bfloat16", 2.0 ** -7)])
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (0.5, 2.0)])
-@pytest.mark.parametrize("shape", [(8, 128, 32, 32, 512), (16, 256, 64, 64, 64)])
+@pytest.mark.parametrize("shape", [(8, 128, 32, 32, 512), (16, 256, 64, 64, 64), (9, 128, 31, 31, 512)])
 def test_pointwise_convolution_on_the_gemm_kernel(gpu, dtype, tol, alpha, beta, shape):
     """1x1, stride 1, unpadded, 8192 pixels x 512 channels = 256 tiles of 128x128 and K = 128 (or 65536 pixels x 64
     channels = 256 tiles of 256x64, K = 256): the channels-last entry point hands these shapes to the direct-to-LDS

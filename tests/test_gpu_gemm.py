@@ -113,7 +113,10 @@ def test_16bit_mfma_path_all_layouts(gpu, kind, ta, tb):
 @pytest.mark.parametrize("batch,m,n,k", [(1, 4096, 3072, 128),   # 192 tiles of 256x256: the 8-wavefront kernel
                                          (1, 1536, 1536, 256),   # 144 tiles of 128x128: the 4-wavefront kernel, four stages
                                          (1, 2304, 2304, 192),   # 324 tiles of 128x128: two stages, two blocks per CU
-                                         (2, 1024, 1024, 320)])  # the same with two batches, B broadcast, an odd number of K steps
+                                         (2, 1024, 1024, 320),   # the same with two batches, B broadcast, an odd number of K steps
+                                         (1, 4000, 3000, 128),   # 16 x 12 tiles of 256x256, the last row and column partly outside
+                                         (1, 1500, 1400, 256),   # 12 x 11 tiles of 128x128, ragged both ways
+                                         (2, 1000, 1000, 320)])  # ragged, two batches
 def test_16bit_direct_to_lds_kernel(gpu, kind, tb, alpha, beta, batch, m, n, k):
     """Shapes the direct-to-LDS kernels take (A stored [M][K], K % 64 == 0, enough 256x256 or 128x128 tiles): both
     layouts of B, the staged epilogue (beta == 0) and the read-modify-write one."""
