@@ -1169,10 +1169,10 @@ bool TryDma16(const GemmProblem& p, hipStream_t stream) {
       LaunchDma16<T, true, 256, 256, 2, 4, true>(p, stream);
       return true;
     }
-    // measured on ResNet-50 at batch 32 (fp16): with fewer than two 128x128 tiles per CU the 64x64 tiles of the
-    // convolution kernel are faster (19 against 26 us at 196 tiles, K = 1152) unless K is long (68 against 74 us at
-    // 196 tiles, K = 4608)
-    if (tiles128 >= 256 || (tiles128 >= 128 && p.k >= 4096) || (forced == 128 && tiles128 > 0)) {
+    // measured on ResNet-50 at batch 32 (fp16): from 192 tiles of 128x128 (four stages up to 256 tiles) the network
+    // is 0.5-1 % faster with these layers here than on the 64x64 tiles of the convolution kernel, with 96 tiles 2 %
+    // slower; a long K (52 against 73 us at 196 tiles, K = 4608) pays from 128 tiles
+    if (tiles128 >= 192 || (tiles128 >= 128 && p.k >= 4096) || (forced == 128 && tiles128 > 0)) {
       if (stages == 4) {
         LaunchDma16<T, true, 128, 128, 2, 2, true, 4>(p, stream);
       } else {
@@ -1411,10 +1411,10 @@ bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream) {
   GemmProblem p;
   ConvGeom geom{};
   if (pointwise) {
-    // measured inside ResNet-50 at batch 32: the GEMM kernels win only with at least one 128x128 tile per CU and a K
-    // loop of two steps or more; smaller grids are better served by the 64x64 tiles and split K of the convolution kernel
+    // measured inside ResNet-50 at batch 32: the GEMM kernels win from 192 tiles of 128x128 and a K loop of two steps
+    // or more; smaller grids are better served by the 64x64 tiles and split K of the convolution kernel
     const bool narrow = a.oc % 128 != 0 && a.oc % 64 == 0 && ((pixels + 255) / 256) * (a.oc / 64) >= 256;
-    if (a.c < 128 || (!narrow && ((pixels + 127) / 128) * ((a.oc + 127) / 128) < 256)) return false;
+    if (a.c < 128 || (!narrow && ((pixels + 127) / 128) * ((a.oc + 127) / 128) < 192)) return false;
     p.k = a.c;
   } else {
     // any filter, stride, padding, dilation: implicit GEMM, K = kh * kw * c with 64-channel steps inside a tap
