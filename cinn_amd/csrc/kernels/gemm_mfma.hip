@@ -1479,14 +1479,21 @@ void cinn_call_cublas(void* v_args, int num_args, bool trans_a, bool trans_b, bo
   p.type  = TypeOf(A);
   p.alpha = alpha;
   p.beta  = beta;
-  // one launch per leading index o1; the second batch dim goes to the grid
+  // The batch goes to the grid.  Both batch dims fold into one when every operand is either batched over both or
+  // broadcast over both (one stride per operand describes it); otherwise one launch per leading index o1.
   const int64_t a_mat = (int64_t)a3 * a4, b_mat = (int64_t)b3 * b4, c_mat = (int64_t)m * n;
   const int elem = A->type.bits / CHAR_BIT;
-  for (int i1 = 0; i1 < o1; ++i1) {
+  const bool a_full = a1 == o1 && a2 == o2, a_bcast = a1 == 1 && a2 == 1;
+  const bool b_full = b1 == o1 && b2 == o2, b_bcast = b1 == 1 && b2 == 1;
+  const bool fold   = o1 > 1 && (a_full || a_bcast) && (b_full || b_bcast) && (int64_t)o1 * o2 <= 65535;
+  const int launches = fold ? 1 : o1;
+  const int batch    = fold ? o1 * o2 : o2;
+  for (int i1 = 0; i1 < launches; ++i1) {
     const char* a_base = reinterpret_cast<const char*>(A->memory) + (a1 == 1 ? 0 : (int64_t)i1 * a2 * a_mat) * elem;
     const char* b_base = reinterpret_cast<const char*>(B->memory) + (b1 == 1 ? 0 : (int64_t)i1 * b2 * b_mat) * elem;
     char* c_base       = reinterpret_cast<char*>(C->memory) + (int64_t)i1 * o2 * c_mat * elem;
-    const int64_t sa = a2 == 1 ? 0 : a_mat, sb = b2 == 1 ? 0 : b_mat;
+    const int64_t sa = fold ? (a_full ? a_mat : 0) : (a2 == 1 ? 0 : a_mat);
+    const int64_t sb = fold ? (b_full ? b_mat : 0) : (b2 == 1 ? 0 : b_mat);
     if (!trans_o) {
       p.a = a_base, p.b = b_base, p.c = c_base;
       p.m = m, p.n = n, p.k = k;
@@ -1499,7 +1506,7 @@ void cinn_call_cublas(void* v_args, int num_args, bool trans_a, bool trans_b, bo
       p.trans_a = !trans_b, p.trans_b = !trans_a;
       p.stride_a = sb, p.stride_b = sa;
     }
-    p.batch    = o2;
+    p.batch    = batch;
     p.stride_c = c_mat;
     RunGemm(p, static_cast<hipStream_t>(stream));
   }

@@ -232,6 +232,22 @@ def test_batched_and_broadcast_leading_dims(gpu):
     np.testing.assert_allclose(got, a.astype(np.float64) @ b3.astype(np.float64), rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("b_dims", [(4, 6), (1, 1), (1, 6), (4, 1)])
+@pytest.mark.parametrize("tb", [False, True])
+def test_two_batch_dims_fp16(gpu, b_dims, tb):
+    """[4,6] batches of 512x512x128 (24 x 16 tiles of 128x128 in one launch when B is batched over both dims or
+    broadcast over both; one launch per leading index when it is broadcast over one of them)."""
+    rng = np.random.default_rng(59)
+    a = (rng.standard_normal((4, 6, 512, 128)) * 0.1).astype(np.float16)
+    b = (rng.standard_normal(b_dims + ((512, 128) if tb else (128, 512))) * 0.1).astype(np.float16)
+    got = call_cublas(a, b, (4, 6, 512, 512), "float16", False, tb).astype(np.float64)
+    bf = b.astype(np.float64)
+    bm = np.swapaxes(bf, -1, -2) if tb else bf
+    exact = a.astype(np.float64) @ bm
+    scale = np.abs(a.astype(np.float64)) @ np.abs(bm)
+    assert np.all(np.abs(got - exact) <= 2.0 ** -10 * np.maximum(np.abs(exact), 1e-3 * scale) + 2.0 ** -24)
+
+
 def test_fp64_generic_path(gpu):
     rng = np.random.default_rng(41)
     a, b = rng.standard_normal((33, 47)), rng.standard_normal((47, 21))
