@@ -1104,9 +1104,11 @@ template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool 
 void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
   int64_t ldb = p.trans_b ? p.k : p.n;
   const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
+  // XCD rectangles for tile grids large enough to have panels to share; a small grid per batch entry is numbered
+  // linearly (padded rectangles would leave whole XCDs with nothing but blocks that return at once)
   int xcd_cols = 0, sub_rows = 0, sub_cols = 0;
-  XcdRectanglesPadded(tiles_m, tiles_n, &xcd_cols, &sub_rows, &sub_cols);
-  dim3 grid(8 * sub_rows * sub_cols, p.batch, 1);
+  if (tiles_m * tiles_n >= 64) XcdRectanglesPadded(tiles_m, tiles_n, &xcd_cols, &sub_rows, &sub_cols);
+  dim3 grid(sub_rows > 0 ? 8 * sub_rows * sub_cols : tiles_m * tiles_n, p.batch, 1);
   DmaEpilogue epi;
   epi.scale          = p.scale;
   epi.shift          = p.shift;
@@ -1182,7 +1184,12 @@ bool TryDma16(const GemmProblem& p, hipStream_t stream) {
     }
     return false;
   }
-  if (tiles256 >= 192 && forced != 128) {
+  // rows and columns a tiling computes beyond M and N: 256x256 tiles are passed over when they would compute a fifth
+  // more than 128x128 tiles (a [512,64] result is a quarter of one 256x256 tile)
+  const double area256 = (double)((p.m + 255) / 256) * ((p.n + 255) / 256) * 4.0;
+  const double area128 = (double)((p.m + 127) / 128) * ((p.n + 127) / 128);
+  const bool wasteful256 = area256 > 1.2 * area128 && tiles128 >= 128;
+  if (tiles256 >= 192 && forced != 128 && !wasteful256) {
     if (p.trans_b) {
       LaunchDma16<T, true, 256, 256, 2, 4>(p, stream);
     } else {
