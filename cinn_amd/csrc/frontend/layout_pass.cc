@@ -111,10 +111,13 @@ class LayoutConverter {
       bool nchw    = GetAttr<std::string>(ins->attrs, "data_format", "NCHW") == "NCHW";
       bool forward = GetAttr<std::string>(ins->attrs, "conv_type", "forward") == "forward";
       int groups   = GetAttr<int>(ins->attrs, "groups", 1);
-      if (nchw && forward && groups == 1 && x->shape.size() == 4 && MfmaType(x->type)) {
+      const int chunk = 16 / x->type.bytes();
+      // depthwise: one filter per channel (the channels-last kernel wants whole 16-byte channel vectors)
+      const bool depthwise = groups > 1 && x->shape.size() == 4 && w->shape.size() == 4 && groups == x->shape[1] &&
+                             groups == w->shape[0] && w->shape[1] == 1 && x->shape[1] % chunk == 0;
+      if (nchw && forward && (groups == 1 || depthwise) && x->shape.size() == 4 && MfmaType(x->type)) {
         AttributeMap attrs   = ins->attrs;
         attrs["data_format"] = std::string("NHWC");
-        const int chunk      = 16 / x->type.bytes();
         Variable y;
         if (HasTwin(x) || x->shape[1] % chunk == 0) {
           y = emit_.Emit1("conv2d", {GetNhwc(x), FilterToOhwi(w)}, attrs);
@@ -245,7 +248,8 @@ Program FuseConvBatchNorm(const Program& program, const std::set<std::string>& f
     auto& conv = instrs[i];
     if (conv->op_type != "conv2d" || dropped[i]) continue;
     if (GetAttr<std::string>(conv->attrs, "data_format", "NCHW") != "NHWC") continue;
-    if (GetAttr<int>(conv->attrs, "groups", 1) != 1) continue;
+    // grouped convolutions in channels-last form are depthwise ones (the layout pass converts no others); their kernel
+    // has the same epilogue
     int bn_at = single_user(conv->outputs[0]);
     if (bn_at < 0 || instrs[bn_at]->op_type != "batch_norm" || !(instrs[bn_at]->inputs[0] == conv->outputs[0])) continue;
     auto& bn = instrs[bn_at];

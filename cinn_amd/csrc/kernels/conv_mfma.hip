@@ -304,7 +304,13 @@ void RunConv(cinn_buffer_t* x, cinn_buffer_t* w, cinn_buffer_t* y, const float* 
     a.oc = fn, a.kh = fh, a.kw = fw, a.oh = oh, a.ow = ow;
     a.pad_h = ph, a.pad_w = pw, a.stride_h = sh, a.stride_w = sw, a.dil_h = dh, a.dil_w = dw;
     a.type = x->type;
-    CINN_RT_CHECK(groups == 1, "conv2d: the channels-last kernels do not support groups (got %d)", groups);
+    if (groups != 1) {
+      CINN_RT_CHECK(cinn_hip_kernels::DepthwiseNhwcSupported(a, groups),
+                    "conv2d: of grouped convolutions the channels-last kernels take depthwise ones only (groups %d, channels %d -> %d)",
+                    groups, ic, fn);
+      cinn_hip_kernels::RunDepthwiseNhwc(a, stream);
+      return;
+    }
     CINN_RT_CHECK(cinn_hip_kernels::ConvNhwcSupported(a), "conv2d: channels-last needs the channel count (%d) to be a multiple of 16 bytes", ic);
     cinn_hip_kernels::RunConvNhwc(a, stream);
     return;

@@ -37,6 +37,11 @@ bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream);
 // 256 bytes of zeros in device memory (what masked-out chunks are read from)
 const void* ConvZeroPage();
 
+// depthwise convolutions (groups == channels in == channels out) on channels-last tensors, filter [C][KH][KW]
+// (conv_depthwise.hip): same epilogue; false when the shape does not qualify
+bool DepthwiseNhwcSupported(const ConvNhwcArgs& a, int groups);
+void RunDepthwiseNhwc(const ConvNhwcArgs& a, hipStream_t stream);
+
 // NCHW-input convolutions whose filter and input patch fit LDS (conv_stem_mfma.hip): staged instead of gathered
 bool ConvStemSupported(const ConvNhwcArgs& a);
 void RunConvStem(const ConvNhwcArgs& a, hipStream_t stream);

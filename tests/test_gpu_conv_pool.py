@@ -249,7 +249,7 @@ def test_matmul_of_a_matrix_with_itself(gpu):
 
 
 # ---- the channels-last kernels through the C-ABI (tensor formats 1 and 2 of cinn_call_cudnn_conv2d_forward) --------
-def call_conv_nhwc(x_nchw, w_oihw, stride, pad, fmt, dtype, alpha=1.0, beta=0.0, y_init=None, dilation=1):
+def call_conv_nhwc(x_nchw, w_oihw, stride, pad, fmt, dtype, alpha=1.0, beta=0.0, y_init=None, dilation=1, groups=1):
     """x / w are fp32 arrays in NCHW / OIHW; they are converted to `dtype` and to the layout `fmt` asks for.
     Returns the output as fp32 NCHW."""
     from cinn_amd.common import bfloat16_bits_to_float32, float32_to_bfloat16_bits
@@ -274,8 +274,8 @@ def call_conv_nhwc(x_nchw, w_oihw, stride, pad, fmt, dtype, alpha=1.0, beta=0.0,
     y0 = np.zeros((n, oc, oh, ow), np.float32) if y_init is None else y_init
     Y.copy_from(to_dev(y0.transpose(0, 2, 3, 1)))
     args = runtime.pod_args([X, W, Y])
-    lib.cinn_call_cudnn_conv2d_forward(args, 3, fmt, alpha, beta, n, ic, ih, iw, oc, ic, kh, kw, pad, pad, stride, stride,
-                                       dilation, dilation, 1, n, oc, oh, ow, None)
+    lib.cinn_call_cudnn_conv2d_forward(args, 3, fmt, alpha, beta, n, ic, ih, iw, oc, ic // groups, kh, kw, pad, pad, stride,
+                                       stride, dilation, dilation, groups, n, oc, oh, ow, None)
     runtime.synchronize()
     out = Y.numpy()
     out = bfloat16_bits_to_float32(out) if dtype == "bfloat16" else out.astype(np.float32)
@@ -370,6 +370,70 @@ def test_convolution_as_implicit_gemm(gpu, case, dtype, tol):
     want = oracle.conv2d_nchw(x, w, (s, s), (p, p))
     scale = oracle.conv2d_nchw(np.abs(x), np.abs(w), (s, s), (p, p))
     assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+
+
+DEPTHWISE_CASES = [
+    # (n, c, h, w, k, stride, pad, dilation)
+    (2, 32, 14, 15, 3, 1, 1, 1),
+    (3, 64, 17, 9, 3, 2, 1, 1),
+    (1, 16, 12, 12, 5, 1, 2, 1),
+    (2, 24, 11, 13, 3, 1, 2, 2),      # fp32 vectors are 4 channels: 24 is a multiple of 4 and of 8
+    (1, 256, 7, 7, 7, 1, 0, 1),       # global filter: one output pixel
+]
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 1e-5), ("float16", 1e-2), ("bfloat16", 2e-2)])
+@pytest.mark.parametrize("case", DEPTHWISE_CASES)
+def test_depthwise_convolution_channels_last(gpu, case, dtype, tol):
+    """groups == channels: the channels-last entry point runs the depthwise kernel (filter [C][KH][KW] in, one fp32
+    accumulation per output in tap order); alpha / beta through its epilogue."""
+    n, c, h, w_, k, s, p, d = case
+    rng = np.random.default_rng(sum(case) + 13)
+    x = round_to(rng.standard_normal((n, c, h, w_)), dtype)
+    w = round_to(rng.standard_normal((c, 1, k, k)) * np.sqrt(2.0 / (k * k)), dtype)
+    oh = oracle.conv_out_dim(h, k, p, s, d)
+    ow = oracle.conv_out_dim(w_, k, p, s, d)
+    y0 = round_to(rng.standard_normal((n, c, oh, ow)), dtype)
+    got = call_conv_nhwc(x, w, s, p, 1, dtype, alpha=0.5, beta=2.0, y_init=y0, dilation=d, groups=c)
+    conv = oracle.conv2d_nchw(x, w, (s, s), (p, p), (d, d), c).astype(np.float64)
+    want = 0.5 * conv + 2.0 * y0
+    scale = 0.5 * oracle.conv2d_nchw(np.abs(x), np.abs(w), (s, s), (p, p), (d, d), c) + 2.0 * np.abs(y0)
+    if dtype == "float32":
+        assert np.all(np.abs(got - want) <= tol * scale + 1e-30)
+    else:
+        assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_depthwise_conv_bn_relu_through_netbuilder(gpu, dtype):
+    """A MobileNet-style layer: depthwise 3x3 -> batch norm -> relu at batch 32.  The layout pass keeps it channels-last
+    and the batch norm and relu fold into the depthwise kernel's epilogue; equal images give equal outputs."""
+    n, c, hw = 32, 128, 28
+    rng = np.random.default_rng(71)
+    x = rng.standard_normal((n, c, hw, hw)).astype(dtype)
+    x[19] = x[3]
+    w = (rng.standard_normal((c, 1, 3, 3)) * np.sqrt(2.0 / 9)).astype(dtype)
+    scale = rng.uniform(0.5, 1.5, c).astype(dtype)
+    bias = rng.uniform(-0.5, 0.5, c).astype(dtype)
+    mean = (rng.standard_normal(c) * 0.1).astype(dtype)
+    var = rng.uniform(0.5, 1.5, c).astype(dtype)
+    b = NetBuilder("dw")
+    T = Float(32) if dtype == "float32" else Float(16)
+    X, W = b.create_input(T, x.shape, "x"), b.create_input(T, w.shape, "w")
+    S, Bi, M, V = [b.create_input(T, [c], nm) for nm in ("scale", "bias", "mean", "var")]
+    for v in (W, S, Bi, M, V):
+        v.set_const(True)
+    conv = b.conv2d(X, W, strides=[1, 1], paddings=[1, 1], groups=c)
+    y = b.relu(b.batchnorm(conv, S, Bi, M, V, epsilon=1e-5)[0])
+    (got,), comp = run(b, {X: x, W: w, S: scale, Bi: bias, M: mean, V: var}, [y])
+    sample = [0, 3, 31]
+    want_conv = oracle.conv2d_nchw(x[sample], w, (1, 1), (1, 1), (1, 1), c)
+    want = oracle.batch_norm_relu_nchw(want_conv, scale, bias, mean, var, 1e-5, relu=True)
+    tol = 1e-4 if dtype == "float32" else 2e-2
+    np.testing.assert_allclose(got[sample].astype(np.float64), want.astype(np.float64), rtol=tol, atol=tol)
+    assert np.array_equal(got[19], got[3])
+    # transposes of x in and y out, and the fused convolution
+    assert comp.num_instructions() == 3, comp.fusion_groups()
 
 
 @pytest.mark.parametrize("dtype,tol", [("float16", 1e-2), ("bfloat16", 2e-2)])
