@@ -185,6 +185,35 @@ void cinn_call_cudnn_softmax_forward(void* v_args, int num_args, int mode, int f
                                      int input_n, int input_c, int input_h, int input_w, int output_n, int output_c,
                                      int output_h, int output_w, void* stream);
 
+/* Gradients of the three calls above, with the reference's argument lists.  Gather-form kernels (one thread or block
+ * per gradient element, fp32 accumulation), formats 0 = NCHW / [F][C][KH][KW] and 1 = NHWC / [F][KH][KW][C]; every result
+ * is out = alpha * gradient + beta * out.
+ * cinn_call_cudnn_conv2d_backward_data (cuda_util.cc:722-843): v_args = {w, dy, dx}.
+ * cinn_call_cudnn_conv2d_backward_filter (cuda_util.cc:845-967): v_args = {x, dy, dw}. */
+void cinn_call_cudnn_conv2d_backward_data(void* v_args, int num_args, int format, float alpha, float beta, int input_n,
+                                          int input_c, int input_h, int input_w, int filter_n, int filter_c,
+                                          int filter_h, int filter_w, int pad_h, int pad_w, int stride_h, int stride_w,
+                                          int dilation_h, int dilation_w, int groups, int output_n, int output_c,
+                                          int output_h, int output_w, void* stream);
+void cinn_call_cudnn_conv2d_backward_filter(void* v_args, int num_args, int format, float alpha, float beta, int input_n,
+                                            int input_c, int input_h, int input_w, int filter_n, int filter_c,
+                                            int filter_h, int filter_w, int pad_h, int pad_w, int stride_h,
+                                            int stride_w, int dilation_h, int dilation_w, int groups, int output_n,
+                                            int output_c, int output_h, int output_w, void* stream);
+
+/* Replaces cinn_call_cudnn_pool2d_backward (cuda_util.cc:1043-1119).  v_args = {x, y, dy, dx}; modes as in the
+ * forward call.  Max pooling sends a window's gradient to its first maximum (rows, then columns; x == y decides). */
+void cinn_call_cudnn_pool2d_backward(void* v_args, int num_args, int mode, int format, float alpha, float beta,
+                                     int input_n, int input_c, int input_h, int input_w, int kernel_h, int kernel_w,
+                                     int pad_h, int pad_w, int stride_h, int stride_w, int output_n, int output_c,
+                                     int output_h, int output_w, void* stream);
+
+/* Replaces cinn_call_cudnn_softmax_backward (cuda_util.cc:1169-1217), which always runs CUDNN_SOFTMAX_LOG:
+ * dx = alpha * (dy - exp(y) * sum(dy)) + beta * dx over C (mode 1) or C*H*W (mode 0).  v_args = {y, dy, dx}. */
+void cinn_call_cudnn_softmax_backward(void* v_args, int num_args, int mode, int format, float alpha, float beta,
+                                      int input_n, int input_c, int input_h, int input_w, int output_n, int output_c,
+                                      int output_h, int output_w, void* stream);
+
 /* Replace cinn_call_cuda_memset / cinn_call_cuda_memcpy (cuda_util.cc:439-462). */
 void cinn_call_cuda_memset(void* v_args, int num_args, int value, size_t count, void* stream);
 void cinn_call_cuda_memcpy(void* v_args, int num_args, size_t count, void* stream);
