@@ -18,8 +18,9 @@ One JSON line is printed; besides the contract fields it carries
   cpu_baseline - the CPU oracle (a port of the reference's compute definitions, OpenMP) timed on this
                  box's host cores on the same workload
   kernels      - per-kernel event timings of the step
-  extra        - configs[0] (relu(add)) latency, the scaled element-wise streaming rate, configs[2] GEMM TFLOP/s and
-                 configs[4] ResNet-50 images/s
+  extra        - configs[0] (relu(add)) latency, the scaled element-wise streaming rate, configs[2] GEMM TFLOP/s,
+                 configs[3] convolution layers, configs[4] ResNet-50 images/s, and under "cpu_baseline" the CPU oracle
+                 timed on bounded samples of those configs
 """
 import argparse
 import json
@@ -127,6 +128,81 @@ def cpu_baseline(kernels, repeats=3):
     return dict(value=round(total / med / 1e9, 3), unit="GB/s", cores=threads, kind="port",
                 sample="full configs[1] workload (6 kernels, %d bytes), median of %d passes, %.3f s per pass, "
                        "OpenMP over rows" % (total, repeats, med))
+
+
+def extra_cpu_baselines():
+    """The CPU oracle on bounded samples of the other configs (the same threads as cpu_baseline): configs[0] whole,
+    configs[2]'s fp32 1024^3 product whole, configs[3]'s layers and configs[4]'s network on 2 of the 32 images."""
+    import oracle
+    import bench_conv
+    import bench_resnet50 as rn
+    threads = oracle.num_threads()
+    out = {}
+
+    def median_time(fn, budget_s, most=200):
+        fn()
+        t0 = time.perf_counter()
+        fn()
+        one = time.perf_counter() - t0
+        times = [one]
+        for _ in range(max(0, min(most, int(budget_s / max(one, 1e-6))) - 1)):
+            t0 = time.perf_counter()
+            fn()
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        return times[len(times) // 2], len(times)
+
+    rng = np.random.default_rng(1000)
+    a = rng.uniform(-1, 1, (1, 3, 224, 224)).astype(np.float32)
+    t, n = median_time(lambda: oracle.add_relu(a, a), 1.0)
+    out["config0_add_relu_1x3x224x224"] = dict(value=round(3 * a.nbytes / t / 1e9, 3), unit="GB/s", cores=threads,
+                                               kind="port", sample="whole tensor, median of %d passes" % n)
+    m = (rng.standard_normal((1024, 1024)) * 0.02).astype(np.float32)
+    t, n = median_time(lambda: oracle.matmul(m, m), 3.0, most=5)
+    out["config2_matmul_fp32_1024"] = dict(value=round(2 * 1024 ** 3 / t / 1e9, 2), unit="GFLOP/s", cores=threads,
+                                           kind="port", sample="whole product, median of %d passes" % n)
+    images = 2
+    for name, ic, oc, k, st, pad, hw in bench_conv.LAYERS:
+        x = rng.standard_normal((images, ic, hw, hw)).astype(np.float32)
+        w = (rng.standard_normal((oc, ic, k, k)) * np.sqrt(2.0 / (ic * k * k))).astype(np.float32)
+        v = rng.uniform(0.5, 1.5, oc).astype(np.float32)
+
+        def layer():
+            y = oracle.conv2d_nchw(x, w, (st, st), (pad, pad))
+            return oracle.batch_norm_relu_nchw(y, v, v, v, v, 1e-5, relu=True)
+
+        t, n = median_time(layer, 2.0, most=5)
+        oh = (hw + 2 * pad - k) // st + 1
+        out["config3_%s_float32" % name] = dict(value=round(2 * images * oc * oh * oh * ic * k * k / t / 1e9, 2),
+                                                unit="GFLOP/s", cores=threads, kind="port",
+                                                sample="%d of the 32 images, median of %d passes" % (images, n))
+    params = rn.random_params(0, "float32")
+    x = rng.standard_normal((images, 3, 224, 224)).astype(np.float32)
+    specs = {sp[0]: sp for sp in rn.layer_specs()}
+
+    def conv_bn(inp, name, relu):
+        _, _, _, _, st, pad = specs[name]
+        y = oracle.conv2d_nchw(inp, params[name + "_w"], (st, st), (pad, pad))
+        return oracle.batch_norm_relu_nchw(y, params[name + "_scale"], params[name + "_bias"], params[name + "_mean"],
+                                           params[name + "_var"], 1e-5, relu=relu)
+
+    def network():
+        y = oracle.pool2d_nchw(conv_bn(x, "conv1", True), (3, 3), (2, 2), (1, 1, 1, 1), "max")
+        for si, (blocks, _, _) in enumerate(rn.STAGES):
+            for bi in range(blocks):
+                tag = "s%db%d" % (si + 2, bi)
+                short = conv_bn(y, tag + "_sc", False) if bi == 0 else y
+                z = conv_bn(conv_bn(conv_bn(y, tag + "_a", True), tag + "_b", True), tag + "_c", False)
+                y = np.maximum(z + short, np.float32(0))
+        y = oracle.pool2d_nchw(y, (7, 7), (1, 1), (0, 0, 0, 0), "avg").reshape(images, 2048)
+        return oracle.matmul(y, params["fc_w"]) + params["fc_b"]
+
+    t0 = time.perf_counter()
+    network()
+    t = time.perf_counter() - t0
+    out["resnet50_v1.5_float32"] = dict(value=round(images / t, 3), unit="images/s", cores=threads, kind="port",
+                                        sample="%d of the 32 images, one pass of %.1f s" % (images, t))
+    return out
 
 
 def read_traffic(kernel_name):
@@ -278,6 +354,8 @@ def main():
         result["cpu_baseline"] = cpu_baseline(kernels)
     if not args.no_extra:
         result["extra"] = extra_measurements(stream, runtime)
+        if not args.no_cpu_baseline:
+            result["extra"]["cpu_baseline"] = extra_cpu_baselines()
     print(json.dumps(result))
 
 
