@@ -699,6 +699,21 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   static_assert(PASS_ROWS * kRowFloats * 4 <= NS * STAGE, "the staged result does not fit the operand stages");
   static_assert(PASS_ROWS * CPR % THREADS == 0, "the copy-out loop assumes whole rounds");
   float* stage = reinterpret_cast<float*>(lds);
+  // The residual chunks of a pass are requested one pass ahead (those of the first pass before the first barrier), so
+  // that their latency runs under the staging of the accumulators instead of after it.
+  constexpr int EPT = PASS_ROWS * CPR / THREADS;  // chunks per thread and pass
+  vec8 res[2][EPT];
+  auto request_residual = [&](int pass, vec8* out) {
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+      const int chunk = e * THREADS + tid;
+      const int lrow  = chunk / CPR;
+      const int c8    = chunk % CPR;
+      const int row   = m0 + (lrow / (IB * 16)) * (TM * 16) + pass * (IB * 16) + lrow % (IB * 16);
+      if (row < M && n0 + c8 * 8 < N) out[e] = *reinterpret_cast<const vec8*>(Rt + (int64_t)row * ldc + n0 + c8 * 8);
+    }
+  };
+  request_residual(0, res[0]);
 #pragma unroll
   for (int pass = 0; pass < TM / IB; ++pass) {
     __syncthreads();
@@ -713,8 +728,9 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
           stage[lrow * kRowFloats + col] = __builtin_fmaf(acc[IB * pass + ii][j][r], sc[j], sh[j]);
         }
     __syncthreads();
+    if (pass + 1 < TM / IB) request_residual(pass + 1, res[(pass + 1) & 1]);
 #pragma unroll
-    for (int e = 0; e < PASS_ROWS * CPR / THREADS; ++e) {
+    for (int e = 0; e < EPT; ++e) {
       const int chunk = e * THREADS + tid;
       const int lrow  = chunk / CPR;
       const int c8    = chunk % CPR;
@@ -723,11 +739,11 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
       const int64_t o = (int64_t)row * ldc + n0 + c8 * 8;
       const f32x4 lo  = *reinterpret_cast<const f32x4*>(stage + lrow * kRowFloats + c8 * 8);
       const f32x4 hi  = *reinterpret_cast<const f32x4*>(stage + lrow * kRowFloats + c8 * 8 + 4);
-      const vec8 res  = *reinterpret_cast<const vec8*>(Rt + o);
+      const vec8& rq  = res[pass & 1][e];
       vec8 out;
 #pragma unroll
       for (int q = 0; q < 8; ++q) {
-        float v = __builtin_fmaf(epi.residual_scale, (float)res[q], q < 4 ? lo[q] : hi[q - 4]);
+        float v = __builtin_fmaf(epi.residual_scale, (float)rq[q], q < 4 ? lo[q] : hi[q - 4]);
         asm volatile("" : "+v"(v));
         if (epi.relu) v = v > 0.0f ? v : 0.0f;
         out[q] = (T)v;
@@ -737,6 +753,140 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
       } else {
         *reinterpret_cast<vec8*>(Ct + o) = out;
       }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Short reductions (K = 64 .. 256) with B stored [N][K] - 1x1 convolutions over few channels, attention scores:
+// 2 * K flop per output element make these products a stream of C (and of the residual), and a tiled kernel, whose
+// block waits for its operands, computes for a moment and then writes its tile, never has enough bytes in flight.
+// Here nothing is staged and nobody waits for a neighbour: a wavefront keeps its NT * 16 filter rows in registers as
+// MFMA operands for the whole kernel and walks over groups of 16 rows of A, computing the transposed tile
+// D[n][m] = sum_k B[n][k] * A[m][k] on v_mfma_f32_16x16x32, so that a lane ends up with 4 consecutive columns of one
+// row of C: the residual arrives as 8-byte loads in that layout, the finished 16-bit tile turns into whole rows in a
+// piece of LDS private to the wavefront and leaves as 16-byte stores.
+// Both operands are read from global memory straight in fragment layout (16 bytes of one row per lane); the rows and
+// the residual of the next group are requested before the current group is computed.  Per-column scale / shift sit
+// in LDS.  No block barrier after the start-up.
+// ---------------------------------------------------------------------------------------------------
+template <typename T, int NT, int KH, bool RES>
+__global__ void __launch_bounds__(256)
+gemm16_shortk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ C, int M, int N,
+                     int64_t lda, int64_t ldb, int64_t ldc, DmaEpilogue epi, int64_t stride_a, int64_t stride_b,
+                     int64_t stride_c, int ny) {
+  typedef typename Half16<T>::vec8 vec8;
+  constexpr int NW = NT * 16;  // columns per wavefront
+  __shared__ __attribute__((aligned(16))) float s_scale[NW];
+  __shared__ __attribute__((aligned(16))) float s_shift[NW];
+  constexpr int kStageRow     = NW * 2 + 16;  // bytes; the pad spreads the 16 rows of an 8-byte write over the banks
+  constexpr int kChunksPerRow = NW / 8;       // 16-byte chunks
+  constexpr int kRowsPerStore = 64 / kChunksPerRow;
+  __shared__ __attribute__((aligned(16))) char s_stage[4 * 16 * kStageRow];
+  const int tid  = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  char* my_stage = s_stage + wave * 16 * kStageRow;  // private to the wavefront: no block barrier in the loop
+  // consecutive block ids go round-robin to the 8 XCDs: the ny column panels of one row range stay on one XCD
+  const int lin = blockIdx.x, xcd = lin & 7, idx = lin >> 3;
+  const int n0    = (idx % ny) * NW;
+  const int slot  = (idx / ny) * 8 + xcd;
+  const int slots = gridDim.x / ny;
+  A += (int64_t)blockIdx.y * stride_a;
+  B += (int64_t)blockIdx.y * stride_b;
+  C += (int64_t)blockIdx.y * stride_c;
+  const T* Rt = reinterpret_cast<const T*>(epi.residual);
+  if (RES) Rt += (int64_t)blockIdx.y * stride_c;
+  for (int i = tid; i < NW; i += 256) {
+    s_scale[i] = epi.scale ? epi.scale[n0 + i] : epi.alpha;
+    s_shift[i] = epi.shift ? epi.shift[n0 + i] : 0.0f;
+  }
+  const int frow = lane & 15;        // row of the fragment this lane reads
+  const int fk   = (lane >> 4) * 8;  // its 8 elements of a 32-deep k block
+  vec8 wf[NT][KH];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int kh = 0; kh < KH; ++kh)
+      wf[j][kh] = *reinterpret_cast<const vec8*>(B + (int64_t)(n0 + j * 16 + frow) * ldb + kh * 32 + fk);
+  __syncthreads();
+
+  const int groups  = (M + 15) >> 4;
+  const int gstride = slots * 4;
+  int g             = slot * 4 + wave;
+  if (g >= groups) return;
+  struct alignas(8) Res4 { T v[4]; };
+  auto request = [&](int grp, vec8* xa, Res4* rr) {
+    int row = grp * 16 + frow;
+    row     = row < M ? row : M - 1;
+#pragma unroll
+    for (int kh = 0; kh < KH; ++kh) xa[kh] = *reinterpret_cast<const vec8*>(A + (int64_t)row * lda + kh * 32 + fk);
+    if (RES) {
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        rr[j] = *reinterpret_cast<const Res4*>(Rt + (int64_t)row * ldc + n0 + j * 16 + 4 * (lane >> 4));
+    }
+  };
+  // a ring of D groups: the rows (and residual) of the group D - 1 steps ahead are requested while the current one is
+  // computed (three steps ahead measured the same as one: 17.6 against 17.0 us for 100352 x 256 x 64)
+  constexpr int D = 2;
+  vec8 xa[D][KH];
+  Res4 rr[D][RES ? NT : 1];
+#pragma unroll
+  for (int d = 0; d < D - 1; ++d)
+    if (g + d * gstride < groups) request(g + d * gstride, xa[d], rr[d]);
+  for (;;) {
+#pragma unroll
+    for (int u = 0; u < D; ++u) {
+      const int gn        = g + gstride;
+      const bool has_next = gn < groups;
+      if (g + (D - 1) * gstride < groups) request(g + (D - 1) * gstride, xa[(u + D - 1) % D], rr[(u + D - 1) % D]);
+      f32x4 acc[NT];
+#pragma unroll
+      for (int j = 0; j < NT; ++j) acc[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int kh = 0; kh < KH; ++kh)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[j] = Half16<T>::mfma16(wf[j][kh], xa[u][kh], acc[j]);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const f32x4 sc = *reinterpret_cast<const f32x4*>(&s_scale[j * 16 + 4 * (lane >> 4)]);
+        const f32x4 sh = *reinterpret_cast<const f32x4*>(&s_shift[j * 16 + 4 * (lane >> 4)]);
+        Res4 out;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float v = __builtin_fmaf(acc[j][r], sc[r], sh[r]);
+          if (RES) v = __builtin_fmaf(epi.residual_scale, (float)rr[u][RES ? j : 0].v[r], v);
+          asm volatile("" : "+v"(v));  // one rounding to T for every element, see gemm16_dma_kernel's epilogue
+          if (epi.relu) v = v > 0.0f ? v : 0.0f;
+          out.v[r] = (T)v;
+        }
+        *reinterpret_cast<Res4*>(my_stage + frow * kStageRow + (j * 16 + 4 * (lane >> 4)) * 2) = out;
+      }
+      // the wavefront's own 16 x NW tile comes back as whole rows: 16 bytes per lane, full lines per store
+      // (8-byte pieces of 32 contiguous bytes per row write at little more than half the rate)
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int i = 0; i < 16 / kRowsPerStore; ++i) {
+        const int srow = i * kRowsPerStore + lane / kChunksPerRow;
+        const int ch   = lane % kChunksPerRow;
+        const u32x4 v  = *reinterpret_cast<const u32x4*>(my_stage + srow * kStageRow + ch * 16);
+        const int row  = g * 16 + srow;
+        if (row < M) {
+          u32x4* dst = reinterpret_cast<u32x4*>(reinterpret_cast<T*>(C) + (int64_t)row * ldc + n0 + ch * 8);
+          if (epi.streaming) {
+            __builtin_nontemporal_store(v, dst);
+          } else {
+            *dst = v;
+          }
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      if (!has_next) return;
+      g = gn;
     }
   }
 }
@@ -1126,12 +1276,60 @@ void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
                      p.stride_b, p.stride_c, xcd_cols, sub_rows, sub_cols, geom);
 }
 
+// gemm16_shortk_kernel: K = 64, B stored [N][K], N a multiple of the 128 columns of a wavefront, at least 16384 rows.
+// FLAGS_cinn_hip_gemm_shortk=0 switches it off.
+template <typename T, int NT, int KH>
+void LaunchShortK(const GemmProblem& p, hipStream_t stream) {
+  const int ny     = p.n / (NT * 16);
+  const int groups = (p.m + 15) / 16;
+  // two blocks of four wavefronts per CU, spread evenly over the XCDs and the column panels
+  int slots = (groups + 3) / 4;
+  slots     = slots < 512 / ny ? slots : 512 / ny;
+  slots     = (slots + 7) / 8 * 8;
+  DmaEpilogue epi;
+  epi.scale          = p.scale;
+  epi.shift          = p.shift;
+  epi.alpha          = p.alpha;
+  epi.relu           = p.relu ? 1 : 0;
+  epi.residual       = p.residual ? p.residual : (p.beta != 0.0f ? p.c : nullptr);
+  epi.residual_scale = p.residual ? p.residual_scale : p.beta;
+  epi.streaming      = !p.keep_in_cache && (int64_t)p.batch * p.m * p.n * 2 >= (16 << 20);
+  dim3 grid(slots * ny, p.batch, 1);
+#define CINN_SHORTK(RES)                                                                                             \
+  hipLaunchKernelGGL((gemm16_shortk_kernel<T, NT, KH, RES>), grid, dim3(256), 0, stream,                              \
+                     static_cast<const uint16_t*>(p.a), static_cast<const uint16_t*>(p.b), static_cast<uint16_t*>(p.c), \
+                     p.m, p.n, (int64_t)p.k, (int64_t)p.k, (int64_t)p.n, epi, p.stride_a, p.stride_b, p.stride_c, ny)
+  if (epi.residual) {
+    CINN_SHORTK(true);
+  } else {
+    CINN_SHORTK(false);
+  }
+#undef CINN_SHORTK
+}
+
+template <typename T>
+bool TryShortK(const GemmProblem& p, hipStream_t stream) {
+  static const bool enabled = !(getenv("FLAGS_cinn_hip_gemm_shortk") && atoi(getenv("FLAGS_cinn_hip_gemm_shortk")) == 0);
+  if (!enabled || p.conv || p.trans_a || !p.trans_b) return false;
+  // measured against the tiled kernels (fp16, B [N][K]): 100352 x 256 x 64 17.0 against 22.7 us; with 64 columns, or a
+  // K of 128 or 256, or many small batch entries (the filter fragments are reloaded per block) the tiled kernels win
+  if (p.k != 64 || p.n % 128 != 0 || p.m < 16384 || p.batch > 65535) return false;
+  // 8-byte accesses to C and the residual, 16-byte accesses to A and B
+  if (reinterpret_cast<uintptr_t>(p.a) % 16 != 0 || reinterpret_cast<uintptr_t>(p.b) % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(p.c) % 8 != 0 || reinterpret_cast<uintptr_t>(p.residual) % 8 != 0 ||
+      p.stride_a % 8 != 0 || p.stride_b % 8 != 0 || p.stride_c % 4 != 0)
+    return false;
+  LaunchShortK<T, 8, 2>(p, stream);
+  return true;
+}
+
 // A stored [M][K], K % 64 == 0, N % 8 == 0 (whole 16-byte chunks per row of C and of a row-major B): 256x256 tiles
 // when they fill the chip, else 128x128 tiles when there are enough of those; M and N need not be multiples of the
 // tile (the last tile row / column computes some rows / columns that are not stored); false when neither applies
 template <typename T>
 bool TryDma16(const GemmProblem& p, hipStream_t stream) {
   if (p.trans_a || p.k % 64 != 0 || p.n % 8 != 0) return false;
+  if (TryShortK<T>(p, stream)) return true;
   // every access moves 16 bytes
   if (reinterpret_cast<uintptr_t>(p.a) % 16 != 0 || reinterpret_cast<uintptr_t>(p.b) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(p.c) % 16 != 0 || reinterpret_cast<uintptr_t>(p.residual) % 16 != 0 ||
@@ -1421,7 +1619,9 @@ bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream) {
     // measured inside ResNet-50 at batch 32: the GEMM kernels win from 192 tiles of 128x128 and a K loop of two steps
     // or more; smaller grids are better served by the 64x64 tiles and split K of the convolution kernel
     const bool narrow = a.oc % 128 != 0 && a.oc % 64 == 0 && ((pixels + 255) / 256) * (a.oc / 64) >= 256;
-    if (a.c < 128 || (!narrow && ((pixels + 127) / 128) * ((a.oc + 127) / 128) < 192)) return false;
+    static const bool shortk_on = !(getenv("FLAGS_cinn_hip_gemm_shortk") && atoi(getenv("FLAGS_cinn_hip_gemm_shortk")) == 0);
+    const bool shortk = shortk_on && a.c == 64 && a.oc % 128 == 0 && pixels >= 16384;
+    if (!shortk && (a.c < 128 || (!narrow && ((pixels + 127) / 128) * ((a.oc + 127) / 128) < 192))) return false;
     p.k = a.c;
   } else {
     // any filter, stride, padding, dilation: implicit GEMM, K = kh * kw * c with 64-channel steps inside a tap

@@ -466,7 +466,8 @@ def test_implicit_gemm_convolution_with_residual_epilogue(gpu):
 
 @pytest.mark.parametrize("dtype,tol", [("float16", 2.0 ** -10), ("bfloat16", 2.0 ** -7)])
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (0.5, 2.0)])
-@pytest.mark.parametrize("shape", [(8, 128, 32, 32, 512), (16, 256, 64, 64, 64), (9, 128, 31, 31, 512)])
+@pytest.mark.parametrize("shape", [(8, 128, 32, 32, 512), (16, 256, 64, 64, 64), (9, 128, 31, 31, 512),
+                                   (6, 64, 56, 56, 256)])  # 18816 pixels, K = 64: the streaming short-K kernel
 def test_pointwise_convolution_on_the_gemm_kernel(gpu, dtype, tol, alpha, beta, shape):
     """1x1, stride 1, unpadded, 8192 pixels x 512 channels = 256 tiles of 128x128 and K = 128 (or 65536 pixels x 64
     channels = 256 tiles of 256x64, K = 256): the channels-last entry point hands these shapes to the direct-to-LDS

@@ -116,7 +116,9 @@ def test_16bit_mfma_path_all_layouts(gpu, kind, ta, tb):
                                          (2, 1024, 1024, 320),   # the same with two batches, B broadcast, an odd number of K steps
                                          (1, 4000, 3000, 128),   # 16 x 12 tiles of 256x256, the last row and column partly outside
                                          (1, 1500, 1400, 256),   # 12 x 11 tiles of 128x128, ragged both ways
-                                         (2, 1000, 1000, 320)])  # ragged, two batches
+                                         (2, 1000, 1000, 320),   # ragged, two batches
+                                         (1, 16500, 256, 64),    # K = 64, many rows: the streaming short-K kernel
+                                         (2, 16389, 128, 64)])   # (B stored [N][K]); last group of 16 rows ragged
 def test_16bit_direct_to_lds_kernel(gpu, kind, tb, alpha, beta, batch, m, n, k):
     """Shapes the direct-to-LDS kernels take (A stored [M][K], K % 64 == 0, enough 256x256 or 128x128 tiles): both
     layouts of B, the staged epilogue (beta == 0) and the read-modify-write one."""
