@@ -764,8 +764,8 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 // Here nothing is staged and nobody waits for a neighbour: a wavefront keeps its NT * 16 filter rows in registers as
 // MFMA operands for the whole kernel and walks over groups of 16 rows of A, computing the transposed tile
 // D[n][m] = sum_k B[n][k] * A[m][k] on v_mfma_f32_16x16x32, so that a lane ends up with 4 consecutive columns of one
-// row of C: the residual arrives as 8-byte loads in that layout, the finished 16-bit tile turns into whole rows in a
-// piece of LDS private to the wavefront and leaves as 16-byte stores.
+// row of C; the tile turns into whole rows in a piece of LDS private to the wavefront (as finished 16-bit values, or
+// as fp32 when a residual - read as whole rows, 16 bytes per lane - is still to be added) and leaves as 16-byte stores.
 // Both operands are read from global memory straight in fragment layout (16 bytes of one row per lane); the rows and
 // the residual of the next group are requested before the current group is computed.  Per-column scale / shift sit
 // in LDS.  No block barrier after the start-up.
@@ -779,8 +779,10 @@ gemm16_shortk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict_
   constexpr int NW = NT * 16;  // columns per wavefront
   __shared__ __attribute__((aligned(16))) float s_scale[NW];
   __shared__ __attribute__((aligned(16))) float s_shift[NW];
-  constexpr int kStageRow     = NW * 2 + 16;  // bytes; the pad spreads the 16 rows of an 8-byte write over the banks
-  constexpr int kChunksPerRow = NW / 8;       // 16-byte chunks
+  // staging row in bytes, padded so that the 16 rows of a write spread over the banks: the finished 16-bit tile, or -
+  // with a residual, which arrives as whole rows and is added before the rounding - the fp32 tile
+  constexpr int kStageRow     = RES ? (NW + 4) * 4 : NW * 2 + 16;
+  constexpr int kChunksPerRow = NW / 8;  // 8 columns: 16 bytes of C per lane
   constexpr int kRowsPerStore = 64 / kChunksPerRow;
   __shared__ __attribute__((aligned(16))) char s_stage[4 * 16 * kStageRow];
   const int tid  = threadIdx.x;
@@ -816,22 +818,25 @@ gemm16_shortk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict_
   int g             = slot * 4 + wave;
   if (g >= groups) return;
   struct alignas(8) Res4 { T v[4]; };
-  auto request = [&](int grp, vec8* xa, Res4* rr) {
+  auto request = [&](int grp, vec8* xa, vec8* rr) {
     int row = grp * 16 + frow;
     row     = row < M ? row : M - 1;
 #pragma unroll
     for (int kh = 0; kh < KH; ++kh) xa[kh] = *reinterpret_cast<const vec8*>(A + (int64_t)row * lda + kh * 32 + fk);
     if (RES) {
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
-        rr[j] = *reinterpret_cast<const Res4*>(Rt + (int64_t)row * ldc + n0 + j * 16 + 4 * (lane >> 4));
+      for (int i = 0; i < 16 / kRowsPerStore; ++i) {
+        int rrow = grp * 16 + i * kRowsPerStore + lane / kChunksPerRow;
+        rrow     = rrow < M ? rrow : M - 1;
+        rr[i]    = *reinterpret_cast<const vec8*>(Rt + (int64_t)rrow * ldc + n0 + (lane % kChunksPerRow) * 8);
+      }
     }
   };
   // a ring of D groups: the rows (and residual) of the group D - 1 steps ahead are requested while the current one is
   // computed (three steps ahead measured the same as one: 17.6 against 17.0 us for 100352 x 256 x 64)
   constexpr int D = 2;
   vec8 xa[D][KH];
-  Res4 rr[D][RES ? NT : 1];
+  vec8 rr[D][RES ? 16 / kRowsPerStore : 1];
 #pragma unroll
   for (int d = 0; d < D - 1; ++d)
     if (g + d * gstride < groups) request(g + d * gstride, xa[d], rr[d]);
@@ -852,18 +857,24 @@ gemm16_shortk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict_
       for (int j = 0; j < NT; ++j) {
         const f32x4 sc = *reinterpret_cast<const f32x4*>(&s_scale[j * 16 + 4 * (lane >> 4)]);
         const f32x4 sh = *reinterpret_cast<const f32x4*>(&s_shift[j * 16 + 4 * (lane >> 4)]);
-        Res4 out;
+        if (RES) {
+          f32x4 v4;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float v = __builtin_fmaf(acc[j][r], sc[r], sh[r]);
-          if (RES) v = __builtin_fmaf(epi.residual_scale, (float)rr[u][RES ? j : 0].v[r], v);
-          asm volatile("" : "+v"(v));  // one rounding to T for every element, see gemm16_dma_kernel's epilogue
-          if (epi.relu) v = v > 0.0f ? v : 0.0f;
-          out.v[r] = (T)v;
+          for (int r = 0; r < 4; ++r) v4[r] = __builtin_fmaf(acc[j][r], sc[r], sh[r]);
+          *reinterpret_cast<f32x4*>(my_stage + frow * kStageRow + (j * 16 + 4 * (lane >> 4)) * 4) = v4;
+        } else {
+          Res4 out;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float v = __builtin_fmaf(acc[j][r], sc[r], sh[r]);
+            asm volatile("" : "+v"(v));  // one rounding to T for every element, see gemm16_dma_kernel's epilogue
+            if (epi.relu) v = v > 0.0f ? v : 0.0f;
+            out.v[r] = (T)v;
+          }
+          *reinterpret_cast<Res4*>(my_stage + frow * kStageRow + (j * 16 + 4 * (lane >> 4)) * 2) = out;
         }
-        *reinterpret_cast<Res4*>(my_stage + frow * kStageRow + (j * 16 + 4 * (lane >> 4)) * 2) = out;
       }
-      // the wavefront's own 16 x NW tile comes back as whole rows: 16 bytes per lane, full lines per store
+      // the wavefront's own 16 x NW tile comes back as whole rows: 16 bytes of C per lane, full lines per store
       // (8-byte pieces of 32 contiguous bytes per row write at little more than half the rate)
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
@@ -872,8 +883,23 @@ gemm16_shortk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict_
       for (int i = 0; i < 16 / kRowsPerStore; ++i) {
         const int srow = i * kRowsPerStore + lane / kChunksPerRow;
         const int ch   = lane % kChunksPerRow;
-        const u32x4 v  = *reinterpret_cast<const u32x4*>(my_stage + srow * kStageRow + ch * 16);
-        const int row  = g * 16 + srow;
+        u32x4 v;
+        if (RES) {
+          const f32x4 lo = *reinterpret_cast<const f32x4*>(my_stage + srow * kStageRow + ch * 32);
+          const f32x4 hi = *reinterpret_cast<const f32x4*>(my_stage + srow * kStageRow + ch * 32 + 16);
+          vec8 out;
+#pragma unroll
+          for (int q = 0; q < 8; ++q) {
+            float t = __builtin_fmaf(epi.residual_scale, (float)rr[u][RES ? i : 0][q], q < 4 ? lo[q] : hi[q - 4]);
+            asm volatile("" : "+v"(t));
+            if (epi.relu) t = t > 0.0f ? t : 0.0f;
+            out[q] = (T)t;
+          }
+          v = *reinterpret_cast<const u32x4*>(&out);
+        } else {
+          v = *reinterpret_cast<const u32x4*>(my_stage + srow * kStageRow + ch * 16);
+        }
+        const int row = g * 16 + srow;
         if (row < M) {
           u32x4* dst = reinterpret_cast<u32x4*>(reinterpret_cast<T*>(C) + (int64_t)row * ldc + n0 + ch * 8);
           if (epi.streaming) {
