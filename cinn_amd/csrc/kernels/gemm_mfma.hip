@@ -758,7 +758,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Short reductions (K = 64 .. 256) with B stored [N][K] - 1x1 convolutions over few channels, attention scores:
+// Short reductions (K = 64; B stored [N][K], or [K][N] gathered once per block) - 1x1 convolutions over few channels:
 // 2 * K flop per output element make these products a stream of C (and of the residual), and a tiled kernel, whose
 // block waits for its operands, computes for a moment and then writes its tile, never has enough bytes in flight.
 // Here nothing is staged and nobody waits for a neighbour: a wavefront keeps its NT * 16 filter rows in registers as
@@ -770,7 +770,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 // the residual of the next group are requested before the current group is computed.  Per-column scale / shift sit
 // in LDS.  No block barrier after the start-up.
 // ---------------------------------------------------------------------------------------------------
-template <typename T, int NT, int KH, bool RES>
+template <typename T, int NT, int KH, bool RES, bool B_KC>
 __global__ void __launch_bounds__(256)
 gemm16_shortk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ C, int M, int N,
                      int64_t lda, int64_t ldb, int64_t ldc, DmaEpilogue epi, int64_t stride_a, int64_t stride_b,
@@ -810,7 +810,15 @@ gemm16_shortk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict_
   for (int j = 0; j < NT; ++j)
 #pragma unroll
     for (int kh = 0; kh < KH; ++kh)
-      wf[j][kh] = *reinterpret_cast<const vec8*>(B + (int64_t)(n0 + j * 16 + frow) * ldb + kh * 32 + fk);
+      if (B_KC) {
+        wf[j][kh] = *reinterpret_cast<const vec8*>(B + (int64_t)(n0 + j * 16 + frow) * ldb + kh * 32 + fk);
+      } else {
+        // B stored [K][N]: the 8 k values of a fragment are a column, gathered once per block
+        uint16_t col[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) col[q] = B[(int64_t)(kh * 32 + fk + q) * ldb + n0 + j * 16 + frow];
+        __builtin_memcpy(&wf[j][kh], col, 16);
+      }
   __syncthreads();
 
   const int groups  = (M + 15) >> 4;
@@ -1302,7 +1310,7 @@ void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
                      p.stride_b, p.stride_c, xcd_cols, sub_rows, sub_cols, geom);
 }
 
-// gemm16_shortk_kernel: K = 64, B stored [N][K], N a multiple of the 128 columns of a wavefront, at least 16384 rows.
+// gemm16_shortk_kernel: K = 64, either layout of B, N a multiple of the 128 columns of a wavefront, at least 16384 rows.
 // FLAGS_cinn_hip_gemm_shortk=0 switches it off.
 template <typename T, int NT, int KH>
 void LaunchShortK(const GemmProblem& p, hipStream_t stream) {
@@ -1321,14 +1329,21 @@ void LaunchShortK(const GemmProblem& p, hipStream_t stream) {
   epi.residual_scale = p.residual ? p.residual_scale : p.beta;
   epi.streaming      = !p.keep_in_cache && (int64_t)p.batch * p.m * p.n * 2 >= (16 << 20);
   dim3 grid(slots * ny, p.batch, 1);
-#define CINN_SHORTK(RES)                                                                                             \
-  hipLaunchKernelGGL((gemm16_shortk_kernel<T, NT, KH, RES>), grid, dim3(256), 0, stream,                              \
+#define CINN_SHORTK(RES, B_KC)                                                                                       \
+  hipLaunchKernelGGL((gemm16_shortk_kernel<T, NT, KH, RES, B_KC>), grid, dim3(256), 0, stream,                        \
                      static_cast<const uint16_t*>(p.a), static_cast<const uint16_t*>(p.b), static_cast<uint16_t*>(p.c), \
-                     p.m, p.n, (int64_t)p.k, (int64_t)p.k, (int64_t)p.n, epi, p.stride_a, p.stride_b, p.stride_c, ny)
+                     p.m, p.n, (int64_t)p.k, (int64_t)(B_KC ? p.k : p.n), (int64_t)p.n, epi, p.stride_a, p.stride_b,    \
+                     p.stride_c, ny)
   if (epi.residual) {
-    CINN_SHORTK(true);
+    if (p.trans_b) {
+      CINN_SHORTK(true, true);
+    } else {
+      CINN_SHORTK(true, false);
+    }
+  } else if (p.trans_b) {
+    CINN_SHORTK(false, true);
   } else {
-    CINN_SHORTK(false);
+    CINN_SHORTK(false, false);
   }
 #undef CINN_SHORTK
 }
@@ -1336,8 +1351,8 @@ void LaunchShortK(const GemmProblem& p, hipStream_t stream) {
 template <typename T>
 bool TryShortK(const GemmProblem& p, hipStream_t stream) {
   static const bool enabled = !(getenv("FLAGS_cinn_hip_gemm_shortk") && atoi(getenv("FLAGS_cinn_hip_gemm_shortk")) == 0);
-  if (!enabled || p.conv || p.trans_a || !p.trans_b) return false;
-  // measured against the tiled kernels (fp16, B [N][K]): 100352 x 256 x 64 17.0 against 22.7 us; with 64 columns, or a
+  if (!enabled || p.conv || p.trans_a) return false;
+  // measured against the tiled kernels (fp16): 100352 x 256 x 64 17.0 against 22.7 us; with 64 columns, or a
   // K of 128 or 256, or many small batch entries (the filter fragments are reloaded per block) the tiled kernels win
   if (p.k != 64 || p.n % 128 != 0 || p.m < 16384 || p.batch > 65535) return false;
   // 8-byte accesses to C and the residual, 16-byte accesses to A and B
