@@ -1354,7 +1354,7 @@ bool TryShortK(const GemmProblem& p, hipStream_t stream) {
   if (!enabled || p.conv || p.trans_a) return false;
   // measured against the tiled kernels (fp16): 100352 x 256 x 64 17.0 against 22.7 us; with 64 columns, or a
   // K of 128 or 256, or many small batch entries (the filter fragments are reloaded per block) the tiled kernels win
-  if (p.k != 64 || p.n % 128 != 0 || p.m < 16384 || p.batch > 65535) return false;
+  if (p.k != 64 || p.n % 128 != 0 || p.n > 8192 || p.m < 16384 || p.batch > 65535) return false;
   // 8-byte accesses to C and the residual, 16-byte accesses to A and B
   if (reinterpret_cast<uintptr_t>(p.a) % 16 != 0 || reinterpret_cast<uintptr_t>(p.b) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(p.c) % 8 != 0 || reinterpret_cast<uintptr_t>(p.residual) % 8 != 0 ||
