@@ -5,6 +5,7 @@
 #include <map>
 #include <sstream>
 
+#include "backends/host_stub.h"
 #include "frontend/computation.h"
 #include "frontend/net_builder.h"
 #include "hlir/op.h"
@@ -385,6 +386,43 @@ int cinn_amd_computation_run_instruction(cinn_amd_computation_t c, int32_t index
 
 int cinn_amd_list_operators(char* out, size_t cap, size_t* needed) {
   return Guard([&] { CopyOut(Join(cinn::hlir::framework::OpRegistry::Global().ListAllNames()), out, cap, needed); });
+}
+
+int cinn_amd_extern_api_names(char* out, size_t cap, size_t* needed) {
+  return Guard([&] { CopyOut(Join(cinn::backends::ExternApiRegistry::Global().Names()), out, cap, needed); });
+}
+
+int cinn_amd_host_stub_create(const char* api, const char* constants, void** fn) {
+  return Guard([&] {
+    namespace ir = cinn::ir;
+    CINN_CHECK(api && fn) << "null argument";
+    std::vector<ir::Expr> args = {ir::MakeVar("kernel_args", cinn::common::Handle()),
+                                  ir::MakeVar("kernel_args_num", cinn::common::Int(32))};
+    std::stringstream items(constants ? constants : "");
+    std::string item;
+    while (std::getline(items, item, ',')) {
+      if (item.empty()) continue;
+      CINN_CHECK(item.size() > 2 && item[1] == ':') << "bad constant '" << item << "' (want i:<int>, f:<float> or b:<0|1>)";
+      const std::string value = item.substr(2);
+      switch (item[0]) {
+        case 'i': args.push_back(ir::MakeIntImm(cinn::common::Int(64), std::stoll(value))); break;
+        case 'f': args.push_back(ir::Expr(static_cast<float>(std::stod(value)))); break;
+        case 'b': args.push_back(ir::Expr(value != "0")); break;
+        default: CINN_CHECK(false) << "bad constant '" << item << "'";
+      }
+    }
+    args.push_back(ir::MakeVar("kernel_stream", cinn::common::Handle()));
+    ir::LoweredFunc func;
+    func.name      = std::string("stub_of_") + api;
+    func.is_device = false;
+    func.body      = ir::MakeCall(cinn::common::Type(), api, args, ir::CallType::Extern);
+    auto closure   = cinn::backends::LowerHostFunction(func, {});
+    *fn            = reinterpret_cast<void*>(cinn::backends::HostStubPool::Global().Acquire(std::move(closure)));
+  });
+}
+
+int cinn_amd_host_stub_release(void* fn) {
+  return Guard([&] { cinn::backends::HostStubPool::Global().Release(reinterpret_cast<lower_func_ptr_g>(fn)); });
 }
 
 }  // extern "C"

@@ -44,6 +44,25 @@ void InvokeSoftmaxForward(const std::vector<BakedArg>& a, void* args, int32_t n,
   cinn_call_cudnn_softmax_forward(args, n, I(a[2]), I(a[3]), F(a[4]), F(a[5]), I(a[6]), I(a[7]), I(a[8]), I(a[9]),
                                   I(a[10]), I(a[11]), I(a[12]), I(a[13]), stream);
 }
+void InvokeBatchedCublas(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
+  cinn_call_batched_cublas(args, n, I(a[2]), B(a[3]), B(a[4]), B(a[5]), F(a[6]), F(a[7]), I(a[8]), I(a[9]), I(a[10]),
+                           I(a[11]), I(a[12]), I(a[13]), I(a[14]), I(a[15]), stream);
+}
+// the two convolution gradients share the forward call's argument list (format, alpha, beta, 19 extents)
+template <decltype(&cinn_call_cudnn_conv2d_backward_data) Fn>
+void InvokeConv2dBackward(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
+  Fn(args, n, I(a[2]), F(a[3]), F(a[4]), I(a[5]), I(a[6]), I(a[7]), I(a[8]), I(a[9]), I(a[10]), I(a[11]), I(a[12]),
+     I(a[13]), I(a[14]), I(a[15]), I(a[16]), I(a[17]), I(a[18]), I(a[19]), I(a[20]), I(a[21]), I(a[22]), I(a[23]), stream);
+}
+void InvokePool2dBackward(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
+  cinn_call_cudnn_pool2d_backward(args, n, I(a[2]), I(a[3]), F(a[4]), F(a[5]), I(a[6]), I(a[7]), I(a[8]), I(a[9]),
+                                  I(a[10]), I(a[11]), I(a[12]), I(a[13]), I(a[14]), I(a[15]), I(a[16]), I(a[17]),
+                                  I(a[18]), I(a[19]), stream);
+}
+void InvokeSoftmaxBackward(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
+  cinn_call_cudnn_softmax_backward(args, n, I(a[2]), I(a[3]), F(a[4]), F(a[5]), I(a[6]), I(a[7]), I(a[8]), I(a[9]),
+                                   I(a[10]), I(a[11]), I(a[12]), I(a[13]), stream);
+}
 void InvokeMemset(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
   cinn_call_cuda_memset(args, n, I(a[2]), static_cast<size_t>(a[3].i), stream);
 }
@@ -62,6 +81,12 @@ ExternApiRegistry::ExternApiRegistry() {
   Register("cinn_call_hip_conv2d_bn_relu", InvokeConv2dBnRelu, 24);
   Register("cinn_call_cudnn_pool2d_forward", InvokePool2dForward, 21);
   Register("cinn_call_cudnn_softmax_forward", InvokeSoftmaxForward, 15);
+  // (kernel_args, kernel_args_num, opside, trans_a, trans_b, trans_o, alpha, beta, a1..a4, b1..b4, kernel_stream)
+  Register("cinn_call_batched_cublas", InvokeBatchedCublas, 17);
+  Register("cinn_call_cudnn_conv2d_backward_data", InvokeConv2dBackward<&cinn_call_cudnn_conv2d_backward_data>, 25);
+  Register("cinn_call_cudnn_conv2d_backward_filter", InvokeConv2dBackward<&cinn_call_cudnn_conv2d_backward_filter>, 25);
+  Register("cinn_call_cudnn_pool2d_backward", InvokePool2dBackward, 21);
+  Register("cinn_call_cudnn_softmax_backward", InvokeSoftmaxBackward, 15);
   Register("cinn_call_cuda_memset", InvokeMemset, 5);
   Register("cinn_call_cuda_memcpy", InvokeMemcpy, 4);
 }

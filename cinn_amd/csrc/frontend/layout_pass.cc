@@ -119,10 +119,12 @@ class LayoutConverter {
         AttributeMap attrs   = ins->attrs;
         attrs["data_format"] = std::string("NHWC");
         Variable y;
-        if (HasTwin(x) || x->shape[1] % chunk == 0) {
+        if (x->shape[1] % chunk == 0) {
           y = emit_.Emit1("conv2d", {GetNhwc(x), FilterToOhwi(w)}, attrs);
         } else {
-          // few input channels (an image): the kernel reads the NCHW tensor and the [O][I][KH][KW] filter as they are
+          // a channel count that is not a whole number of 16-byte chunks (an image, or LeNet-style 6 / 12 channels,
+          // also when the producer left only a channels-last twin): the kernel reads the NCHW tensor and the
+          // [O][I][KH][KW] filter as they are
           EnsureNchw(x);
           EnsureNchw(w);
           attrs["input_layout"] = std::string("NCHW");

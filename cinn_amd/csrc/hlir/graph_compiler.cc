@@ -222,9 +222,20 @@ void Program::ExecuteGraph(void* stream) {
     // capturing stream does not allow: run the program once before recording it.
     for (auto& ins : instrs_) ins->Run(stream);
     CINN_HIP_STATUS(static_cast<int>(hipStreamSynchronize(s)));
+    // That run also sized the library's per-stream scratch (split-K partial sums, transposed operands), so the
+    // recorded calls find it large enough; scratch a later call outgrows is retired, never freed, and the addresses
+    // recorded here stay valid for every replay.
     hipGraph_t graph = nullptr;
     CINN_HIP_STATUS(static_cast<int>(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal)));
-    for (auto& ins : instrs_) ins->Run(stream);
+    try {
+      for (auto& ins : instrs_) ins->Run(stream);
+    } catch (...) {
+      // never leave the caller's stream in capture mode
+      hipGraph_t partial = nullptr;
+      (void)hipStreamEndCapture(s, &partial);
+      if (partial) (void)hipGraphDestroy(partial);
+      throw;
+    }
     CINN_HIP_STATUS(static_cast<int>(hipStreamEndCapture(s, &graph)));
     hipGraphExec_t exec = nullptr;
     CINN_HIP_STATUS(static_cast<int>(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0)));

@@ -1306,12 +1306,13 @@ ir::LoweredFuncRef OpLowerer::LowerLibraryCall(const Group& group) const {
     // argument list of CustomCallArgsForCublas (cinn/hlir/op/custom_call.cc:116-217)
     api = "cinn_call_cublas";
     bool ta = false, tb = false;
-    float alpha = 1.0f;
+    const bool trans_out = GetAttr<bool>(n->attrs, "trans_out", false);
+    const float alpha    = GetAttr<float>(n->attrs, "alpha", 1.0f);
+    const float beta     = GetAttr<float>(n->attrs, "beta", 0.0f);
     ShapeType a_shape, b_shape;
     if (op == "matmul") {
       ta      = GetAttr<bool>(n->attrs, "trans_a", false);
       tb      = GetAttr<bool>(n->attrs, "trans_b", false);
-      alpha   = GetAttr<float>(n->attrs, "alpha", 1.0f);
       a_shape = n->inputs[0]->shape;
       b_shape = n->inputs[1]->shape;
       if (a_shape.size() == 1) a_shape = ta ? ShapeType{a_shape[0], 1} : ShapeType{1, a_shape[0]};
@@ -1320,19 +1321,29 @@ ir::LoweredFuncRef OpLowerer::LowerLibraryCall(const Group& group) const {
       int xn = GetAttr<int>(n->attrs, "x_num_col_dims", 1), yn = GetAttr<int>(n->attrs, "y_num_col_dims", 1);
       const auto& xs = n->inputs[0]->shape;
       const auto& ys = n->inputs[1]->shape;
-      int m = 1, kk = 1, nn = 1;
-      for (int i = 0; i < xn; ++i) m *= xs[i];
-      for (size_t i = xn; i < xs.size(); ++i) kk *= xs[i];
-      for (size_t i = yn; i < ys.size(); ++i) nn *= ys[i];
-      a_shape = {m, kk};
-      b_shape = {kk, nn};
+      if (xn < 0) xn += static_cast<int>(xs.size());
+      if (yn < 0) yn += static_cast<int>(ys.size());
+      int a_height = 1, a_width = 1, b_height = 1, b_width = 1;
+      for (int i = 0; i < xn; ++i) a_height *= xs[i];
+      for (size_t i = xn; i < xs.size(); ++i) a_width *= xs[i];
+      for (int i = 0; i < yn; ++i) b_height *= ys[i];
+      for (size_t i = yn; i < ys.size(); ++i) b_width *= ys[i];
+      a_shape = {a_height, a_width};
+      b_shape = {b_height, b_width};
+      if (GetAttr<bool>(n->attrs, "is_infer", false)) {
+        // y is the transposed weight [N, K] (custom_call.cc:199-202)
+        CINN_CHECK_EQ(a_width, b_width) << "mul (is_infer): the K dimensions differ";
+        tb = true;
+      } else {
+        CINN_CHECK_EQ(a_width, b_height) << "mul: the K dimensions differ";
+      }
     }
     auto a4 = PadTo4(a_shape), b4 = PadTo4(b_shape);
     args.push_back(Expr(ta));
     args.push_back(Expr(tb));
-    args.push_back(Expr(false));  // trans_o
+    args.push_back(Expr(trans_out));
     args.push_back(Expr(alpha));
-    args.push_back(Expr(0.0f));  // beta
+    args.push_back(Expr(beta));
     push_ints({a4[0], a4[1], a4[2], a4[3], b4[0], b4[1], b4[2], b4[3]});
   } else if (op == "conv2d" || op == "hip_conv2d_bn_relu") {
     // argument list of CustomCallArgsForCudnnConvForward (custom_call.cc:338-388)

@@ -484,19 +484,32 @@ OpRegistry::OpRegistry() {
     op.infer_dtype = SameTypeAsFirst;
   }
   {
-    // mul (fc): x flattened at x_num_col_dims times y flattened at y_num_col_dims, y given as [N, K]
-    // when is_infer-style transposed weights are not used here: y is [K, N]
+    // mul (fc): x flattened at x_num_col_dims times y flattened at y_num_col_dims.  y is [K, N]; with is_infer it
+    // is the transposed weight [N, K] and the output takes y's leading dims (GetMulNewShapes,
+    // cinn/hlir/pe/transform.cc:186-250; InferShapeForMul, cinn/hlir/op/transform.cc:592-621)
     auto& op       = r->Register("mul");
     op.pattern     = OpPatternKind::kNonFusible;
     op.num_inputs  = 2;
     op.infer_shape = [](const std::vector<ShapeType>& in, const AttributeMap& a) {
       int xn = GetAttr<int>(a, "x_num_col_dims", 1), yn = GetAttr<int>(a, "y_num_col_dims", 1);
+      bool is_infer = GetAttr<bool>(a, "is_infer", false);
+      CINN_CHECK(in[0].size() >= 2 && in[1].size() >= 2) << "mul: operands need at least two dimensions";
+      if (xn < 0) xn += static_cast<int>(in[0].size());
+      if (yn < 0) yn += static_cast<int>(in[1].size());
+      CINN_CHECK(xn > 0 && xn < static_cast<int>(in[0].size())) << "mul: x_num_col_dims out of range";
+      CINN_CHECK(yn > 0 && yn < static_cast<int>(in[1].size())) << "mul: y_num_col_dims out of range";
       ShapeType out(in[0].begin(), in[0].begin() + xn);
-      out.insert(out.end(), in[1].begin() + yn, in[1].end());
-      int64_t kx = 1, ky = 1;
+      int64_t kx = 1, y_lead = 1, y_trail = 1;
       for (size_t i = xn; i < in[0].size(); ++i) kx *= in[0][i];
-      for (int i = 0; i < yn; ++i) ky *= in[1][i];
-      CINN_CHECK_EQ(kx, ky) << "mul: flattened inner dimensions differ";
+      for (int i = 0; i < yn; ++i) y_lead *= in[1][i];
+      for (size_t i = yn; i < in[1].size(); ++i) y_trail *= in[1][i];
+      if (is_infer) {
+        out.insert(out.end(), in[1].begin(), in[1].begin() + yn);
+        CINN_CHECK_EQ(kx, y_trail) << "mul (is_infer): the K dimensions of x and the transposed y differ";
+      } else {
+        out.insert(out.end(), in[1].begin() + yn, in[1].end());
+        CINN_CHECK_EQ(kx, y_lead) << "mul: flattened inner dimensions differ";
+      }
       return std::vector<ShapeType>{out};
     };
     op.infer_dtype = SameTypeAsFirst;

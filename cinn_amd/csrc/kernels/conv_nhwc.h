@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include "cinn_hip_runtime.h"
+#include "runtime/scratch.h"
 
 namespace cinn_hip_kernels {
 
@@ -35,7 +36,7 @@ void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream);
 // (K = kh * kw * c); both with this epilogue.  false when the shape does not qualify.
 bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream);
 // 256 bytes of zeros in device memory (what masked-out chunks are read from)
-const void* ConvZeroPage();
+inline const void* ConvZeroPage() { return ZeroPage(); }
 
 // depthwise convolutions (groups == channels in == channels out) on channels-last tensors, filter [C][KH][KW]
 // (conv_depthwise.hip): same epilogue; false when the shape does not qualify

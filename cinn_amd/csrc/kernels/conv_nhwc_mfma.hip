@@ -22,6 +22,7 @@
 
 #include <climits>
 #include <cstdint>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -502,39 +503,6 @@ TileChoice ChooseTile(int pixels, int oc) {
   return options[2];
 }
 
-// 256 bytes of zeros that masked-out chunks are read from
-const void* ZeroPage() {
-  static void* page = nullptr;
-  if (!page) {
-    CINN_HIP_CALL(hipMalloc(&page, 256));
-    CINN_HIP_CALL(hipMemset(page, 0, 256));
-    CINN_HIP_CALL(hipDeviceSynchronize());
-  }
-  return page;
-}
-
-// fp32 scratch for split-K partial sums, one buffer per stream (launches on different streams may overlap); grown on
-// demand and kept (the first, eager execution of a program sizes it, so graph capture never sees an allocation)
-float* Workspace(size_t bytes, hipStream_t stream) {
-  struct Buffer {
-    float* data{nullptr};
-    size_t capacity{0};
-  };
-  static std::mutex mu;
-  static std::map<hipStream_t, Buffer> buffers;
-  std::lock_guard<std::mutex> lock(mu);
-  Buffer& b = buffers[stream];
-  if (bytes > b.capacity) {
-    if (b.data) {
-      CINN_HIP_CALL(hipDeviceSynchronize());
-      CINN_HIP_CALL(hipFree(b.data));
-    }
-    CINN_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&b.data), bytes));
-    b.capacity = bytes;
-  }
-  return b.data;
-}
-
 // K splits: layers whose tile grid cannot fill the 256 CUs spend their time waiting for one block's serial chain of
 // loads; splitting the reduction puts several blocks of the same tile on different CUs
 int ChooseSplits(int tiles, int steps) {
@@ -550,28 +518,51 @@ int ChooseSplits(int tiles, int steps) {
   return splits;
 }
 
+// Where a launch takes its scratch from: the library's per-stream arena (the default), or a caller-fixed region that
+// must be large enough (the entry point that allocates nothing).
+struct ScratchSource {
+  float* fixed_partials{nullptr};   // null: the arena
+  size_t fixed_partials_bytes{0};
+  const void* zero_page{nullptr};   // null: the arena's page
+};
+
+// split count and K steps per split of one launch
+void PlanSplits(Params* p, int bm, int bn, int elem_bytes) {
+  const int bk    = 128 / elem_bytes;
+  const int tiles = ((p->pixels + bm - 1) / bm) * ((p->oc + bn - 1) / bn);
+  const int steps = (p->k_total + bk - 1) / bk;
+  p->splits          = ChooseSplits(tiles, steps);
+  p->steps_per_split = (steps + p->splits - 1) / p->splits;
+  p->splits          = (steps + p->steps_per_split - 1) / p->steps_per_split;
+}
+
 template <typename T, int BM, int BN, int WM, int WN, bool NCHW_IN>
-void Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream) {
+void Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream, const ScratchSource& src) {
   constexpr int PF = 2;  // K steps in flight per block
   auto kernel      = conv_nhwc_mfma_kernel<T, BM, BN, WM, WN, NCHW_IN, PF>;
   const int bytes  = LdsBytes(BM, BN, WM);
-  static bool configured = false;
-  if (!configured) {
+  static const bool configured = [&] {  // once per instantiation, thread-safe
     CINN_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
-    configured = true;
+    return true;
+  }();
+  (void)configured;
+  Params p = p_in;
+  PlanSplits(&p, BM, BN, sizeof(T));
+  const int tiles  = ((p.pixels + BM - 1) / BM) * ((p.oc + BN - 1) / BN);
+  float* workspace = nullptr;
+  // fp32 partial sums [split][pixel][oc]
+  if (p.splits > 1) {
+    const size_t need = (size_t)p.splits * p.pixels * p.oc * sizeof(float);
+    if (src.fixed_partials) {
+      CINN_RT_CHECK(need <= src.fixed_partials_bytes, "conv2d: %zu bytes of partial sums do not fit the fixed scratch", need);
+      workspace = src.fixed_partials;
+    } else {
+      workspace = static_cast<float*>(Scratch(ScratchKind::kSplitK, need, stream));
+    }
   }
-  Params p              = p_in;
-  constexpr int BK      = 128 / sizeof(T);
-  const int tiles       = ((p.pixels + BM - 1) / BM) * ((p.oc + BN - 1) / BN);
-  const int steps       = (p.k_total + BK - 1) / BK;
-  p.splits              = ChooseSplits(tiles, steps);
-  p.steps_per_split     = (steps + p.splits - 1) / p.splits;
-  p.splits              = (steps + p.steps_per_split - 1) / p.steps_per_split;
-  float* workspace      = nullptr;
-  if (p.splits > 1) workspace = Workspace((size_t)p.splits * p.pixels * p.oc * sizeof(float), stream);
   hipLaunchKernelGGL(kernel, dim3(tiles, p.splits), dim3(64 * WM * WN), bytes, stream, static_cast<const T*>(a.x),
                      static_cast<const T*>(a.w), static_cast<T*>(a.y), a.scale, a.shift, static_cast<const T*>(a.residual),
-                     workspace, ZeroPage(), p);
+                     workspace, src.zero_page ? src.zero_page : ZeroPage(), p);
   CINN_HIP_CALL(hipGetLastError());
   if (p.splits > 1) {
     if (p.oc % 4 == 0) {
@@ -587,24 +578,37 @@ void Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream) {
   }
 }
 
-template <typename T>
-void Dispatch(const ConvNhwcArgs& a, const Params& p, hipStream_t stream) {
+// block tile and wavefront grid of a launch: {BM, BN, WM, WN}
+struct TileShape {
+  int bm, bn, wm, wn;
+};
+TileShape TileFor(const ConvNhwcArgs& a, const Params& p) {
   TileChoice t = ChooseTile(p.pixels, p.oc);
+  if (a.nchw_input) return t.bm == 128 ? TileShape{128, 64, 2, 2} : TileShape{64, 64, 2, 2};
+  if (t.bm == 128 && t.bn == 128 && t.waves == 8) return {128, 128, 2, 4};
+  if (t.bm == 128 && t.bn == 128) return {128, 128, 2, 2};
+  if (t.bm == 128) return {128, 64, 2, 2};
+  return {64, 64, 2, 2};
+}
+
+template <typename T>
+void Dispatch(const ConvNhwcArgs& a, const Params& p, hipStream_t stream, const ScratchSource& src = ScratchSource()) {
+  const TileShape t = TileFor(a, p);
   if (a.nchw_input) {
     if (t.bm == 128)
-      Launch<T, 128, 64, 2, 2, true>(a, p, stream);
+      Launch<T, 128, 64, 2, 2, true>(a, p, stream, src);
     else
-      Launch<T, 64, 64, 2, 2, true>(a, p, stream);
+      Launch<T, 64, 64, 2, 2, true>(a, p, stream, src);
     return;
   }
-  if (t.bm == 128 && t.bn == 128 && t.waves == 8)
-    Launch<T, 128, 128, 2, 4, false>(a, p, stream);
+  if (t.bm == 128 && t.bn == 128 && t.wn == 4)
+    Launch<T, 128, 128, 2, 4, false>(a, p, stream, src);
   else if (t.bm == 128 && t.bn == 128)
-    Launch<T, 128, 128, 2, 2, false>(a, p, stream);
+    Launch<T, 128, 128, 2, 2, false>(a, p, stream, src);
   else if (t.bm == 128)
-    Launch<T, 128, 64, 2, 2, false>(a, p, stream);
+    Launch<T, 128, 64, 2, 2, false>(a, p, stream, src);
   else
-    Launch<T, 64, 64, 2, 2, false>(a, p, stream);
+    Launch<T, 64, 64, 2, 2, false>(a, p, stream, src);
 }
 
 int ChunkElems(const cinn_type_t& t) { return 16 / (t.bits / CHAR_BIT); }
@@ -621,27 +625,8 @@ void MagicFor(int d, unsigned* magic, unsigned* shift) {
   }
 }
 
-}  // namespace
-
-const void* ConvZeroPage() { return ZeroPage(); }
-
-bool ConvNhwcSupported(const ConvNhwcArgs& a) {
-  const bool is_float = a.type.code == cinn_type_float && (a.type.bits == 32 || a.type.bits == 16);
-  const bool is_bf16  = a.type.code == cinn_type_bfloat && a.type.bits == 16;
-  if (!is_float && !is_bf16) return false;
-  if (a.nchw_input) return true;
-  return a.c % ChunkElems(a.type) == 0;
-}
-
-void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream) {
-  CINN_RT_CHECK(ConvNhwcSupported(a), "conv2d (channels-last): unsupported type or channel count %d", a.c);
-  CINN_RT_CHECK((int64_t)a.n * a.h * a.w_in * a.c < INT_MAX && (int64_t)a.n * a.oh * a.ow * a.oc < INT_MAX,
-                "conv2d (channels-last): tensor too large for 32-bit offsets");
-  if (ConvStemSupported(a)) {
-    RunConvStem(a, stream);
-    return;
-  }
-  if (TryPointwiseConvAsGemm(a, stream)) return;
+// kernel parameters of one convolution (shapes, magic numbers of the index divisions)
+Params MakeParams(const ConvNhwcArgs& a) {
   Params p;
   p.n = a.n, p.h = a.h, p.w = a.w_in, p.c = a.c;
   p.oc = a.oc, p.kh = a.kh, p.kw = a.kw;
@@ -660,6 +645,29 @@ void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream) {
   MagicFor(a.c, &p.magic_c, &p.shift_c);
   MagicFor(a.kw, &p.magic_kw, &p.shift_kw);
   CINN_RT_CHECK((int64_t)a.oc * p.k_total < INT_MAX, "conv2d (channels-last): filter too large for 32-bit offsets");
+  return p;
+}
+
+}  // namespace
+
+bool ConvNhwcSupported(const ConvNhwcArgs& a) {
+  const bool is_float = a.type.code == cinn_type_float && (a.type.bits == 32 || a.type.bits == 16);
+  const bool is_bf16  = a.type.code == cinn_type_bfloat && a.type.bits == 16;
+  if (!is_float && !is_bf16) return false;
+  if (a.nchw_input) return true;
+  return a.c % ChunkElems(a.type) == 0;
+}
+
+void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream) {
+  CINN_RT_CHECK(ConvNhwcSupported(a), "conv2d (channels-last): unsupported type or channel count %d", a.c);
+  CINN_RT_CHECK((int64_t)a.n * a.h * a.w_in * a.c < INT_MAX && (int64_t)a.n * a.oh * a.ow * a.oc < INT_MAX,
+                "conv2d (channels-last): tensor too large for 32-bit offsets");
+  if (ConvStemSupported(a)) {
+    RunConvStem(a, stream);
+    return;
+  }
+  if (TryPointwiseConvAsGemm(a, stream)) return;
+  const Params p = MakeParams(a);
   if (a.type.code == cinn_type_bfloat) {
     Dispatch<__bf16>(a, p, stream);
   } else if (a.type.bits == 16) {

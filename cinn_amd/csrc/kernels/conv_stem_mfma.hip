@@ -18,6 +18,8 @@
 #include <cstdint>
 #include <cstdlib>
 
+#include <mutex>
+
 #include "kernels/conv_nhwc.h"
 #include "runtime/hip_check.h"
 
@@ -353,10 +355,14 @@ template <typename T, int STEPS>
 void Launch(const ConvNhwcArgs& a, const StemParams& p, hipStream_t stream) {
   auto kernel     = conv_stem_kernel<T, STEPS>;
   const int bytes = LdsBytes(p);
-  static int configured = 0;
-  if (bytes > configured) {
-    CINN_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
-    configured = bytes;
+  {
+    static std::mutex mu;  // per instantiation: the attribute only ever grows
+    static int configured = 0;
+    std::lock_guard<std::mutex> lock(mu);
+    if (bytes > configured) {
+      CINN_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+      configured = bytes;
+    }
   }
   // a few blocks per CU stride over the tiles: the filter staging is amortised and the tail is short
   int per_cu = (160 * 1024) / bytes;

@@ -1178,27 +1178,6 @@ transpose2d_kernel(const T* __restrict__ in, T* __restrict__ out, int rows, int 
   }
 }
 
-// scratch for transposed operands, one buffer per stream; grown on demand and kept
-char* TransposeWorkspace(size_t bytes, hipStream_t stream) {
-  struct Buffer {
-    char* data{nullptr};
-    size_t capacity{0};
-  };
-  static std::mutex mu;
-  static std::map<hipStream_t, Buffer> buffers;
-  std::lock_guard<std::mutex> lock(mu);
-  Buffer& b = buffers[stream];
-  if (bytes > b.capacity) {
-    if (b.data) {
-      CINN_HIP_CALL(hipDeviceSynchronize());
-      CINN_HIP_CALL(hipFree(b.data));
-    }
-    CINN_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&b.data), bytes));
-    b.capacity = bytes;
-  }
-  return b.data;
-}
-
 void LaunchTranspose(const void* in, void* out, int rows, int cols, int batch, int64_t in_stride, int elem_bytes,
                      hipStream_t stream) {
   dim3 grid((cols + 31) / 32, (rows + 31) / 32, batch);
@@ -1241,12 +1220,12 @@ struct GemmProblem {
 template <typename T, bool A_KC, bool B_KC>
 void LaunchFast16(const GemmProblem& p, hipStream_t stream) {
   auto kernel = gemm16_mfma_kernel<T, A_KC, B_KC>;
-  static bool configured = false;  // per instantiation
-  if (!configured) {
+  static const bool configured = [&] {  // once per instantiation, thread-safe
     CINN_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       2 * kStageBytes));
-    configured = true;
-  }
+    return true;
+  }();
+  (void)configured;
   int64_t lda = p.trans_a ? p.m : p.k;
   int64_t ldb = p.trans_b ? p.k : p.n;
   dim3 grid((p.m / kBM) * (p.n / kBN), p.batch, 1);
@@ -1559,7 +1538,7 @@ void RunGemm(const GemmProblem& p, hipStream_t stream) {
       const int batch_b    = !p.trans_b ? (p.stride_b == 0 ? 1 : p.batch) : 0;
       const size_t bytes_a = (size_t)batch_a * p.m * p.k * elem_bytes;
       const size_t bytes_b = (size_t)batch_b * p.k * p.n * elem_bytes;
-      char* scratch        = TransposeWorkspace(bytes_a + bytes_b, stream);
+      char* scratch        = static_cast<char*>(cinn_hip_kernels::Scratch(cinn_hip_kernels::ScratchKind::kTranspose, bytes_a + bytes_b, stream));
       if (p.trans_a) {  // stored [k][m]
         LaunchTranspose(p.a, scratch, p.k, p.m, batch_a, p.stride_a, elem_bytes, stream);
         a_base   = scratch;

@@ -1,4 +1,4 @@
-// Host-side runtime intrinsics that generated host stubs call: kernel launch, memset, memcpy.
+// Host-side runtime intrinsics that generated host stubs call: kernel launch and memcpy (memset: kernels/fill.hip).
 #include <hip/hip_runtime_api.h>
 
 #include "cinn_hip_runtime.h"
@@ -43,13 +43,6 @@ void cinn_call_hip_kernel(void* kernel_fn, void* v_args, int num_args, int grid_
 void cinn_call_cuda_kernel(void* kernel_fn, void* v_args, int num_args, int grid_x, int grid_y, int grid_z,
                            int block_x, int block_y, int block_z, void* stream) {
   cinn_call_hip_kernel(kernel_fn, v_args, num_args, grid_x, grid_y, grid_z, block_x, block_y, block_z, stream);
-}
-
-void cinn_call_cuda_memset(void* v_args, int num_args, int value, size_t count, void* stream) {
-  CINN_RT_CHECK(num_args == 1, "cinn_call_cuda_memset takes one output buffer, got %d arguments", num_args);
-  auto* args = static_cast<cinn_pod_value_t*>(v_args);
-  auto* out  = static_cast<cinn_buffer_t*>(args[0].value_.v_handle);
-  CINN_HIP_CALL(hipMemsetAsync(out->memory, value, count, static_cast<hipStream_t>(stream)));
 }
 
 void cinn_call_cuda_memcpy(void* v_args, int num_args, size_t count, void* stream) {

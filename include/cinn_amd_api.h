@@ -77,6 +77,18 @@ int cinn_amd_computation_run_instruction(cinn_amd_computation_t c, int32_t index
 /* names of all registered operators, ',' separated */
 int cinn_amd_list_operators(char* out, size_t cap, size_t* needed);
 
+/* Host stubs of single runtime-intrinsic calls, built the way a compiled program's library-call instructions are
+ * (the registered extern-function prototypes of cinn/runtime/cuda/cuda_intrinsics.cc:404-733 and the host function
+ * CodeGenCUDA_Host::LowerGPUKernelLauncher makes of such a call, cinn/backends/codegen_cuda_host.cc:35-168).
+ * cinn_amd_extern_api_names lists the intrinsics a host function may call, ',' separated.
+ * cinn_amd_host_stub_create builds the stub of `api(kernel_args, kernel_args_num, <constants>, kernel_stream)`;
+ * `constants` is a ','-separated list of `i:<int>`, `f:<float>` and `b:<0|1>` items in call order.  *fn is a
+ * `void (*)(void* pod_args, int32_t num_args, void* stream)` (lower_func_ptr_g) to be released with
+ * cinn_amd_host_stub_release. */
+int cinn_amd_extern_api_names(char* out, size_t cap, size_t* needed);
+int cinn_amd_host_stub_create(const char* api, const char* constants, void** fn);
+int cinn_amd_host_stub_release(void* fn);
+
 #ifdef __cplusplus
 }
 #endif

@@ -264,6 +264,18 @@ int cinn_hip_event_synchronize(void* event);
 int cinn_hip_event_elapsed_ms(void* start, void* stop, float* ms);
 const char* cinn_hip_error_string(int status);
 
+/* Library-owned device scratch (partial sums of split reductions in the convolution / GEMM kernels, transposed copies
+ * of GEMM operands).  The reference has no such buffer of its own: cuBLAS / cuDNN keep theirs inside their handles
+ * (cinn/runtime/cuda/cuda_util.cc:45-76 CublasHandle, 465-514 CudnnHandle with its workspace).  One buffer per stream
+ * and purpose, grown on demand by the cinn_call_* that needs it; an outgrown buffer is retired, not freed, because a
+ * captured graph may still hold its address, and no call waits for the device.  While a stream is being captured
+ * nothing can be allocated: reserve first (one eager run of the same calls does it, or this call; 0 = leave as is).
+ * cinn_hip_scratch_release_retired frees the retired buffers; only a caller that knows that no instantiated graph
+ * refers to them may call it. */
+int cinn_hip_scratch_reserve(void* stream, size_t split_k_bytes, size_t transpose_bytes);
+int cinn_hip_scratch_info(void* stream, size_t* split_k_capacity, size_t* transpose_capacity, size_t* retired_bytes);
+int cinn_hip_scratch_release_retired(void);
+
 /* Device descriptor consumed by schedules.  Replaces common::Target's cudaDeviceGetAttribute
  * queries (cinn/common/target.cc:55-84, 177-221).  Filled from the live device when one is
  * present, otherwise with the MI355X datasheet values (256 CUs, wave64, 160 KiB LDS per CU). */

@@ -39,6 +39,25 @@ def test_reference_intrinsic_names_present():
         assert hasattr(lib, name), name
 
 
+def test_every_declared_intrinsic_can_be_called_from_a_host_stub():
+    # every cinn_call_* of the header has a registered prototype, so a compiled program's host function can call it
+    # (REGISTER_EXTERN_FUNC_HELPER list, cinn/runtime/cuda/cuda_intrinsics.cc:404-733)
+    lib = _lib.load()
+    registered = set(_lib.read_string(lib.cinn_amd_extern_api_names).split(","))
+    declared = [n for n in _declared_functions("cinn_hip_runtime.h") if n.startswith("cinn_call_")]
+    assert len(declared) >= 14
+    assert not [n for n in declared if n not in registered], registered
+    # a stub is a real function pointer; wrong arity and unknown names are reported, not executed
+    fn = ctypes.c_void_p()
+    _lib.check(lib.cinn_amd_host_stub_create(b"cinn_call_cuda_memcpy", b"i:16", ctypes.byref(fn)))
+    assert fn.value
+    _lib.check(lib.cinn_amd_host_stub_release(fn))
+    assert lib.cinn_amd_host_stub_create(b"cinn_call_cuda_memcpy", b"i:16,i:3", ctypes.byref(fn)) != 0
+    assert "wrong number of arguments" in lib.cinn_amd_last_error().decode()
+    assert lib.cinn_amd_host_stub_create(b"cinn_call_nothing", b"", ctypes.byref(fn)) != 0
+    assert lib.cinn_amd_host_stub_create(b"cinn_call_cuda_memcpy", b"x:1", ctypes.byref(fn)) != 0
+
+
 def test_struct_layout_documented_numbers():
     assert ctypes.sizeof(runtime.cinn_type_t) == 12
     assert ctypes.sizeof(runtime.cinn_buffer_t) == 120

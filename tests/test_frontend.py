@@ -271,3 +271,26 @@ def test_reductions_over_non_trailing_axes_are_split_into_runs_and_steps():
     b = NetBuilder("sm")
     x = b.create_input(Float(32), [512, 1024], "x")
     assert compile_only(b, [b.softmax(x, axes=[-1])]).num_instructions() == 1
+
+
+@pytest.mark.parametrize("dtype,channels", [("float32", (3, 6, 8)), ("float16", (3, 12, 16))])
+def test_conv_with_a_ragged_channel_count_reads_nchw_even_when_a_channels_last_twin_exists(dtype, channels):
+    # LeNet-style chains: the second convolution's input (6 fp32 / 12 fp16 channels) is not a whole number of 16-byte
+    # chunks, so it must take the NCHW-reading form although its producer left a channels-last twin
+    from cinn_amd.common import Float
+    t = Float(32) if dtype == "float32" else Float(16)
+    c0, c1, c2 = channels
+    b = NetBuilder("ragged_" + dtype)
+    x = b.create_input(t, [2, c0, 12, 12], "x")
+    w1 = b.create_input(t, [c1, c0, 3, 3], "w1")
+    w2 = b.create_input(t, [c2, c1, 3, 3], "w2")
+    y = b.conv2d(b.relu(b.conv2d(x, w1, paddings=[1, 1])), w2, paddings=[1, 1])
+    comp = compile_only(b, [y])
+    convs = [g for g in comp.fusion_groups().splitlines() if "conv2d" in g]
+    assert len(convs) == 2, convs
+    for g, (image, filt) in zip(convs, (("x", "w1"), (None, "w2"))):
+        ins = g.split(" in: ")[1].split(" out: ")[0].split()
+        # the filter is taken as it is ([O][I][KH][KW]) and the activations are an NCHW tensor, never a channels-last twin
+        assert ins[1] == filt and not ins[0].startswith("nhwc_"), g
+        if image:
+            assert ins[0] == image, g

@@ -1,0 +1,196 @@
+"""The raw C-ABI path on the GPU, driven with ctypes only, the way the reference's own runtime tests drive theirs:
+hiprtc -> code object -> function handle -> cinn_call_cuda_kernel with buffer AND scalar pod arguments
+(cinn/runtime/cuda/cuda_module_test.cc:31-177, cinn/backends/compiler_test.cc:31-158), then the intrinsics no compiled
+program of the front end reaches: cinn_call_batched_cublas (cuda_util.cc:312-437), cinn_call_cuda_memset /
+cinn_call_cuda_memcpy (cuda_util.cc:439-462), and the same calls through host stubs built from their registered
+prototypes (cuda_intrinsics.cc:404-733).  Integer / byte results are bit-exact, fp32 products within 1e-5 of the sum
+of magnitudes."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from cinn_amd import _lib, runtime
+
+pytestmark = pytest.mark.gpu
+
+LAUNCH_ARGTYPES = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int] + [ctypes.c_int] * 6 + [ctypes.c_void_p]
+
+TWO_KERNELS = r'''
+#include "cinn_hip_runtime_source.h"
+// y[r][c] = a * x[r][c] + shift, on a 2-D grid; rows / cols bound the ragged edge
+extern "C" __global__ void saxpy2d(const float* __restrict__ x, float* __restrict__ y, int rows, int cols, float a, int shift) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int r = blockIdx.y * blockDim.y + threadIdx.y;
+  if (r < rows && c < cols) y[r * cols + c] = a * x[r * cols + c] + (float)shift;
+}
+// one wavefront per row: out[r] = sum of the row through the device library's 64-lane all-reduce
+extern "C" __global__ void row_sum64(const int* __restrict__ x, int* __restrict__ out, int cols) {
+  int acc = 0;
+  for (int c = threadIdx.x; c < cols; c += 64) acc += x[blockIdx.x * cols + c];
+  acc = cinn_wave_shuffle_sum_int32_internal(acc);
+  if (threadIdx.x == 0) out[blockIdx.x] = acc;
+}
+'''
+
+
+def scalar_pods(lib, buffers, scalars):
+    """cinn_pod_value_t[]: buffers first, then ("i", v) / ("f", v) scalars, as a host stub packs kernel arguments"""
+    arr = (runtime.cinn_pod_value_t * (len(buffers) + len(scalars)))()
+    for i, b in enumerate(buffers):
+        lib.cinn_hip_pod_from_buffer(ctypes.byref(arr[i]), ctypes.byref(b.buffer))
+    for j, (kind, v) in enumerate(scalars):
+        slot = ctypes.byref(arr[len(buffers) + j])
+        if kind == "i":
+            lib.cinn_hip_pod_from_int32(slot, ctypes.c_int32(v))
+        else:
+            lib.cinn_hip_pod_from_float(slot, ctypes.c_float(v))
+    return arr
+
+
+def test_rtc_module_get_function_and_launch_with_buffer_and_scalar_args(gpu, rng):
+    lib = _lib.load()
+    lib.cinn_call_cuda_kernel.argtypes = LAUNCH_ARGTYPES
+    image = runtime.rtc_compile(TWO_KERNELS)
+    module = runtime.Module(image)
+    # 2-D grid, ragged on both axes, buffer + int32 + float arguments
+    rows, cols = 37, 150
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    X, Y = runtime.DeviceBuffer.from_numpy(x), runtime.DeviceBuffer((rows, cols), "float32")
+    Y.copy_from(np.full((rows, cols), -7.0, np.float32))
+    args = scalar_pods(lib, [X, Y], [("i", rows), ("i", cols), ("f", 2.5), ("i", -3)])
+    lib.cinn_call_cuda_kernel(module.get_function("saxpy2d"), args, 6, (cols + 31) // 32, (rows + 7) // 8, 1, 32, 8, 1, None)
+    runtime.synchronize()
+    assert np.array_equal(Y.numpy(), np.float32(2.5) * x + np.float32(-3.0))
+    # second kernel of the same module: the device library's wavefront reduction, bit-exact
+    xi = rng.integers(-1000, 1000, (19, 333), dtype=np.int32)
+    XI, OUT = runtime.DeviceBuffer.from_numpy(xi), runtime.DeviceBuffer((19,), "int32")
+    args = scalar_pods(lib, [XI, OUT], [("i", 333)])
+    stream = runtime.Stream()
+    lib.cinn_call_cuda_kernel(module.get_function("row_sum64"), args, 3, 19, 1, 1, 64, 1, 1, stream.handle)
+    stream.synchronize()
+    assert np.array_equal(OUT.numpy(), xi.sum(axis=1, dtype=np.int32))
+    # an unknown kernel name is an error status, not a crash
+    fn = ctypes.c_void_p()
+    assert lib.cinn_hip_module_get_function(module.handle, b"no_such_kernel", ctypes.byref(fn)) != 0
+
+
+BATCHED_ARGTYPES = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_bool, ctypes.c_bool, ctypes.c_bool,
+                    ctypes.c_float, ctypes.c_float] + [ctypes.c_int] * 8 + [ctypes.c_void_p]
+
+
+def batched_case(rng, opside, trans_o, pairs=3, m=48, n=40, k=24):
+    """shared operand S and `pairs` others; opside 0: S is the left operand A [m,k], others are B_i [k,n];
+    opside 1: S is the right operand B [k,n], others are A_i [m,k]"""
+    if opside == 0:
+        shared = rng.standard_normal((m, k)).astype(np.float32)
+        others = [rng.standard_normal((k, n)).astype(np.float32) for _ in range(pairs)]
+        wants = [shared.astype(np.float64) @ o.astype(np.float64) for o in others]
+        scales = [np.abs(shared).astype(np.float64) @ np.abs(o).astype(np.float64) for o in others]
+    else:
+        shared = rng.standard_normal((k, n)).astype(np.float32)
+        others = [rng.standard_normal((m, k)).astype(np.float32) for _ in range(pairs)]
+        wants = [o.astype(np.float64) @ shared.astype(np.float64) for o in others]
+        scales = [np.abs(o).astype(np.float64) @ np.abs(shared).astype(np.float64) for o in others]
+    if trans_o:
+        wants, scales = [w.T for w in wants], [s.T for s in scales]
+    return shared, others, wants, scales
+
+
+@pytest.mark.parametrize("via_stub", [False, True])
+@pytest.mark.parametrize("trans_o", [False, True])
+@pytest.mark.parametrize("opside", [0, 1])
+def test_batched_cublas_shares_one_operand_over_several_products(gpu, rng, opside, trans_o, via_stub):
+    lib = _lib.load()
+    lib.cinn_call_batched_cublas.argtypes = BATCHED_ARGTYPES
+    m, n, k = 48, 40, 24
+    shared, others, wants, scales = batched_case(rng, opside, trans_o, 3, m, n, k)
+    S = runtime.DeviceBuffer.from_numpy(shared)
+    O = [runtime.DeviceBuffer.from_numpy(o) for o in others]
+    C = [runtime.DeviceBuffer(w.shape, "float32") for w in wants]
+    c0 = [rng.standard_normal(w.shape).astype(np.float32) for w in wants]
+    for buf, init in zip(C, c0):
+        buf.copy_from(init)
+    args = runtime.pod_args([S] + O + C)
+    alpha, beta = 0.5, 2.0
+    if via_stub:
+        consts = "i:%d,b:0,b:0,b:%d,f:%r,f:%r,i:1,i:1,i:%d,i:%d,i:1,i:1,i:%d,i:%d" % (opside, int(trans_o), alpha, beta, m, k, k, n)
+        fn = ctypes.c_void_p()
+        _lib.check(lib.cinn_amd_host_stub_create(b"cinn_call_batched_cublas", consts.encode(), ctypes.byref(fn)))
+        stub = ctypes.CFUNCTYPE(None, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p)(fn.value)
+        stub(ctypes.cast(args, ctypes.c_void_p), 7, None)
+        _lib.check(lib.cinn_amd_host_stub_release(fn))
+    else:
+        lib.cinn_call_batched_cublas(args, 7, opside, False, False, trans_o, alpha, beta, 1, 1, m, k, 1, 1, k, n, None)
+    runtime.synchronize()
+    for buf, want, scale, init in zip(C, wants, scales, c0):
+        got = buf.numpy().astype(np.float64)
+        ref = alpha * want + beta * init.astype(np.float64)
+        assert np.all(np.abs(got - ref) <= 1e-5 * (alpha * scale + beta * np.abs(init)) + 1e-30)
+
+
+@pytest.mark.parametrize("count,offset", [(0, 0), (1, 0), (15, 3), (4096, 0), (100003, 5), (1 << 22, 16)])
+def test_memset_intrinsic_writes_exactly_count_bytes(gpu, count, offset):
+    lib = _lib.load()
+    lib.cinn_call_cuda_memset.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p]
+    total = count + 64
+    base = runtime.DeviceBuffer((total,), "uint8")
+    base.copy_from(np.full(total, 0x5A, np.uint8))
+    # a view that starts `offset` bytes into the allocation: unaligned heads and tails must be handled
+    view = runtime.cinn_buffer_t()
+    dims = (ctypes.c_int32 * 1)(total - offset)
+    lib.cinn_hip_buffer_init(ctypes.byref(view), ctypes.c_void_p(base.ptr.value + offset), 1, 8, dims, 1)
+    arr = (runtime.cinn_pod_value_t * 1)()
+    lib.cinn_hip_pod_from_buffer(ctypes.byref(arr[0]), ctypes.byref(view))
+    lib.cinn_call_cuda_memset(arr, 1, 0x1C3, count, None)  # the value is truncated to a byte like memset's
+    runtime.synchronize()
+    want = np.full(total, 0x5A, np.uint8)
+    want[offset:offset + count] = 0xC3
+    assert np.array_equal(base.numpy(), want)
+
+
+def test_memcpy_intrinsic_and_its_host_stub(gpu, rng):
+    lib = _lib.load()
+    lib.cinn_call_cuda_memcpy.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p]
+    x = rng.integers(0, 255, 70001, dtype=np.uint8)
+    X, Y = runtime.DeviceBuffer.from_numpy(x), runtime.DeviceBuffer((70001,), "uint8")
+    Y.copy_from(np.zeros(70001, np.uint8))
+    args = runtime.pod_args([X, Y])
+    lib.cinn_call_cuda_memcpy(args, 2, 60000, None)
+    runtime.synchronize()
+    got = Y.numpy()
+    assert np.array_equal(got[:60000], x[:60000]) and not got[60000:].any()
+    # the same call as a compiled program would make it: through a host stub with the count baked in
+    fn = ctypes.c_void_p()
+    _lib.check(lib.cinn_amd_host_stub_create(b"cinn_call_cuda_memcpy", b"i:70001", ctypes.byref(fn)))
+    stub = ctypes.CFUNCTYPE(None, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p)(fn.value)
+    stream = runtime.Stream()
+    stub(ctypes.cast(args, ctypes.c_void_p), 2, stream.handle)
+    stream.synchronize()
+    _lib.check(lib.cinn_amd_host_stub_release(fn))
+    assert np.array_equal(Y.numpy(), x)
+
+
+def test_memset_in_a_captured_graph_replays_correctly(gpu):
+    """a fill recorded into a HIP graph must do its work on every replay, with eager work in between"""
+    lib = _lib.load()
+    lib.cinn_call_cuda_memset.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p]
+    hip = ctypes.CDLL("libamdhip64.so")
+    n = 1 << 16
+    Y = runtime.DeviceBuffer((n,), "uint8")
+    arr = runtime.pod_args([Y])
+    stream = runtime.Stream()
+    graph, graph_exec = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipStreamBeginCapture(stream.handle, 1) == 0  # hipStreamCaptureModeThreadLocal
+    lib.cinn_call_cuda_memset(arr, 1, 0x11, n - 7, stream.handle)
+    assert hip.hipStreamEndCapture(stream.handle, ctypes.byref(graph)) == 0
+    assert hip.hipGraphInstantiate(ctypes.byref(graph_exec), graph, None, None, ctypes.c_size_t(0)) == 0
+    want = np.full(n, 0xEE, np.uint8)
+    want[:n - 7] = 0x11
+    for replay in range(4):
+        Y.copy_from(np.full(n, 0xEE, np.uint8))  # eager work between the replays
+        assert hip.hipGraphLaunch(graph_exec, stream.handle) == 0
+        stream.synchronize()
+        assert np.array_equal(Y.numpy(), want), "replay %d" % replay
+    hip.hipGraphExecDestroy(graph_exec)
+    hip.hipGraphDestroy(graph)

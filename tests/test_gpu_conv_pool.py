@@ -485,3 +485,27 @@ def test_pointwise_convolution_on_the_gemm_kernel(gpu, dtype, tol, alpha, beta, 
     want = alpha * conv + beta * y0
     scale = alpha * np.einsum("oc,nchw->nohw", np.abs(w2), np.abs(x).astype(np.float64)) + beta * np.abs(y0)
     assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-3 * scale) + 2.0 ** -24)
+
+
+@pytest.mark.parametrize("dtype,channels,tol", [("float32", (3, 6, 8), 1e-5), ("float16", (3, 12, 16), 1e-2)])
+def test_conv_chain_through_a_ragged_channel_count(gpu, dtype, channels, tol):
+    # LeNet-style: the middle tensor has 6 (fp32) / 12 (fp16) channels, not a whole number of 16-byte chunks, so the
+    # second convolution must read NCHW although the first one produced a channels-last tensor
+    npdt = np.dtype(dtype).type
+    c0, c1, c2 = channels
+    rng = np.random.default_rng(c1)
+    x = rng.standard_normal((2, c0, 12, 13)).astype(npdt)
+    w1 = (rng.standard_normal((c1, c0, 3, 3)) * np.sqrt(2.0 / (c0 * 9))).astype(npdt)
+    w2 = (rng.standard_normal((c2, c1, 3, 3)) * np.sqrt(2.0 / (c1 * 9))).astype(npdt)
+    b = NetBuilder("ragged_chain")
+    t = Float(32) if dtype == "float32" else Float(16)
+    X, W1, W2 = b.create_input(t, list(x.shape), "x"), b.create_input(t, list(w1.shape), "w1"), b.create_input(t, list(w2.shape), "w2")
+    y = b.conv2d(b.relu(b.conv2d(X, W1, paddings=[1, 1])), W2, paddings=[1, 1], strides=[2, 2])
+    (got,), _ = run(b, {X: x, W1: w1, W2: w2}, [y])
+    mid = np.maximum(oracle.conv2d_nchw(x, w1, (1, 1), (1, 1)), 0).astype(npdt)
+    want = oracle.conv2d_nchw(mid, w2, (2, 2), (1, 1)).astype(np.float64)
+    scale = conv_scale(mid.astype(np.float32), w2.astype(np.float32), (2, 2), (1, 1))
+    assert got.shape == want.shape
+    # the middle tensor is rounded to the storage type on both sides; fp16 inputs of the second sum may differ by one
+    # ulp, which the magnitude scale absorbs
+    assert np.all(np.abs(got.astype(np.float64) - want) <= tol * np.maximum(np.abs(want), 0.1 * scale) + 2.0 ** -24)
