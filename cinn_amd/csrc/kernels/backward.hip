@@ -272,6 +272,7 @@ void cinn_call_cudnn_conv2d_backward_data(void* v_args, int num_args, int format
                                           int filter_h, int filter_w, int pad_h, int pad_w, int stride_h, int stride_w,
                                           int dilation_h, int dilation_w, int groups, int output_n, int output_c,
                                           int output_h, int output_w, void* stream) {
+  CINN_HIP_CLEAR_STALE_ERROR();
   CINN_RT_CHECK(num_args == 3, "cinn_call_cudnn_conv2d_backward_data takes w, dy and dx, got %d arguments", num_args);
   const ConvDims p = MakeConvDims("conv2d_backward_data", format, alpha, beta, input_n, input_c, input_h, input_w, filter_n,
                                   filter_c, filter_h, filter_w, pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w,
@@ -305,6 +306,7 @@ void cinn_call_cudnn_conv2d_backward_filter(void* v_args, int num_args, int form
                                             int filter_h, int filter_w, int pad_h, int pad_w, int stride_h,
                                             int stride_w, int dilation_h, int dilation_w, int groups, int output_n,
                                             int output_c, int output_h, int output_w, void* stream) {
+  CINN_HIP_CLEAR_STALE_ERROR();
   CINN_RT_CHECK(num_args == 3, "cinn_call_cudnn_conv2d_backward_filter takes x, dy and dw, got %d arguments", num_args);
   const ConvDims p = MakeConvDims("conv2d_backward_filter", format, alpha, beta, input_n, input_c, input_h, input_w,
                                   filter_n, filter_c, filter_h, filter_w, pad_h, pad_w, stride_h, stride_w, dilation_h,
@@ -338,6 +340,7 @@ void cinn_call_cudnn_pool2d_backward(void* v_args, int num_args, int mode, int f
                                      int input_n, int input_c, int input_h, int input_w, int kernel_h, int kernel_w,
                                      int pad_h, int pad_w, int stride_h, int stride_w, int output_n, int output_c,
                                      int output_h, int output_w, void* stream) {
+  CINN_HIP_CLEAR_STALE_ERROR();
   CINN_RT_CHECK(num_args == 4, "cinn_call_cudnn_pool2d_backward takes x, y, dy and dx, got %d arguments", num_args);
   CINN_RT_CHECK(format == 0 || format == 1, "pool2d_backward: unknown tensor format %d", format);
   CINN_RT_CHECK(mode >= 0 && mode <= 3, "pool2d_backward: unknown pooling mode %d", mode);
@@ -380,6 +383,7 @@ void cinn_call_cudnn_pool2d_backward(void* v_args, int num_args, int mode, int f
 void cinn_call_cudnn_softmax_backward(void* v_args, int num_args, int mode, int format, float alpha, float beta,
                                       int input_n, int input_c, int input_h, int input_w, int output_n, int output_c,
                                       int output_h, int output_w, void* stream) {
+  CINN_HIP_CLEAR_STALE_ERROR();
   CINN_RT_CHECK(num_args == 3, "cinn_call_cudnn_softmax_backward takes y, dy and dx, got %d arguments", num_args);
   CINN_RT_CHECK(format == 0, "softmax_backward: only NCHW (format 0) is implemented, got format %d", format);
   CINN_RT_CHECK(mode == 0 || mode == 1, "softmax_backward: unknown mode %d", mode);

@@ -360,6 +360,7 @@ void cinn_call_cudnn_conv2d_forward(void* v_args, int num_args, int format, floa
                                     int filter_w, int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h,
                                     int dilation_w, int groups, int output_n, int output_c, int output_h,
                                     int output_w, void* stream) {
+  CINN_HIP_CLEAR_STALE_ERROR();
   CINN_RT_CHECK(num_args == 3, "cinn_call_cudnn_conv2d_forward takes x, w and y, got %d arguments", num_args);
   RunConv(BufferArg(v_args, 0), BufferArg(v_args, 1), BufferArg(v_args, 2), nullptr, nullptr, nullptr, 0, format, alpha, beta,
           input_n, input_c, input_h, input_w, filter_n, filter_c, filter_h, filter_w, pad_h, pad_w, stride_h, stride_w,
@@ -370,6 +371,7 @@ void cinn_call_hip_conv2d_bn_relu(void* v_args, int num_args, int format, int re
                                   int input_h, int input_w, int filter_n, int filter_c, int filter_h, int filter_w,
                                   int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
                                   int groups, int output_n, int output_c, int output_h, int output_w, void* stream) {
+  CINN_HIP_CLEAR_STALE_ERROR();
   CINN_RT_CHECK(num_args == 5 || num_args == 6,
                 "cinn_call_hip_conv2d_bn_relu takes x, w, scale, shift, [residual] and y, got %d arguments", num_args);
   cinn_buffer_t* scale = BufferArg(v_args, 2);

@@ -31,6 +31,7 @@ fill_bytes_kernel(unsigned char* dst, unsigned char value, size_t count, size_t 
 }  // namespace
 
 extern "C" void cinn_call_cuda_memset(void* v_args, int num_args, int value, size_t count, void* stream) {
+  CINN_HIP_CLEAR_STALE_ERROR();
   CINN_RT_CHECK(num_args == 1, "cinn_call_cuda_memset takes one output buffer, got %d arguments", num_args);
   auto* args = static_cast<cinn_pod_value_t*>(v_args);
   CINN_RT_CHECK(args[0].type_code_ == CINN_POD_BUFFER_P, "cinn_call_cuda_memset: the argument is not a buffer");

@@ -1690,6 +1690,7 @@ extern "C" {
 // Leading dimensions broadcast: an operand whose leading dims are 1 is shared by every batch.
 void cinn_call_cublas(void* v_args, int num_args, bool trans_a, bool trans_b, bool trans_o, float alpha, float beta,
                       int a1, int a2, int a3, int a4, int b1, int b2, int b3, int b4, void* stream) {
+  CINN_HIP_CLEAR_STALE_ERROR();
   CINN_RT_CHECK(num_args == 3, "cinn_call_cublas takes A, B and C, got %d arguments", num_args);
   cinn_buffer_t* A = BufferArg(v_args, 0);
   cinn_buffer_t* B = BufferArg(v_args, 1);

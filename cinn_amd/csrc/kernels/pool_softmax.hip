@@ -267,6 +267,7 @@ void cinn_call_cudnn_pool2d_forward(void* v_args, int num_args, int mode, int fo
                                     int input_n, int input_c, int input_h, int input_w, int kernel_h, int kernel_w,
                                     int pad_h, int pad_w, int stride_h, int stride_w, int output_n, int output_c,
                                     int output_h, int output_w, void* stream) {
+  CINN_HIP_CLEAR_STALE_ERROR();
   CINN_RT_CHECK(num_args == 2, "cinn_call_cudnn_pool2d_forward takes x and y, got %d arguments", num_args);
   CINN_RT_CHECK(format == 0 || format == 1, "pool2d: unknown tensor format %d", format);
   CINN_RT_CHECK(mode >= 0 && mode <= 3, "pool2d: unknown pooling mode %d", mode);
@@ -313,6 +314,7 @@ void cinn_call_cudnn_pool2d_forward(void* v_args, int num_args, int mode, int fo
 void cinn_call_cudnn_softmax_forward(void* v_args, int num_args, int mode, int format, float alpha, float beta,
                                      int input_n, int input_c, int input_h, int input_w, int output_n, int output_c,
                                      int output_h, int output_w, void* stream) {
+  CINN_HIP_CLEAR_STALE_ERROR();
   CINN_RT_CHECK(num_args == 2, "cinn_call_cudnn_softmax_forward takes x and y, got %d arguments", num_args);
   CINN_RT_CHECK(format == 0, "softmax: only NCHW (format 0) is implemented, got format %d", format);
   CINN_RT_CHECK(mode == 0 || mode == 1, "softmax: unknown mode %d", mode);

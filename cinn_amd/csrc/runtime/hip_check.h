@@ -26,3 +26,8 @@
       abort();                                                                    \
     }                                                                             \
   } while (0)
+
+// A kernel launched with hipLaunchKernelGGL reports failure through the thread's sticky "last error", which an earlier,
+// unrelated HIP call (the application's own, or a status-returning cinn_hip_* call that failed) may have left set.
+// Every cinn_call_* intrinsic starts by clearing it, so that the check after its launches sees its own errors only.
+#define CINN_HIP_CLEAR_STALE_ERROR() (void)hipGetLastError()

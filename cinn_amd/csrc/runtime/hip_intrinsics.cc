@@ -12,6 +12,7 @@ extern "C" {
 
 void cinn_call_hip_kernel(void* kernel_fn, void* v_args, int num_args, int grid_x, int grid_y, int grid_z,
                           int block_x, int block_y, int block_z, void* stream) {
+  CINN_HIP_CLEAR_STALE_ERROR();
   CINN_RT_CHECK(kernel_fn != nullptr, "cinn_call_hip_kernel: null kernel function");
   CINN_RT_CHECK(num_args >= 0 && (num_args == 0 || v_args != nullptr), "cinn_call_hip_kernel: bad argument list");
   CINN_RT_CHECK(grid_x > 0 && grid_y > 0 && grid_z > 0 && block_x > 0 && block_y > 0 && block_z > 0,

@@ -36,11 +36,17 @@ int cinn_hip_module_get_function(cinn_hip_module_t m, const char* name, void** k
   }
   if (!m->module) {
     hipError_t st = hipModuleLoadData(&m->module, m->image.data());
-    if (st != hipSuccess) return static_cast<int>(st);
+    if (st != hipSuccess) {
+      (void)hipGetLastError();  // reported through the status, not left behind as the thread's sticky error
+      return static_cast<int>(st);
+    }
   }
   hipFunction_t fn = nullptr;
   hipError_t st    = hipModuleGetFunction(&fn, m->module, name);
-  if (st != hipSuccess) return static_cast<int>(st);
+  if (st != hipSuccess) {
+    (void)hipGetLastError();
+    return static_cast<int>(st);
+  }
   m->functions[name] = fn;
   *kernel_fn         = fn;
   return 0;

@@ -17,6 +17,15 @@ static_assert(offsetof(cinn_buffer_t, memory_size) == 88, "cinn_buffer_t::memory
 static_assert(sizeof(cinn_pod_value_t) == 16, "cinn_pod_value_t must stay 16 bytes");
 static_assert(offsetof(cinn_pod_value_t, value_) == 8, "cinn_pod_value_t::value_ offset");
 
+namespace {
+// status of a HIP call for a status-returning entry point: the error is reported through the return value, so the
+// thread's sticky "last error" is cleared - it must not surface later in an unrelated launch check
+int Status(hipError_t st) {
+  if (st != hipSuccess) (void)hipGetLastError();
+  return static_cast<int>(st);
+}
+}  // namespace
+
 extern "C" {
 
 void cinn_hip_buffer_init(cinn_buffer_t* buf, void* device_ptr, int32_t type_code, int32_t bits, const int32_t* dims,
@@ -64,36 +73,36 @@ int cinn_hip_device_count(int* count) {
   return static_cast<int>(st);
 }
 
-int cinn_hip_malloc(void** dptr, size_t bytes) { return static_cast<int>(hipMalloc(dptr, bytes ? bytes : 1)); }
-int cinn_hip_free(void* dptr) { return static_cast<int>(hipFree(dptr)); }
+int cinn_hip_malloc(void** dptr, size_t bytes) { return Status(hipMalloc(dptr, bytes ? bytes : 1)); }
+int cinn_hip_free(void* dptr) { return Status(hipFree(dptr)); }
 int cinn_hip_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream) {
-  if (stream) return static_cast<int>(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)));
-  return static_cast<int>(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+  if (stream) return Status(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)));
+  return Status(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
 }
 int cinn_hip_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream) {
   if (stream) {
     hipError_t st = hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream));
     if (st != hipSuccess) return static_cast<int>(st);
-    return static_cast<int>(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    return Status(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
   }
-  return static_cast<int>(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+  return Status(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
 }
 int cinn_hip_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream) {
-  return static_cast<int>(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)));
+  return Status(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)));
 }
 int cinn_hip_memset(void* dst, int value, size_t bytes, void* stream) {
-  return static_cast<int>(hipMemsetAsync(dst, value, bytes, static_cast<hipStream_t>(stream)));
+  return Status(hipMemsetAsync(dst, value, bytes, static_cast<hipStream_t>(stream)));
 }
-int cinn_hip_device_synchronize(void) { return static_cast<int>(hipDeviceSynchronize()); }
+int cinn_hip_device_synchronize(void) { return Status(hipDeviceSynchronize()); }
 int cinn_hip_stream_create(void** stream) {
   hipStream_t s = nullptr;
   hipError_t st = hipStreamCreate(&s);  // default priority only
   *stream       = s;
   return static_cast<int>(st);
 }
-int cinn_hip_stream_destroy(void* stream) { return static_cast<int>(hipStreamDestroy(static_cast<hipStream_t>(stream))); }
+int cinn_hip_stream_destroy(void* stream) { return Status(hipStreamDestroy(static_cast<hipStream_t>(stream))); }
 int cinn_hip_stream_synchronize(void* stream) {
-  return static_cast<int>(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  return Status(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
 }
 int cinn_hip_event_create(void** event) {
   hipEvent_t e  = nullptr;
@@ -101,13 +110,13 @@ int cinn_hip_event_create(void** event) {
   *event        = e;
   return static_cast<int>(st);
 }
-int cinn_hip_event_destroy(void* event) { return static_cast<int>(hipEventDestroy(static_cast<hipEvent_t>(event))); }
+int cinn_hip_event_destroy(void* event) { return Status(hipEventDestroy(static_cast<hipEvent_t>(event))); }
 int cinn_hip_event_record(void* event, void* stream) {
-  return static_cast<int>(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
+  return Status(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
 }
-int cinn_hip_event_synchronize(void* event) { return static_cast<int>(hipEventSynchronize(static_cast<hipEvent_t>(event))); }
+int cinn_hip_event_synchronize(void* event) { return Status(hipEventSynchronize(static_cast<hipEvent_t>(event))); }
 int cinn_hip_event_elapsed_ms(void* start, void* stop, float* ms) {
-  return static_cast<int>(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+  return Status(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
 }
 const char* cinn_hip_error_string(int status) { return hipGetErrorString(static_cast<hipError_t>(status)); }
 void cinn_hip_free_host(void* p) { free(p); }

@@ -44,7 +44,9 @@ def test_every_declared_intrinsic_can_be_called_from_a_host_stub():
     # (REGISTER_EXTERN_FUNC_HELPER list, cinn/runtime/cuda/cuda_intrinsics.cc:404-733)
     lib = _lib.load()
     registered = set(_lib.read_string(lib.cinn_amd_extern_api_names).split(","))
-    declared = [n for n in _declared_functions("cinn_hip_runtime.h") if n.startswith("cinn_call_")]
+    # (the status-returning entry point for callers that cannot allocate is not a host-stub prototype)
+    declared = [n for n in _declared_functions("cinn_hip_runtime.h")
+                if n.startswith("cinn_call_") and not n.endswith("_noalloc")]
     assert len(declared) >= 14
     assert not [n for n in declared if n not in registered], registered
     # a stub is a real function pointer; wrong arity and unknown names are reported, not executed

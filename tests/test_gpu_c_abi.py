@@ -18,11 +18,13 @@ LAUNCH_ARGTYPES = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int] + [ctypes.c_i
 
 TWO_KERNELS = r'''
 #include "cinn_hip_runtime_source.h"
-// y[r][c] = a * x[r][c] + shift, on a 2-D grid; rows / cols bound the ragged edge
-extern "C" __global__ void saxpy2d(const float* __restrict__ x, float* __restrict__ y, int rows, int cols, float a, int shift) {
+// y[r][c] = a * x[r][c] + shift, on a 2-D grid; rows / cols bound the ragged edge.  A floating-point pod value
+// travels as a double (cinn_pod_value_t(float) stores v_float64 and data_addr() hands out its address,
+// cinn/runtime/cinn_runtime.cc:274, 394-412), so the kernel parameter that receives it is a double.
+extern "C" __global__ void saxpy2d(const float* __restrict__ x, float* __restrict__ y, int rows, int cols, double a, int shift) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   const int r = blockIdx.y * blockDim.y + threadIdx.y;
-  if (r < rows && c < cols) y[r * cols + c] = a * x[r * cols + c] + (float)shift;
+  if (r < rows && c < cols) y[r * cols + c] = (float)a * x[r * cols + c] + (float)shift;
 }
 // one wavefront per row: out[r] = sum of the row through the device library's 64-lane all-reduce
 extern "C" __global__ void row_sum64(const int* __restrict__ x, int* __restrict__ out, int cols) {
