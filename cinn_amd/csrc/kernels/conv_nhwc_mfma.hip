@@ -678,3 +678,133 @@ void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream) {
 }
 
 }  // namespace cinn_hip_kernels
+
+// ---- the entry point that allocates nothing -------------------------------------------------------------------
+// cinn_call_hip_conv2d_forward_noalloc: cinn_call_cudnn_conv2d_forward for callers that cannot call hipMalloc (code
+// under graph capture, tight serving loops).  Its scratch - the page of zeros that masked-out chunks are read from and
+// the fp32 partial sums of a split reduction - lives in this file-scope device array instead of the library's arena.
+// Every GPU the library runs on holds its own copy, at its own address, until the process ends; the host-side name
+// `scratch` is only a handle for hipGetSymbolAddress, never a device address.
+namespace {
+
+constexpr size_t kNoAllocZeroBytes     = 256;                 // never written by any kernel: stays zero
+constexpr size_t kNoAllocPartialsBytes = (size_t)16 << 20;    // split-K partial sums, rewritten by every call
+static __device__ __align__(256) unsigned char scratch[kNoAllocZeroBytes + kNoAllocPartialsBytes];
+
+constexpr int kNoAllocMaxDevices = 64;
+std::mutex g_noalloc_mu;
+unsigned char* g_noalloc_ptr[kNoAllocMaxDevices];  // device address of `scratch` on each device, once looked up
+
+// device address of this device's copy of `scratch`; 0 = ok
+int NoAllocScratch(unsigned char** out) {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kNoAllocMaxDevices) {
+    fprintf(stderr, "cinn_call_hip_conv2d_forward_noalloc: no current device (or more than %d devices)\n", kNoAllocMaxDevices);
+    return 1;
+  }
+  std::lock_guard<std::mutex> lock(g_noalloc_mu);
+  if (!g_noalloc_ptr[device]) {
+    void* ptr      = nullptr;
+    hipError_t err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || !ptr) {
+      fprintf(stderr, "cinn_call_hip_conv2d_forward_noalloc: hipGetSymbolAddress(scratch) failed on device %d: %s\n", device,
+              hipGetErrorString(err));
+      return 1;
+    }
+    g_noalloc_ptr[device] = static_cast<unsigned char*>(ptr);
+  }
+  *out = g_noalloc_ptr[device];
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t cinn_hip_conv2d_forward_noalloc_scratch_limit(void) { return kNoAllocPartialsBytes; }
+
+int cinn_hip_conv2d_forward_noalloc_init(void) {
+  unsigned char* base = nullptr;
+  return NoAllocScratch(&base);
+}
+
+int cinn_call_hip_conv2d_forward_noalloc(void* v_args, int num_args, int format, float alpha, float beta, int input_n,
+                                         int input_c, int input_h, int input_w, int filter_n, int filter_c, int filter_h,
+                                         int filter_w, int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h,
+                                         int dilation_w, int groups, int output_n, int output_c, int output_h,
+                                         int output_w, void* stream) {
+  CINN_HIP_CLEAR_STALE_ERROR();
+  using namespace cinn_hip_kernels;
+  const char* const me = "cinn_call_hip_conv2d_forward_noalloc";
+#define CINN_NOALLOC_REJECT(code, ...)  \
+  do {                                  \
+    fprintf(stderr, "%s: ", me);        \
+    fprintf(stderr, __VA_ARGS__);       \
+    fprintf(stderr, "\n");              \
+    return code;                        \
+  } while (0)
+  if (num_args != 3 || !v_args) CINN_NOALLOC_REJECT(1, "takes x, w and y, got %d arguments", num_args);
+  auto* pods = static_cast<cinn_pod_value_t*>(v_args);
+  cinn_buffer_t* bufs[3];
+  for (int i = 0; i < 3; ++i) {
+    if (pods[i].type_code_ != CINN_POD_BUFFER_P || !pods[i].value_.v_handle) CINN_NOALLOC_REJECT(1, "argument %d is not a buffer", i);
+    bufs[i] = static_cast<cinn_buffer_t*>(pods[i].value_.v_handle);
+    if (!bufs[i]->memory) CINN_NOALLOC_REJECT(1, "argument %d has no device memory", i);
+  }
+  if (format != 1 && format != 2)
+    CINN_NOALLOC_REJECT(1, "format %d: only channels-last outputs (1, or 2 with an NCHW input) run without allocation", format);
+  if (groups != 1) CINN_NOALLOC_REJECT(1, "groups = %d: only ungrouped convolutions", groups);
+  if (filter_c != input_c || output_n != input_n || output_c != filter_n)
+    CINN_NOALLOC_REJECT(1, "inconsistent extents (filter channels %d vs %d, output [%d,%d] vs [%d,%d])", filter_c, input_c,
+                        output_n, output_c, input_n, filter_n);
+  if (stride_h <= 0 || stride_w <= 0 || dilation_h <= 0 || dilation_w <= 0)
+    CINN_NOALLOC_REJECT(1, "strides and dilations must be positive");
+  const int want_oh = (input_h - ((filter_h - 1) * dilation_h + 1) + 2 * pad_h) / stride_h + 1;
+  const int want_ow = (input_w - ((filter_w - 1) * dilation_w + 1) + 2 * pad_w) / stride_w + 1;
+  if (output_h != want_oh || output_w != want_ow || want_oh <= 0 || want_ow <= 0)
+    CINN_NOALLOC_REJECT(1, "output is %dx%d, the shapes give %dx%d", output_h, output_w, want_oh, want_ow);
+  if ((int64_t)input_n * input_c * input_h * input_w >= INT_MAX || (int64_t)output_n * output_c * output_h * output_w >= INT_MAX ||
+      (int64_t)filter_n * filter_c * filter_h * filter_w * 8 >= INT_MAX)
+    CINN_NOALLOC_REJECT(1, "tensor too large for 32-bit offsets");
+  ConvNhwcArgs a;
+  a.x = bufs[0]->memory, a.w = bufs[1]->memory, a.y = bufs[2]->memory;
+  a.scale = a.shift = nullptr;
+  a.residual        = beta != 0.0f ? bufs[2]->memory : nullptr;
+  a.alpha           = alpha;
+  a.residual_scale  = beta;
+  a.relu            = false;
+  a.nchw_input      = format == 2;
+  a.n = input_n, a.h = input_h, a.w_in = input_w, a.c = input_c;
+  a.oc = filter_n, a.kh = filter_h, a.kw = filter_w, a.oh = output_h, a.ow = output_w;
+  a.pad_h = pad_h, a.pad_w = pad_w, a.stride_h = stride_h, a.stride_w = stride_w, a.dil_h = dilation_h, a.dil_w = dilation_w;
+  a.type = bufs[0]->type;
+  if (!ConvNhwcSupported(a))
+    CINN_NOALLOC_REJECT(1, "unsupported element type (code %d, %d bits) or %d input channels are not whole 16-byte chunks",
+                        a.type.code, a.type.bits, input_c);
+  // the size check comes before any launch: the partial sums of the split this shape gets must fit
+  Params p          = MakeParams(a);
+  const TileShape t = TileFor(a, p);
+  PlanSplits(&p, t.bm, t.bn, a.type.bits / CHAR_BIT);
+  const size_t need = p.splits > 1 ? (size_t)p.splits * p.pixels * p.oc * sizeof(float) : 0;
+  if (need > kNoAllocPartialsBytes)
+    CINN_NOALLOC_REJECT(2, "this shape splits its reduction %d ways and needs %zu bytes of partial sums; the static scratch holds %zu",
+                        p.splits, need, kNoAllocPartialsBytes);
+#undef CINN_NOALLOC_REJECT
+  unsigned char* base = nullptr;
+  if (NoAllocScratch(&base) != 0) return 1;
+  ScratchSource src;
+  src.zero_page            = base;
+  src.fixed_partials       = reinterpret_cast<float*>(base + kNoAllocZeroBytes);
+  src.fixed_partials_bytes = kNoAllocPartialsBytes;
+  const Params fresh = MakeParams(a);  // Launch plans the split itself, identically
+  if (a.type.code == cinn_type_bfloat) {
+    Dispatch<__bf16>(a, fresh, static_cast<hipStream_t>(stream), src);
+  } else if (a.type.bits == 16) {
+    Dispatch<_Float16>(a, fresh, static_cast<hipStream_t>(stream), src);
+  } else {
+    Dispatch<float>(a, fresh, static_cast<hipStream_t>(stream), src);
+  }
+  return 0;
+}
+
+}  // extern "C"

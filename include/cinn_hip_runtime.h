@@ -170,6 +170,25 @@ void cinn_call_hip_conv2d_bn_relu(void* v_args, int num_args, int format, int re
                                   int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
                                   int groups, int output_n, int output_c, int output_h, int output_w, void* stream);
 
+/* cinn_call_cudnn_conv2d_forward for callers that cannot allocate.  No counterpart in the reference: it exists for
+ * code that runs under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  Same arguments and
+ * results as the call above for format 1 and 2 with groups == 1 (always on the general channels-last MFMA kernel);
+ * it calls no hipMalloc / hipFree and no allocating library routine.  What the kernels need beyond x, w and y (a page
+ * of zeros, the fp32 partial sums of a split reduction) lives in a static device array of
+ * cinn_hip_conv2d_forward_noalloc_scratch_limit() = 16 MiB (+ 256 bytes) that every GPU the library runs on holds
+ * until the process ends.  Returns 0 on success; 1 for an unsupported format, type, group count or shape; 2 when the
+ * shape's partial sums exceed the limit (nothing is launched in either case; the reason is printed to stderr).
+ * All calls on one GPU share that array: calls that overlap on one GPU (two streams, two threads) race.
+ * cinn_hip_conv2d_forward_noalloc_init looks the array's device address up for the current device ahead of time
+ * (otherwise the first call on a device does). */
+int cinn_call_hip_conv2d_forward_noalloc(void* v_args, int num_args, int format, float alpha, float beta, int input_n,
+                                         int input_c, int input_h, int input_w, int filter_n, int filter_c, int filter_h,
+                                         int filter_w, int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h,
+                                         int dilation_w, int groups, int output_n, int output_c, int output_h,
+                                         int output_w, void* stream);
+int cinn_hip_conv2d_forward_noalloc_init(void);
+size_t cinn_hip_conv2d_forward_noalloc_scratch_limit(void);
+
 /* Replaces cinn_call_cudnn_pool2d_forward (cuda_util.cc:969-1041).  mode: 0 = max,
  * 1 = avg counting padding, 2 = avg excluding padding, 3 = max (deterministic) — the
  * cudnnPoolingMode_t values.  v_args = {x, y}. */
