@@ -602,6 +602,21 @@ class RowReduceEmitter {
     k_   = ir::MakeVar("k", common::Int(32));
     col_ = ir::MakeVar("col", common::Int(32));
     ComputePhases();
+    // Column operands (gamma / beta of a layer norm) that only later phases use are requested in the first phase,
+    // together with the row itself, and kept in registers: otherwise their latency is paid after the reductions,
+    // once more per row.  Budget: 64 registers per lane for all of them.
+    if (plan_.cached && num_phases_ > 1) {
+      int64_t dwords = 0;
+      for (auto& kv : kinds_) {
+        if (kv.second != RowKind::kCol || ctx_->produced.count(kv.first)) continue;
+        dwords += (static_cast<int64_t>(plan_.chunks) * plan_.vec * kv.first->dtype.bytes() + 3) / 4;
+        prefetched_cols_.push_back(const_cast<NodeData*>(kv.first));
+      }
+      static const bool enabled = EnvInt("FLAGS_cinn_hip_prefetch_columns", 1) != 0;
+      if (!enabled || dwords > 64) prefetched_cols_.clear();
+      std::sort(prefetched_cols_.begin(), prefetched_cols_.end(),
+                [](const NodeData* a, const NodeData* b) { return a->id < b->id; });
+    }
   }
 
   Expr row() const { return row_; }
@@ -736,7 +751,7 @@ class RowReduceEmitter {
   // vector, or any operand in streaming mode, is re-read in every phase that uses it.
   Expr StagedInput(NodeData* v, bool is_col) {
     auto& slot      = stage_[v];
-    bool persistent = plan_.cached && !is_col;
+    bool persistent = plan_.cached && (!is_col || std::find(prefetched_cols_.begin(), prefetched_cols_.end(), v) != prefetched_cols_.end());
     if (!slot.buffer) {
       int64_t size = persistent ? static_cast<int64_t>(plan_.chunks) * plan_.vec : plan_.vec;
       slot.buffer  = ctx_->NewLocal(CName(v->id) + "_reg", v->dtype, size);
@@ -875,6 +890,9 @@ class RowReduceEmitter {
         lane_stmts.push_back(ir::MakeStore(a.value, Combine(a.kind, cur, ir::MakeCast(a.acc_type, v)), I32(0)));
       }
     }
+    // column operands of later phases, requested now
+    if (p == 0 && !accs.empty())
+      for (NodeData* v : prefetched_cols_) StagedInput(v, true);
     // values that later phases need (cached mode)
     for (Node* n : ctx_->group.nodes) {
       for (auto* v : n->outputs)
@@ -955,6 +973,7 @@ class RowReduceEmitter {
   std::set<const NodeData*> stored_rows_;
   std::map<const NodeData*, Expr> elem_cache_;
   std::map<const NodeData*, Stage> stage_;
+  std::vector<NodeData*> prefetched_cols_;
   std::map<const NodeData*, BufferRef> materialized_buf_;
   std::map<const NodeData*, int> materialized_phase_;
 };

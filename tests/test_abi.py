@@ -204,3 +204,60 @@ def test_bench_refuses_more_than_one_gpu():
     assert r.returncode != 0
     assert "ONE GPU" in (r.stdout + r.stderr)
     assert not any(line.startswith("{") for line in r.stdout.splitlines())
+
+
+FLOAT_FNS = ["sin", "cos", "tan", "sinh", "cosh", "tanh", "asin", "acos", "atan", "asinh", "acosh", "atanh", "ceil", "round",
+             "trunc", "abs", "floor", "log", "log2", "log10", "exp", "erf", "sigmoid", "sqrt", "rsqrt", "cbrt"]
+
+
+def reference_spelling_calls():
+    """One call of every device-library name an unchanged CINN lowering can emit (the cinn_nvgpu_<fn>_<type> table of
+    cinn/runtime/cuda/cinn_cuda_runtime_source.cuh:12-370 and the cinn_cuda_* / counting / index helpers of :619-843),
+    as statements that accumulate into `double acc`."""
+    calls = []
+    ctype = {"fp32": "float", "fp64": "double", "fp16": "float16", "bf16": "bfloat16"}
+    for sfx, t in ctype.items():
+        v = "(%s)0.5f" % t
+        for fn in FLOAT_FNS:
+            calls.append("acc += (double)(float)cinn_nvgpu_%s_%s(%s);" % (fn, sfx, v))
+        for fn in ("isfinite", "isinf", "isnan"):
+            calls.append("acc += cinn_nvgpu_%s_%s(%s) ? 1.0 : 0.0;" % (fn, sfx, v))
+        for fn in ("pow", "mod"):
+            calls.append("acc += (double)(float)cinn_nvgpu_%s_%s(%s, (%s)3.0f);" % (fn, sfx, v, t))
+    ints = {"uint8": "uint8_t", "int8": "int8_t", "int16": "int16_t", "int32": "int", "int64": "long long"}
+    for sfx, t in ints.items():
+        for fn in ("bitwise_and", "bitwise_or", "bitwise_xor", "logical_right_shift"):
+            calls.append("acc += (double)cinn_nvgpu_%s_%s((%s)12, (%s)2);" % (fn, sfx, t, t))
+        calls.append("acc += (double)cinn_nvgpu_bitwise_not_%s((%s)12);" % (sfx, t))
+    for fn in ("bitwise_and", "bitwise_or", "bitwise_xor"):
+        calls.append("acc += cinn_nvgpu_%s_bool(true, false) ? 1.0 : 0.0;" % fn)
+    calls.append("acc += cinn_nvgpu_bitwise_not_bool(true) ? 1.0 : 0.0;")
+    for fn in ("pow", "left_shift", "right_shift", "max", "min", "mod"):
+        calls.append("acc += (double)cinn_nvgpu_%s_int32(7, 2);" % fn)
+    for fn in ("clz", "popc", "trunc"):
+        calls.append("acc += (double)cinn_nvgpu_%s_int32(7);" % fn)
+        calls.append("acc += (double)cinn_nvgpu_%s_int64(7ll);" % fn)
+    calls.append("acc += (double)cinn_nvgpu_mod_int64(7ll, 2ll) + (double)cinn_nvgpu_pow_int64(7ll, 2ll);")
+    calls.append("acc += cinn_cuda_find_int(ibuf, 4, 1) + cinn_cuda_find_float(fbuf, 4, 1.0f);")
+    calls.append("acc += cinn_cuda_find_int_nd(ibuf, 2, 1, 0, 2) + cinn_cuda_find_float_nd(fbuf, 2, 1.0f, 0, 2);")
+    calls.append("acc += cinn_cuda_find_int_from(ibuf, 4, 1, 1) + cinn_cuda_find_float_from(fbuf, 4, 1.0f, 1);")
+    calls.append("acc += cinn_nvgpu_next_smallest_int32(ibuf, 4, 0, 0, 1);")
+    for sfx, buf, v in (("fp32", "fbuf", "1.0f"), ("fp64", "dbuf", "1.0"), ("int32", "ibuf", "1"), ("int64", "lbuf", "1ll"),
+                        ("fp16", "hbuf", "(float16)1.0f")):
+        calls.append("acc += cinn_nvgpu_lt_num_%s(%s, 4, %s, 0, 1) + cinn_nvgpu_gt_num_%s(%s, 4, %s, 0, 1);" % (sfx, buf, v, sfx, buf, v))
+    for sfx, buf, v in (("fp32", "fbuf", "1.0f"), ("fp64", "dbuf", "1.0"), ("int32", "ibuf", "1"), ("int64", "lbuf", "1ll"),
+                        ("fp16", "hbuf", "(float16)1.0f"), ("int8", "cbuf", "(int8_t)1"), ("bool", "bbuf", "true")):
+        calls.append("acc += (double)(float)cinn_nvgpu_index_add_%s(%s, 1, %s, 0, 1, ibuf, 4);" % (sfx, v, buf))
+    calls.append("acc += cinn_cuda_resize_bilinear(ibuf, 1, 2, 2, 4, 4, 0, 0, 1, 1) + cinn_cuda_resize_bicubic(ibuf, 1, 2, 2, 4, 4, 0, 0, 1, 1);")
+    return calls
+
+
+def test_device_library_defines_the_reference_spellings():
+    calls = reference_spelling_calls()
+    assert len(calls) > 180
+    src = ('#include "cinn_hip_runtime_source.h"\n'
+           'extern "C" __global__ void every_name(int* ibuf, float* fbuf, double* dbuf, long long* lbuf, float16* hbuf, '
+           'int8_t* cbuf, bool* bbuf, double* out) {\n  double acc = 0.0;\n  ' + "\n  ".join(calls) +
+           "\n  out[threadIdx.x] = acc;\n}\n")
+    image = runtime.rtc_compile(src)
+    assert image[:4] == b"\x7fELF"

@@ -196,3 +196,112 @@ def test_memset_in_a_captured_graph_replays_correctly(gpu):
         assert np.array_equal(Y.numpy(), want), "replay %d" % replay
     hip.hipGraphExecDestroy(graph_exec)
     hip.hipGraphDestroy(graph)
+
+
+RESIZE_KERNELS = r'''
+#include "cinn_hip_runtime_source.h"
+// out[n][c][y][x] = resize(in)[n][c][y][x], one thread per output element, through the reference-named entry points
+extern "C" __global__ void resize_both(const int* __restrict__ in, int* __restrict__ lin, int* __restrict__ cub,
+                                       int n_size, int c_size, int in_h, int in_w, int out_h, int out_w) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n_size * c_size * out_h * out_w) return;
+  const int x = idx % out_w, y = (idx / out_w) % out_h, c = (idx / (out_w * out_h)) % c_size, n = idx / (out_w * out_h * c_size);
+  lin[idx] = cinn_cuda_resize_bilinear(in, c_size, in_h, in_w, out_h, out_w, n, c, y, x);
+  cub[idx] = cinn_cuda_resize_bicubic(in, c_size, in_h, in_w, out_h, out_w, n, c, y, x);
+}
+// a few of the cinn_nvgpu_* / cinn_cuda_* spellings with results that pin their semantics
+extern "C" __global__ void spellings(const int* __restrict__ v, int* __restrict__ out, int size) {
+  if (threadIdx.x != 0) return;
+  out[0] = cinn_nvgpu_mod_int32(-7, 3);                      // result takes the divisor's sign: 2
+  out[1] = cinn_cuda_find_int(v, size, 5);                   // last position of 5
+  out[2] = cinn_cuda_find_int_from(v, size, 5, 0);           // first position of 5
+  out[3] = cinn_nvgpu_gt_num_int32(v, size, 4, 0, 1);        // how many are greater than 4
+  out[4] = cinn_nvgpu_lt_num_int32(v, size / 2, 4, 1, 2);    // odd positions only
+  out[5] = (int)cinn_nvgpu_floor_fp32(-1.5f);
+  out[6] = cinn_nvgpu_clz_int32(1);
+  out[7] = cinn_nvgpu_index_add_int32(100, 5, v, 0, 1, v, size);  // adds v[i] for every i with v[i] == 5
+}
+'''
+
+
+def resize_brute_force(img, out_h, out_w, cubic):
+    """cinn_cuda_resize_bilinear / _bicubic restated in numpy fp32, one operation per rounding
+    (cinn/runtime/cuda/cinn_cuda_runtime_source.cuh:748-843)"""
+    f = np.float32
+    n_size, c_size, in_h, in_w = img.shape
+    out = np.zeros((n_size, c_size, out_h, out_w), np.int32)
+
+    def source(dst, in_extent, out_extent):
+        scale = f(in_extent) / f(out_extent)
+        src = f(f(f(dst) + f(0.5)) * scale) - f(0.5)
+        low = np.floor(src)
+        return int(low), f(src - low)
+
+    def weights(t):
+        a = f(-0.5)
+        t2 = f(t * t)
+        t3 = f(f(t * t) * t)
+        return [f(a * f(f(t3 - f(f(2) * t2)) + t)),
+                f(f(f(f(a + f(2)) * t3) - f(f(f(3) + a) * t2)) + f(1)),
+                f(f(f(-f(a + f(2))) * t3 + f(f(f(3) + f(f(2) * a)) * t2)) - f(a * t)),
+                f(f(f(-a) * t3) + f(a * t2))]
+
+    for y in range(out_h):
+        by, fy = source(y, in_h, out_h)
+        for x in range(out_w):
+            bx, fx = source(x, in_w, out_w)
+            for n in range(n_size):
+                for c in range(c_size):
+                    plane = img[n, c]
+                    if not cubic:
+                        rows = []
+                        for i in range(2):
+                            line = plane[min(max(by + i, 0), in_h - 1)]
+                            left, right = f(line[min(max(bx, 0), in_w - 1)]), f(line[min(max(bx + 1, 0), in_w - 1)])
+                            rows.append(f(f(left * f(f(1) - fx)) + f(right * fx)))
+                        value = f(f(rows[0] * f(f(1) - fy)) + f(rows[1] * fy))
+                    else:
+                        wx, wy = weights(fx), weights(fy)
+                        value = f(0)
+                        for i in range(4):
+                            line = plane[min(max(by + i - 1, 0), in_h - 1)]
+                            acc = f(0)
+                            for j in range(4):
+                                acc = f(acc + f(f(line[min(max(bx + j - 1, 0), in_w - 1)]) * wx[j]))
+                            value = f(value + f(acc * wy[i]))
+                    out[n, c, y, x] = int(value)  # truncation toward zero, as the float -> int conversion does
+    return out
+
+
+@pytest.mark.parametrize("shape,out_hw", [((2, 3, 5, 7), (9, 4)), ((1, 2, 8, 8), (3, 16))])
+def test_resize_device_functions_match_a_brute_force(gpu, shape, out_hw):
+    lib = _lib.load()
+    lib.cinn_call_cuda_kernel.argtypes = LAUNCH_ARGTYPES
+    rng = np.random.default_rng(sum(shape))
+    img = rng.integers(-200, 200, shape, dtype=np.int32)
+    out_h, out_w = out_hw
+    total = shape[0] * shape[1] * out_h * out_w
+    module = runtime.Module(runtime.rtc_compile(RESIZE_KERNELS))
+    IN = runtime.DeviceBuffer.from_numpy(img)
+    LIN, CUB = runtime.DeviceBuffer((total,), "int32"), runtime.DeviceBuffer((total,), "int32")
+    args = scalar_pods(lib, [IN, LIN, CUB], [("i", shape[0]), ("i", shape[1]), ("i", shape[2]), ("i", shape[3]), ("i", out_h), ("i", out_w)])
+    lib.cinn_call_cuda_kernel(module.get_function("resize_both"), args, 9, (total + 63) // 64, 1, 1, 64, 1, 1, None)
+    runtime.synchronize()
+    want_lin = resize_brute_force(img, out_h, out_w, cubic=False).reshape(-1)
+    want_cub = resize_brute_force(img, out_h, out_w, cubic=True).reshape(-1)
+    assert np.array_equal(LIN.numpy(), want_lin)
+    assert np.array_equal(CUB.numpy(), want_cub)
+    # bilinear interpolation never leaves the range of the image
+    assert LIN.numpy().min() >= img.min() and LIN.numpy().max() <= img.max()
+
+
+def test_reference_spellings_keep_their_semantics(gpu):
+    lib = _lib.load()
+    lib.cinn_call_cuda_kernel.argtypes = LAUNCH_ARGTYPES
+    v = np.array([5, 1, 9, 5, 0, 7, 5, 2], np.int32)
+    module = runtime.Module(runtime.rtc_compile(RESIZE_KERNELS))
+    V, OUT = runtime.DeviceBuffer.from_numpy(v), runtime.DeviceBuffer((8,), "int32")
+    args = scalar_pods(lib, [V, OUT], [("i", 8)])
+    lib.cinn_call_cuda_kernel(module.get_function("spellings"), args, 3, 1, 1, 1, 64, 1, 1, None)
+    runtime.synchronize()
+    assert OUT.numpy().tolist() == [2, 6, 0, 5, 2, -2, 31, 115]
