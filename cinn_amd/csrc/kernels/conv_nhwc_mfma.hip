@@ -536,9 +536,9 @@ void PlanSplits(Params* p, int bm, int bn, int elem_bytes) {
   p->splits          = (steps + p->steps_per_split - 1) / p->steps_per_split;
 }
 
-template <typename T, int BM, int BN, int WM, int WN, bool NCHW_IN>
+template <typename T, int BM, int BN, int WM, int WN, bool NCHW_IN, int PF = 2>
 void Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream, const ScratchSource& src) {
-  constexpr int PF = 2;  // K steps in flight per block
+  // PF: K steps in flight per block
   auto kernel      = conv_nhwc_mfma_kernel<T, BM, BN, WM, WN, NCHW_IN, PF>;
   const int bytes  = LdsBytes(BM, BN, WM);
   static const bool configured = [&] {  // once per instantiation, thread-safe
@@ -607,8 +607,17 @@ void Dispatch(const ConvNhwcArgs& a, const Params& p, hipStream_t stream, const 
     Launch<T, 128, 128, 2, 2, false>(a, p, stream, src);
   else if (t.bm == 128)
     Launch<T, 128, 64, 2, 2, false>(a, p, stream, src);
-  else
-    Launch<T, 64, 64, 2, 2, false>(a, p, stream, src);
+  else {
+    static const int pf = getenv("FLAGS_cinn_hip_conv_pf") ? atoi(getenv("FLAGS_cinn_hip_conv_pf")) : 2;
+    if (pf == 4)
+      Launch<T, 64, 64, 2, 2, false, 4>(a, p, stream, src);
+    else if (pf == 6)
+      Launch<T, 64, 64, 2, 2, false, 6>(a, p, stream, src);
+    else if (pf == 8)
+      Launch<T, 64, 64, 2, 2, false, 8>(a, p, stream, src);
+    else
+      Launch<T, 64, 64, 2, 2, false>(a, p, stream, src);
+  }
 }
 
 int ChunkElems(const cinn_type_t& t) { return 16 / (t.bits / CHAR_BIT); }

@@ -315,13 +315,19 @@ struct ConvGeom {
 
 // BM x BN block tile on a WAVES_M x WAVES_N grid of wavefronts: 256x256 on 2x4 (8 wavefronts of 128x64) for large
 // problems, 128x128 on 2x2 (4 wavefronts of 64x64, two blocks per CU) when 256x256 tiles would leave CUs idle.
-template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false, int NS = 2>
-__global__ void __launch_bounds__(64 * WAVES_M * WAVES_N)
+// FEED: the block carries WAVES_M x WAVES_N more wavefronts that only issue the direct-to-LDS loads, wait for them and
+// take part in the barriers, while the first WAVES_M x WAVES_N only compute.  A wavefront that issues a load
+// instruction stalls until the address unit has taken it (about 16 clocks per KiB and CU), and with one computing
+// wavefront per SIMD nobody else is there to issue MFMAs meanwhile: measured on the 128x128 tile (four stages,
+// implicit GEMM, K = 4608) a K step took 1102 clocks for 512 of MFMA with the loads issued by the computing
+// wavefronts and 531 without any loads.
+template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false, int NS = 2, bool FEED = false>
+__global__ void __launch_bounds__(64 * WAVES_M * WAVES_N * (FEED ? 2 : 1))
 gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* C, int M, int N, int K,
                   int64_t lda, int64_t ldb, int64_t ldc, DmaEpilogue epi, int64_t stride_a, int64_t stride_b,
                   int64_t stride_c, int xcd_cols, int sub_rows, int sub_cols, ConvGeom geom) {
-  constexpr int NW      = WAVES_M * WAVES_N;
-  constexpr int THREADS = 64 * NW;
+  constexpr int NW      = WAVES_M * WAVES_N;                // computing wavefronts
+  constexpr int THREADS = 64 * NW * (FEED ? 2 : 1);
   constexpr int TM      = BM / WAVES_M / 16;  // 16x16 accumulator tiles per wavefront along M and N
   constexpr int TN      = BN / WAVES_N / 16;
   constexpr int A_TILE  = BM * kD64BK * 2;    // bytes of one operand tile of a stage
@@ -329,7 +335,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   // With two wavefronts per SIMD the older one of each pair (wavefronts 0 .. NW/2-1) wins the MFMA arbitration, runs
   // ahead and then waits at the step's barrier; it issues all the loads (their issue stalls cost it nothing), so the
   // younger one, which the barrier waits for, has no loads to issue or wait for.
-  constexpr int LW      = (TM == 8 && !CONV) ? NW / 2 : NW;  // wavefronts that issue loads
+  constexpr int LW      = FEED ? NW : ((TM == 8 && !CONV) ? NW / 2 : NW);  // wavefronts that issue loads
   constexpr int LPA     = BM / 8 / LW;                        // loads (of 1 KiB per wavefront) per thread, operand and step
   constexpr int LPB     = BN / 8 / LW;
   static_assert(LPA >= 1 && LPB >= 1 && LPA <= 8 && LPB <= 8 && TM % 4 == 0 && TN == 4, "unsupported tile shape");
@@ -345,8 +351,9 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm   = wave / WAVES_N;
-  const int wn   = wave % WAVES_N;
+  const bool feeder = FEED && wave >= NW;  // loads only
+  const int wm   = (wave % NW) / WAVES_N;
+  const int wn   = (wave % NW) % WAVES_N;
 
   int tile_row, tile_col;
   if (sub_rows > 0) {
@@ -371,8 +378,8 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   // of row 0 (B stored [K][N]), less the instruction offset 1024 t of load t (which the LDS address needs)
   // (an instruction offset is below 4 KiB: loads t and t + 4 differ in m0 instead)
   unsigned a_off[LPA], b_off[LPB];
-  const bool loader = LW == NW || wave < LW;
-  const int lwave   = loader ? wave : 0;
+  const bool loader = FEED ? feeder : (LW == NW || wave < LW);
+  const int lwave   = loader ? (FEED ? wave - NW : wave) : 0;
   // The last tile row / column may reach beyond M / N: its lanes fetch the last valid row (or 8-column chunk)
   // instead - what they compute is not stored.  The bases lie kBias bytes below the tile and every lane offset
   // includes kBias, so that an offset less its instruction offset never wraps below zero.
@@ -529,7 +536,55 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   constexpr int L = LPA + LPB;  // loads of a loader wavefront per stage
   // vmcnt(n): at most n of the wavefront's loads still in flight; they complete in the order they were issued
 #define CINN_VMCNT(n) ((((n) & 15) | (((n) >> 4) << 14)) | 0x0F70)
-  if (loader) {
+  if (FEED) {
+    // Feeding wavefronts: every slot is free at the start, so all NS stages go out at once; then, per K step, wait
+    // for the next stage (the NS - 2 requested after it may stay in flight), meet the computing wavefronts at the
+    // step's barrier - which also tells that the step's own slot has been read - and refill that slot.
+    if (feeder) {
+#pragma unroll
+      for (int st = 0; st < NS; ++st) {
+        if (st < nk) {
+#pragma unroll
+          for (int t = 0; t < L; ++t) issue_one(sa(st), sb(st), st, t);
+          if (CONV) advance_tap();
+        }
+      }
+      if (nk >= NS) {
+        __builtin_amdgcn_s_waitcnt(CINN_VMCNT((NS - 1) * L));  // stage 0 has landed
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      }
+      __syncthreads();
+      int kt = 0;
+      for (; kt + NS < nk; ++kt) {  // steps that have a stage to request
+        __builtin_amdgcn_s_waitcnt(CINN_VMCNT((NS - 2) * L));  // stage kt + 1 has landed
+        __syncthreads();
+        switch (kt % NS) {  // slot of stage kt, now read by everyone
+          case 0:
+#pragma unroll
+            for (int t = 0; t < L; ++t) issue_one(sa(0), sb(0), kt + NS, t);
+            break;
+          case 1:
+#pragma unroll
+            for (int t = 0; t < L; ++t) issue_one(sa(1 % NS), sb(1 % NS), kt + NS, t);
+            break;
+          case 2:
+#pragma unroll
+            for (int t = 0; t < L; ++t) issue_one(sa(2 % NS), sb(2 % NS), kt + NS, t);
+            break;
+          default:
+#pragma unroll
+            for (int t = 0; t < L; ++t) issue_one(sa(3 % NS), sb(3 % NS), kt + NS, t);
+            break;
+        }
+        if (CONV) advance_tap();
+      }
+      for (; kt + 1 < nk; ++kt) {  // the last steps: everything is requested, wait for all of it
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+      }
+    }
+  } else if (loader) {
 #pragma unroll
     for (int st = 0; st < NS - 1; ++st) {
       if (st < nk) {
@@ -547,11 +602,13 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     }
   }
+  if (!feeder) {
   __syncthreads();
 #pragma unroll
   for (int i = 0; i < 3; ++i) ring[i] = read_a(sa(0), 0, i);
 #pragma unroll
   for (int j = 0; j < TN; ++j) bf[0][j] = read_b(sb(0), 0, j);
+  }
 
   // Step u of a group of NS (slot of its stage: u).  After its barrier the slot is free for stage s + NS: the first
   // EARLY loads go out in the three rows after the barrier, the others in the first rows of step s + 1 (there: stage
@@ -619,7 +676,9 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
       }                                                                                                      \
     }                                                                                                        \
   }
-  if (loader) {
+  if (feeder) {
+    // nothing to compute
+  } else if (loader) {
     CINN_GEMM_LOOP(true)
   } else {
     CINN_GEMM_LOOP(false)
@@ -658,6 +717,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 #pragma unroll
     for (int pass = 0; pass < TM / IB; ++pass) {
       __syncthreads();  // the last stage (or the previous pass) has been read
+      if (!feeder)
 #pragma unroll
       for (int ii = 0; ii < IB; ++ii)
 #pragma unroll
@@ -717,6 +777,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 #pragma unroll
   for (int pass = 0; pass < TM / IB; ++pass) {
     __syncthreads();
+    if (!feeder)
 #pragma unroll
     for (int ii = 0; ii < IB; ++ii)
 #pragma unroll
@@ -1263,7 +1324,7 @@ void XcdRectanglesPadded(int tiles_m, int tiles_n, int* xcd_cols, int* sub_rows,
   }
 }
 
-template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false, int NS = 2>
+template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false, int NS = 2, bool FEED = false>
 void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
   int64_t ldb = p.trans_b ? p.k : p.n;
   const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
@@ -1283,7 +1344,8 @@ void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
   epi.streaming = !p.keep_in_cache && (int64_t)p.batch * p.m * p.n * 2 >= (16 << 20);
   ConvGeom geom{};
   if (CONV) geom = *p.conv;
-  hipLaunchKernelGGL((gemm16_dma_kernel<T, B_KC, BM, BN, WAVES_M, WAVES_N, CONV, NS>), grid, dim3(64 * WAVES_M * WAVES_N), 0,
+  hipLaunchKernelGGL((gemm16_dma_kernel<T, B_KC, BM, BN, WAVES_M, WAVES_N, CONV, NS, FEED>), grid,
+                     dim3(64 * WAVES_M * WAVES_N * (FEED ? 2 : 1)), 0,
                      stream, static_cast<const uint16_t*>(p.a), static_cast<const uint16_t*>(p.b),
                      static_cast<uint16_t*>(p.c), p.m, p.n, p.k, (int64_t)p.k, ldb, (int64_t)p.n, epi, p.stride_a,
                      p.stride_b, p.stride_c, xcd_cols, sub_rows, sub_cols, geom);
@@ -1343,6 +1405,12 @@ bool TryShortK(const GemmProblem& p, hipStream_t stream) {
   return true;
 }
 
+// FLAGS_cinn_hip_gemm_feed=0: the four-stage 128x128 instances issue their loads from the computing wavefronts
+bool FeedWavefronts() {
+  static const bool on = !(getenv("FLAGS_cinn_hip_gemm_feed") && atoi(getenv("FLAGS_cinn_hip_gemm_feed")) == 0);
+  return on;
+}
+
 // A stored [M][K], K % 64 == 0, N % 8 == 0 (whole 16-byte chunks per row of C and of a row-major B): 256x256 tiles
 // when they fill the chip, else 128x128 tiles when there are enough of those; M and N need not be multiples of the
 // tile (the last tile row / column computes some rows / columns that are not stored); false when neither applies
@@ -1393,7 +1461,9 @@ bool TryDma16(const GemmProblem& p, hipStream_t stream) {
     // is 0.5-1 % faster with these layers here than on the 64x64 tiles of the convolution kernel, with 96 tiles 2 %
     // slower; a long K (52 against 73 us at 196 tiles, K = 4608) pays from 128 tiles
     if (tiles128 >= 192 || (tiles128 >= 128 && p.k >= 4096) || (forced == 128 && tiles128 > 0)) {
-      if (stages == 4) {
+      if (stages == 4 && FeedWavefronts()) {
+        LaunchDma16<T, true, 128, 128, 2, 2, true, 4, true>(p, stream);
+      } else if (stages == 4) {
         LaunchDma16<T, true, 128, 128, 2, 2, true, 4>(p, stream);
       } else {
         LaunchDma16<T, true, 128, 128, 2, 2, true>(p, stream);
@@ -1416,7 +1486,13 @@ bool TryDma16(const GemmProblem& p, hipStream_t stream) {
     return true;
   }
   if ((tiles128 >= 128 && forced != 256) || (forced == 128 && tiles128 > 0)) {
-    if (stages == 4) {
+    if (stages == 4 && FeedWavefronts()) {
+      if (p.trans_b) {
+        LaunchDma16<T, true, 128, 128, 2, 2, false, 4, true>(p, stream);
+      } else {
+        LaunchDma16<T, false, 128, 128, 2, 2, false, 4, true>(p, stream);
+      }
+    } else if (stages == 4) {
       if (p.trans_b) {
         LaunchDma16<T, true, 128, 128, 2, 2, false, 4>(p, stream);
       } else {
