@@ -1460,7 +1460,10 @@ bool TryDma16(const GemmProblem& p, hipStream_t stream) {
     // measured on ResNet-50 at batch 32 (fp16): from 192 tiles of 128x128 (four stages up to 256 tiles) the network
     // is 0.5-1 % faster with these layers here than on the 64x64 tiles of the convolution kernel, with 96 tiles 2 %
     // slower; a long K (52 against 73 us at 196 tiles, K = 4608) pays from 128 tiles
-    if (tiles128 >= 192 || (tiles128 >= 128 && p.k >= 4096) || (forced == 128 && tiles128 > 0)) {
+    // with the loads issued by wavefronts of their own, a long reduction pays from 96 tiles (256 -> 256 3x3 on 14x14
+    // at batch 32, 98 tiles, K = 2304: 21.0 against 22.4 us)
+    if (tiles128 >= 192 || (tiles128 >= 128 && p.k >= 4096) || (tiles128 >= 96 && p.k >= 2048 && FeedWavefronts()) ||
+        (forced == 128 && tiles128 > 0)) {
       if (stages == 4 && FeedWavefronts()) {
         LaunchDma16<T, true, 128, 128, 2, 2, true, 4, true>(p, stream);
       } else if (stages == 4) {
