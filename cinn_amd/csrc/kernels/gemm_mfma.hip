@@ -523,9 +523,11 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   // A wavefront tile of 64 rows has short steps (8 rows): all its loads go into the three rows after the barrier.
   // Loader wavefronts that carry their partner's loads too issue two per row.
   constexpr int EPR   = TM == 4 ? 3 : (LW < NW ? 2 : 1);  // loads per row: after the barrier ...
-  constexpr int LPR   = LW < NW ? 2 : 1;                  // ... and in the first rows of the next step
   constexpr int EARLY = 3 * EPR < LPA + LPB ? 3 * EPR : LPA + LPB;
   constexpr int LATE  = LPA + LPB - EARLY;
+  // ... and in the first rows of the next step (two per row also when one per row would not get them all out before
+  // the barrier that waits for them)
+  constexpr int LPR   = (LW < NW || LATE > ROWS - 3) ? 2 : 1;
   static_assert(LATE >= 0 && (LATE + LPR - 1) / LPR <= BAR + 1, "the late loads are issued before the barrier that waits for them");
   // slot of a row's per-row loads that follows MFMA j (-1: none)
 #define CINN_LOAD_SLOT(P, j) ((P) == 1 ? ((j) == 3 ? 0 : -1) : (P) == 2 ? ((j) == 1 ? 0 : (j) == 3 ? 1 : -1) : (j) - 1)
@@ -1450,6 +1452,13 @@ bool TryDma16(const GemmProblem& p, hipStream_t stream) {
     }
     return true;
   }
+  // Few tiles and a long reduction over K-contiguous operands (2048 -> 512 1x1 on 7x7 at batch 32: 52 tiles of 128x128,
+  // K = 2048): 64x64 tiles, one computing and one feeding wavefront per block, four stages - 14.1 against 21.0 us on the
+  // 64x64 tiles of the convolution kernel with split K and its reduce kernel.  (3x3 layers measured slower here.)
+  if (p.trans_b && !p.conv && ((forced == 0 && FeedWavefronts() && tiles128 < 96 && p.k >= 2048 && p.batch == 1) || forced == 64)) {
+    LaunchDma16<T, true, 64, 64, 1, 1, false, 4, true>(p, stream);
+    return true;
+  }
   if (p.conv) {
     // implicit-GEMM convolution: filters are [OC][K]
     if (!p.trans_b) return false;
@@ -1720,7 +1729,10 @@ bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream) {
     const bool narrow = a.oc % 128 != 0 && a.oc % 64 == 0 && ((pixels + 255) / 256) * (a.oc / 64) >= 256;
     static const bool shortk_on = !(getenv("FLAGS_cinn_hip_gemm_shortk") && atoi(getenv("FLAGS_cinn_hip_gemm_shortk")) == 0);
     const bool shortk = shortk_on && a.c == 64 && a.oc % 128 == 0 && pixels >= 16384;
-    if (!shortk && (a.c < 128 || (!narrow && ((pixels + 127) / 128) * ((a.oc + 127) / 128) < 192))) return false;
+    static const int forced_tile = getenv("FLAGS_cinn_hip_gemm_tile") ? atoi(getenv("FLAGS_cinn_hip_gemm_tile")) : 0;
+    // few tiles but a long reduction: the single-wavefront 64x64 tiles of the GEMM kernel (see TryDma16)
+    const bool long_k = forced_tile == 64 || (forced_tile == 0 && a.c >= 2048 && a.oc % 64 == 0);
+    if (!shortk && !long_k && (a.c < 128 || (!narrow && ((pixels + 127) / 128) * ((a.oc + 127) / 128) < 192))) return false;
     p.k = a.c;
   } else {
     // any filter, stride, padding, dilation: implicit GEMM, K = kh * kw * c with 64-channel steps inside a tap
