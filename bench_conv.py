@@ -3,7 +3,7 @@ NetBuilder with const parameters (the batch norm folds into the convolution epil
 launch stream.  Imported by bench.py (extra measurements); also runnable on its own:
     python bench_conv.py [float16|float32]
 Reports microseconds per launch, TFLOP/s (2 * N * OC * OH * OW * IC * KH * KW flop) and the layer's roofline: its bound
-is the larger of the HBM time of its algorithmic bytes (input + filter + output, once each) at 8 TB/s and the MFMA time
+is the larger of the HBM time of its algorithmic bytes (the input pixels it reads + filter + output, once each) at 8 TB/s and the MFMA time
 of its flop at the dense peak of the type; `frac` = that bound / the measured time.  Launches cycle through enough
 separate input / output sets to put 512 MiB between two uses of the same buffers (cold caches), after 30 ms of
 warm-up; the figure is the median of three runs of 200 launches."""
@@ -41,7 +41,9 @@ def measure(stream, runtime, dtype="float16", batch=32, launches=200):
                   "mean": rng.standard_normal(oc) * 0.1, "var": rng.uniform(0.5, 1.5, oc)}
         oh = (hw + 2 * p - k) // s + 1
         flop = 2 * batch * oc * oh * oh * ic * k * k
-        nbytes = (x.size + w.size + batch * oc * oh * oh) * elem + 2 * oc * 4
+        # input elements the layer reads at all: a filter smaller than its stride skips pixels (1x1 stride 2 reads one in four)
+        touched = x.size if k >= s else batch * ic * (oh * k) * (oh * k)
+        nbytes = (touched + w.size + batch * oc * oh * oh) * elem + 2 * oc * 4
         comps = []
         for _ in range(cold_sets(nbytes)):
             b = NetBuilder(name)
