@@ -1301,6 +1301,11 @@ ShapeType PadTo4(const ShapeType& s) {
 
 ir::LoweredFuncRef OpLowerer::LowerLibraryCall(const Group& group) const {
   CINN_CHECK_EQ(group.nodes.size(), 1u);
+  // The reference lowers contractions through generated compute bodies when FLAGS_cinn_use_custom_call is 0
+  // (cinn/hlir/framework/op_lowering.cc); here they exist only as library calls, so that setting is an error rather
+  // than a silently different path.
+  CINN_CHECK(EnvInt("FLAGS_cinn_use_custom_call", 1) != 0)
+      << "FLAGS_cinn_use_custom_call=0 is not supported: matmul / conv2d / pool2d are lowered to library calls only";
   Node* n         = group.nodes[0];
   auto func       = std::make_shared<ir::LoweredFunc>();
   func->name      = group.func_name;

@@ -607,17 +607,8 @@ void Dispatch(const ConvNhwcArgs& a, const Params& p, hipStream_t stream, const 
     Launch<T, 128, 128, 2, 2, false>(a, p, stream, src);
   else if (t.bm == 128)
     Launch<T, 128, 64, 2, 2, false>(a, p, stream, src);
-  else {
-    static const int pf = getenv("FLAGS_cinn_hip_conv_pf") ? atoi(getenv("FLAGS_cinn_hip_conv_pf")) : 2;
-    if (pf == 4)
-      Launch<T, 64, 64, 2, 2, false, 4>(a, p, stream, src);
-    else if (pf == 6)
-      Launch<T, 64, 64, 2, 2, false, 6>(a, p, stream, src);
-    else if (pf == 8)
-      Launch<T, 64, 64, 2, 2, false, 8>(a, p, stream, src);
-    else
-      Launch<T, 64, 64, 2, 2, false>(a, p, stream, src);
-  }
+  else
+    Launch<T, 64, 64, 2, 2, false>(a, p, stream, src);
 }
 
 int ChunkElems(const cinn_type_t& t) { return 16 / (t.bits / CHAR_BIT); }

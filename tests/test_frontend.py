@@ -164,6 +164,21 @@ def test_unknown_operator_and_bad_fetch_are_reported():
         b.reshape(x, [3])
 
 
+def test_contractions_without_library_calls_are_refused(monkeypatch):
+    """FLAGS_cinn_use_custom_call=0 asks the reference for generated matmul / conv2d bodies
+    (cinn/hlir/framework/op_lowering.cc); this backend has library calls only and says so."""
+    b = NetBuilder("no_custom_call")
+    x = b.create_input(Float(32), [16, 32], "x")
+    y = b.create_input(Float(32), [32, 8], "y")
+    out = b.matmul(x, y)
+    monkeypatch.setenv("FLAGS_cinn_use_custom_call", "0")
+    with pytest.raises(_lib.CinnError) as e:
+        compile_only(b, [out])
+    assert "FLAGS_cinn_use_custom_call" in str(e.value)
+    monkeypatch.setenv("FLAGS_cinn_use_custom_call", "1")
+    compile_only(b, [out])
+
+
 def test_generated_source_idioms():
     b = NetBuilder("t")
     x = b.create_input(Float(32), [1000, 3], "x")  # 3000 elements: not a multiple of 256*4 -> guarded tail
