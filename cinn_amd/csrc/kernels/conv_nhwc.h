@@ -35,6 +35,10 @@ void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream);
 // convolution is the GEMM pixels x channels; any other one with a multiple of 64 input channels runs as an implicit GEMM
 // (K = kh * kw * c); both with this epilogue.  false when the shape does not qualify.
 bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream);
+// 3x3, stride 1, padding 1 convolutions with 16-bit operands and multiples of 64 channels on both sides whose input
+// rows fit LDS (conv_patch_mfma.hip): the input patch of a band of output rows stays resident in LDS, only the filter
+// streams; same epilogue.  false when the shape does not qualify.
+bool TryConvPatch(const ConvNhwcArgs& a, hipStream_t stream);
 // 256 bytes of zeros in device memory (what masked-out chunks are read from)
 inline const void* ConvZeroPage() { return ZeroPage(); }
 

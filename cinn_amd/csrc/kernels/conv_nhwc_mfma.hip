@@ -666,6 +666,7 @@ void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream) {
     RunConvStem(a, stream);
     return;
   }
+  if (TryConvPatch(a, stream)) return;
   if (TryPointwiseConvAsGemm(a, stream)) return;
   const Params p = MakeParams(a);
   if (a.type.code == cinn_type_bfloat) {

@@ -295,6 +295,13 @@ int cinn_hip_scratch_reserve(void* stream, size_t split_k_bytes, size_t transpos
 int cinn_hip_scratch_info(void* stream, size_t* split_k_capacity, size_t* transpose_capacity, size_t* retired_bytes);
 int cinn_hip_scratch_release_retired(void);
 
+/* Kernel choice of cinn_call_cudnn_conv2d_forward / cinn_call_hip_conv2d_bn_relu for 3x3, stride 1, padding 1
+ * convolutions on channels-last 16-bit tensors: 0 = never the kernel that keeps the input patch resident in LDS,
+ * 1 = where it is expected to win (default; FLAGS_cinn_hip_conv_patch sets the initial value), 2 = wherever the shape
+ * qualifies.  Returns the previous mode; any other argument only reads it.  No counterpart in the reference (cuDNN picks
+ * its algorithm inside cudnnConvolutionForward, cinn/runtime/cuda/cuda_util.cc:560-640); a tuning and test switch. */
+int cinn_hip_conv_patch_mode(int mode);
+
 /* Device descriptor consumed by schedules.  Replaces common::Target's cudaDeviceGetAttribute
  * queries (cinn/common/target.cc:55-84, 177-221).  Filled from the live device when one is
  * present, otherwise with the MI355X datasheet values (256 CUs, wave64, 160 KiB LDS per CU). */

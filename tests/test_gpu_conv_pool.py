@@ -509,3 +509,58 @@ def test_conv_chain_through_a_ragged_channel_count(gpu, dtype, channels, tol):
     # the middle tensor is rounded to the storage type on both sides; fp16 inputs of the second sum may differ by one
     # ulp, which the magnitude scale absorbs
     assert np.all(np.abs(got.astype(np.float64) - want) <= tol * np.maximum(np.abs(want), 0.1 * scale) + 2.0 ** -24)
+
+
+@pytest.fixture
+def patch_kernel_everywhere():
+    """3x3 convolutions go to the LDS-resident-patch kernel whenever their shape qualifies, however few blocks."""
+    lib = _lib.load()
+    lib.cinn_hip_conv_patch_mode.argtypes = [ctypes.c_int]
+    before = lib.cinn_hip_conv_patch_mode(2)
+    yield lib
+    lib.cinn_hip_conv_patch_mode(before)
+
+
+PATCH_CASES = [
+    # (n, ic, h, w, oc): 3x3, stride 1, padding 1, 64 input channels
+    (2, 64, 56, 56, 64),     # 7 bands of 8 rows: first, inner and last bands
+    (2, 64, 28, 28, 128),    # two bands of 14 rows (392 of 448 pixel slots), two groups of output channels
+    (3, 64, 14, 14, 192),    # does not qualify (196 of 448 slots): stays on the other kernels
+    (2, 64, 43, 20, 64),     # ragged: bands of 22 and 21 rows; tiles that straddle image rows
+    (1, 64, 8, 56, 128),     # a single band: halo rows above and below are both outside the image
+    (2, 64, 16, 27, 64),     # odd width: 432 pixels, the last tile is half empty
+    (5, 64, 7, 64, 64),      # 448 pixels in 7 rows
+    (1, 64, 1, 400, 64),     # a single image row: every tap row but the middle one is halo
+]
+
+
+@pytest.mark.parametrize("dtype,tol", [("float16", 1e-2), ("bfloat16", 2e-2)])
+@pytest.mark.parametrize("case", PATCH_CASES)
+def test_convolution_with_the_input_patch_resident_in_lds(gpu, patch_kernel_everywhere, case, dtype, tol):
+    """The kernel of conv_patch_mfma.hip against the oracle, and bit for bit against the implicit-GEMM kernel, which
+    adds the same products in the same order."""
+    n, ic, h, w_, oc = case
+    rng = np.random.default_rng(sum(case) + 5)
+    x = round_to(rng.standard_normal((n, ic, h, w_)), dtype)
+    w = round_to(rng.standard_normal((oc, ic, 3, 3)) * np.sqrt(2.0 / (ic * 9)), dtype)
+    got = call_conv_nhwc(x, w, 1, 1, 1, dtype)
+    want = oracle.conv2d_nchw(x, w, (1, 1), (1, 1))
+    scale = oracle.conv2d_nchw(np.abs(x), np.abs(w), (1, 1), (1, 1))
+    assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+    patch_kernel_everywhere.cinn_hip_conv_patch_mode(0)
+    other = call_conv_nhwc(x, w, 1, 1, 1, dtype)
+    patch_kernel_everywhere.cinn_hip_conv_patch_mode(2)
+    assert np.all(np.abs(got - other) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+
+
+def test_patch_convolution_with_residual_epilogue(gpu, patch_kernel_everywhere):
+    """alpha / beta through the in-register epilogue: y = 0.5 conv(x, w) + 2 y0."""
+    n, ic, h, w_, oc = 2, 64, 30, 28, 128
+    rng = np.random.default_rng(197)
+    x = round_to(rng.standard_normal((n, ic, h, w_)), "float16")
+    w = round_to(rng.standard_normal((oc, ic, 3, 3)) * np.sqrt(2.0 / (ic * 9)), "float16")
+    y0 = round_to(rng.standard_normal((n, oc, h, w_)), "float16")
+    got = call_conv_nhwc(x, w, 1, 1, 1, "float16", alpha=0.5, beta=2.0, y_init=y0).astype(np.float64)
+    want = 0.5 * oracle.conv2d_nchw(x, w, (1, 1), (1, 1)).astype(np.float64) + 2.0 * y0
+    scale = 0.5 * oracle.conv2d_nchw(np.abs(x), np.abs(w), (1, 1), (1, 1)) + 2.0 * np.abs(y0)
+    assert np.all(np.abs(got - want) <= 2.0 ** -10 * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
