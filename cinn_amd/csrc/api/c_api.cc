@@ -336,6 +336,13 @@ int cinn_amd_computation_pre_run(cinn_amd_computation_t c) {
 int cinn_amd_computation_num_instructions(cinn_amd_computation_t c, int32_t* n) {
   return Guard([&] { *n = static_cast<int32_t>(c->comp->num_instructions()); });
 }
+int cinn_amd_computation_graph_lanes(cinn_amd_computation_t c, int32_t* lanes, int32_t capacity, int32_t* count) {
+  return Guard([&] {
+    const std::vector<int>& l = c->comp->GraphLanes();
+    *count                    = static_cast<int32_t>(l.size());
+    for (int32_t i = 0; i < capacity && i < *count; ++i) lanes[i] = l[i];
+  });
+}
 int cinn_amd_computation_set_tensor(cinn_amd_computation_t c, const char* name, const void* data, size_t bytes) {
   return Guard([&] { c->comp->SetTensorData(name, const_cast<void*>(data), bytes); });
 }

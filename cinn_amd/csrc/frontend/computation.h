@@ -61,6 +61,8 @@ class CinnComputation {
   const std::string& source_code() const { return source_code_; }
   std::string group_debug_string() const { return graph_->DebugGroupString(); }
   size_t num_instructions() const { return program_->size(); }
+  // stream lane (0 / 1) of every run instruction in a graph replay
+  const std::vector<int>& GraphLanes() { return program_->GraphLanes(); }
   const std::vector<std::string>& output_names() const { return output_names_; }
   const std::vector<std::string>& input_names() const { return input_names_; }
   void* stream() const { return stream_; }

@@ -103,6 +103,12 @@ void Instruction::UpdateArgsCache() {
   for (auto& a : out_args_) add(a);
 }
 
+std::vector<const void*> Instruction::ArgAddresses(bool outputs) const {
+  std::vector<const void*> out;
+  for (auto& a : outputs ? out_args_ : in_args_) out.push_back(scope_->GetTensor(a)->mutable_data(target_));
+  return out;
+}
+
 namespace {
 
 // Debug switches of Instruction::Run, read once from the environment like the reference's flags
@@ -186,6 +192,105 @@ Program::Program(std::shared_ptr<Scope> scope, std::vector<std::unique_ptr<Instr
 Program::~Program() {
   if (graph_exec_) (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec_));
   if (graph_) (void)hipGraphDestroy(static_cast<hipGraph_t>(graph_));
+  for (void* e : done_event_)
+    if (e) (void)hipEventDestroy(static_cast<hipEvent_t>(e));
+  if (fork_event_) (void)hipEventDestroy(static_cast<hipEvent_t>(fork_event_));
+  if (join_event_) (void)hipEventDestroy(static_cast<hipEvent_t>(join_event_));
+  if (side_stream_) (void)hipStreamDestroy(static_cast<hipStream_t>(side_stream_));
+}
+
+// Two stream lanes for a graph replay.  Instruction i depends on an earlier one that wrote what i reads or writes, or
+// read what i writes (by device address, so two names for one allocation count as one).  In program order, an
+// instruction that depends - directly or through others - on the last instruction of lane 0 continues lane 0; one
+// that does not can run next to it and goes to lane 1.  Across lanes an instruction waits for the latest instruction
+// of the other lane it depends on (stream order covers the earlier ones).
+void Program::PlanLanes() {
+  if (lanes_planned_) return;
+  lanes_planned_ = true;
+  const int n    = static_cast<int>(instrs_.size());
+  lane_.assign(n, 0);
+  wait_for_.assign(n, -1);
+  done_event_.assign(n, nullptr);
+  // Off unless asked for: on ResNet-50 (batch 32, fp16) the four forks and joins cost more than the overlap of the
+  // shortcut convolutions with their main branches gains (1.022 ms per batch against 1.004 ms as a single chain).
+  const char* flag = getenv("FLAGS_cinn_hip_graph_branches");
+  if (!flag || std::strcmp(flag, "1") != 0) return;
+  std::map<const void*, int> last_writer;
+  std::map<const void*, std::vector<int>> readers;  // since the last write
+  std::vector<std::vector<bool>> reach(n);          // reach[i][j]: i depends on j, directly or not
+  int tail[2] = {-1, -1};
+  for (int i = 0; i < n; ++i) {
+    std::vector<int> deps;
+    const auto ins  = instrs_[i]->ArgAddresses(false);
+    const auto outs = instrs_[i]->ArgAddresses(true);
+    for (const void* a : ins) {
+      auto w = last_writer.find(a);
+      if (w != last_writer.end()) deps.push_back(w->second);
+    }
+    for (const void* a : outs) {
+      auto w = last_writer.find(a);
+      if (w != last_writer.end()) deps.push_back(w->second);
+      for (int r : readers[a]) deps.push_back(r);
+    }
+    reach[i].assign(n, false);
+    for (int j : deps) {
+      reach[i][j] = true;
+      for (int k = 0; k < j; ++k)
+        if (reach[j][k]) reach[i][k] = true;
+    }
+    const int l = (tail[0] < 0 || reach[i][tail[0]]) ? 0 : 1;
+    lane_[i]    = l;
+    tail[l]     = i;
+    for (int j : deps)
+      if (lane_[j] != l && j > wait_for_[i]) wait_for_[i] = j;
+    for (const void* a : ins) readers[a].push_back(i);
+    for (const void* a : outs) {
+      last_writer[a] = i;
+      readers[a].clear();
+    }
+    if (l == 1) any_side_ = true;
+  }
+  if (!any_side_) return;
+  auto new_event = [] {
+    hipEvent_t e = nullptr;
+    CINN_HIP_STATUS(static_cast<int>(hipEventCreateWithFlags(&e, hipEventDisableTiming)));
+    return static_cast<void*>(e);
+  };
+  for (int i = 0; i < n; ++i)
+    if (wait_for_[i] >= 0 && !done_event_[wait_for_[i]]) done_event_[wait_for_[i]] = new_event();
+  fork_event_ = new_event();
+  join_event_ = new_event();
+  hipStream_t side = nullptr;
+  CINN_HIP_STATUS(static_cast<int>(hipStreamCreateWithFlags(&side, hipStreamNonBlocking)));  // default priority
+  side_stream_ = side;
+}
+
+const std::vector<int>& Program::GraphLanes() {
+  PlanLanes();
+  return lane_;
+}
+
+// every run instruction on its lane; the side stream starts after what `stream` holds so far and is joined at the end
+// (the fork / join a stream capture needs to take the second stream in and to end on the first)
+void Program::RunLanes(void* stream) {
+  PlanLanes();
+  if (!any_side_) {
+    for (auto& ins : instrs_) ins->Run(stream);
+    return;
+  }
+  auto main_s = static_cast<hipStream_t>(stream);
+  auto side_s = static_cast<hipStream_t>(side_stream_);
+  CINN_HIP_STATUS(static_cast<int>(hipEventRecord(static_cast<hipEvent_t>(fork_event_), main_s)));
+  CINN_HIP_STATUS(static_cast<int>(hipStreamWaitEvent(side_s, static_cast<hipEvent_t>(fork_event_), 0)));
+  for (size_t i = 0; i < instrs_.size(); ++i) {
+    hipStream_t s = lane_[i] ? side_s : main_s;
+    if (wait_for_[i] >= 0)
+      CINN_HIP_STATUS(static_cast<int>(hipStreamWaitEvent(s, static_cast<hipEvent_t>(done_event_[wait_for_[i]]), 0)));
+    instrs_[i]->Run(s);
+    if (done_event_[i]) CINN_HIP_STATUS(static_cast<int>(hipEventRecord(static_cast<hipEvent_t>(done_event_[i]), s)));
+  }
+  CINN_HIP_STATUS(static_cast<int>(hipEventRecord(static_cast<hipEvent_t>(join_event_), side_s)));
+  CINN_HIP_STATUS(static_cast<int>(hipStreamWaitEvent(main_s, static_cast<hipEvent_t>(join_event_), 0)));
 }
 
 void Program::PreRun(const common::Target& target) {
@@ -219,8 +324,9 @@ void Program::ExecuteGraph(void* stream) {
   if (!prerun_done_) RunPreRunInstructions(stream);
   if (!graph_exec_) {
     // Library-call kernels build per-shape tables and set function attributes on their first launch, which a
-    // capturing stream does not allow: run the program once before recording it.
-    for (auto& ins : instrs_) ins->Run(stream);
+    // capturing stream does not allow: run the program once before recording it, on the streams it will be recorded
+    // on.
+    RunLanes(stream);
     CINN_HIP_STATUS(static_cast<int>(hipStreamSynchronize(s)));
     // That run also sized the library's per-stream scratch (split-K partial sums, transposed operands), so the
     // recorded calls find it large enough; scratch a later call outgrows is retired, never freed, and the addresses
@@ -228,7 +334,7 @@ void Program::ExecuteGraph(void* stream) {
     hipGraph_t graph = nullptr;
     CINN_HIP_STATUS(static_cast<int>(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal)));
     try {
-      for (auto& ins : instrs_) ins->Run(stream);
+      RunLanes(stream);
     } catch (...) {
       // never leave the caller's stream in capture mode
       hipGraph_t partial = nullptr;

@@ -79,6 +79,9 @@ class Instruction {
   const std::string& function_name() const { return function_name_; }
   const std::vector<std::string>& in_args() const { return in_args_; }
   const std::vector<std::string>& out_args() const { return out_args_; }
+  // device addresses of the input / output tensors (allocates them if need be): what two instructions must not share
+  // to run side by side
+  std::vector<const void*> ArgAddresses(bool outputs) const;
   // runs once ahead of the first execution instead of in every one (cinn/hlir/framework/instruction.h:129)
   bool pre_run{false};
 
@@ -112,7 +115,12 @@ class Program {
   void Execute(void* stream = nullptr);
   // Same work replayed from a HIP graph captured on first use (removes the per-kernel launch cost
   // of programs with many small kernels).  Falls back to Execute when capture is not possible.
+  // With FLAGS_cinn_hip_graph_branches=1, instructions that do not depend on the one before them (the projection
+  // shortcut of a residual block next to the block's main branch) are recorded on a second stream, so the graph holds
+  // them as parallel branches; by default the graph is a single chain.
   void ExecuteGraph(void* stream);
+  // stream lane (0: the caller's stream, 1: the side stream) of every run instruction in a graph replay
+  const std::vector<int>& GraphLanes();
   size_t size() const { return instrs_.size(); }
   const std::vector<std::unique_ptr<Instruction>>& GetRunInstructions() const { return instrs_; }
   const std::vector<std::unique_ptr<Instruction>>& GetPreRunInstructions() const { return prerun_instrs_; }
@@ -125,6 +133,17 @@ class Program {
   bool prerun_done_{false};
   void* graph_exec_{nullptr};
   void* graph_{nullptr};
+  // two-lane schedule of a graph replay
+  void PlanLanes();
+  void RunLanes(void* stream);
+  bool lanes_planned_{false};
+  bool any_side_{false};
+  std::vector<int> lane_;                  // per run instruction
+  std::vector<int> wait_for_;              // instruction on the other lane to wait for, or -1
+  std::vector<void*> done_event_;          // recorded after the instruction when the other lane waits for it
+  void* side_stream_{nullptr};
+  void* fork_event_{nullptr};
+  void* join_event_{nullptr};
 };
 
 struct GraphCompileOptions {

@@ -357,6 +357,15 @@ class Computation(object):
     def output_names(self):
         return self._names(1)
 
+    def graph_lanes(self):
+        """stream lane (0 / 1) of every run instruction in a graph replay"""
+        n = ctypes.c_int32(0)
+        lib = _lib.load()
+        _lib.check(lib.cinn_amd_computation_graph_lanes(self._handle, None, 0, ctypes.byref(n)))
+        lanes = (ctypes.c_int32 * max(1, n.value))()
+        _lib.check(lib.cinn_amd_computation_graph_lanes(self._handle, lanes, n.value, ctypes.byref(n)))
+        return list(lanes)[:n.value]
+
     def num_instructions(self):
         n = ctypes.c_int32(0)
         _lib.check(_lib.load().cinn_amd_computation_num_instructions(self._handle, ctypes.byref(n)))

@@ -58,6 +58,9 @@ int cinn_amd_computation_execute_graph(cinn_amd_computation_t c);
  * execute does it by itself; call it again after replacing the data of a const input. */
 int cinn_amd_computation_pre_run(cinn_amd_computation_t c);
 int cinn_amd_computation_num_instructions(cinn_amd_computation_t c, int32_t* n);
+/* Stream lane of every run instruction in a graph replay (0: the computation's stream, 1: the side stream that holds
+ * instructions independent of their predecessor); writes min(capacity, *count) entries. */
+int cinn_amd_computation_graph_lanes(cinn_amd_computation_t c, int32_t* lanes, int32_t capacity, int32_t* count);
 /* SetTensorData / GetTensorData: synchronous host <-> device copies of exactly the tensor's byte size */
 int cinn_amd_computation_set_tensor(cinn_amd_computation_t c, const char* name, const void* data, size_t bytes);
 int cinn_amd_computation_get_tensor(cinn_amd_computation_t c, const char* name, void* data, size_t bytes);

@@ -136,16 +136,38 @@ def test_resnet50_batch32(gpu, dtype, tol):
     assert top1 >= (1.0 if dtype == "float32" else 0.9)
 
 
-def test_resnet50_hip_graph_replay_matches_eager(gpu):
+def test_resnet50_hip_graph_replay_matches_eager(gpu, monkeypatch):
+    """With FLAGS_cinn_hip_graph_branches=1 graph replay records the projection shortcuts next to the main branch of
+    their blocks (a second stream lane); every replay must equal eager execution on one stream bit for bit, also with
+    new input data, and so must the default graph, a single chain."""
     params = rn.random_params(4, "float16")
-    x = np.random.default_rng(5).standard_normal((4, 3, 224, 224)).astype(np.float16)
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((4, 3, 224, 224)).astype(np.float16)
+    x2 = rng.standard_normal((4, 3, 224, 224)).astype(np.float16)
     eager, _ = gpu_forward(params, x)
+    eager2, _ = gpu_forward(params, x2)
+    assert not np.array_equal(eager, eager2)
+    monkeypatch.setenv("FLAGS_cinn_hip_graph_branches", "1")
     stream = runtime.Stream()
     _, comp = gpu_forward(params, x, stream=stream)
-    for _ in range(3):
+    lanes = comp.graph_lanes()
+    assert len(lanes) == comp.num_instructions()
+    # four blocks have a projection shortcut: in each, either it or the main branch leaves the first lane
+    assert lanes[0] == 0 and sum(1 for a, b in zip(lanes, lanes[1:]) if a == 0 and b == 1) >= 4, lanes
+    out = comp.output_names()[0]
+    for data, want in ((x, eager), (x, eager), (x2, eager2), (x, eager)):
+        comp.get_tensor("image").from_numpy(data)
         comp.execute_graph()
         stream.synchronize()
-        assert np.array_equal(comp.get_tensor(comp.output_names()[0]).numpy(), eager)
+        assert np.array_equal(comp.get_tensor(out).numpy(), want)
+    monkeypatch.delenv("FLAGS_cinn_hip_graph_branches")
+    stream1 = runtime.Stream()
+    _, chain = gpu_forward(params, x, stream=stream1)
+    assert set(chain.graph_lanes()) == {0}
+    for _ in range(2):
+        chain.execute_graph()
+        stream1.synchronize()
+        assert np.array_equal(chain.get_tensor(out).numpy(), eager)
 
 
 def test_const_weights_are_prepared_once_and_pre_run_refreshes_them(gpu):
