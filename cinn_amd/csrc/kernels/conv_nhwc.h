@@ -51,4 +51,9 @@ void RunDepthwiseNhwc(const ConvNhwcArgs& a, hipStream_t stream);
 bool ConvStemSupported(const ConvNhwcArgs& a);
 void RunConvStem(const ConvNhwcArgs& a, hipStream_t stream);
 
+// the 7x7, stride 2, padding 3 convolution of a 3-channel NCHW image in 16-bit types (conv_stem7_mfma.hip): persistent
+// blocks with the next tile's input rows fetched while the current tile is multiplied; false when the shape does not
+// qualify
+bool TryConvStem7(const ConvNhwcArgs& a, hipStream_t stream);
+
 }  // namespace cinn_hip_kernels

@@ -662,6 +662,7 @@ void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream) {
   CINN_RT_CHECK(ConvNhwcSupported(a), "conv2d (channels-last): unsupported type or channel count %d", a.c);
   CINN_RT_CHECK((int64_t)a.n * a.h * a.w_in * a.c < INT_MAX && (int64_t)a.n * a.oh * a.ow * a.oc < INT_MAX,
                 "conv2d (channels-last): tensor too large for 32-bit offsets");
+  if (TryConvStem7(a, stream)) return;
   if (ConvStemSupported(a)) {
     RunConvStem(a, stream);
     return;

@@ -564,3 +564,55 @@ def test_patch_convolution_with_residual_epilogue(gpu, patch_kernel_everywhere):
     want = 0.5 * oracle.conv2d_nchw(x, w, (1, 1), (1, 1)).astype(np.float64) + 2.0 * y0
     scale = 0.5 * oracle.conv2d_nchw(np.abs(x), np.abs(w), (1, 1), (1, 1)) + 2.0 * np.abs(y0)
     assert np.all(np.abs(got - want) <= 2.0 ** -10 * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+
+
+STEM7_CASES = [
+    # (n, h, w, oc): 7x7, stride 2, padding 3 over 3 channels, NCHW input -> NHWC output
+    (1, 224, 224, 64),    # 28 tiles of 4 output rows
+    (2, 96, 80, 128),     # tiles of 10 rows of 40 pixels, the last one 8 rows; two groups of output channels
+    (3, 56, 128, 64),     # 7 rows of 64 pixels per tile
+    (10, 224, 224, 64),   # 280 tiles on 256 persistent blocks: some blocks take a second tile into the other buffer
+]
+
+
+@pytest.mark.parametrize("dtype,tol", [("float16", 1e-2), ("bfloat16", 2e-2)])
+@pytest.mark.parametrize("case", STEM7_CASES)
+def test_image_convolution_7x7_stride2(gpu, case, dtype, tol):
+    """conv_stem7_mfma.hip against the oracle; a NaN two columns left of a window's first filter column (the slot
+    the kernel's fragments carry with a zero weight) must not reach that window's output."""
+    n, h, w_, oc = case
+    rng = np.random.default_rng(sum(case) + 3)
+    x = round_to(rng.standard_normal((n, 3, h, w_)), dtype)
+    w = round_to(rng.standard_normal((oc, 3, 7, 7)) * np.sqrt(2.0 / 147), dtype)
+    got = call_conv_nhwc(x, w, 2, 3, 2, dtype)
+    want = oracle.conv2d_nchw(x, w, (2, 2), (3, 3))
+    scale = oracle.conv2d_nchw(np.abs(x), np.abs(w), (2, 2), (3, 3))
+    assert got.shape == want.shape
+    assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+    if n == 1:
+        x[0, 1, 20, 36] = np.nan  # column 36 = 2 * 20 - 4: slot 0 of output column 20, a real tap of columns 17..19
+        got = call_conv_nhwc(x, w, 2, 3, 2, dtype)
+        bad = np.isnan(got[0, 0])
+        assert not bad[:, 20].any() and bad[10, 19] and bad[10, 17] and not bad[10, 16]
+
+
+def test_image_convolution_7x7_with_folded_epilogue(gpu):
+    """batch norm + relu folded into the image convolution, through NetBuilder (scale / shift table in LDS)."""
+    rng = np.random.default_rng(29)
+    x = rng.standard_normal((2, 3, 224, 224)).astype(np.float16)
+    w = (rng.standard_normal((64, 3, 7, 7)) * np.sqrt(2.0 / 147)).astype(np.float16)
+    scale, bias = rng.uniform(0.5, 1.5, 64).astype(np.float16), rng.standard_normal(64).astype(np.float16)
+    mean, var = (rng.standard_normal(64) * 0.1).astype(np.float16), rng.uniform(0.5, 1.5, 64).astype(np.float16)
+    b = NetBuilder("stem7")
+    X = b.create_input(Float(16), x.shape, "x")
+    W = b.create_input(Float(16), w.shape, "w").set_const()
+    P = [b.create_input(Float(16), [64], nm).set_const() for nm in ("scale", "bias", "mean", "var")]
+    y = b.pool2d(b.relu(b.batchnorm(b.conv2d(X, W, strides=[2, 2], paddings=[3, 3]), *P)[0]), "max", [3, 3], [2, 2],
+                 [1, 1, 1, 1])
+    (got,), comp = run(b, {X: x, W: w, P[0]: scale, P[1]: bias, P[2]: mean, P[3]: var}, [y])
+    conv = oracle.conv2d_nchw(x.astype(np.float32), w.astype(np.float32), (2, 2), (3, 3))
+    act = oracle.batch_norm_relu_nchw(conv, scale.astype(np.float32), bias.astype(np.float32), mean.astype(np.float32),
+                                      var.astype(np.float32), 1e-5, relu=True)
+    want = oracle.pool2d_nchw(act.astype(np.float16), (3, 3), (2, 2), (1, 1, 1, 1), "max")
+    # relative to the value or, where the convolution's terms cancel, to a twentieth of the activations' unit scale
+    assert np.all(np.abs(got.astype(np.float64) - want) <= 1e-2 * np.maximum(np.abs(want), 0.05))
