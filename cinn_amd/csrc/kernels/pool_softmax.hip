@@ -8,6 +8,8 @@
 // the exclusive mode, kh*kw otherwise), window rows then columns in ascending order.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include <climits>
 #include <cstdint>
 
@@ -75,11 +77,15 @@ __global__ void __launch_bounds__(256) pool2d_nchw_kernel(const T* __restrict__ 
 // Channels-last pooling: one thread per output pixel and group of V consecutive channels (V elements = 16 bytes
 // when the channel count allows), so that every access is one contiguous vector and consecutive lanes read
 // consecutive vectors.  Arithmetic and order of operations are those of the NCHW kernel.
+// Blocks are dispatched round-robin to the 8 XCDs, each with an L2 of its own; the grid (a multiple of 8 blocks) is
+// renumbered so that an XCD works on one contiguous eighth of the output, and overlapping windows of neighbouring
+// output rows find their shared input rows in that XCD's L2 instead of fetching them once per XCD.
 template <typename T, int V>
 __global__ void __launch_bounds__(256) pool2d_nhwc_kernel(const T* __restrict__ in, T* __restrict__ out, PoolParams p) {
   const int groups    = p.c / V;
   const int64_t total = (int64_t)p.n * p.oh * p.ow * groups;
-  const int64_t idx   = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const unsigned block = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  const int64_t idx   = (int64_t)block * 256 + threadIdx.x;
   if (idx >= total) return;
   const int g         = (int)(idx % groups);
   const int64_t pixel = idx / groups;
@@ -129,6 +135,54 @@ __global__ void __launch_bounds__(256) pool2d_nhwc_kernel(const T* __restrict__ 
   __builtin_memcpy(dst, res, V * sizeof(T));
 }
 
+
+// Max pooling of fp16 channels-last tensors with a small window (3x3 stride 2 after the first convolution of an image
+// network): the generic kernel above spends ~800 instructions per thread - 64-bit index divisions, a float conversion
+// and a compare / select pair per element and tap - and is bound by them, not by memory (25 us for 64 MB at batch 32).
+// Here the indices are 32-bit, the window is unrolled with clamped, unconditional loads (all in flight together), taps
+// outside the image are replaced by -inf, and the maximum is taken on packed halves.  The maximum of halves is exact,
+// so results equal the generic kernel's (which compares the same values as floats) except that max(+0, -0) may carry
+// either sign.
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+template <int KH, int KW>
+__global__ void __launch_bounds__(256) maxpool_nhwc_f16_kernel(const _Float16* __restrict__ in, _Float16* __restrict__ out,
+                                                               PoolParams p) {
+  const unsigned groups = (unsigned)p.c >> 3;
+  const unsigned total  = (unsigned)p.n * p.oh * p.ow * groups;
+  const unsigned block  = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);  // an XCD works on one eighth
+  const unsigned idx    = block * 256u + threadIdx.x;
+  if (idx >= total) return;
+  const unsigned pixel = idx / groups, g = idx - pixel * groups;
+  const unsigned t = pixel / (unsigned)p.ow, x = pixel - t * p.ow;
+  const unsigned n = t / (unsigned)p.oh, y = t - n * p.oh;
+  const _Float16* src = in + (int64_t)n * p.ih * p.iw * p.c + g * 8;
+  const int ys = (int)y * p.sh - p.ph, xs = (int)x * p.sw - p.pw;
+  const _Float16 ninf = -__builtin_huge_valf();
+  half8 v[KH][KW];
+#pragma unroll
+  for (int ry = 0; ry < KH; ++ry) {
+    const int yy = ys + ry, yc = yy < 0 ? 0 : (yy < p.ih ? yy : p.ih - 1);
+#pragma unroll
+    for (int rx = 0; rx < KW; ++rx) {
+      const int xx = xs + rx, xc = xx < 0 ? 0 : (xx < p.iw ? xx : p.iw - 1);
+      v[ry][rx]    = *reinterpret_cast<const half8*>(src + (unsigned)((yc * p.iw + xc) * p.c));
+    }
+  }
+  half8 acc;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = ninf;
+#pragma unroll
+  for (int ry = 0; ry < KH; ++ry)
+#pragma unroll
+    for (int rx = 0; rx < KW; ++rx) {
+      const bool ok = (unsigned)(ys + ry) < (unsigned)p.ih && (unsigned)(xs + rx) < (unsigned)p.iw;
+      half8 tap     = v[ry][rx];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) tap[e] = ok ? tap[e] : ninf;
+      acc = __builtin_elementwise_max(acc, tap);
+    }
+  *reinterpret_cast<half8*>(out + (int64_t)pixel * p.c + g * 8) = acc;
+}
 
 // Channels-last pooling whose window is the whole image (global average / max pooling): the generic kernel would give
 // each thread the entire image of its channels to walk through.  Here a block of 256 threads takes one image and 64
@@ -194,13 +248,24 @@ void LaunchPoolNhwc(const void* x, void* y, const PoolParams& p, hipStream_t s) 
                        static_cast<const T*>(x), static_cast<T*>(y), p);
     return;
   }
+  if (sizeof(T) == 2 && p.c % 8 == 0) {
+    // fp16 max pooling with a 3x3 window and no alpha / beta: the packed-half kernel
+    const int64_t total = (int64_t)p.n * p.oh * p.ow * (p.c / 8);
+    const bool is_f16   = std::is_same<T, _Float16>::value;
+    if (is_f16 && (p.mode == 0 || p.mode == 3) && p.kh == 3 && p.kw == 3 && p.alpha == 1.0f && p.beta == 0.0f &&
+        total < (1ll << 31) && (int64_t)p.ih * p.iw * p.c < (1ll << 31)) {
+      hipLaunchKernelGGL((maxpool_nhwc_f16_kernel<3, 3>), dim3((unsigned)(((total + 255) / 256 + 7) / 8 * 8)), dim3(256), 0, s,
+                         static_cast<const _Float16*>(x), static_cast<_Float16*>(y), p);
+      return;
+    }
+  }
   if (p.c % V == 0) {
     const int64_t total = (int64_t)p.n * p.oh * p.ow * (p.c / V);
-    hipLaunchKernelGGL((pool2d_nhwc_kernel<T, V>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+    hipLaunchKernelGGL((pool2d_nhwc_kernel<T, V>), dim3((unsigned)(((total + 255) / 256 + 7) / 8 * 8)), dim3(256), 0, s,
                        static_cast<const T*>(x), static_cast<T*>(y), p);
   } else {
     const int64_t total = (int64_t)p.n * p.oh * p.ow * p.c;
-    hipLaunchKernelGGL((pool2d_nhwc_kernel<T, 1>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+    hipLaunchKernelGGL((pool2d_nhwc_kernel<T, 1>), dim3((unsigned)(((total + 255) / 256 + 7) / 8 * 8)), dim3(256), 0, s,
                        static_cast<const T*>(x), static_cast<T*>(y), p);
   }
 }

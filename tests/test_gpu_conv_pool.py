@@ -178,6 +178,34 @@ def test_pool2d_intrinsic(gpu, pool_type, exclusive, mode):
         np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-7)
 
 
+@pytest.mark.parametrize("shape,stride,pad", [((3, 64, 29, 31), 2, 1), ((2, 8, 7, 9), 1, 1), ((2, 136, 12, 12), 2, 0)])
+def test_max_pool_3x3_fp16_channels_last(gpu, shape, stride, pad):
+    """The packed-half 3x3 max-pooling kernel (format 1, fp16): bit-equal to the oracle, also with infinities and
+    with rows / columns of the window outside the image."""
+    rng = np.random.default_rng(sum(shape))
+    x = rng.standard_normal(shape).astype(np.float16)
+    x[0, :, 0, 0] = -np.inf
+    x[0, :, 1, :3] = -np.inf
+    x[0, :, 0, 1:3] = -np.inf   # a corner window whose taps inside the image are all -inf
+    x[1, 0, 3, 3] = np.inf
+    # the oracle starts from the lowest float, as the reference does: as a half that is -inf
+    want = oracle.pool2d_nchw(x, (3, 3), (stride, stride), (pad, pad, pad, pad), "max").astype(np.float16)
+    lib = _lib.load()
+    lib.cinn_call_cudnn_pool2d_forward.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                   ctypes.c_float, ctypes.c_float] + [ctypes.c_int] * 14 + [ctypes.c_void_p]
+    n, c, ih, iw = shape
+    oh, ow = want.shape[2:]
+    X = runtime.DeviceBuffer.from_numpy(np.ascontiguousarray(x.transpose(0, 2, 3, 1)), "float16")
+    Y = runtime.DeviceBuffer((n, oh, ow, c), "float16")
+    lib.cinn_call_cudnn_pool2d_forward(runtime.pod_args([X, Y]), 2, 0, 1, 1.0, 0.0, n, c, ih, iw, 3, 3, pad, pad, stride,
+                                       stride, n, c, oh, ow, None)
+    runtime.synchronize()
+    got = Y.numpy().transpose(0, 3, 1, 2)
+    assert np.array_equal(got, want)
+    if pad == 1:
+        assert np.isneginf(got[0, :, 0, 0]).all()
+
+
 def test_pool2d_through_netbuilder_resnet_layers_and_golden(gpu):
     f = load("pool2d")
     b = NetBuilder("p")
