@@ -299,6 +299,10 @@ struct DmaEpilogue {
   float residual_scale;
   int relu;
   int streaming;          // store the result with non-temporal stores (large outputs nobody re-reads from L2)
+  // Split reduction: blockIdx.z = s takes the K steps [s * steps_per_split, (s + 1) * steps_per_split) and writes its
+  // raw fp32 sums to partials[s][M][N]; the epilogue is applied by gemm16_split_reduce_kernel.  Null: no split.
+  float* partials;
+  int steps_per_split;
 };
 
 // Implicit-GEMM view of a channels-last convolution for gemm16_dma_kernel<.., CONV = true>: row m of A is output pixel
@@ -384,8 +388,12 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   // instead - what they compute is not stored.  The bases lie kBias bytes below the tile and every lane offset
   // includes kBias, so that an offset less its instruction offset never wraps below zero.
   constexpr int kBias = 4096;
-  const char* const a_base = reinterpret_cast<const char*>(A + (int64_t)m0 * lda) - kBias;
-  const char* const b_base = reinterpret_cast<const char*>(B + (B_KC ? (int64_t)n0 * ldb : (int64_t)n0)) - kBias;
+  // this block's K steps: all of them, or the split's share
+  const int kt0 = epi.partials ? (int)blockIdx.z * epi.steps_per_split : 0;
+  const int64_t b_step = (B_KC ? kD64BK : (int64_t)kD64BK * ldb) * 2;  // bytes per K step
+  const char* const a_base = reinterpret_cast<const char*>(A + (int64_t)m0 * lda) - kBias + (int64_t)kt0 * (kD64BK * 2);
+  const char* const b_base =
+      reinterpret_cast<const char*>(B + (B_KC ? (int64_t)n0 * ldb : (int64_t)n0)) - kBias + kt0 * b_step;
   const int a_last = M - 1 - m0;  // last valid row of this tile (>= 0)
   const int b_last = N - 1 - n0;
   // CONV: a_off is the byte offset of the lane's chunk at the top-left corner of the pixel's window (it may lie before
@@ -414,6 +422,13 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   // CONV: filter tap and first channel of the K step whose loads are being issued (all loads of one step are issued
   // between two advances)
   int tap_dy = 0, tap_dx = 0, tap_c0 = 0;
+  if (CONV && kt0 > 0) {
+    const int k0  = kt0 * kD64BK;
+    const int tap = k0 / geom.c;
+    tap_c0        = k0 - tap * geom.c;
+    tap_dy        = tap / geom.kw;
+    tap_dx        = tap - tap_dy * geom.kw;
+  }
   auto advance_tap = [&]() {
     tap_c0 += kD64BK;
     if (tap_c0 == geom.c) {
@@ -441,7 +456,6 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
       b_off[t]         = (unsigned)(((int64_t)krow * ldb + (chunk_c << 3)) * 2 + kBias - 1024 * (t & 3));
     }
   }
-  const int64_t b_step = (B_KC ? kD64BK : (int64_t)kD64BK * ldb) * 2;  // bytes per K step
   // load t of step kt: first the LPA loads of the A tile, then the LPB loads of the B tile
   auto issue_one = [&](char* a_tile, char* b_tile, int kt, int t) {
     if (t < LPA) {
@@ -534,7 +548,8 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   vec8 ring[4];
   vec8 bf[2][TN];
 
-  const int nk = K / kD64BK;
+  const int nk_all = K / kD64BK;
+  const int nk     = epi.partials ? (nk_all - kt0 < epi.steps_per_split ? nk_all - kt0 : epi.steps_per_split) : nk_all;
   constexpr int L = LPA + LPB;  // loads of a loader wavefront per stage
   // vmcnt(n): at most n of the wavefront's loads still in flight; they complete in the order they were issued
 #define CINN_VMCNT(n) ((((n) & 15) | (((n) >> 4) << 14)) | 0x0F70)
@@ -698,6 +713,46 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   // optional relu, one rounding to T.  The tile goes through LDS so that every lane moves 16 bytes and a store
   // instruction covers whole rows of the C tile instead of 64 two-byte pieces: as 16-bit values, 64 rows of every
   // wavefront per pass, or - with a residual, which is added before the rounding - as fp32, 32 rows per pass.
+  if (epi.partials) {
+    // split reduction: the raw sums as fp32 rows (through LDS, 32 rows per wavefront row and pass, so that a lane
+    // stores 2 x 16 contiguous bytes)
+    constexpr int kRowFloats = BN + 4;
+    constexpr int IB         = 2;
+    constexpr int PASS_ROWS  = WAVES_M * IB * 16;
+    constexpr int CPR8       = BN / 8;
+    static_assert(PASS_ROWS * kRowFloats * 4 <= NS * STAGE, "the staged partial sums do not fit the operand stages");
+    static_assert(PASS_ROWS * CPR8 % THREADS == 0, "the copy-out loop assumes whole rounds");
+    float* stage = reinterpret_cast<float*>(lds);
+    float* P     = epi.partials + (int64_t)blockIdx.z * M * N;
+#pragma unroll
+    for (int pass = 0; pass < TM / IB; ++pass) {
+      __syncthreads();
+      if (!feeder)
+#pragma unroll
+      for (int ii = 0; ii < IB; ++ii)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int lrow = wm * (IB * 16) + ii * 16 + 4 * (lane >> 4) + r;
+            const int col  = wn * (TN * 16) + j * 16 + (lane & 15);
+            stage[lrow * kRowFloats + col] = acc[IB * pass + ii][j][r];
+          }
+      __syncthreads();
+#pragma unroll
+      for (int e = 0; e < PASS_ROWS * CPR8 / THREADS; ++e) {
+        const int chunk = e * THREADS + tid;
+        const int lrow  = chunk / CPR8;
+        const int c8    = chunk % CPR8;
+        const int row   = m0 + (lrow / (IB * 16)) * (TM * 16) + pass * (IB * 16) + lrow % (IB * 16);
+        if (row >= M || n0 + c8 * 8 >= N) continue;
+        float* dst = P + (int64_t)row * N + n0 + c8 * 8;
+        *reinterpret_cast<f32x4*>(dst)     = *reinterpret_cast<const f32x4*>(stage + lrow * kRowFloats + c8 * 8);
+        *reinterpret_cast<f32x4*>(dst + 4) = *reinterpret_cast<const f32x4*>(stage + lrow * kRowFloats + c8 * 8 + 4);
+      }
+    }
+    return;
+  }
   T* Ct       = reinterpret_cast<T*>(C);
   const T* Rt = reinterpret_cast<const T*>(epi.residual);
   if (Rt) Rt += (int64_t)blockIdx.y * stride_c;
@@ -1297,6 +1352,41 @@ void LaunchFast16(const GemmProblem& p, hipStream_t stream) {
                      (int64_t)p.n, p.alpha, p.beta, p.stride_a, p.stride_b, p.stride_c);
 }
 
+// Sum of the fp32 partial tiles of a split reduction, then the epilogue of gemm16_dma_kernel: 8 columns per thread
+// (N % 8 == 0), the same fused multiply-adds and the single rounding to T.
+template <typename T>
+__global__ void __launch_bounds__(256)
+gemm16_split_reduce_kernel(const float* __restrict__ partials, T* C, int64_t total8, int N, int64_t plane, int splits,
+                           DmaEpilogue epi) {
+  typedef typename Half16<T>::vec8 vec8;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total8) return;
+  const int64_t off = idx * 8;
+  const int col     = (int)(off % N);
+  float v[8];
+#pragma unroll
+  for (int q = 0; q < 8; ++q) v[q] = 0.0f;
+  for (int s = 0; s < splits; ++s) {
+    const f32x4 lo = *reinterpret_cast<const f32x4*>(partials + s * plane + off);
+    const f32x4 hi = *reinterpret_cast<const f32x4*>(partials + s * plane + off + 4);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) v[q] += lo[q], v[4 + q] += hi[q];
+  }
+  const T* Rt = reinterpret_cast<const T*>(epi.residual);
+  vec8 rq;
+  if (Rt) rq = *reinterpret_cast<const vec8*>(Rt + off);
+  vec8 out;
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    float t = __builtin_fmaf(v[q], epi.scale ? epi.scale[col + q] : epi.alpha, epi.shift ? epi.shift[col + q] : 0.0f);
+    if (Rt) t = __builtin_fmaf(epi.residual_scale, (float)rq[q], t);
+    asm volatile("" : "+v"(t));
+    if (epi.relu) t = t > 0.0f ? t : 0.0f;
+    out[q] = (T)t;
+  }
+  *reinterpret_cast<vec8*>(C + off) = out;
+}
+
 // split a tiles_m x tiles_n grid over the 8 XCDs as gr x gc rectangles with the smallest half-perimeter; sub_rows
 // stays 0 when the grid does not divide
 void XcdRectangles(int tiles_m, int tiles_n, int* xcd_cols, int* sub_rows, int* sub_cols) {
@@ -1327,15 +1417,22 @@ void XcdRectanglesPadded(int tiles_m, int tiles_n, int* xcd_cols, int* sub_rows,
 }
 
 template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false, int NS = 2, bool FEED = false>
-void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
+void LaunchDma16(const GemmProblem& p, hipStream_t stream, int splits = 1) {
   int64_t ldb = p.trans_b ? p.k : p.n;
   const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
   // XCD rectangles for tile grids large enough to have panels to share; a small grid per batch entry is numbered
   // linearly (padded rectangles would leave whole XCDs with nothing but blocks that return at once)
   int xcd_cols = 0, sub_rows = 0, sub_cols = 0;
   if (tiles_m * tiles_n >= 64) XcdRectanglesPadded(tiles_m, tiles_n, &xcd_cols, &sub_rows, &sub_cols);
-  dim3 grid(sub_rows > 0 ? 8 * sub_rows * sub_cols : tiles_m * tiles_n, p.batch, 1);
+  dim3 grid(sub_rows > 0 ? 8 * sub_rows * sub_cols : tiles_m * tiles_n, p.batch, splits);
   DmaEpilogue epi;
+  epi.partials        = nullptr;
+  epi.steps_per_split = 0;
+  if (splits > 1) {
+    CINN_RT_CHECK(p.batch == 1 && p.beta == 0.0f, "a split reduction takes one unbatched product without a beta term");
+    epi.partials        = static_cast<float*>(cinn_hip_kernels::Scratch(cinn_hip_kernels::ScratchKind::kSplitK, (size_t)splits * p.m * p.n * sizeof(float), stream));
+    epi.steps_per_split = (p.k / kD64BK + splits - 1) / splits;
+  }
   epi.scale          = p.scale;
   epi.shift          = p.shift;
   epi.alpha          = p.alpha;
@@ -1351,6 +1448,11 @@ void LaunchDma16(const GemmProblem& p, hipStream_t stream) {
                      stream, static_cast<const uint16_t*>(p.a), static_cast<const uint16_t*>(p.b),
                      static_cast<uint16_t*>(p.c), p.m, p.n, p.k, (int64_t)p.k, ldb, (int64_t)p.n, epi, p.stride_a,
                      p.stride_b, p.stride_c, xcd_cols, sub_rows, sub_cols, geom);
+  if (splits > 1) {
+    const int64_t total8 = (int64_t)p.m * p.n / 8;
+    hipLaunchKernelGGL((gemm16_split_reduce_kernel<T>), dim3((unsigned)((total8 + 255) / 256)), dim3(256), 0, stream,
+                       epi.partials, static_cast<T*>(p.c), total8, p.n, (int64_t)p.m * p.n, splits, epi);
+  }
 }
 
 // gemm16_shortk_kernel: K = 64, either layout of B, N a multiple of the 128 columns of a wavefront, at least 16384 rows.
@@ -1465,6 +1567,20 @@ bool TryDma16(const GemmProblem& p, hipStream_t stream) {
     if (tiles256 >= 192 && forced != 128) {
       LaunchDma16<T, true, 256, 256, 2, 4, true>(p, stream);
       return true;
+    }
+    // Few tiles and a long reduction (512 -> 512 3x3 on 7x7 at batch 32: 52 tiles of 128x128, K = 4608): the
+    // reduction is split over blockIdx.z so that about 200 blocks run, each at least 8 K steps long; a second kernel
+    // adds the partial sums.
+    // FLAGS_cinn_hip_gemm_split_k: 0 switches it off, a value of 2 or more forces that many splits
+    static const int split_flag = getenv("FLAGS_cinn_hip_gemm_split_k") ? atoi(getenv("FLAGS_cinn_hip_gemm_split_k")) : 1;
+    if (split_flag != 0 && FeedWavefronts() && forced == 0 && tiles128 >= 32 && tiles128 < 96 && p.k >= 2048 && p.batch == 1 &&
+        p.n % 8 == 0) {
+      int splits = split_flag >= 2 ? split_flag : (int)((208 + tiles128 - 1) / tiles128);
+      while (splits > 1 && p.k / kD64BK / splits < 8) --splits;
+      if (splits > 1) {
+        LaunchDma16<T, true, 128, 128, 2, 2, true, 4, true>(p, stream, splits);
+        return true;
+      }
     }
     // measured on ResNet-50 at batch 32 (fp16): from 192 tiles of 128x128 (four stages up to 256 tiles) the network
     // is 0.5-1 % faster with these layers here than on the 64x64 tiles of the convolution kernel, with 96 tiles 2 %

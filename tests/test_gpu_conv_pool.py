@@ -189,7 +189,8 @@ def test_max_pool_3x3_fp16_channels_last(gpu, shape, stride, pad):
     x[0, :, 0, 1:3] = -np.inf   # a corner window whose taps inside the image are all -inf
     x[1, 0, 3, 3] = np.inf
     # the oracle starts from the lowest float, as the reference does: as a half that is -inf
-    want = oracle.pool2d_nchw(x, (3, 3), (stride, stride), (pad, pad, pad, pad), "max").astype(np.float16)
+    with np.errstate(over="ignore"):
+        want = oracle.pool2d_nchw(x, (3, 3), (stride, stride), (pad, pad, pad, pad), "max").astype(np.float16)
     lib = _lib.load()
     lib.cinn_call_cudnn_pool2d_forward.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
                                                    ctypes.c_float, ctypes.c_float] + [ctypes.c_int] * 14 + [ctypes.c_void_p]
@@ -644,3 +645,22 @@ def test_image_convolution_7x7_with_folded_epilogue(gpu):
     want = oracle.pool2d_nchw(act.astype(np.float16), (3, 3), (2, 2), (1, 1, 1, 1), "max")
     # relative to the value or, where the convolution's terms cancel, to a twentieth of the activations' unit scale
     assert np.all(np.abs(got.astype(np.float64) - want) <= 1e-2 * np.maximum(np.abs(want), 0.05))
+
+
+@pytest.mark.parametrize("dtype,tol", [("float16", 1e-2), ("bfloat16", 2e-2)])
+@pytest.mark.parametrize("case", [(32, 512, 7, 7, 512), (20, 256, 9, 9, 384)])
+def test_implicit_gemm_convolution_with_split_reduction(gpu, case, dtype, tol):
+    """Few 128x128 tiles and a long reduction (the 3x3 layers of the last ResNet stage): K is split over the grid's
+    third dimension, fp32 partial sums are added by a second kernel, which also applies alpha / beta."""
+    n, ic, h, w_, oc = case
+    rng = np.random.default_rng(sum(case) + 1)
+    x = round_to(rng.standard_normal((n, ic, h, w_)), dtype)
+    w = round_to(rng.standard_normal((oc, ic, 3, 3)) * np.sqrt(2.0 / (ic * 9)), dtype)
+    y0 = round_to(rng.standard_normal((n, oc, h, w_)), dtype)
+    want = oracle.conv2d_nchw(x, w, (1, 1), (1, 1)).astype(np.float64)
+    scale = oracle.conv2d_nchw(np.abs(x), np.abs(w), (1, 1), (1, 1))
+    got = call_conv_nhwc(x, w, 1, 1, 1, dtype)
+    assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+    got = call_conv_nhwc(x, w, 1, 1, 1, dtype, alpha=0.5, beta=2.0, y_init=y0)
+    want2 = 0.5 * want + 2.0 * y0
+    assert np.all(np.abs(got - want2) <= tol * np.maximum(np.abs(want2), 1e-2 * (0.5 * scale + 2.0 * np.abs(y0))) + 1e-6)
