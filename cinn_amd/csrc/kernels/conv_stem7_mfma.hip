@@ -87,6 +87,15 @@ __device__ __forceinline__ unsigned RowShift8(unsigned v) {
   return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, SHR ? 0x118 : 0x108, 0xf, 0xf, true);
 }
 
+// Block barrier that orders LDS accesses only.  __syncthreads() also waits until every global store of the wavefront
+// has completed (its release covers global memory); here that would stall the computing wavefronts at every tile until
+// the tile's 57 KB of results have left, instead of letting them drain under the next tile's MFMAs.
+__device__ __forceinline__ void BarrierLds() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 template <typename T>
 __global__ void __launch_bounds__(128 * kWaves) conv_stem7_kernel(Stem7Params p) {
   typedef typename Mfma16<T>::vec8 vec8;
@@ -149,7 +158,7 @@ __global__ void __launch_bounds__(128 * kWaves) conv_stem7_kernel(Stem7Params p)
 #pragma unroll
       for (int e = 0; e < kMaxVectors; ++e)
         if (dst[e] >= 0) *reinterpret_cast<u32x4*>(buf + dst[e]) = regs[e];
-      __syncthreads();  // tile k is in its buffer; the other buffer's tile (k - 1) has been multiplied
+      BarrierLds();  // tile k is in its buffer; the other buffer's tile (k - 1) has been multiplied
     }
     return;
   }
@@ -202,7 +211,7 @@ __global__ void __launch_bounds__(128 * kWaves) conv_stem7_kernel(Stem7Params p)
     const int oy0  = (t - img * p.strips) * p.rows;
     const int npix = min(p.rows, p.oh - oy0) * p.ow;
     const char* const buf = patch0 + (k & 1) * p.patch_bytes;
-    __syncthreads();  // tile k is in its buffer
+    BarrierLds();  // tile k is in its buffer
 
     f32x4 acc[kTMW][4];
 #pragma unroll
