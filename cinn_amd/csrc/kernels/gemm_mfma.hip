@@ -1366,19 +1366,33 @@ gemm16_split_reduce_kernel(const float* __restrict__ partials, T* C, int64_t tot
   float v[8];
 #pragma unroll
   for (int q = 0; q < 8; ++q) v[q] = 0.0f;
-  for (int s = 0; s < splits; ++s) {
-    const f32x4 lo = *reinterpret_cast<const f32x4*>(partials + s * plane + off);
-    const f32x4 hi = *reinterpret_cast<const f32x4*>(partials + s * plane + off + 4);
-#pragma unroll
-    for (int q = 0; q < 4; ++q) v[q] += lo[q], v[4 + q] += hi[q];
-  }
+  // four partial tiles at a time, all their loads in flight together (a fifth split and beyond repeat the round)
   const T* Rt = reinterpret_cast<const T*>(epi.residual);
   vec8 rq;
   if (Rt) rq = *reinterpret_cast<const vec8*>(Rt + off);
+  f32x4 sc[2], sh[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    sc[h] = epi.scale ? *reinterpret_cast<const f32x4*>(epi.scale + col + 4 * h) : f32x4{epi.alpha, epi.alpha, epi.alpha, epi.alpha};
+    sh[h] = epi.shift ? *reinterpret_cast<const f32x4*>(epi.shift + col + 4 * h) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  }
+  for (int s0 = 0; s0 < splits; s0 += 4) {
+    f32x4 part[4][2];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+        part[u][h] = s0 + u < splits ? *reinterpret_cast<const f32x4*>(partials + (s0 + u) * plane + off + 4 * h)
+                                     : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v[q] += part[u][0][q], v[4 + q] += part[u][1][q];
+  }
   vec8 out;
 #pragma unroll
   for (int q = 0; q < 8; ++q) {
-    float t = __builtin_fmaf(v[q], epi.scale ? epi.scale[col + q] : epi.alpha, epi.shift ? epi.shift[col + q] : 0.0f);
+    float t = __builtin_fmaf(v[q], sc[q >> 2][q & 3], sh[q >> 2][q & 3]);
     if (Rt) t = __builtin_fmaf(epi.residual_scale, (float)rq[q], t);
     asm volatile("" : "+v"(t));
     if (epi.relu) t = t > 0.0f ? t : 0.0f;
