@@ -25,6 +25,7 @@ class CinnComputation {
     // epilogue applies the folded batch norm in fp32 on the accumulators (frontend/layout_pass.h).  The result
     // differs from the unfused operation order by rounding only; switch it off to get that order exactly.
     bool fuse_conv_bn_relu{true};
+    bool fuse_stem_pool{true};  // fold the max pooling after an image convolution into it
     // move conv2d chains written in NCHW to channels-last tensors, the layout the MFMA convolution kernels read
     // with 16-byte accesses (frontend/layout_pass.h); off: every conv2d runs in the layout it was written in
     bool conv_layout_nhwc{true};

@@ -3,8 +3,10 @@
 #include <algorithm>
 #include <map>
 
+#include "cinn_hip_runtime.h"
 #include "frontend/pass_util.h"
 #include "hlir/op.h"
+#include "kernels/stem_pool.h"
 
 namespace cinn {
 namespace frontend {
@@ -227,7 +229,37 @@ Program PretransposeConstMatmulWeights(const Program& program) {
   return Program(std::move(out), program.GetInputs(), program.name());
 }
 
-Program FuseConvBatchNorm(const Program& program, const std::set<std::string>& fetch_ids) {
+namespace {
+// conv: channels-last convolution of an NCHW image; pool: its only consumer (after batch norm and relu).  True when the
+// image-convolution kernel can take the pooling along (conv_stem7_mfma.hip): 7x7 / stride 2 / padding 3 over three
+// channels in a 16-bit type, followed by max pooling 3x3 / stride 2 / padding 1 without ceil mode.
+bool StemMaxPoolFusable(const Instruction& conv, const Instruction& pool) {
+  if (GetAttr<std::string>(conv->attrs, "input_layout", "NHWC") != "NCHW") return false;
+  if (GetAttr<std::string>(pool->attrs, "data_format", "NCHW") != "NHWC") return false;
+  if (GetAttr<std::string>(pool->attrs, "pool_type", "max") != "max" || GetAttr<bool>(pool->attrs, "global_pooling", false) ||
+      GetAttr<bool>(pool->attrs, "adaptive", false) || GetAttr<bool>(pool->attrs, "ceil_mode", false))
+    return false;
+  auto ksize = GetAttr<std::vector<int>>(pool->attrs, "kernel_size", {1, 1});
+  auto pstr  = GetAttr<std::vector<int>>(pool->attrs, "stride_size", {1, 1});
+  auto ppad  = GetAttr<std::vector<int>>(pool->attrs, "padding_size", {0, 0, 0, 0});
+  if (ksize != std::vector<int>{3, 3} || pstr != std::vector<int>{2, 2}) return false;
+  for (int v : ppad)
+    if (v != 1) return false;
+  auto stride   = GetAttr<std::vector<int>>(conv->attrs, "stride", {1, 1});
+  auto padding  = GetAttr<std::vector<int>>(conv->attrs, "padding", {0, 0});
+  auto dilation = GetAttr<std::vector<int>>(conv->attrs, "dilation", {1, 1});
+  const auto& x = conv->inputs[0]->shape;  // NCHW
+  const auto& w = conv->inputs[1]->shape;  // OIHW
+  if (x.size() != 4 || w.size() != 4 || GetAttr<int>(conv->attrs, "groups", 1) != 1) return false;
+  const auto& t = conv->inputs[0]->type;
+  if (!t.is_floating()) return false;
+  return cinn_hip_kernels::StemPoolFusableShape(x[0], x[1], x[2], x[3], w[0], w[2], w[3], stride[0], stride[1], padding[0],
+                                                padding[1], dilation[0], dilation[1],
+                                                t.is_bfloat16() ? cinn_type_bfloat : cinn_type_float, t.bits);
+}
+}  // namespace
+
+Program FuseConvBatchNorm(const Program& program, const std::set<std::string>& fetch_ids, bool fuse_stem_pool) {
   const auto& instrs = program.instructions();
   // consumers of every variable
   std::map<std::string, std::vector<size_t>> users;
@@ -281,6 +313,16 @@ Program FuseConvBatchNorm(const Program& program, const std::set<std::string>& f
       dropped[next] = true;
       last          = next;
       result        = instrs[next]->outputs[0];
+      next          = single_user(result);
+    }
+    // a 3x3, stride 2, padding 1 max pooling after the image convolution's relu runs inside the convolution kernel
+    bool max_pool = false;
+    if (fuse_stem_pool && relu && !residual.defined() && next >= 0 && !dropped[next] && instrs[next]->op_type == "pool2d" &&
+        StemMaxPoolFusable(conv, instrs[next])) {
+      max_pool      = true;
+      dropped[next] = true;
+      last          = next;
+      result        = instrs[next]->outputs[0];
     }
     dropped[i]     = true;
     dropped[bn_at] = true;
@@ -302,6 +344,7 @@ Program FuseConvBatchNorm(const Program& program, const std::set<std::string>& f
     auto t     = e.Emit1("subtract", {bias, e.Emit1("elementwise_mul", {mean, s}, {{"axis", -1}})}, {{"axis", -1}});
     AttributeMap attrs = conv->attrs;
     attrs["relu"]      = relu;
+    attrs["max_pool"]  = max_pool;
     std::vector<Variable> inputs = {conv->inputs[0], conv->inputs[1], s, t};
     if (residual.defined()) inputs.push_back(residual);
     e.EmitInto(result, "hip_conv2d_bn_relu", inputs, attrs);

@@ -22,7 +22,10 @@ namespace cinn {
 namespace frontend {
 
 Program ConvertConvLayoutToNHWC(const Program& program, const std::set<std::string>& fetch_ids);
-Program FuseConvBatchNorm(const Program& program, const std::set<std::string>& fetch_ids);
+// With fuse_stem_pool, a 3x3 / stride 2 / padding 1 max pooling that follows the relu of a folded image convolution
+// (7x7 / stride 2 / padding 3 over 3 NCHW channels, 16-bit) is folded in as well (attribute max_pool): the
+// full-resolution activation then never reaches memory.
+Program FuseConvBatchNorm(const Program& program, const std::set<std::string>& fetch_ids, bool fuse_stem_pool = true);
 // matmul(x, W) with a const 2-D W stored [K][N]: multiply by a pre-run transposed copy instead (trans_b), so that
 // both operands of the GEMM kernel have K contiguous whatever the sizes of x
 Program PretransposeConstMatmulWeights(const Program& program);

@@ -1391,7 +1391,8 @@ ir::LoweredFuncRef OpLowerer::LowerLibraryCall(const Group& group) const {
     } else {
       api = "cinn_call_hip_conv2d_bn_relu";
       args.push_back(I32(format));
-      args.push_back(I32(GetAttr<bool>(n->attrs, "relu", false) ? 1 : 0));
+      // bit 0: relu; bit 1: 3x3 / stride 2 / padding 1 max pooling after it, inside the kernel
+      args.push_back(I32((GetAttr<bool>(n->attrs, "relu", false) ? 1 : 0) | (GetAttr<bool>(n->attrs, "max_pool", false) ? 2 : 0)));
     }
     // extents are always passed in n, c, h, w order
     if (nchw_input) {
@@ -1404,6 +1405,12 @@ ir::LoweredFuncRef OpLowerer::LowerLibraryCall(const Group& group) const {
     push_ints({padding[0], padding[1], stride[0], stride[1], dilation[0], dilation[1], groups});
     if (nchw) {
       push_ints({y[0], y[1], y[2], y[3]});
+    } else if (GetAttr<bool>(n->attrs, "max_pool", false)) {
+      // the output tensor is the pooled one; the intrinsic takes the convolution's own output extents
+      const int xh = nchw_input ? x[2] : x[1], xw = nchw_input ? x[3] : x[2];
+      const int kh = nchw_input ? w[2] : w[1], kw = nchw_input ? w[3] : w[2];
+      push_ints({y[0], y[3], (xh + 2 * padding[0] - ((kh - 1) * dilation[0] + 1)) / stride[0] + 1,
+                 (xw + 2 * padding[1] - ((kw - 1) * dilation[1] + 1)) / stride[1] + 1});
     } else {
       push_ints({y[0], y[3], y[1], y[2]});
     }

@@ -559,7 +559,13 @@ OpRegistry::OpRegistry() {
     const auto* cv = r->Find("conv2d");
     auto conv_shape = cv->infer_shape;
     op.infer_shape = [conv_shape](const std::vector<ShapeType>& in, const AttributeMap& a) {
-      return conv_shape({in[0], in[1]}, a);
+      auto out = conv_shape({in[0], in[1]}, a);
+      if (GetAttr<bool>(a, "max_pool", false)) {
+        // the 3x3 / stride 2 / padding 1 max pooling folded into an image convolution (channels-last output)
+        out[0][1] = (out[0][1] + 2 - 3) / 2 + 1;
+        out[0][2] = (out[0][2] + 2 - 3) / 2 + 1;
+      }
+      return out;
     };
     op.infer_dtype = SameTypeAsFirst;
   }

@@ -298,7 +298,8 @@ void RunConv(cinn_buffer_t* x, cinn_buffer_t* w, cinn_buffer_t* y, const float* 
     a.residual       = residual ? residual->memory : (epilogue == 0 && beta != 0.0f ? y->memory : nullptr);
     a.alpha          = epilogue == 0 ? alpha : 1.0f;
     a.residual_scale = residual ? 1.0f : beta;
-    a.relu           = epilogue == 2;
+    a.relu           = epilogue >= 2;
+    a.pool_after     = epilogue == 3;
     a.nchw_input     = format == 2;
     a.n = in, a.h = ih, a.w_in = iw, a.c = ic;
     a.oc = fn, a.kh = fh, a.kw = fw, a.oh = oh, a.ow = ow;
@@ -316,6 +317,7 @@ void RunConv(cinn_buffer_t* x, cinn_buffer_t* w, cinn_buffer_t* y, const float* 
     return;
   }
   CINN_RT_CHECK(residual == nullptr, "conv2d: a residual input needs the channels-last format");
+  CINN_RT_CHECK(epilogue != 3, "conv2d: a fused max pooling needs the channels-last format");
 
   ConvParams p;
   p.n = in, p.c = ic, p.ih = ih, p.iw = iw;
@@ -380,7 +382,7 @@ void cinn_call_hip_conv2d_bn_relu(void* v_args, int num_args, int format, int re
                 "cinn_call_hip_conv2d_bn_relu: scale / shift must be fp32");
   RunConv(BufferArg(v_args, 0), BufferArg(v_args, 1), BufferArg(v_args, num_args - 1),
           reinterpret_cast<const float*>(scale->memory), reinterpret_cast<const float*>(shift->memory),
-          num_args == 6 ? BufferArg(v_args, 4) : nullptr, relu ? 2 : 1, format, 1.0f, 0.0f, input_n, input_c, input_h,
+          num_args == 6 ? BufferArg(v_args, 4) : nullptr, (relu & 2) ? 3 : ((relu & 1) ? 2 : 1), format, 1.0f, 0.0f, input_n, input_c, input_h,
           input_w, filter_n, filter_c, filter_h, filter_w, pad_h, pad_w, stride_h, stride_w, dilation_h, dilation_w,
           groups, output_n, output_c, output_h, output_w, static_cast<hipStream_t>(stream));
 }

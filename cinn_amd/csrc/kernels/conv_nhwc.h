@@ -19,6 +19,9 @@ struct ConvNhwcArgs {
   float residual_scale;  // factor of the residual (beta of the alpha / beta form)
   bool relu;
   bool nchw_input;
+  // a 3x3, stride 2, padding 1 max pooling follows the epilogue inside the kernel: y is the pooled tensor, oh / ow stay
+  // the convolution's own output extents.  Only conv_stem7_mfma.hip implements it (StemPoolFusableShape says when).
+  bool pool_after = false;
   int n, h, w_in, c;  // input extents
   int oc, kh, kw;
   int oh, ow;

@@ -15,6 +15,14 @@
 //     the transposed tile, so that the epilogue runs in registers and, after an exchange between lanes (DPP row shifts
 //     by 8), every store instruction writes 8 pixels x 128 contiguous bytes;
 //   * the filter is staged once per block as [64 channels][192], rows swizzled as in conv3x3_c64_patch_kernel.
+// POOL: the 3x3, stride 2, padding 1 max pooling that follows such a convolution (after batch norm and relu) runs in
+// the same kernel, so that the full-resolution tensor (51 MB at batch 32) never reaches memory.  A tile is then five
+// convolution rows (one per computing wavefront, five of them; three wavefronts fetch), which give two pooled rows; the
+// rows are staged in LDS as 16-bit values after the epilogue, and all eight wavefronts take the maxima.  (Four
+// computing wavefronts with nine tiles of 16 pixels each were tried: the 144 accumulators leave too few registers,
+// 58 us against 38.)  One row in
+// four is computed twice (by the tile above as well).  Values are non-negative after the relu, so taps outside the
+// image count as zeros.
 #include <hip/hip_runtime.h>
 
 #include <climits>
@@ -22,6 +30,7 @@
 #include <cstdlib>
 
 #include "kernels/conv_nhwc.h"
+#include "kernels/stem_pool.h"
 #include "runtime/hip_check.h"
 
 namespace cinn_hip_kernels {
@@ -57,8 +66,8 @@ constexpr int kSlices    = 6;                  // MFMA slices of 4 segments
 constexpr int kFilterRow = kSlices * 4 * 16;   // bytes of a filter row: 24 segments of 8 halves
 constexpr int kFilterBytes = 64 * kFilterRow;
 constexpr int kTableBytes  = 2 * 64 * 4;       // scale and shift of the block's 64 channels
-constexpr int kMaxVectors  = 6;                // 16-byte vectors a fetching thread holds per tile
 constexpr int kLdsLimit    = 160 * 1024;
+constexpr int kStagePitch  = 144;              // bytes between staged pixels (POOL): 64 channels + 16
 
 struct Stem7Params {
   const uint16_t* x;  // [N][3][H][W]
@@ -78,6 +87,7 @@ struct Stem7Params {
   int patch_bytes;
   unsigned ow_magic, ow_shift;    // n / OW
   unsigned vec_magic, vec_shift;  // n / (W / 8)
+  int pool_h, pool_w;             // POOL: extents of the pooled output (y is [N][pool_h][pool_w][OC])
 };
 
 __device__ __forceinline__ int FilterKey(int r) { return ((r >> 1) & 1) * 2 + ((r >> 3) & 1) * 4 + ((r >> 2) & 1); }
@@ -96,13 +106,27 @@ __device__ __forceinline__ void BarrierLds() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-template <typename T>
-__global__ void __launch_bounds__(128 * kWaves) conv_stem7_kernel(Stem7Params p) {
+// element-wise maximum of eight 16-bit values (exact in either type)
+__device__ __forceinline__ f16x8 Max8(f16x8 a, f16x8 b) { return __builtin_elementwise_max(a, b); }
+__device__ __forceinline__ bf16x8 Max8(bf16x8 a, bf16x8 b) {
+  bf16x8 r;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) r[e] = (float)a[e] > (float)b[e] ? a[e] : b[e];
+  return r;
+}
+
+template <typename T, bool POOL>
+__global__ void __launch_bounds__(512) conv_stem7_kernel(Stem7Params p) {
+  constexpr int CW   = POOL ? 5 : kWaves;  // computing wavefronts (POOL: one per convolution row of a tile)
+  constexpr int TM   = kTMW;               // 16-pixel tiles per computing wavefront
+  constexpr int FT   = 512 - 64 * CW;      // fetching threads
+  constexpr int MAXV = POOL ? 7 : 6;       // 16-byte vectors a fetching thread holds per tile
   typedef typename Mfma16<T>::vec8 vec8;
   extern __shared__ __attribute__((aligned(16))) char lds[];
   char* const filter = lds;
   float* const table = reinterpret_cast<float*>(lds + kFilterBytes);  // [scale | shift][64]
   char* const patch0 = lds + kFilterBytes + kTableBytes;
+  char* const stage  = patch0 + 2 * p.patch_bytes;  // POOL: [5 rows][OW] pixels of kStagePitch bytes
   const int tid      = threadIdx.x;
   const int lane     = tid & 63;
   const int wave     = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -110,8 +134,8 @@ __global__ void __launch_bounds__(128 * kWaves) conv_stem7_kernel(Stem7Params p)
   const int row_vecs = p.w_in >> 3;  // 16-byte vectors per image row
 
   // ---- once per block: both patch buffers zero (the halo columns stay so), the filter slice in fragment order
-  for (int v = tid; v < (2 * p.patch_bytes) >> 4; v += 128 * kWaves) *reinterpret_cast<u32x4*>(patch0 + v * 16) = u32x4{0u, 0u, 0u, 0u};
-  for (int q = tid; q < 64 * 4 * kSlices; q += 128 * kWaves) {
+  for (int v = tid; v < (2 * p.patch_bytes) >> 4; v += 512) *reinterpret_cast<u32x4*>(patch0 + v * 16) = u32x4{0u, 0u, 0u, 0u};
+  for (int q = tid; q < 64 * 4 * kSlices; q += 512) {
     const int row = q / (4 * kSlices), seg = q - row * (4 * kSlices);
     uint16_t taps[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     if (seg < kSegments) {
@@ -128,21 +152,46 @@ __global__ void __launch_bounds__(128 * kWaves) conv_stem7_kernel(Stem7Params p)
   }
   __syncthreads();
 
-  if (wave >= kWaves) {
+  // tile t: image t / strips, strip t % strips; its first input row
+  auto first_input_row = [&](int strip) { return POOL ? 8 * strip - 5 : strip * p.rows * 2 - 3; };
+  // POOL: maxima of the staged tile - 2 pooled rows x pool_w pixels x 8 channel groups over all 512 threads
+  auto pool_tile = [&](int img, int strip) {
+    T* const Yp = reinterpret_cast<T*>(p.y);
+    const int items = 2 * p.pool_w * 8;
+    for (int it = tid; it < items; it += 512) {
+      const int grp  = it & 7, q = it >> 3;
+      const int prow = q >= p.pool_w ? 1 : 0, px = q - prow * p.pool_w;
+      const int py   = 2 * strip + prow;
+      if (py >= p.pool_h) continue;
+      vec8 best = {};
+#pragma unroll
+      for (int dy = 0; dy < 3; ++dy)
+#pragma unroll
+        for (int dx = 0; dx < 3; ++dx) {
+          const int cx = 2 * px - 1 + dx;
+          vec8 v = {};
+          if ((unsigned)cx < (unsigned)p.ow)
+            v = *reinterpret_cast<const vec8*>(stage + ((2 * prow + dy) * p.ow + cx) * kStagePitch + grp * 16);
+          best = Max8(best, v);
+        }
+      *reinterpret_cast<vec8*>(Yp + (((int64_t)img * p.pool_h + py) * p.pool_w + px) * p.oc + n0 + grp * 8) = best;
+    }
+  };
+
+  if (wave >= CW) {
     // ---- fetching wavefronts: vector v of a tile = 8 columns of one (channel, patch row)
-    const int ft      = tid - 64 * kWaves;
+    const int ft      = tid - 64 * CW;
     const int vectors = 3 * p.patch_rows * row_vecs;
-    int k = 0;
-    for (int t = blockIdx.x; t < p.tiles; t += gridDim.x, ++k) {
+    auto fetch = [&](int t, int k) {
       const int img   = t / p.strips;
-      const int iy0   = (t - img * p.strips) * p.rows * 2 - 3;
+      const int iy0   = first_input_row(t - img * p.strips);
       const uint16_t* image = p.x + (int64_t)img * 3 * p.h * p.w_in;
       char* const buf = patch0 + (k & 1) * p.patch_bytes;
-      u32x4 regs[kMaxVectors];
-      int dst[kMaxVectors];
+      u32x4 regs[MAXV];
+      int dst[MAXV];
 #pragma unroll
-      for (int e = 0; e < kMaxVectors; ++e) {
-        const int v = ft + 64 * kWaves * e;
+      for (int e = 0; e < MAXV; ++e) {
+        const int v = ft + FT * e;
         dst[e]      = -1;
         regs[e]     = u32x4{0u, 0u, 0u, 0u};
         if (v < vectors) {
@@ -156,25 +205,45 @@ __global__ void __launch_bounds__(128 * kWaves) conv_stem7_kernel(Stem7Params p)
         }
       }
 #pragma unroll
-      for (int e = 0; e < kMaxVectors; ++e)
+      for (int e = 0; e < MAXV; ++e)
         if (dst[e] >= 0) *reinterpret_cast<u32x4*>(buf + dst[e]) = regs[e];
-      BarrierLds();  // tile k is in its buffer; the other buffer's tile (k - 1) has been multiplied
+    };
+    int k = 0;
+    if (POOL) {
+      // tile k + 1 is fetched while tile k is multiplied; then these wavefronts help with tile k's maxima
+      if ((int)blockIdx.x < p.tiles) fetch(blockIdx.x, 0);
+      for (int t = blockIdx.x; t < p.tiles; t += gridDim.x, ++k) {
+        BarrierLds();  // tile k is in its buffer; the staged tile k - 1 has been pooled
+        if (t + (int)gridDim.x < p.tiles) fetch(t + gridDim.x, k + 1);
+        BarrierLds();  // tile k's convolution rows are staged
+        pool_tile(t / p.strips, t % p.strips);
+      }
+    } else {
+      for (int t = blockIdx.x; t < p.tiles; t += gridDim.x, ++k) {
+        fetch(t, k);
+        BarrierLds();  // tile k is in its buffer; the other buffer's tile (k - 1) has been multiplied
+      }
     }
     return;
   }
 
   // ---- computing wavefronts
   const int kgc  = ((lane >> 4) & 1) * 2 + (lane >> 5);  // k chunk of this lane group: 0, 2, 1, 3
-  const int pix0 = wave * (kTMW * 16) + (lane & 15);
   // byte offset of the window's first column (2 ox - 4, patch column 2 ox + 4) in the patch row of the window's first
   // input row (2 ly), per tile; pixels beyond the tile read offset 0, their results are not stored
-  int a_pix[kTMW];
+  const int pix0 = wave * (TM * 16) + (lane & 15);
+  int a_pix[TM];
 #pragma unroll
-  for (int i = 0; i < kTMW; ++i) {
-    const int pix = pix0 + 16 * i;
-    const int ly  = (int)(((uint64_t)(unsigned)pix * p.ow_magic) >> p.ow_shift);
-    const int ox  = pix - ly * p.ow;
-    a_pix[i]      = ly < p.rows ? 2 * ly * p.pitch + (2 * ox + 4) * 2 : 0;
+  for (int i = 0; i < TM; ++i) {
+    if (POOL) {  // wavefront w multiplies convolution row w of the tile
+      const int ox = 16 * i + (lane & 15);
+      a_pix[i]     = ox < p.ow ? 2 * wave * p.pitch + (2 * ox + 4) * 2 : 0;
+    } else {
+      const int pix = pix0 + 16 * i;
+      const int ly  = (int)(((uint64_t)(unsigned)pix * p.ow_magic) >> p.ow_shift);
+      const int ox  = pix - ly * p.ow;
+      a_pix[i]      = ly < p.rows ? 2 * ly * p.pitch + (2 * ox + 4) * 2 : 0;
+    }
   }
   // segment 4 s + kgc = (channel, dy) of slice s; the padding segments 21..23 read segment 0 and are cleared
   int seg_off[kSlices];
@@ -213,21 +282,18 @@ __global__ void __launch_bounds__(128 * kWaves) conv_stem7_kernel(Stem7Params p)
     const char* const buf = patch0 + (k & 1) * p.patch_bytes;
     BarrierLds();  // tile k is in its buffer
 
-    f32x4 acc[kTMW][4];
+    f32x4 acc[TM][4];
 #pragma unroll
-    for (int i = 0; i < kTMW; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    // 42 rows of 4 MFMAs: row 7 s + i multiplies the pixel fragment of tile i, slice s, with the slice's four filter
-    // fragments.  Pixel fragments are requested three rows ahead into one register set per tile, the next slice's
+    // 6 TM rows of 4 MFMAs: row TM s + i multiplies the pixel fragment of tile i, slice s, with the slice's four filter
+    // fragments.  Pixel fragments are requested three rows ahead into a ring of four register sets, the next slice's
     // filter fragments during rows 0 and 1 of a slice; scheduling barriers pin that order.
-    // the raw dwords of a fragment are requested early and patched when the row that uses them starts: slot 0 (the
-    // column left of the window) is cleared, and so are the padding segments of the last slice
-    const char* a_tile[kTMW];
-#pragma unroll
-    for (int i = 0; i < kTMW; ++i) a_tile[i] = buf + a_pix[i];
+    // The raw dwords of a fragment are requested early and patched when the row that uses them starts: slot 0 (the
+    // column left of the window) is cleared, and so are the padding segments of the last slice.
     auto read_a = [&](int s, int i) -> u32x4 {
-      const uint32_t* src = reinterpret_cast<const uint32_t*>(a_tile[i] + seg_off[s]);
+      const uint32_t* src = reinterpret_cast<const uint32_t*>(buf + (a_pix[i] + seg_off[s]));
       u32x4 d;
 #pragma unroll
       for (int e = 0; e < 4; ++e) d[e] = src[e];
@@ -242,7 +308,7 @@ __global__ void __launch_bounds__(128 * kWaves) conv_stem7_kernel(Stem7Params p)
       return __builtin_bit_cast(vec8, d);
     };
     auto read_b = [&](int s, int j) -> vec8 { return *reinterpret_cast<const vec8*>(b_base[s & 1][j] + (s >> 1) * 128); };
-    u32x4 ar[kTMW];
+    u32x4 ar[4];
     vec8 bf[2][4];
 #pragma unroll
     for (int r = 0; r < 3; ++r) ar[r] = read_a(0, r);
@@ -252,16 +318,16 @@ __global__ void __launch_bounds__(128 * kWaves) conv_stem7_kernel(Stem7Params p)
 #pragma unroll
     for (int s = 0; s < kSlices; ++s) {
 #pragma unroll
-      for (int i = 0; i < kTMW; ++i) {
+      for (int i = 0; i < TM; ++i) {
         CINN_SB;
-        const vec8 af = patched(s, ar[i]);
+        const vec8 af = patched(s, ar[(TM * s + i) % 4]);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           CINN_SB;
           acc[i][j] = Mfma16<T>::mma(bf[s & 1][j], af, acc[i][j]);
           CINN_SB;
-          const int rr = kTMW * s + i + 3;
-          if (j == 0 && rr < kTMW * kSlices) ar[rr % kTMW] = read_a(rr / kTMW, rr % kTMW);
+          const int rr = TM * s + i + 3;
+          if (j == 0 && rr < TM * kSlices) ar[rr % 4] = read_a(rr / TM, rr % TM);
           if ((j == 1 || j == 2) && i < 2 && s + 1 < kSlices) bf[(s + 1) & 1][i * 2 + j - 1] = read_b(s + 1, i * 2 + j - 1);
         }
       }
@@ -279,8 +345,33 @@ __global__ void __launch_bounds__(128 * kWaves) conv_stem7_kernel(Stem7Params p)
         sc[s][e] = table[8 * g + 32 * s + e];
         sh[s][e] = table[64 + 8 * g + 32 * s + e];
       }
+    if (POOL) {
+      // this wavefront's convolution row, after scale, shift and relu, into the staging tile (zeros for a row outside
+      // the image); then the maxima
+      const int strip  = t - img * p.strips;
+      const bool valid = (unsigned)(4 * strip - 1 + wave) < (unsigned)p.oh;  // this wavefront's row exists
 #pragma unroll
-    for (int i = 0; i < kTMW; ++i) {
+      for (int i = 0; i < TM; ++i) {
+        const int ox = 16 * i + px;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+          vec8 o8;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            float v = __builtin_fmaf(acc[i][2 * s + (e >> 2)][e & 3], sc[s][e], sh[s][e]);
+            asm volatile("" : "+v"(v));
+            v     = valid && v > 0.0f ? v : 0.0f;
+            o8[e] = (T)v;
+          }
+          if (ox < p.ow) *reinterpret_cast<vec8*>(stage + (wave * p.ow + ox) * kStagePitch + (g + 4 * s) * 16) = o8;
+        }
+      }
+      BarrierLds();  // the five rows are staged
+      pool_tile(img, strip);
+      continue;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
       const int pix = pix0 + 16 * i;
       vec8 res[2] = {};
       if (R && pix < npix) {
@@ -338,24 +429,36 @@ bool FillParams(const ConvNhwcArgs& a, Stem7Params* out) {
       a.dil_h != 1 || a.dil_w != 1)
     return false;
   if (a.oc % 64 != 0 || a.w_in % 8 != 0 || a.ow > kCapacity) return false;
+  if (a.pool_after && (!a.relu || a.residual || a.ow > kTMW * 16)) return false;
   if (a.oh != (a.h + 6 - 7) / 2 + 1 || a.ow != (a.w_in + 6 - 7) / 2 + 1) return false;
   if ((int64_t)a.n * 3 * a.h * a.w_in >= INT_MAX || (int64_t)a.n * a.oh * a.ow * a.oc >= INT_MAX) return false;
   if (reinterpret_cast<uintptr_t>(a.x) % 16 != 0 || reinterpret_cast<uintptr_t>(a.y) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(a.residual) % 16 != 0)
     return false;
   Stem7Params p;
-  int rows = kCapacity / a.ow;
-  rows     = rows < a.oh ? rows : a.oh;
-  p.strips = (a.oh + rows - 1) / rows;
-  rows     = (a.oh + p.strips - 1) / p.strips;
-  if ((int64_t)a.oh * a.ow * 5 < (int64_t)p.strips * kCapacity * 4) return false;  // mostly empty tiles
+  p.pool_h = p.pool_w = 0;
+  int rows;
+  if (a.pool_after) {
+    // 3x3, stride 2, padding 1 pooling: a tile is 5 convolution rows -> 2 pooled rows
+    p.pool_h = (a.oh + 2 - 3) / 2 + 1;
+    p.pool_w = (a.ow + 2 - 3) / 2 + 1;
+    rows     = 5;
+    p.strips = (p.pool_h + 1) / 2;
+  } else {
+    rows     = kCapacity / a.ow;
+    rows     = rows < a.oh ? rows : a.oh;
+    p.strips = (a.oh + rows - 1) / rows;
+    rows     = (a.oh + p.strips - 1) / p.strips;
+    if ((int64_t)a.oh * a.ow * 5 < (int64_t)p.strips * kCapacity * 4) return false;  // mostly empty tiles
+  }
   p.rows       = rows;
   p.tiles      = a.n * p.strips;
   p.patch_rows = 2 * (rows - 1) + 7;
   p.pitch      = ((a.w_in + 16) * 2 + 255 - 64) / 256 * 256 + 64;
   p.patch_bytes = 3 * p.patch_rows * p.pitch;
-  if (kFilterBytes + kTableBytes + 2 * p.patch_bytes > kLdsLimit) return false;
-  if (3 * p.patch_rows * (a.w_in / 8) > kMaxVectors * 64 * kWaves) return false;
+  const int stage_bytes = a.pool_after ? 5 * a.ow * kStagePitch : 0;
+  if (kFilterBytes + kTableBytes + 2 * p.patch_bytes + stage_bytes > kLdsLimit) return false;
+  if (3 * p.patch_rows * (a.w_in / 8) > (a.pool_after ? 7 * 192 : 6 * 256)) return false;
   p.x = static_cast<const uint16_t*>(a.x), p.w = static_cast<const uint16_t*>(a.w), p.y = static_cast<uint16_t*>(a.y);
   p.scale = a.scale, p.shift = a.shift, p.residual = static_cast<const uint16_t*>(a.residual);
   p.alpha = a.alpha, p.residual_scale = a.residual_scale, p.relu = a.relu ? 1 : 0;
@@ -366,9 +469,9 @@ bool FillParams(const ConvNhwcArgs& a, Stem7Params* out) {
   return true;
 }
 
-template <typename T>
+template <typename T, bool POOL>
 void Launch(const Stem7Params& p, hipStream_t stream) {
-  auto kernel = conv_stem7_kernel<T>;
+  auto kernel = conv_stem7_kernel<T, POOL>;
   static const bool configured = [&] {  // once per instantiation, thread-safe
     CINN_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
     return true;
@@ -377,20 +480,43 @@ void Launch(const Stem7Params& p, hipStream_t stream) {
   // persistent blocks: one per CU (its eight wavefronts use the register file of a CU's four SIMDs two by two)
   const int per_group = 256 / (p.oc / 64) > 0 ? 256 / (p.oc / 64) : 1;
   dim3 grid(p.tiles < per_group ? p.tiles : per_group, p.oc / 64);
-  hipLaunchKernelGGL(kernel, grid, dim3(128 * kWaves), kFilterBytes + kTableBytes + 2 * p.patch_bytes, stream, p);
+  const int stage_bytes = POOL ? 5 * p.ow * kStagePitch : 0;
+  hipLaunchKernelGGL(kernel, grid, dim3(512), kFilterBytes + kTableBytes + 2 * p.patch_bytes + stage_bytes, stream, p);
 }
 
 }  // namespace
 
-bool TryConvStem7(const ConvNhwcArgs& a, hipStream_t stream) {
+namespace {
+bool Stem7Enabled() {
   static const bool enabled = !(getenv("FLAGS_cinn_hip_conv_stem7") && atoi(getenv("FLAGS_cinn_hip_conv_stem7")) == 0);
-  if (!enabled) return false;
+  return enabled;
+}
+}  // namespace
+
+bool StemPoolFusableShape(int n, int c, int h, int w, int oc, int kh, int kw, int stride_h, int stride_w, int pad_h,
+                          int pad_w, int dil_h, int dil_w, int type_code, int type_bits) {
+  if (!Stem7Enabled() || stride_h < 1 || stride_w < 1) return false;
+  ConvNhwcArgs a{};
+  a.nchw_input = true, a.relu = true, a.pool_after = true;
+  a.n = n, a.c = c, a.h = h, a.w_in = w, a.oc = oc, a.kh = kh, a.kw = kw;
+  a.pad_h = pad_h, a.pad_w = pad_w, a.stride_h = stride_h, a.stride_w = stride_w, a.dil_h = dil_h, a.dil_w = dil_w;
+  a.oh = (h + 2 * pad_h - ((kh - 1) * dil_h + 1)) / stride_h + 1;
+  a.ow = (w + 2 * pad_w - ((kw - 1) * dil_w + 1)) / stride_w + 1;
+  a.type.code  = static_cast<cinn_type_code_t>(type_code);
+  a.type.bits  = static_cast<uint8_t>(type_bits);
+  a.type.lanes = 1;
+  Stem7Params p;
+  return FillParams(a, &p);
+}
+
+bool TryConvStem7(const ConvNhwcArgs& a, hipStream_t stream) {
+  if (!Stem7Enabled()) return false;
   Stem7Params p;
   if (!FillParams(a, &p)) return false;
   if (a.type.code == cinn_type_bfloat) {
-    Launch<__bf16>(p, stream);
+    a.pool_after ? Launch<__bf16, true>(p, stream) : Launch<__bf16, false>(p, stream);
   } else {
-    Launch<_Float16>(p, stream);
+    a.pool_after ? Launch<_Float16, true>(p, stream) : Launch<_Float16, false>(p, stream);
   }
   CINN_HIP_CALL(hipGetLastError());
   return true;

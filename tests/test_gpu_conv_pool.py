@@ -625,42 +625,48 @@ def test_image_convolution_7x7_stride2(gpu, case, dtype, tol):
         assert not bad[:, 20].any() and bad[10, 19] and bad[10, 17] and not bad[10, 16]
 
 
-def test_image_convolution_7x7_with_folded_epilogue(gpu):
-    """batch norm + relu folded into the image convolution, through NetBuilder (scale / shift table in LDS)."""
-    rng = np.random.default_rng(29)
-    x = rng.standard_normal((2, 3, 224, 224)).astype(np.float16)
-    w = (rng.standard_normal((64, 3, 7, 7)) * np.sqrt(2.0 / 147)).astype(np.float16)
-    scale, bias = rng.uniform(0.5, 1.5, 64).astype(np.float16), rng.standard_normal(64).astype(np.float16)
-    mean, var = (rng.standard_normal(64) * 0.1).astype(np.float16), rng.uniform(0.5, 1.5, 64).astype(np.float16)
-    b = NetBuilder("stem7")
-    X = b.create_input(Float(16), x.shape, "x")
-    W = b.create_input(Float(16), w.shape, "w").set_const()
-    P = [b.create_input(Float(16), [64], nm).set_const() for nm in ("scale", "bias", "mean", "var")]
-    y = b.pool2d(b.relu(b.batchnorm(b.conv2d(X, W, strides=[2, 2], paddings=[3, 3]), *P)[0]), "max", [3, 3], [2, 2],
-                 [1, 1, 1, 1])
-    (got,), comp = run(b, {X: x, W: w, P[0]: scale, P[1]: bias, P[2]: mean, P[3]: var}, [y])
-    conv = oracle.conv2d_nchw(x.astype(np.float32), w.astype(np.float32), (2, 2), (3, 3))
-    act = oracle.batch_norm_relu_nchw(conv, scale.astype(np.float32), bias.astype(np.float32), mean.astype(np.float32),
-                                      var.astype(np.float32), 1e-5, relu=True)
-    want = oracle.pool2d_nchw(act.astype(np.float16), (3, 3), (2, 2), (1, 1, 1, 1), "max")
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("shape", [(2, 224, 224), (3, 108, 88), (9, 224, 224)])
+def test_image_convolution_7x7_with_folded_epilogue_and_max_pooling(gpu, dtype, shape):
+    """conv -> batch norm -> relu -> 3x3 max pooling as one kernel (scale / shift table and the staged convolution rows
+    in LDS): against the oracle, and bit for bit against the unfused pair of kernels (the maximum of rounded values is
+    exact).  108 rows give 27 pooled rows: the last tile holds one; 9 images give 252 + tiles on 256 blocks."""
+    from cinn_amd.common import BFloat16
+    n, h, w_ = shape
+    rng = np.random.default_rng(29 + n)
+    x = round_to(rng.standard_normal((n, 3, h, w_)), dtype)
+    w = round_to(rng.standard_normal((64, 3, 7, 7)) * np.sqrt(2.0 / 147), dtype)
+    scale, bias = round_to(rng.uniform(0.5, 1.5, 64), dtype), round_to(rng.standard_normal(64), dtype)
+    mean, var = round_to(rng.standard_normal(64) * 0.1, dtype), round_to(rng.uniform(0.5, 1.5, 64), dtype)
+    ty = Float(16) if dtype == "float16" else BFloat16()
+
+    def build(**options):
+        b = NetBuilder("stem7")
+        X = b.create_input(ty, x.shape, "x")
+        W = b.create_input(ty, w.shape, "w").set_const()
+        P = [b.create_input(ty, [64], nm).set_const() for nm in ("scale", "bias", "mean", "var")]
+        y = b.pool2d(b.relu(b.batchnorm(b.conv2d(X, W, strides=[2, 2], paddings=[3, 3]), *P)[0]), "max", [3, 3], [2, 2],
+                     [1, 1, 1, 1])
+        feeds = {X: x, W: w, P[0]: scale, P[1]: bias, P[2]: mean, P[3]: var}
+        if dtype == "bfloat16":
+            from cinn_amd.common import float32_to_bfloat16_bits
+            feeds = {k: float32_to_bfloat16_bits(v.astype(np.float32)) for k, v in feeds.items()}
+        else:
+            feeds = {k: v.astype(np.float16) for k, v in feeds.items()}
+        (got,), comp = run(b, feeds, [y], **options)
+        if dtype == "bfloat16":
+            from cinn_amd.common import bfloat16_bits_to_float32
+            got = bfloat16_bits_to_float32(got)
+        return got.astype(np.float32), comp
+
+    fused, comp = build()
+    assert comp.num_instructions() == 2, comp.fusion_groups()  # the convolution, the transpose back to NCHW
+    apart, comp2 = build(fuse_stem_pool=0)
+    assert comp2.num_instructions() == 3
+    assert np.array_equal(fused, apart)
+    conv = oracle.conv2d_nchw(x, w, (2, 2), (3, 3))
+    act = oracle.batch_norm_relu_nchw(conv, scale, bias, mean, var, 1e-5, relu=True)
+    want = oracle.pool2d_nchw(round_to(act, dtype), (3, 3), (2, 2), (1, 1, 1, 1), "max")
+    tol = 1e-2 if dtype == "float16" else 2e-2
     # relative to the value or, where the convolution's terms cancel, to a twentieth of the activations' unit scale
-    assert np.all(np.abs(got.astype(np.float64) - want) <= 1e-2 * np.maximum(np.abs(want), 0.05))
-
-
-@pytest.mark.parametrize("dtype,tol", [("float16", 1e-2), ("bfloat16", 2e-2)])
-@pytest.mark.parametrize("case", [(32, 512, 7, 7, 512), (20, 256, 9, 9, 384)])
-def test_implicit_gemm_convolution_with_split_reduction(gpu, case, dtype, tol):
-    """Few 128x128 tiles and a long reduction (the 3x3 layers of the last ResNet stage): K is split over the grid's
-    third dimension, fp32 partial sums are added by a second kernel, which also applies alpha / beta."""
-    n, ic, h, w_, oc = case
-    rng = np.random.default_rng(sum(case) + 1)
-    x = round_to(rng.standard_normal((n, ic, h, w_)), dtype)
-    w = round_to(rng.standard_normal((oc, ic, 3, 3)) * np.sqrt(2.0 / (ic * 9)), dtype)
-    y0 = round_to(rng.standard_normal((n, oc, h, w_)), dtype)
-    want = oracle.conv2d_nchw(x, w, (1, 1), (1, 1)).astype(np.float64)
-    scale = oracle.conv2d_nchw(np.abs(x), np.abs(w), (1, 1), (1, 1))
-    got = call_conv_nhwc(x, w, 1, 1, 1, dtype)
-    assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
-    got = call_conv_nhwc(x, w, 1, 1, 1, dtype, alpha=0.5, beta=2.0, y_init=y0)
-    want2 = 0.5 * want + 2.0 * y0
-    assert np.all(np.abs(got - want2) <= tol * np.maximum(np.abs(want2), 1e-2 * (0.5 * scale + 2.0 * np.abs(y0))) + 1e-6)
+    assert np.all(np.abs(fused.astype(np.float64) - want) <= tol * np.maximum(np.abs(want), 0.05))

@@ -81,9 +81,13 @@ def test_resnet50_fp16_batch2_matches_oracle(gpu):
     # one within 1e-2 of a tenth of the logit scale (a sum of O(scale) terms cannot be resolved below that in halves)
     assert_logits_close_fp16(got, want)
     fused, comp = gpu_forward(params, x, fuse_conv_bn_relu=True)
-    # every batch norm, residual addition and relu now lives in a convolution epilogue
-    assert comp.num_instructions() == 53 + 2 + 3, comp.fusion_groups()
+    # every batch norm, residual addition and relu now lives in a convolution epilogue, and the max pooling in the
+    # image convolution: 53 convolutions, the global pooling, reshape + classifier + bias
+    assert comp.num_instructions() == 53 + 1 + 3, comp.fusion_groups()
     assert_logits_close_fp16(fused, want)
+    apart, comp = gpu_forward(params, x, fuse_stem_pool=False)
+    assert comp.num_instructions() == 53 + 2 + 3
+    assert np.array_equal(apart, fused)
 
 
 def torch_forward(params, x):
