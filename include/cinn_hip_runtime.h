@@ -164,7 +164,11 @@ void cinn_call_cudnn_conv2d_forward(void* v_args, int num_args, int format, floa
  * applied in the kernel epilogue on the fp32 accumulators, so an inference batch_norm (+ shortcut
  * + relu) that follows a convolution costs no extra pass over HBM.
  * v_args = {x, w, scale, shift, y} or {x, w, scale, shift, residual, y}; scale / shift are fp32
- * [output_c]; residual has y's shape, type and layout and needs format 1 or 2. */
+ * [output_c]; residual has y's shape, type and layout and needs format 1 or 2.
+ * relu: bit 0 = ReLU; bit 1 = a 3x3 / stride 2 / padding 1 max pooling follows the ReLU inside the kernel: y is then
+ * the pooled tensor [n][(output_h - 1) / 2 + 1][(output_w - 1) / 2 + 1][output_c] while output_h / output_w stay the
+ * convolution's own extents.  Bit 1 needs bit 0, format 2, no residual and the 7x7 / stride 2 / padding 3 convolution
+ * of a 3-channel image in a 16-bit type (anything else aborts with a message); the graph rewrite sets it only then. */
 void cinn_call_hip_conv2d_bn_relu(void* v_args, int num_args, int format, int relu, int input_n, int input_c,
                                   int input_h, int input_w, int filter_n, int filter_c, int filter_h, int filter_w,
                                   int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,

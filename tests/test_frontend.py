@@ -309,3 +309,30 @@ def test_conv_with_a_ragged_channel_count_reads_nchw_even_when_a_channels_last_t
         assert ins[1] == filt and not ins[0].startswith("nhwc_"), g
         if image:
             assert ins[0] == image, g
+
+
+def _image_stem(dtype, h=224, w=224, oc=64, k=7, stride=2, pad=3, pool=("max", [3, 3], [2, 2], [1, 1, 1, 1])):
+    b = NetBuilder("stem")
+    X = b.create_input(dtype, [4, 3, h, w], "image")
+    W = b.create_input(dtype, [oc, 3, k, k], "w").set_const()
+    P = [b.create_input(dtype, [oc], nm).set_const() for nm in ("scale", "bias", "mean", "var")]
+    y = b.relu(b.batchnorm(b.conv2d(X, W, strides=[stride, stride], paddings=[pad, pad]), *P)[0])
+    return b, b.pool2d(y, pool[0], pool[1], pool[2], pool[3])
+
+
+def test_max_pooling_after_the_image_convolution_is_folded_into_it():
+    """conv 7x7 / 2 -> batch norm -> relu -> max pool 3x3 / 2 on a 16-bit image becomes one library call whose output
+    is the pooled tensor; other pooling windows, fp32 and the option fuse_stem_pool=0 keep the pooling kernel."""
+    b, y = _image_stem(Float(16))
+    comp = compile_only(b, [y])
+    run = [g for g in comp.fusion_groups().splitlines() if " pre_run " not in g and g.strip()]
+    assert comp.num_instructions() == 2 and "pool2d" not in " ".join(run), run  # convolution, transpose back to NCHW
+    assert comp.get_tensor(str(y)).shape() == [4, 64, 56, 56]
+    for kwargs, opts in (({}, {"fuse_stem_pool": 0}), ({"pool": ("max", [2, 2], [2, 2], [0, 0, 0, 0])}, {}),
+                         ({"pool": ("avg", [3, 3], [2, 2], [1, 1, 1, 1])}, {}), ({"k": 5, "pad": 2}, {}),
+                         ({"w": 220}, {})):
+        b, y = _image_stem(Float(16), **kwargs)
+        groups = compile_only(b, [y], **opts).fusion_groups()
+        assert "pool2d" in groups, (kwargs, opts)
+    b, y = _image_stem(Float(32))
+    assert "pool2d" in compile_only(b, [y]).fusion_groups()
