@@ -20,11 +20,11 @@ from bench_timing import sustained_ms  # noqa: E402
 PEAK_TFLOPS = {"bfloat16": 2500.0, "float16": 2500.0, "float32": 157.3}
 
 
-def _time_gemm(lib, runtime, stream, dtype, m, n, k):
+def _time_gemm(lib, runtime, stream, dtype, m, n, k, b_stored_nk=False):
     from cinn_amd.common import float32_to_bfloat16_bits
     rng = np.random.default_rng(3000)
     a = (rng.standard_normal((m, k)) * 0.02).astype(np.float32)
-    b = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+    b = (rng.standard_normal((n, k) if b_stored_nk else (k, n)) * 0.02).astype(np.float32)
     if dtype == "float16":
         a, b = a.astype(np.float16), b.astype(np.float16)
     elif dtype == "bfloat16":
@@ -34,7 +34,10 @@ def _time_gemm(lib, runtime, stream, dtype, m, n, k):
     args = runtime.pod_args([A, B, C])
 
     def launch(_i=0):
-        lib.cinn_call_cublas(args, 3, False, False, False, 1.0, 0.0, 1, 1, m, k, 1, 1, k, n, stream.handle)
+        if b_stored_nk:  # trans_b: what a const weight becomes once the program pass has transposed it ahead of time
+            lib.cinn_call_cublas(args, 3, False, True, False, 1.0, 0.0, 1, 1, m, k, 1, 1, n, k, stream.handle)
+        else:
+            lib.cinn_call_cublas(args, 3, False, False, False, 1.0, 0.0, 1, 1, m, k, 1, 1, k, n, stream.handle)
 
     # the short loop first, from idle
     for _ in range(5):
@@ -64,6 +67,7 @@ def measure(stream, runtime):
     out = {}
     out["config2_matmul_bf16_4096"] = _time_gemm(lib, runtime, stream, "bfloat16", 4096, 4096, 4096)
     out["config2_matmul_fp16_4096"] = _time_gemm(lib, runtime, stream, "float16", 4096, 4096, 4096)
+    out["matmul_bf16_4096_b_stored_nk"] = _time_gemm(lib, runtime, stream, "bfloat16", 4096, 4096, 4096, b_stored_nk=True)
     out["config2_matmul_fp32_1024"] = _time_gemm(lib, runtime, stream, "float32", 1024, 1024, 1024)
     return out
 
