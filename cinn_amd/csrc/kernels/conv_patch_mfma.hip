@@ -34,32 +34,13 @@
 #include <cstdlib>
 
 #include "kernels/conv_nhwc.h"
+#include "kernels/mfma_tile.h"
 #include "runtime/hip_check.h"
 
 namespace cinn_hip_kernels {
 namespace {
 
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-
-template <typename T>
-struct Mfma16;
-template <>
-struct Mfma16<__bf16> {
-  typedef bf16x8 vec8;
-  static __device__ __forceinline__ f32x4 mma(vec8 a, vec8 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
-  }
-};
-template <>
-struct Mfma16<_Float16> {
-  typedef f16x8 vec8;
-  static __device__ __forceinline__ f32x4 mma(vec8 a, vec8 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
-  }
-};
+using namespace tile;
 
 constexpr int kTMW      = 7;            // 16-pixel tiles per computing wavefront
 constexpr int kWaves    = 4;            // computing wavefronts (as many feeding ones)
@@ -87,21 +68,6 @@ struct PatchParams {
   unsigned w_magic, w_shift;    // n / W == (n * w_magic) >> w_shift
   unsigned pw_magic, pw_shift;  // the same for W + 2
 };
-
-// 16 bytes per lane from global memory straight into LDS at lds_addr_uniform + 16 * lane.  Inline assembly, so that
-// the compiler does not track the load (tracked, every later LDS read would wait for vmcnt(0)).
-__device__ __forceinline__ void AsyncCopy16(const void* src, unsigned lds_addr_uniform) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr_uniform), "v"(src) : "memory");
-}
-
-// swizzle key of filter-stage row r (see the file comment)
-__device__ __forceinline__ int FilterKey(int r) { return ((r >> 1) & 1) * 2 + ((r >> 3) & 1) * 4 + ((r >> 2) & 1); }
-
-// the value lane (l & 15) - 8 (SHR) or + 8 of the same row of 16 lanes holds; 0 where that lane does not exist
-template <bool SHR>
-__device__ __forceinline__ unsigned RowShift8(unsigned v) {
-  return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, SHR ? 0x118 : 0x108, 0xf, 0xf, true);
-}
 
 // vmcnt(n): at most n of the wavefront's loads still in flight (they complete in issue order); lgkmcnt / expcnt open
 #define CINN_VMCNT(n) ((((n) & 15) | (((n) >> 4) << 14)) | 0x0F70)
@@ -331,18 +297,6 @@ __global__ void __launch_bounds__(128 * kWaves) conv3x3_c64_patch_kernel(PatchPa
   }
 }
 #undef CINN_VMCNT
-
-// q = (n * magic) >> shift == n / d for 0 <= n < 2^31
-void MagicFor(int d, unsigned* magic, unsigned* shift) {
-  int l = 0;
-  while ((1ll << l) < d) ++l;
-  *shift = 31 + l;
-  *magic = (unsigned)(((1ull << *shift) / (unsigned)d) + 1);
-  if (d == 1) {
-    *shift = 0;
-    *magic = 1;
-  }
-}
 
 struct PatchPlan {
   int rows, bands, patch_loads, lds_bytes;

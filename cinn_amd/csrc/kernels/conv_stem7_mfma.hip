@@ -30,33 +30,14 @@
 #include <cstdlib>
 
 #include "kernels/conv_nhwc.h"
+#include "kernels/mfma_tile.h"
 #include "kernels/stem_pool.h"
 #include "runtime/hip_check.h"
 
 namespace cinn_hip_kernels {
 namespace {
 
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-
-template <typename T>
-struct Mfma16;
-template <>
-struct Mfma16<__bf16> {
-  typedef bf16x8 vec8;
-  static __device__ __forceinline__ f32x4 mma(vec8 a, vec8 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
-  }
-};
-template <>
-struct Mfma16<_Float16> {
-  typedef f16x8 vec8;
-  static __device__ __forceinline__ f32x4 mma(vec8 a, vec8 b, f32x4 c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
-  }
-};
+using namespace tile;
 
 constexpr int kTMW       = 7;                  // 16-pixel tiles per computing wavefront
 constexpr int kWaves     = 4;                  // computing wavefronts (as many fetching ones)
@@ -89,22 +70,6 @@ struct Stem7Params {
   unsigned vec_magic, vec_shift;  // n / (W / 8)
   int pool_h, pool_w;             // POOL: extents of the pooled output (y is [N][pool_h][pool_w][OC])
 };
-
-__device__ __forceinline__ int FilterKey(int r) { return ((r >> 1) & 1) * 2 + ((r >> 3) & 1) * 4 + ((r >> 2) & 1); }
-
-template <bool SHR>
-__device__ __forceinline__ unsigned RowShift8(unsigned v) {
-  return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, SHR ? 0x118 : 0x108, 0xf, 0xf, true);
-}
-
-// Block barrier that orders LDS accesses only.  __syncthreads() also waits until every global store of the wavefront
-// has completed (its release covers global memory); here that would stall the computing wavefronts at every tile until
-// the tile's 57 KB of results have left, instead of letting them drain under the next tile's MFMAs.
-__device__ __forceinline__ void BarrierLds() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-  __builtin_amdgcn_s_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
 
 // element-wise maximum of eight 16-bit values (exact in either type)
 __device__ __forceinline__ f16x8 Max8(f16x8 a, f16x8 b) { return __builtin_elementwise_max(a, b); }
@@ -406,18 +371,6 @@ __global__ void __launch_bounds__(512) conv_stem7_kernel(Stem7Params p) {
       if (p_first < npix) *reinterpret_cast<u32x4*>(Y + (out_row0 + p_first) * p.oc + n0 + 8 * st_chunk) = first;
       if (p_second < npix) *reinterpret_cast<u32x4*>(Y + (out_row0 + p_second) * p.oc + n0 + 8 * st_chunk) = second;
     }
-  }
-}
-
-// q = (n * magic) >> shift == n / d for 0 <= n < 2^31
-void MagicFor(int d, unsigned* magic, unsigned* shift) {
-  int l = 0;
-  while ((1ll << l) < d) ++l;
-  *shift = 31 + l;
-  *magic = (unsigned)(((1ull << *shift) / (unsigned)d) + 1);
-  if (d == 1) {
-    *shift = 0;
-    *magic = 1;
   }
 }
 
