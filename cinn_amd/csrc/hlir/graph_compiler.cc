@@ -24,7 +24,17 @@ namespace framework {
 _Tensor_::_Tensor_() { cinn_hip_buffer_init(&buffer_, nullptr, cinn_type_float, 32, nullptr, 0); }
 _Tensor_::~_Tensor_() { Free(); }
 
+void _Tensor_::ShareBufferWith(const std::shared_ptr<_Tensor_>& source) {
+  CINN_CHECK(source && source.get() != this) << "a tensor cannot be a view of itself";
+  Free();
+  source_ = source;
+}
+
 void _Tensor_::Free() {
+  if (source_) {  // a view owns nothing
+    buffer_.memory = nullptr;
+    return;
+  }
   if (buffer_.memory) {
     cinn_hip_free(buffer_.memory);
     buffer_.memory = nullptr;
@@ -42,6 +52,16 @@ void _Tensor_::set_type(const common::Type& t) { type_ = t; }
 void* _Tensor_::mutable_data(const common::Target& target) {
   CINN_CHECK(target.arch == common::Target::Arch::AMDGPU) << "device tensors need the AMDGPU target";
   size_t need = bytes();
+  if (source_) {
+    CINN_CHECK_EQ(need, source_->bytes()) << "a view must cover exactly its source's bytes";
+    void* p = source_->mutable_data(target);
+    if (buffer_.memory != p) {
+      int code = type_.is_bool() ? cinn_type_int : (type_.is_bfloat16() ? cinn_type_bfloat : static_cast<int>(type_.code));
+      cinn_hip_buffer_init(&buffer_, p, code, type_.is_bool() ? 1 : type_.bits, shape_.data(), static_cast<int>(shape_.size()));
+      buffer_.memory_size = need;
+    }
+    return buffer_.memory;
+  }
   if (!buffer_.memory || allocated_ < need) {
     Free();
     void* p = nullptr;
@@ -62,8 +82,8 @@ void _Tensor_::CopyFromHost(const void* src, size_t n, const common::Target& tar
 }
 void _Tensor_::CopyToHost(void* dst, size_t n) const {
   CINN_CHECK_EQ(n, bytes()) << "host buffer size does not match the tensor";
-  CINN_CHECK(buffer_.memory) << "tensor has no device memory yet";
-  CINN_HIP_STATUS(cinn_hip_memcpy_d2h(dst, buffer_.memory, n, nullptr));
+  CINN_CHECK(data()) << "tensor has no device memory yet";
+  CINN_HIP_STATUS(cinn_hip_memcpy_d2h(dst, data(), n, nullptr));
 }
 
 // ---- Scope ----------------------------------------------------------------------------------------
@@ -385,6 +405,18 @@ std::string GraphCompiler::GenSourceCode(const CompileOptions& options) {
   return source_code_;
 }
 
+namespace {
+// one input, one output of the same type and size, and nothing but reshape operators in between
+bool IsReshapeOnly(const Group& g) {
+  if (g.inputs.size() != 1 || g.outputs.size() != 1 || g.nodes.empty()) return false;
+  for (auto* n : g.nodes)
+    if (n->op_type() != "reshape") return false;
+  const auto* in  = g.inputs[0];
+  const auto* out = g.outputs[0];
+  return in->dtype == out->dtype && in->numel() == out->numel();
+}
+}  // namespace
+
 std::unique_ptr<Program> GraphCompiler::Build(const CompileOptions& options) {
   auto module = LowerGraph(options);
   compiler_   = backends::Compiler::Create(target_);
@@ -393,6 +425,12 @@ std::unique_ptr<Program> GraphCompiler::Build(const CompileOptions& options) {
 
   std::vector<std::unique_ptr<Instruction>> instrs;
   for (auto& g : graph_->groups) {
+    if (options.reshape_as_view && IsReshapeOnly(*g)) {
+      // a reshape of a dense row-major tensor moves nothing: the result shares its operand's memory and no kernel
+      // runs (the reference copies, cinn/hlir/op/transform.cc Reshape)
+      scope_->Var(g->outputs[0]->id)->ShareBufferWith(scope_->Var(g->inputs[0]->id));
+      continue;
+    }
     std::vector<std::string> ins, outs;
     for (auto* v : g->inputs) ins.push_back(v->id);
     for (auto* v : g->outputs) outs.push_back(v->id);

@@ -38,7 +38,11 @@ class _Tensor_ {
 
   // device pointer; allocates on first use
   void* mutable_data(const common::Target& target);
-  void* data() const { return buffer_.memory; }
+  // This tensor becomes another view (its own shape, the same number of bytes) of `source`'s device memory: no
+  // allocation of its own, `source` stays the owner.  What a reshape of a dense row-major tensor is.
+  void ShareBufferWith(const std::shared_ptr<_Tensor_>& source);
+  bool is_view() const { return source_ != nullptr; }
+  void* data() const { return source_ ? source_->data() : buffer_.memory; }
   cinn_buffer_t* buffer() { return &buffer_; }
 
   // synchronous copies between host memory and the device buffer
@@ -51,6 +55,7 @@ class _Tensor_ {
   common::Type type_{common::Float(32)};
   cinn_buffer_t buffer_;
   size_t allocated_{0};
+  std::shared_ptr<_Tensor_> source_;  // set by ShareBufferWith
 };
 using Tensor = std::shared_ptr<_Tensor_>;
 
@@ -148,6 +153,7 @@ class Program {
 
 struct GraphCompileOptions {
   bool with_instantiate_variables{true};
+  bool reshape_as_view{true};  // groups made of reshapes only become views of their operand instead of copy kernels
   LoweringOptions lowering{LoweringOptions::FromEnv()};
 };
 

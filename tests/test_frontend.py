@@ -239,7 +239,9 @@ def test_const_inputs_make_pre_run_groups_and_broadcasts_stay_in_place():
     assert any("transpose" in g and " fc" in g for g in pre), pre
     # replicating a const vector is never materialised ahead of time
     assert not any("broadcast_to" in g for g in pre), pre
-    assert comp.num_instructions() == len(run)
+    # one instruction per group, except groups of reshapes only: those are views of their operand
+    views = [g for g in run if re.search(r"\{ (reshape )+\}", g)]
+    assert comp.num_instructions() == len(run) - len(views)
 
 
 def test_conv_batch_norm_residual_relu_fold_into_convolution_epilogues():

@@ -113,7 +113,8 @@ def test_config4_conv_bn_relu_batch32(gpu, dtype, name, ic, oc, k, s, p, hw, nhw
     (got_conv, got), comp = run(b, {X: x, W: w, S: scale, Bi: bias, M: mean, V: var}, [conv, y], conv_layout_nhwc=nhwc)
     # conv (MFMA) + per-channel sqrt + one fused bn/relu kernel; the channels-last form adds the transposes of x and
     # w and one back to NCHW for the fetched convolution output (the one of y is fused into the bn/relu kernel)
-    assert comp.num_instructions() == (6 if nhwc else 3), comp.fusion_groups()
+    # (a 1x1 filter changes layout by a reshape, which is a view and no instruction)
+    assert comp.num_instructions() == ((5 if k == 1 else 6) if nhwc else 3), comp.fusion_groups()
     sample = [0, 17, 31]
     want_conv = oracle.conv2d_nchw(x[sample], w, (s, s), (p, p))
     want = oracle.batch_norm_relu_nchw(want_conv, scale, bias, mean, var, 1e-5, relu=True)

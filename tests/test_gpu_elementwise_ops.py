@@ -188,3 +188,48 @@ def test_sixteen_bit_elementwise(gpu, dtype):
     tol = 1e-2
     np.testing.assert_allclose(to_f(z), (to_f(x) + to_f(y)) / to_f(y), rtol=tol, atol=1e-3)
     np.testing.assert_allclose(to_f(e), np.exp(to_f(x)), rtol=tol, atol=1e-3)
+
+
+def test_reshape_alone_is_a_view_of_its_operand(gpu):
+    """A group made of reshapes only runs no kernel: its result shares the operand's device memory (one instruction
+    fewer), follows new input data, works in the middle of a program and under graph replay, and can be switched back
+    to a copy kernel."""
+    from cinn_amd import runtime
+    from helpers import compile_only
+    rng = np.random.default_rng(41)
+    x = rng.standard_normal((4, 6, 10)).astype(np.float32)
+    w = rng.standard_normal((30, 7)).astype(np.float32)
+
+    def program(stream=None, **options):
+        b = NetBuilder("views")
+        X = b.create_input(Float(32), list(x.shape), "x")
+        W = b.create_input(Float(32), list(w.shape), "w")
+        flat = b.reshape(b.reshape(X, [24, 10]), [8, 30])          # reshapes only: a view of x
+        y = b.matmul(flat, W)                                      # a library call reads the view
+        z = b.reshape(b.relu(y), [4, 14])                          # fused with the relu: an ordinary kernel
+        comp = compile_only(b, [flat, y, z], stream=stream, **options)
+        comp.get_tensor("x").from_numpy(x)
+        comp.get_tensor("w").from_numpy(w)
+        return comp, (flat, y, z)
+
+    comp, (flat, y, z) = program()
+    copies, _ = program(reshape_as_view=0)
+    assert comp.num_instructions() == copies.num_instructions() - 1
+    comp.execute()
+    copies.execute()
+    for c in (comp, copies):
+        assert np.array_equal(c.get_tensor(flat.id).numpy(), x.reshape(8, 30))
+        np.testing.assert_allclose(c.get_tensor(y.id).numpy(), x.reshape(8, 30) @ w, rtol=1e-5, atol=1e-5)
+        np.testing.assert_allclose(c.get_tensor(z.id).numpy(), np.maximum(x.reshape(8, 30) @ w, 0).reshape(4, 14),
+                                   rtol=1e-5, atol=1e-5)
+    # new input data shows through the view without any instruction having to run
+    x2 = rng.standard_normal(x.shape).astype(np.float32)
+    comp.get_tensor("x").from_numpy(x2)
+    assert np.array_equal(comp.get_tensor(flat.id).numpy(), x2.reshape(8, 30))
+    stream = runtime.Stream()
+    replay, (flat, y, z) = program(stream=stream)
+    for data in (x, x2):
+        replay.get_tensor("x").from_numpy(data)
+        replay.execute_graph()
+        stream.synchronize()
+        np.testing.assert_allclose(replay.get_tensor(y.id).numpy(), data.reshape(8, 30) @ w, rtol=1e-5, atol=1e-5)
