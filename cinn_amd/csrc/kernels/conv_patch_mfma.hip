@@ -26,6 +26,14 @@
 //     instruction writes 8 pixels x 128 contiguous bytes.  No LDS staging, no barrier after the K loop.
 //   * Filter stage rows are swizzled with a key made of bits 1, 3 and 2 of the row, which keeps those permuted
 //     fragment reads conflict free.
+//
+// More than 64 input channels (conv3x3_patch_chunks_kernel): the K loop walks the channels 64 at a time and, inside a
+// chunk, the nine taps.  The patch of a chunk is what the single-chunk kernel keeps; two such buffers alternate, and
+// the feeding wavefronts fetch the next chunk's patch a few loads per K step while the current one is multiplied.  A
+// K step is still one filter stage of 64 x 64 (chunk c, tap t: the columns t C + 64 c .. + 63 of a filter row), the
+// ring slot is the tap modulo 3 whatever the chunk, and switching buffers is one add per pixel tile and chunk.  The
+// input then travels L2 -> LDS once instead of nine times, which is what bounds the implicit-GEMM tiles on the 14 x 14
+// and 28 x 28 layers (their blocks are few and small, so the filter is re-fetched per 128 pixels there as well).
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -62,15 +70,108 @@ struct PatchParams {
   float alpha, residual_scale;
   int relu;
   int n, h, w_in, oc;
+  int c;            // input channels (a multiple of 64)
   int rows;         // output rows per band
   int bands;        // bands per image
   int patch_loads;  // 1 KiB loads that cover the (rows + 2) (W + 2) positions of 10 slots
-  unsigned w_magic, w_shift;    // n / W == (n * w_magic) >> w_shift
+  unsigned w_magic, w_shift;    // n / W == (n * w_magic) >> w_shift (chunked kernel: W rounded up to a multiple of 8)
   unsigned pw_magic, pw_shift;  // the same for W + 2
 };
 
 // vmcnt(n): at most n of the wavefront's loads still in flight (they complete in issue order); lgkmcnt / expcnt open
 #define CINN_VMCNT(n) ((((n) & 15) | (((n) >> 4) << 14)) | 0x0F70)
+
+// The folded scale and shift of a lane's output channels (8 g .. 8 g + 7 and 32 + 8 g .. + 7 of the block's 64; alpha
+// and 0 without a table), fetched before the K loop so that the epilogue does not start with a trip to memory.  The
+// empty asm pins the loads there: the compiler would otherwise sink them to their first use.
+struct LaneScaleShift {
+  float sc[2][8], sh[2][8];
+};
+__device__ __forceinline__ void LoadScaleShift(const PatchParams& p, int n0, int lane, LaneScaleShift* out) {
+  const int oc0 = n0 + 8 * (lane >> 4);
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      out->sc[s][e] = p.scale ? p.scale[oc0 + 32 * s + e] : p.alpha;
+      out->sh[s][e] = p.shift ? p.shift[oc0 + 32 * s + e] : 0.0f;
+    }
+#pragma unroll
+  for (int s = 0; s < 2; ++s)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) asm volatile("" : "+v"(out->sc[s][e]), "+v"(out->sh[s][e]));
+}
+
+// Epilogue in registers (scale, shift, residual, relu), then whole 128-byte lines to global memory.  acc[i][j]: tile i
+// of 16 pixel slots (this lane: slot pix0 + 16 i of the band), transposed result tile j.  Slots are the band's pixels
+// in order (PADDED false: npix of them are real), or image rows padded to wp slots, a multiple of 8 (PADDED true: slot
+// q is column q % wp of the band's row q / wp; p.w_magic / p.w_shift divide by wp).
+template <typename T, int TMW, bool PADDED>
+__device__ __forceinline__ void PatchEpilogue(const PatchParams& p, const f32x4 (&acc)[TMW][4], const LaneScaleShift& ss,
+                                              int img, int y0, int n0, int rows, int wp, int pix0, int lane) {
+  typedef typename Mfma16<T>::vec8 vec8;
+  const int W    = p.w_in;
+  const int npix = rows * W;
+  // the band's pixel in slot q, or -1
+  auto pixel_of = [&](int q) -> int {
+    if (!PADDED) return q < npix ? q : -1;
+    const int ly = (int)(((uint64_t)(unsigned)q * p.w_magic) >> p.w_shift);
+    const int lx = q - ly * wp;
+    return ly < rows && lx < W ? ly * W + lx : -1;
+  };
+  // lane = (slot lane & 15 of each tile; channels 8 g .. 8 g + 7 and 32 + 8 g .. + 7)
+  const int g   = lane >> 4;
+  const int px  = lane & 15;
+  const int oc0 = n0 + 8 * g;
+  const int64_t out_row0 = ((int64_t)img * p.h + y0) * W;
+  T* const Y       = reinterpret_cast<T*>(p.y);
+  const T* const R = reinterpret_cast<const T*>(p.residual);
+  const int st_chunk = g + 4 * (px >> 3);  // 16-byte chunk of a pixel's 64 channels that this lane stores
+#pragma unroll
+  for (int i = 0; i < TMW; ++i) {
+    const int slot = pix0 + 16 * i;
+    vec8 res[2] = {};
+    if (R) {
+      const int pix = pixel_of(slot);
+      if (pix >= 0) {
+        const int64_t o = (out_row0 + pix) * p.oc + oc0;
+        res[0] = *reinterpret_cast<const vec8*>(R + o);
+        res[1] = *reinterpret_cast<const vec8*>(R + o + 32);
+      }
+    }
+    u32x4 out[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      vec8 o8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        // explicit fused multiply-adds rounded to fp32 and an empty asm before the conversion: the same arithmetic,
+        // in the same order, as the epilogues of the other convolution kernels
+        float v = __builtin_fmaf(acc[i][2 * s + (e >> 2)][e & 3], ss.sc[s][e], ss.sh[s][e]);
+        if (R) v = __builtin_fmaf(p.residual_scale, (float)res[s][e], v);
+        asm volatile("" : "+v"(v));
+        if (p.relu) v = v > 0.0f ? v : 0.0f;
+        o8[e] = (T)v;
+      }
+      out[s] = __builtin_bit_cast(u32x4, o8);
+    }
+    // first store: slots 0..7 of the tile as whole 128-byte lines (lanes px < 8: their own channels 8 g ..; lanes
+    // px >= 8: the channels 32 + 8 g .. of slot px - 8); second store: slots 8..15 (lanes px >= 8: their own channels
+    // 32 + 8 g ..; lanes px < 8: the channels 8 g .. of slot px + 8)
+    u32x4 first, second;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const unsigned from_below = RowShift8<true>(out[1][d]);   // second half of lane px - 8
+      const unsigned from_above = RowShift8<false>(out[0][d]);  // first half of lane px + 8
+      first[d]  = px < 8 ? out[0][d] : from_below;
+      second[d] = px < 8 ? from_above : out[1][d];
+    }
+    const int p_first  = pixel_of(slot - px + (px & 7));
+    const int p_second = pixel_of(slot - px + (px & 7) + 8);
+    if (p_first >= 0) *reinterpret_cast<u32x4*>(Y + (out_row0 + p_first) * p.oc + n0 + 8 * st_chunk) = first;
+    if (p_second >= 0) *reinterpret_cast<u32x4*>(Y + (out_row0 + p_second) * p.oc + n0 + 8 * st_chunk) = second;
+  }
+}
 
 template <typename T>
 __global__ void __launch_bounds__(128 * kWaves) conv3x3_c64_patch_kernel(PatchParams p) {
@@ -238,63 +339,306 @@ __global__ void __launch_bounds__(128 * kWaves) conv3x3_c64_patch_kernel(PatchPa
   }
 #undef CINN_SB
 
-  // ---- epilogue in registers: lane = (pixel lane & 15 of each tile; channels 8 g .. 8 g + 7 and 32 + 8 g .. + 7)
-  const int g   = lane >> 4;
-  const int px  = lane & 15;
-  const int oc0 = n0 + 8 * g;
-  float sc[2][8], sh[2][8];
-#pragma unroll
-  for (int s = 0; s < 2; ++s)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      sc[s][e] = p.scale ? p.scale[oc0 + 32 * s + e] : p.alpha;
-      sh[s][e] = p.shift ? p.shift[oc0 + 32 * s + e] : 0.0f;
-    }
-  const int64_t out_row0 = ((int64_t)img * p.h + y0) * W;
-  T* const Y       = reinterpret_cast<T*>(p.y);
-  const T* const R = reinterpret_cast<const T*>(p.residual);
-  const int st_chunk = g + 4 * (px >> 3);  // 16-byte chunk of a pixel's 64 channels that this lane stores
-#pragma unroll
-  for (int i = 0; i < kTMW; ++i) {
-    const int pix = pix0 + 16 * i;
-    vec8 res[2] = {};
-    if (R && pix < npix) {
-      const int64_t o = (out_row0 + pix) * p.oc + oc0;
-      res[0] = *reinterpret_cast<const vec8*>(R + o);
-      res[1] = *reinterpret_cast<const vec8*>(R + o + 32);
-    }
-    u32x4 out[2];
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      vec8 o8;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        // explicit fused multiply-adds rounded to fp32 and an empty asm before the conversion: the same arithmetic,
-        // in the same order, as the epilogues of the other convolution kernels
-        float v = __builtin_fmaf(acc[i][2 * s + (e >> 2)][e & 3], sc[s][e], sh[s][e]);
-        if (R) v = __builtin_fmaf(p.residual_scale, (float)res[s][e], v);
-        asm volatile("" : "+v"(v));
-        if (p.relu) v = v > 0.0f ? v : 0.0f;
-        o8[e] = (T)v;
-      }
-      out[s] = __builtin_bit_cast(u32x4, o8);
-    }
-    // first store: pixels 0..7 of the tile as whole 128-byte lines (lanes px < 8: their own channels 8 g ..; lanes
-    // px >= 8: the channels 32 + 8 g .. of pixel px - 8); second store: pixels 8..15 (lanes px >= 8: their own channels
-    // 32 + 8 g ..; lanes px < 8: the channels 8 g .. of pixel px + 8)
-    u32x4 first, second;
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      const unsigned from_below = RowShift8<true>(out[1][d]);   // second half of lane px - 8
-      const unsigned from_above = RowShift8<false>(out[0][d]);  // first half of lane px + 8
-      first[d]  = px < 8 ? out[0][d] : from_below;
-      second[d] = px < 8 ? from_above : out[1][d];
-    }
-    const int p_first  = pix - px + (px & 7);
-    const int p_second = p_first + 8;
-    if (p_first < npix) *reinterpret_cast<u32x4*>(Y + (out_row0 + p_first) * p.oc + n0 + 8 * st_chunk) = first;
-    if (p_second < npix) *reinterpret_cast<u32x4*>(Y + (out_row0 + p_second) * p.oc + n0 + 8 * st_chunk) = second;
+  LaneScaleShift ss;
+  LoadScaleShift(p, n0, lane, &ss);
+  PatchEpilogue<T, kTMW, false>(p, acc, ss, img, y0, n0, rows, W, pix0, lane);
+}
+// s_waitcnt vmcnt(n) for a count that is a constant only after unrolling (the builtin wants a literal)
+__device__ __forceinline__ void WaitLoadsInFlight(int n) {
+  switch (n) {
+    case 0: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(0)); break;
+    case 1: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(1)); break;
+    case 2: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(2)); break;
+    case 3: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(3)); break;
+    case 4: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(4)); break;
+    case 5: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(5)); break;
+    case 6: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(6)); break;
+    case 7: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(7)); break;
+    case 8: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(8)); break;
+    case 9: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(9)); break;
+    case 10: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(10)); break;
+    case 11: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(11)); break;
+    case 12: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(12)); break;
+    case 13: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(13)); break;
+    case 14: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(14)); break;
+    case 15: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(15)); break;
+    case 16: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(16)); break;
+    case 17: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(17)); break;
+    case 18: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(18)); break;
+    case 19: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(19)); break;
+    case 20: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(20)); break;
+    case 21: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(21)); break;
+    case 22: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(22)); break;
+    case 23: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(23)); break;
+    case 24: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(24)); break;
+    case 25: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(25)); break;
+    case 26: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(26)); break;
+    case 27: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(27)); break;
+    case 28: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(28)); break;
+    case 29: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(29)); break;
+    case 30: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(30)); break;
+    case 31: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(31)); break;
+    case 32: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(32)); break;
+    case 33: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(33)); break;
+    case 34: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(34)); break;
+    case 35: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(35)); break;
+    case 36: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(36)); break;
+    case 37: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(37)); break;
+    case 38: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(38)); break;
+    case 39: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(39)); break;
+    case 40: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(40)); break;
+    default: __builtin_amdgcn_s_waitcnt(CINN_VMCNT(0)); break;
   }
+}
+
+template <bool B>
+struct BoolTag {
+  static constexpr bool value = B;
+};
+
+constexpr int kPatchSteps = 4;  // K steps of a chunk after whose barriers the feeding wavefronts fetch patch loads
+constexpr int kRing       = kTaps;  // filter stages in the chunked kernel's ring: the slot of a stage is its tap
+
+// Loads a feeding wavefront of the chunked kernel may still have in flight when it arrives at the barrier of K step
+// (chunk, tap t): everything it issued after filter stage s + 1, which must have landed.  After the barrier of a step u
+// it issues pl patch loads (taps below kPatchSteps of a chunk that is not the last) and then the l loads of stage
+// u + kRing (while that stage exists, i.e. in chunks that are not the last); stage s + 1 was issued after barrier
+// s + 1 - kRing, so the steps s - 7 .. s - 1 count.  In the first chunk the steps before step 0 stand for the stages
+// 1 .. 8, issued in that order before the loop (after the first patch and stage 0, and without patch loads between
+// them).  At tap 8 of a chunk that is not the last, the next chunk's patch must have landed as well: only the stages
+// issued after the last patch load may be in flight.
+__device__ __forceinline__ constexpr int ChunkLoadsInFlight(int t, bool first, bool last, int pl, int l) {
+  int n = 0;
+  for (int u = t - (kRing - 2); u < t; ++u) {
+    const bool before = u < 0;  // a step of the previous chunk, or a stage fetched before the loop
+    const int tap     = before ? u + kTaps : u;
+    if (before && first) {
+      n += l;
+    } else if (before || !last) {
+      n += (tap < kPatchSteps ? pl : 0) + l;
+    }
+  }
+  if (!last && t == kTaps - 1) {
+    const int after_patch = (kTaps - kPatchSteps) * l;
+    n                     = n < after_patch ? n : after_patch;
+  }
+  return n;
+}
+
+// C = 64 * chunks input channels.  TMW: 16-pixel tiles per computing wavefront (the block holds 64 TMW pixels of one
+// band); PL: patch loads a feeding wavefront issues per K step, so a chunk's patch is at most 4 * kPatchSteps * PL KiB.
+// LDS: a ring of nine filter stages (a whole chunk: the slot of a stage is its tap, and a stage is requested eight K
+// steps before its use - the filters of a layer are read once per launch and XCD, from memory rather than from L2, and
+// with the two steps of lead that suffice for the single-chunk kernel's 72 KiB filter every step waited for its
+// loads), then two patch buffers of patch_loads KiB each.  At least two chunks.  The loop starts as soon as the first
+// patch and stage 0 have landed.
+//
+// Order of events around the barrier of K step s = 9 c + t (one per step but the last, after MFMA row RB of the step):
+//   computing wavefronts   every fragment of filter stage s is in registers before it; after it they read the first
+//                          fragments of stage s + 1 and, in step t = 8, of the next chunk's patch;
+//   feeding wavefronts     before it: stage s + 1 has landed and, at t = 8, the next chunk's patch (loads complete in
+//                          order: ChunkLoadsInFlight counts what was issued later and may still be in flight); after
+//                          it: PL patch loads of chunk c + 1 (steps t < kPatchSteps; the buffer was last read in step
+//                          9 c - 1, whose MFMAs everyone has issued before barrier 9 c), then stage s + 9 into the
+//                          slot of stage s.
+template <typename T, int TMW, int PL>
+__global__ void __launch_bounds__(128 * kWaves) conv3x3_patch_chunks_kernel(PatchParams p) {
+  constexpr int L   = 64 / 8 / kWaves;       // 1 KiB filter loads per feeding wavefront and stage
+  constexpr int NPL = PL * kPatchSteps;       // patch loads per feeding wavefront and chunk
+  constexpr int R   = 2 * TMW;                // MFMA rows (of four) per K step
+  constexpr int RB  = TMW > 2 * TMW - 5 ? TMW : 2 * TMW - 5;  // the barrier follows this row
+  constexpr int NB  = TMW < 6 ? RB + 1 : RB + 2;              // rows NB, NB + 1 request the next stage's slice 0
+  static_assert(TMW >= 4 && NB + 1 < R, "the schedule of a K step needs at least eight rows");
+  typedef typename Mfma16<T>::vec8 vec8;
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  char* const ring  = lds;
+  char* const patch = lds + kRing * kBTile;
+  const unsigned lds_addr = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) char*)lds);
+  const unsigned patch_addr = lds_addr + kRing * kBTile;
+
+  const int tid     = threadIdx.x;
+  const int lane    = tid & 63;
+  const int wave    = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int band    = blockIdx.x % p.bands;
+  const int img     = blockIdx.x / p.bands;
+  const int n0      = blockIdx.y * 64;
+  const int W       = p.w_in;
+  const int PW      = W + 2;
+  const int C       = p.c;
+  const int chunks  = C >> 6;
+  const int y0      = band * p.rows;
+  const int rows    = min(p.rows, p.h - y0);
+  const int WP      = (W + 7) & ~7;           // pixel slots per image row: a 16-lane tile is two halves of one row each
+  const int npos    = (p.rows + 2) * PW;
+  const int ktot    = kTaps * C;              // filter row length
+  const int patch_bytes = p.patch_loads * 1024;
+
+  if (wave >= kWaves) {
+    const int f = wave - kWaves;
+    // ---- the patch: load q fills the slots 64 q .. 64 q + 63 of a buffer, slot s = chunk s % 10 of position s / 10;
+    // this wavefront issues the loads q = f + 4 i.  Source pointers are kept per load and move on by 128 bytes per
+    // chunk (lanes that fetch halo or dummy slots stay on the page of zeros).  Loads beyond the last one repeat it: the
+    // count per K step stays a constant, which the vmcnt waits rely on.
+    const char* src[NPL];
+    unsigned step_bytes[NPL];
+    unsigned dst[NPL];
+    {
+      const char* const ximg  = reinterpret_cast<const char*>(p.x + (int64_t)img * p.h * W * C);
+      const char* const zeros = static_cast<const char*>(p.zero_page);
+#pragma unroll
+      for (int i = 0; i < NPL; ++i) {
+        const int q          = min(f + kWaves * i, p.patch_loads - 1);
+        const unsigned slot  = 64u * q + lane;
+        const unsigned pos   = (slot * 52429u) >> 19;  // slot / 10 for slot < 2^16
+        const unsigned chunk = slot - 10u * pos;
+        const int pr         = (int)(((uint64_t)pos * p.pw_magic) >> p.pw_shift);
+        const int iy         = y0 - 1 + pr;
+        const int ix         = (int)pos - pr * PW - 1;
+        const bool inside    = chunk < 8u && (unsigned)iy < (unsigned)p.h && (unsigned)ix < (unsigned)W && (int)pos < npos;
+        src[i]        = inside ? ximg + ((int64_t)(iy * W + ix) * C * 2 + chunk * 16u) : zeros + ((lane & 7) << 4);
+        step_bytes[i] = inside ? 128u : 0u;
+        dst[i]        = (unsigned)q * 1024u;
+      }
+    }
+    auto issue_patch = [&](int first, int count, unsigned buffer) {
+#pragma unroll
+      for (int i = first; i < first + count; ++i) {
+        AsyncCopy16(src[i], buffer + dst[i]);
+        src[i] += step_bytes[i];
+      }
+    };
+    // ---- filter stages: load t covers rows 8 (f L + t) .. + 7 of the stage
+    unsigned b_off[L];
+#pragma unroll
+    for (int t = 0; t < L; ++t) {
+      const int row = 8 * (f * L + t) + (lane >> 3);
+      b_off[t]      = (unsigned)(row * ktot + (((lane & 7) ^ FilterKey(row)) << 3)) * 2u;
+    }
+    const char* const wbase = reinterpret_cast<const char*>(p.w + (int64_t)n0 * ktot);
+    auto issue_stage = [&](int slot, int chunk, int tap) {
+      const char* const w0 = wbase + (tap * C + chunk * 64) * 2;
+#pragma unroll
+      for (int t = 0; t < L; ++t) AsyncCopy16(w0 + b_off[t], lds_addr + slot * kBTile + (f * L + t) * 1024);
+    };
+    // the first patch and stage 0 are all the first K step needs; the stages 1 .. 8 land while it runs
+    issue_patch(0, NPL, patch_addr);
+#pragma unroll
+    for (int st = 0; st < kRing; ++st) issue_stage(st, 0, st);
+    WaitLoadsInFlight((kRing - 1) * L);
+    BarrierLds();
+    auto feed_chunk = [&](auto first_tag, auto last_tag, int c) {
+      constexpr bool FIRST = decltype(first_tag)::value;
+      constexpr bool LAST  = decltype(last_tag)::value;
+      const unsigned next_buffer = patch_addr + ((c + 1) & 1) * patch_bytes;
+#pragma unroll
+      for (int t = 0; t + (LAST ? 1 : 0) < kTaps; ++t) {
+        WaitLoadsInFlight(ChunkLoadsInFlight(t, FIRST, LAST, PL, L));
+        BarrierLds();
+        if (!LAST) {
+          if (t < kPatchSteps) issue_patch(t * PL, PL, next_buffer);
+          issue_stage(t, c + 1, t);
+        }
+      }
+    };
+    feed_chunk(BoolTag<true>{}, BoolTag<false>{}, 0);
+    for (int c = 1; c + 1 < chunks; ++c) feed_chunk(BoolTag<false>{}, BoolTag<false>{}, c);
+    feed_chunk(BoolTag<false>{}, BoolTag<true>{}, chunks - 1);
+    return;
+  }
+
+  // ---- computing wavefronts
+  const int frag_kg = ((lane >> 4) & 1) * 2 + (lane >> 5);  // k chunks 0, 2, 1, 3 for the lane groups 0..3
+  const int pix0    = wave * (TMW * 16) + (lane & 15);
+  // LDS address of this lane's chunk of K slice 0 under tap (0, 0) in the patch buffer of the current chunk, per tile.
+  // The eight lanes LDS serves together hold consecutive slots of one image row, i.e. consecutive positions: with
+  // tiles that straddle rows (positions two apart at the seam) a third of the reads of a 14-wide image took two
+  // passes, and LDS reads, half an instruction per MFMA here, are what the K loop waits for.  Slots beyond the row's
+  // last pixel read that pixel's position again (a broadcast, no conflict); slots beyond the band read position 0.
+  const char* a_base[TMW];
+#pragma unroll
+  for (int i = 0; i < TMW; ++i) {
+    const int slot = pix0 + 16 * i;
+    const int ly   = (int)(((uint64_t)(unsigned)slot * p.w_magic) >> p.w_shift);
+    const int lx   = min(slot - ly * WP, W - 1);
+    const int pos  = ly < rows ? ly * PW + lx : 0;
+    a_base[i]      = patch + pos * kPitch + frag_kg * 16;
+  }
+  LaneScaleShift ss;
+  LoadScaleShift(p, n0, lane, &ss);
+  const char* b_base[2][4];
+  {
+    const int q = lane & 15;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int row = 32 * (j >> 1) + 8 * (q >> 2) + 4 * (j & 1) + (q & 3);
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) b_base[kk][j] = ring + row * 128 + (((kk * 4 + frag_kg) ^ FilterKey(row)) << 4);
+    }
+  }
+  const int row_pitch = PW * kPitch;
+
+  f32x4 acc[TMW][4];
+#pragma unroll
+  for (int i = 0; i < TMW; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+  // A K step is R rows of 4 MFMAs: row r multiplies the pixel fragment of tile r % TMW, slice r / TMW, with the four
+  // filter fragments of that slice.  Pixel fragments are requested three rows ahead, across the ends of steps and of
+  // chunks; filter fragments: slice 1 in rows 0 and 1, the next stage's slice 0 in rows NB and NB + 1.
+  vec8 ar[TMW];
+  vec8 bf[2][4];
+  auto read_b = [&](int slot, int kk, int j) -> vec8 { return *reinterpret_cast<const vec8*>(b_base[kk][j] + slot * kBTile); };
+  BarrierLds();  // the first patch and the first filter stages are in LDS
+#pragma unroll
+  for (int r = 0; r < 3; ++r) ar[r] = *reinterpret_cast<const vec8*>(a_base[r]);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) bf[0][j] = read_b(0, 0, j);
+#define CINN_SB __builtin_amdgcn_sched_barrier(0)
+  // to_next: from tap (2, 0) of this chunk's buffer to tap (0, 0) of the other buffer
+  auto multiply_chunk = [&](auto last_tag, int to_next) {
+    constexpr bool LAST = decltype(last_tag)::value;
+#pragma unroll
+    for (int kt = 0; kt < kTaps; ++kt) {
+      const bool has_next = !(LAST && kt + 1 == kTaps);
+      const int dx        = kt % 3;
+      const int next_dx   = dx == 2 ? 0 : dx + 1;
+      const int next_off  = kt + 1 == kTaps ? to_next : (dx == 2 ? row_pitch : 0);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          CINN_SB;
+          acc[r % TMW][j] = Mfma16<T>::mma(bf[r / TMW][j], ar[r % TMW], acc[r % TMW][j]);
+          CINN_SB;
+          if (j == 0) {
+            if (r + 3 < R) {
+              ar[(r + 3) % TMW] = *reinterpret_cast<const vec8*>(a_base[(r + 3) % TMW] + dx * kPitch + ((r + 3) / TMW) * 64);
+            } else if (has_next) {
+              ar[r + 3 - R] = *reinterpret_cast<const vec8*>(a_base[r + 3 - R] + next_off + next_dx * kPitch);
+            }
+          }
+          if ((j == 1 || j == 2) && r < 2) bf[1][r * 2 + j - 1] = read_b(kt, 1, r * 2 + j - 1);
+          if ((j == 1 || j == 2) && r >= NB && r < NB + 2 && has_next)
+            bf[0][(r - NB) * 2 + j - 1] = read_b((kt + 1) % kRing, 0, (r - NB) * 2 + j - 1);
+        }
+        if (r == RB && has_next) {
+          CINN_SB;
+          BarrierLds();
+        }
+      }
+      if (has_next && (dx == 2)) {
+        CINN_SB;
+#pragma unroll
+        for (int i = 0; i < TMW; ++i) a_base[i] += next_off;
+      }
+    }
+  };
+  for (int c = 0; c + 1 < chunks; ++c) multiply_chunk(BoolTag<false>{}, ((c & 1) ? -patch_bytes : patch_bytes) - 2 * row_pitch);
+  multiply_chunk(BoolTag<true>{}, 0);
+#undef CINN_SB
+
+  PatchEpilogue<T, TMW, true>(p, acc, ss, img, y0, n0, rows, WP, pix0, lane);
 }
 #undef CINN_VMCNT
 
@@ -318,6 +662,43 @@ bool PlanFor(const ConvNhwcArgs& a, PatchPlan* plan) {
   if (bytes > kLdsLimit) return false;
   *plan = PatchPlan{rows, bands, patch_loads, bytes};
   return true;
+}
+
+// The same for more than 64 channels: bands of at most 64 TMW pixel slots (image rows padded to a multiple of 8
+// slots) and two patch buffers; rows are given up until
+// the buffers fit.  *per_step: patch loads per feeding wavefront and K step (2 or 3).  False when more than three tenths
+// of the pixel slots would stay empty.
+template <int TMW>
+bool PlanChunksFor(const ConvNhwcArgs& a, PatchPlan* plan, int* per_step) {
+  constexpr int capacity = kWaves * TMW * 16;
+  const int wp = (a.w_in + 7) & ~7;  // pixel slots per image row
+  int rows     = capacity / wp;
+  rows         = rows < a.h ? rows : a.h;
+  for (; rows >= 1; --rows) {
+    const int bands       = (a.h + rows - 1) / rows;
+    const int even        = (a.h + bands - 1) / bands;
+    const int slots       = (even + 2) * (a.w_in + 2) * 10;
+    const int patch_loads = (slots + 63) / 64;
+    const int bytes       = kRing * kBTile + 2 * patch_loads * 1024;
+    if (patch_loads > kWaves * kPatchSteps * 3 || bytes > kLdsLimit) continue;
+    if ((int64_t)a.h * a.w_in * 10 < (int64_t)bands * capacity * 7) return false;
+    *plan     = PatchPlan{even, bands, patch_loads, bytes};
+    *per_step = patch_loads > kWaves * kPatchSteps * 2 ? 3 : 2;  // 32 KiB, else 48 KiB of patch per buffer
+    return true;
+  }
+  return false;
+}
+
+template <typename T, int TMW, int PL>
+void LaunchChunks(const PatchParams& p, const PatchPlan& plan, hipStream_t stream) {
+  auto kernel = conv3x3_patch_chunks_kernel<T, TMW, PL>;
+  static const bool configured = [&] {  // once per instantiation, thread-safe
+    CINN_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
+    return true;
+  }();
+  (void)configured;
+  dim3 grid(p.n * p.bands, p.oc / 64);
+  hipLaunchKernelGGL(kernel, grid, dim3(128 * kWaves), plan.lds_bytes, stream, p);
 }
 
 template <typename T>
@@ -356,13 +737,16 @@ bool TryConvPatch(const ConvNhwcArgs& a, hipStream_t stream) {
   if (a.kh != 3 || a.kw != 3 || a.stride_h != 1 || a.stride_w != 1 || a.pad_h != 1 || a.pad_w != 1 || a.dil_h != 1 ||
       a.dil_w != 1 || a.oh != a.h || a.ow != a.w_in)
     return false;
-  if (a.c != 64 || a.oc % 64 != 0) return false;
+  if (a.c % 64 != 0 || a.c > 2048 || a.oc % 64 != 0) return false;  // one chunk, or two and more
   if ((int64_t)a.n * a.h * a.w_in * a.c >= INT_MAX || (int64_t)a.n * a.h * a.w_in * a.oc >= INT_MAX) return false;
   if (reinterpret_cast<uintptr_t>(a.x) % 16 != 0 || reinterpret_cast<uintptr_t>(a.w) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(a.y) % 16 != 0 || reinterpret_cast<uintptr_t>(a.residual) % 16 != 0)
     return false;
+  constexpr int kChunksTMW = 4;
+  const bool chunked = a.c != 64;
+  int per_step       = 0;
   PatchPlan plan;
-  if (!PlanFor(a, &plan)) return false;
+  if (!(chunked ? PlanChunksFor<kChunksTMW>(a, &plan, &per_step) : PlanFor(a, &plan))) return false;
   // one block per band, image and 64 output channels; below ~100 blocks most of the chip would idle and the
   // implicit-GEMM tiles are the better choice
   if (flag != 2 && (int64_t)a.n * plan.bands * (a.oc / 64) < 96) return false;
@@ -371,11 +755,23 @@ bool TryConvPatch(const ConvNhwcArgs& a, hipStream_t stream) {
   p.scale = a.scale, p.shift = a.shift, p.residual = static_cast<const uint16_t*>(a.residual);
   p.zero_page = ConvZeroPage();
   p.alpha = a.alpha, p.residual_scale = a.residual_scale, p.relu = a.relu ? 1 : 0;
-  p.n = a.n, p.h = a.h, p.w_in = a.w_in, p.oc = a.oc;
+  p.n = a.n, p.h = a.h, p.w_in = a.w_in, p.oc = a.oc, p.c = a.c;
   p.rows = plan.rows, p.bands = plan.bands, p.patch_loads = plan.patch_loads;
-  MagicFor(a.w_in, &p.w_magic, &p.w_shift);
+  MagicFor(chunked ? (a.w_in + 7) & ~7 : a.w_in, &p.w_magic, &p.w_shift);
   MagicFor(a.w_in + 2, &p.pw_magic, &p.pw_shift);
-  if (is_bf16) {
+  if (chunked && per_step == 2) {
+    if (is_bf16) {
+      LaunchChunks<__bf16, kChunksTMW, 2>(p, plan, stream);
+    } else {
+      LaunchChunks<_Float16, kChunksTMW, 2>(p, plan, stream);
+    }
+  } else if (chunked) {
+    if (is_bf16) {
+      LaunchChunks<__bf16, kChunksTMW, 3>(p, plan, stream);
+    } else {
+      LaunchChunks<_Float16, kChunksTMW, 3>(p, plan, stream);
+    }
+  } else if (is_bf16) {
     Launch<__bf16>(p, plan, stream);
   } else {
     Launch<_Float16>(p, plan, stream);

@@ -583,6 +583,51 @@ def test_convolution_with_the_input_patch_resident_in_lds(gpu, patch_kernel_ever
     assert np.all(np.abs(got - other) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
 
 
+PATCH_CHUNK_CASES = [
+    # (n, ic, h, w, oc): 3x3, stride 1, padding 1, more than 64 input channels (walked 64 at a time, two patch buffers)
+    (2, 128, 28, 28, 128),   # 4 bands of 7 rows, two chunks
+    (2, 256, 14, 14, 256),   # one band = the whole image (halo rows above and below both outside), four chunks
+    (1, 512, 14, 14, 64),    # eight chunks
+    (2, 192, 12, 16, 64),    # three chunks (odd count: the last chunk sits in the first buffer again)
+    (1, 128, 16, 25, 64),    # odd width, bands of 8 rows: 25 of the 32 pixel slots of a row are real
+    (2, 128, 12, 32, 64),    # bands of 6 rows of 32 pixels
+    (1, 128, 27, 28, 64),    # bands of 7, 7, 7 and 6 rows: first, inner and a shorter last band
+    (2, 128, 7, 7, 64),      # does not qualify (49 of 256 pixel slots): stays on the other kernels
+]
+
+
+@pytest.mark.parametrize("dtype,tol", [("float16", 1e-2), ("bfloat16", 2e-2)])
+@pytest.mark.parametrize("case", PATCH_CHUNK_CASES)
+def test_convolution_with_the_input_patch_resident_in_lds_by_channel_chunks(gpu, patch_kernel_everywhere, case, dtype, tol):
+    """conv3x3_patch_chunks_kernel against the oracle and against the implicit-GEMM kernel (which adds the same
+    products tap by tap instead of chunk by chunk: equal within rounding, not bit for bit)."""
+    n, ic, h, w_, oc = case
+    rng = np.random.default_rng(sum(case) + 11)
+    x = round_to(rng.standard_normal((n, ic, h, w_)), dtype)
+    w = round_to(rng.standard_normal((oc, ic, 3, 3)) * np.sqrt(2.0 / (ic * 9)), dtype)
+    got = call_conv_nhwc(x, w, 1, 1, 1, dtype)
+    want = oracle.conv2d_nchw(x, w, (1, 1), (1, 1))
+    scale = oracle.conv2d_nchw(np.abs(x), np.abs(w), (1, 1), (1, 1))
+    assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+    patch_kernel_everywhere.cinn_hip_conv_patch_mode(0)
+    other = call_conv_nhwc(x, w, 1, 1, 1, dtype)
+    patch_kernel_everywhere.cinn_hip_conv_patch_mode(2)
+    assert np.all(np.abs(got - other) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+
+
+def test_chunked_patch_convolution_with_residual_epilogue(gpu, patch_kernel_everywhere):
+    """alpha / beta through the in-register epilogue of the chunked kernel: y = 0.5 conv(x, w) + 2 y0."""
+    n, ic, h, w_, oc = 2, 256, 14, 14, 128
+    rng = np.random.default_rng(198)
+    x = round_to(rng.standard_normal((n, ic, h, w_)), "float16")
+    w = round_to(rng.standard_normal((oc, ic, 3, 3)) * np.sqrt(2.0 / (ic * 9)), "float16")
+    y0 = round_to(rng.standard_normal((n, oc, h, w_)), "float16")
+    got = call_conv_nhwc(x, w, 1, 1, 1, "float16", alpha=0.5, beta=2.0, y_init=y0).astype(np.float64)
+    want = 0.5 * oracle.conv2d_nchw(x, w, (1, 1), (1, 1)).astype(np.float64) + 2.0 * y0
+    scale = 0.5 * oracle.conv2d_nchw(np.abs(x), np.abs(w), (1, 1), (1, 1)) + 2.0 * np.abs(y0)
+    assert np.all(np.abs(got - want) <= 2.0 ** -10 * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+
+
 def test_patch_convolution_with_residual_epilogue(gpu, patch_kernel_everywhere):
     """alpha / beta through the in-register epilogue: y = 0.5 conv(x, w) + 2 y0."""
     n, ic, h, w_, oc = 2, 64, 30, 28, 128
