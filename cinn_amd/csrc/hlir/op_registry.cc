@@ -53,8 +53,11 @@ std::vector<ShapeType> SameShapeAsFirst(const std::vector<ShapeType>& in, const 
 std::vector<Type> SameTypeAsFirst(const std::vector<Type>& in, const AttributeMap&) { return {in[0]}; }
 std::vector<Type> BoolType(const std::vector<Type>&, const AttributeMap&) { return {common::Bool()}; }
 
+// A call of a math function by its target-independent name; optim::MapExternCall picks the device library's function
+// for the type of the first argument when the group's kernel is built (cinn/optim/map_extern_call.cc:45-115).
 Expr CallExtern(const std::string& fn, const Type& t, std::vector<Expr> args, const Type& ret) {
-  return ir::MakeCall(ret, ExternFuncName(fn, t), std::move(args));
+  CINN_CHECK(!args.empty() && args.front().type() == t) << fn << ": the first argument selects the library function";
+  return ir::MakeCall(ret, fn, std::move(args));
 }
 
 void RegisterUnaryMath(OpRegistry* r, const std::string& op_name, const std::string& fn) {

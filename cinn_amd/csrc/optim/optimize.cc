@@ -1,7 +1,9 @@
 #include "optim/optimize.h"
 
 #include <algorithm>
+#include <set>
 
+#include "common/type.h"
 #include "ir/ir_mutator.h"
 
 namespace cinn {
@@ -99,7 +101,82 @@ class GpuLoopBinder : public IrMutator {
   GpuAxisInfo* info_;
 };
 
+// cinn/optim/map_extern_call.cc:25-40
+const std::set<std::string>& FloatMathNames() {
+  static const std::set<std::string> names = {
+      "exp",   "erf",  "sigmoid",  "sqrt",  "log",       "log2",  "log10", "floor", "ceil",  "round", "trunc",
+      "cos",   "cosh", "tan",      "sin",   "sinh",      "acos",  "acosh", "asin",  "asinh", "atan",  "atanh",
+      "isnan", "tanh", "isfinite", "isinf", "remainder", "rsqrt", "cbrt",  "abs",   "pow",   "mod"};
+  return names;
+}
+const std::set<std::string>& IntMathNames() {
+  static const std::set<std::string> names = {"left_shift",  "right_shift", "bitwise_or", "bitwise_and",
+                                              "bitwise_xor", "bitwise_not", "pow",        "logical_right_shift",
+                                              "clz",         "popc",        "mod"};
+  return names;
+}
+
+bool IsFloatConstant(const Expr& e, double value) {
+  if (auto* f = e.As<FloatImm>()) return f->value == value;
+  if (auto* c = e.As<Cast>()) return IsFloatConstant(c->v, value);  // a constant rounded to a 16-bit type
+  return false;
+}
+
+class ExternCallMapper : public IrMutator {
+ public:
+  Expr Mutate(const Expr& e) override {
+    if (!e.defined()) return e;
+    Expr out   = MutateChildren(e);
+    auto* call = out.As<Call>();
+    if (!call || call->args.empty()) return out;
+    std::string name        = call->name;
+    std::vector<Expr> args  = call->args;
+    if (name == "pow" && args.size() >= 2 && IsFloatConstant(args[1], 0.5)) {
+      name = "sqrt";
+      args.erase(args.begin() + 1);
+    } else if (name == "pow" && args.size() >= 2 && IsFloatConstant(args[1], -0.5)) {
+      name = "rsqrt";
+      args.erase(args.begin() + 1);
+    }
+    if (!FloatMathNames().count(name) && !IntMathNames().count(name)) return out;
+    const std::string library_name = "cinn_hip_" + name + "_" + common::TypeSuffix(args.front().type());
+    Expr mapped                    = MakeCall(out.type(), library_name, std::move(args), call->call_type);
+    mapped.As<Call>()->buffer_args = call->buffer_args;
+    return mapped;
+  }
+};
+
+class SyncThreadsUnguard : public IrMutator {
+ public:
+  Expr Mutate(const Expr& e) override {
+    if (!e.defined()) return e;
+    Expr out = MutateChildren(e);
+    auto* br = out.As<IfThenElse>();
+    if (!br || br->false_case.defined() || br->condition.node_type() != IrNodeTy::EQ) return out;
+    if (!static_cast<Binary*>(br->condition.get())->b.is_int_imm(0)) return out;
+    Expr body = br->true_case;
+    if (auto* b = body.As<Block>()) {
+      if (b->stmts.size() != 1) return out;
+      body = b->stmts[0];
+    }
+    auto* call = body.As<Call>();
+    if (call && call->name == "__syncthreads") return body;
+    return out;
+  }
+};
+
 }  // namespace
+
+Expr MapExternCall(const Expr& body, const common::Target& target) {
+  if (target.arch != common::Target::Arch::AMDGPU) return body;
+  ExternCallMapper m;
+  return m.Mutate(body);
+}
+
+Expr SyncThreadsDropIfThenElse(const Expr& body) {
+  SyncThreadsUnguard m;
+  return m.Mutate(body);
+}
 
 Expr VectorizeLoops(const Expr& body) {
   Vectorizer v;
@@ -113,8 +190,10 @@ Expr TransformGpuForloops(const Expr& body, GpuAxisInfo* axis_info) {
 }
 
 void OptimizeFuncGPU(LoweredFunc* func) {
+  func->body = MapExternCall(func->body, common::DefaultAMDGPUTarget());
   func->body = VectorizeLoops(func->body);
   func->body = TransformGpuForloops(func->body, &func->axis_info);
+  func->body = SyncThreadsDropIfThenElse(func->body);
   CINN_CHECK(func->axis_info.valid) << "kernel " << func->name << " has no loop bound to a GPU axis";
 }
 

@@ -192,6 +192,22 @@ def test_generated_source_idioms():
     assert re.search(r"if \(.*< 750\)", src)  # 3000 / 4 vectors
 
 
+def test_math_calls_are_mapped_to_the_device_library_by_operand_type():
+    """Operators emit target-independent names; the extern-call pass picks cinn_hip_<name>_<type> from the type of the
+    first argument (the reference's MapExternCall, cinn/optim/map_extern_call.cc:45-115)."""
+    from cinn_amd.common import Float, Int
+    b = NetBuilder("t")
+    x = b.create_input(Float(32), [64, 8], "x")
+    h = b.create_input(Float(16), [64, 8], "h")
+    n = b.create_input(Int(32), [64, 8], "n")
+    outs = [b.exp(b.tanh(x)), b.erf(h), b.bitwise_and(n, b.left_shift(n, n)), b.is_nan(x)]
+    src = compile_only(b, outs).source_code()
+    for name in ("cinn_hip_exp_fp32(", "cinn_hip_tanh_fp32(", "cinn_hip_erf_fp16(", "cinn_hip_bitwise_and_int32(",
+                 "cinn_hip_left_shift_int32(", "cinn_hip_isnan_fp32("):
+        assert name in src, name
+    assert not re.search(r"[^_a-z]exp\(", src)  # no unmapped call is left
+
+
 # ---- program passes for convolutional networks (compile only: hiprtc needs no GPU) -------------------------------------
 def _conv_net(const_params, dtype=None):
     from cinn_amd.common import Float
