@@ -90,6 +90,12 @@ const std::map<std::string, Method>& Methods() {
     m["Argmin"] = [](NetBuilder& b, const std::vector<Variable>& in, const AttributeMap& a) {
       return std::vector<Variable>{b.Argmin(in.at(0), GetAttr<int>(a, "axis", 0), GetAttr<bool>(a, "keep_dim", false))};
     };
+    m["ArgSort"] = [](NetBuilder& b, const std::vector<Variable>& in, const AttributeMap& a) {
+      return b.ArgSort(in.at(0), GetAttr<int>(a, "axis", 0), GetAttr<bool>(a, "is_ascend", true));
+    };
+    m["Sort"] = [](NetBuilder& b, const std::vector<Variable>& in, const AttributeMap& a) {
+      return std::vector<Variable>{b.Sort(in.at(0), GetAttr<int>(a, "axis", 0), GetAttr<bool>(a, "is_ascend", true))};
+    };
     m["Select"] = [](NetBuilder& b, const std::vector<Variable>& in, const AttributeMap&) {
       return std::vector<Variable>{b.Select(in.at(0), in.at(1), in.at(2))};
     };

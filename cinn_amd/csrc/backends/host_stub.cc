@@ -44,6 +44,9 @@ void InvokeSoftmaxForward(const std::vector<BakedArg>& a, void* args, int32_t n,
   cinn_call_cudnn_softmax_forward(args, n, I(a[2]), I(a[3]), F(a[4]), F(a[5]), I(a[6]), I(a[7]), I(a[8]), I(a[9]),
                                   I(a[10]), I(a[11]), I(a[12]), I(a[13]), stream);
 }
+void InvokeArgsort(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
+  cinn_call_hip_argsort(args, n, I(a[2]), I(a[3]), I(a[4]), I(a[5]), I(a[6]), stream);
+}
 void InvokeBatchedCublas(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
   cinn_call_batched_cublas(args, n, I(a[2]), B(a[3]), B(a[4]), B(a[5]), F(a[6]), F(a[7]), I(a[8]), I(a[9]), I(a[10]),
                            I(a[11]), I(a[12]), I(a[13]), I(a[14]), I(a[15]), stream);
@@ -81,6 +84,8 @@ ExternApiRegistry::ExternApiRegistry() {
   Register("cinn_call_hip_conv2d_bn_relu", InvokeConv2dBnRelu, 24);
   Register("cinn_call_cudnn_pool2d_forward", InvokePool2dForward, 21);
   Register("cinn_call_cudnn_softmax_forward", InvokeSoftmaxForward, 15);
+  // (kernel_args, kernel_args_num, outer, size, inner, is_ascend, outputs, kernel_stream)
+  Register("cinn_call_hip_argsort", InvokeArgsort, 8);
   // (kernel_args, kernel_args_num, opside, trans_a, trans_b, trans_o, alpha, beta, a1..a4, b1..b4, kernel_stream)
   Register("cinn_call_batched_cublas", InvokeBatchedCublas, 17);
   Register("cinn_call_cudnn_conv2d_backward_data", InvokeConv2dBackward<&cinn_call_cudnn_conv2d_backward_data>, 25);

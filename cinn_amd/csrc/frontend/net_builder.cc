@@ -170,6 +170,13 @@ Variable NetBuilder::Argmin(const Variable& x, const int& axis, const bool& keep
   return CustomInstr("argmin", {x}, {{"axis", axis}, {"keep_dim", keep_dim}}).front();
 }
 
+std::vector<Variable> NetBuilder::ArgSort(const Variable& operand, const int& axis, const bool& is_ascend) {
+  return CustomInstr("argsort", {operand}, {{"axis", axis}, {"is_ascend", is_ascend}});
+}
+Variable NetBuilder::Sort(const Variable& operand, const int& axis, const bool& is_ascend) {
+  return CustomInstr("sort", {operand}, {{"axis", axis}, {"is_ascend", is_ascend}}).front();
+}
+
 Variable NetBuilder::BroadcastTo(const Variable& x, const ShapeType& out_shape) {
   // numpy alignment: the operand's dimensions map onto the trailing output dimensions
   auto x_rank = x->shape.size();

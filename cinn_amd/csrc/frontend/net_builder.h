@@ -69,6 +69,9 @@ class NetBuilder {
   Variable ReduceAny(const Variable& x, const utils::ShapeType& dim = {}, bool keep_dim = false);
   Variable Argmax(const Variable& x, const int& axis = 0, const bool& keep_dim = false);
   Variable Argmin(const Variable& x, const int& axis = 0, const bool& keep_dim = false);
+  // cinn/frontend/net_builder.h:1028-1046: {indices, positions} resp. the sorted values, both of the operand's shape
+  std::vector<Variable> ArgSort(const Variable& operand, const int& axis, const bool& is_ascend = true);
+  Variable Sort(const Variable& operand, const int& axis, const bool& is_ascend = true);
 
   // ---- shape manipulation -----------------------------------------------------------------------
   Variable BroadcastTo(const Variable& x, const utils::ShapeType& out_shape);

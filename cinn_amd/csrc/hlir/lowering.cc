@@ -1457,6 +1457,18 @@ ir::LoweredFuncRef OpLowerer::LowerLibraryCall(const Group& group) const {
     } else {
       push_ints({y[0], y[3], y[1], y[2]});
     }
+  } else if (op == "argsort" || op == "sort") {
+    // [outer][size][inner] around the sorted axis; argsort writes indices and positions, sort the values
+    api            = "cinn_call_hip_argsort";
+    const auto& x  = n->inputs[0]->shape;
+    int axis       = GetAttr<int>(n->attrs, "axis", 0);
+    if (axis < 0) axis += static_cast<int>(x.size());
+    CINN_CHECK(axis >= 0 && axis < static_cast<int>(x.size())) << op << ": axis out of range";
+    int64_t outer = 1, inner = 1;
+    for (int d = 0; d < axis; ++d) outer *= x[d];
+    for (size_t d = axis + 1; d < x.size(); ++d) inner *= x[d];
+    push_ints({static_cast<int>(outer), x[axis], static_cast<int>(inner), GetAttr<bool>(n->attrs, "is_ascend", true) ? 1 : 0,
+               op == "argsort" ? 3 : 4});
   } else {
     CINN_CHECK(false) << "op " << op << " has no GPU lowering";
   }

@@ -573,6 +573,30 @@ OpRegistry::OpRegistry() {
     op.infer_dtype = SameTypeAsFirst;
   }
   {
+    // cinn/hlir/op/contrib/sort.cc:307-350: both keep the operand's shape; argsort has two int32 outputs (indices,
+    // positions), sort one of the operand's type
+    auto check_axis = [](const std::vector<ShapeType>& in, const AttributeMap& a) {
+      CINN_CHECK_EQ(in.size(), 1u) << "sort / argsort take one operand";
+      int axis = GetAttr<int>(a, "axis", 0);
+      if (axis < 0) axis += static_cast<int>(in[0].size());
+      CINN_CHECK(axis >= 0 && axis < static_cast<int>(in[0].size())) << "sort / argsort: axis " << axis << " out of range";
+    };
+    auto& arg       = r->Register("argsort");
+    arg.pattern     = OpPatternKind::kNonFusible;
+    arg.infer_shape = [check_axis](const std::vector<ShapeType>& in, const AttributeMap& a) {
+      check_axis(in, a);
+      return std::vector<ShapeType>{in[0], in[0]};
+    };
+    arg.infer_dtype = [](const std::vector<Type>&, const AttributeMap&) { return std::vector<Type>{common::Int(32), common::Int(32)}; };
+    auto& srt       = r->Register("sort");
+    srt.pattern     = OpPatternKind::kNonFusible;
+    srt.infer_shape = [check_axis](const std::vector<ShapeType>& in, const AttributeMap& a) {
+      check_axis(in, a);
+      return std::vector<ShapeType>{in[0]};
+    };
+    srt.infer_dtype = SameTypeAsFirst;
+  }
+  {
     // pooling output size and attribute meaning as cinn/hlir/pe/nn.cc:956-1109 (PoolImpl)
     auto& op       = r->Register("pool2d");
     op.pattern     = OpPatternKind::kNonFusible;

@@ -155,6 +155,14 @@ class NetBuilder(object):
     def argmin(self, x, axis=0, keep_dim=False):
         return self._call1("Argmin", [x], axis=axis, keep_dim=keep_dim)
 
+    def argsort(self, x, axis, is_ascend=True):
+        """[indices, positions]: the stable order along `axis` and, per element, the count of smaller (descending:
+        larger) elements of its row (cinn/frontend/net_builder.h:1028-1035)."""
+        return self._call("ArgSort", [x], axis=axis, is_ascend=is_ascend)
+
+    def sort(self, x, axis, is_ascend=True):
+        return self._call1("Sort", [x], axis=axis, is_ascend=is_ascend)
+
     def broadcast_to(self, x, out_shape, broadcast_axes=None):
         if broadcast_axes is None:
             return self._call1("BroadcastTo", [x], out_shape=list(out_shape))

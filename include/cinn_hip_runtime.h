@@ -208,6 +208,19 @@ void cinn_call_cudnn_softmax_forward(void* v_args, int num_args, int mode, int f
                                      int input_n, int input_c, int input_h, int input_w, int output_n, int output_c,
                                      int output_h, int output_w, void* stream);
 
+/* argsort / sort along one axis.  The reference has no library call for them: its `argsort` and `sort` operators
+ * (cinn/hlir/op/contrib/sort.cc:50-139) are generated loops over the device functions cinn_nvgpu_lt_num_* /
+ * cinn_nvgpu_gt_num_* and cinn_nvgpu_next_smallest_int32 (cinn_cuda_runtime_source.cuh:645-715), whose second step
+ * mutates one shared buffer from every thread.  This call gives the result that algorithm defines when run in order -
+ * the stable order by (count of smaller elements, index); descending: count of larger elements - without shared
+ * state.  The tensor is [outer][size][inner], sorted along `size`.  outputs: bit 0 = int32 indices, bit 1 = int32
+ * positions (the count of smaller / larger elements of every element, the reference's second `argsort` output before
+ * its second step consumes it), bit 2 = sorted values (the input's type); v_args = {x, then the requested outputs in
+ * that order}.  fp16 / bf16 / fp32 / fp64 / int32 / int64; at most 16384 (8-byte types: 10922) elements along the
+ * sorted axis. */
+void cinn_call_hip_argsort(void* v_args, int num_args, int outer, int size, int inner, int is_ascend, int outputs,
+                           void* stream);
+
 /* Gradients of the three calls above, with the reference's argument lists.  Gather-form kernels (one thread or block
  * per gradient element, fp32 accumulation), formats 0 = NCHW / [F][C][KH][KW] and 1 = NHWC / [F][KH][KW][C]; every result
  * is out = alpha * gradient + beta * out.

@@ -157,6 +157,24 @@ def argmax_by_argsort_i32(row, stride=1):
     return int(fn(_p(row), _L(row.size // stride), _L(stride)))
 
 
+def argsort(x, axis, is_ascend=True):
+    """(indices, positions, sorted) along `axis` by the reference's three loop nests.  Integers go through int64,
+    everything else (float16 / float32 / float64 values) through float64, which holds them exactly."""
+    x = np.asarray(x)
+    axis = axis % x.ndim
+    outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+    size = x.shape[axis]
+    inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    integer = np.issubdtype(x.dtype, np.integer)
+    wide = _c(x, np.int64 if integer else np.float64)
+    index = np.empty(x.shape, np.int32)
+    positions = np.empty(x.shape, np.int32)
+    out = np.empty(x.shape, wide.dtype)
+    fn = require().oracle_argsort_i64 if integer else require().oracle_argsort_f64
+    fn(_p(wide), _p(index), _p(positions), _p(out), _L(outer), _L(size), _L(inner), _I(1 if is_ascend else 0))
+    return index, positions, out.astype(x.dtype)
+
+
 # ---- config 3 -----------------------------------------------------------------------------------
 def matmul(a, b, trans_a=False, trans_b=False, alpha=1.0, beta=0.0, c=None, acc64=False, kind=None):
     """Row-major matmul.  float32 arrays; or uint16 bit patterns with kind='float16' / 'bfloat16'."""

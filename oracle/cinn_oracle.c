@@ -336,6 +336,46 @@ int32_t oracle_argmax_by_argsort_i32(const int32_t* x, long size, long stride) {
   return (int32_t)id;
 }
 
+/* argsort / sort along one axis of [outer][size][inner], the literal three loop nests of the reference
+ * (cinn/hlir/op/contrib/sort.cc:50-139; the generated host code is spelled out in sort_test.cc:96-124):
+ *   positions[k] = cinn_host_lt_num(x, size, x[k], offset, stride)   (gt_num when descending: the count of larger
+ *                  elements; host_intrinsics.cc:99-118 scan from the last element down, which changes nothing)
+ *   index[j]     = cinn_host_next_smallest_int32(positions, size, j, offset, stride) for j = 0 .. size - 1 in order:
+ *                  the first entry with the smallest value, which the call then overwrites with INT32_MAX
+ *                  (host_intrinsics.cc:67-79)
+ *   sorted[j]    = x[index[j]]
+ * `positions_out` receives the positions as computed by the first nest (the second nest consumes a copy).  Doubles
+ * carry fp32 / fp64 / 16-bit values exactly; int64 values beyond 2^53 are not meant for this helper. */
+#define ORACLE_ARGSORT(NAME, T)                                                                                         \
+  void NAME(const T* x, int32_t* index, int32_t* positions_out, T* sorted, long outer, long size, long inner,           \
+            int is_ascend) {                                                                                            \
+    int32_t* work = (int32_t*)malloc(sizeof(int32_t) * (size_t)(size > 0 ? size : 1));                                  \
+    for (long o = 0; o < outer; ++o)                                                                                    \
+      for (long i = 0; i < inner; ++i) {                                                                                \
+        const long offset = o * size * inner + i, stride = inner;                                                       \
+        for (long k = 0; k < size; ++k) {                                                                               \
+          const T num = x[offset + k * stride];                                                                         \
+          int32_t out = 0;                                                                                              \
+          for (long j = (size - 1) * stride + offset; j >= offset; j -= stride)                                         \
+            if (is_ascend ? x[j] < num : x[j] > num) out++;                                                             \
+          work[k] = out;                                                                                                \
+          if (positions_out) positions_out[offset + k * stride] = out;                                                  \
+        }                                                                                                               \
+        for (long slot = 0; slot < size; ++slot) {                                                                      \
+          long id = -1;                                                                                                 \
+          for (long k = 0; k < size; ++k)                                                                               \
+            if (id == -1 || work[k] < work[id]) id = k;                                                                 \
+          work[id] = 2147483647;                                                                                        \
+          if (index) index[offset + slot * stride] = (int32_t)id;                                                       \
+          if (sorted) sorted[offset + slot * stride] = x[offset + id * stride];                                         \
+        }                                                                                                               \
+      }                                                                                                                 \
+    free(work);                                                                                                         \
+  }
+ORACLE_ARGSORT(oracle_argsort_f64, double)
+ORACLE_ARGSORT(oracle_argsort_i64, int64_t)
+#undef ORACLE_ARGSORT
+
 /* ------------------------------------------------------------------------------------------------
  * Matmul, row-major: C[M,N] = alpha * op(A) * op(B) (+ beta * C), op = optional transpose.
  * pe::Matmul (cinn/hlir/pe/transform.cc:252-310): sum over ascending k, then multiplied by alpha when

@@ -192,6 +192,22 @@ def test_generated_source_idioms():
     assert re.search(r"if \(.*< 750\)", src)  # 3000 / 4 vectors
 
 
+def test_argsort_and_sort_shapes_types_and_lowering():
+    """argsort: two int32 outputs of the operand's shape (indices, positions); sort: the operand's type
+    (cinn/hlir/op/contrib/sort.cc:307-350).  Each is one library-call instruction."""
+    from cinn_amd.common import Float
+    b = NetBuilder("t")
+    x = b.create_input(Float(16), [4, 30, 6], "x")
+    index, positions = b.argsort(x, 1, False)
+    values = b.sort(x, -1)
+    assert index.shape() == [4, 30, 6] and positions.shape() == [4, 30, 6] and values.shape() == [4, 30, 6]
+    assert str(index.type()) == "int32" and str(positions.type()) == "int32" and str(values.type()) == "float16"
+    comp = compile_only(b, [index, positions, values])
+    assert comp.num_instructions() == 2
+    with pytest.raises(Exception, match="axis"):
+        b.sort(x, 3)
+
+
 def test_math_calls_are_mapped_to_the_device_library_by_operand_type():
     """Operators emit target-independent names; the extern-call pass picks cinn_hip_<name>_<type> from the type of the
     first argument (the reference's MapExternCall, cinn/optim/map_extern_call.cc:45-115)."""

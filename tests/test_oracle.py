@@ -238,6 +238,40 @@ def test_argmax_first_maximum_wins_and_matches_argsort_definition(rng):
     assert np.array_equal(oracle.argmax_last(f), f.argmax(1).astype(np.int32))
 
 
+def test_argsort_is_the_stable_order_and_sort_gathers_it(rng):
+    """The three loop nests of the reference's argsort / sort against numpy's stable argsort: ascending directly;
+    descending is the stable order of the negated values (ties keep ascending indices either way, because
+    next_smallest takes the first of equal positions).  Values from a tiny range give many ties."""
+    for shape, axis in [((7, 33), 1), ((7, 33), 0), ((3, 5, 4), 1), ((2, 3, 4, 5), -1), ((1, 1), 0), ((6, 1, 9), 2)]:
+        for make in (lambda: rng.integers(-3, 3, shape).astype(np.int32), lambda: rng.standard_normal(shape).astype(np.float32),
+                     lambda: rng.integers(-2, 2, shape).astype(np.float32)):
+            x = make()
+            for ascend in (True, False):
+                index, positions, out = oracle.argsort(x, axis, ascend)
+                want = np.argsort(x if ascend else -x.astype(np.float64), axis=axis, kind="stable")
+                assert np.array_equal(index, want.astype(np.int32))
+                assert np.array_equal(out, np.take_along_axis(x, want, axis))
+                # positions: the count of strictly smaller (larger) elements along the axis, by brute force
+                xm = np.moveaxis(x, axis, -1)
+                less = (xm[..., None, :] < xm[..., :, None]) if ascend else (xm[..., None, :] > xm[..., :, None])
+                assert np.array_equal(np.moveaxis(positions, axis, -1), less.sum(-1).astype(np.int32))
+
+
+def test_argsort_with_nans_follows_the_position_rule():
+    """No comparison with a NaN is true, so a NaN has position 0 and counts for nobody: it shares position 0 with the
+    row's extreme value and they come out in index order.  Worked by hand from the loop nests:
+    [2, nan, 1, nan] ascending: positions 1 0 0 0 -> indices 1 2 3 0; descending: positions 0 0 1 0 -> 0 1 3 2."""
+    x = np.array([[2, np.nan, 1, np.nan]], np.float32)
+    index, positions, out = oracle.argsort(x, 1, True)
+    assert index.tolist() == [[1, 2, 3, 0]] and positions.tolist() == [[1, 0, 0, 0]]
+    assert np.array_equal(out, x[:, [1, 2, 3, 0]], equal_nan=True)
+    index, positions, _ = oracle.argsort(x, 1, False)
+    assert index.tolist() == [[0, 1, 3, 2]] and positions.tolist() == [[0, 0, 1, 0]]
+    # -0.0 and +0.0 are equal: a tie, kept in index order
+    z = np.array([[0.0, -0.0, -1.0, 0.0]], np.float32)
+    assert oracle.argsort(z, 1, True)[0].tolist() == [[2, 0, 1, 3]]
+
+
 # ---- matmul ---------------------------------------------------------------------------------------
 @pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
 def test_matmul_fp32_vs_float64(rng, ta, tb):
