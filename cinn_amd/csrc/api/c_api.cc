@@ -96,6 +96,9 @@ const std::map<std::string, Method>& Methods() {
     m["Sort"] = [](NetBuilder& b, const std::vector<Variable>& in, const AttributeMap& a) {
       return std::vector<Variable>{b.Sort(in.at(0), GetAttr<int>(a, "axis", 0), GetAttr<bool>(a, "is_ascend", true))};
     };
+    m["TopK"] = [](NetBuilder& b, const std::vector<Variable>& in, const AttributeMap& a) {
+      return b.TopK(in.at(0), GetAttr<int>(a, "k", 1), GetAttr<int>(a, "axis", -1), GetAttr<bool>(a, "largest", true));
+    };
     m["Select"] = [](NetBuilder& b, const std::vector<Variable>& in, const AttributeMap&) {
       return std::vector<Variable>{b.Select(in.at(0), in.at(1), in.at(2))};
     };

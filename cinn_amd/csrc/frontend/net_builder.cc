@@ -177,6 +177,17 @@ Variable NetBuilder::Sort(const Variable& operand, const int& axis, const bool& 
   return CustomInstr("sort", {operand}, {{"axis", axis}, {"is_ascend", is_ascend}}).front();
 }
 
+std::vector<Variable> NetBuilder::TopK(const Variable& x, int k, int axis, bool largest) {
+  (void)largest;
+  CINN_CHECK_GT(k, 0) << "The attribute k must be greater than 0.";
+  if (axis < 0) axis += static_cast<int>(x->shape.size());
+  CINN_CHECK(axis >= 0 && axis < static_cast<int>(x->shape.size())) << "top_k: axis out of range";
+  CINN_CHECK_LE(k, x->shape[axis]) << "top_k: k exceeds the extent of the axis";
+  Variable values  = Slice(Sort(x, axis, false), {axis}, {0}, {k});
+  Variable indices = Cast(Slice(ArgSort(x, axis, false).at(0), {axis}, {0}, {k}), "int64");
+  return {values, indices};
+}
+
 Variable NetBuilder::BroadcastTo(const Variable& x, const ShapeType& out_shape) {
   // numpy alignment: the operand's dimensions map onto the trailing output dimensions
   auto x_rank = x->shape.size();

@@ -72,6 +72,10 @@ class NetBuilder {
   // cinn/frontend/net_builder.h:1028-1046: {indices, positions} resp. the sorted values, both of the operand's shape
   std::vector<Variable> ArgSort(const Variable& operand, const int& axis, const bool& is_ascend = true);
   Variable Sort(const Variable& operand, const int& axis, const bool& is_ascend = true);
+  // {values, int64 indices} of the k largest entries along `axis`, as the reference's decomposer composes them
+  // (cinn/frontend/decomposer/top_k.cc:22-47: descending sort / argsort, slice, cast); like there, `largest` is
+  // accepted and not consulted
+  std::vector<Variable> TopK(const Variable& x, int k, int axis, bool largest);
 
   // ---- shape manipulation -----------------------------------------------------------------------
   Variable BroadcastTo(const Variable& x, const utils::ShapeType& out_shape);

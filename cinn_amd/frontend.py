@@ -163,6 +163,11 @@ class NetBuilder(object):
     def sort(self, x, axis, is_ascend=True):
         return self._call1("Sort", [x], axis=axis, is_ascend=is_ascend)
 
+    def top_k(self, x, k, axis=-1, largest=True):
+        """[values, int64 indices] of the k largest entries along `axis` (cinn/frontend/decomposer/top_k.cc:22-47,
+        where - as here - `largest` is not consulted)."""
+        return self._call("TopK", [x], k=int(k), axis=int(axis), largest=bool(largest))
+
     def broadcast_to(self, x, out_shape, broadcast_axes=None):
         if broadcast_axes is None:
             return self._call1("BroadcastTo", [x], out_shape=list(out_shape))

@@ -136,3 +136,21 @@ def test_argsort_at_the_reduce_configuration_size(gpu):
     assert np.array_equal(got_values, np.take_along_axis(x, want, 1))
     assert np.array_equal(np.sort(got_index, axis=1), np.broadcast_to(np.arange(512, dtype=np.int32), x.shape))
     assert np.array_equal(got_index[:, 0], x.argmax(1).astype(np.int32))  # element 0 is the reference's argmax
+
+
+def test_top_k_is_the_reference_composition(gpu):
+    """top_k = slice(sort descending), int64(slice(argsort descending)) (cinn/frontend/decomposer/top_k.cc:22-47).  The
+    reference's own test checks it against a plain top-k of the largest entries whatever `largest` says
+    (python/tests/ops/test_top_k_op.py:44), so both settings give the largest k here as well."""
+    rng = np.random.default_rng(8)
+    x = rng.integers(-6, 6, (7, 40, 3)).astype(np.float32)
+    for largest in (True, False):
+        b = NetBuilder("s")
+        v = b.create_input(Float(32), list(x.shape), "x")
+        values, indices = b.top_k(v, 5, 1, largest)
+        (got_values, got_indices), _ = run(b, {v: x}, [values, indices])
+        order, _, ordered = oracle.argsort(x, 1, False)
+        assert got_indices.dtype == np.int64 and got_values.shape == (7, 5, 3)
+        assert np.array_equal(got_indices, order[:, :5, :].astype(np.int64))
+        assert np.array_equal(got_values, ordered[:, :5, :])
+        assert np.array_equal(got_values[:, 0, :], x.max(1))
