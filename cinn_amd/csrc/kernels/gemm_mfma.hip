@@ -1044,6 +1044,88 @@ gemm16_shortk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict_
 }
 
 // ---------------------------------------------------------------------------------------------------
+// Few rows (M <= 64: a classifier at inference batch sizes, a decoding step): C[M][N] = A[M][K] . B[N][K]^T is bound by
+// one pass over B.  The tiled kernels give such a product M-tiles that are mostly padding and a handful of blocks; here
+// a block owns 16 output columns and its eight wavefronts split K.  A lane's share of a 16x16x32 fragment is 8
+// consecutive k of one row - 16 contiguous bytes in both operands - so fragments come straight from global memory, no
+// LDS on the way: every wavefront keeps U k-blocks of loads in flight (two register sets), B is read exactly once
+// from memory, A (at most 64 rows) comes out of L2.  The eight partial tiles meet in LDS; wavefront t finishes row
+// tile t (scale / shift, residual, relu - the epilogue of gemm16_dma_kernel - then 2-byte stores: the result is small).
+template <typename T, int MT>
+__global__ void __launch_bounds__(512)
+gemm16_skinny_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ C, int M, int N,
+                     int K, DmaEpilogue epi) {
+  typedef typename Half16<T>::vec8 vec8;
+  constexpr int NWAVES = 8;
+  constexpr int U      = 4;  // k-blocks per register set
+  __shared__ __attribute__((aligned(16))) float s_part[NWAVES][MT][64][4];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n0   = blockIdx.x * 16;
+  const int fr   = lane & 15;        // row of the fragment this lane reads (a row of A, a column of C for B)
+  const int fk   = (lane >> 4) * 8;  // its 8 elements of a 32-deep k block
+  const int kw   = K / NWAVES;       // this wavefront's share of K, a multiple of 32
+  const int nkb  = kw / 32;
+  const int bcol = min(n0 + fr, N - 1);
+  const uint16_t* bp = B + (int64_t)bcol * K + wave * kw + fk;
+  const uint16_t* ap[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) ap[t] = A + (int64_t)min(t * 16 + fr, M - 1) * K + wave * kw + fk;
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  vec8 bf[2][U], af[2][U][MT];
+  auto request = [&](int set, int kb0) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kb = min(kb0 + u, nkb - 1);  // beyond the share: the last block again, not multiplied
+      bf[set][u]   = *reinterpret_cast<const vec8*>(bp + kb * 32);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) af[set][u][t] = *reinterpret_cast<const vec8*>(ap[t] + kb * 32);
+    }
+  };
+  auto multiply = [&](int set, int kb0) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (kb0 + u < nkb) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[t] = Half16<T>::mfma16(af[set][u][t], bf[set][u], acc[t]);
+      }
+  };
+  request(0, 0);
+  for (int kb0 = 0; kb0 < nkb; kb0 += 2 * U) {
+    if (kb0 + U < nkb) request(1, kb0 + U);
+    multiply(0, kb0);
+    if (kb0 + 2 * U < nkb) request(0, kb0 + 2 * U);
+    multiply(1, kb0 + U);
+  }
+#pragma unroll
+  for (int t = 0; t < MT; ++t) *reinterpret_cast<f32x4*>(&s_part[wave][t][lane][0]) = acc[t];
+  __syncthreads();
+  if (wave >= MT) return;
+  // wavefront t: row tile t.  Lane = (column n0 + lane % 16, rows 16 t + 4 (lane / 16) .. + 3)
+  f32x4 sum = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int w = 0; w < NWAVES; ++w) sum += *reinterpret_cast<const f32x4*>(&s_part[w][wave][lane][0]);
+  const int col = n0 + fr;
+  if (col >= N) return;
+  const float sc = epi.scale ? epi.scale[col] : epi.alpha;
+  const float sh = epi.shift ? epi.shift[col] : 0.0f;
+  T* Ct          = reinterpret_cast<T*>(C);
+  const T* Rt    = reinterpret_cast<const T*>(epi.residual);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int row = wave * 16 + 4 * (lane >> 4) + r;
+    if (row >= M) continue;
+    float v = __builtin_fmaf(sum[r], sc, sh);
+    if (Rt) v = __builtin_fmaf(epi.residual_scale, (float)Rt[(int64_t)row * N + col], v);
+    asm volatile("" : "+v"(v));  // one rounding to T, see gemm16_dma_kernel's epilogue
+    if (epi.relu) v = v > 0.0f ? v : 0.0f;
+    Ct[(int64_t)row * N + col] = (T)v;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------
 // fp32 on v_mfma_f32_32x32x2f32: 128x128 (or 64x64) tile, K step KS = 32 or 64, 4 wavefronts each a quarter of the tile.
 // LDS holds A as [k][m] and B as [k][n] (row stride TILE + 4 floats) so that a fragment read is one conflict-free
 // ds_read_b32 per lane; the K step is deep enough (16 MFMAs of 64 clocks per accumulator) to cover the latency of
@@ -1523,6 +1605,40 @@ bool TryShortK(const GemmProblem& p, hipStream_t stream) {
   return true;
 }
 
+// gemm16_skinny_kernel: at most 64 rows, A [M][K] and B stored [N][K] (a const weight after the program pass has
+// transposed it), one unbatched product, K a multiple of 256 (eight wavefronts of 32-deep blocks).
+// FLAGS_cinn_hip_gemm_skinny=0 switches it off.
+template <typename T>
+bool TrySkinny(const GemmProblem& p, hipStream_t stream) {
+  static const bool enabled = !(getenv("FLAGS_cinn_hip_gemm_skinny") && atoi(getenv("FLAGS_cinn_hip_gemm_skinny")) == 0);
+  if (!enabled || p.conv || p.trans_a || !p.trans_b || p.batch != 1) return false;
+  if (p.m > 64 || p.k % 256 != 0 || (int64_t)p.n * p.k >= INT_MAX) return false;
+  if (reinterpret_cast<uintptr_t>(p.a) % 16 != 0 || reinterpret_cast<uintptr_t>(p.b) % 16 != 0) return false;
+  DmaEpilogue epi;
+  epi.partials        = nullptr;
+  epi.steps_per_split = 0;
+  epi.scale           = p.scale;
+  epi.shift           = p.shift;
+  epi.alpha           = p.alpha;
+  epi.relu            = p.relu ? 1 : 0;
+  epi.residual        = p.residual ? p.residual : (p.beta != 0.0f ? p.c : nullptr);
+  epi.residual_scale  = p.residual ? p.residual_scale : p.beta;
+  epi.streaming       = 0;
+  const dim3 grid((unsigned)((p.n + 15) / 16));
+  const int mt = (p.m + 15) / 16;
+#define CINN_SKINNY(MT)                                                                                        \
+  hipLaunchKernelGGL((gemm16_skinny_kernel<T, MT>), grid, dim3(512), 0, stream, static_cast<const uint16_t*>(p.a), \
+                     static_cast<const uint16_t*>(p.b), static_cast<uint16_t*>(p.c), p.m, p.n, p.k, epi)
+  switch (mt) {
+    case 1: CINN_SKINNY(1); break;
+    case 2: CINN_SKINNY(2); break;
+    case 3: CINN_SKINNY(3); break;
+    default: CINN_SKINNY(4); break;
+  }
+#undef CINN_SKINNY
+  return true;
+}
+
 // FLAGS_cinn_hip_gemm_feed=0: the four-stage 128x128 instances issue their loads from the computing wavefronts
 bool FeedWavefronts() {
   static const bool on = !(getenv("FLAGS_cinn_hip_gemm_feed") && atoi(getenv("FLAGS_cinn_hip_gemm_feed")) == 0);
@@ -1534,6 +1650,7 @@ bool FeedWavefronts() {
 // tile (the last tile row / column computes some rows / columns that are not stored); false when neither applies
 template <typename T>
 bool TryDma16(const GemmProblem& p, hipStream_t stream) {
+  if (TrySkinny<T>(p, stream)) return true;
   if (p.trans_a || p.k % 64 != 0 || p.n % 8 != 0) return false;
   if (TryShortK<T>(p, stream)) return true;
   // every access moves 16 bytes

@@ -144,6 +144,39 @@ def test_16bit_direct_to_lds_kernel(gpu, kind, tb, alpha, beta, batch, m, n, k):
     assert np.all(np.abs(got - exact) <= ulp * np.maximum(np.abs(exact), 1e-3 * scale) + 2.0 ** -24)
 
 
+@pytest.mark.parametrize("kind", ["float16", "bfloat16"])
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (0.5, 2.0)])
+@pytest.mark.parametrize("m,n,k", [(32, 1000, 2048),   # the classifier of a batch of 32: 63 blocks, the last one 8 columns wide
+                                   (1, 4096, 4096),    # one row: a decoding step
+                                   (64, 520, 256),     # four row tiles, one k block per wavefront
+                                   (17, 8, 512),       # ragged rows, a single block of 8 columns
+                                   (48, 24, 768),      # three row tiles
+                                   (5, 3, 8192),       # long K: both register sets of every wavefront in use; 3 columns
+                                   (33, 136, 4352)])   # 17 k blocks per wavefront: a set that is only partly multiplied
+def test_16bit_products_with_few_rows(gpu, kind, alpha, beta, m, n, k):
+    """gemm16_skinny_kernel: at most 64 rows, B stored [N][K], K a multiple of 256 - one block per 16 columns, K split
+    over its wavefronts, fragments straight from global memory.  Same bar as the tiled kernels: fp32 accumulation and
+    epilogue, one rounding to the 16-bit type."""
+    rng = np.random.default_rng(m * 7 + n + k)
+    a = (rng.standard_normal((m, k)) * 0.05).astype(np.float32)
+    b = (rng.standard_normal((n, k)) * 0.05).astype(np.float32)
+    c0 = rng.standard_normal((m, n)).astype(np.float32)
+    if kind == "float16":
+        ab, bb, cb = a.astype(np.float16), b.astype(np.float16), c0.astype(np.float16)
+        af, bf, cf = ab.astype(np.float64), bb.astype(np.float64), cb.astype(np.float64)
+        got = call_cublas(ab, bb, (m, n), kind, False, True, alpha=alpha, beta=beta, c_init=cb).astype(np.float64)
+        ulp = 2.0 ** -10
+    else:
+        ab, bb, cb = float32_to_bfloat16_bits(a), float32_to_bfloat16_bits(b), float32_to_bfloat16_bits(c0)
+        af, bf, cf = (bfloat16_bits_to_float32(x).astype(np.float64) for x in (ab, bb, cb))
+        got = bfloat16_bits_to_float32(
+            call_cublas(ab, bb, (m, n), kind, False, True, alpha=alpha, beta=beta, c_init=cb)).astype(np.float64)
+        ulp = 2.0 ** -7
+    exact = alpha * (af @ bf.T) + beta * cf
+    scale = abs(alpha) * (np.abs(af) @ np.abs(bf.T)) + abs(beta) * np.abs(cf)
+    assert np.all(np.abs(got - exact) <= ulp * np.maximum(np.abs(exact), 1e-3 * scale) + 2.0 ** -24)
+
+
 @pytest.mark.parametrize("tb", [False, True])
 @pytest.mark.parametrize("m,n", [(4096, 3072), (1536, 1536)])
 @pytest.mark.parametrize("k", [64, 192, 448])
