@@ -407,7 +407,7 @@ constexpr int kRing       = kTaps;  // filter stages in the chunked kernel's rin
 // 1 .. 8, issued in that order before the loop (after the first patch and stage 0, and without patch loads between
 // them).  At tap 8 of a chunk that is not the last, the next chunk's patch must have landed as well: only the stages
 // issued after the last patch load may be in flight.
-__device__ __forceinline__ constexpr int ChunkLoadsInFlight(int t, bool first, bool last, int pl, int l) {
+__host__ __device__ __forceinline__ constexpr int ChunkLoadsInFlight(int t, bool first, bool last, int pl, int l) {
   int n = 0;
   for (int u = t - (kRing - 2); u < t; ++u) {
     const bool before = u < 0;  // a step of the previous chunk, or a stage fetched before the loop
@@ -781,6 +781,10 @@ bool TryConvPatch(const ConvNhwcArgs& a, hipStream_t stream) {
 }
 
 }  // namespace cinn_hip_kernels
+
+extern "C" int cinn_hip_conv_patch_loads_in_flight(int tap, int first_chunk, int last_chunk, int patch_loads_per_step) {
+  return cinn_hip_kernels::ChunkLoadsInFlight(tap, first_chunk != 0, last_chunk != 0, patch_loads_per_step, 64 / 8 / cinn_hip_kernels::kWaves);
+}
 
 extern "C" int cinn_hip_conv_patch_mode(int mode) {
   const int before = cinn_hip_kernels::PatchMode();

@@ -318,6 +318,10 @@ int cinn_hip_scratch_release_retired(void);
  * qualifies.  Returns the previous mode; any other argument only reads it.  No counterpart in the reference (cuDNN picks
  * its algorithm inside cudnnConvolutionForward, cinn/runtime/cuda/cuda_util.cc:560-640); a tuning and test switch. */
 int cinn_hip_conv_patch_mode(int mode);
+/* For tests of the chunked kernel's synchronisation: the `s_waitcnt vmcnt` count a feeding wavefront uses before the
+ * barrier of K step (chunk, tap) - how many of its loads may still be in flight while the next filter stage (and, at
+ * tap 8, the next chunk's patch) is known to have landed.  Host-side evaluation of the kernel's own constexpr. */
+int cinn_hip_conv_patch_loads_in_flight(int tap, int first_chunk, int last_chunk, int patch_loads_per_step);
 
 /* Device descriptor consumed by schedules.  Replaces common::Target's cudaDeviceGetAttribute
  * queries (cinn/common/target.cc:55-84, 177-221).  Filled from the live device when one is

@@ -261,3 +261,36 @@ def test_device_library_defines_the_reference_spellings():
            "\n  out[threadIdx.x] = acc;\n}\n")
     image = runtime.rtc_compile(src)
     assert image[:4] == b"\x7fELF"
+
+
+def test_chunked_patch_kernel_wait_counts_match_a_simulation_of_its_issue_order():
+    """conv3x3_patch_chunks_kernel's feeding wavefronts wait with `s_waitcnt vmcnt(n)` before every barrier: loads
+    complete in issue order, so "at most n in flight" means that everything issued earlier than the last n loads has
+    landed.  n comes from a closed formula in the kernel; here the issue order is replayed load by load (the first
+    patch, the nine stages of chunk 0, then per K step the next chunk's patch loads and the stage nine steps ahead) and
+    the exact largest safe n is counted at every barrier.  The formula may never exceed it (a race), and equals it."""
+    lib = _lib.load()
+    lib.cinn_hip_conv_patch_loads_in_flight.argtypes = [ctypes.c_int] * 4
+    lib.cinn_hip_conv_patch_loads_in_flight.restype = ctypes.c_int
+    taps, ring, patch_steps, stage_loads = 9, 9, 4, 2
+    for chunks in range(2, 7):
+        for per_step in (2, 3):
+            log = [("patch", 0)] * (per_step * patch_steps)
+            for st in range(ring):
+                log += [("stage", st)] * stage_loads
+            for c in range(chunks):
+                last = c == chunks - 1
+                for t in range(taps):
+                    if last and t == taps - 1:
+                        break  # the last K step has no barrier
+                    s = c * taps + t
+                    needed = [("stage", s + 1)] + ([("patch", c + 1)] if (not last and t == taps - 1) else [])
+                    newest = max(max(i for i, e in enumerate(log) if e == what) for what in needed)
+                    exact = len(log) - 1 - newest
+                    got = lib.cinn_hip_conv_patch_loads_in_flight(t, int(c == 0), int(last), per_step)
+                    assert got == exact, (chunks, per_step, c, t, got, exact)
+                    assert got <= 40  # the kernel's table of s_waitcnt immediates
+                    if not last:
+                        if t < patch_steps:
+                            log += [("patch", c + 1)] * per_step
+                        log += [("stage", s + ring)] * stage_loads
