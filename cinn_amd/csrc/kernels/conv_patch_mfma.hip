@@ -398,18 +398,24 @@ struct BoolTag {
 
 constexpr int kPatchSteps = 4;  // K steps of a chunk after whose barriers the feeding wavefronts fetch patch loads
 constexpr int kRing       = kTaps;  // filter stages in the chunked kernel's ring: the slot of a stage is its tap
+constexpr int kChunkStagesAhead = 2;  // a stage has landed this many K steps before the step that multiplies with it
 
-// Loads a feeding wavefront of the chunked kernel may still have in flight when it arrives at the barrier of K step
-// (chunk, tap t): everything it issued after filter stage s + 1, which must have landed.  After the barrier of a step u
-// it issues pl patch loads (taps below kPatchSteps of a chunk that is not the last) and then the l loads of stage
-// u + kRing (while that stage exists, i.e. in chunks that are not the last); stage s + 1 was issued after barrier
-// s + 1 - kRing, so the steps s - 7 .. s - 1 count.  In the first chunk the steps before step 0 stand for the stages
-// 1 .. 8, issued in that order before the loop (after the first patch and stage 0, and without patch loads between
-// them).  At tap 8 of a chunk that is not the last, the next chunk's patch must have landed as well: only the stages
-// issued after the last patch load may be in flight.
-__host__ __device__ __forceinline__ constexpr int ChunkLoadsInFlight(int t, bool first, bool last, int pl, int l) {
+// Loads a feeding wavefront of the chunked kernel may still have in flight when it arrives at the barrier that closes
+// K step (chunk, tap t): everything it issued after filter stage s + ahead, which must have landed (the computing
+// wavefronts read a stage's fragments one step before they multiply with them, so ahead = 2).  After the barrier of a
+// step u the wavefront issues pl patch loads (taps below kPatchSteps of a chunk that is not the last) and then the l
+// loads of stage u + kRing (while that stage exists, i.e. in chunks that are not the last); stage s + ahead was issued
+// after barrier s + ahead - kRing, so the steps from there to s - 1 count.  In the first chunk the steps before step 0
+// stand for the stages issued before the loop, in order and without patch loads between them.  At the last barrier
+// before the computing wavefronts touch the next chunk's patch (tap 9 - ahead of a chunk that is not the last) that
+// patch must have landed as well: only the stages issued after the last patch load may be in flight.  In the last
+// chunk a stage beyond its tap 8 does not exist: the count is the one for the last stage that does.
+__host__ __device__ __forceinline__ constexpr int ChunkLoadsInFlight(int t, bool first, bool last, int pl, int l,
+                                                                     int ahead = kChunkStagesAhead) {
+  if (last && t + ahead > kTaps - 1) ahead = kTaps - 1 - t;
+  if (ahead <= 0) return 0;
   int n = 0;
-  for (int u = t - (kRing - 2); u < t; ++u) {
+  for (int u = t - (kRing - 1 - ahead); u < t; ++u) {
     const bool before = u < 0;  // a step of the previous chunk, or a stage fetched before the loop
     const int tap     = before ? u + kTaps : u;
     if (before && first) {
@@ -418,37 +424,40 @@ __host__ __device__ __forceinline__ constexpr int ChunkLoadsInFlight(int t, bool
       n += (tap < kPatchSteps ? pl : 0) + l;
     }
   }
-  if (!last && t == kTaps - 1) {
-    const int after_patch = (kTaps - kPatchSteps) * l;
+  const int patch_tap = kTaps - ahead;
+  if (!last && t == patch_tap) {
+    const int after_patch = (patch_tap - (kPatchSteps - 1)) * l;
     n                     = n < after_patch ? n : after_patch;
   }
   return n;
 }
 
-// C = 64 * chunks input channels.  TMW: 16-pixel tiles per computing wavefront (the block holds 64 TMW pixels of one
-// band); PL: patch loads a feeding wavefront issues per K step, so a chunk's patch is at most 4 * kPatchSteps * PL KiB.
+// C = 64 * chunks input channels.  TMW: 16-slot tiles per computing wavefront (the block holds 64 TMW pixel slots of
+// one band: 4 for 256, or 2 for 128 where larger blocks would be too few); PL: patch loads a feeding wavefront issues
+// per K step, so a chunk's patch is at most 4 * kPatchSteps * PL KiB.
 // LDS: a ring of nine filter stages (a whole chunk: the slot of a stage is its tap, and a stage is requested eight K
-// steps before its use - the filters of a layer are read once per launch and XCD, from memory rather than from L2, and
-// with the two steps of lead that suffice for the single-chunk kernel's 72 KiB filter every step waited for its
-// loads), then two patch buffers of patch_loads KiB each.  At least two chunks.  The loop starts as soon as the first
-// patch and stage 0 have landed.
+// steps before its use - the filters of a layer are read once per launch and XCD, from memory rather than from L2),
+// then two patch buffers of patch_loads KiB each.  At least two chunks.  The loop starts as soon as the first patch
+// and the stages 0 and 1 have landed.
 //
-// Order of events around the barrier of K step s = 9 c + t (one per step but the last, after MFMA row RB of the step):
-//   computing wavefronts   every fragment of filter stage s is in registers before it; after it they read the first
-//                          fragments of stage s + 1 and, in step t = 8, of the next chunk's patch;
-//   feeding wavefronts     before it: stage s + 1 has landed and, at t = 8, the next chunk's patch (loads complete in
+// A K step (one tap of one chunk) is 2 TMW rows of four MFMAs - 256 clocks with two tiles, less than an LDS read
+// takes to return under load - so the filter fragments of a step are read during the step before it, into one of
+// three register sets (the tap modulo 3: an immediate whatever the chunk); pixel fragments sit in a ring of four,
+// requested three rows ahead.  One barrier closes every step s = 9 c + t but the last:
+//   computing wavefronts   have multiplied with every fragment of stage s before it (its slot may be refilled); after
+//                          it they read the fragments of stage s + 2 during step s + 1, and in the last rows of
+//                          step t = 8 the first pixel fragments of the next chunk's patch;
+//   feeding wavefronts     before it: stage s + 2 has landed and, at t = 7, the next chunk's patch (loads complete in
 //                          order: ChunkLoadsInFlight counts what was issued later and may still be in flight); after
 //                          it: PL patch loads of chunk c + 1 (steps t < kPatchSteps; the buffer was last read in step
-//                          9 c - 1, whose MFMAs everyone has issued before barrier 9 c), then stage s + 9 into the
-//                          slot of stage s.
+//                          9 c - 1, which its barrier has closed), then stage s + 9 into the slot of stage s.
 template <typename T, int TMW, int PL>
 __global__ void __launch_bounds__(128 * kWaves) conv3x3_patch_chunks_kernel(PatchParams p) {
-  constexpr int L   = 64 / 8 / kWaves;       // 1 KiB filter loads per feeding wavefront and stage
-  constexpr int NPL = PL * kPatchSteps;       // patch loads per feeding wavefront and chunk
-  constexpr int R   = 2 * TMW;                // MFMA rows (of four) per K step
-  constexpr int RB  = TMW > 2 * TMW - 5 ? TMW : 2 * TMW - 5;  // the barrier follows this row
-  constexpr int NB  = TMW < 6 ? RB + 1 : RB + 2;              // rows NB, NB + 1 request the next stage's slice 0
-  static_assert(TMW >= 4 && NB + 1 < R, "the schedule of a K step needs at least eight rows");
+  constexpr int L     = 64 / 8 / kWaves;     // 1 KiB filter loads per feeding wavefront and stage
+  constexpr int NPL   = PL * kPatchSteps;     // patch loads per feeding wavefront and chunk
+  constexpr int R     = 2 * TMW;              // MFMA rows (of four) per K step
+  constexpr int AHEAD = kChunkStagesAhead;
+  static_assert(TMW % 2 == 0 && TMW >= 2, "the ring of four pixel fragments wants an even number of tiles");
   typedef typename Mfma16<T>::vec8 vec8;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   char* const ring  = lds;
@@ -520,11 +529,11 @@ __global__ void __launch_bounds__(128 * kWaves) conv3x3_patch_chunks_kernel(Patc
 #pragma unroll
       for (int t = 0; t < L; ++t) AsyncCopy16(w0 + b_off[t], lds_addr + slot * kBTile + (f * L + t) * 1024);
     };
-    // the first patch and stage 0 are all the first K step needs; the stages 1 .. 8 land while it runs
+    // the first patch and the stages 0 and 1 are all the first K step needs; the other stages land while it runs
     issue_patch(0, NPL, patch_addr);
 #pragma unroll
     for (int st = 0; st < kRing; ++st) issue_stage(st, 0, st);
-    WaitLoadsInFlight((kRing - 1) * L);
+    WaitLoadsInFlight((kRing - AHEAD) * L);
     BarrierLds();
     auto feed_chunk = [&](auto first_tag, auto last_tag, int c) {
       constexpr bool FIRST = decltype(first_tag)::value;
@@ -532,7 +541,7 @@ __global__ void __launch_bounds__(128 * kWaves) conv3x3_patch_chunks_kernel(Patc
       const unsigned next_buffer = patch_addr + ((c + 1) & 1) * patch_bytes;
 #pragma unroll
       for (int t = 0; t + (LAST ? 1 : 0) < kTaps; ++t) {
-        WaitLoadsInFlight(ChunkLoadsInFlight(t, FIRST, LAST, PL, L));
+        WaitLoadsInFlight(ChunkLoadsInFlight(t, FIRST, LAST, PL, L, AHEAD));
         BarrierLds();
         if (!LAST) {
           if (t < kPatchSteps) issue_patch(t * PL, PL, next_buffer);
@@ -583,59 +592,64 @@ __global__ void __launch_bounds__(128 * kWaves) conv3x3_patch_chunks_kernel(Patc
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-  // A K step is R rows of 4 MFMAs: row r multiplies the pixel fragment of tile r % TMW, slice r / TMW, with the four
-  // filter fragments of that slice.  Pixel fragments are requested three rows ahead, across the ends of steps and of
-  // chunks; filter fragments: slice 1 in rows 0 and 1, the next stage's slice 0 in rows NB and NB + 1.
-  vec8 ar[TMW];
-  vec8 bf[2][4];
-  auto read_b = [&](int slot, int kk, int j) -> vec8 { return *reinterpret_cast<const vec8*>(b_base[kk][j] + slot * kBTile); };
-  BarrierLds();  // the first patch and the first filter stages are in LDS
-#pragma unroll
-  for (int r = 0; r < 3; ++r) ar[r] = *reinterpret_cast<const vec8*>(a_base[r]);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) bf[0][j] = read_b(0, 0, j);
 #define CINN_SB __builtin_amdgcn_sched_barrier(0)
-  // to_next: from tap (2, 0) of this chunk's buffer to tap (0, 0) of the other buffer
-  auto multiply_chunk = [&](auto last_tag, int to_next) {
-    constexpr bool LAST = decltype(last_tag)::value;
+  {
+    // Row r of a step multiplies the pixel fragment of tile r % TMW, slice r / TMW (ring entry r % 4) with the four
+    // filter fragments of that slice from the set of this tap.  After the first MFMA of a row the pixel fragment three
+    // rows on is requested, after its second and third MFMA two filter fragments of the NEXT tap (slice 0 first).
+    vec8 ar[4];
+    vec8 bf[3][2][4];
+    auto read_b = [&](int slot, int kk, int j) -> vec8 { return *reinterpret_cast<const vec8*>(b_base[kk][j] + slot * kBTile); };
+    auto row_base = [&](int q) -> const char* { return a_base[q % TMW] + (q / TMW) * 64; };  // row q of a step: tile, slice
+    BarrierLds();  // the first patch and the filter stages 0 and 1 are in LDS
 #pragma unroll
-    for (int kt = 0; kt < kTaps; ++kt) {
-      const bool has_next = !(LAST && kt + 1 == kTaps);
-      const int dx        = kt % 3;
-      const int next_dx   = dx == 2 ? 0 : dx + 1;
-      const int next_off  = kt + 1 == kTaps ? to_next : (dx == 2 ? row_pitch : 0);
+    for (int r = 0; r < 3; ++r) ar[r] = *reinterpret_cast<const vec8*>(row_base(r));
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
+    for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          CINN_SB;
-          acc[r % TMW][j] = Mfma16<T>::mma(bf[r / TMW][j], ar[r % TMW], acc[r % TMW][j]);
-          CINN_SB;
-          if (j == 0) {
-            if (r + 3 < R) {
-              ar[(r + 3) % TMW] = *reinterpret_cast<const vec8*>(a_base[(r + 3) % TMW] + dx * kPitch + ((r + 3) / TMW) * 64);
-            } else if (has_next) {
-              ar[r + 3 - R] = *reinterpret_cast<const vec8*>(a_base[r + 3 - R] + next_off + next_dx * kPitch);
+      for (int j = 0; j < 4; ++j) bf[0][kk][j] = read_b(0, kk, j);
+    auto multiply_chunk = [&](auto last_tag, int to_next) {
+      constexpr bool LAST = decltype(last_tag)::value;
+#pragma unroll
+      for (int kt = 0; kt < kTaps; ++kt) {
+        const bool has_next = !(LAST && kt + 1 == kTaps);
+        const int dx        = kt % 3;
+        const int next_dx   = dx == 2 ? 0 : dx + 1;
+        const int next_off  = kt + 1 == kTaps ? to_next : (dx == 2 ? row_pitch : 0);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            CINN_SB;
+            acc[r % TMW][j] = Mfma16<T>::mma(bf[kt % 3][r / TMW][j], ar[r % 4], acc[r % TMW][j]);
+            CINN_SB;
+            if (j == 0) {
+              if (r + 3 < R) {
+                ar[(r + 3) % 4] = *reinterpret_cast<const vec8*>(row_base(r + 3) + dx * kPitch);
+              } else if (has_next) {
+                ar[(r + 3) % 4] = *reinterpret_cast<const vec8*>(row_base(r + 3 - R) + next_off + next_dx * kPitch);
+              }
+            }
+            if ((j == 1 || j == 2) && r < 4 && has_next) {
+              const int f = r * 2 + j - 1;  // 0..7: slice f / 4, filter tile f % 4
+              bf[(kt + 1) % 3][f / 4][f % 4] = read_b((kt + 1) % kRing, f / 4, f % 4);
             }
           }
-          if ((j == 1 || j == 2) && r < 2) bf[1][r * 2 + j - 1] = read_b(kt, 1, r * 2 + j - 1);
-          if ((j == 1 || j == 2) && r >= NB && r < NB + 2 && has_next)
-            bf[0][(r - NB) * 2 + j - 1] = read_b((kt + 1) % kRing, 0, (r - NB) * 2 + j - 1);
         }
-        if (r == RB && has_next) {
+        if (has_next) {
           CINN_SB;
           BarrierLds();
         }
-      }
-      if (has_next && (dx == 2)) {
-        CINN_SB;
+        if (has_next && (dx == 2)) {
+          CINN_SB;
 #pragma unroll
-        for (int i = 0; i < TMW; ++i) a_base[i] += next_off;
+          for (int i = 0; i < TMW; ++i) a_base[i] += next_off;
+        }
       }
-    }
-  };
-  for (int c = 0; c + 1 < chunks; ++c) multiply_chunk(BoolTag<false>{}, ((c & 1) ? -patch_bytes : patch_bytes) - 2 * row_pitch);
-  multiply_chunk(BoolTag<true>{}, 0);
+    };
+    for (int c = 0; c + 1 < chunks; ++c) multiply_chunk(BoolTag<false>{}, ((c & 1) ? -patch_bytes : patch_bytes) - 2 * row_pitch);
+    multiply_chunk(BoolTag<true>{}, 0);
+  }
 #undef CINN_SB
 
   PatchEpilogue<T, TMW, true>(p, acc, ss, img, y0, n0, rows, WP, pix0, lane);
@@ -726,6 +740,20 @@ int PatchMode() {
   return mode;
 }
 
+// 0: chosen per shape, 2 / 4: 16-slot tiles per computing wavefront of the chunked kernel; -1: not read yet
+std::atomic<int> g_patch_tiles{-1};
+
+int PatchTiles() {
+  int tiles = g_patch_tiles.load(std::memory_order_relaxed);
+  if (tiles < 0) {
+    const char* v = getenv("FLAGS_cinn_hip_conv_patch_tiles");
+    tiles         = v && *v ? atoi(v) : 0;
+    if (tiles != 2 && tiles != 4) tiles = 0;
+    g_patch_tiles.store(tiles, std::memory_order_relaxed);
+  }
+  return tiles;
+}
+
 }  // namespace
 
 bool TryConvPatch(const ConvNhwcArgs& a, hipStream_t stream) {
@@ -742,11 +770,31 @@ bool TryConvPatch(const ConvNhwcArgs& a, hipStream_t stream) {
   if (reinterpret_cast<uintptr_t>(a.x) % 16 != 0 || reinterpret_cast<uintptr_t>(a.w) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(a.y) % 16 != 0 || reinterpret_cast<uintptr_t>(a.residual) % 16 != 0)
     return false;
-  constexpr int kChunksTMW = 4;
   const bool chunked = a.c != 64;
   int per_step       = 0;
+  int tiles          = 4;  // 16-slot tiles per computing wavefront of the chunked kernel
   PatchPlan plan;
-  if (!(chunked ? PlanChunksFor<kChunksTMW>(a, &plan, &per_step) : PlanFor(a, &plan))) return false;
+  if (chunked) {
+    // Blocks of 256 pixel slots; when those leave most of the chip idle (256 -> 256 on 14x14 at batch 32: 128 blocks)
+    // and blocks of 128 slots give more, the kernel with the schedule for short K steps takes them.
+    // FLAGS_cinn_hip_conv_patch_tiles=2|4 (or cinn_hip_conv_patch_tiles) forces one form.
+    const int forced_tiles = PatchTiles();
+    const bool fits4 = forced_tiles != 2 && PlanChunksFor<4>(a, &plan, &per_step);
+    const int64_t blocks4 = fits4 ? (int64_t)a.n * plan.bands * (a.oc / 64) : 0;
+    if (forced_tiles == 2 || (forced_tiles == 0 && blocks4 < 192)) {
+      PatchPlan plan2;
+      int per_step2 = 0;
+      if (PlanChunksFor<2>(a, &plan2, &per_step2) && per_step2 == 2 && (int64_t)a.n * plan2.bands * (a.oc / 64) > blocks4) {
+        plan = plan2, per_step = per_step2, tiles = 2;
+      } else if (!fits4) {
+        return false;
+      }
+    } else if (!fits4) {
+      return false;
+    }
+  } else if (!PlanFor(a, &plan)) {
+    return false;
+  }
   // one block per band, image and 64 output channels; below ~100 blocks most of the chip would idle and the
   // implicit-GEMM tiles are the better choice
   if (flag != 2 && (int64_t)a.n * plan.bands * (a.oc / 64) < 96) return false;
@@ -759,17 +807,23 @@ bool TryConvPatch(const ConvNhwcArgs& a, hipStream_t stream) {
   p.rows = plan.rows, p.bands = plan.bands, p.patch_loads = plan.patch_loads;
   MagicFor(chunked ? (a.w_in + 7) & ~7 : a.w_in, &p.w_magic, &p.w_shift);
   MagicFor(a.w_in + 2, &p.pw_magic, &p.pw_shift);
-  if (chunked && per_step == 2) {
+  if (chunked && tiles == 2) {
     if (is_bf16) {
-      LaunchChunks<__bf16, kChunksTMW, 2>(p, plan, stream);
+      LaunchChunks<__bf16, 2, 2>(p, plan, stream);
     } else {
-      LaunchChunks<_Float16, kChunksTMW, 2>(p, plan, stream);
+      LaunchChunks<_Float16, 2, 2>(p, plan, stream);
+    }
+  } else if (chunked && per_step == 2) {
+    if (is_bf16) {
+      LaunchChunks<__bf16, 4, 2>(p, plan, stream);
+    } else {
+      LaunchChunks<_Float16, 4, 2>(p, plan, stream);
     }
   } else if (chunked) {
     if (is_bf16) {
-      LaunchChunks<__bf16, kChunksTMW, 3>(p, plan, stream);
+      LaunchChunks<__bf16, 4, 3>(p, plan, stream);
     } else {
-      LaunchChunks<_Float16, kChunksTMW, 3>(p, plan, stream);
+      LaunchChunks<_Float16, 4, 3>(p, plan, stream);
     }
   } else if (is_bf16) {
     Launch<__bf16>(p, plan, stream);
@@ -784,6 +838,12 @@ bool TryConvPatch(const ConvNhwcArgs& a, hipStream_t stream) {
 
 extern "C" int cinn_hip_conv_patch_loads_in_flight(int tap, int first_chunk, int last_chunk, int patch_loads_per_step) {
   return cinn_hip_kernels::ChunkLoadsInFlight(tap, first_chunk != 0, last_chunk != 0, patch_loads_per_step, 64 / 8 / cinn_hip_kernels::kWaves);
+}
+
+extern "C" int cinn_hip_conv_patch_tiles(int tiles) {
+  const int before = cinn_hip_kernels::PatchTiles();
+  if (tiles == 0 || tiles == 2 || tiles == 4) cinn_hip_kernels::g_patch_tiles.store(tiles, std::memory_order_relaxed);
+  return before;
 }
 
 extern "C" int cinn_hip_conv_patch_mode(int mode) {

@@ -318,6 +318,10 @@ int cinn_hip_scratch_release_retired(void);
  * qualifies.  Returns the previous mode; any other argument only reads it.  No counterpart in the reference (cuDNN picks
  * its algorithm inside cudnnConvolutionForward, cinn/runtime/cuda/cuda_util.cc:560-640); a tuning and test switch. */
 int cinn_hip_conv_patch_mode(int mode);
+/* Block size of that kernel for more than 64 input channels: 4 or 2 tiles of 16 pixel slots per computing wavefront
+ * (256 or 128 slots per block); 0 = chosen per shape (2 when 4 would give fewer than 192 blocks and 2 gives more).
+ * Returns the previous setting; another value only reads it.  Initial value from FLAGS_cinn_hip_conv_patch_tiles. */
+int cinn_hip_conv_patch_tiles(int tiles);
 /* For tests of the chunked kernel's synchronisation: the `s_waitcnt vmcnt` count a feeding wavefront uses before the
  * barrier of K step (chunk, tap) - how many of its loads may still be in flight while the next filter stage (and, at
  * tap 8, the next chunk's patch) is known to have landed.  Host-side evaluation of the kernel's own constexpr. */

@@ -266,14 +266,17 @@ def test_device_library_defines_the_reference_spellings():
 def test_chunked_patch_kernel_wait_counts_match_a_simulation_of_its_issue_order():
     """conv3x3_patch_chunks_kernel's feeding wavefronts wait with `s_waitcnt vmcnt(n)` before every barrier: loads
     complete in issue order, so "at most n in flight" means that everything issued earlier than the last n loads has
-    landed.  n comes from a closed formula in the kernel; here the issue order is replayed load by load (the first
-    patch, the nine stages of chunk 0, then per K step the next chunk's patch loads and the stage nine steps ahead) and
-    the exact largest safe n is counted at every barrier.  The formula may never exceed it (a race), and equals it."""
+    landed.  What must have landed at the barrier that closes K step s: filter stage s + 2 (its fragments are read
+    during step s + 1) and, at tap 7, the next chunk's patch (read in the last rows of tap 8).  n comes from a closed
+    formula in the kernel; here the issue order is replayed load by load (the first patch, the nine stages of chunk 0,
+    then per K step the next chunk's patch loads and the stage nine steps ahead) and the exact largest safe n is
+    counted at every barrier.  The formula may never exceed it (a race), and equals it."""
     lib = _lib.load()
     lib.cinn_hip_conv_patch_loads_in_flight.argtypes = [ctypes.c_int] * 4
     lib.cinn_hip_conv_patch_loads_in_flight.restype = ctypes.c_int
-    taps, ring, patch_steps, stage_loads = 9, 9, 4, 2
+    taps, ring, patch_steps, stage_loads, ahead = 9, 9, 4, 2, 2
     for chunks in range(2, 7):
+        total = chunks * taps
         for per_step in (2, 3):
             log = [("patch", 0)] * (per_step * patch_steps)
             for st in range(ring):
@@ -284,7 +287,9 @@ def test_chunked_patch_kernel_wait_counts_match_a_simulation_of_its_issue_order(
                     if last and t == taps - 1:
                         break  # the last K step has no barrier
                     s = c * taps + t
-                    needed = [("stage", s + 1)] + ([("patch", c + 1)] if (not last and t == taps - 1) else [])
+                    needed = [("stage", min(s + ahead, total - 1))]
+                    if not last and t == taps - ahead:
+                        needed.append(("patch", c + 1))
                     newest = max(max(i for i, e in enumerate(log) if e == what) for what in needed)
                     exact = len(log) - 1 - newest
                     got = lib.cinn_hip_conv_patch_loads_in_flight(t, int(c == 0), int(last), per_step)

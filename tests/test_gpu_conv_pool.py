@@ -596,11 +596,24 @@ PATCH_CHUNK_CASES = [
 ]
 
 
+@pytest.mark.parametrize("tiles", [4, 2])
 @pytest.mark.parametrize("dtype,tol", [("float16", 1e-2), ("bfloat16", 2e-2)])
 @pytest.mark.parametrize("case", PATCH_CHUNK_CASES)
-def test_convolution_with_the_input_patch_resident_in_lds_by_channel_chunks(gpu, patch_kernel_everywhere, case, dtype, tol):
+def test_convolution_with_the_input_patch_resident_in_lds_by_channel_chunks(gpu, patch_kernel_everywhere, case, dtype, tol,
+                                                                            tiles):
     """conv3x3_patch_chunks_kernel against the oracle and against the implicit-GEMM kernel (which adds the same
-    products tap by tap instead of chunk by chunk: equal within rounding, not bit for bit)."""
+    products tap by tap instead of chunk by chunk: equal within rounding, not bit for bit).  Both block sizes: four
+    tiles per computing wavefront (barrier inside a K step) and two (filter fragments read a step early, barrier at
+    the end of the step); a shape whose bands do not fill blocks of that size stays on the other kernels."""
+    patch_kernel_everywhere.cinn_hip_conv_patch_tiles.argtypes = [ctypes.c_int]
+    before = patch_kernel_everywhere.cinn_hip_conv_patch_tiles(tiles)
+    try:
+        _check_chunked_patch_case(patch_kernel_everywhere, case, dtype, tol)
+    finally:
+        patch_kernel_everywhere.cinn_hip_conv_patch_tiles(before)
+
+
+def _check_chunked_patch_case(patch_kernel_everywhere, case, dtype, tol):
     n, ic, h, w_, oc = case
     rng = np.random.default_rng(sum(case) + 11)
     x = round_to(rng.standard_normal((n, ic, h, w_)), dtype)
