@@ -71,7 +71,8 @@ struct PatchParams {
   int relu;
   int n, h, w_in, oc;
   int c;            // input channels (a multiple of 64)
-  int rows;         // output rows per band
+  int stack;        // chunked kernel: images per block, stacked with one row of zeros between them (1: bands of one image)
+  int rows;         // output rows per band (stacked images: their rows and the separating rows)
   int bands;        // bands per image
   int patch_loads;  // 1 KiB loads that cover the (rows + 2) (W + 2) positions of 10 slots
   unsigned w_magic, w_shift;    // n / W == (n * w_magic) >> w_shift (chunked kernel: W rounded up to a multiple of 8)
@@ -112,12 +113,16 @@ __device__ __forceinline__ void PatchEpilogue(const PatchParams& p, const f32x4 
   typedef typename Mfma16<T>::vec8 vec8;
   const int W    = p.w_in;
   const int npix = rows * W;
-  // the band's pixel in slot q, or -1
+  // the band's pixel in slot q (counted from the first pixel of the band's first image row), or -1
   auto pixel_of = [&](int q) -> int {
     if (!PADDED) return q < npix ? q : -1;
     const int ly = (int)(((uint64_t)(unsigned)q * p.w_magic) >> p.w_shift);
     const int lx = q - ly * wp;
-    return ly < rows && lx < W ? ly * W + lx : -1;
+    if (ly >= rows || lx >= W) return -1;
+    if (p.stack == 1) return ly * W + lx;
+    // stacked images: row ly of the band is row ly % (H + 1) of image ly / (H + 1); row H is the separator
+    const int k = ly / (p.h + 1), iy = ly - k * (p.h + 1);
+    return iy < p.h ? (k * p.h + iy) * W + lx : -1;
   };
   // lane = (slot lane & 15 of each tile; channels 8 g .. 8 g + 7 and 32 + 8 g .. + 7)
   const int g   = lane >> 4;
@@ -469,14 +474,15 @@ __global__ void __launch_bounds__(128 * kWaves) conv3x3_patch_chunks_kernel(Patc
   const int lane    = tid & 63;
   const int wave    = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int band    = blockIdx.x % p.bands;
-  const int img     = blockIdx.x / p.bands;
+  const int img     = (blockIdx.x / p.bands) * p.stack;  // the block's (first) image
   const int n0      = blockIdx.y * 64;
   const int W       = p.w_in;
   const int PW      = W + 2;
   const int C       = p.c;
   const int chunks  = C >> 6;
   const int y0      = band * p.rows;
-  const int rows    = min(p.rows, p.h - y0);
+  // a band of one image, or min(stack, images left) whole images with a row of zeros after each but the last
+  const int rows    = p.stack == 1 ? min(p.rows, p.h - y0) : min(p.stack, p.n - img) * (p.h + 1) - 1;
   const int WP      = (W + 7) & ~7;           // pixel slots per image row: a 16-lane tile is two halves of one row each
   const int npos    = (p.rows + 2) * PW;
   const int ktot    = kTaps * C;              // filter row length
@@ -501,10 +507,16 @@ __global__ void __launch_bounds__(128 * kWaves) conv3x3_patch_chunks_kernel(Patc
         const unsigned pos   = (slot * 52429u) >> 19;  // slot / 10 for slot < 2^16
         const unsigned chunk = slot - 10u * pos;
         const int pr         = (int)(((uint64_t)pos * p.pw_magic) >> p.pw_shift);
-        const int iy         = y0 - 1 + pr;
+        int iy               = y0 - 1 + pr;  // row of the image, or of the stack
+        int k                = 0;            // image of the stack
+        if (p.stack > 1 && iy >= 0) {
+          k  = iy / (p.h + 1);
+          iy = iy - k * (p.h + 1);           // H: the row of zeros between two images
+        }
         const int ix         = (int)pos - pr * PW - 1;
-        const bool inside    = chunk < 8u && (unsigned)iy < (unsigned)p.h && (unsigned)ix < (unsigned)W && (int)pos < npos;
-        src[i]        = inside ? ximg + ((int64_t)(iy * W + ix) * C * 2 + chunk * 16u) : zeros + ((lane & 7) << 4);
+        const bool inside    = chunk < 8u && (unsigned)iy < (unsigned)p.h && (unsigned)ix < (unsigned)W && (int)pos < npos &&
+                            img + k < p.n;
+        src[i]        = inside ? ximg + ((int64_t)((k * p.h + iy) * W + ix) * C * 2 + chunk * 16u) : zeros + ((lane & 7) << 4);
         step_bytes[i] = inside ? 128u : 0u;
         dst[i]        = (unsigned)q * 1024u;
       }
@@ -658,6 +670,8 @@ __global__ void __launch_bounds__(128 * kWaves) conv3x3_patch_chunks_kernel(Patc
 
 struct PatchPlan {
   int rows, bands, patch_loads, lds_bytes;
+  int stack{1};  // images per block (chunked kernel, small images)
+  int blocks(int n) const { return ((n + stack - 1) / stack) * bands; }  // per group of 64 output channels
 };
 
 // rows per band and LDS footprint; false when the patch does not fit or more than a fifth of the blocks' pixel slots
@@ -674,7 +688,7 @@ bool PlanFor(const ConvNhwcArgs& a, PatchPlan* plan) {
   const int patch_loads = (slots + 63) / 64;
   const int bytes       = kNS * kBTile + patch_loads * 1024;
   if (bytes > kLdsLimit) return false;
-  *plan = PatchPlan{rows, bands, patch_loads, bytes};
+  *plan = PatchPlan{rows, bands, patch_loads, bytes, 1};
   return true;
 }
 
@@ -687,7 +701,20 @@ bool PlanChunksFor(const ConvNhwcArgs& a, PatchPlan* plan, int* per_step) {
   constexpr int capacity = kWaves * TMW * 16;
   const int wp = (a.w_in + 7) & ~7;  // pixel slots per image row
   int rows     = capacity / wp;
-  rows         = rows < a.h ? rows : a.h;
+  // small images: several whole images per block, stacked with a row of zeros between them (the bottom halo of one
+  // and the top halo of the next); that row is computed and not stored
+  for (int stack = (rows + 1) / (a.h + 1) < a.n ? (rows + 1) / (a.h + 1) : a.n; stack >= 2; --stack) {
+    const int stacked     = stack * (a.h + 1) - 1;
+    const int slots       = (stacked + 2) * (a.w_in + 2) * 10;
+    const int patch_loads = (slots + 63) / 64;
+    const int bytes       = kRing * kBTile + 2 * patch_loads * 1024;
+    if (patch_loads > kWaves * kPatchSteps * 3 || bytes > kLdsLimit) continue;
+    if ((int64_t)stack * a.h * a.w_in * 10 < (int64_t)capacity * 7) break;
+    *plan     = PatchPlan{stacked, 1, patch_loads, bytes, stack};
+    *per_step = patch_loads > kWaves * kPatchSteps * 2 ? 3 : 2;
+    return true;
+  }
+  rows = rows < a.h ? rows : a.h;
   for (; rows >= 1; --rows) {
     const int bands       = (a.h + rows - 1) / rows;
     const int even        = (a.h + bands - 1) / bands;
@@ -696,7 +723,7 @@ bool PlanChunksFor(const ConvNhwcArgs& a, PatchPlan* plan, int* per_step) {
     const int bytes       = kRing * kBTile + 2 * patch_loads * 1024;
     if (patch_loads > kWaves * kPatchSteps * 3 || bytes > kLdsLimit) continue;
     if ((int64_t)a.h * a.w_in * 10 < (int64_t)bands * capacity * 7) return false;
-    *plan     = PatchPlan{even, bands, patch_loads, bytes};
+    *plan     = PatchPlan{even, bands, patch_loads, bytes, 1};
     *per_step = patch_loads > kWaves * kPatchSteps * 2 ? 3 : 2;  // 32 KiB, else 48 KiB of patch per buffer
     return true;
   }
@@ -711,7 +738,7 @@ void LaunchChunks(const PatchParams& p, const PatchPlan& plan, hipStream_t strea
     return true;
   }();
   (void)configured;
-  dim3 grid(p.n * p.bands, p.oc / 64);
+  dim3 grid(plan.blocks(p.n), p.oc / 64);
   hipLaunchKernelGGL(kernel, grid, dim3(128 * kWaves), plan.lds_bytes, stream, p);
 }
 
@@ -780,11 +807,11 @@ bool TryConvPatch(const ConvNhwcArgs& a, hipStream_t stream) {
     // FLAGS_cinn_hip_conv_patch_tiles=2|4 (or cinn_hip_conv_patch_tiles) forces one form.
     const int forced_tiles = PatchTiles();
     const bool fits4 = forced_tiles != 2 && PlanChunksFor<4>(a, &plan, &per_step);
-    const int64_t blocks4 = fits4 ? (int64_t)a.n * plan.bands * (a.oc / 64) : 0;
+    const int64_t blocks4 = fits4 ? (int64_t)plan.blocks(a.n) * (a.oc / 64) : 0;
     if (forced_tiles == 2 || (forced_tiles == 0 && blocks4 < 192)) {
       PatchPlan plan2;
       int per_step2 = 0;
-      if (PlanChunksFor<2>(a, &plan2, &per_step2) && per_step2 == 2 && (int64_t)a.n * plan2.bands * (a.oc / 64) > blocks4) {
+      if (PlanChunksFor<2>(a, &plan2, &per_step2) && per_step2 == 2 && (int64_t)plan2.blocks(a.n) * (a.oc / 64) > blocks4) {
         plan = plan2, per_step = per_step2, tiles = 2;
       } else if (!fits4) {
         return false;
@@ -797,14 +824,14 @@ bool TryConvPatch(const ConvNhwcArgs& a, hipStream_t stream) {
   }
   // one block per band, image and 64 output channels; below ~100 blocks most of the chip would idle and the
   // implicit-GEMM tiles are the better choice
-  if (flag != 2 && (int64_t)a.n * plan.bands * (a.oc / 64) < 96) return false;
+  if (flag != 2 && (int64_t)plan.blocks(a.n) * (a.oc / 64) < 96) return false;
   PatchParams p;
   p.x = static_cast<const uint16_t*>(a.x), p.w = static_cast<const uint16_t*>(a.w), p.y = static_cast<uint16_t*>(a.y);
   p.scale = a.scale, p.shift = a.shift, p.residual = static_cast<const uint16_t*>(a.residual);
   p.zero_page = ConvZeroPage();
   p.alpha = a.alpha, p.residual_scale = a.residual_scale, p.relu = a.relu ? 1 : 0;
   p.n = a.n, p.h = a.h, p.w_in = a.w_in, p.oc = a.oc, p.c = a.c;
-  p.rows = plan.rows, p.bands = plan.bands, p.patch_loads = plan.patch_loads;
+  p.rows = plan.rows, p.bands = plan.bands, p.patch_loads = plan.patch_loads, p.stack = plan.stack;
   MagicFor(chunked ? (a.w_in + 7) & ~7 : a.w_in, &p.w_magic, &p.w_shift);
   MagicFor(a.w_in + 2, &p.pw_magic, &p.pw_shift);
   if (chunked && tiles == 2) {

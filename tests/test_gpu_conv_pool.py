@@ -592,7 +592,10 @@ PATCH_CHUNK_CASES = [
     (1, 128, 16, 25, 64),    # odd width, bands of 8 rows: 25 of the 32 pixel slots of a row are real
     (2, 128, 12, 32, 64),    # bands of 6 rows of 32 pixels
     (1, 128, 27, 28, 64),    # bands of 7, 7, 7 and 6 rows: first, inner and a shorter last band
-    (2, 128, 7, 7, 64),      # does not qualify (49 of 256 pixel slots): stays on the other kernels
+    (2, 128, 7, 7, 64),      # two images stacked in a block of 128 slots (a row of zeros between them); 256: no
+    (5, 128, 7, 7, 128),     # blocks of 128 slots: stacks of 2, 2 and 1 images
+    (4, 128, 7, 14, 64),     # blocks of 256 slots: two images of 7 x 14 per block; 128 slots: one image per block
+    (9, 512, 7, 7, 64),      # eight chunks over stacked images
 ]
 
 
