@@ -825,6 +825,9 @@ bool TryConvPatch(const ConvNhwcArgs& a, hipStream_t stream) {
   // one block per band, image and 64 output channels; below ~100 blocks most of the chip would idle and the
   // implicit-GEMM tiles are the better choice
   if (flag != 2 && (int64_t)plan.blocks(a.n) * (a.oc / 64) < 96) return false;
+  // stacked small images (512 -> 512 on 7x7 at batch 32: 128 blocks of two images, 23.1 us inside ResNet-50) lose to the
+  // implicit GEMM with its reduction split four ways (16.6 + 4.8 us) until they fill most of the chip
+  if (flag != 2 && plan.stack > 1 && (int64_t)plan.blocks(a.n) * (a.oc / 64) < 192) return false;
   PatchParams p;
   p.x = static_cast<const uint16_t*>(a.x), p.w = static_cast<const uint16_t*>(a.w), p.y = static_cast<uint16_t*>(a.y);
   p.scale = a.scale, p.shift = a.shift, p.residual = static_cast<const uint16_t*>(a.residual);
