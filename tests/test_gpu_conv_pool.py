@@ -631,8 +631,19 @@ def _check_chunked_patch_case(patch_kernel_everywhere, case, dtype, tol):
     assert np.all(np.abs(got - other) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
 
 
-def test_chunked_patch_convolution_with_residual_epilogue(gpu, patch_kernel_everywhere):
-    """alpha / beta through the in-register epilogue of the chunked kernel: y = 0.5 conv(x, w) + 2 y0."""
+@pytest.mark.parametrize("tiles", [4, 2])
+def test_chunked_patch_convolution_with_residual_epilogue(gpu, patch_kernel_everywhere, tiles):
+    """alpha / beta through the in-register epilogue of the chunked kernel: y = 0.5 conv(x, w) + 2 y0, with blocks of
+    256 and of 128 pixel slots."""
+    patch_kernel_everywhere.cinn_hip_conv_patch_tiles.argtypes = [ctypes.c_int]
+    before = patch_kernel_everywhere.cinn_hip_conv_patch_tiles(tiles)
+    try:
+        _check_chunked_residual()
+    finally:
+        patch_kernel_everywhere.cinn_hip_conv_patch_tiles(before)
+
+
+def _check_chunked_residual():
     n, ic, h, w_, oc = 2, 256, 14, 14, 128
     rng = np.random.default_rng(198)
     x = round_to(rng.standard_normal((n, ic, h, w_)), "float16")
