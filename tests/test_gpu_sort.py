@@ -154,3 +154,23 @@ def test_top_k_is_the_reference_composition(gpu):
         assert np.array_equal(got_indices, order[:, :5, :].astype(np.int64))
         assert np.array_equal(got_values, ordered[:, :5, :])
         assert np.array_equal(got_values[:, 0, :], x.max(1))
+
+
+@pytest.mark.parametrize("shape", [[512], [1024], [1200], [64, 16], [4, 32, 8], [16, 8, 4, 2], [2, 8, 4, 2, 5],
+                                   [4, 8, 1, 2, 16], [1], [1, 1, 1, 1], [1, 1, 1, 1, 1]])
+def test_sort_on_the_shapes_of_the_reference_suite(gpu, shape):
+    """The shape list of python/tests/ops/test_sort_op.py (axis 0, ascending, float32; its descending and duplicate
+    element cases are covered above) and of test_top_k_op.py: sort, argsort and top_k (k = 1) against the oracle."""
+    rng = np.random.default_rng(sum(shape) + len(shape))
+    x = rng.random(shape).astype(np.float32)
+    b = NetBuilder("s")
+    v = b.create_input(Float(32), shape, "x")
+    values = b.sort(v, 0, True)
+    index, _ = b.argsort(v, 0, True)
+    top_values, top_index = b.top_k(v, 1, 0, True)
+    (got_values, got_index, got_top, got_top_index), _ = run(b, {v: x}, [values, index, top_values, top_index])
+    want_index, _, want_values = oracle.argsort(x, 0, True)
+    assert np.array_equal(got_values, want_values) and np.array_equal(got_values, np.sort(x, axis=0, kind="stable"))
+    assert np.array_equal(got_index, want_index)
+    assert np.array_equal(got_top, x.max(axis=0, keepdims=True))
+    assert np.array_equal(got_top_index, x.argmax(axis=0)[None].astype(np.int64))
