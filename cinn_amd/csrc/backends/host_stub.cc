@@ -1,8 +1,13 @@
 #include "backends/host_stub.h"
 
+#include <sys/mman.h>
+
 #include <array>
+#include <cstring>
+#include <map>
 #include <mutex>
 #include <utility>
+#include <vector>
 
 namespace cinn {
 namespace backends {
@@ -145,6 +150,73 @@ const std::array<lower_func_ptr_g, HostStubPool::kSlots>& Table() {
 }
 }  // namespace
 
+// ---- stubs beyond the pre-compiled slots: generated thunks ---------------------------------------------------------
+namespace {
+#if defined(__x86_64__)
+void ThunkDispatch(void* args, int32_t num_args, void* stream, HostStubPool::Closure* closure) {
+  (*closure)(args, num_args, stream);
+}
+
+// movabs rcx, <closure>; movabs rax, <ThunkDispatch>; jmp rax  - the stub's own three arguments stay in rdi, esi, rdx
+constexpr size_t kThunkBytes = 32;
+constexpr size_t kThunkPage  = 1 << 16;
+
+struct ThunkState {
+  std::vector<unsigned char*> pages;
+  size_t used_in_last{kThunkPage};
+  std::vector<unsigned char*> free_list;
+  std::map<lower_func_ptr_g, HostStubPool::Closure*> live;
+};
+ThunkState& Thunks() {
+  static ThunkState* s = new ThunkState;  // leaked like the pool: stubs may run during static teardown
+  return *s;
+}
+
+// caller holds the pool's mutex; null when the system does not hand out executable memory
+lower_func_ptr_g NewThunk(HostStubPool::Closure closure) {
+  auto& t = Thunks();
+  unsigned char* code = nullptr;
+  if (!t.free_list.empty()) {
+    code = t.free_list.back();
+    t.free_list.pop_back();
+  } else {
+    if (t.used_in_last + kThunkBytes > kThunkPage) {
+      void* page = mmap(nullptr, kThunkPage, PROT_READ | PROT_WRITE | PROT_EXEC, MAP_PRIVATE | MAP_ANONYMOUS, -1, 0);
+      if (page == MAP_FAILED) return nullptr;
+      t.pages.push_back(static_cast<unsigned char*>(page));
+      t.used_in_last = 0;
+    }
+    code = t.pages.back() + t.used_in_last;
+    t.used_in_last += kThunkBytes;
+  }
+  auto* owned            = new HostStubPool::Closure(std::move(closure));
+  const uint64_t ctx     = reinterpret_cast<uint64_t>(owned);
+  const uint64_t target  = reinterpret_cast<uint64_t>(&ThunkDispatch);
+  unsigned char bytes[22] = {0x48, 0xB9, 0, 0, 0, 0, 0, 0, 0, 0, 0x48, 0xB8, 0, 0, 0, 0, 0, 0, 0, 0, 0xFF, 0xE0};
+  std::memcpy(bytes + 2, &ctx, 8);
+  std::memcpy(bytes + 12, &target, 8);
+  std::memcpy(code, bytes, sizeof(bytes));
+  __builtin___clear_cache(reinterpret_cast<char*>(code), reinterpret_cast<char*>(code) + sizeof(bytes));
+  auto fn    = reinterpret_cast<lower_func_ptr_g>(code);
+  t.live[fn] = owned;
+  return fn;
+}
+
+bool ReleaseThunk(lower_func_ptr_g fn) {
+  auto& t = Thunks();
+  auto it = t.live.find(fn);
+  if (it == t.live.end()) return false;
+  delete it->second;
+  t.live.erase(it);
+  t.free_list.push_back(reinterpret_cast<unsigned char*>(fn));
+  return true;
+}
+#else
+lower_func_ptr_g NewThunk(HostStubPool::Closure) { return nullptr; }
+bool ReleaseThunk(lower_func_ptr_g) { return false; }
+#endif
+}  // namespace
+
 HostStubPool& HostStubPool::Global() {
   static HostStubPool pool;
   return pool;
@@ -153,7 +225,12 @@ HostStubPool& HostStubPool::Global() {
 lower_func_ptr_g HostStubPool::Acquire(Closure closure) {
   auto& s = State();
   std::lock_guard<std::mutex> lock(s.mu);
-  CINN_CHECK_LT(s.in_use, kSlots) << "all " << kSlots << " host stub slots are in use; release compiled programs";
+  if (s.in_use >= kSlots) {
+    lower_func_ptr_g fn = NewThunk(std::move(closure));
+    CINN_CHECK(fn) << "all " << kSlots << " pre-compiled host stub slots are in use and no executable memory could be "
+                   << "mapped for more; release compiled programs";
+    return fn;
+  }
   for (int probe = 0; probe < kSlots; ++probe) {
     int slot = (s.next_hint + probe) % kSlots;
     if (!s.used[slot]) {
@@ -182,12 +259,23 @@ void HostStubPool::Release(lower_func_ptr_g fn) {
       return;
     }
   }
+  ReleaseThunk(fn);
 }
 
 int HostStubPool::in_use() const {
   auto& s = State();
   std::lock_guard<std::mutex> lock(s.mu);
   return s.in_use;
+}
+
+int HostStubPool::thunks_in_use() const {
+  auto& s = State();
+  std::lock_guard<std::mutex> lock(s.mu);
+#if defined(__x86_64__)
+  return static_cast<int>(Thunks().live.size());
+#else
+  return 0;
+#endif
 }
 
 // ---------------------------------------------------------------------------------------------------

@@ -51,7 +51,9 @@ class ExternApiRegistry {
 };
 
 // Pool of trampolines.  Acquire() binds a closure to a free slot and returns the slot's function
-// pointer; Release() frees it.
+// pointer; Release() frees it.  kSlots functions are pre-compiled; when all of them are taken, further stubs are a few
+// bytes of machine code each in an executable page (x86-64: load the closure's address into the fourth argument
+// register and jump to a common dispatcher), so the number of live compiled functions is bounded by memory only.
 class HostStubPool {
  public:
   static constexpr int kSlots = 4096;
@@ -60,6 +62,7 @@ class HostStubPool {
   lower_func_ptr_g Acquire(Closure closure);
   void Release(lower_func_ptr_g fn);
   int in_use() const;
+  int thunks_in_use() const;  // stubs beyond the pre-compiled slots
 };
 
 // Resolves the symbols a host function refers to (kernel handles by name) and builds its closure.
