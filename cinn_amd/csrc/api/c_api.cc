@@ -165,6 +165,15 @@ const std::map<std::string, Method>& Methods() {
                                             GetAttr<std::string>(a, "data_format", "NCHW"),
                                             GetAttr<std::string>(a, "padding_algorithm", "EXPLICIT"))};
     };
+    m["Conv"] = [](NetBuilder& b, const std::vector<Variable>& in, const AttributeMap& a) {
+      return std::vector<Variable>{b.Conv(in.at(0), in.at(1), GetAttr<std::vector<int>>(a, "strides", {1, 1}),
+                                          GetAttr<std::vector<int>>(a, "paddings", {0, 0}),
+                                          GetAttr<std::vector<int>>(a, "dilations", {1, 1}), GetAttr<int>(a, "groups", 1),
+                                          GetAttr<std::string>(a, "conv_type", "forward"),
+                                          GetAttr<std::string>(a, "data_format", "NCHW"),
+                                          GetAttr<std::string>(a, "padding_algorithm", "EXPLICIT"),
+                                          GetAttr<std::vector<int>>(a, "output_shape", {}))};
+    };
     m["BatchNorm"] = [](NetBuilder& b, const std::vector<Variable>& in, const AttributeMap& a) {
       return b.BatchNorm(in.at(0), in.at(1), in.at(2), in.at(3), in.at(4), GetAttr<float>(a, "epsilon", 1e-5f),
                          GetAttr<float>(a, "momentum", 0.9f), GetAttr<std::string>(a, "data_layout", "NCHW"),
@@ -177,6 +186,15 @@ const std::map<std::string, Method>& Methods() {
                    GetAttr<bool>(a, "ceil_mode", false), GetAttr<bool>(a, "exclusive", true),
                    GetAttr<bool>(a, "global_pooling", false), GetAttr<std::string>(a, "data_format", "NCHW"),
                    GetAttr<bool>(a, "adaptive", false), GetAttr<std::string>(a, "padding_algorithm", "EXPLICIT"))};
+    };
+    m["Pool2dGrad"] = [](NetBuilder& b, const std::vector<Variable>& in, const AttributeMap& a) {
+      return std::vector<Variable>{b.Pool2dGrad(
+          in.at(0), in.at(1), in.at(2), GetAttr<std::string>(a, "pooling_type", "max"),
+          GetAttr<std::vector<int>>(a, "ksize", {1, 1}), GetAttr<std::vector<int>>(a, "strides", {1, 1}),
+          GetAttr<std::vector<int>>(a, "paddings", {0, 0}), GetAttr<bool>(a, "ceil_mode", false),
+          GetAttr<bool>(a, "exclusive", true), GetAttr<bool>(a, "global_pooling", false),
+          GetAttr<std::string>(a, "data_format", "NCHW"), GetAttr<bool>(a, "adaptive", false),
+          GetAttr<std::string>(a, "padding_algorithm", "EXPLICIT"))};
     };
     // inputs: x [, scale [, bias]]
     m["PaddleLayerNorm"] = [](NetBuilder& b, const std::vector<Variable>& in, const AttributeMap& a) {

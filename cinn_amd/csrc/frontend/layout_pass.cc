@@ -282,6 +282,7 @@ Program FuseConvBatchNorm(const Program& program, const std::set<std::string>& f
     auto& conv = instrs[i];
     if (conv->op_type != "conv2d" || dropped[i]) continue;
     if (GetAttr<std::string>(conv->attrs, "data_format", "NCHW") != "NHWC") continue;
+    if (GetAttr<std::string>(conv->attrs, "conv_type", "forward") != "forward") continue;
     // grouped convolutions in channels-last form are depthwise ones (the layout pass converts no others); their kernel
     // has the same epilogue
     int bn_at = single_user(conv->outputs[0]);

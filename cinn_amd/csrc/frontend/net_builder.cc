@@ -278,14 +278,23 @@ Variable NetBuilder::Mul(const Variable& x, const Variable& y, int x_num_col_dim
 Variable NetBuilder::Conv2d(const Variable& x, const Variable& w, const std::vector<int>& strides,
                             const std::vector<int>& paddings, const std::vector<int>& dilations, int groups,
                             const std::string& data_format, const std::string& padding_algorithm) {
-  return CustomInstr("conv2d", {x, w},
+  return Conv(x, w, strides, paddings, dilations, groups, "forward", data_format, padding_algorithm, {});
+}
+// cinn/frontend/net_builder.cc:465-486: forward takes (x, w); backward_data (w, dy) and gives dx of `output_shape`;
+// backward_filter (x, dy) and gives dw of `output_shape`
+Variable NetBuilder::Conv(const Variable& lhs, const Variable& rhs, const std::vector<int>& strides,
+                          const std::vector<int>& paddings, const std::vector<int>& dilations, int groups,
+                          const std::string& conv_type, const std::string& data_format,
+                          const std::string& padding_algorithm, const std::vector<int>& output_shape) {
+  return CustomInstr("conv2d", {lhs, rhs},
                      {{"stride", strides},
                       {"padding", paddings},
                       {"dilation", dilations},
                       {"groups", groups},
-                      {"conv_type", std::string("forward")},
+                      {"conv_type", conv_type},
                       {"data_format", data_format},
-                      {"padding_algorithm", padding_algorithm}})
+                      {"padding_algorithm", padding_algorithm},
+                      {"output_shape", output_shape}})
       .front();
 }
 std::vector<Variable> NetBuilder::BatchNorm(const Variable& x, const Variable& scale, const Variable& bias,
@@ -296,10 +305,11 @@ std::vector<Variable> NetBuilder::BatchNorm(const Variable& x, const Variable& s
                      {{"epsilon", epsilon}, {"momentum", momentum}, {"data_layout", data_layout}});
 }
 
-Variable NetBuilder::Pool2d(const Variable& x, const std::string& pooling_type, const std::vector<int>& ksize,
-                            const std::vector<int>& strides, const std::vector<int>& paddings, bool ceil_mode,
-                            bool exclusive, bool global_pooling, const std::string& data_format, bool adaptive,
-                            const std::string& padding_algorithm) {
+namespace {
+utils::AttributeMap Pool2dAttrs(const Variable& x, const std::string& pooling_type, const std::vector<int>& ksize,
+                         const std::vector<int>& strides, const std::vector<int>& paddings, bool ceil_mode,
+                         bool exclusive, bool global_pooling, const std::string& data_format, bool adaptive,
+                         const std::string& padding_algorithm) {
   // attribute normalisation of cinn/frontend/net_builder.cc:538-684
   CINN_CHECK_EQ(x->shape.size(), 4u) << "Input's dim must be 4";
   std::string pool_type;
@@ -335,8 +345,7 @@ Variable NetBuilder::Pool2d(const Variable& x, const std::string& pooling_type, 
   }
   if (global_pooling || adaptive) p = {0, 0, 0, 0};
   if (global_pooling) k = {x->shape[hi], x->shape[wi]};
-  return CustomInstr("pool2d", {x},
-                     {{"pool_type", pool_type},
+  return utils::AttributeMap{{"pool_type", pool_type},
                       {"kernel_size", k},
                       {"stride_size", s},
                       {"padding_size", p},
@@ -345,7 +354,27 @@ Variable NetBuilder::Pool2d(const Variable& x, const std::string& pooling_type, 
                       {"global_pooling", global_pooling},
                       {"data_format", layout},
                       {"adaptive", adaptive},
-                      {"padding_algorithm", padding_algorithm}})
+                      {"padding_algorithm", padding_algorithm}};
+}
+}  // namespace
+
+Variable NetBuilder::Pool2d(const Variable& x, const std::string& pooling_type, const std::vector<int>& ksize,
+                            const std::vector<int>& strides, const std::vector<int>& paddings, bool ceil_mode,
+                            bool exclusive, bool global_pooling, const std::string& data_format, bool adaptive,
+                            const std::string& padding_algorithm) {
+  return CustomInstr("pool2d", {x},
+                     Pool2dAttrs(x, pooling_type, ksize, strides, paddings, ceil_mode, exclusive, global_pooling,
+                                 data_format, adaptive, padding_algorithm))
+      .front();
+}
+// cinn/frontend/net_builder.cc:686-755: the same attribute normalisation as pool2d, inputs x, y = pool2d(x), dy
+Variable NetBuilder::Pool2dGrad(const Variable& x, const Variable& y, const Variable& dy, const std::string& pooling_type,
+                                const std::vector<int>& ksize, const std::vector<int>& strides,
+                                const std::vector<int>& paddings, bool ceil_mode, bool exclusive, bool global_pooling,
+                                const std::string& data_format, bool adaptive, const std::string& padding_algorithm) {
+  return CustomInstr("pool2d_grad", {x, y, dy},
+                     Pool2dAttrs(x, pooling_type, ksize, strides, paddings, ceil_mode, exclusive, global_pooling,
+                                 data_format, adaptive, padding_algorithm))
       .front();
 }
 

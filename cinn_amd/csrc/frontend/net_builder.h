@@ -99,6 +99,12 @@ class NetBuilder {
                   const std::vector<int>& paddings = {0, 0}, const std::vector<int>& dilations = {1, 1},
                   int groups = 1, const std::string& data_format = "NCHW",
                   const std::string& padding_algorithm = "EXPLICIT");
+  // conv_type "forward" (x, w), "backward_data" (w, dy -> dx of output_shape) or "backward_filter" (x, dy -> dw of
+  // output_shape), cinn/frontend/net_builder.h (Conv)
+  Variable Conv(const Variable& lhs, const Variable& rhs, const std::vector<int>& strides = {1, 1},
+                const std::vector<int>& paddings = {0, 0}, const std::vector<int>& dilations = {1, 1}, int groups = 1,
+                const std::string& conv_type = "forward", const std::string& data_format = "NCHW",
+                const std::string& padding_algorithm = "EXPLICIT", const std::vector<int>& output_shape = {});
   std::vector<Variable> BatchNorm(const Variable& x, const Variable& scale, const Variable& bias,
                                   const Variable& mean, const Variable& variance, float epsilon = 1e-5f,
                                   float momentum = 0.9f, const std::string& data_layout = "NCHW", bool is_test = true);
@@ -107,6 +113,11 @@ class NetBuilder {
                   bool ceil_mode = false, bool exclusive = true, bool global_pooling = false,
                   const std::string& data_format = "NCHW", bool adaptive = false,
                   const std::string& padding_algorithm = "EXPLICIT");
+  Variable Pool2dGrad(const Variable& x, const Variable& y, const Variable& dy, const std::string& pooling_type,
+                      const std::vector<int>& ksize, const std::vector<int>& strides = {1, 1},
+                      const std::vector<int>& paddings = {0, 0}, bool ceil_mode = false, bool exclusive = true,
+                      bool global_pooling = false, const std::string& data_format = "NCHW", bool adaptive = false,
+                      const std::string& padding_algorithm = "EXPLICIT");
 
  protected:
   Variable UnaryOp(const std::string& op_type, const Variable& x);

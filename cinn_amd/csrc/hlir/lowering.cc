@@ -1369,6 +1369,27 @@ ir::LoweredFuncRef OpLowerer::LowerLibraryCall(const Group& group) const {
     args.push_back(Expr(alpha));
     args.push_back(Expr(beta));
     push_ints({a4[0], a4[1], a4[2], a4[3], b4[0], b4[1], b4[2], b4[3]});
+  } else if (op == "conv2d" && GetAttr<std::string>(n->attrs, "conv_type", "forward") != "forward") {
+    // argument lists of CustomCallArgsForCudnnConvBackwardData / ...BackwardFilter (custom_call.cc:390-500): the
+    // extents of x, w and dy in n, c, h, w order, whichever of them is the output
+    const bool data = GetAttr<std::string>(n->attrs, "conv_type", "forward") == "backward_data";
+    api             = data ? "cinn_call_cudnn_conv2d_backward_data" : "cinn_call_cudnn_conv2d_backward_filter";
+    auto stride     = GetAttr<std::vector<int>>(n->attrs, "stride", {1, 1});
+    auto padding    = GetAttr<std::vector<int>>(n->attrs, "padding", {0, 0});
+    auto dilation   = GetAttr<std::vector<int>>(n->attrs, "dilation", {1, 1});
+    int groups      = GetAttr<int>(n->attrs, "groups", 1);
+    const bool nchw = GetAttr<std::string>(n->attrs, "data_format", "NCHW") == "NCHW";
+    ShapeType x  = data ? n->outputs[0]->shape : n->inputs[0]->shape;
+    ShapeType w  = data ? n->inputs[0]->shape : n->outputs[0]->shape;
+    ShapeType dy = n->inputs[1]->shape;
+    auto ordered = [&](const ShapeType& s) { return nchw ? s : ShapeType{s[0], s[3], s[1], s[2]}; };
+    x = ordered(x), w = ordered(w), dy = ordered(dy);
+    args.push_back(I32(nchw ? 0 : 1));
+    args.push_back(Expr(1.0f));
+    args.push_back(Expr(0.0f));
+    push_ints({x[0], x[1], x[2], x[3], w[0], w[1], w[2], w[3]});
+    push_ints({padding[0], padding[1], stride[0], stride[1], dilation[0], dilation[1], groups});
+    push_ints({dy[0], dy[1], dy[2], dy[3]});
   } else if (op == "conv2d" || op == "hip_conv2d_bn_relu") {
     // argument list of CustomCallArgsForCudnnConvForward (custom_call.cc:338-388)
     auto stride   = GetAttr<std::vector<int>>(n->attrs, "stride", {1, 1});
@@ -1414,9 +1435,10 @@ ir::LoweredFuncRef OpLowerer::LowerLibraryCall(const Group& group) const {
     } else {
       push_ints({y[0], y[3], y[1], y[2]});
     }
-  } else if (op == "pool2d") {
-    // argument list of CustomCallArgsForCudnnPoolForward (custom_call.cc:520-590)
-    api            = "cinn_call_cudnn_pool2d_forward";
+  } else if (op == "pool2d" || op == "pool2d_grad") {
+    // argument list of CustomCallArgsForCudnnPoolForward / ...PoolBackward (custom_call.cc:520-640): the gradient
+    // takes x, y and dy and passes the extents of x and y
+    api            = op == "pool2d" ? "cinn_call_cudnn_pool2d_forward" : "cinn_call_cudnn_pool2d_backward";
     auto ksize     = GetAttr<std::vector<int>>(n->attrs, "kernel_size", {1, 1});
     auto stride    = GetAttr<std::vector<int>>(n->attrs, "stride_size", {1, 1});
     auto padding   = GetAttr<std::vector<int>>(n->attrs, "padding_size", {0, 0, 0, 0});
@@ -1427,7 +1449,7 @@ ir::LoweredFuncRef OpLowerer::LowerLibraryCall(const Group& group) const {
     auto layout    = GetAttr<std::string>(n->attrs, "data_format", "NCHW");
     bool nchw      = layout == "NCHW";
     const auto& x  = n->inputs[0]->shape;
-    const auto& y  = n->outputs[0]->shape;
+    const auto& y  = op == "pool2d" ? n->outputs[0]->shape : n->inputs[1]->shape;
     int ih = nchw ? x[2] : x[1], iw = nchw ? x[3] : x[2];
     int oh = nchw ? y[2] : y[1], ow = nchw ? y[3] : y[2];
     if (global) {
@@ -1435,7 +1457,9 @@ ir::LoweredFuncRef OpLowerer::LowerLibraryCall(const Group& group) const {
       stride  = {ih, iw};
       padding = {0, 0, 0, 0};
     } else if (adaptive) {
-      CINN_CHECK(ih % oh == 0 && iw % ow == 0) << "adaptive pool2d needs output sizes that divide the input";
+      // windows of floor(extent / outputs), side by side from the first row / column; what is left over at the end is
+      // not read (PoolImpl, cinn/hlir/pe/nn.cc:1073-1112)
+      CINN_CHECK(oh > 0 && ow > 0 && ih >= oh && iw >= ow) << "adaptive pool2d: more outputs than inputs";
       ksize   = {ih / oh, iw / ow};
       stride  = ksize;
       padding = {0, 0, 0, 0};

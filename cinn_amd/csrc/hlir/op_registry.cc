@@ -529,6 +529,27 @@ OpRegistry::OpRegistry() {
       CINN_CHECK(in[0].size() == 4 && in[1].size() == 4) << "conv2d: 4-D input and filter expected";
       CINN_CHECK(layout == "NCHW" || layout == "NHWC") << "conv2d: unknown data_format " << layout;
       ShapeType out(4);
+      // the gradients (InferShapeForConv2d, cinn/hlir/op/nn.cc:529-552): backward_data takes (w, dy) and gives dx with
+      // the spatial extents of `output_shape`; backward_filter takes (x, dy) and gives dw with those of `output_shape`
+      auto conv_type = GetAttr<std::string>(a, "conv_type", "forward");
+      CINN_CHECK(conv_type == "forward" || conv_type == "backward_data" || conv_type == "backward_filter")
+          << "The conv type should be one of {forward, backward_data, backward_filter}.";
+      if (conv_type != "forward") {
+        auto wanted = GetAttr<std::vector<int>>(a, "output_shape", {});
+        CINN_CHECK_EQ(wanted.size(), 4u) << "conv2d " << conv_type << ": output_shape must have rank 4";
+        int groups = GetAttr<int>(a, "groups", 1);
+        int c = layout == "NCHW" ? 1 : 3, h = layout == "NCHW" ? 2 : 1, w = h + 1;
+        if (conv_type == "backward_data") {
+          out[0] = in[1][0];
+          out[c] = in[0][c] * groups;
+        } else {
+          out[0] = in[1][c];
+          out[c] = in[0][c] / groups;
+        }
+        out[h] = wanted[h];
+        out[w] = wanted[w];
+        return std::vector<ShapeType>{out};
+      }
       // "input_layout" = "NCHW" on a channels-last convolution: the input (and the [O][I][KH][KW] filter) are still
       // NCHW, only the output is NHWC (the convolution of a network's image input)
       bool nchw_input = GetAttr<std::string>(a, "input_layout", layout) == "NCHW";
@@ -626,6 +647,21 @@ OpRegistry::OpRegistry() {
         out[wi] = od(in[0][wi], ksize[1], padding[1], padding[3], stride[1]);
       }
       return std::vector<ShapeType>{out};
+    };
+    op.infer_dtype = SameTypeAsFirst;
+  }
+  {
+    // inputs x, y = pool2d(x), dy; the gradient has x's shape (cinn/hlir/op/nn.cc pool2d_grad)
+    auto& op       = r->Register("pool2d_grad");
+    op.pattern     = OpPatternKind::kNonFusible;
+    op.num_inputs  = 3;
+    op.infer_shape = [](const std::vector<ShapeType>& in, const AttributeMap&) {
+      CINN_CHECK(in[0].size() == 4 && in[1].size() == 4 && in[2].size() == 4) << "pool2d_grad: x, y and dy must be 4-D";
+      int64_t ny = 1, ndy = 1;
+      for (int d : in[1]) ny *= d;
+      for (int d : in[2]) ndy *= d;
+      CINN_CHECK(ndy >= ny) << "pool2d_grad: dy holds fewer elements than y";
+      return std::vector<ShapeType>{in[0]};
     };
     op.infer_dtype = SameTypeAsFirst;
   }

@@ -2,7 +2,7 @@
 // cinn_call_cudnn_conv2d_backward_filter (cinn/runtime/cuda/cuda_util.cc:722-967), cinn_call_cudnn_pool2d_backward
 // (1043-1119) and cinn_call_cudnn_softmax_backward (1169-1217).  Same argument lists and tensor formats
 // (0 = NCHW with [F][C][KH][KW] filters, 1 = NHWC with [F][KH][KW][C] filters), results
-// out = alpha * gradient + beta * out, fp32 accumulation for fp32 / fp16 / bf16 tensors.
+// out = alpha * gradient + beta * out, fp32 accumulation for fp32 / fp16 / bf16 tensors, fp64 for fp64 tensors.
 //
 // These are the straightforward gather forms - one thread (or, for the filter gradient, one block) per gradient
 // element, summing its contributions in a fixed order - not tiled MFMA kernels: the inference path never calls them.
@@ -31,15 +31,28 @@ cinn_buffer_t* Arg(void* v_args, int index) {
   return static_cast<cinn_buffer_t*>(args[index].value_.v_handle);
 }
 
-enum class Elem { kF32, kF16, kBF16 };
+enum class Elem { kF32, kF16, kBF16, kF64 };
 Elem ElemOf(const cinn_buffer_t* b) {
   const int bytes = b->type.bits / CHAR_BIT;
+  if (b->type.code == cinn_type_float && bytes == 8) return Elem::kF64;
   if (b->type.code == cinn_type_float && bytes == 4) return Elem::kF32;
   if (b->type.code == cinn_type_float && bytes == 2) return Elem::kF16;
   if (b->type.code == cinn_type_bfloat) return Elem::kBF16;
   fprintf(stderr, "backward intrinsic: unsupported data type code %d bits %d\n", b->type.code, b->type.bits);
   abort();
 }
+
+// the type sums are kept in
+template <typename T>
+struct AccOf {
+  typedef float type;
+};
+template <>
+struct AccOf<double> {
+  typedef double type;
+};
+__device__ __forceinline__ float Fma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double Fma(double a, double b, double c) { return __builtin_fma(a, b, c); }
 
 struct ConvDims {
   int n, c, ih, iw;      // input
@@ -79,7 +92,8 @@ conv_backward_data_kernel(const T* __restrict__ w, const T* __restrict__ dy, T* 
   }
   const int g = c / p.fc, cl = c - g * p.fc;
   const int fg = p.f / p.groups;
-  float acc = 0.0f;
+  typedef typename AccOf<T>::type Acc;
+  Acc acc = 0;
   for (int fl = 0; fl < fg; ++fl) {
     const int f = g * fg + fl;
     for (int ky = 0; ky < p.kh; ++ky) {
@@ -92,13 +106,13 @@ conv_backward_data_kernel(const T* __restrict__ w, const T* __restrict__ dy, T* 
         if (tx < 0 || tx % p.sw != 0) continue;
         const int ox = tx / p.sw;
         if (ox >= p.ow) continue;
-        acc = __builtin_fmaf((float)dy[TensorAt(p.nhwc, p.f, p.oh, p.ow, n, f, oy, ox)],
-                             (float)w[FilterAt(p.nhwc, p.fc, p.kh, p.kw, f, cl, ky, kx)], acc);
+        acc = Fma((Acc)dy[TensorAt(p.nhwc, p.f, p.oh, p.ow, n, f, oy, ox)],
+                  (Acc)w[FilterAt(p.nhwc, p.fc, p.kh, p.kw, f, cl, ky, kx)], acc);
       }
     }
   }
-  float v = p.alpha * acc;
-  if (p.beta != 0.0f) v += p.beta * (float)dx[idx];
+  Acc v = (Acc)p.alpha * acc;
+  if (p.beta != 0.0f) v += (Acc)p.beta * (Acc)dx[idx];
   dx[idx] = (T)v;
 }
 
@@ -106,7 +120,8 @@ conv_backward_data_kernel(const T* __restrict__ w, const T* __restrict__ dy, T* 
 template <typename T>
 __global__ void __launch_bounds__(256)
 conv_backward_filter_kernel(const T* __restrict__ x, const T* __restrict__ dy, T* __restrict__ dw, ConvDims p) {
-  __shared__ float partial[256];
+  typedef typename AccOf<T>::type Acc;
+  __shared__ Acc partial[256];
   const int64_t e = blockIdx.x;  // dw in its own memory order
   int f, cl, ky, kx;
   if (p.nhwc) {
@@ -123,15 +138,15 @@ conv_backward_filter_kernel(const T* __restrict__ x, const T* __restrict__ dy, T
   const int fg = p.f / p.groups;
   const int c  = (f / fg) * p.fc + cl;
   const int64_t positions = (int64_t)p.n * p.oh * p.ow;
-  float acc = 0.0f;
+  Acc acc = 0;
   for (int64_t q = threadIdx.x; q < positions; q += 256) {
     const int ox = (int)(q % p.ow);
     const int oy = (int)((q / p.ow) % p.oh);
     const int n  = (int)(q / ((int64_t)p.ow * p.oh));
     const int iy = oy * p.sh - p.ph + ky * p.dh, ix = ox * p.sw - p.pw + kx * p.dw;
     if (iy < 0 || iy >= p.ih || ix < 0 || ix >= p.iw) continue;
-    acc = __builtin_fmaf((float)x[TensorAt(p.nhwc, p.c, p.ih, p.iw, n, c, iy, ix)],
-                         (float)dy[TensorAt(p.nhwc, p.f, p.oh, p.ow, n, f, oy, ox)], acc);
+    acc = Fma((Acc)x[TensorAt(p.nhwc, p.c, p.ih, p.iw, n, c, iy, ix)],
+              (Acc)dy[TensorAt(p.nhwc, p.f, p.oh, p.ow, n, f, oy, ox)], acc);
   }
   partial[threadIdx.x] = acc;
   __syncthreads();
@@ -140,8 +155,8 @@ conv_backward_filter_kernel(const T* __restrict__ x, const T* __restrict__ dy, T
     __syncthreads();
   }
   if (threadIdx.x == 0) {
-    float v = p.alpha * partial[0];
-    if (p.beta != 0.0f) v += p.beta * (float)dw[e];
+    Acc v = (Acc)p.alpha * partial[0];
+    if (p.beta != 0.0f) v += (Acc)p.beta * (Acc)dw[e];
     dw[e] = (T)v;
   }
 }
@@ -171,9 +186,10 @@ pool_backward_kernel(const T* __restrict__ x, const T* __restrict__ y, const T* 
     c  = (int)((idx / ((int64_t)p.iw * p.ih)) % p.c);
     n  = (int)(idx / ((int64_t)p.iw * p.ih * p.c));
   }
+  typedef typename AccOf<T>::type Acc;
   const bool is_max = p.mode == 0 || p.mode == 3;
-  const float mine  = (float)x[idx];
-  float acc = 0.0f;
+  const Acc mine    = (Acc)x[idx];
+  Acc acc = 0;
   // windows (oy, ox) that contain (iy, ix): oy * sh - ph <= iy < oy * sh - ph + kh
   for (int oy = 0; oy < p.oh; ++oy) {
     const int ys = oy * p.sh - p.ph;
@@ -182,9 +198,9 @@ pool_backward_kernel(const T* __restrict__ x, const T* __restrict__ y, const T* 
       const int xs = ox * p.sw - p.pw;
       if (ix < xs || ix >= xs + p.kw) continue;
       const int64_t o = TensorAt(p.nhwc, p.c, p.oh, p.ow, n, c, oy, ox);
-      const float g   = (float)dy[o];
+      const Acc g     = (Acc)dy[o];
       if (is_max) {
-        const float m = (float)y[o];
+        const Acc m = (Acc)y[o];
         if (mine != m) continue;
         // the first element of the window (rows, then columns) that equals the maximum takes the gradient
         bool first = true;
@@ -195,24 +211,24 @@ pool_backward_kernel(const T* __restrict__ x, const T* __restrict__ y, const T* 
             const int xx = xs + rx;
             if (xx < 0 || xx >= p.iw) continue;
             if (yy == iy && xx == ix) { ry = p.kh; break; }
-            if ((float)x[TensorAt(p.nhwc, p.c, p.ih, p.iw, n, c, yy, xx)] == m) { first = false; break; }
+            if ((Acc)x[TensorAt(p.nhwc, p.c, p.ih, p.iw, n, c, yy, xx)] == m) { first = false; break; }
           }
         }
         if (first) acc += g;
       } else {
-        float factor = (float)(p.kh * p.kw);
+        Acc factor = (Acc)(p.kh * p.kw);
         if (p.mode == 2) {
           const int y0 = ys > 0 ? ys : 0, x0 = xs > 0 ? xs : 0;
           const int y1 = ys + p.kh < p.ih ? ys + p.kh : p.ih, x1 = xs + p.kw < p.iw ? xs + p.kw : p.iw;
           const int count = (y1 - y0) * (x1 - x0);
-          factor          = (float)(count > 1 ? count : 1);
+          factor          = (Acc)(count > 1 ? count : 1);
         }
         acc += g / factor;
       }
     }
   }
-  float v = p.alpha * acc;
-  if (p.beta != 0.0f) v += p.beta * (float)dx[idx];
+  Acc v = (Acc)p.alpha * acc;
+  if (p.beta != 0.0f) v += (Acc)p.beta * (Acc)dx[idx];
   dx[idx] = (T)v;
 }
 
@@ -284,6 +300,9 @@ void cinn_call_cudnn_conv2d_backward_data(void* v_args, int num_args, int format
   dim3 grid((unsigned)((total + 255) / 256));
   auto s = static_cast<hipStream_t>(stream);
   switch (ElemOf(dx)) {
+    case Elem::kF64:
+      hipLaunchKernelGGL(conv_backward_data_kernel<double>, grid, dim3(256), 0, s, reinterpret_cast<const double*>(w->memory), reinterpret_cast<const double*>(dy->memory), reinterpret_cast<double*>(dx->memory), p);
+      break;
     case Elem::kF32:
       hipLaunchKernelGGL(conv_backward_data_kernel<float>, grid, dim3(256), 0, s, reinterpret_cast<const float*>(w->memory),
                          reinterpret_cast<const float*>(dy->memory), reinterpret_cast<float*>(dx->memory), p);
@@ -319,6 +338,9 @@ void cinn_call_cudnn_conv2d_backward_filter(void* v_args, int num_args, int form
   dim3 grid((unsigned)total);
   auto s = static_cast<hipStream_t>(stream);
   switch (ElemOf(dw)) {
+    case Elem::kF64:
+      hipLaunchKernelGGL(conv_backward_filter_kernel<double>, grid, dim3(256), 0, s, reinterpret_cast<const double*>(x->memory), reinterpret_cast<const double*>(dy->memory), reinterpret_cast<double*>(dw->memory), p);
+      break;
     case Elem::kF32:
       hipLaunchKernelGGL(conv_backward_filter_kernel<float>, grid, dim3(256), 0, s, reinterpret_cast<const float*>(x->memory),
                          reinterpret_cast<const float*>(dy->memory), reinterpret_cast<float*>(dw->memory), p);
@@ -361,6 +383,10 @@ void cinn_call_cudnn_pool2d_backward(void* v_args, int num_args, int mode, int f
   dim3 grid((unsigned)((total + 255) / 256));
   auto s = static_cast<hipStream_t>(stream);
   switch (ElemOf(dx)) {
+    case Elem::kF64:
+      hipLaunchKernelGGL(pool_backward_kernel<double>, grid, dim3(256), 0, s, reinterpret_cast<const double*>(x->memory), reinterpret_cast<const double*>(y->memory), reinterpret_cast<const double*>(dy->memory),
+                         reinterpret_cast<double*>(dx->memory), p);
+      break;
     case Elem::kF32:
       hipLaunchKernelGGL(pool_backward_kernel<float>, grid, dim3(256), 0, s, reinterpret_cast<const float*>(x->memory),
                          reinterpret_cast<const float*>(y->memory), reinterpret_cast<const float*>(dy->memory),
@@ -399,6 +425,7 @@ void cinn_call_cudnn_softmax_backward(void* v_args, int num_args, int mode, int 
   dim3 grid((unsigned)groups);
   auto s = static_cast<hipStream_t>(stream);
   switch (ElemOf(dx)) {
+    case Elem::kF64: CINN_RT_CHECK(false, "softmax_backward: fp64 tensors are not implemented"); break;
     case Elem::kF32:
       hipLaunchKernelGGL(log_softmax_backward_kernel<float>, grid, dim3(256), 0, s, reinterpret_cast<const float*>(y->memory),
                          reinterpret_cast<const float*>(dy->memory), reinterpret_cast<float*>(dx->memory), len, inner, alpha, beta);

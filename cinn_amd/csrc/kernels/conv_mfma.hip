@@ -271,6 +271,52 @@ const KEntry* GetTable(const ConvParams& p, int dh, int dw) {
   return dev;
 }
 
+// fp64 tensors (no matrix-core path is wired for them): one thread per output element, products added in
+// (channel, filter row, filter column) order.  nhwc: x [N][H][W][C], w [F][KH][KW][C/groups], y [N][OH][OW][F].
+struct DirectConvDims {
+  int n, c, ih, iw, f, fc, kh, kw, oh, ow, ph, pw, sh, sw, dh, dw, groups, nhwc;
+  double alpha, beta;
+};
+__global__ void __launch_bounds__(256)
+conv2d_f64_kernel(const double* __restrict__ x, const double* __restrict__ w, double* __restrict__ y, DirectConvDims p) {
+  const int64_t total = (int64_t)p.n * p.f * p.oh * p.ow;
+  const int64_t idx   = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  int n, f, oy, ox;
+  if (p.nhwc) {
+    f  = (int)(idx % p.f);
+    ox = (int)((idx / p.f) % p.ow);
+    oy = (int)((idx / ((int64_t)p.f * p.ow)) % p.oh);
+    n  = (int)(idx / ((int64_t)p.f * p.ow * p.oh));
+  } else {
+    ox = (int)(idx % p.ow);
+    oy = (int)((idx / p.ow) % p.oh);
+    f  = (int)((idx / ((int64_t)p.ow * p.oh)) % p.f);
+    n  = (int)(idx / ((int64_t)p.ow * p.oh * p.f));
+  }
+  const int c0 = (f / (p.f / p.groups)) * p.fc;
+  double acc   = 0.0;
+  for (int cl = 0; cl < p.fc; ++cl) {
+    const int c = c0 + cl;
+    for (int ky = 0; ky < p.kh; ++ky) {
+      const int iy = oy * p.sh - p.ph + ky * p.dh;
+      if (iy < 0 || iy >= p.ih) continue;
+      for (int kx = 0; kx < p.kw; ++kx) {
+        const int ix = ox * p.sw - p.pw + kx * p.dw;
+        if (ix < 0 || ix >= p.iw) continue;
+        const int64_t xi = p.nhwc ? (((int64_t)n * p.ih + iy) * p.iw + ix) * p.c + c
+                                  : (((int64_t)n * p.c + c) * p.ih + iy) * p.iw + ix;
+        const int64_t wi = p.nhwc ? (((int64_t)f * p.kh + ky) * p.kw + kx) * p.fc + cl
+                                  : (((int64_t)f * p.fc + cl) * p.kh + ky) * p.kw + kx;
+        acc = __builtin_fma(x[xi], w[wi], acc);
+      }
+    }
+  }
+  double v = p.alpha * acc;
+  if (p.beta != 0.0) v += p.beta * y[idx];
+  y[idx] = v;
+}
+
 cinn_buffer_t* BufferArg(void* v_args, int index) {
   auto* args = static_cast<cinn_pod_value_t*>(v_args);
   CINN_RT_CHECK(args[index].type_code_ == CINN_POD_BUFFER_P, "conv2d: argument %d is not a buffer", index);
@@ -290,6 +336,16 @@ void RunConv(cinn_buffer_t* x, cinn_buffer_t* w, cinn_buffer_t* y, const float* 
   CINN_RT_CHECK(oh == want_oh && ow == want_ow, "conv2d: output is %dx%d, the shapes give %dx%d", oh, ow, want_oh, want_ow);
   CINN_RT_CHECK((int64_t)in * ic * ih * iw < INT_MAX && (int64_t)on * oc * oh * ow < INT_MAX, "conv2d: tensor too large");
   CINN_RT_CHECK(fh * dh < 32768 && fw * dw < 32768, "conv2d: filter extent too large");
+  if (x->type.code == cinn_type_float && x->type.bits == 64) {
+    CINN_RT_CHECK(format != 2 && epilogue == 0, "conv2d: fp64 tensors take the plain convolution in NCHW or NHWC only");
+    DirectConvDims d{in, ic, ih, iw, fn, fc, fh, fw, oh, ow, ph, pw, sh, sw, dh, dw, groups, format == 1, alpha, beta};
+    const int64_t total = (int64_t)on * oc * oh * ow;
+    hipLaunchKernelGGL(conv2d_f64_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                       reinterpret_cast<const double*>(x->memory), reinterpret_cast<const double*>(w->memory),
+                       reinterpret_cast<double*>(y->memory), d);
+    CINN_HIP_CALL(hipGetLastError());
+    return;
+  }
   if (format != 0) {
     // channels-last output; format 2 reads an NCHW input and [OC][IC][KH][KW] weights
     cinn_hip_kernels::ConvNhwcArgs a;

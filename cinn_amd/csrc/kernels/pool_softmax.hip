@@ -74,6 +74,68 @@ __global__ void __launch_bounds__(256) pool2d_nchw_kernel(const T* __restrict__ 
 }
 
 
+// fp64 tensors, either layout: one thread per output element, the arithmetic of the kernel above in double
+__global__ void __launch_bounds__(256) pool2d_f64_kernel(const double* __restrict__ in, double* __restrict__ out, PoolParams p,
+                                                         int nhwc) {
+  const int64_t total = (int64_t)p.n * p.c * p.oh * p.ow;
+  const int64_t idx   = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  int x, y, c;
+  int64_t n;
+  if (nhwc) {
+    c = (int)(idx % p.c);
+    x = (int)((idx / p.c) % p.ow);
+    y = (int)((idx / ((int64_t)p.c * p.ow)) % p.oh);
+    n = idx / ((int64_t)p.c * p.ow * p.oh);
+  } else {
+    x = (int)(idx % p.ow);
+    y = (int)((idx / p.ow) % p.oh);
+    c = (int)((idx / ((int64_t)p.ow * p.oh)) % p.c);
+    n = idx / ((int64_t)p.ow * p.oh * p.c);
+  }
+  auto at = [&](int yy, int xx) -> double {
+    return nhwc ? in[((n * p.ih + yy) * p.iw + xx) * p.c + c] : in[((n * p.c + c) * p.ih + yy) * p.iw + xx];
+  };
+  const int ys = y * p.sh - p.ph, xs = x * p.sw - p.pw;
+  double result;
+  if (p.mode == 0 || p.mode == 3) {
+    double m = -1.7976931348623157e+308;
+    for (int ry = 0; ry < p.kh; ++ry) {
+      const int yy = ys + ry;
+      if (yy < 0 || yy >= p.ih) continue;
+      for (int rx = 0; rx < p.kw; ++rx) {
+        const int xx = xs + rx;
+        if (xx < 0 || xx >= p.iw) continue;
+        const double v = at(yy, xx);
+        m              = v > m ? v : m;
+      }
+    }
+    result = m;
+  } else {
+    double factor = (double)(p.kh * p.kw);
+    if (p.mode == 2) {
+      const int y0 = ys > 0 ? ys : 0, x0 = xs > 0 ? xs : 0;
+      const int y1 = ys + p.kh < p.ih ? ys + p.kh : p.ih, x1 = xs + p.kw < p.iw ? xs + p.kw : p.iw;
+      const int count = (y1 - y0) * (x1 - x0);
+      factor          = (double)(count > 1 ? count : 1);
+    }
+    double acc = 0.0;
+    for (int ry = 0; ry < p.kh; ++ry) {
+      const int yy = ys + ry;
+      for (int rx = 0; rx < p.kw; ++rx) {
+        const int xx = xs + rx;
+        double v     = 0.0;
+        if (yy >= 0 && yy < p.ih && xx >= 0 && xx < p.iw) v = at(yy, xx);
+        acc += v / factor;
+      }
+    }
+    result = acc;
+  }
+  double v = (double)p.alpha * result;
+  if (p.beta != 0.0f) v += (double)p.beta * out[idx];
+  out[idx] = v;
+}
+
 // Channels-last pooling: one thread per output pixel and group of V consecutive channels (V elements = 16 bytes
 // when the channel count allows), so that every access is one contiguous vector and consecutive lanes read
 // consecutive vectors.  Arithmetic and order of operations are those of the NCHW kernel.
@@ -314,9 +376,10 @@ cinn_buffer_t* BufferArg(void* v_args, int index) {
   return static_cast<cinn_buffer_t*>(args[index].value_.v_handle);
 }
 
-enum class Elem { kF32, kF16, kBF16 };
+enum class Elem { kF32, kF16, kBF16, kF64 };
 Elem ElemOf(const cinn_buffer_t* b) {
   const int bytes = b->type.bits / CHAR_BIT;
+  if (b->type.code == cinn_type_float && bytes == 8) return Elem::kF64;
   if (b->type.code == cinn_type_float && bytes == 4) return Elem::kF32;
   if (b->type.code == cinn_type_float && bytes == 2) return Elem::kF16;
   if (b->type.code == cinn_type_bfloat) return Elem::kBF16;
@@ -350,8 +413,15 @@ void cinn_call_cudnn_pool2d_forward(void* v_args, int num_args, int mode, int fo
   CINN_RT_CHECK((int64_t)input_c * input_h * input_w * input_n < INT_MAX && total < INT_MAX, "pool2d: tensor too large");
   dim3 grid((unsigned)((total + 255) / 256));
   auto s = static_cast<hipStream_t>(stream);
+  if (ElemOf(x) == Elem::kF64) {
+    hipLaunchKernelGGL(pool2d_f64_kernel, grid, dim3(256), 0, s, reinterpret_cast<const double*>(x->memory),
+                       reinterpret_cast<double*>(y->memory), p, format);
+    CINN_HIP_CALL(hipGetLastError());
+    return;
+  }
   if (format == 1) {
     switch (ElemOf(x)) {
+      case Elem::kF64: break;  // taken above
       case Elem::kF32: LaunchPoolNhwc<float>(x->memory, y->memory, p, s); break;
       case Elem::kF16: LaunchPoolNhwc<_Float16>(x->memory, y->memory, p, s); break;
       case Elem::kBF16: LaunchPoolNhwc<__bf16>(x->memory, y->memory, p, s); break;
@@ -360,6 +430,7 @@ void cinn_call_cudnn_pool2d_forward(void* v_args, int num_args, int mode, int fo
     return;
   }
   switch (ElemOf(x)) {
+    case Elem::kF64: break;  // taken above
     case Elem::kF32:
       hipLaunchKernelGGL(pool2d_nchw_kernel<float>, grid, dim3(256), 0, s, reinterpret_cast<const float*>(x->memory),
                          reinterpret_cast<float*>(y->memory), p);
@@ -395,6 +466,7 @@ void cinn_call_cudnn_softmax_forward(void* v_args, int num_args, int mode, int f
   dim3 grid((unsigned)groups);
   auto s = static_cast<hipStream_t>(stream);
   switch (ElemOf(x)) {
+    case Elem::kF64: CINN_RT_CHECK(false, "softmax: fp64 tensors are not implemented"); break;
     case Elem::kF32:
       hipLaunchKernelGGL(log_softmax_kernel<float>, grid, dim3(256), 0, s, reinterpret_cast<const float*>(x->memory),
                          reinterpret_cast<float*>(y->memory), len, inner, alpha, beta);

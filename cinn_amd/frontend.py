@@ -195,8 +195,9 @@ class NetBuilder(object):
     def softmax(self, x, axes=(-1,), mode="fast", data_format="AnyLayout"):
         return self._call1("Softmax", [x], axes=list(axes), mode=mode, data_format=data_format)
 
-    def matmul(self, x, y, trans_x=False, trans_y=False, alpha=1.0):
-        return self._call1("Matmul", [x, y], trans_x=trans_x, trans_y=trans_y, alpha=float(alpha))
+    def matmul(self, x, y, transpose_x=False, transpose_y=False, alpha=1.0):
+        """Argument names of cinn/pybind/frontend.cc:653-659."""
+        return self._call1("Matmul", [x, y], trans_x=transpose_x, trans_y=transpose_y, alpha=float(alpha))
 
     def mul(self, x, y, x_num_col_dims=1, y_num_col_dims=1, is_infer=False):
         return self._call1("Mul", [x, y], x_num_col_dims=x_num_col_dims, y_num_col_dims=y_num_col_dims,
@@ -208,14 +209,32 @@ class NetBuilder(object):
                            dilations=list(dilations), groups=groups, data_format=data_format,
                            padding_algorithm=padding_algorithm)
 
+    def conv(self, x, w, strides=(1, 1), paddings=(0, 0), dilations=(1, 1), groups=1, conv_type="forward",
+             data_format="NCHW", padding_algorithm="EXPLICIT", output_shape=()):
+        """conv2d (x, w), its data gradient (w, dy -> dx of `output_shape`) or its filter gradient (x, dy -> dw of
+        `output_shape`): cinn/pybind/frontend.cc `conv`."""
+        return self._call1("Conv", [x, w], strides=list(strides), paddings=list(paddings),
+                           dilations=list(dilations), groups=groups, conv_type=conv_type, data_format=data_format,
+                           padding_algorithm=padding_algorithm, output_shape=list(output_shape))
+
     def batchnorm(self, x, scale, bias, mean, variance, epsilon=1e-5, momentum=0.9, data_layout="NCHW", is_test=True):
         return self._call("BatchNorm", [x, scale, bias, mean, variance], epsilon=float(epsilon),
                           momentum=float(momentum), data_layout=data_layout, is_test=is_test)
 
-    def pool2d(self, x, pooling_type, ksize, strides=(1, 1), paddings=(0, 0), ceil_mode=False, exclusive=True,
+    def pool2d(self, x, pooling_type, kernel_size, stride=(1, 1), padding=(0, 0), ceil_mode=False, exclusive=True,
                global_pooling=False, data_format="NCHW", adaptive=False, padding_algorithm="EXPLICIT"):
-        return self._call1("Pool2d", [x], pooling_type=pooling_type, ksize=list(ksize), strides=list(strides),
-                           paddings=list(paddings), ceil_mode=ceil_mode, exclusive=exclusive,
+        """Argument names of cinn/pybind/frontend.cc:586-598."""
+        return self._call1("Pool2d", [x], pooling_type=pooling_type, ksize=list(kernel_size), strides=list(stride),
+                           paddings=list(padding), ceil_mode=ceil_mode, exclusive=exclusive,
+                           global_pooling=global_pooling, data_format=data_format, adaptive=adaptive,
+                           padding_algorithm=padding_algorithm)
+
+    def pool2d_grad(self, x, y, dy, pooling_type, kernel_size, stride=(1, 1), padding=(0, 0), ceil_mode=False,
+                    exclusive=True, global_pooling=False, data_format="NCHW", adaptive=False,
+                    padding_algorithm="EXPLICIT"):
+        """Gradient of pool2d with respect to x (cinn/pybind/frontend.cc:599-613)."""
+        return self._call1("Pool2dGrad", [x, y, dy], pooling_type=pooling_type, ksize=list(kernel_size),
+                           strides=list(stride), paddings=list(padding), ceil_mode=ceil_mode, exclusive=exclusive,
                            global_pooling=global_pooling, data_format=data_format, adaptive=adaptive,
                            padding_algorithm=padding_algorithm)
 

@@ -68,7 +68,7 @@ def test_matmul_conv_pool_shapes():
     a = b.create_input(Float(32), [8, 16], "a")
     w = b.create_input(Float(32), [16, 4], "w")
     assert b.matmul(a, w).shape() == [8, 4]
-    assert b.matmul(w, a, trans_x=True, trans_y=True).shape() == [4, 8]
+    assert b.matmul(w, a, transpose_x=True, transpose_y=True).shape() == [4, 8]
     ba = b.create_input(Float(32), [3, 8, 16], "ba")
     assert b.matmul(ba, w).shape() == [3, 8, 4]
     x = b.create_input(Float(32), [32, 256, 56, 56], "xc")
@@ -370,3 +370,35 @@ def test_max_pooling_after_the_image_convolution_is_folded_into_it():
         assert "pool2d" in groups, (kwargs, opts)
     b, y = _image_stem(Float(32))
     assert "pool2d" in compile_only(b, [y]).fusion_groups()
+
+
+def test_conv_gradients_and_pool2d_grad_shapes_and_lowering():
+    """builder.conv with conv_type backward_data takes (w, dy) and gives dx, backward_filter takes (x, dy) and gives dw,
+    with the extents of `output_shape` (InferShapeForConv2d, cinn/hlir/op/nn.cc:529-552); pool2d_grad takes x, y, dy
+    and gives x's shape.  Each is one library-call instruction; a wrong conv_type or a missing output_shape is refused."""
+    from cinn_amd.common import Float
+    for fmt, xs, ws, dys in (("NCHW", [3, 16, 32, 32], [8, 16, 3, 3], [3, 8, 15, 15]),
+                             ("NHWC", [3, 32, 32, 16], [8, 3, 3, 16], [3, 15, 15, 8])):
+        b = NetBuilder("t")
+        x, w, dy = b.create_input(Float(32), xs, "x"), b.create_input(Float(32), ws, "w"), b.create_input(Float(32), dys, "dy")
+        y = b.conv(x, w, strides=[2, 2], data_format=fmt)
+        assert y.shape() == dys
+        dx = b.conv(w, dy, strides=[2, 2], conv_type="backward_data", data_format=fmt, output_shape=xs)
+        dw = b.conv(x, dy, strides=[2, 2], conv_type="backward_filter", data_format=fmt, output_shape=ws)
+        assert dx.shape() == xs and dw.shape() == ws
+        comp = compile_only(b, [y, dx, dw])
+        names = [comp.instruction_info(i)[0] for i in range(comp.num_instructions())]
+        assert sum("_conv2d_" in n for n in names) == 3  # beside them: layout changes around the forward convolution
+        with pytest.raises(Exception, match="conv type"):
+            b.conv(x, w, conv_type="sideways", data_format=fmt)
+        with pytest.raises(Exception, match="output_shape"):
+            b.conv(w, dy, conv_type="backward_data", data_format=fmt)
+    b = NetBuilder("t")
+    x = b.create_input(Float(16), [2, 4, 9, 9], "x")
+    y = b.pool2d(x, "max", [3, 3], stride=[2, 2], padding=[1, 1])
+    dy = b.create_input(Float(16), y.shape(), "dy")
+    dx = b.pool2d_grad(x, y, dy, "max", [3, 3], stride=[2, 2], padding=[1, 1])
+    assert y.shape() == [2, 4, 5, 5] and dx.shape() == [2, 4, 9, 9] and str(dx.type()) == "float16"
+    assert compile_only(b, [y, dx]).num_instructions() == 2
+    # adaptive average pooling: windows of floor(extent / outputs) (PoolImpl, cinn/hlir/pe/nn.cc:1073-1112)
+    assert b.pool2d(x, "avg", [4, 4], adaptive=True).shape() == [2, 4, 4, 4]

@@ -298,7 +298,7 @@ def test_golden_fixtures_through_netbuilder(gpu):
     assert comp.instruction_info(0)[0].startswith("fn_mm_matmul")
     b = NetBuilder("mmt")
     A, B = b.create_input(Float(32), f["a"].T.shape, "a"), b.create_input(Float(32), f["b"].T.shape, "b")
-    (c,), _ = run(b, {A: f["a"].T.copy(), B: f["b"].T.copy()}, [b.matmul(A, B, trans_x=True, trans_y=True)])
+    (c,), _ = run(b, {A: f["a"].T.copy(), B: f["b"].T.copy()}, [b.matmul(A, B, transpose_x=True, transpose_y=True)])
     np.testing.assert_allclose(c, f["c_tt"], rtol=1e-4, atol=1e-7)
     f = load("cfg3_matmul_bf16")
     b = NetBuilder("mmb")

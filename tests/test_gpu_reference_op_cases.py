@@ -1,0 +1,305 @@
+"""The case lists of the reference's own operator tests for the library-backed operators of this path, built with the
+same NetBuilder calls and run through the compiled program (host stubs -> cinn_call_cublas /
+cinn_call_cudnn_conv2d_forward / _backward_data / _backward_filter / cinn_call_cudnn_pool2d_forward / _backward):
+
+  * python/tests/ops/test_matmul_op.py:84-243  - shapes with 1-D operands, broadcast batch dimensions, every transpose
+    combination, fp16 / fp32 / fp64, and the matmul + transpose pair;
+  * python/tests/ops/test_conv2d_op.py:127-195 - 3x3 convolutions in NCHW and NHWC with both gradients
+    (builder.conv(..., conv_type="backward_data" / "backward_filter", output_shape=...)), fp16 / fp32 / fp64;
+  * python/tests/ops/test_pool2d_op.py:80-330  - six forward attribute sets on four shapes and the four gradient sets.
+
+The reference compares with Paddle at the same precision; here the expected values are float64 numpy (matmul), the
+CPU oracle (convolution and its gradients, pooling in fp32 / fp16) or float64 window loops written out below (fp64
+pooling).  Inputs are uniform in [0, 1) as OpTest.random draws them (python/tests/ops/op_test.py).  Tolerances are
+the reference's: matmul fp16 1e-2, fp32 1e-5, fp64 1e-5 (relative, absolute part 1e-6 scaled by the size of the
+sums); convolution fp16 1e-3, fp32 / fp64 1e-5; max pooling exact, average pooling 1e-6 (fp16 1e-3)."""
+import numpy as np
+import pytest
+
+from cinn_amd.common import Float
+from cinn_amd.frontend import NetBuilder
+
+import oracle
+from oracle import backward as ob
+from helpers import run
+
+pytestmark = pytest.mark.gpu
+
+NP_OF = {"float16": (np.float16, 16), "float32": (np.float32, 32), "float64": (np.float64, 64)}
+
+
+def uniform(seed, shape, dtype):
+    return np.random.default_rng(seed).uniform(0.0, 1.0, shape).astype(NP_OF[dtype][0])
+
+
+def close(got, want, rtol, atol):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    assert got.shape == want.shape, (got.shape, want.shape)
+    err = np.abs(got - want)
+    bound = rtol * np.abs(want) + atol
+    assert np.all(err <= bound), "max excess %g at %s" % ((err - bound).max(),
+                                                          np.unravel_index(np.argmax(err - bound), err.shape))
+
+
+# ---- matmul ------------------------------------------------------------------------------------------------------
+MATMUL_SHAPES = [
+    ([1024], [1024]),
+    ([4, 4], [4, 4]),
+    ([4, 16], [16, 32]),
+    ([5, 4, 16], [5, 16, 32]),
+    ([4, 16], [16]),          # matrix times row vector
+    ([4, 16], [16, 1]),       # matrix times column vector
+    ([8, 16, 4], [1, 4, 16]),
+    ([1, 1, 1, 1], [1, 1, 1, 1]),
+]
+MATMUL_TRANS = [
+    ([16, 4], [16, 32], True, False),
+    ([5, 16, 4], [5, 16, 32], True, False),
+    ([8, 4, 16], [4, 16], True, False),
+    ([4, 16], [32, 16], False, True),
+    ([10, 12, 128, 64], [10, 12, 128, 64], False, True),
+    ([16, 4], [32, 16], True, True),
+    ([10, 12, 64, 128], [10, 12, 128, 64], True, True),
+    ([128], [10, 12, 128, 64], True, False),
+]
+
+
+def matmul_f64(x, y, tx, ty):
+    """paddle.matmul / numpy.matmul with the transposes applied to the last two dimensions (a 1-D operand is left
+    as it is: transposing a vector is the identity)."""
+    x, y = x.astype(np.float64), y.astype(np.float64)
+    if tx and x.ndim > 1:
+        x = np.swapaxes(x, -1, -2)
+    if ty and y.ndim > 1:
+        y = np.swapaxes(y, -1, -2)
+    out = np.matmul(x, y)
+    return out.reshape([1]) if out.ndim == 0 else out
+
+
+def run_matmul(x_shape, y_shape, tx, ty, dtype, perm=None):
+    x, y = uniform(1, x_shape, dtype), uniform(2, y_shape, dtype)
+    b = NetBuilder("matmul")
+    X = b.create_input(Float(NP_OF[dtype][1]), x_shape, "x")
+    Y = b.create_input(Float(NP_OF[dtype][1]), y_shape, "y")
+    out = b.matmul(X, Y, transpose_x=tx, transpose_y=ty)
+    if perm is not None:
+        out = b.transpose(out, perm)
+    (got,), _ = run(b, {X: x, Y: y}, [out])
+    want = matmul_f64(x, y, tx, ty)
+    if perm is not None:
+        want = want.transpose(perm)
+    assert got.dtype == NP_OF[dtype][0]
+    k = x_shape[-2] if (tx and len(x_shape) > 1) else x_shape[-1]
+    rtol = 1e-2 if dtype == "float16" else 1e-5
+    atol = (1e-2 if dtype == "float16" else 1e-6) * max(1.0, k / 4.0)   # the sums are about k / 4
+    close(got, want, rtol, atol)
+
+
+@pytest.mark.parametrize("dtype", ["float16", "float32", "float64"])
+@pytest.mark.parametrize("x_shape,y_shape", MATMUL_SHAPES)
+def test_matmul_shapes_and_types(gpu, x_shape, y_shape, dtype):
+    run_matmul(x_shape, y_shape, False, False, dtype)
+
+
+@pytest.mark.parametrize("x_shape,y_shape,tx,ty", MATMUL_TRANS)
+def test_matmul_transposes(gpu, x_shape, y_shape, tx, ty):
+    run_matmul(x_shape, y_shape, tx, ty, "float32")
+
+
+@pytest.mark.parametrize("x_shape,y_shape,perm", [([32, 64], [64, 128], [1, 0]),
+                                                  ([10, 1, 128, 64], [10, 12, 64, 128], [0, 1, 3, 2])])
+def test_matmul_then_transpose(gpu, x_shape, y_shape, perm):
+    run_matmul(x_shape, y_shape, False, False, "float32", perm)
+
+
+# ---- conv2d and its gradients -------------------------------------------------------------------------------------
+CONV_CASES = [
+    ([3, 16, 32, 32], [16, 16, 3, 3], [3, 16, 30, 30], "NCHW"),
+    ([3, 16, 64, 64], [16, 16, 3, 3], [3, 16, 62, 62], "NCHW"),
+    ([3, 32, 32, 16], [16, 16, 3, 3], [3, 30, 30, 16], "NHWC"),
+    ([3, 64, 64, 16], [16, 16, 3, 3], [3, 62, 62, 16], "NHWC"),
+]
+
+
+@pytest.mark.parametrize("dtype", ["float16", "float32", "float64"])
+@pytest.mark.parametrize("x_shape,w_shape,dy_shape,fmt", CONV_CASES)
+def test_conv2d_with_gradients(gpu, x_shape, w_shape, dy_shape, fmt, dtype):
+    if dtype == "float64" and fmt == "NHWC":
+        pytest.skip("the reference's fp64 list holds the NCHW cases only")
+    x, w, dy = uniform(3, x_shape, dtype), uniform(4, w_shape, dtype), uniform(5, dy_shape, dtype)
+    t = Float(NP_OF[dtype][1])
+    b = NetBuilder("cv")
+    X, W, DY = b.create_input(t, x_shape, "x"), b.create_input(t, w_shape, "weight"), b.create_input(t, dy_shape, "dy")
+    if fmt == "NCHW":
+        y = b.conv2d(X, W, strides=[1, 1], paddings=[0, 0], dilations=[1, 1], groups=1, data_format=fmt)
+        dx = b.conv(W, DY, data_format=fmt, conv_type="backward_data", output_shape=X.shape())
+        dw = b.conv(X, DY, data_format=fmt, conv_type="backward_filter", output_shape=W.shape())
+    else:
+        Wt = b.transpose(W, [0, 2, 3, 1])
+        y = b.conv2d(X, Wt, strides=[1, 1], paddings=[0, 0], dilations=[1, 1], groups=1, data_format=fmt)
+        dx = b.conv(Wt, DY, data_format=fmt, conv_type="backward_data", output_shape=X.shape())
+        dw = b.transpose(b.conv(X, DY, data_format=fmt, conv_type="backward_filter", output_shape=Wt.shape()),
+                         [0, 3, 1, 2])
+    (got_y, got_dx, got_dw), comp = run(b, {X: x, W: w, DY: dy}, [y, dx, dw])
+    names = [comp.instruction_info(i)[0] for i in range(comp.num_instructions())]
+    assert sum("_conv2d_" in n for n in names) == 3
+    to_nchw = (lambda a: a.transpose(0, 3, 1, 2)) if fmt == "NHWC" else (lambda a: a)
+    x64, w64, dy64 = to_nchw(x).astype(np.float64), w.astype(np.float64), to_nchw(dy).astype(np.float64)
+    if dtype == "float64":
+        # float64 expected values: the gradients of the oracle work in float64; the forward sum written out
+        want_y = np.zeros(dy64.shape)
+        for ky in range(3):
+            for kx in range(3):
+                want_y += np.einsum("nchw,fc->nfhw", x64[:, :, ky:ky + dy64.shape[2], kx:kx + dy64.shape[3]],
+                                    w64[:, :, ky, kx])
+    else:
+        want_y = oracle.conv2d_nchw(to_nchw(x).astype(np.float32), w.astype(np.float32), (1, 1), (0, 0))
+    want_dx = ob.conv2d_backward_data(w64, dy64, x64.shape)
+    want_dw = ob.conv2d_backward_filter(x64, dy64, w64.shape)
+    rtol = 1e-3 if dtype == "float16" else 1e-5
+    close(to_nchw(got_y), want_y, rtol, rtol)
+    close(to_nchw(got_dx), want_dx, rtol, rtol)
+    close(got_dw, want_dw, rtol, rtol * 10)
+
+
+# ---- pool2d -------------------------------------------------------------------------------------------------------
+POOL_SHAPES = [([1, 3, 32, 32], "NCHW"), ([32, 3, 64, 64], "NCHW"), ([1, 32, 32, 3], "NHWC"), ([32, 64, 64, 3], "NHWC")]
+POOL_ATTRS = [
+    dict(pooling_type="max", kernel_size=[2, 2], stride=[1, 1], padding=[0, 0], padding_algorithm="VALID",
+         global_pooling=False, ceil_mode=False, exclusive=True, adaptive=False),
+    dict(pooling_type="max", kernel_size=[3, 3], stride=[2, 2], padding=[1, 1], padding_algorithm="SAME",
+         global_pooling=False, ceil_mode=True, exclusive=True, adaptive=False),
+    dict(pooling_type="max", kernel_size=[5, 5], stride=[3, 3], padding=[2, 2], padding_algorithm="EXPLICIT",
+         global_pooling=False, ceil_mode=False, exclusive=False, adaptive=False),
+    dict(pooling_type="avg", kernel_size=[2, 2], stride=[1, 1], padding=[0, 0], padding_algorithm="VALID",
+         global_pooling=False, ceil_mode=False, exclusive=True, adaptive=False),
+    dict(pooling_type="avg", kernel_size=[3, 3], stride=[2, 2], padding=[1, 1], padding_algorithm="SAME",
+         global_pooling=True, ceil_mode=False, exclusive=True, adaptive=False),
+    dict(pooling_type="avg", kernel_size=[5, 5], stride=[3, 3], padding=[1, 1], padding_algorithm="EXPLICIT",
+         global_pooling=False, ceil_mode=False, exclusive=True, adaptive=True),
+]
+POOL_GRAD_SHAPES = [([1, 3, 32, 32], "NCHW"), ([1, 32, 32, 3], "NHWC")]
+POOL_GRAD_ATTRS = [
+    dict(pooling_type="max", kernel_size=[5, 5], stride=[2, 2], padding=[0, 0], padding_algorithm="SAME",
+         global_pooling=False, ceil_mode=False, exclusive=True, adaptive=False),
+    dict(pooling_type="max", kernel_size=[3, 3], stride=[2, 2], padding=[1, 1], padding_algorithm="VALID",
+         global_pooling=False, ceil_mode=True, exclusive=False, adaptive=False),
+    dict(pooling_type="avg", kernel_size=[2, 2], stride=[2, 2], padding=[0, 0], padding_algorithm="SAME",
+         global_pooling=True, ceil_mode=False, exclusive=True, adaptive=False),
+    dict(pooling_type="avg", kernel_size=[3, 3], stride=[2, 2], padding=[1, 1], padding_algorithm="EXPLICIT",
+         global_pooling=False, ceil_mode=False, exclusive=True, adaptive=True),
+]
+
+
+def pool_windows(h, w, a):
+    """Kernel, stride and (top, left, bottom, right) padding the operator works with, and its output extents, after
+    the attribute rules of NetBuilder::Pool2d (cinn/frontend/net_builder.cc:538-684) and the adaptive / global forms
+    of PoolImpl (cinn/hlir/pe/nn.cc:956-1112)."""
+    k, s, p = list(a["kernel_size"]), list(a["stride"]), list(a["padding"]) * 2
+    if a["global_pooling"]:
+        return [h, w], [h, w], [0, 0, 0, 0], 1, 1
+    if a["adaptive"]:
+        return [h // k[0], w // k[1]], [h // k[0], w // k[1]], [0, 0, 0, 0], k[0], k[1]
+    if a["padding_algorithm"] == "VALID":
+        p = [0, 0, 0, 0]
+    elif a["padding_algorithm"] == "SAME":
+        oh, ow = -(-h // s[0]), -(-w // s[1])
+        ph, pw = max((oh - 1) * s[0] + k[0] - h, 0), max((ow - 1) * s[1] + k[1] - w, 0)
+        p = [ph // 2, pw // 2, ph - ph // 2, pw - pw // 2]
+
+    def out(n, kk, p0, p1, ss):
+        num = n - kk + p0 + p1
+        return (-(-num // ss) if a["ceil_mode"] else num // ss) + 1
+    return k, s, p, out(h, k[0], p[0], p[2], s[0]), out(w, k[1], p[1], p[3], s[1])
+
+
+def pool_f64(x, k, s, p, oh, ow, is_max, exclusive):
+    """float64 pooling over NCHW: max over the window positions inside the input; average of position / divisor
+    added row by row, the divisor counting the positions inside the input (exclusive) or the whole window."""
+    n, c, h, w = x.shape
+    out = np.empty((n, c, oh, ow))
+    for oy in range(oh):
+        y0, y1 = max(oy * s[0] - p[0], 0), min(oy * s[0] - p[0] + k[0], h)
+        for ox in range(ow):
+            x0, x1 = max(ox * s[1] - p[1], 0), min(ox * s[1] - p[1] + k[1], w)
+            win = x[:, :, y0:y1, x0:x1]
+            if is_max:
+                out[:, :, oy, ox] = win.max(axis=(2, 3))
+            else:
+                div = max((y1 - y0) * (x1 - x0), 1) if exclusive else k[0] * k[1]
+                acc = np.zeros((n, c))
+                for yy in range(y1 - y0):
+                    for xx in range(x1 - x0):
+                        acc += win[:, :, yy, xx] / div
+                out[:, :, oy, ox] = acc
+    return out
+
+
+def expected_pool(x_nchw, a, dtype):
+    k, s, p, oh, ow = pool_windows(x_nchw.shape[2], x_nchw.shape[3], a)
+    is_max = a["pooling_type"] == "max"
+    if dtype == "float64":
+        return pool_f64(x_nchw, k, s, p, oh, ow, is_max, a["exclusive"]), (k, s, p)
+    want = oracle.pool2d_nchw(x_nchw.astype(np.float32), k, s, p, a["pooling_type"], a["exclusive"], a["ceil_mode"])
+    return want[:, :, :oh, :ow], (k, s, p)
+
+
+@pytest.mark.parametrize("dtype", ["float16", "float32", "float64"])
+@pytest.mark.parametrize("attrs", POOL_ATTRS, ids=lambda a: "%s%d%s" % (
+    a["pooling_type"], a["kernel_size"][0], "g" if a["global_pooling"] else ("a" if a["adaptive"] else "")))
+@pytest.mark.parametrize("shape,fmt", POOL_SHAPES)
+def test_pool2d_forward(gpu, shape, fmt, attrs, dtype):
+    x = uniform(6, shape, dtype)
+    b = NetBuilder("pool2d")
+    X = b.create_input(Float(NP_OF[dtype][1]), shape, "x")
+    out = b.pool2d(X, data_format=fmt, **attrs)
+    (got,), _ = run(b, {X: x}, [out])
+    x_nchw = x.transpose(0, 3, 1, 2) if fmt == "NHWC" else x
+    want, _ = expected_pool(x_nchw, attrs, dtype)
+    got_nchw = got.transpose(0, 3, 1, 2) if fmt == "NHWC" else got
+    assert got_nchw.shape == want.shape, (got_nchw.shape, want.shape)
+    if attrs["pooling_type"] == "max":
+        assert np.array_equal(got_nchw.astype(np.float64), want.astype(np.float64))
+    else:
+        tol = 1e-3 if dtype == "float16" else 1e-6
+        close(got_nchw, want, tol, tol)
+
+
+@pytest.mark.parametrize("dtype", ["float16", "float32", "float64"])
+@pytest.mark.parametrize("attrs", POOL_GRAD_ATTRS, ids=lambda a: "%s%d%s" % (
+    a["pooling_type"], a["kernel_size"][0], "g" if a["global_pooling"] else ("a" if a["adaptive"] else "")))
+@pytest.mark.parametrize("shape,fmt", POOL_GRAD_SHAPES)
+def test_pool2d_gradient(gpu, shape, fmt, attrs, dtype):
+    x = uniform(7, shape, dtype)
+    t = Float(NP_OF[dtype][1])
+    b = NetBuilder("pool2d")
+    X = b.create_input(t, shape, "x")
+    y = b.pool2d(X, data_format=fmt, **attrs)
+    dy = uniform(8, y.shape(), dtype)
+    DY = b.create_input(t, y.shape(), "dy")
+    dx = b.pool2d_grad(X, y, DY, data_format=fmt, **attrs)
+    (got_y, got_dx), _ = run(b, {X: x, DY: dy}, [y, dx])
+    to_nchw = (lambda v: v.transpose(0, 3, 1, 2)) if fmt == "NHWC" else (lambda v: v)
+    x_nchw, dy_nchw = to_nchw(x), to_nchw(dy)
+    want_y, (k, s, p) = expected_pool(x_nchw, attrs, dtype)
+    # the gradient intrinsic takes the top / left padding only (cinn/hlir/op/custom_call.cc:590-640)
+    want_dx = ob.pool2d_backward(x_nchw, dy_nchw, k, s, (p[0], p[1]), attrs["pooling_type"], attrs["exclusive"])
+    tol = 1e-2 if dtype == "float16" else 1e-5
+    close(to_nchw(got_y), want_y, tol if attrs["pooling_type"] == "avg" else 0.0, tol if attrs["pooling_type"] == "avg" else 0.0)
+    close(to_nchw(got_dx), want_dx, tol, tol)
+
+
+def test_pool2d_gradient_with_an_input_sized_dy_buffer(gpu):
+    """The reference's gradient test feeds a dy of x's shape (python/tests/ops/test_pool2d_op.py:186-189); the
+    intrinsic reads the leading elements of that buffer as the [N, C, OH, OW] tensor."""
+    shape, attrs = [1, 3, 32, 32], POOL_GRAD_ATTRS[0]
+    x, dy_big = uniform(9, shape, "float32"), uniform(10, shape, "float32")
+    b = NetBuilder("pool2d")
+    X, DY = b.create_input(Float(32), shape, "x"), b.create_input(Float(32), shape, "dy")
+    y = b.pool2d(X, data_format="NCHW", **attrs)
+    dx = b.pool2d_grad(X, y, DY, data_format="NCHW", **attrs)
+    (got_dx,), _ = run(b, {X: x, DY: dy_big}, [dx])
+    k, s, p, oh, ow = pool_windows(32, 32, attrs)
+    dy = dy_big.reshape(-1)[:3 * oh * ow].reshape(1, 3, oh, ow)
+    want_dx = ob.pool2d_backward(x, dy, k, s, (p[0], p[1]), "max", True)
+    close(got_dx, want_dx, 1e-5, 1e-5)
