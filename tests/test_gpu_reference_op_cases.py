@@ -303,3 +303,136 @@ def test_pool2d_gradient_with_an_input_sized_dy_buffer(gpu):
     dy = dy_big.reshape(-1)[:3 * oh * ow].reshape(1, 3, oh, ow)
     want_dx = ob.pool2d_backward(x, dy, k, s, (p[0], p[1]), "max", True)
     close(got_dx, want_dx, 1e-5, 1e-5)
+
+
+# ---- reductions ---------------------------------------------------------------------------------------------------
+# python/tests/ops/test_reduce_op.py:71-677 (shape, element type, value range, axes, keep_dim; [] = every axis)
+REDUCE_SUM = [
+    ([10, 10, 10], "float32", (-1.0, 1.0), [], False), ([10, 10, 10], "float32", (-1.0, 1.0), [1], False),
+    ([10, 10, 10], "float32", (-1.0, 1.0), [0, 1], False), ([10, 10, 10], "float32", (-1.0, 1.0), [0, 2], False),
+    ([10, 10, 10], "float32", (-1.0, 1.0), [0], True), ([1, 16, 256], "float32", (-1.0, 1.0), [0], False),
+    ([1, 12, 9, 9], "float32", (-1.0, 1.0), [-1], False), ([1, 1, 10, 10, 10], "float32", (-1.0, 1.0), [0], False),
+    ([1, 10, 1, 10, 10], "float32", (-1.0, 1.0), [0, 2], False), ([1, 1, 10], "float32", (-1.0, 1.0), [0, 2], False),
+    ([1, 1, 10], "float32", (-1.0, 1.0), [0, 2], True), ([32, 32, 32, 32], "float32", (-0.1, 0.1), [0, 2, 3], False),
+    ([10, 1024], "float32", (-1.0, 1.0), [], False), ([10, 1024], "float32", (-1.0, 1.0), [0], False),
+    ([10, 1024], "float32", (-1.0, 1.0), [1], False), ([32, 64, 56, 56], "float32", (-0.1, 0.1), [0, 2, 3], False),
+    ([32, 56, 56, 64], "float32", (-0.1, 0.1), [0, 1, 2], False), ([1, 64, 56, 56], "float32", (-0.1, 0.1), [0, 2, 3], False),
+    ([1, 56, 56, 64], "float32", (-0.1, 0.1), [0, 1, 2], False), ([10, 10, 10], "float64", (-1.0, 1.0), [], False),
+    ([10], "int32", (-100, 100), [], False), ([10, 1024], "int32", (-100, 100), [1], False),
+    ([10, 10, 10], "int32", (-100, 100), [], False), ([1, 56, 56, 64], "int32", (-100, 100), [0, 1, 2], False),
+    ([10], "int64", (-100, 100), [], False), ([10, 1024], "int64", (-100, 100), [1], False),
+    ([10, 10, 10], "int64", (-100, 100), [], False), ([1, 56, 56, 64], "int64", (-100, 100), [0, 1, 2], False),
+]
+REDUCE_PROD = [
+    ([10, 10, 10], "float32", (-1.0, 1.0), [0, 1], False), ([10, 10, 10], "float32", (-1.0, 1.0), [0, 1], True),
+    ([10, 10, 10], "float32", (-1.0, 1.0), [0], False), ([10, 10, 10], "float32", (-1.0, 1.0), [], False),
+    ([10, 10, 10], "float64", (-1.0, 1.0), [], False), ([10], "int32", (-10, 10), [], False),
+    ([10, 1024], "int64", (-10, 10), [], False), ([1, 56, 56, 64], "int64", (-10, 10), [0, 1, 2], False),
+]
+REDUCE_MAX_MIN = [
+    ([10, 10, 10], "float32", (-1.0, 1.0), [0, 1], False), ([10, 10, 10], "float32", (-1.0, 1.0), [0, 1], True),
+    ([10, 10, 10], "float32", (-1.0, 1.0), [0], False), ([10, 10, 10], "float32", (-10.0, -1.0), [], False),
+    ([10, 10, 10], "float32", (1.0, 10.0), [], False), ([10, 10, 10], "float64", (-1.0, 1.0), [], False),
+    ([2, 3, 4, 5], "float64", (-1.0, 1.0), [0, 1], False), ([10], "int32", (-100, 100), [], False),
+    ([10, 10], "int64", (-100, 100), [], False), ([1, 56, 56, 64], "int64", (-100, 100), [0, 1, 2], False),
+]
+# python/tests/ops/test_reduce_op_new.py:96-215 and test_reduce_op_other.py (axes lists of TestReduceAxis)
+REDUCE_NEW = [([1], [-1]), ([1024], [0]), ([512, 256], [1]), ([128, 64, 32], [2]), ([16, 8, 4, 2], [3]),
+              ([16, 8, 4, 2, 1], [3]), ([1, 1, 1, 1, 1], [3]), ([1, 512, 1], [1]), ([1, 1024, 1], [1]), ([1, 2048, 1], [1]),
+              ([64, 32, 16, 8, 4], [0, 2]), ([64, 32, 16, 8, 4], [1, 2, 3]), ([64, 32, 16, 8, 4], [])]
+TYPE_OF = {"float32": (np.float32, lambda: Float(32)), "float64": (np.float64, lambda: Float(64)),
+           "int32": (np.int32, None), "int64": (np.int64, None), "bool": (np.bool_, None)}
+
+
+def cinn_type(dtype):
+    from cinn_amd.common import Bool, Int
+    return {"float32": Float(32), "float64": Float(64), "int32": Int(32), "int64": Int(64), "bool": Bool()}[dtype]
+
+
+def reduce_input(seed, shape, dtype, rng_range):
+    rng = np.random.default_rng(seed)
+    if dtype == "bool":
+        return rng.integers(0, 2, shape).astype(np.bool_)
+    if dtype.startswith("int"):
+        return rng.integers(rng_range[0], rng_range[1], shape).astype(TYPE_OF[dtype][0])
+    return rng.uniform(rng_range[0], rng_range[1], shape).astype(TYPE_OF[dtype][0])
+
+
+def run_reduce(op, shape, dtype, rng_range, axes, keep, x=None):
+    x = reduce_input(12, shape, dtype, rng_range) if x is None else x
+    b = NetBuilder("reduce")
+    X = b.create_input(cinn_type(dtype), shape, "x")
+    out = getattr(b, "reduce_" + op)(X, axes, keep)
+    (got,), _ = run(b, {X: x}, [out])
+    ax = tuple(range(len(shape))) if not axes else tuple(axes)
+    fn = {"sum": np.sum, "prod": np.prod, "max": np.max, "min": np.min, "all": np.all, "any": np.any}[op]
+    wide = x.astype(np.float64) if dtype.startswith("float") else x
+    want = np.asarray(fn(wide, axis=ax, keepdims=keep))
+    if want.ndim == 0:
+        want = want.reshape([1])   # a reduction over every axis leaves one element (paddle gives shape [1] too)
+    assert list(got.shape) == list(want.shape), (got.shape, want.shape)
+    assert got.dtype == TYPE_OF[dtype][0]
+    if dtype.startswith("float") and op in ("sum", "prod"):
+        if op == "sum":
+            scale = np.abs(wide).sum(axis=ax, keepdims=keep).reshape(want.shape)
+            close(got, want, 0.0, 1e-5 * scale + 1e-30 if dtype == "float32" else 1e-12 * scale + 1e-300)
+        else:
+            close(got, want, 1e-4 if dtype == "float32" else 1e-10, 1e-38)
+    else:
+        assert np.array_equal(got, want.astype(TYPE_OF[dtype][0]))
+
+
+@pytest.mark.parametrize("shape,dtype,rng_range,axes,keep", REDUCE_SUM)
+def test_reduce_sum_cases(gpu, shape, dtype, rng_range, axes, keep):
+    run_reduce("sum", shape, dtype, rng_range, axes, keep)
+
+
+@pytest.mark.parametrize("shape,dtype,rng_range,axes,keep", REDUCE_PROD)
+def test_reduce_prod_cases(gpu, shape, dtype, rng_range, axes, keep):
+    if dtype.startswith("int") and int(np.prod(shape)) > 10:
+        # the reference's products of hundreds of integers from [-10, 10) overflow; with a zero among them the
+        # result is 0 either way, which is all this case can check
+        x = reduce_input(12, shape, dtype, rng_range)
+        x.reshape(-1)[::7] = 0
+        run_reduce("prod", shape, dtype, rng_range, axes, keep, x)
+    else:
+        run_reduce("prod", shape, dtype, rng_range, axes, keep)
+
+
+@pytest.mark.parametrize("op", ["max", "min"])
+@pytest.mark.parametrize("shape,dtype,rng_range,axes,keep", REDUCE_MAX_MIN)
+def test_reduce_max_min_cases(gpu, shape, dtype, rng_range, axes, keep, op):
+    run_reduce(op, shape, dtype, rng_range, axes, keep)
+
+
+@pytest.mark.parametrize("op", ["all", "any"])
+@pytest.mark.parametrize("axes,keep", [([], False), ([], True), ([0, 1], False), ([0, 1], True), ([0], False)])
+def test_reduce_all_any_cases(gpu, axes, keep, op):
+    run_reduce(op, [10, 10, 10], "bool", None, axes, keep)
+    constant = np.full([10, 10, 10], op == "all", np.bool_)   # TestAllCase5 / TestAnyCase5
+    run_reduce(op, [10, 10, 10], "bool", None, axes, keep, constant)
+
+
+@pytest.mark.parametrize("keep", [True, False])
+@pytest.mark.parametrize("op", ["sum", "prod", "max", "min"])
+@pytest.mark.parametrize("shape,axes", REDUCE_NEW)
+def test_reduce_new_cases(gpu, shape, axes, op, keep):
+    if op == "prod":
+        # uniform [0, 1) products of hundreds of factors underflow: keep the factors near one
+        x = np.random.default_rng(13).uniform(0.9, 1.1, shape).astype(np.float32)
+        run_reduce(op, shape, "float32", None, axes, keep, x)
+    else:
+        run_reduce(op, shape, "float32", (0.0, 1.0), axes, keep)
+
+
+@pytest.mark.parametrize("keep", [True, False])
+@pytest.mark.parametrize("dtype", ["int32", "int64", "float32", "float64"])
+def test_reduce_sum_element_types(gpu, dtype, keep):
+    run_reduce("sum", [16, 8, 4, 2, 1], dtype, (0, 100) if dtype.startswith("int") else (0.0, 1.0), [3], keep)
+
+
+@pytest.mark.parametrize("keep", [True, False])
+@pytest.mark.parametrize("op", ["all", "any"])
+@pytest.mark.parametrize("shape,axes", REDUCE_NEW[:7])
+def test_reduce_bool_new_cases(gpu, shape, axes, op, keep):
+    run_reduce(op, shape, "bool", None, axes, keep)
