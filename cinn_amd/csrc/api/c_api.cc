@@ -179,6 +179,10 @@ const std::map<std::string, Method>& Methods() {
                          GetAttr<float>(a, "momentum", 0.9f), GetAttr<std::string>(a, "data_layout", "NCHW"),
                          GetAttr<bool>(a, "is_test", true));
     };
+    m["BatchNormGrad"] = [](NetBuilder& b, const std::vector<Variable>& in, const AttributeMap& a) {
+      return b.BatchNormGrad(in.at(0), in.at(1), in.at(2), in.at(3), in.at(4), GetAttr<float>(a, "epsilon", 1e-5f),
+                             GetAttr<std::string>(a, "data_layout", "NCHW"));
+    };
     m["Pool2d"] = [](NetBuilder& b, const std::vector<Variable>& in, const AttributeMap& a) {
       return std::vector<Variable>{
           b.Pool2d(in.at(0), GetAttr<std::string>(a, "pooling_type", "max"), GetAttr<std::vector<int>>(a, "ksize", {1, 1}),

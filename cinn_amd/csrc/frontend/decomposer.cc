@@ -15,16 +15,22 @@ class SubBuilder : public NetBuilder {
  public:
   explicit SubBuilder(int serial) : NetBuilder("decomposer"), prefix_("dcp" + std::to_string(serial) + "_") {}
   std::vector<Instruction> TakeInstructions(const Variable& result, const Variable& origin) {
+    return TakeInstructions(std::vector<std::pair<Variable, Variable>>{{result, origin}});
+  }
+  // results[i].first is mapped back to results[i].second, the variable the original instruction defined
+  std::vector<Instruction> TakeInstructions(const std::vector<std::pair<Variable, Variable>>& results) {
     Program p = Build();
     std::vector<Instruction> out;
     for (auto& ins : p.instructions()) {
       for (auto& o : ins->outputs) {
-        if (o == result) {
-          // map the result back to the variable the original instruction defined
-          o->id = origin->id;
-        } else if (o->id.rfind(prefix_, 0) != 0) {
-          o->id = prefix_ + o->id;
+        bool mapped = false;
+        for (auto& r : results) {
+          if (o == r.first) {
+            o->id  = r.second->id;
+            mapped = true;
+          }
         }
+        if (!mapped && o->id.rfind(prefix_, 0) != 0) o->id = prefix_ + o->id;
       }
       out.push_back(ins);
     }
@@ -91,6 +97,111 @@ void DecomposeBatchNorm(const Instruction& instr, int serial, std::vector<Instru
   out->insert(out->end(), ins.begin(), ins.end());
 }
 
+// The training form and the gradient (cinn/frontend/decomposer/batch_norm.cc:22-262): statistics over n, h, w as
+// E(x) and E(x^2) - E(x)^2, y = (x - mean) * rsqrt(variance + eps) * scale + bias, moving averages
+// moving * momentum + saved * (1 - momentum); 16-bit x / dy are computed in fp32 and y / x_grad cast back, the
+// per-channel tensors stay fp32 (the reference's AutoCast pass, cinn/frontend/pass/auto_cast.cc:120-190).
+struct BatchNormParts {
+  SubBuilder* b;
+  std::vector<int> x_shape, reduce_dim, c_axis;
+  float element_count;
+  BatchNormParts(SubBuilder* builder, const std::vector<int>& shape, const std::string& layout) : b(builder), x_shape(shape) {
+    CINN_CHECK_EQ(shape.size(), 4u) << "Only 4-D input tensor is supported, but get " << shape.size() << "-D input tensor.";
+    CINN_CHECK(layout == "NCHW" || layout == "NHWC") << layout << " setting is not support!";
+    if (layout == "NCHW") {
+      c_axis = {1}, reduce_dim = {0, 2, 3};
+      element_count = static_cast<float>(shape[0] * shape[2] * shape[3]);
+    } else {
+      c_axis = {3}, reduce_dim = {0, 1, 2};
+      element_count = static_cast<float>(shape[0] * shape[1] * shape[2]);
+    }
+  }
+  Variable Reduce(const Variable& v) { return b->ReduceSum(v, reduce_dim); }
+  Variable To4d(const Variable& v) { return b->BroadcastTo(v, x_shape, c_axis); }
+  Variable Constant(const Variable& like, float value, const char* name) {
+    return b->FillConstant(like->shape, value, name, common::Type2Str(like->type));
+  }
+  Variable Mean(const Variable& x) {
+    auto sum = Reduce(x);
+    return b->Divide(sum, Constant(sum, element_count, "element_count"));
+  }
+  Variable Variance(const Variable& x, const Variable& mean) {
+    auto sq_sum  = Reduce(b->Multiply(x, b->Identity(x)));
+    auto sq_mean = b->Divide(sq_sum, Constant(sq_sum, element_count, "element_count"));
+    return b->Subtract(sq_mean, b->Multiply(mean, b->Identity(mean)));
+  }
+  Variable StdVarianceInv(const Variable& variance, float epsilon) {
+    return b->Rsqrt(b->Add(variance, Constant(variance, epsilon, "epsilon")));
+  }
+  Variable Moving(const Variable& moving, const Variable& saved, float momentum) {
+    return b->Add(b->Multiply(moving, Constant(moving, momentum, "factor_0")),
+                  b->Multiply(saved, Constant(saved, 1.0f - momentum, "factor_1")));
+  }
+};
+
+bool Is16Bit(const common::Type& t) { return t.is_float16() || t.is_bfloat16(); }
+
+void DecomposeBatchNormTrain(const Instruction& instr, int serial, std::vector<Instruction>* out) {
+  CINN_CHECK_EQ(instr->inputs.size(), 5u) << "batch_norm_train takes x, scale, bias, moving_mean, moving_variance";
+  CINN_CHECK_EQ(instr->outputs.size(), 5u);
+  auto x = instr->inputs[0], scale = instr->inputs[1], bias = instr->inputs[2], moving_mean = instr->inputs[3],
+       moving_variance = instr->inputs[4];
+  float epsilon  = hlir::framework::GetAttr<float>(instr->attrs, "epsilon", 1e-5f);
+  float momentum = hlir::framework::GetAttr<float>(instr->attrs, "momentum", 0.9f);
+  auto layout    = hlir::framework::GetAttr<std::string>(instr->attrs, "data_layout", "NCHW");
+  SubBuilder b(serial);
+  BatchNormParts h(&b, x->shape, layout);
+  const bool narrow = Is16Bit(x->type);
+  Variable xf       = narrow ? b.Cast(x, "float32") : x;
+  auto mean         = h.Mean(xf);
+  auto variance     = h.Variance(xf, mean);
+  // the 4-D form of rsqrt(variance + eps), as the reference builds it
+  auto variance_4d  = h.To4d(variance);
+  auto inv_std_4d   = b.Rsqrt(b.Add(variance_4d, h.Constant(variance_4d, epsilon, "epsilon")));
+  auto normalized   = b.Multiply(b.Subtract(xf, h.To4d(mean)), inv_std_4d);
+  auto y            = b.Add(b.Multiply(normalized, h.To4d(scale)), h.To4d(bias));
+  if (narrow) y = b.Cast(y, common::Type2Str(x->type));
+  auto new_mean     = h.Moving(moving_mean, mean, momentum);
+  auto new_variance = h.Moving(moving_variance, variance, momentum);
+  auto ins = b.TakeInstructions({{y, instr->outputs[0]},
+                                 {mean, instr->outputs[1]},
+                                 {variance, instr->outputs[2]},
+                                 {new_mean, instr->outputs[3]},
+                                 {new_variance, instr->outputs[4]}});
+  out->insert(out->end(), ins.begin(), ins.end());
+}
+
+void DecomposeBatchNormGrad(const Instruction& instr, int serial, std::vector<Instruction>* out) {
+  CINN_CHECK_EQ(instr->inputs.size(), 5u) << "batch_norm_grad takes dy, x, scale, save_mean, save_variance";
+  CINN_CHECK_EQ(instr->outputs.size(), 3u);
+  auto y_grad = instr->inputs[0], x = instr->inputs[1], scale = instr->inputs[2], save_mean = instr->inputs[3],
+       save_variance = instr->inputs[4];
+  float epsilon = hlir::framework::GetAttr<float>(instr->attrs, "epsilon", 1e-5f);
+  auto layout   = hlir::framework::GetAttr<std::string>(instr->attrs, "data_layout", "NCHW");
+  SubBuilder b(serial);
+  BatchNormParts h(&b, x->shape, layout);
+  const bool narrow = Is16Bit(x->type);
+  Variable xf  = narrow ? b.Cast(x, "float32") : x;
+  Variable dyf = Is16Bit(y_grad->type) ? b.Cast(y_grad, "float32") : y_grad;
+  // bias_grad = sum(dy); scale_grad = sum(dy * (x - mean)) * rsqrt(variance + eps)
+  auto x_mean_diff = b.Subtract(xf, h.To4d(save_mean));
+  auto bias_grad   = h.Reduce(dyf);
+  auto dy_xmd_sum  = h.Reduce(b.Multiply(dyf, x_mean_diff));
+  auto scale_grad  = b.Multiply(dy_xmd_sum, h.StdVarianceInv(save_variance, epsilon));
+  // x_grad = scale * rsqrt(variance + eps) / nhw * (nhw * dy - sum(dy) - (x - mean) * sum(dy * (x - mean)) / (variance + eps))
+  auto scaled_inv_std = b.Multiply(scale, h.StdVarianceInv(save_variance, epsilon));
+  auto tmp0 = h.To4d(b.Divide(scaled_inv_std, h.Constant(scaled_inv_std, h.element_count, "element_count_1d")));
+  auto tmp1 = b.Multiply(dyf, h.Constant(dyf, h.element_count, "element_count_4d"));
+  auto tmp2 = h.To4d(bias_grad);
+  auto x_mean_diff2 = b.Subtract(xf, h.To4d(save_mean));
+  auto tmp3_0 = b.Multiply(x_mean_diff2, h.To4d(dy_xmd_sum));
+  auto tmp3   = b.Divide(tmp3_0, h.To4d(b.Add(save_variance, h.Constant(save_variance, epsilon, "epsilon"))));
+  auto x_grad = b.Multiply(tmp0, b.Subtract(b.Subtract(tmp1, tmp2), tmp3));
+  if (narrow) x_grad = b.Cast(x_grad, common::Type2Str(x->type));
+  auto ins = b.TakeInstructions({{x_grad, instr->outputs[0]}, {scale_grad, instr->outputs[1]}, {bias_grad, instr->outputs[2]}});
+  out->insert(out->end(), ins.begin(), ins.end());
+}
+
 }  // namespace
 
 Program ApplyDecomposer(const Program& program) {
@@ -101,6 +212,10 @@ Program ApplyDecomposer(const Program& program) {
       DecomposeSoftmax(ins, serial++, &out);
     } else if (ins->op_type == "batch_norm") {
       DecomposeBatchNorm(ins, serial++, &out);
+    } else if (ins->op_type == "batch_norm_train") {
+      DecomposeBatchNormTrain(ins, serial++, &out);
+    } else if (ins->op_type == "batch_norm_grad") {
+      DecomposeBatchNormGrad(ins, serial++, &out);
     } else {
       out.push_back(ins);
     }

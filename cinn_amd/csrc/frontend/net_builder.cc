@@ -300,9 +300,16 @@ Variable NetBuilder::Conv(const Variable& lhs, const Variable& rhs, const std::v
 std::vector<Variable> NetBuilder::BatchNorm(const Variable& x, const Variable& scale, const Variable& bias,
                                             const Variable& mean, const Variable& variance, float epsilon,
                                             float momentum, const std::string& data_layout, bool is_test) {
-  CINN_CHECK(is_test) << "only the inference form of batch_norm is lowered by this backend";
-  return CustomInstr("batch_norm", {x, scale, bias, mean, variance},
+  // cinn/frontend/net_builder.cc:760-773: one output when is_test, else y, saved mean / variance, moving mean / variance
+  return CustomInstr(is_test ? "batch_norm" : "batch_norm_train", {x, scale, bias, mean, variance},
                      {{"epsilon", epsilon}, {"momentum", momentum}, {"data_layout", data_layout}});
+}
+// outputs x_grad, scale_grad, bias_grad (cinn/frontend/net_builder.cc:776-786)
+std::vector<Variable> NetBuilder::BatchNormGrad(const Variable& dy, const Variable& x, const Variable& scale,
+                                                const Variable& save_mean, const Variable& save_variance,
+                                                float epsilon, const std::string& data_layout) {
+  return CustomInstr("batch_norm_grad", {dy, x, scale, save_mean, save_variance},
+                     {{"epsilon", epsilon}, {"data_layout", data_layout}});
 }
 
 namespace {

@@ -108,6 +108,9 @@ class NetBuilder {
   std::vector<Variable> BatchNorm(const Variable& x, const Variable& scale, const Variable& bias,
                                   const Variable& mean, const Variable& variance, float epsilon = 1e-5f,
                                   float momentum = 0.9f, const std::string& data_layout = "NCHW", bool is_test = true);
+  std::vector<Variable> BatchNormGrad(const Variable& dy, const Variable& x, const Variable& scale,
+                                      const Variable& save_mean, const Variable& save_variance, float epsilon = 1e-5f,
+                                      const std::string& data_layout = "NCHW");
   Variable Pool2d(const Variable& x, const std::string& pooling_type, const std::vector<int>& ksize,
                   const std::vector<int>& strides = {1, 1}, const std::vector<int>& paddings = {0, 0},
                   bool ceil_mode = false, bool exclusive = true, bool global_pooling = false,

@@ -453,6 +453,33 @@ OpRegistry::OpRegistry() {
     op.infer_dtype = SameTypeAsFirst;
   }
 
+  {
+    // training form: x, scale, bias, moving_mean, moving_variance -> y, saved_mean, saved_variance, moving_mean,
+    // moving_variance (cinn/hlir/op/nn.cc batch_norm_train)
+    auto& op       = r->Register("batch_norm_train");
+    op.pattern     = OpPatternKind::kNonFusible;
+    op.num_inputs  = 5;
+    op.infer_shape = [](const std::vector<ShapeType>& in, const AttributeMap&) {
+      return std::vector<ShapeType>{in[0], in[1], in[1], in[1], in[1]};
+    };
+    op.infer_dtype = [](const std::vector<Type>& in, const AttributeMap&) {
+      return std::vector<Type>{in[0], in[1], in[1], in[1], in[1]};
+    };
+  }
+  {
+    // dy, x, scale, save_mean, save_variance -> x_grad, scale_grad, bias_grad (cinn/hlir/op/nn.cc batch_norm_grad)
+    auto& op       = r->Register("batch_norm_grad");
+    op.pattern     = OpPatternKind::kNonFusible;
+    op.num_inputs  = 5;
+    op.infer_shape = [](const std::vector<ShapeType>& in, const AttributeMap&) {
+      CINN_CHECK(in[0] == in[1]) << "batch_norm_grad: dy and x differ in shape";
+      return std::vector<ShapeType>{in[1], in[2], in[2]};
+    };
+    op.infer_dtype = [](const std::vector<Type>& in, const AttributeMap&) {
+      return std::vector<Type>{in[1], in[2], in[2]};
+    };
+  }
+
   // ---- library-backed ops ------------------------------------------------------------------------
   {
     // row-major matmul with numpy batch broadcasting; output shape as NetBuilder::GetMatmulOutputShape

@@ -221,6 +221,11 @@ class NetBuilder(object):
         return self._call("BatchNorm", [x, scale, bias, mean, variance], epsilon=float(epsilon),
                           momentum=float(momentum), data_layout=data_layout, is_test=is_test)
 
+    def batch_norm_grad(self, dy, x, scale, save_mean, save_variance, epsilon=1e-5, data_layout="NCHW"):
+        """Returns [x_grad, scale_grad, bias_grad] (cinn/pybind/frontend.cc `batch_norm_grad`)."""
+        return self._call("BatchNormGrad", [dy, x, scale, save_mean, save_variance], epsilon=float(epsilon),
+                          data_layout=data_layout)
+
     def pool2d(self, x, pooling_type, kernel_size, stride=(1, 1), padding=(0, 0), ceil_mode=False, exclusive=True,
                global_pooling=False, data_format="NCHW", adaptive=False, padding_algorithm="EXPLICIT"):
         """Argument names of cinn/pybind/frontend.cc:586-598."""

@@ -402,3 +402,24 @@ def test_conv_gradients_and_pool2d_grad_shapes_and_lowering():
     assert compile_only(b, [y, dx]).num_instructions() == 2
     # adaptive average pooling: windows of floor(extent / outputs) (PoolImpl, cinn/hlir/pe/nn.cc:1073-1112)
     assert b.pool2d(x, "avg", [4, 4], adaptive=True).shape() == [2, 4, 4, 4]
+
+
+def test_batch_norm_training_form_and_gradient_decompose_into_primitives():
+    """batchnorm(is_test=False) gives y, the saved mean / variance and the new moving mean / variance; batch_norm_grad
+    gives x_grad, scale_grad, bias_grad (cinn/frontend/net_builder.cc:760-786).  Both are rewritten into reductions and
+    elementwise operators before the graph is built (cinn/frontend/decomposer/batch_norm.cc:139-262): no instruction of
+    the compiled program carries their name.  16-bit x keeps fp32 statistics."""
+    from cinn_amd.common import Float
+    b = NetBuilder("t")
+    x = b.create_input(Float(16), [4, 8, 6, 6], "x")
+    dy = b.create_input(Float(16), [4, 8, 6, 6], "dy")
+    params = [b.fill_constant([8], v, n, "float32") for v, n in ((1.0, "s"), (0.0, "b"), (0.0, "m"), (1.0, "v"))]
+    outs = b.batchnorm(x, *params, is_test=False)
+    assert [o.shape() for o in outs] == [[4, 8, 6, 6]] + [[8]] * 4
+    assert [str(o.type()) for o in outs] == ["float16"] + ["float32"] * 4
+    grads = b.batch_norm_grad(dy, x, params[0], outs[1], outs[2])
+    assert [g.shape() for g in grads] == [[4, 8, 6, 6], [8], [8]]
+    assert [str(g.type()) for g in grads] == ["float16", "float32", "float32"]
+    comp = compile_only(b, outs + grads)
+    names = [comp.instruction_info(i)[0] for i in range(comp.num_instructions())]
+    assert not any("batch_norm" in n for n in names) and any("reduce" in n for n in names)

@@ -6,11 +6,13 @@ cinn_call_cudnn_conv2d_forward / _backward_data / _backward_filter / cinn_call_c
     combination, fp16 / fp32 / fp64, and the matmul + transpose pair;
   * python/tests/ops/test_conv2d_op.py:127-195 - 3x3 convolutions in NCHW and NHWC with both gradients
     (builder.conv(..., conv_type="backward_data" / "backward_filter", output_shape=...)), fp16 / fp32 / fp64;
-  * python/tests/ops/test_pool2d_op.py:80-330  - six forward attribute sets on four shapes and the four gradient sets.
+  * python/tests/ops/test_pool2d_op.py:80-330  - six forward attribute sets on four shapes and the four gradient sets;
+  * python/tests/ops/test_reduce_op.py, test_reduce_op_new.py, test_reduce_op_other.py - every reduction case;
+  * python/tests/ops/test_batch_norm_op.py:15-275 - the training form, its gradient and the inference form.
 
 The reference compares with Paddle at the same precision; here the expected values are float64 numpy (matmul), the
 CPU oracle (convolution and its gradients, pooling in fp32 / fp16) or float64 window loops written out below (fp64
-pooling).  Inputs are uniform in [0, 1) as OpTest.random draws them (python/tests/ops/op_test.py).  Tolerances are
+pooling), torch's CPU batch_norm and its autograd in float64 (batch norm).  Inputs are uniform in [0, 1) as OpTest.random draws them (python/tests/ops/op_test.py).  Tolerances are
 the reference's: matmul fp16 1e-2, fp32 1e-5, fp64 1e-5 (relative, absolute part 1e-6 scaled by the size of the
 sums); convolution fp16 1e-3, fp32 / fp64 1e-5; max pooling exact, average pooling 1e-6 (fp16 1e-3)."""
 import numpy as np
@@ -436,3 +438,94 @@ def test_reduce_sum_element_types(gpu, dtype, keep):
 @pytest.mark.parametrize("shape,axes", REDUCE_NEW[:7])
 def test_reduce_bool_new_cases(gpu, shape, axes, op, keep):
     run_reduce(op, shape, "bool", None, axes, keep)
+
+
+# ---- batch_norm: training form, gradient, inference ----------------------------------------------------------------
+BN_SHAPES = [[2, 16, 8, 8], [2, 16, 8, 1], [2, 16, 2048, 8]]
+
+
+def bn_tensor(seed, shape, dtype):
+    x = np.random.default_rng(seed).uniform(0.0, 1.0, shape).astype(np.float32)
+    if dtype == "bfloat16":
+        from cinn_amd.common import bfloat16_bits_to_float32, float32_to_bfloat16_bits
+        bits = float32_to_bfloat16_bits(x)
+        return bits, bfloat16_bits_to_float32(bits)
+    x = x.astype(NP_OF[dtype][0])
+    return x, x.astype(np.float32)
+
+
+def bn_type(dtype):
+    from cinn_amd.common import BFloat16
+    return BFloat16() if dtype == "bfloat16" else Float(NP_OF[dtype][1])
+
+
+def bn_result(a, dtype):
+    from cinn_amd.common import bfloat16_bits_to_float32
+    return bfloat16_bits_to_float32(a) if dtype == "bfloat16" else a.astype(np.float64)
+
+
+def bn_params(b, c):
+    return (b.fill_constant([c], 1.0, "scale", "float32"), b.fill_constant([c], 0.0, "bias", "float32"),
+            b.fill_constant([c], 0.0, "mean", "float32"), b.fill_constant([c], 1.0, "variance", "float32"))
+
+
+@pytest.mark.parametrize("dtype,tol", [("float16", 1e-3), ("float32", 1e-5), ("bfloat16", 1e-2)])
+@pytest.mark.parametrize("shape", BN_SHAPES)
+def test_batch_norm_train(gpu, shape, dtype, tol):
+    import torch
+    raw, x = bn_tensor(14, shape, dtype)
+    b = NetBuilder("batch_norm")
+    X = b.create_input(bn_type(dtype), shape, "x")
+    outs = b.batchnorm(X, *bn_params(b, shape[1]), is_test=False)
+    assert len(outs) == 5
+    got, _ = run(b, {X: raw}, outs)
+    xt = torch.from_numpy(x.astype(np.float64))
+    want_y = torch.nn.functional.batch_norm(xt, None, None, training=True, eps=1e-5).numpy()
+    mean = x.astype(np.float64).mean(axis=(0, 2, 3))
+    var = x.astype(np.float64).var(axis=(0, 2, 3))   # the biased variance, as the normalisation uses it
+    close(bn_result(got[0], dtype), want_y, tol, tol)
+    close(got[1], mean, 1e-5, 1e-6)
+    close(got[2], var, 1e-4, 1e-6)                   # E(x^2) - E(x)^2 in fp32 loses digits of a variance of 1/12
+    close(got[3], 0.9 * 0.0 + 0.1 * mean, 1e-5, 1e-6)
+    close(got[4], 0.9 * 1.0 + 0.1 * var, 1e-5, 1e-6)
+
+
+@pytest.mark.parametrize("dtype,tol", [("float16", 1e-3), ("float32", 1e-5)])
+@pytest.mark.parametrize("shape", BN_SHAPES)
+def test_batch_norm_gradient(gpu, shape, dtype, tol):
+    import torch
+    raw_x, x = bn_tensor(15, shape, dtype)
+    raw_dy, dy = bn_tensor(16, shape, dtype)
+    x64 = x.astype(np.float64)
+    mean, var = x64.mean(axis=(0, 2, 3)).astype(np.float32), x64.var(axis=(0, 2, 3)).astype(np.float32)
+    b = NetBuilder("batch_norm_grad")
+    DY, X = b.create_input(bn_type(dtype), shape, "dout"), b.create_input(bn_type(dtype), shape, "x_g")
+    scale = b.fill_constant([shape[1]], 1.0, "scale_g", "float32")
+    M, V = b.create_input(Float(32), [shape[1]], "save_mean"), b.create_input(Float(32), [shape[1]], "save_variance")
+    outs = b.batch_norm_grad(DY, X, scale, M, V)
+    assert len(outs) == 3
+    (gx, gscale, gbias), _ = run(b, {DY: raw_dy, X: raw_x, M: mean, V: var}, outs)
+    xt = torch.from_numpy(x64).requires_grad_(True)
+    wt = torch.ones(shape[1], dtype=torch.float64, requires_grad=True)
+    bt = torch.zeros(shape[1], dtype=torch.float64, requires_grad=True)
+    torch.nn.functional.batch_norm(xt, None, None, wt, bt, training=True, eps=1e-5).backward(
+        torch.from_numpy(dy.astype(np.float64)))
+    n = shape[0] * shape[2] * shape[3]
+    # x_grad is a difference of terms of the size of dy: the bound is relative to that size, not to the result
+    close(bn_result(gx, dtype), xt.grad.numpy(), tol, tol * 4.0)
+    close(gscale, wt.grad.numpy(), 1e-4, 1e-6 * n)
+    close(gbias, bt.grad.numpy(), 1e-5, 1e-6 * n)
+
+
+@pytest.mark.parametrize("shape", BN_SHAPES)
+def test_batch_norm_inference(gpu, shape):
+    import torch
+    raw, x = bn_tensor(17, shape, "float32")
+    b = NetBuilder("batch_norm")
+    X = b.create_input(Float(32), shape, "x")
+    (y,) = b.batchnorm(X, *bn_params(b, shape[1]), is_test=True)
+    (got,), _ = run(b, {X: raw}, [y])
+    c = shape[1]
+    want = torch.nn.functional.batch_norm(torch.from_numpy(x.astype(np.float64)), torch.zeros(c, dtype=torch.float64),
+                                          torch.ones(c, dtype=torch.float64), training=False, eps=1e-5).numpy()
+    close(got, want, 1e-5, 1e-6)
