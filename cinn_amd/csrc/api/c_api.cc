@@ -179,6 +179,12 @@ const std::map<std::string, Method>& Methods() {
                          GetAttr<float>(a, "momentum", 0.9f), GetAttr<std::string>(a, "data_layout", "NCHW"),
                          GetAttr<bool>(a, "is_test", true));
     };
+    m["ReluGrad"] = [](NetBuilder& b, const std::vector<Variable>& in, const AttributeMap&) {
+      return std::vector<Variable>{b.ReluGrad(in.at(0), in.at(1))};
+    };
+    m["ElementwiseAddGrad"] = [](NetBuilder& b, const std::vector<Variable>& in, const AttributeMap& a) {
+      return b.ElementwiseAddGrad(in.at(0), in.at(1), in.at(2), GetAttr<int>(a, "axis", -1));
+    };
     m["BatchNormGrad"] = [](NetBuilder& b, const std::vector<Variable>& in, const AttributeMap& a) {
       return b.BatchNormGrad(in.at(0), in.at(1), in.at(2), in.at(3), in.at(4), GetAttr<float>(a, "epsilon", 1e-5f),
                              GetAttr<std::string>(a, "data_layout", "NCHW"));

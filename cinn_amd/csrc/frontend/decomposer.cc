@@ -202,6 +202,56 @@ void DecomposeBatchNormGrad(const Instruction& instr, int serial, std::vector<In
   out->insert(out->end(), ins.begin(), ins.end());
 }
 
+// relu_grad(dout, out) = select(out > 0, dout, 0) (cinn/frontend/decomposer/activation.cc:40-55)
+void DecomposeReluGrad(const Instruction& instr, int serial, std::vector<Instruction>* out) {
+  CINN_CHECK_EQ(instr->inputs.size(), 2u) << " 2 input tensors for " << instr->op_type;
+  auto dout = instr->inputs[0], y = instr->inputs[1];
+  SubBuilder b(serial);
+  auto zero = b.FillConstant(y->shape, 0.0f, "zero", common::Type2Str(y->type));
+  auto res  = b.Select(b.GreaterThan(y, zero), dout, zero);
+  auto ins  = b.TakeInstructions(res, instr->outputs[0]);
+  out->insert(out->end(), ins.begin(), ins.end());
+}
+
+// elementwise_add_grad(dout, x, y; axis) -> dx, dy: dout itself where the shapes agree, else its sum over the
+// broadcast dimensions (kept for dx, reshaped to y's shape for dy) - cinn/frontend/decomposer/broadcast.cc:22-159
+void DecomposeElementwiseAddGrad(const Instruction& instr, int serial, std::vector<Instruction>* out) {
+  CINN_CHECK_EQ(instr->inputs.size(), 3u) << " 3 input tensors for " << instr->op_type;
+  CINN_CHECK_EQ(instr->outputs.size(), 2u) << "2 output tensors for " << instr->op_type;
+  auto dout = instr->inputs[0];
+  auto dx = instr->outputs[0], dy = instr->outputs[1];
+  int axis = hlir::framework::GetAttr<int>(instr->attrs, "axis", -1);
+  CINN_CHECK(!(axis < 0 && dx->shape.size() < dy->shape.size()))
+      << "Please make sure x'rank greater than or equal to y'rank when axis = -1";
+  if (axis < 0) axis = static_cast<int>(dx->shape.size()) - static_cast<int>(dy->shape.size());
+  SubBuilder b(serial);
+  Variable dx_t, dy_t;
+  if (dx->shape == dout->shape) {
+    dx_t = b.Identity(dout);
+  } else {
+    std::vector<int> dims;
+    for (size_t i = 0; i < dout->shape.size(); ++i)
+      if (dx->shape[i] == 1 && dout->shape[i] != 1) dims.push_back(static_cast<int>(i));
+    dx_t = b.ReduceSum(dout, dims, true);
+  }
+  if (dy->shape == dout->shape) {
+    dy_t = b.Identity(dout);
+  } else {
+    std::vector<int> dims;
+    const int y_rank = static_cast<int>(dy->shape.size());
+    for (int i = 0; i < static_cast<int>(dout->shape.size()); ++i) {
+      if (i < axis || i >= axis + y_rank) {
+        dims.push_back(i);
+      } else if (dy->shape[i - axis] == 1 && dout->shape[i] != 1) {
+        dims.push_back(i);
+      }
+    }
+    dy_t = b.Reshape(b.ReduceSum(dout, dims, true), dy->shape);
+  }
+  auto ins = b.TakeInstructions({{dx_t, dx}, {dy_t, dy}});
+  out->insert(out->end(), ins.begin(), ins.end());
+}
+
 }  // namespace
 
 Program ApplyDecomposer(const Program& program) {
@@ -212,6 +262,10 @@ Program ApplyDecomposer(const Program& program) {
       DecomposeSoftmax(ins, serial++, &out);
     } else if (ins->op_type == "batch_norm") {
       DecomposeBatchNorm(ins, serial++, &out);
+    } else if (ins->op_type == "relu_grad") {
+      DecomposeReluGrad(ins, serial++, &out);
+    } else if (ins->op_type == "elementwise_add_grad") {
+      DecomposeElementwiseAddGrad(ins, serial++, &out);
     } else if (ins->op_type == "batch_norm_train") {
       DecomposeBatchNormTrain(ins, serial++, &out);
     } else if (ins->op_type == "batch_norm_grad") {

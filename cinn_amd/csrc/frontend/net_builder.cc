@@ -253,6 +253,12 @@ Variable NetBuilder::Squeeze(const Variable& x, const ShapeType& axes) {
   if (shape.empty()) shape.push_back(1);
   return Reshape(x, shape);
 }
+Variable NetBuilder::ReluGrad(const Variable& dout, const Variable& out) {
+  return CustomInstr("relu_grad", {dout, out}, {}).front();
+}
+std::vector<Variable> NetBuilder::ElementwiseAddGrad(const Variable& dout, const Variable& x, const Variable& y, int axis) {
+  return CustomInstr("elementwise_add_grad", {dout, x, y}, {{"axis", axis}});
+}
 Variable NetBuilder::ExpandDims(const Variable& x, const ShapeType& axes) {
   ShapeType shape = x->shape;
   for (int a : axes) {

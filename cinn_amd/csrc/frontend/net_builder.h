@@ -108,6 +108,9 @@ class NetBuilder {
   std::vector<Variable> BatchNorm(const Variable& x, const Variable& scale, const Variable& bias,
                                   const Variable& mean, const Variable& variance, float epsilon = 1e-5f,
                                   float momentum = 0.9f, const std::string& data_layout = "NCHW", bool is_test = true);
+  // cinn/frontend/net_builder.cc:419-432
+  Variable ReluGrad(const Variable& dout, const Variable& out);
+  std::vector<Variable> ElementwiseAddGrad(const Variable& dout, const Variable& x, const Variable& y, int axis = -1);
   std::vector<Variable> BatchNormGrad(const Variable& dy, const Variable& x, const Variable& scale,
                                       const Variable& save_mean, const Variable& save_variance, float epsilon = 1e-5f,
                                       const std::string& data_layout = "NCHW");

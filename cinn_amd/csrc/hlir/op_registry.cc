@@ -454,6 +454,24 @@ OpRegistry::OpRegistry() {
   }
 
   {
+    // relu_grad(dout, out) -> dx
+    auto& op       = r->Register("relu_grad");
+    op.pattern     = OpPatternKind::kNonFusible;
+    op.num_inputs  = 2;
+    op.infer_shape = SameShapeAsFirst;
+    op.infer_dtype = SameTypeAsFirst;
+  }
+  {
+    // elementwise_add_grad(dout, x, y) -> dx, dy with the shapes of x and y
+    auto& op       = r->Register("elementwise_add_grad");
+    op.pattern     = OpPatternKind::kNonFusible;
+    op.num_inputs  = 3;
+    op.infer_shape = [](const std::vector<ShapeType>& in, const AttributeMap&) {
+      return std::vector<ShapeType>{in[1], in[2]};
+    };
+    op.infer_dtype = [](const std::vector<Type>& in, const AttributeMap&) { return std::vector<Type>{in[1], in[2]}; };
+  }
+  {
     // training form: x, scale, bias, moving_mean, moving_variance -> y, saved_mean, saved_variance, moving_mean,
     // moving_variance (cinn/hlir/op/nn.cc batch_norm_train)
     auto& op       = r->Register("batch_norm_train");

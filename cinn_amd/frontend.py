@@ -221,6 +221,13 @@ class NetBuilder(object):
         return self._call("BatchNorm", [x, scale, bias, mean, variance], epsilon=float(epsilon),
                           momentum=float(momentum), data_layout=data_layout, is_test=is_test)
 
+    def relu_grad(self, dout, out):
+        return self._call1("ReluGrad", [dout, out])
+
+    def elementwise_add_grad(self, dout, x, y, axis=-1):
+        """Returns [dx, dy]."""
+        return self._call("ElementwiseAddGrad", [dout, x, y], axis=axis)
+
     def batch_norm_grad(self, dy, x, scale, save_mean, save_variance, epsilon=1e-5, data_layout="NCHW"):
         """Returns [x_grad, scale_grad, bias_grad] (cinn/pybind/frontend.cc `batch_norm_grad`)."""
         return self._call("BatchNormGrad", [dy, x, scale, save_mean, save_variance], epsilon=float(epsilon),

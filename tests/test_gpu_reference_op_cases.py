@@ -8,7 +8,9 @@ cinn_call_cudnn_conv2d_forward / _backward_data / _backward_filter / cinn_call_c
     (builder.conv(..., conv_type="backward_data" / "backward_filter", output_shape=...)), fp16 / fp32 / fp64;
   * python/tests/ops/test_pool2d_op.py:80-330  - six forward attribute sets on four shapes and the four gradient sets;
   * python/tests/ops/test_reduce_op.py, test_reduce_op_new.py, test_reduce_op_other.py - every reduction case;
-  * python/tests/ops/test_batch_norm_op.py:15-275 - the training form, its gradient and the inference form.
+  * python/tests/ops/test_batch_norm_op.py:15-275 - the training form, its gradient and the inference form;
+  * python/tests/ops/test_add_op.py:84-260 and test_relu_op.py:60-137 - add with elementwise_add_grad (equal shapes and
+    y of ones), relu with relu_grad, over their shape and type lists (the operators of the first configuration).
 
 The reference compares with Paddle at the same precision; here the expected values are float64 numpy (matmul), the
 CPU oracle (convolution and its gradients, pooling in fp32 / fp16) or float64 window loops written out below (fp64
@@ -529,3 +531,78 @@ def test_batch_norm_inference(gpu, shape):
     want = torch.nn.functional.batch_norm(torch.from_numpy(x.astype(np.float64)), torch.zeros(c, dtype=torch.float64),
                                           torch.ones(c, dtype=torch.float64), training=False, eps=1e-5).numpy()
     close(got, want, 1e-5, 1e-6)
+
+
+# ---- add / relu with their gradients --------------------------------------------------------------------------------
+ADD_SHAPES = [([1], 0), ([1024], -1), ([512, 256], 0), ([128, 64, 32], -1), ([16, 8, 4, 2], 0), ([16, 8, 4, 2, 1], -1)]
+ADD_TYPES = ["int32", "int64", "float16", "float32", "float64"]
+ALL_NP = dict(TYPE_OF, float16=(np.float16, None))
+
+
+def any_type(dtype):
+    return Float(16) if dtype == "float16" else cinn_type(dtype)
+
+
+def add_input(seed, shape, dtype):
+    rng = np.random.default_rng(seed)
+    if dtype.startswith("int"):
+        return rng.integers(0, 100, shape).astype(ALL_NP[dtype][0])
+    return rng.uniform(0.0, 1.0, shape).astype(ALL_NP[dtype][0])
+
+
+@pytest.mark.parametrize("broadcast", [False, True])
+@pytest.mark.parametrize("dtype", ADD_TYPES)
+@pytest.mark.parametrize("shape,axis", ADD_SHAPES)
+def test_add_with_gradients(gpu, shape, axis, dtype, broadcast):
+    y_shape = [1] * len(shape) if broadcast else shape
+    x, y, dout = add_input(18, shape, dtype), add_input(19, y_shape, dtype), add_input(20, shape, dtype)
+    b = NetBuilder("add")
+    X, Y, D = (b.create_input(any_type(dtype), s, n) for s, n in ((shape, "x"), (y_shape, "y"), (shape, "dout")))
+    out = b.add(X, Y, axis=axis)
+    dx, dy = b.elementwise_add_grad(D, X, Y, axis=axis)
+    (got, got_dx, got_dy), _ = run(b, {X: x, Y: y, D: dout}, [out, dx, dy])
+    assert got.dtype == x.dtype and got_dx.dtype == x.dtype and got_dy.dtype == x.dtype
+    assert np.array_equal(got, x + y)          # one rounding of an exact sum in every type
+    assert np.array_equal(got_dx, dout)
+    if not broadcast:
+        assert np.array_equal(got_dy, dout)
+    elif dtype.startswith("int"):
+        assert list(got_dy.shape) == y_shape and got_dy.reshape(-1)[0] == dout.sum(dtype=dout.dtype)
+    else:
+        want = dout.astype(np.float64).sum()
+        assert list(got_dy.shape) == y_shape
+        tol = {"float16": 1e-3, "float32": 1e-5, "float64": 1e-12}[dtype]
+        if dtype == "float16" and want > 65504.0:
+            # [512, 256] and [128, 64, 32] values of mean 1/2 add up beyond the largest half: the sum, taken in fp32,
+            # rounds to infinity in the result type
+            assert np.isposinf(got_dy.reshape(-1)[0])
+        else:
+            assert abs(float(got_dy.reshape(-1)[0]) - want) <= tol * want + 1e-6
+
+
+RELU_SHAPES = [[10], [8, 5], [10, 3, 5], [80, 40, 5, 7], [80, 1, 5, 7], [80, 3, 1024, 7], [10, 5, 1024, 2048], [1], [512],
+               [1024], [2048], [1, 1, 1, 1]]
+
+
+def run_relu(shape, dtype):
+    rng = np.random.default_rng(21)
+    x = rng.uniform(-1.0, 1.0, shape).astype(ALL_NP[dtype][0])
+    dout = rng.uniform(-1.0, 1.0, shape).astype(ALL_NP[dtype][0])
+    b = NetBuilder("relu")
+    X, D = b.create_input(any_type(dtype), shape, "x"), b.create_input(any_type(dtype), shape, "dout")
+    out = b.relu(X)
+    x_grad = b.relu_grad(D, out)
+    (got, got_grad), _ = run(b, {X: x, D: dout}, [out, x_grad])
+    assert np.array_equal(got, np.maximum(x, 0))
+    assert np.array_equal(got_grad, np.where(x > 0, dout, 0).astype(x.dtype))
+
+
+@pytest.mark.parametrize("shape", RELU_SHAPES)
+def test_relu_with_gradient_shapes(gpu, shape):
+    run_relu(shape, "float32")
+
+
+@pytest.mark.parametrize("dtype", ["float16", "float32", "float64"])
+@pytest.mark.parametrize("shape", [[1], [5], [80, 40, 5, 7]])
+def test_relu_with_gradient_types(gpu, shape, dtype):
+    run_relu(shape, dtype)
