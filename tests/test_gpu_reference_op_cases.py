@@ -10,7 +10,9 @@ cinn_call_cudnn_conv2d_forward / _backward_data / _backward_filter / cinn_call_c
   * python/tests/ops/test_reduce_op.py, test_reduce_op_new.py, test_reduce_op_other.py - every reduction case;
   * python/tests/ops/test_batch_norm_op.py:15-275 - the training form, its gradient and the inference form;
   * python/tests/ops/test_add_op.py:84-260 and test_relu_op.py:60-137 - add with elementwise_add_grad (equal shapes and
-    y of ones), relu with relu_grad, over their shape and type lists (the operators of the first configuration).
+    y of ones), relu with relu_grad, over their shape and type lists (the operators of the first configuration);
+  * python/tests/ops/test_transpose_op.py, test_reshape_op.py, test_concat_op.py, test_cast_op.py, test_scale_op.py -
+    data movement and type conversion, bit for bit.
 
 The reference compares with Paddle at the same precision; here the expected values are float64 numpy (matmul), the
 CPU oracle (convolution and its gradients, pooling in fp32 / fp16) or float64 window loops written out below (fp64
@@ -606,3 +608,147 @@ def test_relu_with_gradient_shapes(gpu, shape):
 @pytest.mark.parametrize("shape", [[1], [5], [80, 40, 5, 7]])
 def test_relu_with_gradient_types(gpu, shape, dtype):
     run_relu(shape, dtype)
+
+
+# ---- transpose / reshape / concat / cast / scale ---------------------------------------------------------------------
+# python/tests/ops/test_transpose_op.py:48-196, test_reshape_op.py:46-182, test_concat_op.py:65-300,
+# test_cast_op.py:50-137, test_scale_op.py:46-140: data movement and type conversion are exact, so every case is
+# compared bit for bit with numpy.
+TRANSPOSE_CASES = [([512], [0]), ([1024], [-1]), ([1200], [0]), ([64, 16], [1, 0]), ([4, 32, 8], [1, 0, 2]),
+                   ([16, 8, 4, 2], [0, 2, 1, 3]), ([2, 8, 4, 2, 5], [0, 2, 3, 1, 4]), ([4, 8, 1, 2, 16], [0, 2, 4, 1, 3]),
+                   ([1], [0]), ([1, 1, 1, 1], [0, 2, 3, 1]), ([1, 1, 1, 1, 1], [0, 2, 3, 1, 4]),
+                   ([1, 1, 512, 1, 1], [0, 2, 3, 1, 4]), ([1, 2048, 1, 1], [0, 2, 3, 1]), ([2048], [0]),
+                   ([1, 1, 65536, 1], [0, 2, 3, 1]), ([1, 1, 131072, 1, 1], [0, 2, 3, 1, 4]),
+                   ([1, 1048576, 1, 1], [0, 2, 3, 1]), ([16, 32, 64, 32], [0, 2, 3, 1])]
+TRANSPOSE_TYPED = [([1024], [0]), ([64, 16], [1, 0]), ([4, 32, 8], [0, 2, 1]), ([16, 8, 4, 2], [1, 2, 3, 0])]
+RESHAPE_CASES = [([100], [100]), ([100], [10, 10]), ([125], [5, 5, 5]), ([256], [4, 4, 4, 4]), ([1024], [8, 8, 4, 4]),
+                 ([5, 5], [25]), ([6, 8], [4, 12]), ([10, 20], [5, 10, 4]), ([4, 8], [2, 2, 2, 4]),
+                 ([16, 16], [4, 2, 2, 1, 16]), ([1, 1, 1], [1]), ([1, 2, 3], [6, 1]), ([4, 8, 16], [16, 8, 4]),
+                 ([6, 6, 6], [4, 9, 2, 3]), ([8, 1, 8], [2, 2, 2, 2, 4]), ([4, 1, 2, 1], [8]), ([2, 2, 4, 8], [4, 32]),
+                 ([6, 7, 8, 9], [42, 36, 2]), ([1024, 1, 1, 1], [4, 4, 8, 8]), ([10, 20, 30, 40], [8, 6, 4, 2, 625]),
+                 ([1, 1024, 4], [1, 2048, 2]), ([2048, 2, 2], [256, 8, 4]), ([1, 1, 256], [16, 1, 16]),
+                 ([1, 1, 1, 1], [1, 1]), ([1, 1, 1], [1]), ([1], [1, 1, 1, 1])]
+CONCAT_CASES = [([[10], [6]], 0), ([[8, 5], [8, 5]], 0), ([[10, 3, 5], [4, 3, 5]], 0), ([[80, 40, 5, 7], [20, 40, 5, 7]], 0),
+                ([[80, 1, 5, 7], [8, 1, 5, 7]], 0), ([[80, 3, 1024, 7], [100, 3, 1024, 7]], 0),
+                ([[1, 5, 1024, 2048], [2, 5, 1024, 2048]], 0), ([[1], [1]], 0), ([[512], [512]], 0), ([[1024], [512]], 0),
+                ([[2048], [4096]], 0), ([[1, 1, 1, 1], [1, 1, 1, 1]], 0), ([[10]], 0), ([[10], [6], [8]], 0),
+                ([[10], [6], [10], [6]], 0), ([[8, 5]], 1), ([[8, 5], [8, 8]], 1), ([[8, 5], [8, 5], [16, 5]], 0),
+                ([[8, 5], [8, 5], [8, 5], [8, 5]], 0), ([[10, 3, 5]], 0), ([[10, 3, 5], [10, 7, 5]], 1),
+                ([[10, 3, 5], [10, 3, 6], [10, 3, 7]], 2), ([[10, 3, 5], [4, 3, 5], [2, 3, 5]], 0), ([[80, 1, 5, 7]], 0),
+                ([[80, 1, 5, 7], [80, 79, 5, 7]], 1), ([[80, 1, 50, 7], [80, 1, 5, 7], [80, 1, 10, 7]], 2),
+                ([[80, 1, 5, 17], [80, 1, 5, 27], [80, 1, 5, 37]], 3), ([[10], [6]], -1), ([[8, 5], [10, 5]], 0),
+                ([[10, 3, 15], [10, 3, 5]], 2), ([[10, 3, 7], [10, 3, 5]], -1), ([[10, 3, 5], [10, 7, 5]], -2),
+                ([[10, 7, 5], [20, 7, 5]], -3)]
+CONCAT_TYPES = ["float16", "float32", "float64", "bool", "uint8", "int8", "int32", "int64"]
+CAST_TYPES = ["bool", "int8", "int16", "int32", "int64", "float16", "float32", "float64"]
+WIDE_NP = {"bool": np.bool_, "uint8": np.uint8, "int8": np.int8, "int16": np.int16, "int32": np.int32, "int64": np.int64,
+           "float16": np.float16, "float32": np.float32, "float64": np.float64}
+
+
+def wide_type(dtype):
+    from cinn_amd.common import Bool, Int, UInt
+    if dtype == "bool":
+        return Bool()
+    if dtype.startswith("uint"):
+        return UInt(int(dtype[4:]))
+    if dtype.startswith("int"):
+        return Int(int(dtype[3:]))
+    return Float(int(dtype[5:]))
+
+
+def wide_input(seed, shape, dtype):
+    """OpTest.random: uniform [0, 1) for floating types, integers of [0, 100) for integer types (int8 / uint8 too),
+    coin flips for bool."""
+    rng = np.random.default_rng(seed)
+    if dtype == "bool":
+        return rng.integers(0, 2, shape).astype(np.bool_)
+    if "int" in dtype:
+        return rng.integers(0, 100, shape).astype(WIDE_NP[dtype])
+    return rng.uniform(0.0, 1.0, shape).astype(WIDE_NP[dtype])
+
+
+@pytest.mark.parametrize("shape,axes", TRANSPOSE_CASES)
+def test_transpose_cases(gpu, shape, axes):
+    x = wide_input(22, shape, "float32")
+    b = NetBuilder("transpose")
+    X = b.create_input(Float(32), shape, "x")
+    (got,), _ = run(b, {X: x}, [b.transpose(X, axes)])
+    assert np.array_equal(got, x.transpose([a % len(shape) for a in axes]))
+
+
+@pytest.mark.parametrize("dtype", ["float16", "float32", "float64"])
+@pytest.mark.parametrize("shape,axes", TRANSPOSE_TYPED)
+def test_transpose_types(gpu, shape, axes, dtype):
+    x = wide_input(23, shape, dtype)
+    b = NetBuilder("transpose")
+    X = b.create_input(wide_type(dtype), shape, "x")
+    (got,), _ = run(b, {X: x}, [b.transpose(X, axes)])
+    assert got.dtype == x.dtype and np.array_equal(got, x.transpose(axes))
+
+
+@pytest.mark.parametrize("shape,target", RESHAPE_CASES)
+def test_reshape_cases(gpu, shape, target):
+    x = wide_input(24, shape, "float32")
+    b = NetBuilder("reshape")
+    X = b.create_input(Float(32), shape, "x")
+    (got,), _ = run(b, {X: x}, [b.reshape(X, target)])
+    assert np.array_equal(got, x.reshape(target))
+
+
+@pytest.mark.parametrize("shapes,axis", CONCAT_CASES)
+def test_concat_cases(gpu, shapes, axis):
+    xs = [wide_input(25 + i, s, "float32") for i, s in enumerate(shapes)]
+    b = NetBuilder("concat")
+    X = [b.create_input(Float(32), s, "x%d" % i) for i, s in enumerate(shapes)]
+    (got,), _ = run(b, dict(zip(X, xs)), [b.concat(X, axis=axis)])
+    assert np.array_equal(got, np.concatenate(xs, axis=axis))
+
+
+@pytest.mark.parametrize("dtype", CONCAT_TYPES)
+@pytest.mark.parametrize("shapes", [[[10], [6]], [[8, 5], [8, 5]], [[10, 3, 5], [4, 3, 5]], [[80, 40, 5, 7], [20, 40, 5, 7]]])
+def test_concat_types(gpu, shapes, dtype):
+    xs = [wide_input(30 + i, s, dtype) for i, s in enumerate(shapes)]
+    b = NetBuilder("concat")
+    X = [b.create_input(wide_type(dtype), s, "x%d" % i) for i, s in enumerate(shapes)]
+    (got,), _ = run(b, dict(zip(X, xs)), [b.concat(X, axis=0)])
+    assert got.dtype == xs[0].dtype and np.array_equal(got, np.concatenate(xs, axis=0))
+
+
+@pytest.mark.parametrize("shape", [[1], [1024], [32, 64], [16, 8, 4, 2]])
+def test_cast_shapes(gpu, shape):
+    x = wide_input(35, shape, "float32")
+    b = NetBuilder("cast")
+    X = b.create_input(Float(32), shape, "x")
+    (got,), _ = run(b, {X: x}, [b.cast(X, "float64")])
+    assert got.dtype == np.float64 and np.array_equal(got, x.astype(np.float64))
+
+
+@pytest.mark.parametrize("to", CAST_TYPES)
+@pytest.mark.parametrize("frm", CAST_TYPES)
+def test_cast_every_pair_of_types(gpu, frm, to):
+    x = wide_input(36, [32, 64], frm)
+    b = NetBuilder("cast")
+    X = b.create_input(wide_type(frm), [32, 64], "x")
+    (got,), _ = run(b, {X: x}, [b.cast(X, to)])
+    assert got.dtype == WIDE_NP[to]
+    assert np.array_equal(got, x.astype(WIDE_NP[to]))   # values of [0, 100) / [0, 1): every conversion is exact or one rounding
+
+
+@pytest.mark.parametrize("shape", [[1], [1024], [512, 256], [128, 64, 32], [16, 8, 4, 2], [16, 8, 4, 2, 1]])
+def test_scale_shapes(gpu, shape):
+    x = wide_input(37, shape, "float32")
+    b = NetBuilder("scale")
+    X = b.create_input(Float(32), shape, "x")
+    (got,), _ = run(b, {X: x}, [b.scale(X, -0.1, 10, False)])
+    close(got, (x.astype(np.float64) + 10.0) * np.float64(np.float32(-0.1)), 1e-6, 1e-6)
+
+
+@pytest.mark.parametrize("scale,bias,after", [(0, 0, True), (0, 0, False), (0.1, 10, True), (-0.1, 10, False)])
+def test_scale_attributes(gpu, scale, bias, after):
+    x = wide_input(38, [32, 64], "float32")
+    b = NetBuilder("scale")
+    X = b.create_input(Float(32), [32, 64], "x")
+    (got,), _ = run(b, {X: x}, [b.scale(X, scale, bias, after)])
+    s = np.float64(np.float32(scale))
+    want = x.astype(np.float64) * s + bias if after else (x.astype(np.float64) + bias) * s
+    close(got, want, 1e-6, 1e-6)
