@@ -38,6 +38,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 template <typename T>
 struct Half16;
@@ -61,6 +62,15 @@ struct Half16<_Float16> {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
 };
+
+// two fp32 values rounded to nearest even into one dword of two T (v_cvt_pk_f16_f32 / v_cvt_pk_bf16_f32)
+template <typename T>
+__device__ __forceinline__ uint32_t PackPair(float a, float b) {
+  typedef T pair_t __attribute__((ext_vector_type(2)));
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  const f32x2 f = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, pair_t));
+}
 
 constexpr int kBM      = 256;
 constexpr int kBN      = 256;
@@ -887,8 +897,15 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 // Both operands are read from global memory straight in fragment layout (16 bytes of one row per lane); the rows and
 // the residual of the next group are requested before the current group is computed.  Per-column scale / shift sit
 // in LDS.  No block barrier after the start-up.
+// Measured on [100352, 64] x [256, 64]^T (51 MB of results, fp16; 19.4 us): the same stores alone, in this kernel's
+// pattern of four 256-byte row pieces per instruction, take 9.6 us (5.3 TB/s), a copy of 12.8 MB into 51 MB 13.5 us;
+// with the stores removed the kernel takes 12.2 us, with the row loads removed 15.4 us.  Start-up (launch, 16 KB of
+// filter fragments per wavefront) is 5 us of that.  Neither the instruction count of the epilogue (219 -> 122 vector
+// instructions per group with packed conversions, a max for the relu and scalar group addresses), nor exact waits
+// (loads in inline assembly, vmcnt counted by hand), nor 12 or 16 wavefronts per CU changed the time: the loop is
+// bound by stores and loads taking turns on the memory side, not by issue.
 // ---------------------------------------------------------------------------------------------------
-template <typename T, int NT, int KH, bool RES, bool B_KC>
+template <typename T, int NT, int KH, bool RES, bool B_KC, bool RELU>
 __global__ void __launch_bounds__(256)
 gemm16_shortk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* __restrict__ C, int M, int N,
                      int64_t lda, int64_t ldb, int64_t ldc, DmaEpilogue epi, int64_t stride_a, int64_t stride_b,
@@ -905,7 +922,7 @@ gemm16_shortk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict_
   __shared__ __attribute__((aligned(16))) char s_stage[4 * 16 * kStageRow];
   const int tid  = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   char* my_stage = s_stage + wave * 16 * kStageRow;  // private to the wavefront: no block barrier in the loop
   // consecutive block ids go round-robin to the 8 XCDs: the ny column panels of one row range stay on one XCD
   const int lin = blockIdx.x, xcd = lin & 7, idx = lin >> 3;
@@ -937,41 +954,58 @@ gemm16_shortk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict_
         for (int q = 0; q < 8; ++q) col[q] = B[(int64_t)(kh * 32 + fk + q) * ldb + n0 + j * 16 + frow];
         __builtin_memcpy(&wf[j][kh], col, 16);
       }
+  // The filter fragments are complete before the loop starts; left to the compiler, the waits for them sit at their
+  // first use, inside the loop, where they would also wait for the rows just requested.
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int kh = 0; kh < KH; ++kh) asm volatile("" : "+v"(wf[j][kh]));
   __syncthreads();
 
   const int groups  = (M + 15) >> 4;
   const int gstride = slots * 4;
   int g             = slot * 4 + wave;
   if (g >= groups) return;
-  struct alignas(8) Res4 { T v[4]; };
+  // A group's first row is the same for the whole wavefront: its address is scalar arithmetic, and what a lane adds
+  // (its row inside the group, its columns) is computed once - 32-bit element offsets, 16 rows of a matrix being far
+  // below 2^31 elements.  Only the last group of a matrix whose rows are not a multiple of 16 clamps its rows.
+  constexpr int kStores = 16 / kRowsPerStore;
+  const int a_lane = frow * (int)lda + fk;
+  int c_lane[kStores];
+#pragma unroll
+  for (int i = 0; i < kStores; ++i)
+    c_lane[i] = (i * kRowsPerStore + lane / kChunksPerRow) * (int)ldc + n0 + (lane % kChunksPerRow) * 8;
   auto request = [&](int grp, vec8* xa, vec8* rr) {
-    int row = grp * 16 + frow;
-    row     = row < M ? row : M - 1;
+    const int valid           = M - grp * 16;  // rows of the group inside the matrix
+    const uint16_t* const a_g = A + (int64_t)grp * 16 * lda;
+    const int a_at            = valid >= 16 ? a_lane : min(frow, valid - 1) * (int)lda + fk;
 #pragma unroll
-    for (int kh = 0; kh < KH; ++kh) xa[kh] = *reinterpret_cast<const vec8*>(A + (int64_t)row * lda + kh * 32 + fk);
+    for (int kh = 0; kh < KH; ++kh) xa[kh] = *reinterpret_cast<const vec8*>(a_g + a_at + kh * 32);
     if (RES) {
+      const T* const r_g = Rt + (int64_t)grp * 16 * ldc;
 #pragma unroll
-      for (int i = 0; i < 16 / kRowsPerStore; ++i) {
-        int rrow = grp * 16 + i * kRowsPerStore + lane / kChunksPerRow;
-        rrow     = rrow < M ? rrow : M - 1;
-        rr[i]    = *reinterpret_cast<const vec8*>(Rt + (int64_t)rrow * ldc + n0 + (lane % kChunksPerRow) * 8);
+      for (int i = 0; i < kStores; ++i) {
+        const int at = valid >= 16 ? c_lane[i]
+                                   : min(i * kRowsPerStore + lane / kChunksPerRow, valid - 1) * (int)ldc + n0 +
+                                         (lane % kChunksPerRow) * 8;
+        rr[i] = *reinterpret_cast<const vec8*>(r_g + at);
       }
     }
   };
   // a ring of D groups: the rows (and residual) of the group D - 1 steps ahead are requested while the current one is
   // computed (three steps ahead measured the same as one: 17.6 against 17.0 us for 100352 x 256 x 64)
   constexpr int D = 2;
+  static_assert(D == 2, "the loop below requests exactly one group ahead");
   vec8 xa[D][KH];
-  vec8 rr[D][RES ? 16 / kRowsPerStore : 1];
-#pragma unroll
-  for (int d = 0; d < D - 1; ++d)
-    if (g + d * gstride < groups) request(g + d * gstride, xa[d], rr[d]);
+  vec8 rr[D][RES ? kStores : 1];
+  request(g, xa[0], rr[0]);
   for (;;) {
 #pragma unroll
     for (int u = 0; u < D; ++u) {
       const int gn        = g + gstride;
       const bool has_next = gn < groups;
-      if (g + (D - 1) * gstride < groups) request(g + (D - 1) * gstride, xa[(u + D - 1) % D], rr[(u + D - 1) % D]);
+      if (has_next) request(gn, xa[(u + 1) % D], rr[(u + 1) % D]);
       f32x4 acc[NT];
 #pragma unroll
       for (int j = 0; j < NT; ++j) acc[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -979,6 +1013,12 @@ gemm16_shortk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict_
       for (int kh = 0; kh < KH; ++kh)
 #pragma unroll
         for (int j = 0; j < NT; ++j) acc[j] = Half16<T>::mfma16(wf[j][kh], xa[u][kh], acc[j]);
+      // the sums are wanted in ordinary registers: the epilogue's arithmetic cannot read the accumulation registers,
+      // and a copy per value is a fifth of this loop's instructions
+#pragma unroll
+      for (int j = 0; j < NT; ++j) asm volatile("" : "+v"(acc[j]));
+      const int valid   = M - g * 16;
+      T* const c_g      = reinterpret_cast<T*>(C) + (int64_t)g * 16 * ldc;
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
         const f32x4 sc = *reinterpret_cast<const f32x4*>(&s_scale[j * 16 + 4 * (lane >> 4)]);
@@ -989,15 +1029,15 @@ gemm16_shortk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict_
           for (int r = 0; r < 4; ++r) v4[r] = __builtin_fmaf(acc[j][r], sc[r], sh[r]);
           *reinterpret_cast<f32x4*>(my_stage + frow * kStageRow + (j * 16 + 4 * (lane >> 4)) * 4) = v4;
         } else {
-          Res4 out;
+          float v[4];
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            float v = __builtin_fmaf(acc[j][r], sc[r], sh[r]);
-            asm volatile("" : "+v"(v));  // one rounding to T for every element, see gemm16_dma_kernel's epilogue
-            if (epi.relu) v = v > 0.0f ? v : 0.0f;
-            out.v[r] = (T)v;
+            v[r] = __builtin_fmaf(acc[j][r], sc[r], sh[r]);
+            if (RELU) v[r] = __builtin_fmaxf(v[r], 0.0f);  // a NaN becomes 0, as with v > 0 ? v : 0
+            asm volatile("" : "+v"(v[r]));  // one rounding to T for every element, see gemm16_dma_kernel's epilogue
           }
-          *reinterpret_cast<Res4*>(my_stage + frow * kStageRow + (j * 16 + 4 * (lane >> 4)) * 2) = out;
+          u32x2 out = {PackPair<T>(v[0], v[1]), PackPair<T>(v[2], v[3])};
+          *reinterpret_cast<u32x2*>(my_stage + frow * kStageRow + (j * 16 + 4 * (lane >> 4)) * 2) = out;
         }
       }
       // the wavefront's own 16 x NW tile comes back as whole rows: 16 bytes of C per lane, full lines per store
@@ -1006,28 +1046,27 @@ gemm16_shortk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict_
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-      for (int i = 0; i < 16 / kRowsPerStore; ++i) {
+      for (int i = 0; i < kStores; ++i) {
         const int srow = i * kRowsPerStore + lane / kChunksPerRow;
         const int ch   = lane % kChunksPerRow;
         u32x4 v;
         if (RES) {
           const f32x4 lo = *reinterpret_cast<const f32x4*>(my_stage + srow * kStageRow + ch * 32);
           const f32x4 hi = *reinterpret_cast<const f32x4*>(my_stage + srow * kStageRow + ch * 32 + 16);
-          vec8 out;
+          float t[8];
 #pragma unroll
           for (int q = 0; q < 8; ++q) {
-            float t = __builtin_fmaf(epi.residual_scale, (float)rr[u][RES ? i : 0][q], q < 4 ? lo[q] : hi[q - 4]);
-            asm volatile("" : "+v"(t));
-            if (epi.relu) t = t > 0.0f ? t : 0.0f;
-            out[q] = (T)t;
+            t[q] = __builtin_fmaf(epi.residual_scale, (float)rr[u][RES ? i : 0][q], q < 4 ? lo[q] : hi[q - 4]);
+            if (RELU) t[q] = __builtin_fmaxf(t[q], 0.0f);
+            asm volatile("" : "+v"(t[q]));
           }
-          v = *reinterpret_cast<const u32x4*>(&out);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] = PackPair<T>(t[2 * q], t[2 * q + 1]);
         } else {
           v = *reinterpret_cast<const u32x4*>(my_stage + srow * kStageRow + ch * 16);
         }
-        const int row = g * 16 + srow;
-        if (row < M) {
-          u32x4* dst = reinterpret_cast<u32x4*>(reinterpret_cast<T*>(C) + (int64_t)row * ldc + n0 + ch * 8);
+        if (srow < valid) {
+          u32x4* dst = reinterpret_cast<u32x4*>(c_g + c_lane[i]);
           if (epi.streaming) {
             __builtin_nontemporal_store(v, dst);
           } else {
@@ -1570,11 +1609,19 @@ void LaunchShortK(const GemmProblem& p, hipStream_t stream) {
   epi.residual_scale = p.residual ? p.residual_scale : p.beta;
   epi.streaming      = !p.keep_in_cache && (int64_t)p.batch * p.m * p.n * 2 >= (16 << 20);
   dim3 grid(slots * ny, p.batch, 1);
-#define CINN_SHORTK(RES, B_KC)                                                                                       \
-  hipLaunchKernelGGL((gemm16_shortk_kernel<T, NT, KH, RES, B_KC>), grid, dim3(256), 0, stream,                        \
+#define CINN_SHORTK_R(RES, B_KC, RELU)                                                                              \
+  hipLaunchKernelGGL((gemm16_shortk_kernel<T, NT, KH, RES, B_KC, RELU>), grid, dim3(256), 0, stream,                  \
                      static_cast<const uint16_t*>(p.a), static_cast<const uint16_t*>(p.b), static_cast<uint16_t*>(p.c), \
                      p.m, p.n, (int64_t)p.k, (int64_t)(B_KC ? p.k : p.n), (int64_t)p.n, epi, p.stride_a, p.stride_b,    \
                      p.stride_c, ny)
+#define CINN_SHORTK(RES, B_KC)      \
+  do {                              \
+    if (epi.relu) {                 \
+      CINN_SHORTK_R(RES, B_KC, true);  \
+    } else {                        \
+      CINN_SHORTK_R(RES, B_KC, false); \
+    }                               \
+  } while (0)
   if (epi.residual) {
     if (p.trans_b) {
       CINN_SHORTK(true, true);
@@ -1587,6 +1634,7 @@ void LaunchShortK(const GemmProblem& p, hipStream_t stream) {
     CINN_SHORTK(false, false);
   }
 #undef CINN_SHORTK
+#undef CINN_SHORTK_R
 }
 
 template <typename T>
