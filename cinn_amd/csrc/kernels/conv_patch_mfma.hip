@@ -147,18 +147,19 @@ __device__ __forceinline__ void PatchEpilogue(const PatchParams& p, const f32x4 
     u32x4 out[2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      vec8 o8;
+      float v[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         // explicit fused multiply-adds rounded to fp32 and an empty asm before the conversion: the same arithmetic,
-        // in the same order, as the epilogues of the other convolution kernels
-        float v = __builtin_fmaf(acc[i][2 * s + (e >> 2)][e & 3], ss.sc[s][e], ss.sh[s][e]);
-        if (R) v = __builtin_fmaf(p.residual_scale, (float)res[s][e], v);
-        asm volatile("" : "+v"(v));
-        if (p.relu) v = v > 0.0f ? v : 0.0f;
-        o8[e] = (T)v;
+        // in the same order, as the epilogues of the other convolution kernels; the relu is a max (a NaN becomes 0,
+        // as with v > 0 ? v : 0) under a select on the flag, the conversion takes two values at a time
+        v[e] = __builtin_fmaf(acc[i][2 * s + (e >> 2)][e & 3], ss.sc[s][e], ss.sh[s][e]);
+        if (R) v[e] = __builtin_fmaf(p.residual_scale, (float)res[s][e], v[e]);
+        const float m = __builtin_fmaxf(v[e], 0.0f);
+        v[e]          = p.relu ? m : v[e];
+        asm volatile("" : "+v"(v[e]));
       }
-      out[s] = __builtin_bit_cast(u32x4, o8);
+      out[s] = u32x4{PackPair<T>(v[0], v[1]), PackPair<T>(v[2], v[3]), PackPair<T>(v[4], v[5]), PackPair<T>(v[6], v[7])};
     }
     // first store: slots 0..7 of the tile as whole 128-byte lines (lanes px < 8: their own channels 8 g ..; lanes
     // px >= 8: the channels 32 + 8 g .. of slot px - 8); second store: slots 8..15 (lanes px >= 8: their own channels

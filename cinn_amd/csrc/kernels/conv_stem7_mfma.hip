@@ -320,15 +320,17 @@ __global__ void __launch_bounds__(512) conv_stem7_kernel(Stem7Params p) {
         const int ox = 16 * i + px;
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-          vec8 o8;
+          float v[8];
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
-            float v = __builtin_fmaf(acc[i][2 * s + (e >> 2)][e & 3], sc[s][e], sh[s][e]);
-            asm volatile("" : "+v"(v));
-            v     = valid && v > 0.0f ? v : 0.0f;
-            o8[e] = (T)v;
+            // relu as a max (a NaN becomes 0, as with v > 0 ? v : 0), zero for a row outside the image; the empty asm
+            // keeps the fused multiply-add and the conversion apart (one rounding each)
+            v[e] = __builtin_fmaxf(__builtin_fmaf(acc[i][2 * s + (e >> 2)][e & 3], sc[s][e], sh[s][e]), 0.0f);
+            v[e] = valid ? v[e] : 0.0f;
+            asm volatile("" : "+v"(v[e]));
           }
-          if (ox < p.ow) *reinterpret_cast<vec8*>(stage + (wave * p.ow + ox) * kStagePitch + (g + 4 * s) * 16) = o8;
+          const u32x4 o8 = {PackPair<T>(v[0], v[1]), PackPair<T>(v[2], v[3]), PackPair<T>(v[4], v[5]), PackPair<T>(v[6], v[7])};
+          if (ox < p.ow) *reinterpret_cast<u32x4*>(stage + (wave * p.ow + ox) * kStagePitch + (g + 4 * s) * 16) = o8;
         }
       }
       BarrierLds();  // the five rows are staged
@@ -347,16 +349,16 @@ __global__ void __launch_bounds__(512) conv_stem7_kernel(Stem7Params p) {
       u32x4 out[2];
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        vec8 o8;
+        float v[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          float v = __builtin_fmaf(acc[i][2 * s + (e >> 2)][e & 3], sc[s][e], sh[s][e]);
-          if (R) v = __builtin_fmaf(p.residual_scale, (float)res[s][e], v);
-          asm volatile("" : "+v"(v));  // keeps the fused multiply-add and the conversion apart (one rounding each)
-          if (p.relu) v = v > 0.0f ? v : 0.0f;
-          o8[e] = (T)v;
+          v[e] = __builtin_fmaf(acc[i][2 * s + (e >> 2)][e & 3], sc[s][e], sh[s][e]);
+          if (R) v[e] = __builtin_fmaf(p.residual_scale, (float)res[s][e], v[e]);
+          const float m = __builtin_fmaxf(v[e], 0.0f);
+          v[e]          = p.relu ? m : v[e];
+          asm volatile("" : "+v"(v[e]));  // keeps the fused multiply-add and the conversion apart (one rounding each)
         }
-        out[s] = __builtin_bit_cast(u32x4, o8);
+        out[s] = u32x4{PackPair<T>(v[0], v[1]), PackPair<T>(v[2], v[3]), PackPair<T>(v[4], v[5]), PackPair<T>(v[6], v[7])};
       }
       u32x4 first, second;
 #pragma unroll

@@ -22,6 +22,8 @@
 // K-contiguous (transpose2d_kernel); gemm_generic_kernel is left with K % (16 bytes) != 0 and fp64.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include <climits>
 #include <cstdint>
 #include <map>
@@ -650,7 +652,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
     _Pragma("unroll") for (int r = 0; r < ROWS; ++r) {                                                       \
       _Pragma("unroll") for (int j = 0; j < TN; ++j) {                                                       \
         CINN_SB;                                                                                             \
-        acc[r % TM][j] = Half16<T>::mfma16(ring[r % 4], bf[r / TM][j], acc[r % TM][j]);                      \
+        acc[r % TM][j] = Half16<T>::mfma16(bf[r / TM][j], ring[r % 4], acc[r % TM][j]);                      \
         CINN_SB;                                                                                             \
         if (j == 0) {                                                                                        \
           if (r + 3 < ROWS) {                                                                                \
@@ -741,12 +743,10 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 #pragma unroll
       for (int ii = 0; ii < IB; ++ii)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int lrow = wm * (IB * 16) + ii * 16 + 4 * (lane >> 4) + r;
-            const int col  = wn * (TN * 16) + j * 16 + (lane & 15);
-            stage[lrow * kRowFloats + col] = acc[IB * pass + ii][j][r];
+        for (int j = 0; j < TN; ++j) {
+            const int lrow = wm * (IB * 16) + ii * 16 + (lane & 15);
+            const int col  = wn * (TN * 16) + j * 16 + 4 * (lane >> 4);
+            *reinterpret_cast<f32x4*>(stage + lrow * kRowFloats + col) = acc[IB * pass + ii][j];
           }
       __syncthreads();
 #pragma unroll
@@ -766,14 +766,16 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   T* Ct       = reinterpret_cast<T*>(C);
   const T* Rt = reinterpret_cast<const T*>(epi.residual);
   if (Rt) Rt += (int64_t)blockIdx.y * stride_c;
-  float sc[TN], sh[TN];
+  float sc[TN][4], sh[TN][4];
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    int col = n0 + wn * (TN * 16) + j * 16 + (lane & 15);
-    col     = col < N ? col : N - 1;
-    sc[j]   = epi.scale ? epi.scale[col] : epi.alpha;
-    sh[j]   = epi.shift ? epi.shift[col] : 0.0f;
-  }
+  for (int j = 0; j < TN; ++j)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      int col  = n0 + wn * (TN * 16) + j * 16 + 4 * (lane >> 4) + r;
+      col      = col < N ? col : N - 1;
+      sc[j][r] = epi.scale ? epi.scale[col] : epi.alpha;
+      sh[j][r] = epi.shift ? epi.shift[col] : 0.0f;
+    }
   constexpr int CPR = BN / 8;  // 8-column chunks per row
   if (!Rt) {
     constexpr int kRowBytes = (BN + 8) * 2;
@@ -784,20 +786,34 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 #pragma unroll
     for (int pass = 0; pass < TM / IB; ++pass) {
       __syncthreads();  // the last stage (or the previous pass) has been read
-      if (!feeder)
+      // a lane's four consecutive columns of a row leave as one 8-byte LDS write; the relu is a max (a NaN becomes 0,
+      // as with v > 0 ? v : 0), chosen by a branch around the pass so that the other form carries no select
+      auto stage_pass = [&](auto relu_tag) {
+        constexpr bool RELU = decltype(relu_tag)::value;
 #pragma unroll
-      for (int ii = 0; ii < IB; ++ii)
+        for (int ii = 0; ii < IB; ++ii)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+          for (int j = 0; j < TN; ++j) {
+            const int lrow = wm * (IB * 16) + ii * 16 + (lane & 15);
+            const int col  = wn * (TN * 16) + j * 16 + 4 * (lane >> 4);
+            float v[4];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int lrow = wm * (IB * 16) + ii * 16 + 4 * (lane >> 4) + r;
-            const int col  = wn * (TN * 16) + j * 16 + (lane & 15);
-            float v        = __builtin_fmaf(acc[IB * pass + ii][j][r], sc[j], sh[j]);
-            asm volatile("" : "+v"(v));  // keeps the fma and the conversion apart, see above
-            if (epi.relu) v = v > 0.0f ? v : 0.0f;
-            *reinterpret_cast<T*>(lds + lrow * kRowBytes + col * 2) = (T)v;
+            for (int r = 0; r < 4; ++r) {
+              v[r] = __builtin_fmaf(acc[IB * pass + ii][j][r], sc[j][r], sh[j][r]);
+              if (RELU) v[r] = __builtin_fmaxf(v[r], 0.0f);
+              asm volatile("" : "+v"(v[r]));  // keeps the fma and the conversion apart, see above
+            }
+            const u32x2 out = {PackPair<T>(v[0], v[1]), PackPair<T>(v[2], v[3])};
+            *reinterpret_cast<u32x2*>(lds + lrow * kRowBytes + col * 2) = out;
           }
+      };
+      if (!feeder) {
+        if (epi.relu) {
+          stage_pass(std::true_type{});
+        } else {
+          stage_pass(std::false_type{});
+        }
+      }
       __syncthreads();
 #pragma unroll
       for (int e = 0; e < PASS_ROWS * CPR / THREADS; ++e) {
@@ -848,12 +864,13 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 #pragma unroll
     for (int ii = 0; ii < IB; ++ii)
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
+      for (int j = 0; j < TN; ++j) {
+          const int lrow = wm * (IB * 16) + ii * 16 + (lane & 15);
+          const int col  = wn * (TN * 16) + j * 16 + 4 * (lane >> 4);
+          f32x4 v4;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int lrow = wm * (IB * 16) + ii * 16 + 4 * (lane >> 4) + r;
-          const int col  = wn * (TN * 16) + j * 16 + (lane & 15);
-          stage[lrow * kRowFloats + col] = __builtin_fmaf(acc[IB * pass + ii][j][r], sc[j], sh[j]);
+          for (int r = 0; r < 4; ++r) v4[r] = __builtin_fmaf(acc[IB * pass + ii][j][r], sc[j][r], sh[j][r]);
+          *reinterpret_cast<f32x4*>(stage + lrow * kRowFloats + col) = v4;
         }
     __syncthreads();
     if (pass + 1 < TM / IB) request_residual(pass + 1, res[(pass + 1) & 1]);
@@ -868,18 +885,20 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
       const f32x4 lo  = *reinterpret_cast<const f32x4*>(stage + lrow * kRowFloats + c8 * 8);
       const f32x4 hi  = *reinterpret_cast<const f32x4*>(stage + lrow * kRowFloats + c8 * 8 + 4);
       const vec8& rq  = res[pass & 1][e];
-      vec8 out;
+      float v[8];
 #pragma unroll
       for (int q = 0; q < 8; ++q) {
-        float v = __builtin_fmaf(epi.residual_scale, (float)rq[q], q < 4 ? lo[q] : hi[q - 4]);
-        asm volatile("" : "+v"(v));
-        if (epi.relu) v = v > 0.0f ? v : 0.0f;
-        out[q] = (T)v;
+        v[q] = __builtin_fmaf(epi.residual_scale, (float)rq[q], q < 4 ? lo[q] : hi[q - 4]);
+        // the relu as a max under a select on the flag: no compare per value
+        const float m = __builtin_fmaxf(v[q], 0.0f);
+        v[q]          = epi.relu ? m : v[q];
+        asm volatile("" : "+v"(v[q]));
       }
+      const u32x4 out = {PackPair<T>(v[0], v[1]), PackPair<T>(v[2], v[3]), PackPair<T>(v[4], v[5]), PackPair<T>(v[6], v[7])};
       if (epi.streaming) {
-        __builtin_nontemporal_store(out, reinterpret_cast<vec8*>(Ct + o));
+        __builtin_nontemporal_store(out, reinterpret_cast<u32x4*>(Ct + o));
       } else {
-        *reinterpret_cast<vec8*>(Ct + o) = out;
+        *reinterpret_cast<u32x4*>(Ct + o) = out;
       }
     }
   }

@@ -14,6 +14,15 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
+// two fp32 values rounded to nearest even into one dword of two T (v_cvt_pk_f16_f32 / v_cvt_pk_bf16_f32)
+template <typename T>
+__device__ __forceinline__ uint32_t PackPair(float a, float b) {
+  typedef T pair_t __attribute__((ext_vector_type(2)));
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  const f32x2 f = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, pair_t));
+}
+
 template <typename T>
 struct Mfma16;
 template <>
