@@ -743,3 +743,46 @@ def test_image_convolution_7x7_with_folded_epilogue_and_max_pooling(gpu, dtype, 
     tol = 1e-2 if dtype == "float16" else 2e-2
     # relative to the value or, where the convolution's terms cancel, to a twentieth of the activations' unit scale
     assert np.all(np.abs(fused.astype(np.float64) - want) <= tol * np.maximum(np.abs(want), 0.05))
+
+
+@pytest.mark.parametrize("dtype", ["float16", "float32"])
+@pytest.mark.parametrize("shape", [(2, 64, 56, 56, 64, 3, 1),     # LDS-resident patch kernel
+                                   (2, 128, 28, 28, 128, 3, 1),   # the same by chunks of 64 channels
+                                   (4, 256, 14, 14, 512, 1, 0),   # direct-to-LDS GEMM tiles
+                                   (32, 64, 56, 56, 256, 1, 0)])  # streaming short-K kernel
+def test_fused_relu_of_nan_and_infinite_sums(gpu, shape, dtype):
+    """relu is max(x, 0) with the C ternary's result for a NaN (cinn/hlir/pe/nn.cc:61-64: relu(NaN) = 0), and without a
+    relu a NaN or an infinite sum reaches the output as it is.  One input pixel is NaN, one +inf, one -inf (different
+    images / corners, so that no sum sees two of them): outputs whose window holds the NaN are 0 with the relu and NaN
+    without; +inf times a weight is +-inf and stays, or becomes 0 under the relu where it is -inf."""
+    n, c, h, w_, oc, k, pad = shape
+    rng = np.random.default_rng(77)
+    np_t = np.float16 if dtype == "float16" else np.float32
+    x = rng.standard_normal((n, c, h, w_)).astype(np_t)
+    w = (rng.standard_normal((oc, c, k, k)) * np.sqrt(2.0 / (c * k * k))).astype(np_t)
+    x[0, 3, 5, 5] = np.nan
+    x[1, 7, 2, h - 3] = np.inf
+    x[1, 9, h - 2, 1] = -np.inf
+    stats = [np.ones(oc, np.float32), np.zeros(oc, np.float32), np.zeros(oc, np.float32), np.ones(oc, np.float32)]
+    for relu in (True, False):
+        b = NetBuilder("nanrelu")
+        X = b.create_input(Float(16 if dtype == "float16" else 32), x.shape, "x")
+        W = b.create_input(Float(16 if dtype == "float16" else 32), w.shape, "w")
+        P = [b.create_input(Float(32), [oc], nm) for nm in ("scale", "bias", "mean", "var")]
+        y = b.batchnorm(b.conv2d(X, W, strides=[1, 1], paddings=[pad, pad]), *P)[0]
+        if relu:
+            y = b.relu(y)
+        feeds = {X: x, W: w}
+        feeds.update(dict(zip(P, stats)))
+        (got,), comp = run(b, feeds, [y], fuse_conv_bn_relu=True)
+        assert comp.fusion_groups().count("hip_conv2d_bn_relu") == 1
+        conv = oracle.conv2d_nchw(x.astype(np.float32), w.astype(np.float32), (1, 1), (pad, pad))
+        want = oracle.batch_norm_relu_nchw(conv, *stats, 1e-5, relu=relu)
+        got = got.astype(np.float32)
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        assert np.array_equal(np.isposinf(got), np.isposinf(want)) and np.array_equal(np.isneginf(got), np.isneginf(want))
+        finite = np.isfinite(want)
+        np.testing.assert_allclose(got[finite], want[finite], rtol=2e-2 if dtype == "float16" else 1e-4,
+                                   atol=2e-2 if dtype == "float16" else 1e-4)
+        if relu:
+            assert not np.isnan(got).any() and np.isnan(conv).any()
