@@ -26,6 +26,9 @@ class CinnComputation {
     // differs from the unfused operation order by rounding only; switch it off to get that order exactly.
     bool fuse_conv_bn_relu{true};
     bool fuse_stem_pool{true};  // fold the max pooling after an image convolution into it
+    // `matmul(x, W) + bias` with a const 2-D W and a const bias in a 16-bit type: the bias is added in the product's
+    // epilogue (frontend/layout_pass.h); the result differs from the two operators by one rounding
+    bool fuse_matmul_bias{true};
     // move conv2d chains written in NCHW to channels-last tensors, the layout the MFMA convolution kernels read
     // with 16-byte accesses (frontend/layout_pass.h); off: every conv2d runs in the layout it was written in
     bool conv_layout_nhwc{true};

@@ -363,5 +363,98 @@ Program FuseConvBatchNorm(const Program& program, const std::set<std::string>& f
   return Program(std::move(out), program.GetInputs(), program.name());
 }
 
+Program FuseMatmulBias(const Program& program, const std::set<std::string>& fetch_ids) {
+  const auto& instrs = program.instructions();
+  std::map<std::string, std::vector<size_t>> users;
+  for (size_t i = 0; i < instrs.size(); ++i)
+    for (auto& in : instrs[i]->inputs) users[in->id].push_back(i);
+  // values known before the first run: const inputs and what is computed from them alone
+  std::set<std::string> known;
+  for (auto& v : program.GetInputs())
+    if (v->is_const) known.insert(v->id);
+  std::map<std::string, size_t> defined_at;
+  for (size_t i = 0; i < instrs.size(); ++i) {
+    bool all = true;
+    for (auto& in : instrs[i]->inputs) all = all && (in->is_const || known.count(in->id));
+    for (auto& o : instrs[i]->outputs) {
+      defined_at[o->id] = i;
+      if (all) known.insert(o->id);
+    }
+  }
+  std::vector<bool> dropped(instrs.size(), false);
+  std::map<size_t, std::vector<Instruction>> replacement;
+  int serial = 0;
+  for (size_t i = 0; i < instrs.size(); ++i) {
+    auto& mm = instrs[i];
+    if (mm->op_type != "matmul" || mm->inputs.size() != 2 || mm->outputs.size() != 1) continue;
+    const Variable &x = mm->inputs[0], &w = mm->inputs[1], &prod = mm->outputs[0];
+    if (x->shape.size() != 2 || w->shape.size() != 2 || prod->shape.size() != 2) continue;
+    if (GetAttr<bool>(mm->attrs, "trans_a", false) || !GetAttr<bool>(mm->attrs, "trans_b", false) ||
+        GetAttr<float>(mm->attrs, "alpha", 1.0f) != 1.0f)
+      continue;
+    if (!(x->type.is_float16() || x->type.is_bfloat16()) || !(w->type == x->type)) continue;
+    const int m = x->shape[0], k = x->shape[1], n = w->shape[0];
+    if (w->shape[1] != k || prod->shape != ShapeType{m, n}) continue;
+    if (fetch_ids.count(prod->id)) continue;
+    auto u = users.find(prod->id);
+    if (u == users.end() || u->second.size() != 1) continue;
+    const size_t add_at = u->second[0];
+    auto& add           = instrs[add_at];
+    if (add->op_type != "elementwise_add" || add->inputs.size() != 2 || dropped[add_at]) continue;
+    Variable bias  = add->inputs[0] == prod ? add->inputs[1] : add->inputs[0];
+    const int axis = GetAttr<int>(add->attrs, "axis", -1);
+    if (bias == prod) continue;
+    // the builder's addition broadcasts the bias to [M][N] first (broadcast_to over axis 1)
+    int bcast_at = -1;
+    auto bdef    = defined_at.find(bias->id);
+    if (bias->shape == ShapeType{m, n} && bdef != defined_at.end() && instrs[bdef->second]->op_type == "broadcast_to") {
+      auto& bc  = instrs[bdef->second];
+      auto axes = GetAttr<std::vector<int>>(bc->attrs, "broadcast_axes", {});
+      auto bu   = users.find(bias->id);
+      if (bc->inputs.size() != 1 || axes.size() != 1 || (axes[0] != 1 && axes[0] != -1) || fetch_ids.count(bias->id) ||
+          bu == users.end() || bu->second.size() != 1 || dropped[bdef->second])
+        continue;
+      bcast_at = static_cast<int>(bdef->second);
+      bias     = bc->inputs[0];
+    } else if (axis != -1 && axis != 1) {
+      continue;
+    }
+    if (bias->shape != ShapeType{n}) continue;
+    if (!(bias->is_const || known.count(bias->id))) continue;
+    auto def = defined_at.find(bias->id);
+    if (def != defined_at.end() && def->second > i) continue;
+    if (add->outputs[0]->shape != ShapeType{m, n} || !(add->outputs[0]->type == x->type)) continue;
+
+    std::vector<Instruction> seq;
+    Emitter e(&seq, "mmb" + std::to_string(serial++) + "_");
+    auto x4   = e.Emit1("reshape", {x}, {{"shape", ShapeType{m, 1, 1, k}}});
+    auto w4   = e.Emit1("reshape", {w}, {{"shape", ShapeType{n, 1, 1, k}}});
+    auto ones = e.Emit1("fill_constant", {},
+                        {{"shape", ShapeType{n}}, {"value", 1.0}, {"dtype", std::string("float32")}, {"force_cpu", false}});
+    auto shift = bias->type == common::Float(32) ? bias : e.Emit1("cast", {bias}, {{"dtype", std::string("float32")}});
+    AttributeMap attrs = {{"stride", std::vector<int>{1, 1}},   {"padding", std::vector<int>{0, 0}},
+                          {"dilation", std::vector<int>{1, 1}}, {"groups", 1},
+                          {"data_format", std::string("NHWC")}, {"relu", false},
+                          {"max_pool", false}};
+    auto y4 = e.Emit1("hip_conv2d_bn_relu", {x4, w4, ones, shift}, attrs);
+    e.EmitInto(add->outputs[0], "reshape", {y4}, {{"shape", ShapeType{m, n}}});
+    dropped[i]      = true;
+    dropped[add_at] = true;
+    if (bcast_at >= 0) dropped[bcast_at] = true;
+    replacement[add_at] = seq;
+  }
+  if (replacement.empty()) return program;
+  std::vector<Instruction> out;
+  for (size_t i = 0; i < instrs.size(); ++i) {
+    auto it = replacement.find(i);
+    if (it != replacement.end()) {
+      out.insert(out.end(), it->second.begin(), it->second.end());
+    } else if (!dropped[i]) {
+      out.push_back(instrs[i]);
+    }
+  }
+  return Program(std::move(out), program.GetInputs(), program.name());
+}
+
 }  // namespace frontend
 }  // namespace cinn

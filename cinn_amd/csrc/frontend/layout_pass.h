@@ -29,6 +29,11 @@ Program FuseConvBatchNorm(const Program& program, const std::set<std::string>& f
 // matmul(x, W) with a const 2-D W stored [K][N]: multiply by a pre-run transposed copy instead (trans_b), so that
 // both operands of the GEMM kernel have K contiguous whatever the sizes of x
 Program PretransposeConstMatmulWeights(const Program& program);
+// matmul(x [M][K], W stored [N][K]) + bias [N] in a 16-bit type, the bias known before the first run: one
+// hip_conv2d_bn_relu call on the operands seen as 1x1 images (x as [M,1,1,K], W as [N,1,1,K]) with scale 1 and the
+// bias in fp32 as shift - a classifier's bias then costs no kernel of its own.  The sum is rounded once, from the
+// fp32 accumulator plus bias, where the two operators round the product first.
+Program FuseMatmulBias(const Program& program, const std::set<std::string>& fetch_ids);
 
 }  // namespace frontend
 }  // namespace cinn

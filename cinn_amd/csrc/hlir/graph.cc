@@ -108,8 +108,10 @@ void Graph::ConstPropagate() {
     Node* n = np.get();
     if (n->op_type() != "fill_constant" || n->outputs[0]->consumers.empty()) continue;
     // with consumers on both sides it is computed once up front and read from memory by the others
+    // a library call cannot fold a literal into its kernel: what it reads is filled once as well
     bool any_pre_run = false;
-    for (Node* c : n->outputs[0]->consumers) any_pre_run = any_pre_run || c->pre_run;
+    for (Node* c : n->outputs[0]->consumers)
+      any_pre_run = any_pre_run || c->pre_run || c->op->pattern == OpPatternKind::kNonFusible;
     n->pre_run = any_pre_run;
   }
 }

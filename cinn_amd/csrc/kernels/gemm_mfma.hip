@@ -2056,7 +2056,11 @@ bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream) {
     // few tiles but a long reduction: the single-wavefront 64x64 tiles of the GEMM kernel (see TryDma16)
     const bool long_k = forced_tile == 64 || (forced_tile == 0 && a.oc % 64 == 0 &&
                                               (a.c >= 2048 || (a.c >= 1024 && ((pixels + 127) / 128) * ((a.oc + 127) / 128) < 128)));
-    if (mode != 2 && !shortk && !long_k && (a.c < 128 || (!narrow && ((pixels + 127) / 128) * ((a.oc + 127) / 128) < 192))) return false;
+    // at most 64 pixels (a matmul with few rows written as a 1x1 layer, its bias as the shift): gemm16_skinny_kernel
+    const bool few_rows = forced_tile == 0 && pixels <= 64 && a.c % 256 == 0;
+    if (mode != 2 && !shortk && !long_k && !few_rows &&
+        (a.c < 128 || (!narrow && ((pixels + 127) / 128) * ((a.oc + 127) / 128) < 192)))
+      return false;
     p.k = a.c;
   } else {
     // any filter, stride, padding, dilation: implicit GEMM, K = kh * kw * c with 64-channel steps inside a tap

@@ -423,3 +423,37 @@ def test_batch_norm_training_form_and_gradient_decompose_into_primitives():
     comp = compile_only(b, outs + grads)
     names = [comp.instruction_info(i)[0] for i in range(comp.num_instructions())]
     assert not any("batch_norm" in n for n in names) and any("reduce" in n for n in names)
+
+
+def _classifier(dtype, m=32, k=512, n=1000, const_bias=True, const_w=True):
+    b = NetBuilder("fc")
+    x = b.create_input(dtype, [m, k], "x")
+    w = b.create_input(dtype, [k, n], "w")
+    c = b.create_input(dtype, [n], "c")
+    if const_w:
+        w.set_const()
+    if const_bias:
+        c.set_const()
+    return b, b.add(b.matmul(x, w), c)
+
+
+def test_bias_after_a_matmul_with_const_weights_is_folded_into_the_product():
+    """matmul(x, W) + bias, W and bias const and 16-bit: one library call at run time (the bias is the shift of the
+    product's epilogue, hip_conv2d_bn_relu on 1x1 images) and no element-wise kernel; the transposed weight, the fp32
+    bias and the scale of ones are computed before the first run.  fp32, a bias that is not const, a weight that is
+    not const (stays [K][N]) and the option fuse_matmul_bias=0 keep the two operators."""
+    from cinn_amd.common import Float
+    b, y = _classifier(Float(16))
+    comp = compile_only(b, [y])
+    groups = [g for g in comp.fusion_groups().splitlines() if g.strip()]
+    # what is left at run time: the call, and two reshapes that are views (no instruction)
+    run = [g for g in groups if " pre_run " not in g and "{ reshape }" not in g]
+    assert len(run) == 1 and "hip_conv2d_bn_relu" in run[0], groups
+    names = [comp.instruction_info(i)[0] for i in range(comp.num_instructions())]
+    assert sum("reshape" in n or "elementwise_add" in n for n in names) == 0, names
+    assert comp.get_tensor(str(y)).shape() == [32, 1000]
+    for dtype, kwargs, opts in ((Float(16), {}, {"fuse_matmul_bias": 0}), (Float(32), {}, {}),
+                                (Float(16), {"const_bias": False}, {}), (Float(16), {"const_w": False}, {})):
+        b, y = _classifier(dtype, **kwargs)
+        text = compile_only(b, [y], **opts).fusion_groups()
+        assert "hip_conv2d_bn_relu" not in text and "matmul" in text, (kwargs, opts, text)

@@ -324,3 +324,40 @@ def test_matmul_fused_with_neighbours(gpu):
     (y,), comp = run(b, {X: x, W: w, Bi: bias}, [out])
     np.testing.assert_allclose(y, np.maximum(x.astype(np.float64) @ w + bias, 0), rtol=1e-4, atol=1e-4)
     assert comp.num_instructions() == 2
+
+
+@pytest.mark.parametrize("kind", ["float16", "bfloat16"])
+@pytest.mark.parametrize("m,n,k", [(32, 1000, 2048), (8, 24, 256), (33, 1000, 512), (64, 4096, 1024), (128, 512, 256),
+                                   (300, 1000, 320)])
+def test_bias_folded_into_the_product_of_a_const_weight(gpu, kind, m, n, k):
+    """matmul(x, W) + bias with const 16-bit W and bias runs as one call (bias = shift of the epilogue, one rounding);
+    against float64 and against the two separate operators (fuse_matmul_bias=0), which round the product first."""
+    from cinn_amd.common import float32_to_bfloat16_bits
+    rng = np.random.default_rng(m * 7 + n + k)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    w = (rng.standard_normal((k, n)) / np.sqrt(k)).astype(np.float32)
+    c = rng.uniform(-1, 1, n).astype(np.float32)
+    if kind == "float16":
+        ty, enc, dec = Float(16), (lambda a: a.astype(np.float16)), (lambda a: a.astype(np.float64))
+    else:
+        ty, enc, dec = BFloat16(), float32_to_bfloat16_bits, (lambda a: bfloat16_bits_to_float32(a).astype(np.float64))
+    xq, wq, cq = enc(x), enc(w), enc(c)
+    want = dec(xq) @ dec(wq) + dec(cq)
+
+    def build(**options):
+        b = NetBuilder("fc")
+        X = b.create_input(ty, [m, k], "x")
+        W = b.create_input(ty, [k, n], "w").set_const()
+        C = b.create_input(ty, [n], "c").set_const()
+        (got,), comp = run(b, {X: xq, W: wq, C: cq}, [b.add(b.matmul(X, W), C)], **options)
+        return dec(got), comp
+
+    fused, comp = build()
+    assert comp.num_instructions() == 1 and "hip_conv2d_bn_relu" in comp.instruction_info(0)[0], comp.fusion_groups()
+    apart, comp2 = build(fuse_matmul_bias=0)
+    assert comp2.num_instructions() == 2
+    eps = 2.0 ** -10 if kind == "float16" else 2.0 ** -7
+    scale = np.abs(dec(xq)) @ np.abs(dec(wq)) + np.abs(dec(cq))
+    assert np.all(np.abs(fused - want) <= eps * np.abs(want) + 1e-5 * scale), np.abs(fused - want).max()
+    # the separate operators add one rounding of the product
+    assert np.all(np.abs(fused - apart) <= 2 * eps * (np.abs(want) + np.abs(dec(cq))) + 1e-5 * scale)
