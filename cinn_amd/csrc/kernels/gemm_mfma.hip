@@ -1695,12 +1695,13 @@ bool TrySkinny(const GemmProblem& p, hipStream_t stream) {
   epi.streaming       = 0;
   int mt = (p.m + 15) / 16;
   dim3 grid((unsigned)((p.n + 15) / 16));
-  // One block per 16 rows as well: a block's traffic is its 16 columns of B plus the rows of A it multiplies, and with
-  // all of A (128 KB at 32 x 2048, against 64 KB of B) the few CUs at work are bound by what one CU can pull in.  Row
-  // blocks read B again, out of L2.  ResNet-50's classifier, 32 x 2048 -> 1000: 126 blocks instead of 63, 2.2 us less.
-  // FLAGS_cinn_hip_gemm_skinny_rows=0: one block for all rows (row tiles in registers).
-  static const bool by_rows = !(getenv("FLAGS_cinn_hip_gemm_skinny_rows") && atoi(getenv("FLAGS_cinn_hip_gemm_skinny_rows")) == 0);
-  if (by_rows) grid.y = mt, mt = 1;
+  // Fewer column blocks than CUs: one block per 16 rows as well.  A block's traffic is its 16 columns of B plus the
+  // rows of A it multiplies, and with all of A (128 KB at 32 x 2048, against 64 KB of B) the few CUs at work are bound
+  // by what one CU can pull in; row blocks read B again, out of L2.  ResNet-50's classifier, 32 x 2048 -> 1000: 126
+  // blocks instead of 63, 2.2 us less.  With the chip full, the row tiles stay in one block's registers (B read once).
+  // FLAGS_cinn_hip_gemm_skinny_rows: 0 never splits the rows, 2 always.
+  static const int rows_flag = getenv("FLAGS_cinn_hip_gemm_skinny_rows") ? atoi(getenv("FLAGS_cinn_hip_gemm_skinny_rows")) : 1;
+  if (rows_flag == 2 || (rows_flag == 1 && grid.x < 256)) grid.y = mt, mt = 1;
 #define CINN_SKINNY(MT)                                                                                        \
   hipLaunchKernelGGL((gemm16_skinny_kernel<T, MT>), grid, dim3(512), 0, stream, static_cast<const uint16_t*>(p.a), \
                      static_cast<const uint16_t*>(p.b), static_cast<uint16_t*>(p.c), p.m, p.n, p.k, epi)

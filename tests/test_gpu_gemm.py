@@ -152,10 +152,12 @@ def test_16bit_direct_to_lds_kernel(gpu, kind, tb, alpha, beta, batch, m, n, k):
                                    (17, 8, 512),       # ragged rows, a single block of 8 columns
                                    (48, 24, 768),      # three row tiles
                                    (5, 3, 8192),       # long K: both register sets of every wavefront in use; 3 columns
-                                   (33, 136, 4352)])   # 17 k blocks per wavefront: a set that is only partly multiplied
+                                   (33, 136, 4352),    # 17 k blocks per wavefront: a set that is only partly multiplied
+                                   (40, 4112, 256),    # 257 column blocks: the three row tiles stay in one block
+                                   (64, 4096, 512)])   # 256 column blocks, four row tiles per block
 def test_16bit_products_with_few_rows(gpu, kind, alpha, beta, m, n, k):
-    """gemm16_skinny_kernel: at most 64 rows, B stored [N][K], K a multiple of 256 - one block per 16 columns, K split
-    over its wavefronts, fragments straight from global memory.  Same bar as the tiled kernels: fp32 accumulation and
+    """gemm16_skinny_kernel: at most 64 rows, B stored [N][K], K a multiple of 256 - one block per 16 columns (and, below 256
+    such blocks, per 16 rows), K split over its wavefronts, fragments straight from global memory.  Same bar as the tiled kernels: fp32 accumulation and
     epilogue, one rounding to the 16-bit type."""
     rng = np.random.default_rng(m * 7 + n + k)
     a = (rng.standard_normal((m, k)) * 0.05).astype(np.float32)
