@@ -269,6 +269,33 @@ def test_residual_that_is_also_the_convolution_input(gpu, fuse):
         assert comp.fusion_groups().count("hip_conv2d_bn_relu") == 2
 
 
+@pytest.mark.parametrize("n,hw", [(1, 7), (4, 4), (2, 5)])
+def test_pointwise_layer_of_at_most_64_pixels_with_residual_and_relu(gpu, n, hw):
+    """1x1 convolution over 512 channels of a 16-bit image of at most 64 pixels, folded batch norm, residual and relu:
+    such a layer runs on the GEMM kernel for products with few rows (every epilogue term in use, ragged row tiles)."""
+    rng = np.random.default_rng(61 + n)
+    c = 512
+    x = rng.standard_normal((n, c, hw, hw)).astype(np.float16)
+    w = (rng.standard_normal((c, c, 1, 1)) / np.sqrt(c)).astype(np.float16)
+    stats = [rng.uniform(0.5, 1.5, c).astype(np.float16), rng.uniform(-0.5, 0.5, c).astype(np.float16),
+             (rng.standard_normal(c) * 0.1).astype(np.float16), rng.uniform(0.5, 1.5, c).astype(np.float16)]
+    b = NetBuilder("few")
+    X = b.create_input(Float(16), x.shape, "x")
+    W = b.create_input(Float(16), w.shape, "w").set_const()
+    P = [b.create_input(Float(16), [c], nm).set_const() for nm in ("scale", "bias", "mean", "var")]
+    y = b.relu(b.add(b.batchnorm(b.conv2d(X, W), *P)[0], X))
+    feeds = {X: x, W: w}
+    feeds.update(dict(zip(P, stats)))
+    (got,), comp = run(b, feeds, [y])
+    assert comp.fusion_groups().count("hip_conv2d_bn_relu") == 1
+    f32 = [a.astype(np.float32) for a in stats]
+    z = oracle.batch_norm_relu_nchw(oracle.conv2d_nchw(x.astype(np.float32), w.astype(np.float32), (1, 1), (0, 0)), *f32,
+                                    1e-5, relu=False)
+    want = np.maximum(z.astype(np.float64) + x.astype(np.float64), 0)
+    np.testing.assert_allclose(got.astype(np.float64), want, rtol=1e-2, atol=1e-2)
+    assert (got == 0).any() and (got > 0).any()
+
+
 def test_matmul_of_a_matrix_with_itself(gpu):
     rng = np.random.default_rng(22)
     a = rng.standard_normal((48, 48)).astype(np.float32)
