@@ -157,19 +157,68 @@ void ThunkDispatch(void* args, int32_t num_args, void* stream, HostStubPool::Clo
   (*closure)(args, num_args, stream);
 }
 
-// movabs rcx, <closure>; movabs rax, <ThunkDispatch>; jmp rax  - the stub's own three arguments stay in rdi, esi, rdx
-constexpr size_t kThunkBytes = 32;
-constexpr size_t kThunkPage  = 1 << 16;
+// A thunk is position-independent code that never changes once written:
+//   mov rcx, [rip + d0]   ; its closure, from the thunk's slot in a data region that follows the code region
+//   mov rax, [rip + d1]   ; &ThunkDispatch, same slot
+//   jmp rax               ; the stub's own three arguments stay in rdi, esi, rdx
+// A region's code is generated in full while it is mapped read + write, then made read + execute for good; only the
+// data slots (never executable) are written afterwards.  No page is ever writable and executable at once, and no
+// page's protection changes while a stub on it may be running.
+constexpr size_t kThunkBytes  = 32;
+constexpr size_t kThunkRegion = 1 << 16;                       // code bytes per region, and data bytes after them
+constexpr size_t kThunksPerRegion = kThunkRegion / kThunkBytes;
+struct ThunkSlot {
+  HostStubPool::Closure* closure;
+  void (*dispatch)(void*, int32_t, void*, HostStubPool::Closure*);
+};
+static_assert(sizeof(ThunkSlot) * kThunksPerRegion <= kThunkRegion, "the data region holds one slot per thunk");
 
 struct ThunkState {
-  std::vector<unsigned char*> pages;
-  size_t used_in_last{kThunkPage};
+  std::vector<unsigned char*> regions;
+  size_t used_in_last{kThunksPerRegion};
   std::vector<unsigned char*> free_list;
   std::map<lower_func_ptr_g, HostStubPool::Closure*> live;
 };
 ThunkState& Thunks() {
   static ThunkState* s = new ThunkState;  // leaked like the pool: stubs may run during static teardown
   return *s;
+}
+
+ThunkSlot* SlotOf(unsigned char* code) {
+  const uintptr_t addr   = reinterpret_cast<uintptr_t>(code);
+  const uintptr_t region = addr & ~static_cast<uintptr_t>(kThunkRegion - 1);  // regions are aligned to their size
+  return reinterpret_cast<ThunkSlot*>(region + kThunkRegion) + (addr - region) / kThunkBytes;
+}
+
+// a new region with all its thunks written; null when the system refuses the mapping or the protection change
+unsigned char* NewThunkRegion() {
+  // twice the span, so that an aligned code + data pair lies inside whatever address comes back
+  const size_t span = 4 * kThunkRegion;
+  void* raw = mmap(nullptr, span, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS, -1, 0);
+  if (raw == MAP_FAILED) return nullptr;
+  const uintptr_t base = (reinterpret_cast<uintptr_t>(raw) + kThunkRegion - 1) & ~static_cast<uintptr_t>(kThunkRegion - 1);
+  auto* code = reinterpret_cast<unsigned char*>(base);
+  // give back what lies before and behind the pair
+  if (base > reinterpret_cast<uintptr_t>(raw)) munmap(raw, base - reinterpret_cast<uintptr_t>(raw));
+  const uintptr_t end = reinterpret_cast<uintptr_t>(raw) + span;
+  if (end > base + 2 * kThunkRegion) munmap(reinterpret_cast<void*>(base + 2 * kThunkRegion), end - (base + 2 * kThunkRegion));
+  for (size_t i = 0; i < kThunksPerRegion; ++i) {
+    unsigned char* t   = code + i * kThunkBytes;
+    const uintptr_t slot = base + kThunkRegion + i * sizeof(ThunkSlot);
+    const int32_t d0 = static_cast<int32_t>(slot - (reinterpret_cast<uintptr_t>(t) + 7));
+    const int32_t d1 = static_cast<int32_t>(slot + 8 - (reinterpret_cast<uintptr_t>(t) + 14));
+    unsigned char bytes[16] = {0x48, 0x8B, 0x0D, 0, 0, 0, 0, 0x48, 0x8B, 0x05, 0, 0, 0, 0, 0xFF, 0xE0};
+    std::memcpy(bytes + 3, &d0, 4);
+    std::memcpy(bytes + 10, &d1, 4);
+    std::memcpy(t, bytes, sizeof(bytes));
+    std::memset(t + sizeof(bytes), 0xCC, kThunkBytes - sizeof(bytes));  // int3 padding
+  }
+  if (mprotect(code, kThunkRegion, PROT_READ | PROT_EXEC) != 0) {
+    munmap(code, 2 * kThunkRegion);
+    return nullptr;
+  }
+  __builtin___clear_cache(reinterpret_cast<char*>(code), reinterpret_cast<char*>(code) + kThunkRegion);
+  return code;
 }
 
 // caller holds the pool's mutex; null when the system does not hand out executable memory
@@ -180,23 +229,19 @@ lower_func_ptr_g NewThunk(HostStubPool::Closure closure) {
     code = t.free_list.back();
     t.free_list.pop_back();
   } else {
-    if (t.used_in_last + kThunkBytes > kThunkPage) {
-      void* page = mmap(nullptr, kThunkPage, PROT_READ | PROT_WRITE | PROT_EXEC, MAP_PRIVATE | MAP_ANONYMOUS, -1, 0);
-      if (page == MAP_FAILED) return nullptr;
-      t.pages.push_back(static_cast<unsigned char*>(page));
+    if (t.used_in_last >= kThunksPerRegion) {
+      unsigned char* region = NewThunkRegion();
+      if (!region) return nullptr;
+      t.regions.push_back(region);
       t.used_in_last = 0;
     }
-    code = t.pages.back() + t.used_in_last;
-    t.used_in_last += kThunkBytes;
+    code = t.regions.back() + t.used_in_last * kThunkBytes;
+    ++t.used_in_last;
   }
-  auto* owned            = new HostStubPool::Closure(std::move(closure));
-  const uint64_t ctx     = reinterpret_cast<uint64_t>(owned);
-  const uint64_t target  = reinterpret_cast<uint64_t>(&ThunkDispatch);
-  unsigned char bytes[22] = {0x48, 0xB9, 0, 0, 0, 0, 0, 0, 0, 0, 0x48, 0xB8, 0, 0, 0, 0, 0, 0, 0, 0, 0xFF, 0xE0};
-  std::memcpy(bytes + 2, &ctx, 8);
-  std::memcpy(bytes + 12, &target, 8);
-  std::memcpy(code, bytes, sizeof(bytes));
-  __builtin___clear_cache(reinterpret_cast<char*>(code), reinterpret_cast<char*>(code) + sizeof(bytes));
+  auto* owned     = new HostStubPool::Closure(std::move(closure));
+  ThunkSlot* slot = SlotOf(code);
+  slot->closure   = owned;
+  slot->dispatch  = &ThunkDispatch;
   auto fn    = reinterpret_cast<lower_func_ptr_g>(code);
   t.live[fn] = owned;
   return fn;

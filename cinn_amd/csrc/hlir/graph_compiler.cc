@@ -216,7 +216,10 @@ Program::~Program() {
     if (e) (void)hipEventDestroy(static_cast<hipEvent_t>(e));
   if (fork_event_) (void)hipEventDestroy(static_cast<hipEvent_t>(fork_event_));
   if (join_event_) (void)hipEventDestroy(static_cast<hipEvent_t>(join_event_));
-  if (side_stream_) (void)hipStreamDestroy(static_cast<hipStream_t>(side_stream_));
+  if (side_stream_) {
+    (void)cinn_hip_scratch_release_stream(side_stream_);  // the library's per-stream scratch does not outlive the stream
+    (void)hipStreamDestroy(static_cast<hipStream_t>(side_stream_));
+  }
 }
 
 // Two stream lanes for a graph replay.  Instruction i depends on an earlier one that wrote what i reads or writes, or

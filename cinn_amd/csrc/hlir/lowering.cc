@@ -1491,6 +1491,15 @@ ir::LoweredFuncRef OpLowerer::LowerLibraryCall(const Group& group) const {
     int64_t outer = 1, inner = 1;
     for (int d = 0; d < axis; ++d) outer *= x[d];
     for (size_t d = axis + 1; d < x.size(); ++d) inner *= x[d];
+    {
+      // cinn_call_hip_argsort keeps a whole row of keys (and, for rows with a NaN, positions) in one block's LDS:
+      // 128 KiB / (key bytes + 4).  Longer rows are refused here, when the program is compiled, not at its first run.
+      const int key_bytes   = n->inputs[0]->dtype.bytes() > 4 ? 8 : 4;
+      const int64_t longest = (128 * 1024) / (key_bytes + 4);
+      CINN_CHECK(((static_cast<int64_t>(x[axis]) + 3) & ~int64_t(3)) <= longest)
+          << op << ": " << x[axis] << " elements along the sorted axis; the GPU kernel sorts rows of at most " << longest
+          << " elements of this type (one block's LDS)";
+    }
     push_ints({static_cast<int>(outer), x[axis], static_cast<int>(inner), GetAttr<bool>(n->attrs, "is_ascend", true) ? 1 : 0,
                op == "argsort" ? 3 : 4});
   } else {

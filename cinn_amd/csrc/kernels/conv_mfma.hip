@@ -5,9 +5,10 @@
 //
 // GEMM view per group: M = output channels, N = n * oh * ow output pixels (flattened over the batch so that
 // small images still fill a tile), K = (c / groups) * kh * kw.  The weight matrix is [M][K] as stored.  The
-// im2col matrix is never materialised: every thread owns one output pixel of the tile, and a small
-// per-shape table (one entry per k: input offset, dy, dx) replaces the div / mod of decoding k into
-// (c, ry, rx), so a gathered element costs one table read, two range checks and one load.
+// im2col matrix is never materialised: every thread owns one output pixel of the tile and decodes k into
+// (c, ry, rx) with two multiply-shift divisions by host-computed magic numbers, so a gathered element costs
+// a few integer instructions, two range checks and one load - and the entry point touches no device memory
+// beyond its operands (nothing to allocate or upload on the first call of a shape, safe under stream capture).
 //
 // Block tile 128 (channels) x 128 (pixels), 256 threads = 4 wavefronts in a 2x2 grid, each 64x64 = 2x2 MFMA
 // tiles of 32x32.
@@ -19,10 +20,6 @@
 
 #include <climits>
 #include <cstdint>
-#include <map>
-#include <mutex>
-#include <string>
-#include <vector>
 
 #include "cinn_hip_runtime.h"
 #include "kernels/conv_nhwc.h"
@@ -35,16 +32,14 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-struct KEntry {
-  int offset;   // c * ih * iw + ry * d * iw + rx * d, relative to the input position of the pixel
-  short dy, dx;  // ry * d, rx * d
-};
-
 struct ConvParams {
   int n, c, ih, iw;        // input
   int f, kh, kw;           // filter: f output channels, c / groups input channels each
   int oh, ow;              // output
-  int ph, pw, sh, sw;      // padding, stride (dilation lives in the table)
+  int ph, pw, sh, sw;      // padding, stride
+  int dh, dw;              // dilation
+  // exact division of 0 <= k < 2^31 by kh * kw and by kw: q = (k * magic) >> shift with a 64-bit product
+  unsigned magic_taps, shift_taps, magic_kw, shift_kw;
   int groups;
   int k_total;             // (c / groups) * kh * kw
   int pixels;              // n * oh * ow
@@ -88,8 +83,7 @@ __device__ __forceinline__ int HalfTileOffset(int row, int chunk) { return row *
 template <typename T>
 __global__ void __launch_bounds__(kThreads)
 conv2d_igemm_kernel(const T* __restrict__ in, const T* __restrict__ w, T* __restrict__ out,
-                    const KEntry* __restrict__ table, const float* __restrict__ scale, const float* __restrict__ shift,
-                    ConvParams p) {
+                    const float* __restrict__ scale, const float* __restrict__ shift, ConvParams p) {
   constexpr int BK = ConvTraits<T>::kStep;
   // fp32: A[BK][128 + 4] and B[BK][128 + 4] floats; 16-bit: A[128][32] and B[128][32] halves (8 KiB each)
   __shared__ __attribute__((aligned(16))) char lds_a[ConvTraits<T>::kHalf ? kTileM * 64 : BK * (kTileM + 4) * 4];
@@ -132,10 +126,13 @@ conv2d_igemm_kernel(const T* __restrict__ in, const T* __restrict__ w, T* __rest
 
   auto gather = [&](int k) -> T {
     if (!pix_ok || k >= K) return (T)0.0f;
-    KEntry e = table[k];
-    int iy = iy0 + e.dy, ix = ix0 + e.dx;
+    const int c   = (int)(((unsigned long long)(unsigned)k * p.magic_taps) >> p.shift_taps);
+    const int tap = k - c * (p.kh * p.kw);
+    const int ry  = (int)(((unsigned long long)(unsigned)tap * p.magic_kw) >> p.shift_kw);
+    const int dy = ry * p.dh, dx = (tap - ry * p.kw) * p.dw;
+    int iy = iy0 + dy, ix = ix0 + dx;
     if (iy < 0 || iy >= p.ih || ix < 0 || ix >= p.iw) return (T)0.0f;
-    return in_pix[e.offset];
+    return in_pix[(c * p.ih + dy) * p.iw + dx];
   };
 
   for (int k0 = 0; k0 < K; k0 += BK) {
@@ -244,31 +241,16 @@ conv2d_igemm_kernel(const T* __restrict__ in, const T* __restrict__ w, T* __rest
   }
 }
 
-// ---- per-shape k table, cached on the device ---------------------------------------------------------
-std::mutex g_table_mu;
-std::map<std::string, KEntry*> g_tables;
-
-const KEntry* GetTable(const ConvParams& p, int dh, int dw) {
-  char key[160];
-  snprintf(key, sizeof(key), "%d,%d,%d,%d,%d,%d,%d,%d", p.c / p.groups, p.ih, p.iw, p.kh, p.kw, dh, dw, p.k_total);
-  std::lock_guard<std::mutex> lock(g_table_mu);
-  auto it = g_tables.find(key);
-  if (it != g_tables.end()) return it->second;
-  std::vector<KEntry> host(p.k_total);
-  int k = 0;
-  for (int c = 0; c < p.c / p.groups; ++c)
-    for (int ry = 0; ry < p.kh; ++ry)
-      for (int rx = 0; rx < p.kw; ++rx) {
-        host[k].offset = (c * p.ih + ry * dh) * p.iw + rx * dw;
-        host[k].dy     = static_cast<short>(ry * dh);
-        host[k].dx     = static_cast<short>(rx * dw);
-        ++k;
-      }
-  KEntry* dev = nullptr;
-  CINN_HIP_CALL(hipMalloc(&dev, sizeof(KEntry) * host.size()));
-  CINN_HIP_CALL(hipMemcpy(dev, host.data(), sizeof(KEntry) * host.size(), hipMemcpyHostToDevice));
-  g_tables[key] = dev;
-  return dev;
+// q = (n * magic) >> shift == n / d for 0 <= n < 2^31 (Granlund-Montgomery with a 64-bit product)
+void MagicFor(int d, unsigned* magic, unsigned* shift) {
+  int l = 0;
+  while ((1ll << l) < d) ++l;
+  *shift = 31 + l;
+  *magic = (unsigned)(((1ull << *shift) / (unsigned)d) + 1);
+  if (d == 1) {  // 2^31 + 1 would round n = 2^31 - 1 up; d == 1 needs no rounding at all
+    *shift = 0;
+    *magic = 1;
+  }
 }
 
 // fp64 tensors (no matrix-core path is wired for them): one thread per output element, products added in
@@ -386,22 +368,24 @@ void RunConv(cinn_buffer_t* x, cinn_buffer_t* w, cinn_buffer_t* y, const float* 
   p.alpha    = alpha;
   p.beta     = beta;
   p.epilogue = epilogue;
-  const KEntry* table = GetTable(p, dh, dw);
+  p.dh = dh, p.dw = dw;
+  MagicFor(fh * fw, &p.magic_taps, &p.shift_taps);
+  MagicFor(fw, &p.magic_kw, &p.shift_kw);
 
   dim3 grid((p.pixels + kTileN - 1) / kTileN, (fn / groups + kTileM - 1) / kTileM, groups);
   CINN_RT_CHECK(grid.y <= 65535 && grid.z <= 65535, "conv2d: grid too large");
   const int bytes = x->type.bits / CHAR_BIT;
   if (x->type.code == cinn_type_float && bytes == 4) {
     hipLaunchKernelGGL(conv2d_igemm_kernel<float>, grid, dim3(kThreads), 0, stream, reinterpret_cast<const float*>(x->memory),
-                       reinterpret_cast<const float*>(w->memory), reinterpret_cast<float*>(y->memory), table, scale, shift, p);
+                       reinterpret_cast<const float*>(w->memory), reinterpret_cast<float*>(y->memory), scale, shift, p);
   } else if (x->type.code == cinn_type_float && bytes == 2) {
     hipLaunchKernelGGL(conv2d_igemm_kernel<_Float16>, grid, dim3(kThreads), 0, stream,
                        reinterpret_cast<const _Float16*>(x->memory), reinterpret_cast<const _Float16*>(w->memory),
-                       reinterpret_cast<_Float16*>(y->memory), table, scale, shift, p);
+                       reinterpret_cast<_Float16*>(y->memory), scale, shift, p);
   } else if (x->type.code == cinn_type_bfloat) {
     hipLaunchKernelGGL(conv2d_igemm_kernel<__bf16>, grid, dim3(kThreads), 0, stream,
                        reinterpret_cast<const __bf16*>(x->memory), reinterpret_cast<const __bf16*>(w->memory),
-                       reinterpret_cast<__bf16*>(y->memory), table, scale, shift, p);
+                       reinterpret_cast<__bf16*>(y->memory), scale, shift, p);
   } else {
     fprintf(stderr, "conv2d: unsupported data type code %d bits %d\n", x->type.code, x->type.bits);
     abort();

@@ -60,3 +60,9 @@ void RunConvStem(const ConvNhwcArgs& a, hipStream_t stream);
 bool TryConvStem7(const ConvNhwcArgs& a, hipStream_t stream);
 
 }  // namespace cinn_hip_kernels
+
+// Test hook, exported from the shared library but deliberately absent from the public header: the `s_waitcnt vmcnt`
+// count a feeding wavefront of conv3x3_patch_chunks_kernel uses before the barrier of K step (chunk, tap) - how many of
+// its loads may still be in flight while the next filter stage (and, at tap 7, the next chunk's patch) is known to have
+// landed.  Host-side evaluation of the kernel's own constexpr, pure (no state).
+extern "C" int cinn_hip_conv_patch_loads_in_flight(int tap, int first_chunk, int last_chunk, int patch_loads_per_step);

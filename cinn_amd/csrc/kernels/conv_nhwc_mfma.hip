@@ -20,6 +20,7 @@
 //     patch fit LDS (the network's first convolution) go to the staged kernel of conv_stem_mfma.hip instead.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <climits>
 #include <cstdint>
 #include <cstdio>
@@ -524,6 +525,7 @@ struct ScratchSource {
   float* fixed_partials{nullptr};   // null: the arena
   size_t fixed_partials_bytes{0};
   const void* zero_page{nullptr};   // null: the arena's page
+  bool status_only{false};          // failed runtime calls are reported and returned instead of aborting
 };
 
 // split count and K steps per split of one launch
@@ -536,16 +538,35 @@ void PlanSplits(Params* p, int bm, int bn, int elem_bytes) {
   p->splits          = (steps + p->steps_per_split - 1) / p->steps_per_split;
 }
 
+// Raises the dynamic LDS limit of one kernel instantiation, once per instantiation and process (a failed attempt is
+// tried again by the next call).  The runtime does not allow the call while a stream is being captured, which is why
+// cinn_hip_conv2d_forward_noalloc_init walks every instantiation ahead of time.
 template <typename T, int BM, int BN, int WM, int WN, bool NCHW_IN, int PF = 2>
-void Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream, const ScratchSource& src) {
+hipError_t Configure() {
+  static std::atomic<bool> done{false};
+  if (done.load(std::memory_order_acquire)) return hipSuccess;
+  const hipError_t status = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(conv_nhwc_mfma_kernel<T, BM, BN, WM, WN, NCHW_IN, PF>),
+      hipFuncAttributeMaxDynamicSharedMemorySize, LdsBytes(BM, BN, WM));
+  if (status == hipSuccess) done.store(true, std::memory_order_release);
+  return status;
+}
+
+// A failed runtime call: the allocating entry points abort with the message (the reference's CUDA_CALL), the entry
+// point that allocates nothing reports and returns a status.
+int LaunchFailed(const ScratchSource& src, hipError_t err, const char* what) {
+  if (!src.status_only) CINN_RT_CHECK(false, "conv2d (channels-last): %s: %s", what, hipGetErrorString(err));
+  fprintf(stderr, "cinn_call_hip_conv2d_forward_noalloc: %s: %s\n", what, hipGetErrorString(err));
+  return 1;
+}
+
+template <typename T, int BM, int BN, int WM, int WN, bool NCHW_IN, int PF = 2>
+int Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream, const ScratchSource& src) {
   // PF: K steps in flight per block
   auto kernel      = conv_nhwc_mfma_kernel<T, BM, BN, WM, WN, NCHW_IN, PF>;
   const int bytes  = LdsBytes(BM, BN, WM);
-  static const bool configured = [&] {  // once per instantiation, thread-safe
-    CINN_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
-    return true;
-  }();
-  (void)configured;
+  if (hipError_t err = Configure<T, BM, BN, WM, WN, NCHW_IN, PF>(); err != hipSuccess)
+    return LaunchFailed(src, err, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
   Params p = p_in;
   PlanSplits(&p, BM, BN, sizeof(T));
   const int tiles  = ((p.pixels + BM - 1) / BM) * ((p.oc + BN - 1) / BN);
@@ -554,7 +575,7 @@ void Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream, const
   if (p.splits > 1) {
     const size_t need = (size_t)p.splits * p.pixels * p.oc * sizeof(float);
     if (src.fixed_partials) {
-      CINN_RT_CHECK(need <= src.fixed_partials_bytes, "conv2d: %zu bytes of partial sums do not fit the fixed scratch", need);
+      if (need > src.fixed_partials_bytes) return LaunchFailed(src, hipErrorOutOfMemory, "partial sums do not fit the fixed scratch");
       workspace = src.fixed_partials;
     } else {
       workspace = static_cast<float*>(Scratch(ScratchKind::kSplitK, need, stream));
@@ -563,7 +584,7 @@ void Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream, const
   hipLaunchKernelGGL(kernel, dim3(tiles, p.splits), dim3(64 * WM * WN), bytes, stream, static_cast<const T*>(a.x),
                      static_cast<const T*>(a.w), static_cast<T*>(a.y), a.scale, a.shift, static_cast<const T*>(a.residual),
                      workspace, src.zero_page ? src.zero_page : ZeroPage(), p);
-  CINN_HIP_CALL(hipGetLastError());
+  if (hipError_t err = hipGetLastError(); err != hipSuccess) return LaunchFailed(src, err, "kernel launch");
   if (p.splits > 1) {
     if (p.oc % 4 == 0) {
       const int64_t total = (int64_t)p.pixels * p.oc / 4;
@@ -574,8 +595,9 @@ void Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream, const
       hipLaunchKernelGGL((SplitReduceKernel<T, 1>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, workspace,
                          static_cast<T*>(a.y), a.scale, a.shift, static_cast<const T*>(a.residual), p);
     }
-    CINN_HIP_CALL(hipGetLastError());
+    if (hipError_t err = hipGetLastError(); err != hipSuccess) return LaunchFailed(src, err, "launch of the split reduction");
   }
+  return 0;
 }
 
 // block tile and wavefront grid of a launch: {BM, BN, WM, WN}
@@ -592,23 +614,27 @@ TileShape TileFor(const ConvNhwcArgs& a, const Params& p) {
 }
 
 template <typename T>
-void Dispatch(const ConvNhwcArgs& a, const Params& p, hipStream_t stream, const ScratchSource& src = ScratchSource()) {
+int Dispatch(const ConvNhwcArgs& a, const Params& p, hipStream_t stream, const ScratchSource& src = ScratchSource()) {
   const TileShape t = TileFor(a, p);
   if (a.nchw_input) {
-    if (t.bm == 128)
-      Launch<T, 128, 64, 2, 2, true>(a, p, stream, src);
-    else
-      Launch<T, 64, 64, 2, 2, true>(a, p, stream, src);
-    return;
+    if (t.bm == 128) return Launch<T, 128, 64, 2, 2, true>(a, p, stream, src);
+    return Launch<T, 64, 64, 2, 2, true>(a, p, stream, src);
   }
-  if (t.bm == 128 && t.bn == 128 && t.wn == 4)
-    Launch<T, 128, 128, 2, 4, false>(a, p, stream, src);
-  else if (t.bm == 128 && t.bn == 128)
-    Launch<T, 128, 128, 2, 2, false>(a, p, stream, src);
-  else if (t.bm == 128)
-    Launch<T, 128, 64, 2, 2, false>(a, p, stream, src);
-  else
-    Launch<T, 64, 64, 2, 2, false>(a, p, stream, src);
+  if (t.bm == 128 && t.bn == 128 && t.wn == 4) return Launch<T, 128, 128, 2, 4, false>(a, p, stream, src);
+  if (t.bm == 128 && t.bn == 128) return Launch<T, 128, 128, 2, 2, false>(a, p, stream, src);
+  if (t.bm == 128) return Launch<T, 128, 64, 2, 2, false>(a, p, stream, src);
+  return Launch<T, 64, 64, 2, 2, false>(a, p, stream, src);
+}
+
+// every instantiation Dispatch<T> can reach
+template <typename T>
+hipError_t ConfigureAll() {
+  const hipError_t all[6] = {Configure<T, 128, 64, 2, 2, true>(),   Configure<T, 64, 64, 2, 2, true>(),
+                             Configure<T, 128, 128, 2, 4, false>(), Configure<T, 128, 128, 2, 2, false>(),
+                             Configure<T, 128, 64, 2, 2, false>(),  Configure<T, 64, 64, 2, 2, false>()};
+  for (hipError_t e : all)
+    if (e != hipSuccess) return e;
+  return hipSuccess;
 }
 
 int ChunkElems(const cinn_type_t& t) { return 16 / (t.bits / CHAR_BIT); }
@@ -727,8 +753,17 @@ extern "C" {
 size_t cinn_hip_conv2d_forward_noalloc_scratch_limit(void) { return kNoAllocPartialsBytes; }
 
 int cinn_hip_conv2d_forward_noalloc_init(void) {
+  using namespace cinn_hip_kernels;
   unsigned char* base = nullptr;
-  return NoAllocScratch(&base);
+  if (NoAllocScratch(&base) != 0) return 1;
+  // the LDS limit of every kernel the entry point can launch: a capturing stream does not allow this set-up call
+  for (hipError_t e : {ConfigureAll<float>(), ConfigureAll<_Float16>(), ConfigureAll<__bf16>()}) {
+    if (e != hipSuccess) {
+      fprintf(stderr, "cinn_hip_conv2d_forward_noalloc_init: hipFuncSetAttribute failed: %s\n", hipGetErrorString(e));
+      return 1;
+    }
+  }
+  return 0;
 }
 
 int cinn_call_hip_conv2d_forward_noalloc(void* v_args, int num_args, int format, float alpha, float beta, int input_n,
@@ -799,15 +834,11 @@ int cinn_call_hip_conv2d_forward_noalloc(void* v_args, int num_args, int format,
   src.zero_page            = base;
   src.fixed_partials       = reinterpret_cast<float*>(base + kNoAllocZeroBytes);
   src.fixed_partials_bytes = kNoAllocPartialsBytes;
+  src.status_only          = true;
   const Params fresh = MakeParams(a);  // Launch plans the split itself, identically
-  if (a.type.code == cinn_type_bfloat) {
-    Dispatch<__bf16>(a, fresh, static_cast<hipStream_t>(stream), src);
-  } else if (a.type.bits == 16) {
-    Dispatch<_Float16>(a, fresh, static_cast<hipStream_t>(stream), src);
-  } else {
-    Dispatch<float>(a, fresh, static_cast<hipStream_t>(stream), src);
-  }
-  return 0;
+  if (a.type.code == cinn_type_bfloat) return Dispatch<__bf16>(a, fresh, static_cast<hipStream_t>(stream), src);
+  if (a.type.bits == 16) return Dispatch<_Float16>(a, fresh, static_cast<hipStream_t>(stream), src);
+  return Dispatch<float>(a, fresh, static_cast<hipStream_t>(stream), src);
 }
 
 }  // extern "C"

@@ -100,7 +100,10 @@ int cinn_hip_stream_create(void** stream) {
   *stream       = s;
   return static_cast<int>(st);
 }
-int cinn_hip_stream_destroy(void* stream) { return Status(hipStreamDestroy(static_cast<hipStream_t>(stream))); }
+int cinn_hip_stream_destroy(void* stream) {
+  (void)cinn_hip_scratch_release_stream(stream);  // its scratch is retired with it, so a recycled handle starts empty
+  return Status(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+}
 int cinn_hip_stream_synchronize(void* stream) {
   return Status(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
 }

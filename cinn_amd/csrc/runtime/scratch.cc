@@ -2,7 +2,7 @@
 
 #include <map>
 #include <mutex>
-#include <utility>
+#include <tuple>
 #include <vector>
 
 #include "cinn_hip_runtime.h"
@@ -18,7 +18,7 @@ struct Buffer {
 
 struct Arena {
   std::mutex mu;
-  std::map<std::pair<hipStream_t, int>, Buffer> live;
+  std::map<std::tuple<int, hipStream_t, int>, Buffer> live;  // (device, stream, kind)
   std::vector<Buffer> retired;
   size_t retired_bytes{0};
 };
@@ -26,6 +26,12 @@ struct Arena {
 Arena& TheArena() {
   static Arena* arena = new Arena;  // leaked on purpose: intrinsics may run during static teardown
   return *arena;
+}
+
+int CurrentDevice() {
+  int device = 0;
+  CINN_HIP_CALL(hipGetDevice(&device));
+  return device;
 }
 
 bool Capturing(hipStream_t stream) {
@@ -37,7 +43,7 @@ bool Capturing(hipStream_t stream) {
 
 // caller holds the arena's mutex
 void* Ensure(Arena& arena, ScratchKind kind, size_t bytes, hipStream_t stream) {
-  Buffer& b = arena.live[{stream, static_cast<int>(kind)}];
+  Buffer& b = arena.live[{CurrentDevice(), stream, static_cast<int>(kind)}];
   if (bytes <= b.capacity) return b.data;
   CINN_RT_CHECK(!Capturing(stream),
                 "library scratch (kind %d) must grow from %zu to %zu bytes while its stream is being captured; run the "
@@ -64,13 +70,18 @@ void* Scratch(ScratchKind kind, size_t bytes, hipStream_t stream) {
 }
 
 const void* ZeroPage() {
-  static void* page = nullptr;
-  static std::once_flag once;
-  std::call_once(once, [] {
-    CINN_HIP_CALL(hipMalloc(&page, 256));
-    CINN_HIP_CALL(hipMemset(page, 0, 256));  // synchronous with respect to the host for device memory
-  });
-  return page;
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static void* pages[kMaxDevices];  // one page per device, allocated and cleared on its first use there
+  const int device = CurrentDevice();
+  CINN_RT_CHECK(device >= 0 && device < kMaxDevices, "device %d: the library keeps a page of zeros for at most %d devices", device,
+                kMaxDevices);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!pages[device]) {
+    CINN_HIP_CALL(hipMalloc(&pages[device], 256));
+    CINN_HIP_CALL(hipMemset(pages[device], 0, 256));  // synchronous with respect to the host for device memory
+  }
+  return pages[device];
 }
 
 }  // namespace cinn_hip_kernels
@@ -91,12 +102,29 @@ int cinn_hip_scratch_info(void* stream, size_t* split_k_capacity, size_t* transp
   Arena& arena = TheArena();
   std::lock_guard<std::mutex> lock(arena.mu);
   auto capacity = [&](ScratchKind kind) -> size_t {
-    auto it = arena.live.find({static_cast<hipStream_t>(stream), static_cast<int>(kind)});
+    auto it = arena.live.find({CurrentDevice(), static_cast<hipStream_t>(stream), static_cast<int>(kind)});
     return it == arena.live.end() ? 0 : it->second.capacity;
   };
   if (split_k_capacity) *split_k_capacity = capacity(ScratchKind::kSplitK);
   if (transpose_capacity) *transpose_capacity = capacity(ScratchKind::kTranspose);
   if (retired_bytes) *retired_bytes = arena.retired_bytes;
+  return 0;
+}
+
+int cinn_hip_scratch_release_stream(void* stream) {
+  using namespace cinn_hip_kernels;
+  Arena& arena = TheArena();
+  std::lock_guard<std::mutex> lock(arena.mu);
+  const int device = CurrentDevice();
+  for (int kind = 0; kind < kScratchKinds; ++kind) {
+    auto it = arena.live.find({device, static_cast<hipStream_t>(stream), kind});
+    if (it == arena.live.end()) continue;
+    if (it->second.data) {  // a graph captured on the stream may still hold the address: retire, do not free
+      arena.retired.push_back(it->second);
+      arena.retired_bytes += it->second.capacity;
+    }
+    arena.live.erase(it);
+  }
   return 0;
 }
 

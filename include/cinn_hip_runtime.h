@@ -311,22 +311,24 @@ const char* cinn_hip_error_string(int status);
 int cinn_hip_scratch_reserve(void* stream, size_t split_k_bytes, size_t transpose_bytes);
 int cinn_hip_scratch_info(void* stream, size_t* split_k_capacity, size_t* transpose_capacity, size_t* retired_bytes);
 int cinn_hip_scratch_release_retired(void);
+/* Lifetime rule: scratch is keyed by (current device, stream handle, kind) and outlives the stream.  Call this before
+ * hipStreamDestroy: the stream's buffers join the retired ones (a graph captured on the stream may still hold their
+ * addresses) and a later stream that happens to get the same handle value starts empty. */
+int cinn_hip_scratch_release_stream(void* stream);
 
 /* Kernel choice of cinn_call_cudnn_conv2d_forward / cinn_call_hip_conv2d_bn_relu for 3x3, stride 1, padding 1
  * convolutions on channels-last 16-bit tensors: 0 = never the kernel that keeps the input patch resident in LDS,
  * 1 = where it is expected to win (default; FLAGS_cinn_hip_conv_patch sets the initial value), 2 = wherever the shape
  * qualifies.  Returns the previous mode; any other argument only reads it.  No counterpart in the reference (cuDNN picks
- * its algorithm inside cudnnConvolutionForward, cinn/runtime/cuda/cuda_util.cc:560-640); a tuning and test switch. */
+ * its algorithm inside cudnnConvolutionForward, cinn/runtime/cuda/cuda_util.cc:560-640); a tuning and test switch.
+ * The setting is one atomic integer of the process: a convolution call that runs concurrently with a change uses the
+ * old or the new value as a whole, never a mixture. */
 int cinn_hip_conv_patch_mode(int mode);
 /* Block size of that kernel for more than 64 input channels: 4 or 2 tiles of 16 pixel slots per computing wavefront
  * (256 or 128 slots per block); 0 = chosen per shape (2 when 4 would give fewer than 192 blocks and 2 gives more).
- * Returns the previous setting; another value only reads it.  Initial value from FLAGS_cinn_hip_conv_patch_tiles. */
+ * Returns the previous setting; another value only reads it.  Initial value from FLAGS_cinn_hip_conv_patch_tiles.
+ * Atomic like the mode above. */
 int cinn_hip_conv_patch_tiles(int tiles);
-/* For tests of the chunked kernel's synchronisation: the `s_waitcnt vmcnt` count a feeding wavefront uses before the
- * barrier of K step (chunk, tap) - how many of its loads may still be in flight while the next filter stage (and, at
- * tap 8, the next chunk's patch) is known to have landed.  Host-side evaluation of the kernel's own constexpr. */
-int cinn_hip_conv_patch_loads_in_flight(int tap, int first_chunk, int last_chunk, int patch_loads_per_step);
-
 /* Device descriptor consumed by schedules.  Replaces common::Target's cudaDeviceGetAttribute
  * queries (cinn/common/target.cc:55-84, 177-221).  Filled from the live device when one is
  * present, otherwise with the MI355X datasheet values (256 CUs, wave64, 160 KiB LDS per CU). */

@@ -206,6 +206,14 @@ def test_argsort_and_sort_shapes_types_and_lowering():
     assert comp.num_instructions() == 2
     with pytest.raises(Exception, match="axis"):
         b.sort(x, 3)
+    # a row longer than one block's LDS holds is refused when the program is compiled, with the limit in the message
+    b = NetBuilder("t")
+    long_rows = b.create_input(Float(32), [2, 16385], "x")
+    with pytest.raises(Exception, match="at most 16384"):
+        compile_only(b, [b.sort(long_rows, 1)])
+    b = NetBuilder("t")
+    fits = b.create_input(Float(32), [2, 16384], "x")
+    assert compile_only(b, [b.sort(fits, 1)]).num_instructions() == 1
 
 
 def test_math_calls_are_mapped_to_the_device_library_by_operand_type():

@@ -198,6 +198,53 @@ def test_memset_in_a_captured_graph_replays_correctly(gpu):
     hip.hipGraphDestroy(graph)
 
 
+def test_nchw_convolution_of_a_new_shape_is_captured_without_an_eager_run(gpu):
+    """cinn_call_cudnn_conv2d_forward in the reference's own NCHW format (0), groups and dilation included, touches no
+    device memory beyond its operands: the first call of a shape may be made while its stream is being captured, after
+    cinn_hip_scratch_reserve only (cinn/runtime/cuda/cuda_util.cc:603-720 is the call it replaces)."""
+    import oracle
+    lib = _lib.load()
+    hip = ctypes.CDLL("libamdhip64.so")
+    conv_argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_float] + [ctypes.c_int] * 19 + [ctypes.c_void_p]
+    lib.cinn_call_cudnn_conv2d_forward.argtypes = conv_argtypes
+    lib.cinn_call_cudnn_conv2d_forward.restype = None
+    rng = np.random.default_rng(31)
+    stream = runtime.Stream()
+    assert lib.cinn_hip_scratch_reserve(stream.handle, ctypes.c_size_t(1 << 20), ctypes.c_size_t(1 << 20)) == 0
+    # odd extents nothing else in the test suite uses; dilation 2, two groups
+    n, c, h, w, f, k, pad, stride, dil, groups = 3, 10, 19, 23, 14, 3, 2, 2, 2, 2
+    x = rng.standard_normal((n, c, h, w)).astype(np.float32)
+    wt = rng.standard_normal((f, c // groups, k, k)).astype(np.float32)
+    oh = (h + 2 * pad - (dil * (k - 1) + 1)) // stride + 1
+    ow = (w + 2 * pad - (dil * (k - 1) + 1)) // stride + 1
+    X, W = runtime.DeviceBuffer.from_numpy(x, "float32"), runtime.DeviceBuffer.from_numpy(wt, "float32")
+    Y = runtime.DeviceBuffer((n, f, oh, ow), "float32")
+    Y.copy_from(np.zeros((n, f, oh, ow), np.float32))
+    args = runtime.pod_args([X, W, Y])
+    graph, graph_exec = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipStreamBeginCapture(stream.handle, 1) == 0  # hipStreamCaptureModeThreadLocal
+    lib.cinn_call_cudnn_conv2d_forward(args, 3, 0, 1.0, 0.0, n, c, h, w, f, c // groups, k, k, pad, pad, stride, stride, dil, dil,
+                                       groups, n, f, oh, ow, stream.handle)
+    assert hip.hipStreamEndCapture(stream.handle, ctypes.byref(graph)) == 0
+    assert hip.hipGraphInstantiate(ctypes.byref(graph_exec), graph, None, None, ctypes.c_size_t(0)) == 0
+    want = oracle.conv2d_nchw(x, wt, (stride, stride), (pad, pad), (dil, dil), groups)
+    scale = oracle.conv2d_nchw(np.abs(x), np.abs(wt), (stride, stride), (pad, pad), (dil, dil), groups)
+    for replay in range(3):
+        Y.copy_from(np.zeros((n, f, oh, ow), np.float32))  # eager work between the replays
+        assert hip.hipGraphLaunch(graph_exec, stream.handle) == 0
+        stream.synchronize()
+        got = Y.numpy()
+        assert np.all(np.abs(got - want) <= 1e-5 * scale), "replay %d" % replay
+    # the eager call gives the same bits as the replays
+    Y.copy_from(np.zeros((n, f, oh, ow), np.float32))
+    lib.cinn_call_cudnn_conv2d_forward(args, 3, 0, 1.0, 0.0, n, c, h, w, f, c // groups, k, k, pad, pad, stride, stride, dil, dil,
+                                       groups, n, f, oh, ow, stream.handle)
+    stream.synchronize()
+    assert np.array_equal(Y.numpy(), got)
+    hip.hipGraphExecDestroy(graph_exec)
+    hip.hipGraphDestroy(graph)
+
+
 RESIZE_KERNELS = r'''
 #include "cinn_hip_runtime_source.h"
 // out[n][c][y][x] = resize(in)[n][c][y][x], one thread per output element, through the reference-named entry points

@@ -95,3 +95,20 @@ def test_reserve_grows_and_never_shrinks(gpu):
     assert lib.cinn_hip_scratch_reserve(stream.handle, 10, transpose0 + 5000) == 0
     split2, transpose2, _ = scratch_info(stream)
     assert split2 == split and transpose2 >= transpose0 + 5000
+
+
+def test_releasing_a_stream_retires_its_scratch(gpu):
+    """cinn_hip_scratch_release_stream (and cinn_hip_stream_destroy, which calls it): the stream's buffers move to the
+    retired list - a graph captured on the stream may still hold them - and the handle starts empty again"""
+    lib = _lib.load()
+    lib.cinn_hip_scratch_reserve.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t]
+    lib.cinn_hip_scratch_release_stream.argtypes = [ctypes.c_void_p]
+    stream = runtime.Stream()
+    assert lib.cinn_hip_scratch_release_stream(stream.handle) == 0  # whatever an earlier owner of the handle left
+    assert scratch_info(stream)[:2] == (0, 0)
+    retired0 = scratch_info(stream)[2]
+    assert lib.cinn_hip_scratch_reserve(stream.handle, 70000, 3000) == 0
+    split, transpose, _ = scratch_info(stream)
+    assert split >= 70000 and transpose >= 3000
+    assert lib.cinn_hip_scratch_release_stream(stream.handle) == 0
+    assert scratch_info(stream) == (0, 0, retired0 + split + transpose)

@@ -3,7 +3,9 @@ outputs, on two calls in a row (the second with a smaller input, so that the sha
 first call's partial sums), with and without a split reduction, plus the error returns.  fp32 cases run on the same
 kernel under both entry points and must agree bit for bit; the fp16 case may be routed to another MFMA kernel by the
 allocating entry point (different summation order) and is held to the 1e-2 bar; every result is also compared with
-the CPU oracle."""
+the CPU oracle.  A last test makes the call while its stream is being captured (after
+cinn_hip_conv2d_forward_noalloc_init, which does the per-kernel set-up a capture does not allow), replays the graph and
+checks that neither the library's arena nor the device's free memory moved across the calls."""
 import ctypes
 
 import numpy as np
@@ -133,3 +135,67 @@ def test_noalloc_rejects_what_it_cannot_run_without_launching(gpu):
     assert lib.cinn_call_hip_conv2d_forward_noalloc(args, 2, 1, 1.0, 0.0, n, c, hw, hw, oc, c, 3, 3, 1, 1, 1, 1, 1, 1, 1, n, oc, hw, hw, None) == 1
     runtime.synchronize()
     assert np.array_equal(Y.numpy(), sentinel)
+
+
+def test_noalloc_allocates_nothing_and_runs_under_stream_capture(gpu):
+    lib = _lib.load()
+    hip = ctypes.CDLL("libamdhip64.so")
+    lib.cinn_call_hip_conv2d_forward_noalloc.argtypes = CONV_ARGTYPES
+    lib.cinn_call_hip_conv2d_forward_noalloc.restype = ctypes.c_int
+    assert lib.cinn_hip_conv2d_forward_noalloc_init() == 0
+    rng = np.random.default_rng(7)
+    stream = runtime.Stream()
+    # fp16 with a split reduction (49 tiles of 64x64, 18 K steps): two kernels, partial sums in the static scratch;
+    # fp32 unsplit with a stride: another instantiation.  Neither shape has run in this process before init.
+    cases = [(np.float16, 4, 128, 28, 64, 3, 1, 1), (np.float32, 4, 16, 40, 96, 3, 2, 1)]
+    for dtype, n, c, hw, oc, k, stride, pad in cases:
+        x, w = case(rng, dtype, n, c, hw, oc, k)
+        oh = oracle.conv_out_dim(hw, k, pad, stride)
+        dt = np.dtype(dtype).name
+        X, W = runtime.DeviceBuffer.from_numpy(nhwc(x), dt), runtime.DeviceBuffer.from_numpy(ohwi(w), dt)
+        Y, Yg = runtime.DeviceBuffer((n, oh, oh, oc), dt), runtime.DeviceBuffer((n, oh, oh, oc), dt)
+
+        def call(out):
+            return lib.cinn_call_hip_conv2d_forward_noalloc(runtime.pod_args([X, W, out]), 3, 1, 1.0, 0.0, n, c, hw, hw, oc, c,
+                                                            k, k, pad, pad, stride, stride, 1, 1, 1, n, oc, oh, oh, stream.handle)
+
+        def arena_state():
+            states = []
+            for st in (stream.handle, None):
+                caps = [ctypes.c_size_t(0) for _ in range(3)]
+                assert lib.cinn_hip_scratch_info(st, *[ctypes.byref(v) for v in caps]) == 0
+                states.append(tuple(v.value for v in caps))
+            return states
+
+        def free_bytes():
+            free, total = ctypes.c_size_t(0), ctypes.c_size_t(0)
+            assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+            return free.value
+
+        arena = arena_state()
+        assert call(Y) == 0                       # first eager call of this shape
+        stream.synchronize()
+        assert arena_state() == arena, "the call grew the library's arena"
+        # (the runtime itself may set up a kernel's first launch; free memory is compared across the next call)
+        free = free_bytes()
+        assert call(Y) == 0
+        stream.synchronize()
+        assert free_bytes() == free and arena_state() == arena, "the call changed the device's free memory"
+        eager = Y.numpy()
+        check_oracle(eager.transpose(0, 3, 1, 2), x, w, stride, pad, 1e-2 if dtype == np.float16 else 1e-5)
+        # the same call while the stream is being captured: nothing may run until the graph is launched
+        Yg.copy_from(np.full((n, oh, oh, oc), 3.0, dtype))
+        graph, graph_exec = ctypes.c_void_p(), ctypes.c_void_p()
+        assert hip.hipStreamBeginCapture(stream.handle, 1) == 0  # hipStreamCaptureModeThreadLocal
+        rc = call(Yg)
+        assert hip.hipStreamEndCapture(stream.handle, ctypes.byref(graph)) == 0
+        assert rc == 0, "the call was refused under capture"
+        assert hip.hipGraphInstantiate(ctypes.byref(graph_exec), graph, None, None, ctypes.c_size_t(0)) == 0
+        for replay in range(3):
+            Yg.copy_from(np.full((n, oh, oh, oc), 3.0, dtype))  # eager work between the replays
+            assert hip.hipGraphLaunch(graph_exec, stream.handle) == 0
+            stream.synchronize()
+            assert np.array_equal(Yg.numpy(), eager), "replay %d" % replay
+        hip.hipGraphExecDestroy(graph_exec)
+        hip.hipGraphDestroy(graph)
+        assert arena_state() == arena
