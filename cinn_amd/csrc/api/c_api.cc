@@ -339,6 +339,12 @@ int cinn_amd_computation_build_and_compile(cinn_amd_builder_t b, const char* con
           opts.fuse_matmul_bias = v != 0;
         } else if (k == "reshape_as_view") {
           opts.reshape_as_view = v != 0;
+        } else if (k == "merge_independent_kernels") {
+          opts.merge_independent_kernels = v != 0;
+        } else if (k == "memory_arena") {
+          opts.memory_arena = v != 0;
+        } else if (k == "reuse_intermediates") {
+          opts.reuse_intermediates = v != 0;
         } else if (k == "conv_layout_nhwc") {
           opts.conv_layout_nhwc = v != 0;
         } else if (k == "split_reductions") {
@@ -375,6 +381,12 @@ int cinn_amd_computation_execute_graph(cinn_amd_computation_t c) {
 }
 int cinn_amd_computation_pre_run(cinn_amd_computation_t c) {
   return Guard([&] { c->comp->PreRun(); });
+}
+int cinn_amd_computation_memory_info(cinn_amd_computation_t c, size_t* arena_bytes, size_t* unshared_bytes) {
+  return Guard([&] {
+    if (arena_bytes) *arena_bytes = c->comp->arena_bytes();
+    if (unshared_bytes) *unshared_bytes = c->comp->unshared_bytes();
+  });
 }
 int cinn_amd_computation_num_instructions(cinn_amd_computation_t c, int32_t* n) {
   return Guard([&] { *n = static_cast<int32_t>(c->comp->num_instructions()); });

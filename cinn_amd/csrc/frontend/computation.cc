@@ -56,6 +56,8 @@ std::shared_ptr<CinnComputation> CinnComputation::Compile(const common::Target& 
   gopts.with_instantiate_variables    = options.do_prerun && options.with_instantiate_variables;
   comp->program_                      = gc.Build(gopts);
   comp->source_code_                  = gc.source_code();
+  comp->arena_bytes_                  = gc.arena_bytes();
+  comp->unshared_bytes_               = gc.unshared_bytes();
   comp->compiler_                     = gc.ReleaseCompiler();
   return comp;
 }
@@ -72,14 +74,30 @@ std::vector<hlir::framework::Tensor> CinnComputation::GetOutputTensors() {
   for (auto& n : output_names_) out.push_back(GetTensor(n));
   return out;
 }
+namespace {
+// An intermediate whose bytes other values of the program reuse holds nothing the host could rely on.
+void CheckHostVisible(const hlir::framework::Tensor& t, const char* what) {
+  const hlir::framework::_Tensor_* root = t.get();
+  while (root->source()) root = root->source().get();
+  CINN_CHECK(!root->is_transient())
+      << what << ": this tensor is an intermediate of the compiled program whose device memory is shared with other "
+      << "intermediates (compile option reuse_intermediates); name it in the outputs of build_and_compile, or compile "
+      << "with reuse_intermediates=0, to give it memory of its own";
+}
+}  // namespace
+
 void CinnComputation::SetTensorData(hlir::framework::Tensor& t, void* data, size_t size) {
+  CheckHostVisible(t, "SetTensorData");
   t->CopyFromHost(data, size, target_);
 }
 void CinnComputation::SetTensorData(const std::string& tname, void* data, size_t size) {
   auto t = GetTensor(tname);
   SetTensorData(t, data, size);
 }
-void CinnComputation::GetTensorData(hlir::framework::Tensor& t, void* data, size_t size) { t->CopyToHost(data, size); }
+void CinnComputation::GetTensorData(hlir::framework::Tensor& t, void* data, size_t size) {
+  CheckHostVisible(t, "GetTensorData");
+  t->CopyToHost(data, size);
+}
 void CinnComputation::GetTensorData(const std::string& tname, void* data, size_t size) {
   auto t = GetTensor(tname);
   GetTensorData(t, data, size);

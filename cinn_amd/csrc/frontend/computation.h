@@ -65,6 +65,10 @@ class CinnComputation {
   const std::string& source_code() const { return source_code_; }
   std::string group_debug_string() const { return graph_->DebugGroupString(); }
   size_t num_instructions() const { return program_->size(); }
+  // size of the program's one device allocation (0: tensors are allocated one by one) and the sum of the sizes its
+  // tensors would have without sharing
+  size_t arena_bytes() const { return arena_bytes_; }
+  size_t unshared_bytes() const { return unshared_bytes_; }
   // stream lane (0 / 1) of every run instruction in a graph replay
   const std::vector<int>& GraphLanes() { return program_->GraphLanes(); }
   const std::vector<std::string>& output_names() const { return output_names_; }
@@ -81,6 +85,7 @@ class CinnComputation {
   std::unique_ptr<backends::Compiler> compiler_;
   std::vector<std::string> input_names_, output_names_;
   std::string source_code_;
+  size_t arena_bytes_{0}, unshared_bytes_{0};
 };
 
 }  // namespace frontend

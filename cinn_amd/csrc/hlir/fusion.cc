@@ -7,8 +7,13 @@
 //     and the merge closes no cycle in the group graph, i.e. there is no other path from the producer
 //     to the consumer; merging repeats until nothing changes.  A value with consumers outside the
 //     merged group simply stays an output of it, so no computation is ever duplicated;
+//   - then sibling groups merge (horizontal fusion, fusion_merge_pass.cc:85-120 and 176-260): two groups that read
+//     the same value, live in the same iteration space (equal flat size, or equal rows x cols) and do not depend
+//     on each other become one kernel that reads the shared value once - `reduce_sum(x)` and `argmax(x)` of one
+//     tensor are one pass over x;
 //   - kNonFusible ops and reductions over non-trailing axes stay alone.
 #include <algorithm>
+#include <cstdlib>
 #include <map>
 #include <set>
 
@@ -239,6 +244,62 @@ void Graph::BuildFusionGroups() {
         p->cols  = merged.cols;
         for (Node* m : c->nodes) group_of[m] = p;
         c->nodes.clear();
+        changed = true;
+      }
+    }
+  }
+
+  // horizontal fusion: sibling groups over a shared input.  `reaches(a, b)`: b depends on a, directly or not.
+  auto reaches = [&](WorkGroup* from, WorkGroup* to) {
+    std::set<WorkGroup*> visited;
+    std::vector<WorkGroup*> stack;
+    for (WorkGroup* s : successors(from)) stack.push_back(s);
+    while (!stack.empty()) {
+      WorkGroup* g = stack.back();
+      stack.pop_back();
+      if (g == to) return true;
+      if (!visited.insert(g).second) continue;
+      for (WorkGroup* s : successors(g)) stack.push_back(s);
+    }
+    return false;
+  };
+  auto group_inputs = [&](WorkGroup* g) {
+    std::set<const NodeData*> produced, ins;
+    for (Node* n : g->nodes)
+      for (auto* o : n->outputs) produced.insert(o);
+    for (Node* n : g->nodes)
+      for (auto* in : n->inputs)
+        if (!produced.count(in)) ins.insert(in);
+    return ins;
+  };
+  // FLAGS_cinn_hip_horizontal_fusion=0 keeps sibling groups apart (one kernel each, the shared value read by each)
+  const char* horizontal_flag = getenv("FLAGS_cinn_hip_horizontal_fusion");
+  changed                     = !(horizontal_flag && horizontal_flag[0] == '0');
+  while (changed) {
+    changed = false;
+    std::vector<WorkGroup*> live;
+    for (auto& g : work)
+      if (!g->nodes.empty() && (g->kind == GroupKind::kElementwise || g->kind == GroupKind::kRowReduce)) live.push_back(g.get());
+    for (size_t i = 0; i < live.size() && !changed; ++i) {
+      const auto ins_a = group_inputs(live[i]);
+      for (size_t j = i + 1; j < live.size() && !changed; ++j) {
+        WorkGroup *a = live[i], *b = live[j];
+        if (a->kind != b->kind) continue;  // an element-wise group next to a row group gains nothing from the row's phases
+        bool shared = false;
+        for (const NodeData* in : group_inputs(b))
+          // the shared value must be one both kernels stream (the whole space), not a per-row or scalar operand
+          if (ins_a.count(in) && in->numel() == (a->kind == GroupKind::kRowReduce ? a->rows * a->cols : a->numel)) shared = true;
+        if (!shared) continue;
+        WorkGroup merged;
+        if (!merged_shape(a, b, &merged)) continue;
+        if (reaches(a, b) || reaches(b, a)) continue;
+        a->kind  = merged.kind;
+        a->nodes = merged.nodes;
+        a->numel = merged.numel;
+        a->rows  = merged.rows;
+        a->cols  = merged.cols;
+        for (Node* m : b->nodes) group_of[m] = a;
+        b->nodes.clear();
         changed = true;
       }
     }

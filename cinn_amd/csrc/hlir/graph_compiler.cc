@@ -6,8 +6,10 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <set>
 
 #include "hlir/accuracy_checker.h"
+#include "hlir/memory_plan.h"
 #include "optim/optimize.h"
 
 namespace cinn {
@@ -20,6 +22,16 @@ namespace framework {
     CINN_CHECK_EQ(cinn_status__, 0) << #expr << " failed: " << cinn_hip_error_string(cinn_status__); \
   } while (0)
 
+// ---- DeviceArena ----------------------------------------------------------------------------------
+DeviceArena::DeviceArena(size_t bytes) : bytes_(bytes) {
+  void* p = nullptr;
+  CINN_HIP_STATUS(cinn_hip_malloc(&p, bytes ? bytes : 256));
+  base_ = static_cast<char*>(p);
+}
+DeviceArena::~DeviceArena() {
+  if (base_) cinn_hip_free(base_);
+}
+
 // ---- Tensor ---------------------------------------------------------------------------------------
 _Tensor_::_Tensor_() { cinn_hip_buffer_init(&buffer_, nullptr, cinn_type_float, 32, nullptr, 0); }
 _Tensor_::~_Tensor_() { Free(); }
@@ -30,8 +42,22 @@ void _Tensor_::ShareBufferWith(const std::shared_ptr<_Tensor_>& source) {
   source_ = source;
 }
 
+void _Tensor_::PlaceIn(std::shared_ptr<DeviceArena> arena, size_t offset, size_t capacity, bool transient) {
+  CINN_CHECK(!source_) << "a view is placed with its source";
+  CINN_CHECK(arena && offset + capacity <= arena->bytes()) << "tensor placed outside its arena";
+  Free();
+  arena_          = std::move(arena);
+  arena_offset_   = offset;
+  arena_capacity_ = capacity;
+  transient_      = transient;
+}
+
 void _Tensor_::Free() {
   if (source_) {  // a view owns nothing
+    buffer_.memory = nullptr;
+    return;
+  }
+  if (arena_ && allocated_ == 0) {  // a slice of the arena: nothing of its own to free
     buffer_.memory = nullptr;
     return;
   }
@@ -61,6 +87,21 @@ void* _Tensor_::mutable_data(const common::Target& target) {
       buffer_.memory_size = need;
     }
     return buffer_.memory;
+  }
+  if (arena_ && allocated_ == 0) {
+    if (need <= arena_capacity_) {
+      void* p = arena_->base() + arena_offset_;
+      if (buffer_.memory != p || buffer_.memory_size != need) {
+        int code = type_.is_bool() ? cinn_type_int : (type_.is_bfloat16() ? cinn_type_bfloat : static_cast<int>(type_.code));
+        cinn_hip_buffer_init(&buffer_, p, code, type_.is_bool() ? 1 : type_.bits, shape_.data(), static_cast<int>(shape_.size()));
+        buffer_.memory_size = need;
+      }
+      return buffer_.memory;
+    }
+    // resized beyond its slice: back to an allocation of its own
+    buffer_.memory = nullptr;
+    arena_.reset();
+    transient_ = false;
   }
   if (!buffer_.memory || allocated_ < need) {
     Free();
@@ -387,27 +428,6 @@ std::shared_ptr<Scope> BuildScope(const common::Target& target, const std::share
   return scope;
 }
 
-ir::Module GraphCompiler::LowerGraph(const CompileOptions& options) {
-  if (graph_->groups.empty()) graph_->BuildFusionGroups();
-  OpLowerer lowerer(target_, options.lowering);
-  ir::Module module;
-  module.name   = "cinn_hip_module";
-  module.target = target_;
-  for (auto& g : graph_->groups) {
-    auto func = lowerer.Lower(*g);
-    if (func->is_device) optim::OptimizeFuncGPU(func.get());
-    module.functions.push_back(func);
-  }
-  return module;
-}
-
-std::string GraphCompiler::GenSourceCode(const CompileOptions& options) {
-  auto module  = LowerGraph(options);
-  auto comp    = backends::Compiler::Create(target_);
-  source_code_ = comp->GetSourceCode(module);
-  return source_code_;
-}
-
 namespace {
 // one input, one output of the same type and size, and nothing but reshape operators in between
 bool IsReshapeOnly(const Group& g) {
@@ -420,6 +440,34 @@ bool IsReshapeOnly(const Group& g) {
 }
 }  // namespace
 
+ir::Module GraphCompiler::LowerGraph(const CompileOptions& options) {
+  if (graph_->groups.empty()) graph_->BuildFusionGroups();
+  OpLowerer lowerer(target_, options.lowering);
+  ir::Module module;
+  module.name   = "cinn_hip_module";
+  module.target = target_;
+  std::vector<ir::LoweredFuncRef> funcs;
+  std::vector<bool> barrier;
+  for (auto& g : graph_->groups) {
+    auto func = lowerer.Lower(*g);
+    if (func->is_device) optim::OptimizeFuncGPU(func.get());
+    funcs.push_back(func);
+    barrier.push_back(options.reshape_as_view && IsReshapeOnly(*g));  // becomes a view: no kernel to merge
+  }
+  KernelMergeOptions merge;
+  const char* flag = getenv("FLAGS_cinn_hip_merge_kernels");
+  merge.enabled    = options.merge_independent_kernels && !(flag && flag[0] == '0');
+  units_           = MergeIndependentKernels(graph_->groups, funcs, barrier, merge, &module.functions);
+  return module;
+}
+
+std::string GraphCompiler::GenSourceCode(const CompileOptions& options) {
+  auto module  = LowerGraph(options);
+  auto comp    = backends::Compiler::Create(target_);
+  source_code_ = comp->GetSourceCode(module);
+  return source_code_;
+}
+
 std::unique_ptr<Program> GraphCompiler::Build(const CompileOptions& options) {
   auto module = LowerGraph(options);
   compiler_   = backends::Compiler::Create(target_);
@@ -427,30 +475,104 @@ std::unique_ptr<Program> GraphCompiler::Build(const CompileOptions& options) {
   source_code_ = compiler_->source_code();
 
   std::vector<std::unique_ptr<Instruction>> instrs;
-  for (auto& g : graph_->groups) {
-    if (options.reshape_as_view && IsReshapeOnly(*g)) {
+  for (auto& u : units_) {
+    if (u.members.size() == 1 && options.reshape_as_view && IsReshapeOnly(*u.members[0])) {
       // a reshape of a dense row-major tensor moves nothing: the result shares its operand's memory and no kernel
       // runs (the reference copies, cinn/hlir/op/transform.cc Reshape)
-      scope_->Var(g->outputs[0]->id)->ShareBufferWith(scope_->Var(g->inputs[0]->id));
+      scope_->Var(u.outputs[0]->id)->ShareBufferWith(scope_->Var(u.inputs[0]->id));
       continue;
     }
     std::vector<std::string> ins, outs;
-    for (auto* v : g->inputs) ins.push_back(v->id);
-    for (auto* v : g->outputs) outs.push_back(v->id);
-    auto instr = std::make_unique<Instruction>(target_, scope_.get(), ins, outs, g->func_name);
-    void* fn   = compiler_->Lookup(g->func_name);
-    CINN_CHECK(fn) << "compiled function " << g->func_name << " not found";
+    for (auto* v : u.inputs) ins.push_back(v->id);
+    for (auto* v : u.outputs) outs.push_back(v->id);
+    auto instr = std::make_unique<Instruction>(target_, scope_.get(), ins, outs, u.func_name);
+    void* fn   = compiler_->Lookup(u.func_name);
+    CINN_CHECK(fn) << "compiled function " << u.func_name << " not found";
     instr->SetLoweredFunc(fn);
-    instr->pre_run = g->pre_run;
+    instr->pre_run = u.pre_run;
     instrs.push_back(std::move(instr));
   }
+  int device_count = 0;
+  if (options.with_instantiate_variables) cinn_hip_device_count(&device_count);
+  if (device_count > 0 && options.memory_arena) arena_bytes_ = PlanMemory(instrs, options);
   auto program = std::make_unique<Program>(scope_, std::move(instrs));
-  if (options.with_instantiate_variables) {
-    int device_count = 0;
-    cinn_hip_device_count(&device_count);
-    if (device_count > 0) program->PreRun(target_);
-  }
+  if (device_count > 0) program->PreRun(target_);
   return program;
+}
+
+// Memory plan of a compiled program.  Every tensor that an instruction reads or writes (views count as their source)
+// and that has no memory yet gets a slice of one allocation:
+//   * persistent slices, one each, for what the host or another execution may look at: fed inputs, fetched outputs,
+//     const values and everything pre-run instructions touch;
+//   * transient slices (PlanMemorySlots, memory_plan.h) for the rest - values produced by run instruction `def` and
+//     last read by run instruction `last`.
+// Slices are 256-byte aligned, the alignment the runtime's allocator gives and the kernels' 16-byte accesses rely on.
+size_t GraphCompiler::PlanMemory(const std::vector<std::unique_ptr<Instruction>>& instrs, const CompileOptions& options) {
+  constexpr size_t kAlign = 256;
+  std::vector<MemorySlot> slots;
+  std::vector<_Tensor_*> tensors;       // tensors[i] owns slots[i]
+  std::map<_Tensor_*, size_t> index_of;
+  std::vector<bool> written;            // by a run instruction
+  auto root_of = [&](const std::string& name) {
+    _Tensor_* t = scope_->GetTensor(name).get();
+    while (t->source()) t = t->source().get();
+    return t;
+  };
+  auto slot_of = [&](const std::string& name) -> size_t {
+    _Tensor_* t = root_of(name);
+    auto it     = index_of.find(t);
+    if (it != index_of.end()) return it->second;
+    MemorySlot s;
+    s.bytes = std::max<size_t>(kAlign, (t->bytes() + kAlign - 1) / kAlign * kAlign);
+    s.def = s.last = 0;
+    slots.push_back(s);
+    tensors.push_back(t);
+    written.push_back(false);
+    index_of[t] = slots.size() - 1;
+    return slots.size() - 1;
+  };
+  // what must keep bytes of its own, by root tensor
+  std::set<_Tensor_*> keep;
+  for (auto* v : graph_->AllVars()) {
+    if (!scope_->FindVar(v->id)) continue;
+    if (v->producer == nullptr || v->is_fetch || v->is_const || !options.reuse_intermediates) keep.insert(root_of(v->id));
+  }
+  int index = 0;
+  for (auto& ins : instrs) {
+    if (ins->pre_run) {
+      for (auto* list : {&ins->in_args(), &ins->out_args()})
+        for (auto& a : *list) slots[slot_of(a)].persistent = true;
+      continue;
+    }
+    for (auto& a : ins->in_args()) {
+      const size_t i = slot_of(a);
+      if (!written[i]) slots[i].persistent = true;  // read before any run instruction wrote it
+      slots[i].last = index;
+    }
+    for (auto& a : ins->out_args()) {
+      const size_t i = slot_of(a);
+      if (!written[i]) slots[i].def = index;
+      written[i]    = true;
+      slots[i].last = index;
+    }
+    ++index;
+  }
+  // tensors the caller gave memory already stay where they are
+  std::vector<MemorySlot> plan;
+  std::vector<_Tensor_*> planned;
+  unshared_bytes_ = 0;
+  for (size_t i = 0; i < slots.size(); ++i) {
+    if (tensors[i]->data() != nullptr) continue;
+    if (keep.count(tensors[i])) slots[i].persistent = true;
+    unshared_bytes_ += slots[i].bytes;
+    plan.push_back(slots[i]);
+    planned.push_back(tensors[i]);
+  }
+  if (plan.empty()) return 0;
+  const size_t total = PlanMemorySlots(&plan);
+  auto arena         = std::make_shared<DeviceArena>(total);
+  for (size_t i = 0; i < plan.size(); ++i) planned[i]->PlaceIn(arena, plan[i].offset, plan[i].bytes, !plan[i].persistent);
+  return total;
 }
 
 }  // namespace framework

@@ -1,7 +1,9 @@
 // Scope / Tensor / Instruction / Program / GraphCompiler of the GPU path.  Interfaces follow
 // cinn/hlir/framework/{scope.h,tensor.h,buffer.h,memory.cc,instruction.h,graph_compiler.h}:
 //   * a Tensor owns a cinn_buffer_t whose `memory` is device memory obtained through the runtime's
-//     allocator (role of CudaMemoryMng, memory.cc:43-64);
+//     allocator (role of CudaMemoryMng, memory.cc:43-64) - or, for the tensors of a compiled program, a
+//     slice of the program's one device allocation (DeviceArena below), in which intermediates whose
+//     lifetimes do not overlap share bytes;
 //   * an Instruction holds the names of its arguments and a lower_func_ptr_g; Run() packs the
 //     cinn_pod_value_t argument array once and calls the function (instruction.cc:77-138);
 //   * Program::Execute runs the instructions in order on one stream and synchronises when no
@@ -17,11 +19,29 @@
 #include "backends/compiler.h"
 #include "cinn_hip_runtime.h"
 #include "hlir/graph.h"
+#include "hlir/kernel_merge.h"
 #include "hlir/lowering.h"
 
 namespace cinn {
 namespace hlir {
 namespace framework {
+
+// One device allocation that holds every tensor of a compiled program (GraphCompiler::Build plans it): a few large
+// pages instead of one allocation per variable, and intermediates placed by lifetime so that a program's working set
+// is the largest set of values alive at once, not the sum of all of them.  Freed when the last tensor placed in it
+// and the scope that made it are gone.
+class DeviceArena {
+ public:
+  explicit DeviceArena(size_t bytes);
+  ~DeviceArena();
+  DeviceArena(const DeviceArena&) = delete;
+  char* base() const { return base_; }
+  size_t bytes() const { return bytes_; }
+
+ private:
+  char* base_{nullptr};
+  size_t bytes_{0};
+};
 
 class _Tensor_ {
  public:
@@ -42,6 +62,14 @@ class _Tensor_ {
   // allocation of its own, `source` stays the owner.  What a reshape of a dense row-major tensor is.
   void ShareBufferWith(const std::shared_ptr<_Tensor_>& source);
   bool is_view() const { return source_ != nullptr; }
+  const std::shared_ptr<_Tensor_>& source() const { return source_; }
+  // This tensor lives at `offset` of `arena` from now on (capacity bytes are its own while it is alive; a tensor that
+  // is later resized beyond them goes back to an allocation of its own).  transient: other tensors of the program
+  // occupy the same bytes before its producer and after its last consumer have run, so its contents mean something
+  // only in between - reading or writing it from the host by name is refused.
+  void PlaceIn(std::shared_ptr<DeviceArena> arena, size_t offset, size_t capacity, bool transient);
+  bool is_transient() const { return arena_ && transient_; }
+  bool in_arena() const { return arena_ != nullptr; }
   void* data() const { return source_ ? source_->data() : buffer_.memory; }
   cinn_buffer_t* buffer() { return &buffer_; }
 
@@ -56,6 +84,9 @@ class _Tensor_ {
   cinn_buffer_t buffer_;
   size_t allocated_{0};
   std::shared_ptr<_Tensor_> source_;  // set by ShareBufferWith
+  std::shared_ptr<DeviceArena> arena_;  // set by PlaceIn
+  size_t arena_offset_{0}, arena_capacity_{0};
+  bool transient_{false};
 };
 using Tensor = std::shared_ptr<_Tensor_>;
 
@@ -154,6 +185,14 @@ class Program {
 struct GraphCompileOptions {
   bool with_instantiate_variables{true};
   bool reshape_as_view{true};  // groups made of reshapes only become views of their operand instead of copy kernels
+  // consecutive generated kernels that do not depend on each other run as one launch (kernel_merge.h);
+  // FLAGS_cinn_hip_merge_kernels=0 switches it off for a process
+  bool merge_independent_kernels{true};
+  // every tensor the instructions touch is a slice of one device allocation (DeviceArena); off: one allocation each
+  bool memory_arena{true};
+  // within the arena, intermediates (produced and consumed by run instructions, neither fed, fetched nor const) whose
+  // lifetimes do not overlap share bytes; such a tensor cannot be read from the host - name it in the outputs
+  bool reuse_intermediates{true};
   LoweringOptions lowering{LoweringOptions::FromEnv()};
 };
 
@@ -167,14 +206,21 @@ class GraphCompiler final {
   // device source of the whole graph without loading anything
   std::string GenSourceCode(const CompileOptions& options = CompileOptions());
   const std::string& source_code() const { return source_code_; }
+  // bytes of the program's device arena after Build (0: none was made), and what one allocation per tensor would take
+  size_t arena_bytes() const { return arena_bytes_; }
+  size_t unshared_bytes() const { return unshared_bytes_; }
 
  private:
+  size_t arena_bytes_{0}, unshared_bytes_{0};
   ir::Module LowerGraph(const CompileOptions& options);
+  // places the tensors of the instructions in one DeviceArena; returns its size
+  size_t PlanMemory(const std::vector<std::unique_ptr<Instruction>>& instrs, const CompileOptions& options);
   common::Target target_;
   std::shared_ptr<Scope> scope_;
   std::shared_ptr<Graph> graph_;
   std::unique_ptr<backends::Compiler> compiler_;
   std::string source_code_;
+  std::vector<LaunchUnit> units_;  // the program's instructions, filled by LowerGraph
 
  public:
   // the Compiler owns the loaded code objects and host stubs; a Program must not outlive it

@@ -410,6 +410,12 @@ class Computation(object):
         _lib.check(lib.cinn_amd_computation_graph_lanes(self._handle, lanes, n.value, ctypes.byref(n)))
         return list(lanes)[:n.value]
 
+    def memory_info(self):
+        """(bytes of the program's one device allocation, bytes its tensors would take with one allocation each)"""
+        arena, unshared = ctypes.c_size_t(0), ctypes.c_size_t(0)
+        _lib.check(_lib.load().cinn_amd_computation_memory_info(self._handle, ctypes.byref(arena), ctypes.byref(unshared)))
+        return arena.value, unshared.value
+
     def num_instructions(self):
         n = ctypes.c_int32(0)
         _lib.check(_lib.load().cinn_amd_computation_num_instructions(self._handle, ctypes.byref(n)))

@@ -47,8 +47,13 @@ int cinn_amd_builder_program_string(cinn_amd_builder_t b, char* out, size_t cap,
 /* ---- CinnComputation (cinn/frontend/computation.h) ---- */
 /* CinnComputation::BuildAndCompile for the AMDGPU target.  outputs: ids to fetch (NULL/0: outputs of the
  * last instruction).  stream: hipStream_t or NULL.  options: "key=value;..." (keys: do_prerun,
- * fuse_conv_bn_relu, conv_layout_nhwc, split_reductions, and the lowering knobs reduce_cached_elems, reduce_wave_elems, elementwise_block,
- * reduce_rows_per_block). */
+ * fuse_conv_bn_relu, conv_layout_nhwc, split_reductions, merge_independent_kernels, memory_arena, reuse_intermediates,
+ * and the lowering knobs
+ * reduce_cached_elems, reduce_wave_elems, elementwise_block, reduce_rows_per_block).
+ * Memory: with memory_arena=1 (default) every tensor the program's instructions touch is a slice of ONE device
+ * allocation (the reference allocates per tensor, cinn/hlir/framework/memory.cc:43-53, tensor.h:64-82), and with
+ * reuse_intermediates=1 (default) values that are neither fed, fetched (named in `outputs`) nor const share bytes when
+ * their lifetimes do not overlap; set_tensor / get_tensor on such a value fail with a message that says so. */
 int cinn_amd_computation_build_and_compile(cinn_amd_builder_t b, const char* const* outputs, int32_t num_outputs,
                                            void* stream, const char* options, cinn_amd_computation_t* out);
 int cinn_amd_computation_destroy(cinn_amd_computation_t c);
@@ -57,6 +62,8 @@ int cinn_amd_computation_execute_graph(cinn_amd_computation_t c);
 /* Program::PreRun (cinn/hlir/framework/graph_compiler.cc:78-87): runs the pre-run instructions.  The first
  * execute does it by itself; call it again after replacing the data of a const input. */
 int cinn_amd_computation_pre_run(cinn_amd_computation_t c);
+/* size of the program's device allocation (0 when memory_arena=0) and the sum of its tensors' sizes without sharing */
+int cinn_amd_computation_memory_info(cinn_amd_computation_t c, size_t* arena_bytes, size_t* unshared_bytes);
 int cinn_amd_computation_num_instructions(cinn_amd_computation_t c, int32_t* n);
 /* Stream lane of every run instruction in a graph replay (0: the computation's stream, 1: the side stream that holds
  * instructions independent of their predecessor); writes min(capacity, *count) entries. */

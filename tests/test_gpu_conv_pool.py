@@ -114,7 +114,9 @@ def test_config4_conv_bn_relu_batch32(gpu, dtype, name, ic, oc, k, s, p, hw, nhw
     # conv (MFMA) + per-channel sqrt + one fused bn/relu kernel; the channels-last form adds the transposes of x and
     # w and one back to NCHW for the fetched convolution output (the one of y is fused into the bn/relu kernel)
     # (a 1x1 filter changes layout by a reshape, which is a view and no instruction)
-    assert comp.num_instructions() == ((5 if k == 1 else 6) if nhwc else 3), comp.fusion_groups()
+    # at most: sibling groups over one value fuse and independent neighbouring kernels share a launch (the two layout
+    # changes of x and w, the transpose of the fetched convolution output with the bn/relu kernel)
+    assert comp.num_instructions() <= ((5 if k == 1 else 6) if nhwc else 3), comp.fusion_groups()
     sample = [0, 17, 31]
     want_conv = oracle.conv2d_nchw(x[sample], w, (s, s), (p, p))
     want = oracle.batch_norm_relu_nchw(want_conv, scale, bias, mean, var, 1e-5, relu=True)

@@ -260,3 +260,46 @@ print("done", float(s[0]))
     assert "input: name=x, dtype=float32, shape={4, 8}, data=[1, 1, ... , 1, 1], One" in text, text
     assert any("input: name=y" in line and line.rstrip().endswith("NaN") for line in text.splitlines()), text
     assert any(line.strip().startswith("output:") and line.rstrip().endswith("NaN") for line in text.splitlines()), text
+
+
+def test_sibling_reductions_over_one_input_are_one_kernel(gpu):
+    """reduce_sum(x) and argmax(x) of one tensor fuse horizontally (cinn/hlir/pass/fusion_merge_pass.cc:85-120,
+    176-260): one instruction, x read once, both results bit-exact against the oracle at the config size; an
+    element-wise consumer of one of them and a third reduction ride along."""
+    rng = np.random.default_rng(29)
+    x = rng.integers(-1000, 1000, (16384, 512), endpoint=True).astype(np.int32)
+    b = NetBuilder("hz")
+    X = b.create_input(Int(32), x.shape, "x")
+    (s, am), comp = run(b, {X: x}, [b.reduce_sum(X, [1]), b.argmax(X, axis=1)])
+    assert comp.num_instructions() == 1, comp.fusion_groups()
+    assert comp.source_code().count("cinn_hip_copy_vec") == 1  # one load statement for x (unrolled twice): the row, once
+    assert np.array_equal(s, oracle.reduce_sum_i32(x))
+    assert am.dtype == np.int32 and np.array_equal(am, oracle.argmax_last(x))
+    # fp32: softmax(x) next to max(x) and argmin(x) of the same rows
+    xf = rng.standard_normal((512, 1000)).astype(np.float32)
+    b = NetBuilder("hz2")
+    X = b.create_input(Float(32), xf.shape, "x")
+    (sm, mx, amin), comp = run(b, {X: xf}, [b.softmax(X, axes=[-1]), b.reduce_max(X, [1]), b.argmin(X, axis=1)])
+    assert comp.num_instructions() == 1, comp.fusion_groups()
+    np.testing.assert_allclose(sm, oracle.softmax(xf), rtol=1e-5, atol=0)
+    assert np.array_equal(mx, xf.max(1)) and np.array_equal(amin, xf.argmin(1).astype(np.int32))
+
+
+def test_sibling_elementwise_groups_share_their_input_and_dependent_ones_stay_apart(gpu):
+    rng = np.random.default_rng(30)
+    a = rng.uniform(-1, 1, (3, 1000)).astype(np.float32)
+    b = NetBuilder("hz3")
+    A = b.create_input(Float(32), a.shape, "A")
+    # two element-wise siblings over A: one kernel, two outputs
+    (p, q), comp = run(b, {A: a}, [b.relu(A), b.exp(A)])
+    assert comp.num_instructions() == 1, comp.fusion_groups()
+    assert np.array_equal(p, np.maximum(a, 0)) and np.allclose(q, np.exp(a), rtol=1e-6)
+    # a row sum and a consumer of it that also reads A: vertical fusion already makes that one kernel; a reduction over
+    # the OTHER axis of A shares the input but not the iteration space and stays a kernel of its own
+    b = NetBuilder("hz4")
+    A = b.create_input(Float(32), a.shape, "A")
+    rows = b.reduce_sum(A, [1], keep_dim=True)
+    (y, cols), comp = run(b, {A: a}, [b.subtract(A, b.broadcast_to(rows, a.shape)), b.reduce_sum(A, [0])])
+    assert comp.num_instructions() >= 2, comp.fusion_groups()
+    np.testing.assert_allclose(y, a - a.sum(1, keepdims=True, dtype=np.float32), rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(cols, a.sum(0), rtol=1e-5, atol=1e-5)

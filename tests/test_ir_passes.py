@@ -1,6 +1,7 @@
 """C++ unit tests against the library's own headers, compiled and run here (no GPU needed): the GPU IR passes
-(csrc/optim) on hand-built loop nests (tests/cpp/test_ir_passes.cc) and the host-stub pool beyond its pre-compiled
-trampolines (tests/cpp/test_host_stubs.cc)."""
+(csrc/optim) on hand-built loop nests (tests/cpp/test_ir_passes.cc), the host-stub pool beyond its pre-compiled
+trampolines (tests/cpp/test_host_stubs.cc) and the placement of a program's tensors in one allocation
+(tests/cpp/test_memory_plan.cc)."""
 import os
 import subprocess
 
@@ -29,3 +30,7 @@ def test_host_stubs_beyond_the_precompiled_trampolines(tmp_path):
     closure, released thunks are reused (the reference JIT-compiles host stubs with LLVM and has no such bound,
     cinn/backends/llvm/execution_engine.cc)."""
     _build_and_run(tmp_path, "test_host_stubs")
+
+
+def test_memory_plan_never_overlaps_values_that_are_alive_together(tmp_path):
+    _build_and_run(tmp_path, "test_memory_plan")
