@@ -2,25 +2,29 @@
 """Benchmark of the gfx950 CINN backend on ONE MI355X.
 
 A "step" is one pass of the hot path over one batch of synthetic input of BASELINE.json configs[1] (fused reduce
-groups): six generated kernels - softmax over the last axis of [4096,4096] (fp32, fp16), Paddle layer_norm over
-[8192,1024] (fp32, fp16, gamma/beta fp32, mean/variance emitted), int32 reduce_sum and argmax over axis 1 of
-[16384,512] - launched in order on ONE stream, the way Program::Execute runs them.  Four batches are resident in HBM
-and step i works on batch i % 4 (1.5 GB of inputs and outputs are touched between two uses of a buffer, so nothing is
-served from the caches).  `value` is the algorithmic bytes of the six kernels divided by the step time.
+groups): ONE compiled program that holds the six fused groups - softmax over the last axis of [4096,4096] (fp32, fp16),
+Paddle layer_norm over [8192,1024] (fp32, fp16, gamma/beta fp32, mean/variance emitted), int32 reduce_sum and argmax
+over axis 1 of [16384,512] (each on its own input tensor) - executed with Program::Execute on ONE stream.  The groups
+do not depend on each other, so the compiler emits them as one launch whose blocks are handed out group by group
+(csrc/hlir/kernel_merge.h); `config.unmerged_*` is the same program compiled with merge_independent_kernels=0, six
+launches in order on the same stream.  Four batches (four compiled instances of the program, each with its own device
+memory) are resident in HBM and step i works on batch i % 4: 1.5 GB of inputs and outputs are touched between two uses
+of a buffer, so nothing is served from the caches.  `value` is the algorithmic bytes of the six groups divided by the
+step time.
 
 One JSON line is printed; besides the contract fields it carries
-  roofline     - the dominant kernel (fp32 softmax, 134 MB per launch): average launch duration measured with HIP
-                 events on the launch stream over runs of 200 back-to-back launches that cycle through 4 separate
-                 input/output buffer sets (537 MB, so every launch streams from HBM), against the 8 TB/s HBM peak
+  roofline     - the dominant kernel, which is the step's one launch (369 MB of algorithmic bytes): average launch
+                 duration measured with HIP events on the launch stream over runs of 200 back-to-back launches cycling
+                 through the four batches, against the 8 TB/s HBM peak
   cpu_baseline - the CPU oracle (a port of the reference's compute definitions, OpenMP) timed on this box's host
                  cores on the same workload
-  kernels      - every kernel of the step timed the same way, each over at least 512 MiB of rotating buffer sets
-  config       - also the step on three free-running streams (`three_stream_GBps`: the six kernels are independent, so
-                 launch gaps of one hide under the body of another; a property of the launch pattern, not of a kernel)
-  extra        - launch floors (an empty kernel, a hand-written cold 32 MiB read and copy), configs[0] (relu(add))
-                 latency, the scaled element-wise streaming rate, configs[2] GEMM, configs[3] convolution layers and
-                 configs[4] ResNet-50, each with its roofline bound and fraction, and under "cpu_baseline" the CPU
-                 oracle timed on bounded samples of those configs
+  kernels      - every fused group compiled and timed alone (one kernel per launch), each over at least 512 MiB of
+                 rotating buffer sets
+  extra        - launch floors (an empty kernel, a hand-written cold 32 MiB read and copy), reduce_sum + argmax of ONE
+                 tensor as one horizontally fused kernel, configs[0] (relu(add)) latency, the scaled element-wise
+                 streaming rate, configs[2] GEMM, configs[3] convolution layers and configs[4] ResNet-50, each with its
+                 roofline bound and fraction, and under "cpu_baseline" the CPU oracle timed on bounded samples of those
+                 configs
 """
 import argparse
 import json
@@ -46,8 +50,6 @@ def parse_args():
     p.add_argument("--warmup", type=int, default=20)
     p.add_argument("--no-cpu-baseline", action="store_true", help="skip timing the CPU oracle")
     p.add_argument("--no-extra", action="store_true", help="skip the configs outside the headline workload")
-    p.add_argument("--step-streams", type=int, default=3,
-                   help="HIP streams of the extra multi-stream step figure (0 or 1: skip it)")
     return p.parse_args()
 
 
@@ -111,13 +113,42 @@ def build_sets(spec, stream, count):
 
 
 def build_workload(stream):
-    """Compiles the six fused groups; every kernel gets enough buffer sets for a cold per-kernel measurement (at least
-    512 MiB between two uses of a set), the first STEP_BATCHES of which are the batches of the timed step."""
+    """Compiles every fused group alone; each gets enough buffer sets for a cold per-kernel measurement (at least
+    512 MiB between two uses of a set)."""
     kernels = []
     for spec in kernel_specs():
-        comps = build_sets(spec, stream, max(STEP_BATCHES, cold_sets(spec["bytes"])))
+        comps = build_sets(spec, stream, cold_sets(spec["bytes"]))
         kernels.append(dict(name=spec["name"], comps=comps, bytes=spec["bytes"], feeds=spec["feeds"], spec=spec))
     return kernels
+
+
+def build_step_program(stream, feeds_by_kernel, **options):
+    """ONE program with the six fused groups of configs[1] (the reduce_sum and the argmax on tensors of their own, so
+    that the step moves the same bytes whether or not sibling groups fuse); returns the compiled computation."""
+    from cinn_amd.common import DefaultAMDGPUTarget, Float, Int
+    from cinn_amd.frontend import Computation, NetBuilder
+    b = NetBuilder("step")
+    outs, feeds = [], {}
+    for tag, T in (("fp32", Float(32)), ("fp16", Float(16))):
+        X = b.create_input(T, [4096, 4096], "softmax_x_" + tag)
+        outs.append(b.softmax(X, axes=[-1]))
+        feeds[X.id] = feeds_by_kernel["softmax_" + tag]["x"]
+    for tag, T in (("fp32", Float(32)), ("fp16", Float(16))):
+        X = b.create_input(T, [8192, 1024], "layer_norm_x_" + tag)
+        G, Be = b.create_input(Float(32), [1024], "gamma_" + tag), b.create_input(Float(32), [1024], "beta_" + tag)
+        outs += b.paddle_layer_norm(X, G, Be, epsilon=1e-5)
+        f = feeds_by_kernel["layer_norm_" + tag]
+        feeds.update({X.id: f["x"], G.id: f["gamma"], Be.id: f["beta"]})
+    X = b.create_input(Int(32), [16384, 512], "reduce_sum_x")
+    outs.append(b.reduce_sum(X, [1]))
+    feeds[X.id] = feeds_by_kernel["reduce_sum_int32"]["x"]
+    X = b.create_input(Int(32), [16384, 512], "argmax_x")
+    outs.append(b.argmax(X, axis=1))
+    feeds[X.id] = feeds_by_kernel["argmax_int32"]["x"]
+    comp = Computation.build_and_compile(DefaultAMDGPUTarget(), b, outputs=outs, stream=stream, **options)
+    for var, data in feeds.items():
+        comp.get_tensor(var).from_numpy(data)
+    return comp
 
 
 def cpu_baseline(kernels, repeats=3):
@@ -319,6 +350,27 @@ def extra_measurements(stream, runtime):
         out[tag] = dict(us=round(ms * 1e3, 2), GBps=round(3 * a.nbytes / ms / 1e6, 1), bytes=3 * a.nbytes,
                         bound="hbm", frac=round(3 * a.nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), buffer_sets=len(comps))
         del comps
+    # reduce_sum(x) and argmax(x) of ONE tensor: sibling groups over a shared input fuse horizontally into one kernel
+    # that reads x once (cinn/hlir/pass/fusion_merge_pass.cc:176-260)
+    from cinn_amd.common import Int
+    xi = np.random.default_rng(2300).integers(-1000, 1000, (16384, 512), endpoint=True).astype(np.int32)
+    nbytes = xi.nbytes + 2 * 16384 * 4
+    comps = []
+    for _ in range(cold_sets(nbytes)):
+        b = NetBuilder("siblings")
+        X = b.create_input(Int(32), [16384, 512], "x")
+        comp = Computation.build_and_compile(DefaultAMDGPUTarget(), b, outputs=[b.reduce_sum(X, [1]), b.argmax(X, axis=1)],
+                                             stream=stream)
+        assert comp.num_instructions() == 1, comp.fusion_groups()
+        comp.get_tensor("x").from_numpy(xi)
+        comps.append(comp)
+    ms = time_comp(comps, 200)
+    out["sibling_reduce_sum_argmax_int32"] = dict(us=round(ms * 1e3, 2), GBps=round(nbytes / ms / 1e6, 1), bytes=nbytes,
+                                                  bound="hbm", frac=round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4),
+                                                  buffer_sets=len(comps), kernels=1,
+                                                  note="both results from one pass over x; as two kernels the same "
+                                                       "results take kernels.reduce_sum_int32 + kernels.argmax_int32")
+    del comps
     out["config0_add_relu_1x3x224x224"]["note"] = ("1.8 MB: latency-bound, 0.23 us at 8 TB/s against the launch period of "
                                                    "an empty kernel (launch_floors.empty_kernel)")
     # plain copy of known size: y = identity(x) over 64 Mi fp32 (256 MiB read, 256 MiB written).  It gives the
@@ -357,11 +409,13 @@ def main():
 
     stream = runtime.Stream()
     kernels = build_workload(stream)
-    dominant = 0  # softmax_fp32: the largest kernel of the step
+    feeds_by_kernel = {k["name"]: k["feeds"] for k in kernels}
+    batches = [build_step_program(stream, feeds_by_kernel) for _ in range(STEP_BATCHES)]
+    launches_per_step = batches[0].num_instructions()
+    assert launches_per_step == 1, "the six independent groups must share one launch:\n" + batches[0].fusion_groups()
 
-    def step(i, ks=kernels):
-        for k in ks:
-            k["comps"][i % STEP_BATCHES].run_instruction(0)
+    def step(i, progs=batches):
+        progs[i % STEP_BATCHES].execute()  # Program::Execute on `stream`: no synchronisation
 
     # the W untimed warm-up steps of the contract, then enough more to reach 30 ms of load: a timed region that starts
     # on an idle GPU measures the clock governor's ramp, not the kernels
@@ -388,36 +442,39 @@ def main():
     total_bytes = sum(k["bytes"] for k in kernels)
     value = total_bytes / (ms_per_step * 1e-3) / 1e9
 
-    # the same step with the six kernels spread round-robin over free-running streams (their own buffer sets)
-    multi = None
-    if args.step_streams > 1:
-        streams = [runtime.Stream() for _ in range(args.step_streams)]
-        mk = [dict(comps=build_sets(k["spec"], streams[n % len(streams)], STEP_BATCHES)) for n, k in enumerate(kernels)]
-        for w in range(60):
-            step(w, mk)
-        runtime.synchronize()
-        runs = []
-        for _ in range(3):
-            t0 = time.perf_counter()
-            for j in range(200):
-                step(j, mk)
-            runtime.synchronize()
-            runs.append((time.perf_counter() - t0) / 200)
-        multi = sorted(runs)[1]
-        del mk
-
-    # per-kernel average launch duration: event pairs around runs of 200 back-to-back launches that cycle through the
-    # kernel's buffer sets (an event pair around every single launch would add microseconds of marker overhead to each)
+    # the dominant kernel is the step's one launch: its average launch duration with HIP events on the launch stream
     launches = 200
+    merged_ms = sustained_ms(lambda n: batches[n % STEP_BATCHES].run_instruction(0), stream, runtime, launches=launches,
+                             warm_ms=10.0)
+
+    # the same program with one launch per group (merge_independent_kernels=0), same stream, same rotation
+    unmerged = [build_step_program(stream, feeds_by_kernel, merge_independent_kernels=0) for _ in range(STEP_BATCHES)]
+    assert unmerged[0].num_instructions() == 6
+    for w in range(60):
+        step(w, unmerged)
+    stream.synchronize()
+    runs = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        for j in range(200):
+            step(j, unmerged)
+        stream.synchronize()
+        runs.append((time.perf_counter() - t0) / 200)
+    unmerged_s = sorted(runs)[1]
+    del unmerged
+
+    # every group alone, per-kernel average launch duration: event pairs around runs of 200 back-to-back launches that
+    # cycle through the kernel's buffer sets (an event pair around every single launch would add microseconds of marker
+    # overhead to each)
     kernel_ms = [sustained_ms(lambda n, c=k["comps"]: c[n % len(c)].run_instruction(0), stream, runtime, launches=launches,
                               warm_ms=10.0) for k in kernels]
-    dom = kernels[dominant]
-    achieved = dom["bytes"] / (kernel_ms[dominant] * 1e-3) / 1e9
+    achieved = total_bytes / (merged_ms * 1e-3) / 1e9
     roofline = dict(bound="hbm", achieved=round(achieved, 1), peak=HBM_PEAK_GBS, unit="GB/s",
-                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=read_traffic(dom["name"]),
-                    traffic_source="profiles/%s_pmc.txt (a committed rocprofv3 --pmc run, not this run)" % dom["name"],
-                    kernel=dom["name"], algorithmic_bytes=dom["bytes"], avg_launch_us=round(kernel_ms[dominant] * 1e3, 2),
-                    launches=launches, buffer_sets=len(dom["comps"]))
+                    frac=round(achieved / HBM_PEAK_GBS, 4), traffic=read_traffic("step_merged"),
+                    traffic_source="profiles/step_merged_pmc.txt (a committed rocprofv3 --pmc run, not this run)",
+                    kernel="the step's one launch (six fused groups, blocks handed out group by group)",
+                    algorithmic_bytes=total_bytes, avg_launch_us=round(merged_ms * 1e3, 2), launches=launches,
+                    buffer_sets=STEP_BATCHES)
 
     result = {
         "metric": "fused-group HBM GB/s",
@@ -433,19 +490,18 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "configs[1] fused reduce groups: softmax [4096,4096] fp32+fp16, layer_norm [8192,1024] "
-                               "fp32+fp16, int32 reduce_sum+argmax [16384,512]; 6 generated kernels per step, in order on "
-                               "one stream, %d batches resident in HBM" % STEP_BATCHES,
+                               "fp32+fp16, int32 reduce_sum+argmax [16384,512]; one compiled program of 6 fused groups per "
+                               "step, Program::Execute on one stream, %d batches resident in HBM" % STEP_BATCHES,
                    "bytes_per_step": total_bytes, "percent_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
-                   "streams": 1, "resident_batches": STEP_BATCHES},
+                   "streams": 1, "resident_batches": STEP_BATCHES, "launches_per_step": launches_per_step,
+                   "unmerged_launches_per_step": 6, "unmerged_us_per_step": round(unmerged_s * 1e6, 2),
+                   "unmerged_GBps": round(total_bytes / unmerged_s / 1e9, 1)},
         "roofline": roofline,
         # each kernel alone, back-to-back launches cycling through at least 512 MiB of its own buffer sets
         "kernels": {k["name"]: dict(us=round(kernel_ms[n] * 1e3, 2), GBps=round(k["bytes"] / kernel_ms[n] / 1e6, 1),
                                     frac=round(k["bytes"] / kernel_ms[n] / 1e6 / HBM_PEAK_GBS, 4), bytes=k["bytes"],
                                     buffer_sets=len(k["comps"])) for n, k in enumerate(kernels)},
     }
-    if multi is not None:
-        result["config"]["three_stream_us_per_step" if args.step_streams == 3 else "multi_stream_us_per_step"] = round(multi * 1e6, 2)
-        result["config"]["three_stream_GBps" if args.step_streams == 3 else "multi_stream_GBps"] = round(total_bytes / multi / 1e9, 1)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(kernels)
     if not args.no_extra:
