@@ -185,7 +185,7 @@ def cpu_baseline(kernels, repeats=3):
 def extra_cpu_baselines():
     """The CPU oracle on bounded samples of the other configs (the same threads as cpu_baseline): configs[0] whole,
     configs[2]'s fp32 1024^3 product whole and 256 rows of the 16-bit 4096^3 products, configs[3]'s layers (fp32 and
-    fp16) and configs[4]'s network on 2 of the 32 images.  The thread count is OpenMP's default on the box (every
+    fp16) and configs[4]'s network (fp32 and fp16) on 2 of the 32 images.  The thread count is OpenMP's default on the box (every
     hardware thread the job may use); the reference's own host runtime would use half of them on x86
     (cinn/runtime/cpu/thread_backend.cc:29-44)."""
     import oracle
@@ -216,32 +216,37 @@ def extra_cpu_baselines():
     out.update(bench_gemm.cpu_baselines())
     out.update(bench_conv.cpu_baselines())
     images = 2
-    params = rn.random_params(0, "float32")
-    x = rng.standard_normal((images, 3, 224, 224)).astype(np.float32)
     specs = {sp[0]: sp for sp in rn.layer_specs()}
+    for dtype in ("float32", "float16"):
+        params = rn.random_params(0, dtype)
+        x = rng.standard_normal((images, 3, 224, 224)).astype(dtype)
+        dt = x.dtype
 
-    def conv_bn(inp, name, relu):
-        _, _, _, _, st, pad = specs[name]
-        y = oracle.conv2d_nchw(inp, params[name + "_w"], (st, st), (pad, pad))
-        return oracle.batch_norm_relu_nchw(y, params[name + "_scale"], params[name + "_bias"], params[name + "_mean"],
-                                           params[name + "_var"], 1e-5, relu=relu)
+        def conv_bn(inp, name, relu):
+            _, _, _, _, st, pad = specs[name]
+            y = oracle.conv2d_nchw(inp, params[name + "_w"], (st, st), (pad, pad))
+            return oracle.batch_norm_relu_nchw(y, params[name + "_scale"], params[name + "_bias"], params[name + "_mean"],
+                                               params[name + "_var"], 1e-5, relu=relu)
 
-    def network():
-        y = oracle.pool2d_nchw(conv_bn(x, "conv1", True), (3, 3), (2, 2), (1, 1, 1, 1), "max")
-        for si, (blocks, _, _) in enumerate(rn.STAGES):
-            for bi in range(blocks):
-                tag = "s%db%d" % (si + 2, bi)
-                short = conv_bn(y, tag + "_sc", False) if bi == 0 else y
-                z = conv_bn(conv_bn(conv_bn(y, tag + "_a", True), tag + "_b", True), tag + "_c", False)
-                y = np.maximum(z + short, np.float32(0))
-        y = oracle.pool2d_nchw(y, (7, 7), (1, 1), (0, 0, 0, 0), "avg").reshape(images, 2048)
-        return oracle.matmul(y, params["fc_w"]) + params["fc_b"]
+        def network():
+            # 16-bit tensors: the oracle's convolution and batch norm round to nearest with fp32 sums; pooling and the
+            # classifier are computed in fp32 and rounded once
+            y = oracle.pool2d_nchw(conv_bn(x, "conv1", True), (3, 3), (2, 2), (1, 1, 1, 1), "max").astype(dt)
+            for si, (blocks, _, _) in enumerate(rn.STAGES):
+                for bi in range(blocks):
+                    tag = "s%db%d" % (si + 2, bi)
+                    short = conv_bn(y, tag + "_sc", False) if bi == 0 else y
+                    z = conv_bn(conv_bn(conv_bn(y, tag + "_a", True), tag + "_b", True), tag + "_c", False)
+                    y = np.maximum((z + short).astype(dt), dt.type(0))
+            y = oracle.pool2d_nchw(y, (7, 7), (1, 1), (0, 0, 0, 0), "avg").reshape(images, 2048)
+            logits = oracle.matmul(y.astype(np.float32), params["fc_w"].astype(np.float32)) + params["fc_b"].astype(np.float32)
+            return logits.astype(dt)
 
-    t0 = time.perf_counter()
-    network()
-    t = time.perf_counter() - t0
-    out["resnet50_v1.5_float32"] = dict(value=round(images / t, 3), unit="images/s", cores=threads, kind="port",
-                                        sample="%d of the 32 images, one pass of %.1f s" % (images, t))
+        t0 = time.perf_counter()
+        network()
+        t = time.perf_counter() - t0
+        out["resnet50_v1.5_" + dtype] = dict(value=round(images / t, 3), unit="images/s", cores=threads, kind="port",
+                                             sample="%d of the 32 images, one pass of %.1f s" % (images, t))
     return out
 
 

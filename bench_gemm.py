@@ -4,7 +4,9 @@ events on the launch stream.  Imported by bench.py (extra measurements); also ru
 Reports TFLOP/s and the fraction of the dense MFMA peak (2.5 PFLOP/s for bf16 / fp16, 157.3 TFLOP/s for fp32): the
 median of three runs of 200 back-to-back launches after 30 ms of the same load (see bench_timing.py for why), and
 beside it `first_20_us`, the average of the first 20 launches after an idle period, which is what a short timing loop
-reads while the clock governor is still ramping."""
+reads while the clock governor is still ramping.
+    python bench_gemm.py --clock
+prints where the time of a 4096^3 launch goes, from time stamps the kernel writes itself (clock_probe).""" 
 import ctypes
 import json
 import os
@@ -72,6 +74,63 @@ def measure(stream, runtime):
     return out
 
 
+def clock_probe(stream, runtime, dtype="bfloat16", size=4096, launches=200):
+    """Where the time of a size^3 launch goes, from the kernel's own time stamps: with cinn_hip_gemm_set_probe every
+    block writes (100 MHz clock, core clock counter) at its start, after its first operands have landed, after its K
+    loop and after its last store was issued.  The launches run back to back after 30 ms of the same load; the stamps
+    of the last one are read.  Returns microseconds per phase (median over the blocks), the core clock the K loop ran
+    at (clock counter ticks per microsecond of the 100 MHz clock), and how far the blocks' starts and ends spread."""
+    from cinn_amd import _lib
+    from cinn_amd.common import float32_to_bfloat16_bits
+    lib = _lib.load()
+    lib.cinn_call_cublas.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_bool, ctypes.c_bool, ctypes.c_bool,
+                                     ctypes.c_float, ctypes.c_float] + [ctypes.c_int] * 8 + [ctypes.c_void_p]
+    lib.cinn_hip_gemm_set_probe.argtypes = [ctypes.c_void_p]
+    lib.cinn_hip_gemm_set_probe.restype = None
+    rng = np.random.default_rng(3000)
+    a = (rng.standard_normal((size, size)) * 0.02).astype(np.float32)
+    b = (rng.standard_normal((size, size)) * 0.02).astype(np.float32)
+    if dtype == "float16":
+        a, b = a.astype(np.float16), b.astype(np.float16)
+    else:
+        a, b = float32_to_bfloat16_bits(a), float32_to_bfloat16_bits(b)
+    A, B = runtime.DeviceBuffer.from_numpy(a, dtype), runtime.DeviceBuffer.from_numpy(b, dtype)
+    C = runtime.DeviceBuffer((size, size), dtype)
+    args = runtime.pod_args([A, B, C])
+    blocks = 4096  # more than any grid of this size has
+    stamps = runtime.DeviceBuffer((blocks, 8), "uint64")
+    stamps.copy_from(np.zeros((blocks, 8), np.uint64))
+
+    def launch(_i=0):
+        lib.cinn_call_cublas(args, 3, False, False, False, 1.0, 0.0, 1, 1, size, size, 1, 1, size, size, stream.handle)
+
+    lib.cinn_hip_gemm_set_probe(stamps.ptr)
+    try:
+        ms = sustained_ms(launch, stream, runtime, launches=launches, runs=3, warm_ms=30.0)
+        stream.synchronize()
+        t = stamps.numpy().astype(np.int64)
+    finally:
+        lib.cinn_hip_gemm_set_probe(None)
+    xcd = np.arange(len(t))[t[:, 0] != 0] % 8      # consecutive block indices go to consecutive XCDs
+    t = t[t[:, 0] != 0]
+    wall, core = t[:, 0::2] / 100.0, t[:, 1::2]   # microseconds, clock ticks
+    loop_us = wall[:, 2] - wall[:, 1]
+    loop_clk = (core[:, 2] - core[:, 1]) / loop_us / 1e3
+    per_xcd = [dict(xcd=int(x), k_loop_us=round(float(np.median(loop_us[xcd == x])), 2),
+                    core_clock_GHz=round(float(np.median(loop_clk[xcd == x])), 3)) for x in range(8)]
+    phase = np.median(np.diff(wall, axis=1), axis=0)
+    loop_ghz = np.median((core[:, 2] - core[:, 1]) / (wall[:, 2] - wall[:, 1])) / 1e3
+    whole_ghz = np.median((core[:, 3] - core[:, 0]) / (wall[:, 3] - wall[:, 0])) / 1e3
+    return dict(dtype=dtype, size=size, blocks=int(len(t)), us_per_launch=round(ms * 1e3, 2),
+                prologue_us=round(float(phase[0]), 2), k_loop_us=round(float(phase[1]), 2), epilogue_us=round(float(phase[2]), 2),
+                k_loop_us_min_max=[round(float(v), 2) for v in (np.diff(wall, axis=1)[:, 1].min(), np.diff(wall, axis=1)[:, 1].max())],
+                k_loop_core_clock_GHz=round(float(loop_ghz), 3), block_core_clock_GHz=round(float(whole_ghz), 3),
+                k_loop_clocks_per_step=round(float(np.median(core[:, 2] - core[:, 1])) / (size // 64), 1),
+                first_to_last_block_start_us=round(float(wall[:, 0].max() - wall[:, 0].min()), 2),
+                first_to_last_block_end_us=round(float(wall[:, 3].max() - wall[:, 3].min()), 2),
+                first_start_to_last_end_us=round(float(wall[:, 3].max() - wall[:, 0].min()), 2), per_xcd=per_xcd)
+
+
 def cpu_baselines(budget_s=4.0):
     """The CPU oracle on bounded samples: the fp32 1024^3 product whole, and 256 rows of the 16-bit 4096^3 products
     (fp32 accumulation, one rounding at the end, as the GPU kernels do)."""
@@ -112,4 +171,9 @@ def cpu_baselines(budget_s=4.0):
 
 if __name__ == "__main__":
     from cinn_amd import runtime as rt
-    print(json.dumps(measure(rt.Stream(), rt)))
+    if "--clock" in sys.argv:
+        # python3 bench_gemm.py --clock : per-phase time stamps of the 4096^3 launches, bf16 and fp16
+        st = rt.Stream()
+        print(json.dumps([clock_probe(st, rt, dt) for dt in ("bfloat16", "float16")]))
+    else:
+        print(json.dumps(measure(rt.Stream(), rt)))

@@ -113,6 +113,37 @@ def flop_per_image(image=224):
     return flops + 2 * 2048 * 1000
 
 
+HBM_PEAK_BPS = 8.0e12
+MFMA_PEAK_FLOPS = {"float16": 2.5e15, "float32": 157.3e12}
+
+
+def roofline_of(comp, dtype):
+    """Lower bound of one execution of a compiled network on MI355X: for every run instruction the larger of the HBM
+    time of its operands (every argument tensor once, at 8 TB/s) and the matrix-core time of its multiply-adds at the
+    dense peak of `dtype`, summed over the instructions (they run one after the other).  Multiply-adds are taken from
+    the arguments of the instruction: a convolution or product call (x, w, ..., y) does numel(y) * numel(w) / w.shape[0]
+    of them (four times that when a 2x2-strided pooling is folded into it: y is then the pooled tensor)."""
+    from cinn_amd.common import np_dtype
+    peak = MFMA_PEAK_FLOPS[dtype]
+    total, rows = 0.0, []
+    for i in range(comp.num_instructions()):
+        fn, args = comp.instruction_info(i)
+        tensors = {a: comp.get_tensor(a) for a in dict.fromkeys(args)}
+        nbytes = sum(int(np.prod(t.shape(), dtype=np.int64)) * np_dtype(str(t.type())).itemsize for t in tensors.values())
+        flop = 0
+        if "conv2d" in fn or "matmul" in fn or "mul" in fn.split("_"):
+            x, w, y = tensors[args[0]].shape(), tensors[args[1]].shape(), tensors[args[-1]].shape()
+            macs_per_output = int(np.prod(w, dtype=np.int64)) // w[0] if "conv2d" in fn else x[-1]
+            outputs = int(np.prod(y, dtype=np.int64))
+            if "conv2d" in fn and len(x) == 4 and x[1] == 3 and x[2] == 4 * y[1]:
+                outputs *= 4  # the image convolution with its max pooling folded in
+            flop = 2 * outputs * macs_per_output
+        t = max(nbytes / HBM_PEAK_BPS, flop / peak)
+        total += t
+        rows.append((fn, nbytes, flop, t))
+    return total, rows
+
+
 def measure(batch=32, dtype="float16", steps=20, warmup=3, graph=True, seed=0, **options):
     from cinn_amd import runtime
     from cinn_amd.common import DefaultAMDGPUTarget
@@ -147,11 +178,20 @@ def measure(batch=32, dtype="float16", steps=20, warmup=3, graph=True, seed=0, *
         times.append((time.perf_counter() - t0) / steps)
     dt = sorted(times)[1]
     flop = flop_per_image() * batch
-    peak = 157.3e12 if dtype == "float32" else 2.5e15
+    peak = MFMA_PEAK_FLOPS[dtype]
+    bound_s, rows = roofline_of(comp, dtype)
+    counted = sum(r[2] for r in rows)
+    assert abs(counted - flop) <= 1e-6 * flop, "multiply-adds of the instructions %d vs of the layer list %d" % (counted, flop)
+    arena, unshared = comp.memory_info()
     return {"workload": "resnet50_v1.5_b%d_%s" % (batch, dtype), "images_per_s": batch / dt, "ms_per_batch": dt * 1e3,
-            "tflops": flop / dt / 1e12, "flop_per_batch": flop, "bound": "mfma", "peak_TFLOPs": peak / 1e12,
-            "frac": flop / dt / peak, "instructions": comp.num_instructions(), "compile_s": compile_s,
-            "hip_graph": bool(graph), "timing": "median of 3 runs of %d batches after 100 ms of the same load" % steps}
+            "tflops": flop / dt / 1e12, "flop_per_batch": flop,
+            # the network's own roofline: per instruction max(HBM time of its operands, MFMA time of its flop), summed
+            "bound": "mixed", "bound_us": bound_s * 1e6, "frac": bound_s / dt,
+            "hbm_bound_instructions": sum(1 for r in rows if r[1] / HBM_PEAK_BPS >= r[2] / peak),
+            "peak_TFLOPs": peak / 1e12, "frac_of_mfma_peak": flop / dt / peak,
+            "instructions": comp.num_instructions(), "device_arena_bytes": arena, "unshared_tensor_bytes": unshared,
+            "compile_s": compile_s, "hip_graph": bool(graph),
+            "timing": "median of 3 runs of %d batches after 100 ms of the same load" % steps}
 
 
 if __name__ == "__main__":

@@ -66,3 +66,9 @@ bool TryConvStem7(const ConvNhwcArgs& a, hipStream_t stream);
 // its loads may still be in flight while the next filter stage (and, at tap 7, the next chunk's patch) is known to have
 // landed.  Host-side evaluation of the kernel's own constexpr, pure (no state).
 extern "C" int cinn_hip_conv_patch_loads_in_flight(int tap, int first_chunk, int last_chunk, int patch_loads_per_step);
+
+// Measurement hook of the direct-to-LDS GEMM kernel (gemm_mfma.hip), exported like the one above: while a device buffer
+// is set, thread 0 of every block of that kernel writes four (100 MHz clock, core clock counter) pairs - block start,
+// first operands landed, K loop done, last store issued - at buffer + 64 bytes * linear block index.  Null switches it
+// off.  bench_gemm.py --clock reads the stamps.
+extern "C" void cinn_hip_gemm_set_probe(void* device_buffer);

@@ -22,6 +22,7 @@
 // K-contiguous (transpose2d_kernel); gemm_generic_kernel is left with K % (16 bytes) != 0 and fp64.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <type_traits>
 
 #include <climits>
@@ -315,7 +316,22 @@ struct DmaEpilogue {
   // raw fp32 sums to partials[s][M][N]; the epilogue is applied by gemm16_split_reduce_kernel.  Null: no split.
   float* partials;
   int steps_per_split;
+  // Measurement hook (cinn_hip_gemm_set_probe): when set, thread 0 of every block writes eight 64-bit words at
+  // probe + 8 * (linear block index) - the constant 100 MHz clock and the core clock counter at block start, after the
+  // first operands have landed, after the K loop and after the last store was issued.  Null in normal use.
+  unsigned long long* probe = nullptr;
 };
+
+// `first_wave` must be wavefront-uniform (a scalar branch: a lane-dependent one ahead of the direct-to-LDS loads makes
+// the compiler move their scalar base addresses into vector registers, which the instruction does not take); every
+// lane of that wavefront stores the same words to the same address.
+__device__ __forceinline__ void ProbeStamp(unsigned long long* probe, bool first_wave, int slot) {
+  if (probe && first_wave) {
+    unsigned long long* at = probe + 8 * (blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)) + 2 * slot;
+    at[0] = __builtin_amdgcn_s_memrealtime();
+    at[1] = __builtin_readcyclecounter();
+  }
+}
 
 // Implicit-GEMM view of a channels-last convolution for gemm16_dma_kernel<.., CONV = true>: row m of A is output pixel
 // m = (n, oy, ox), K runs over (dy, dx, c) with c contiguous; a 64-deep K step lies inside one filter tap (the channel
@@ -387,6 +403,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   A += (int64_t)blockIdx.y * stride_a;
   B += (int64_t)blockIdx.y * stride_b;
   C += (int64_t)blockIdx.y * stride_c;
+  ProbeStamp(epi.probe, wave == 0, 0);
 
   // Load q = LPA wave + t of an operand fills LDS bytes [1024 q, 1024 q + 1024) of its tile: 8 rows of a
   // [row][64 halves] tile, or 512 / BN k-rows of a [k][BN halves] tile.
@@ -633,6 +650,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   }
   if (!feeder) {
   __syncthreads();
+  ProbeStamp(epi.probe, wave == 0, 1);
 #pragma unroll
   for (int i = 0; i < 3; ++i) ring[i] = read_a(sa(0), 0, i);
 #pragma unroll
@@ -717,6 +735,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
 #undef CINN_LOAD_SLOT
 #undef CINN_GEMM_STEP
 #undef CINN_SB
+  ProbeStamp(epi.probe, wave == 0, 2);
 
   // Epilogue on the fp32 accumulators: v = fma(residual_scale, R[row][col], fma(acc, scale[col] or alpha, shift[col]))
   // (explicit fused multiply-adds rounded to fp32, and an empty asm between them and the conversion to T: left to the
@@ -834,6 +853,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
         }
       }
     }
+    ProbeStamp(epi.probe, wave == 0, 3);
     return;
   }
   constexpr int kRowFloats = BN + 4;
@@ -902,6 +922,7 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
       }
     }
   }
+  ProbeStamp(epi.probe, wave == 0, 3);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -1572,6 +1593,9 @@ void XcdRectanglesPadded(int tiles_m, int tiles_n, int* xcd_cols, int* sub_rows,
   }
 }
 
+// device buffer of the time-stamp hook, or null (cinn_hip_gemm_set_probe)
+std::atomic<unsigned long long*> g_gemm_probe{nullptr};
+
 template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false, int NS = 2, bool FEED = false>
 void LaunchDma16(const GemmProblem& p, hipStream_t stream, int splits = 1) {
   int64_t ldb = p.trans_b ? p.k : p.n;
@@ -1582,6 +1606,7 @@ void LaunchDma16(const GemmProblem& p, hipStream_t stream, int splits = 1) {
   if (tiles_m * tiles_n >= 64) XcdRectanglesPadded(tiles_m, tiles_n, &xcd_cols, &sub_rows, &sub_cols);
   dim3 grid(sub_rows > 0 ? 8 * sub_rows * sub_cols : tiles_m * tiles_n, p.batch, splits);
   DmaEpilogue epi;
+  epi.probe           = g_gemm_probe.load(std::memory_order_relaxed);
   epi.partials        = nullptr;
   epi.steps_per_split = 0;
   if (splits > 1) {
@@ -2111,6 +2136,13 @@ bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream) {
 }  // namespace cinn_hip_kernels
 
 extern "C" {
+
+// Measurement hook, exported but deliberately absent from the public header (declared in kernels/conv_nhwc.h): every
+// later launch of the direct-to-LDS GEMM kernel writes four time-stamp pairs per block to `device_buffer` (8 x 8 bytes
+// per block of the launch; the caller sizes it), until it is called again with null.
+void cinn_hip_gemm_set_probe(void* device_buffer) {
+  g_gemm_probe.store(static_cast<unsigned long long*>(device_buffer), std::memory_order_relaxed);
+}
 
 // Shape algebra of cinn_call_cublas (cinn/runtime/cuda/cuda_util.cc:121-310) restated for a row-major kernel:
 // the result is [a1', a2', M, N] with M = trans_a ? a4 : a3, K = trans_a ? a3 : a4, N = trans_b ? b3 : b4;

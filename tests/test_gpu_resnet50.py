@@ -48,9 +48,16 @@ def gpu_forward(params, x, const_params=True, **options):
     return out, comp
 
 
-def assert_logits_close_fp16(got, want, rtol=1e-2, floor=0.1):
+def assert_logits_close_fp16(got, want, rtol=1e-2, ulps=1.5):
+    """Every logit within 1e-2 of itself or within 1.5 half-precision ulps of the LARGEST logit, whichever is larger.
+    The second term is what 53 layers of fp16 activations leave in a 2048-term sum: an absolute error that does not
+    shrink with the logit.  Measured against the oracle (batches of 2 and 4, two seeds, logit scale 21 - 23): the worst
+    error is exactly one ulp of the largest logit (0.0156) in both the unfused and the fused network; 99 % of the
+    logits lie within 0.5 ulp (unfused) and 0.9 ulp (folded batch norms, which round once instead of twice per
+    layer), independent of the logit's own size - so a bar relative to each logit alone would ask more of a logit
+    of 0.2 than half precision can give (its error would have to stay under 0.13 ulp of the scale)."""
     got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
-    bound = rtol * np.maximum(np.abs(want), floor * np.abs(want).max())
+    bound = np.maximum(rtol * np.abs(want), ulps * float(np.spacing(np.float16(np.abs(want).max()))))
     err = np.abs(got - want)
     assert np.all(err <= bound), "worst error / bound = %.3f at %s" % ((err / bound).max(), np.unravel_index(np.argmax(err / bound), err.shape))
 
@@ -77,8 +84,7 @@ def test_resnet50_fp16_batch2_matches_oracle(gpu):
     got, _ = gpu_forward(params, x, fuse_conv_bn_relu=False)
     want = oracle_forward(params, x).astype(np.float64)
     assert np.isfinite(got).all()
-    # 53 half-precision layers: every logit within 1e-2 of its own magnitude, logits much smaller than the largest
-    # one within 1e-2 of a tenth of the logit scale (a sum of O(scale) terms cannot be resolved below that in halves)
+    # 53 half-precision layers: every logit within 1e-2 of its own magnitude or 1.5 ulps of the largest logit
     assert_logits_close_fp16(got, want)
     fused, comp = gpu_forward(params, x, fuse_conv_bn_relu=True)
     # every batch norm, residual addition and relu now lives in a convolution epilogue, and the max pooling in the
@@ -140,8 +146,13 @@ def test_resnet50_batch32(gpu, dtype, tol):
         assert np.abs(got[[0, 31]] - want_ends).max() <= 1e-4 * np.abs(want_ends).max()
     else:
         assert_logits_close_fp16(got[[0, 31]], want_ends)
-    top1 = (np.argmax(got, 1) == np.argmax(want, 1)).mean()
-    assert top1 >= (1.0 if dtype == "float32" else 0.9)
+    # top-1: every image agrees with the float64 reference, unless the reference's two largest logits of that image
+    # lie closer together than twice the bar the logits are held to (then either order is a correct answer)
+    bar = tol * np.abs(want).max()
+    for img in np.nonzero(np.argmax(got, 1) != np.argmax(want, 1))[0]:
+        top2 = np.sort(want[img])[-2:]
+        assert top2[1] - top2[0] <= 2 * bar, "image %d: top-1 differs although the reference's lead is %g (bar %g)" % (
+            img, top2[1] - top2[0], bar)
 
 
 def test_resnet50_hip_graph_replay_matches_eager(gpu, monkeypatch):
