@@ -1223,8 +1223,16 @@ __global__ void __launch_bounds__(256 * KSPLIT)
 gemm32_mfma_kernel(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C, int M, int N, int K,
                    int64_t lda, int64_t ldb, int64_t ldc, float alpha, float beta, int64_t stride_a, int64_t stride_b,
                    int64_t stride_c, int xcd_cols, int sub_rows, int sub_cols) {
-  __shared__ __attribute__((aligned(16))) float As[2][KS][TILE + 4];
-  __shared__ __attribute__((aligned(16))) float Bs[2][KS][TILE + 4];
+  // Row pitch of the [k][row] tiles.  An operand whose contiguous axis is the row index is copied with 16-byte
+  // accesses (pitch a multiple of 4 floats; + 4 keeps the k rows of a fragment read apart).  One whose contiguous axis
+  // is k is scattered, four 4-byte writes per thread: a wavefront's lanes are (k chunk 0..7) x (row 0..7), so the bank
+  // of a write is pitch * 4 * chunk + row (mod 32) - with an odd pitch the eight chunks fall into eight different
+  // groups of four banks (TILE + 5: 20, 8, 28, 16, 4, 24, 12 away from chunk 0) and the scatter is conflict-free; with
+  // TILE + 4 chunks 0, 2, 4, 6 share their banks (SQ_LDS_BANK_CONFLICT / SQ_LDS_IDX_ACTIVE 0.33 on 1024^3).
+  constexpr int PA = TILE + (TRANS_A ? 4 : 5);
+  constexpr int PB = TILE + (TRANS_B ? 5 : 4);
+  __shared__ __attribute__((aligned(16))) float As[2][KS][PA];
+  __shared__ __attribute__((aligned(16))) float Bs[2][KS][PB];
   constexpr int TT      = TILE / 64;  // 32x32 MFMA tiles per wavefront and dimension
   constexpr int THREADS = 256 * KSPLIT;
   const int tid  = threadIdx.x;
@@ -1272,7 +1280,7 @@ gemm32_mfma_kernel(const float* __restrict__ A, const float* __restrict__ B, flo
     const int k = u / (TILE / 4), c = u % (TILE / 4);
     return *reinterpret_cast<const f32x4*>(P + (int64_t)(k0 + k) * ld + row0 + c * 4);
   };
-  auto store_one = [&](float (*S)[TILE + 4], bool k_contig, int i, f32x4 v) {
+  auto store_one = [&](auto* S, bool k_contig, int i, f32x4 v) {  // S: one buffer of As or Bs, float [KS][pitch]
     const int u = tid + THREADS * i;
     if (k_contig) {
       const int r = u / (KS / 4), kc = u % (KS / 4);
