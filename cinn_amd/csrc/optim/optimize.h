@@ -32,8 +32,27 @@ ir::Expr MapExternCall(const ir::Expr& body, const common::Target& target);
 // never completes (cinn/optim/transform_gpu_forloop.cc:628-661).
 ir::Expr SyncThreadsDropIfThenElse(const ir::Expr& body);
 
-// The driver: map extern calls, vectorize, bind, free barriers from their guards, and record launch dimensions into
-// func->axis_info.
+// Temporaries of a kernel (GPUShared / GPULocal buffers) written by a schedule as slices of a full-size tensor get the
+// shape of what one block / one thread really touches (cinn/optim/transform_gpu_forloop.cc, OptimizeExprGPU: 257-342
+// UpdateBufferAxisPass, 376-478 SharedAxisVisitor / LocalAxisVisitor, 562-608 ReplaceVarToZero).  Works on loops that
+// still carry their GPU bindings, i.e. before TransformGpuForloops; indices are flat here, so "dropping an axis" is
+// substituting 0 for its loop variable:
+//   * a GPULocal buffer is private to a thread: the variables of every loop bound to a block or thread axis that
+//     encloses an access, and of every loop that encloses ALL accesses of the buffer, become 0 in its indices;
+//   * a GPUShared buffer is private to a block: the same for loops bound to a block axis and for the serial loops that
+//     enclose all of its accesses; loops bound to a thread axis stay, they distinguish the block's threads;
+//   * in every index, the variable of a loop with extent 1 becomes the loop's first value.
+ir::Expr UpdateBufferAxes(const ir::Expr& body);
+
+// Shrinks the temporaries of `func` to the largest index its accesses can reach plus one (the reference's
+// ResizeBufferSizeVisitor, transform_gpu_forloop.cc:480-560, which enumerates every combination of loop values; here
+// the bound comes from interval arithmetic over the enclosing loops, so it may be larger than the exact maximum, never
+// smaller).  A buffer is never enlarged, and one with an access whose bound is unknown (a loop extent that is not a
+// constant, a variable that is no loop variable) keeps its size.  Run after UpdateBufferAxes, before binding.
+void ResizeBuffersToMaxVarRange(ir::LoweredFunc* func);
+
+// The driver: map extern calls, vectorize, drop the axes a temporary does not need and shrink it, bind, free barriers
+// from their guards, and record launch dimensions into func->axis_info.
 void OptimizeFuncGPU(ir::LoweredFunc* func);
 
 }  // namespace optim

@@ -89,10 +89,119 @@ static void TestBindAndVectorize() {
   if (failures) std::printf("%s\n", s.c_str());
 }
 
+// A schedule writes its temporaries as slices of the full-size tensor: under a block loop i (16) and a thread loop j
+// (64), a per-thread accumulator acc[i*64 + j] and a per-block staging tile[i*512 + j*8 + k].  One thread touches one
+// element of acc, one block 512 of tile: the block / thread terms leave the indices and the buffers shrink
+// (cinn/optim/transform_gpu_forloop.cc:257-560).  Global buffers keep their indices.
+static void TestBufferAxesAndResize() {
+  const common::Type i32 = common::Int(32), f32 = common::Float(32);
+  BufferRef a = MakeBuffer("a", f32, MemoryType::Global, 8192), o = MakeBuffer("o", f32, MemoryType::Global, 1024);
+  BufferRef acc = MakeBuffer("acc", f32, MemoryType::GPULocal, 1024), tile = MakeBuffer("tile", f32, MemoryType::GPUShared, 8192);
+  Expr i = MakeVar("i", i32), j = MakeVar("j", i32), k = MakeVar("k", i32), k2 = MakeVar("k2", i32), u = MakeVar("u", i32);
+  Expr lin = i * Expr(64) + j;
+  Expr stage = MakeFor(k, Expr(0), Expr(8), ForType::Serial,
+                       MakeStore(tile, MakeLoad(a, lin * Expr(8) + k), i * Expr(512) + j * Expr(8) + k));
+  Expr init = MakeStore(acc, MakeFloatImm(f32, 0.0), lin);
+  // a loop that runs once: u is its first value, 3
+  Expr sum = MakeFor(u, Expr(3), Expr(1), ForType::Serial,
+                     MakeFor(k2, Expr(0), Expr(8), ForType::Serial,
+                             MakeStore(acc, MakeLoad(acc, lin) + MakeLoad(tile, i * Expr(512) + j * Expr(8) + k2) * MakeCast(f32, u), lin)));
+  Expr out = MakeStore(o, MakeLoad(acc, lin), lin);
+  BindInfo bind_t{ForType::GPUThread, 0}, bind_b{ForType::GPUBlock, 0};
+  auto func  = std::make_shared<LoweredFunc>();
+  func->name = "k";
+  func->temp_bufs = {acc, tile};
+  func->body = MakeFor(i, Expr(0), Expr(16), ForType::GPUBlock,
+                       MakeFor(j, Expr(0), Expr(64), ForType::GPUThread, MakeBlock({stage, init, sum, out}), bind_t), bind_b);
+  Expr axes = optim::UpdateBufferAxes(func->body);
+  std::string s = ToString(axes);
+  EXPECT(Has(s, "acc[0]") && !Has(s, "acc[(") && !Has(s, "acc[i") );
+  EXPECT(Has(s, "tile[((j * 8) + k)]") && Has(s, "tile[((j * 8) + k2)]"));
+  EXPECT(Has(s, "o[((i * 64) + j)]") && Has(s, "a[((((i * 64) + j) * 8) + k)]"));
+  EXPECT(Has(s, "* 3.0f)") && !Has(s, "u)"));  // the loop over u stays as a scope, its variable is gone from the body
+  if (failures) std::printf("%s\n", s.c_str());
+  func->body = axes;
+  optim::ResizeBuffersToMaxVarRange(func.get());
+  EXPECT(acc->num_elements == 1);
+  EXPECT(tile->num_elements == 512);
+
+  // the driver does the same and binds: no loop variable of a bound loop is left in a temporary's index
+  acc->num_elements = 1024, tile->num_elements = 8192;
+  func->body = MakeFor(i, Expr(0), Expr(16), ForType::GPUBlock,
+                       MakeFor(j, Expr(0), Expr(64), ForType::GPUThread, MakeBlock({stage, init, sum, out}), bind_t), bind_b);
+  optim::OptimizeFuncGPU(func.get());
+  s = ToString(func->body);
+  EXPECT(Has(s, "acc[0]") && Has(s, "tile[((threadIdx.x * 8) + k)]") && Has(s, "o[((blockIdx.x * 64) + threadIdx.x)]"));
+  EXPECT(acc->num_elements == 1 && tile->num_elements == 512);
+  if (failures) std::printf("%s\n", s.c_str());
+
+  // an index whose range is unknown (n is no loop variable) leaves the buffer alone; a buffer is never enlarged
+  BufferRef small = MakeBuffer("small", f32, MemoryType::GPULocal, 4), odd = MakeBuffer("odd", f32, MemoryType::GPULocal, 64);
+  Expr n = MakeVar("n", i32), q = MakeVar("q", i32);
+  auto g  = std::make_shared<LoweredFunc>();
+  g->name = "g";
+  g->temp_bufs = {small, odd};
+  g->body = MakeFor(q, Expr(0), Expr(8), ForType::Serial,
+                    MakeBlock({MakeStore(small, MakeFloatImm(f32, 1.0), q % Expr(4)), MakeStore(odd, MakeFloatImm(f32, 1.0), q + n)}));
+  optim::ResizeBuffersToMaxVarRange(g.get());
+  EXPECT(small->num_elements == 4 && odd->num_elements == 64);
+}
+
+// What must stay as written: the passes only drop a variable when no two accesses that met in an element stop meeting
+// and no value has to survive in the dropped direction.
+static void TestBufferAxesKeepWhatIsNeeded() {
+  const common::Type i32 = common::Int(32), f32 = common::Float(32);
+  BufferRef a = MakeBuffer("a", f32, MemoryType::Global, 4096), o = MakeBuffer("o", f32, MemoryType::Global, 4096);
+  Expr j = MakeVar("j", i32), ko = MakeVar("ko", i32), ki = MakeVar("ki", i32), k2 = MakeVar("k2", i32);
+  BindInfo bind_t{ForType::GPUThread, 0};
+  auto run = [&](Expr inner) { return ToString(optim::UpdateBufferAxes(MakeFor(j, Expr(0), Expr(64), ForType::GPUThread, inner, bind_t))); };
+
+  // one slice per iteration of ko, filled and consumed inside it: the iterations share the slice
+  BufferRef tmp = MakeBuffer("tmp", f32, MemoryType::GPULocal, 64 * 16 * 4);
+  Expr at   = (j * Expr(16) + ko) * Expr(4);
+  Expr fill = MakeFor(ki, Expr(0), Expr(4), ForType::Serial, MakeStore(tmp, MakeLoad(a, at + ki), at + ki));
+  Expr use  = MakeFor(k2, Expr(0), Expr(4), ForType::Serial, MakeStore(o, MakeLoad(tmp, at + k2), at + k2));
+  std::string s = run(MakeFor(ko, Expr(0), Expr(16), ForType::Serial, MakeBlock({fill, use})));
+  EXPECT(Has(s, "tmp[ki] = ") && Has(s, "= tmp[k2]"));
+  if (failures) std::printf("%s\n", s.c_str());
+
+  // a slice that overlaps the next iteration's (step 2, four elements): ko stays, the thread's own offset goes
+  Expr at2 = j * Expr(64) + ko * Expr(2);
+  fill     = MakeFor(ki, Expr(0), Expr(4), ForType::Serial, MakeStore(tmp, MakeLoad(a, at + ki), at2 + ki));
+  use      = MakeFor(k2, Expr(0), Expr(4), ForType::Serial, MakeStore(o, MakeLoad(tmp, at2 + k2), at + k2));
+  s        = run(MakeFor(ko, Expr(0), Expr(16), ForType::Serial, MakeBlock({fill, use})));
+  EXPECT(Has(s, "tmp[((ko * 2) + ki)] = ") && Has(s, "= tmp[((ko * 2) + k2)]"));
+  if (failures) std::printf("%s\n", s.c_str());
+
+  // two halves used in turn (this iteration writes one, reads the other): not a constant step, ko stays
+  Expr half_w = (ko % Expr(2)) * Expr(4), half_r = ((ko + Expr(1)) % Expr(2)) * Expr(4);
+  fill        = MakeFor(ki, Expr(0), Expr(4), ForType::Serial, MakeStore(tmp, MakeLoad(a, at + ki), half_w + ki));
+  use         = MakeFor(k2, Expr(0), Expr(4), ForType::Serial, MakeStore(o, MakeLoad(tmp, half_r + k2), at + k2));
+  s           = run(MakeFor(ko, Expr(0), Expr(16), ForType::Serial, MakeBlock({fill, use})));
+  EXPECT(Has(s, "tmp[(((ko % 2) * 4) + ki)]") && Has(s, "tmp[((((ko + 1) % 2) * 4) + k2)]"));
+  if (failures) std::printf("%s\n", s.c_str());
+
+  // a block's shared buffer keeps the thread's offset and the serial loop: other threads read what this one wrote
+  BufferRef sh = MakeBuffer("sh", f32, MemoryType::GPUShared, 64 * 16 * 4);
+  fill         = MakeFor(ki, Expr(0), Expr(4), ForType::Serial, MakeStore(sh, MakeLoad(a, at + ki), at + ki));
+  use          = MakeFor(k2, Expr(0), Expr(4), ForType::Serial, MakeStore(o, MakeLoad(sh, at + k2), at + k2));
+  s            = run(MakeFor(ko, Expr(0), Expr(16), ForType::Serial, MakeBlock({fill, use})));
+  EXPECT(Has(s, "sh[((((j * 16) + ko) * 4) + ki)] = "));
+  if (failures) std::printf("%s\n", s.c_str());
+
+  // a thread's buffer read with another thread's offset (the schedule's mistake or a rotation): steps differ, untouched
+  BufferRef loc = MakeBuffer("loc", f32, MemoryType::GPULocal, 256);
+  s = run(MakeBlock({MakeStore(loc, MakeLoad(a, j), j), MakeStore(o, MakeLoad(loc, j * Expr(2)), j)}));
+  EXPECT(Has(s, "loc[j] = ") && Has(s, "loc[(j * 2)]"));
+  if (failures) std::printf("%s\n", s.c_str());
+}
+
 int main() {
   TestMapExternCall();
   TestSyncThreadsDropIfThenElse();
   TestBindAndVectorize();
+  TestBufferAxesAndResize();
+  TestBufferAxesKeepWhatIsNeeded();
   if (failures) return 1;
   std::printf("ok\n");
   return 0;
