@@ -72,3 +72,8 @@ extern "C" int cinn_hip_conv_patch_loads_in_flight(int tap, int first_chunk, int
 // first operands landed, K loop done, last store issued - at buffer + 64 bytes * linear block index.  Null switches it
 // off.  bench_gemm.py --clock reads the stamps.
 extern "C" void cinn_hip_gemm_set_probe(void* device_buffer);
+
+// The same for conv3x3_c64_stream_kernel (conv_patch_mfma.hip): six pairs per block at buffer + 128 bytes * linear
+// block index - block start, filter and first patch rows landed, first tile multiplied, whole patch landed, fourth
+// tile stored, last store issued.  bench_conv.py --clock reads the stamps.
+extern "C" void cinn_hip_conv_patch_set_probe(void* device_buffer);

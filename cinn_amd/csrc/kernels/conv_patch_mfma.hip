@@ -75,6 +75,8 @@ struct PatchParams {
   int rows;         // output rows per band (stacked images: their rows and the separating rows)
   int bands;        // bands per image
   int patch_loads;  // 1 KiB loads that cover the (rows + 2) (W + 2) positions of 10 slots
+  int first_loads;  // streaming kernel: the first so many of them cover the rows that the band's first 64 pixels read
+  unsigned long long* probe;  // measurement hook (cinn_hip_conv_patch_set_probe): 16 words per block, or null
   unsigned w_magic, w_shift;    // n / W == (n * w_magic) >> w_shift (chunked kernel: W rounded up to a multiple of 8)
   unsigned pw_magic, pw_shift;  // the same for W + 2
 };
@@ -397,6 +399,264 @@ __device__ __forceinline__ void WaitLoadsInFlight(int n) {
   }
 }
 
+// The same layer with the three phases of conv3x3_c64_patch_kernel - fetch the patch, multiply, store - overlapped
+// inside a block instead of following each other.  That kernel walks the taps in its outer loop (a filter stage is
+// used once, by every pixel), so no pixel is finished before the last tap and all stores come at the end.  Here the
+// pixels are the outer loop: the WHOLE filter sits in registers (eight computing wavefronts, wavefront (pg, h) keeps
+// the 9 x 64 x 32 filter of the output channels 32 h .. 32 h + 31: 144 registers), a wavefront takes one tile of 16
+// pixels through all nine taps (36 MFMAs on two accumulators), converts and stores it, and goes on to the next while
+// those stores drain.  Per MFMA it reads LDS half as often as the tap-major loop needs for the same tile shape, two
+// wavefronts share a SIMD (one's epilogue and LDS waits are covered by the other's MFMAs) and there are no feeding
+// wavefronts and no barrier per K step: the loads are all issued at the start.
+//   * LDS: the patch from 0, as in the other kernel; the filter stages of the taps 0..7 (swizzled rows as there) at
+//     kStreamFilter; the folded scale / shift of the block's 64 channels in the last KiB.  The ninth stage does not
+//     fit beside them; it travels in the two dummy slots that every patch position has behind its 128 bytes (a patch
+//     load fills 64 consecutive slots of 16 bytes, ten per position): dummy slot d = 2 position + (0 | 1), d < 512,
+//     holds chunk d % 8 of filter row d / 8.  Nothing in LDS is written twice, so no load has to wait for a reader.
+//   * Tiles are dealt round-robin, tile 4 s + pg in step s, so the block moves down the band together: step 0 only
+//     reads the first rows of the patch (p.first_loads loads, which also cover the ninth stage) and starts when those
+//     and the filter have landed.  During step 0 a wavefront moves its filter fragments from LDS into registers, each
+//     just ahead of its first MFMA.  Everything else is waited for once, after step 0; then the block runs free.
+//     What a block requests (148 KB: 74 KB of patch, 74 KB of filter) leaves L2 at about 44 GB/s per CU when all CUs
+//     pull at once (direct-to-LDS loads of a load-only kernel land 8 KiB per CU every 0.18 us whatever they hit), so
+//     the first MFMA cannot come before about 3 us into the block and the last row lands about a microsecond later.
+//   * All global loads are the untracked direct-to-LDS ones (also scale / shift): the compiler sees LDS reads and
+//     global stores only and never waits for the latter.  (A residual operand is read with ordinary loads in the
+//     epilogue, which then waits for the stores before it too - correct, slower; 3x3 layers rarely have one.)
+// Sums are formed in the same order as in conv3x3_c64_patch_kernel (tap, then the two halves of the channels) and the
+// epilogue is the same arithmetic: results are bit-identical.
+
+// Measurement hook: with a buffer set, one wavefront of every block stores the 100 MHz counter and the core clock
+// counter at up to eight points (16 words per block).  `chosen` must be wavefront-uniform; every lane stores the same
+// words.  The stores count like any other in vmcnt: a wait of that wavefront for its loads then waits for them as
+// well, never for less (the stamps come from a wavefront that does not wait during step 0).
+__device__ __forceinline__ void PatchStamp(unsigned long long* probe, bool chosen, int slot) {
+  if (probe && chosen) {
+    unsigned long long* at = probe + 16 * (blockIdx.x + gridDim.x * blockIdx.y) + 2 * slot;
+    at[0] = __builtin_amdgcn_s_memrealtime();
+    at[1] = __builtin_readcyclecounter();
+  }
+}
+
+constexpr int kStreamWaves  = 8;
+constexpr int kStreamSteps  = 7;                                       // tiles per wavefront
+constexpr int kStreamScale  = kLdsLimit - 1024;                        // 64 scales, 64 shifts (fp32)
+constexpr int kStreamFilter = kStreamScale - (kTaps - 1) * kBTile;     // eight stages of 8 KiB
+constexpr int kStreamLast   = 64 * 8;                                  // dummy slots that hold the ninth stage
+constexpr int kStreamLastLoads = (kStreamLast / 2 * 10 + 63) / 64;     // patch loads that cover their positions
+
+template <typename T>
+__global__ void __launch_bounds__(64 * kStreamWaves) conv3x3_c64_stream_kernel(PatchParams p) {
+  typedef typename Mfma16<T>::vec8 vec8;
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  char* const patch = lds;
+  char* const filt  = lds + kStreamFilter;
+  const unsigned lds_addr = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) char*)lds);
+
+  const int tid  = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int pg   = wave & 3;   // tiles pg, pg + 4, ...
+  const int half = wave >> 2;  // output channels 32 half .. + 31 of the block's 64
+  const int band = blockIdx.x % p.bands;
+  const int img  = blockIdx.x / p.bands;
+  const int n0   = blockIdx.y * 64;
+  const int W    = p.w_in;
+  const int PW   = W + 2;
+  const int y0   = band * p.rows;
+  const int rows = min(p.rows, p.h - y0);
+  const int npix = rows * W;
+  const int npos = (p.rows + 2) * PW;
+  constexpr int ktot = kTaps * 64;
+  const char* const zeros = static_cast<const char*>(p.zero_page);
+  const char* const wblk  = reinterpret_cast<const char*>(p.w + (int64_t)n0 * ktot);
+  PatchStamp(p.probe, wave == 0, 0);
+
+  // ---- every load of the block, those that step 0 needs first
+  if (wave == 0) {  // lanes 0..15: four scales each, 16..31: four shifts each
+    const char* src = zeros + ((lane & 7) << 4);
+    if (lane < 16 && p.scale) src = reinterpret_cast<const char*>(p.scale + n0 + 4 * lane);
+    if (lane >= 16 && lane < 32 && p.shift) src = reinterpret_cast<const char*>(p.shift + n0 + 4 * (lane - 16));
+    AsyncCopy16(src, lds_addr + kStreamScale);
+  }
+  {  // filter stages 0..7: this wavefront fetches the rows 8 wave .. + 7 of each
+    const int row      = 8 * wave + (lane >> 3);
+    const unsigned off = (unsigned)(row * ktot + (((lane & 7) ^ FilterKey(row)) << 3)) * 2u;
+#pragma unroll
+    for (int t = 0; t + 1 < kTaps; ++t) AsyncCopy16(wblk + off + t * 128, lds_addr + kStreamFilter + t * kBTile + wave * 1024);
+  }
+  // patch loads q = wave, wave + 8, ... of [lo, hi): load q fills the slots 64 q .. 64 q + 63 (slot s = chunk s % 10 of
+  // position s / 10; chunks 8 and 9 are the dummies, of which the first 512 carry the ninth filter stage and the
+  // others are not fetched at all: their lanes sit the load out)
+  auto load_patch = [&](int lo, int hi) {
+    const char* const ximg = reinterpret_cast<const char*>(p.x + (int64_t)img * p.h * W * 64);
+    for (int q = lo + ((wave - lo) & 7); q < hi; q += kStreamWaves) {
+      const unsigned slot  = 64u * q + lane;
+      const unsigned pos   = (slot * 52429u) >> 19;  // slot / 10 for slot < 2^16
+      const unsigned chunk = slot - 10u * pos;
+      const int pr         = (int)(((uint64_t)pos * p.pw_magic) >> p.pw_shift);
+      const int iy         = y0 - 1 + pr;
+      const int ix         = (int)pos - pr * PW - 1;
+      const bool inside    = chunk < 8u && (unsigned)iy < (unsigned)p.h && (unsigned)ix < (unsigned)W && (int)pos < npos;
+      const unsigned d     = 2u * pos + (chunk - 8u);  // dummy slot number
+      const char* src      = inside ? ximg + ((unsigned)(iy * W + ix) * 128u + chunk * 16u) : zeros + ((lane & 7) << 4);
+      if (chunk >= 8u) src = wblk + ((d >> 3) * ktot + (kTaps - 1) * 64 + (d & 7u) * 8u) * 2u;
+      if (chunk < 8u || d < (unsigned)kStreamLast) AsyncCopy16(src, lds_addr + q * 1024);
+    }
+  };
+  // The address unit's queue holds less than the block requests and serves the oldest wavefront first: without the
+  // barrier, one wavefront's loads for the last rows would queue in front of another's loads for the first.  (One
+  // barrier: more of them, a finer order, cost more than the order gains - a round of one load per wavefront with a
+  // barrier takes 0.1 to 0.2 us.)
+  load_patch(0, p.first_loads);
+  __builtin_amdgcn_s_barrier();
+  load_patch(p.first_loads, p.patch_loads);
+  // how many of this wavefront's patch loads lie below load number x
+  auto mine_below = [&](int x) -> int { return x > wave ? (x - wave + kStreamWaves - 1) / kStreamWaves : 0; };
+
+  // ---- addresses
+  const int frag_kg = ((lane >> 4) & 1) * 2 + (lane >> 5);  // k chunks 0, 2, 1, 3 for the lane groups 0..3
+  const int px      = lane & 15;
+  const int g       = lane >> 4;
+  // position of this lane's pixel of step s in the patch (tap (0, 0), K slice 0); lanes beyond the band read position 0
+  const char* a_pos[kStreamSteps];
+#pragma unroll
+  for (int s = 0; s < kStreamSteps; ++s) {
+    const int pix = 16 * (4 * s + pg) + px;
+    const int ly  = (int)(((uint64_t)(unsigned)pix * p.w_magic) >> p.w_shift);
+    const int pos = pix < npix ? ly * PW + (pix - ly * W) : 0;
+    a_pos[s]      = patch + pos * kPitch + frag_kg * 16;
+  }
+  const int row_pitch = PW * kPitch;
+  // filter fragment of tile j (rows 32 half + 8 g' + 4 j + r', q = lane & 15 = 4 g' + r'), K slice kk: in stage 0, and
+  // where the ninth stage has it
+  const char* b_base[2][2];
+  const char* b_last[2][2];
+  {
+    const int q = lane & 15;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int row = 32 * half + 8 * (q >> 2) + 4 * j + (q & 3);
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        b_base[kk][j] = filt + row * 128 + (((kk * 4 + frag_kg) ^ FilterKey(row)) << 4);
+        const int d   = 8 * row + kk * 4 + frag_kg;
+        b_last[kk][j] = patch + (d >> 1) * kPitch + 128 + (d & 1) * 16;
+      }
+    }
+  }
+  // this lane's first output element: pixel 16 pg + px of the band, channels n0 + 32 half + 8 g ..
+  const int oc0 = n0 + 32 * half + 8 * g;
+  T* const Y       = reinterpret_cast<T*>(p.y);
+  const T* const R = reinterpret_cast<const T*>(p.residual);
+  const int64_t out0 = (((int64_t)img * p.h + y0) * W + 16 * pg + px) * p.oc + oc0;
+
+  // ---- the filter and the rows that step 0 reads have landed (this wavefront's part: at most the patch loads it
+  // issued after them are in flight)
+  WaitLoadsInFlight(mine_below(p.patch_loads) - mine_below(p.first_loads));
+  BarrierLds();
+  PatchStamp(p.probe, wave == 0, 1);
+
+  vec8 bf[kTaps][2][2];
+  auto read_b = [&](int t, int kk, int j) -> vec8 {
+    return *reinterpret_cast<const vec8*>(t + 1 < kTaps ? b_base[kk][j] + t * kBTile : b_last[kk][j]);
+  };
+  auto read_a = [&](int s, int u) -> vec8 {  // pixel fragment u = 2 tap + kk of step s
+    const int tap = u >> 1, kk = u & 1;
+    return *reinterpret_cast<const vec8*>(a_pos[s] + (tap / 3) * row_pitch + (tap % 3) * kPitch + kk * 64);
+  };
+  float sc[8], sh[8];
+  // scale, shift, residual, relu, conversion: the arithmetic of PatchEpilogue
+  auto finish = [&](const f32x4 (&acc)[2], int s) -> u32x4 {
+    vec8 res = {};
+    const bool valid = 16 * (4 * s + pg) + px < npix;
+    if (R && valid) res = *reinterpret_cast<const vec8*>(R + out0 + (int64_t)s * 64 * p.oc);
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      v[e] = __builtin_fmaf(acc[e >> 2][e & 3], sc[e], sh[e]);
+      if (R) v[e] = __builtin_fmaf(p.residual_scale, (float)res[e], v[e]);
+      const float m = __builtin_fmaxf(v[e], 0.0f);
+      v[e]          = p.relu ? m : v[e];
+      asm volatile("" : "+v"(v[e]));
+    }
+    return u32x4{PackPair<T>(v[0], v[1]), PackPair<T>(v[2], v[3]), PackPair<T>(v[4], v[5]), PackPair<T>(v[6], v[7])};
+  };
+  auto store = [&](u32x4 out, int s) {
+    if (16 * (4 * s + pg) + px < npix) *reinterpret_cast<u32x4*>(Y + out0 + (int64_t)s * 64 * p.oc) = out;
+  };
+
+#define CINN_SB __builtin_amdgcn_sched_barrier(0)
+  constexpr int kFrags = 2 * kTaps;  // pixel fragments per tile
+  // Pixel fragments go through a ring of four register sets, requested three MFMA pairs ahead; fragment u of step s
+  // has the slot (kFrags s + u) % 4, so the ring runs on across the steps.  In step 0 the filter fragments of pair
+  // u + 2 are requested with them.
+  vec8 ar[4];
+  f32x4 acc[2];
+  u32x4 held;
+#pragma unroll
+  for (int s = 0; s < kStreamSteps; ++s) {
+    if (s == 1) {
+      // Everything else is waited for once, BEFORE the first store is issued: a wait is for "at most n operations in
+      // flight", loads or stores, and with stores among them it would wait for their acknowledgement (most of a
+      // microsecond) where it only needs the loads.  (Waits before each of the next steps, for just the rows they
+      // add, were measured: 14.5 us per launch against 13.5, for that reason.)
+      __builtin_amdgcn_s_waitcnt(CINN_VMCNT(0));  // all of this wavefront's patch loads have landed
+      BarrierLds();                               // ... and everyone else's
+      PatchStamp(p.probe, wave == 0, 3);
+      store(held, 0);
+    }
+    // the first fragments of a step are requested during the step before, except across that wait
+    if (s < 2) {
+#pragma unroll
+      for (int u = 0; u < 3; ++u) ar[(kFrags * s + u) & 3] = read_a(s, u);
+    }
+    if (s == 0) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) bf[u >> 1][u & 1][j] = read_b(u >> 1, u & 1, j);
+    }
+    acc[0] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    acc[1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int u = 0; u < kFrags; ++u) {
+      const int m = kFrags * s + u;
+      CINN_SB;
+      acc[0] = Mfma16<T>::mma(bf[u >> 1][u & 1][0], ar[m & 3], acc[0]);
+      CINN_SB;
+      if (u + 3 < kFrags) {
+        ar[(m + 3) & 3] = read_a(s, u + 3);
+      } else if (s >= 1 && s + 1 < kStreamSteps) {
+        ar[(m + 3) & 3] = read_a(s + 1, u + 3 - kFrags);
+      }
+      if (s == 0 && u + 2 < kFrags) {
+        bf[(u + 2) >> 1][(u + 2) & 1][0] = read_b((u + 2) >> 1, (u + 2) & 1, 0);
+        bf[(u + 2) >> 1][(u + 2) & 1][1] = read_b((u + 2) >> 1, (u + 2) & 1, 1);
+      }
+      CINN_SB;
+      acc[1] = Mfma16<T>::mma(bf[u >> 1][u & 1][1], ar[m & 3], acc[1]);
+      CINN_SB;
+    }
+    if (s == 0) {
+      const float* const tab = reinterpret_cast<const float*>(lds + kStreamScale);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float a = tab[32 * half + 8 * g + e], b = tab[64 + 32 * half + 8 * g + e];
+        sc[e] = p.scale ? a : p.alpha;
+        sh[e] = p.shift ? b : 0.0f;
+      }
+      held = finish(acc, 0);
+      PatchStamp(p.probe, wave == 0, 2);
+    } else {
+      store(finish(acc, s), s);
+      if (s == 3) PatchStamp(p.probe, wave == 0, 4);
+    }
+  }
+#undef CINN_SB
+  PatchStamp(p.probe, wave == 0, 5);
+}
+
 template <bool B>
 struct BoolTag {
   static constexpr bool value = B;
@@ -693,6 +953,30 @@ bool PlanFor(const ConvNhwcArgs& a, PatchPlan* plan) {
   return true;
 }
 
+// The streaming kernel's plan: the same bands; the patch must end below the filter stages, have the 256 positions
+// whose dummy slots carry the ninth stage, and the first loads - the rows that the band's first 64 pixels read, and
+// those positions - are the ones step 0 waits for.
+bool PlanStreamFor(const ConvNhwcArgs& a, PatchPlan* plan, int* first_loads) {
+  int rows = kCapacity / a.w_in;
+  if (rows < 1) return false;
+  rows            = rows < a.h ? rows : a.h;
+  const int bands = (a.h + rows - 1) / rows;
+  rows            = (a.h + bands - 1) / bands;
+  if ((int64_t)a.h * a.w_in * 5 < (int64_t)bands * kCapacity * 4) return false;
+  const int slots = (rows + 2) * (a.w_in + 2) * 10;
+  if (slots >= 65536) return false;
+  const int patch_loads = (slots + 63) / 64;
+  if (patch_loads * 1024 > kStreamFilter || patch_loads < kStreamLastLoads) return false;
+  const int npix     = rows * a.w_in;
+  const int last_row = ((npix < 64 ? npix : 64) - 1) / a.w_in;  // band row of the last pixel of step 0
+  const int need     = (last_row + 3) * (a.w_in + 2) * 10;      // slots of the patch rows 0 .. last_row + 2
+  int first          = (need + 63) / 64;
+  first              = first > kStreamLastLoads ? first : kStreamLastLoads;
+  *first_loads       = first < patch_loads ? first : patch_loads;
+  *plan = PatchPlan{rows, bands, patch_loads, kLdsLimit, 1};
+  return true;
+}
+
 // The same for more than 64 channels: bands of at most 64 TMW pixel slots (image rows padded to a multiple of 8
 // slots) and two patch buffers; rows are given up until
 // the buffers fit.  *per_step: patch loads per feeding wavefront and K step (2 or 3).  False when more than three tenths
@@ -755,6 +1039,33 @@ void Launch(const PatchParams& p, const PatchPlan& plan, hipStream_t stream) {
   hipLaunchKernelGGL(kernel, grid, dim3(128 * kWaves), plan.lds_bytes, stream, p);
 }
 
+template <typename T>
+void LaunchStream(const PatchParams& p, const PatchPlan& plan, hipStream_t stream) {
+  auto kernel = conv3x3_c64_stream_kernel<T>;
+  static const bool configured = [&] {  // once per instantiation, thread-safe
+    CINN_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit));
+    return true;
+  }();
+  (void)configured;
+  dim3 grid(p.n * p.bands, p.oc / 64);
+  hipLaunchKernelGGL(kernel, grid, dim3(64 * kStreamWaves), plan.lds_bytes, stream, p);
+}
+
+// 64 input channels: 1 = the streaming kernel (pixels outermost, filter in registers), 0 = the tap-major one; -1: not read
+std::atomic<int> g_patch_stream{-1};
+
+int PatchStream() {
+  int on = g_patch_stream.load(std::memory_order_relaxed);
+  if (on < 0) {
+    const char* v = getenv("FLAGS_cinn_hip_conv_patch_stream");
+    on            = v && *v ? (atoi(v) != 0) : 1;
+    g_patch_stream.store(on, std::memory_order_relaxed);
+  }
+  return on;
+}
+
+std::atomic<unsigned long long*> g_patch_probe{nullptr};
+
 // 0: never, 1: where it is expected to win, 2: wherever the shape qualifies; -1: not read yet
 std::atomic<int> g_patch_mode{-1};
 
@@ -801,6 +1112,8 @@ bool TryConvPatch(const ConvNhwcArgs& a, hipStream_t stream) {
   const bool chunked = a.c != 64;
   int per_step       = 0;
   int tiles          = 4;  // 16-slot tiles per computing wavefront of the chunked kernel
+  int first_loads    = 0;
+  bool streaming     = false;
   PatchPlan plan;
   if (chunked) {
     // Blocks of 256 pixel slots; when those leave most of the chip idle (256 -> 256 on 14x14 at batch 32: 128 blocks)
@@ -820,6 +1133,8 @@ bool TryConvPatch(const ConvNhwcArgs& a, hipStream_t stream) {
     } else if (!fits4) {
       return false;
     }
+  } else if (PatchStream() && PlanStreamFor(a, &plan, &first_loads)) {
+    streaming = true;
   } else if (!PlanFor(a, &plan)) {
     return false;
   }
@@ -836,6 +1151,8 @@ bool TryConvPatch(const ConvNhwcArgs& a, hipStream_t stream) {
   p.alpha = a.alpha, p.residual_scale = a.residual_scale, p.relu = a.relu ? 1 : 0;
   p.n = a.n, p.h = a.h, p.w_in = a.w_in, p.oc = a.oc, p.c = a.c;
   p.rows = plan.rows, p.bands = plan.bands, p.patch_loads = plan.patch_loads, p.stack = plan.stack;
+  p.first_loads = first_loads;
+  p.probe       = g_patch_probe.load(std::memory_order_relaxed);
   MagicFor(chunked ? (a.w_in + 7) & ~7 : a.w_in, &p.w_magic, &p.w_shift);
   MagicFor(a.w_in + 2, &p.pw_magic, &p.pw_shift);
   if (chunked && tiles == 2) {
@@ -856,6 +1173,12 @@ bool TryConvPatch(const ConvNhwcArgs& a, hipStream_t stream) {
     } else {
       LaunchChunks<_Float16, 4, 3>(p, plan, stream);
     }
+  } else if (streaming) {
+    if (is_bf16) {
+      LaunchStream<__bf16>(p, plan, stream);
+    } else {
+      LaunchStream<_Float16>(p, plan, stream);
+    }
   } else if (is_bf16) {
     Launch<__bf16>(p, plan, stream);
   } else {
@@ -874,6 +1197,16 @@ extern "C" int cinn_hip_conv_patch_loads_in_flight(int tap, int first_chunk, int
 extern "C" int cinn_hip_conv_patch_tiles(int tiles) {
   const int before = cinn_hip_kernels::PatchTiles();
   if (tiles == 0 || tiles == 2 || tiles == 4) cinn_hip_kernels::g_patch_tiles.store(tiles, std::memory_order_relaxed);
+  return before;
+}
+
+extern "C" void cinn_hip_conv_patch_set_probe(void* buffer) {
+  cinn_hip_kernels::g_patch_probe.store(static_cast<unsigned long long*>(buffer), std::memory_order_relaxed);
+}
+
+extern "C" int cinn_hip_conv_patch_stream(int on) {
+  const int before = cinn_hip_kernels::PatchStream();
+  if (on == 0 || on == 1) cinn_hip_kernels::g_patch_stream.store(on, std::memory_order_relaxed);
   return before;
 }
 

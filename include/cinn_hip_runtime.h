@@ -329,6 +329,11 @@ int cinn_hip_conv_patch_mode(int mode);
  * Returns the previous setting; another value only reads it.  Initial value from FLAGS_cinn_hip_conv_patch_tiles.
  * Atomic like the mode above. */
 int cinn_hip_conv_patch_tiles(int tiles);
+/* The same kernel family for exactly 64 input channels: 1 = the form that walks the pixels in its outer loop with the
+ * whole filter in registers, so that a tile's results are stored while the next is multiplied (default), 0 = the form
+ * that walks the filter taps in its outer loop and stores at the end.  Both give the same bits.  Returns the previous
+ * setting; another value only reads it.  Initial value from FLAGS_cinn_hip_conv_patch_stream.  Atomic like the mode. */
+int cinn_hip_conv_patch_stream(int on);
 /* Device descriptor consumed by schedules.  Replaces common::Target's cudaDeviceGetAttribute
  * queries (cinn/common/target.cc:55-84, 177-221).  Filled from the live device when one is
  * present, otherwise with the MI355X datasheet values (256 CUs, wave64, 160 KiB LDS per CU). */

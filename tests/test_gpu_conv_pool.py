@@ -610,6 +610,15 @@ def test_convolution_with_the_input_patch_resident_in_lds(gpu, patch_kernel_ever
     other = call_conv_nhwc(x, w, 1, 1, 1, dtype)
     patch_kernel_everywhere.cinn_hip_conv_patch_mode(2)
     assert np.all(np.abs(got - other) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+    # the two forms of the kernel (pixels outermost with the filter in registers - the default - and taps outermost)
+    # add the same products in the same order: the same bits
+    patch_kernel_everywhere.cinn_hip_conv_patch_stream.argtypes = [ctypes.c_int]
+    before = patch_kernel_everywhere.cinn_hip_conv_patch_stream(0)
+    try:
+        tap_major = call_conv_nhwc(x, w, 1, 1, 1, dtype)
+    finally:
+        patch_kernel_everywhere.cinn_hip_conv_patch_stream(before)
+    assert before == 1 and np.array_equal(got, tap_major)
 
 
 PATCH_CHUNK_CASES = [
@@ -695,6 +704,13 @@ def test_patch_convolution_with_residual_epilogue(gpu, patch_kernel_everywhere):
     want = 0.5 * oracle.conv2d_nchw(x, w, (1, 1), (1, 1)).astype(np.float64) + 2.0 * y0
     scale = 0.5 * oracle.conv2d_nchw(np.abs(x), np.abs(w), (1, 1), (1, 1)) + 2.0 * np.abs(y0)
     assert np.all(np.abs(got - want) <= 2.0 ** -10 * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
+    patch_kernel_everywhere.cinn_hip_conv_patch_stream.argtypes = [ctypes.c_int]
+    before = patch_kernel_everywhere.cinn_hip_conv_patch_stream(0)
+    try:
+        tap_major = call_conv_nhwc(x, w, 1, 1, 1, "float16", alpha=0.5, beta=2.0, y_init=y0).astype(np.float64)
+    finally:
+        patch_kernel_everywhere.cinn_hip_conv_patch_stream(before)
+    assert np.array_equal(got, tap_major)
 
 
 STEM7_CASES = [
