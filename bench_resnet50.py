@@ -122,7 +122,8 @@ def roofline_of(comp, dtype):
     time of its operands (every argument tensor once, at 8 TB/s) and the matrix-core time of its multiply-adds at the
     dense peak of `dtype`, summed over the instructions (they run one after the other).  Multiply-adds are taken from
     the arguments of the instruction: a convolution or product call (x, w, ..., y) does numel(y) * numel(w) / w.shape[0]
-    of them (four times that when a 2x2-strided pooling is folded into it: y is then the pooled tensor)."""
+    of them (four times that when a 2x2-strided pooling is folded into it: y is then the pooled tensor), a call of two
+    1x1 convolutions in a row those of both."""
     from cinn_amd.common import np_dtype
     peak = MFMA_PEAK_FLOPS[dtype]
     total, rows = 0.0, []
@@ -131,7 +132,12 @@ def roofline_of(comp, dtype):
         tensors = {a: comp.get_tensor(a) for a in dict.fromkeys(args)}
         nbytes = sum(int(np.prod(t.shape(), dtype=np.int64)) * np_dtype(str(t.type())).itemsize for t in tensors.values())
         flop = 0
-        if "conv2d" in fn or "matmul" in fn or "mul" in fn.split("_"):
+        if "conv2d_bn_relu_chain" in fn:
+            # (x, w1, scale1, shift1, [residual,] w2, scale2, shift2, e, y): two 1x1 convolutions
+            x, w1, e, y = (tensors[args[j]].shape() for j in (0, 1, -2, -1))
+            pixels = int(np.prod(x[:-1], dtype=np.int64))
+            flop = 2 * pixels * (w1[-1] * e[-1] + e[-1] * y[-1])
+        elif "conv2d" in fn or "matmul" in fn or "mul" in fn.split("_"):
             x, w, y = tensors[args[0]].shape(), tensors[args[1]].shape(), tensors[args[-1]].shape()
             macs_per_output = int(np.prod(w, dtype=np.int64)) // w[0] if "conv2d" in fn else x[-1]
             outputs = int(np.prod(y, dtype=np.int64))

@@ -29,6 +29,9 @@ class CinnComputation {
     // `matmul(x, W) + bias` with a const 2-D W and a const bias in a 16-bit type: the bias is added in the product's
     // epilogue (frontend/layout_pass.h); the result differs from the two operators by one rounding
     bool fuse_matmul_bias{true};
+    // two folded 1x1 convolutions in a row whose channel counts the chain kernel takes become one call that writes
+    // both results (frontend/layout_pass.h); same results as the two calls
+    bool fuse_conv_chain{true};
     // move conv2d chains written in NCHW to channels-last tensors, the layout the MFMA convolution kernels read
     // with 16-byte accesses (frontend/layout_pass.h); off: every conv2d runs in the layout it was written in
     bool conv_layout_nhwc{true};

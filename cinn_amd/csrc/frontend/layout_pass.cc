@@ -2,10 +2,12 @@
 
 #include <algorithm>
 #include <map>
+#include <set>
 
 #include "cinn_hip_runtime.h"
 #include "frontend/pass_util.h"
 #include "hlir/op.h"
+#include "kernels/conv_chain.h"
 #include "kernels/stem_pool.h"
 
 namespace cinn {
@@ -452,6 +454,103 @@ Program FuseMatmulBias(const Program& program, const std::set<std::string>& fetc
     } else if (!dropped[i]) {
       out.push_back(instrs[i]);
     }
+  }
+  return Program(std::move(out), program.GetInputs(), program.name());
+}
+
+Program FuseConvChain(const Program& program, const std::set<std::string>& fetch_ids) {
+  (void)fetch_ids;  // both results of a pair stay outputs of the new call, fetched or not
+  const auto& instrs = program.instructions();
+  std::map<std::string, std::vector<size_t>> users;
+  for (size_t i = 0; i < instrs.size(); ++i)
+    for (auto& in : instrs[i]->inputs) users[in->id].push_back(i);
+  // a folded convolution that is a matrix product over the channels of each pixel
+  auto pointwise = [](const Instruction& ins) {
+    if (ins->op_type != "hip_conv2d_bn_relu" || ins->inputs.size() < 4) return false;
+    const auto& a = ins->attrs;
+    if (GetAttr<std::string>(a, "data_format", "NCHW") != "NHWC" || GetAttr<std::string>(a, "input_layout", "NHWC") != "NHWC") return false;
+    if (GetAttr<bool>(a, "max_pool", false) || GetAttr<int>(a, "groups", 1) != 1) return false;
+    if (GetAttr<std::vector<int>>(a, "stride", {1, 1}) != std::vector<int>{1, 1} ||
+        GetAttr<std::vector<int>>(a, "padding", {0, 0}) != std::vector<int>{0, 0} ||
+        GetAttr<std::vector<int>>(a, "dilation", {1, 1}) != std::vector<int>{1, 1})
+      return false;
+    const auto& x = ins->inputs[0];
+    const auto& w = ins->inputs[1];
+    if (x->shape.size() != 4 || w->shape.size() != 4 || w->shape[1] != 1 || w->shape[2] != 1 || w->shape[3] != x->shape[3]) return false;
+    return x->type.is_floating() && x->type.bits == 16 && w->type == x->type;
+  };
+  std::map<std::string, size_t> defined_at;
+  for (size_t i = 0; i < instrs.size(); ++i)
+    for (auto& o : instrs[i]->outputs) defined_at[o->id] = i;
+  std::vector<bool> dropped(instrs.size(), false);
+  // what is emitted in front of instruction i: hoisted parameter computations of the second convolution, then the call
+  std::map<size_t, std::vector<Instruction>> before;
+  for (size_t i = 0; i < instrs.size(); ++i) {
+    const auto& first = instrs[i];
+    if (dropped[i] || !pointwise(first)) continue;
+    const Variable& e = first->outputs[0];
+    auto it = users.find(e->id);
+    if (it == users.end()) continue;
+    std::vector<size_t> readers = it->second;
+    std::sort(readers.begin(), readers.end());
+    // the second convolution: the first reader of e that qualifies
+    size_t at = instrs.size();
+    for (size_t r : readers) {
+      const auto& c = instrs[r];
+      if (r <= i || dropped[r] || !pointwise(c) || c->inputs.size() != 4) continue;
+      if (!(c->inputs[0] == e) || c->inputs[1] == e || c->inputs[2] == e || c->inputs[3] == e) continue;
+      const int64_t m = static_cast<int64_t>(e->shape[0]) * e->shape[1] * e->shape[2];
+      if (!cinn_hip_kernels::ConvChainShape(m, first->inputs[0]->shape[3], e->shape[3], c->outputs[0]->shape[3])) continue;
+      at = r;
+      break;
+    }
+    if (at == instrs.size()) continue;
+    const auto& second = instrs[at];
+    // The call produces e, so it goes in front of e's earliest reader.  What the second convolution's filter, scale and
+    // shift are computed from between there and its own position comes along, provided none of it reads e.
+    const size_t where = readers.front();
+    if (where <= i || before.count(where)) continue;
+    std::set<size_t> hoist;
+    bool ok = true;
+    std::vector<Variable> work(second->inputs.begin() + 1, second->inputs.end());
+    while (ok && !work.empty()) {
+      Variable v = work.back();
+      work.pop_back();
+      auto def = defined_at.find(v->id);
+      if (def == defined_at.end() || def->second < where) continue;  // a program input, or ready in time
+      if (def->second >= at || dropped[def->second]) {
+        ok = false;
+        break;
+      }
+      if (!hoist.insert(def->second).second) continue;
+      for (auto& in : instrs[def->second]->inputs) {
+        if (in == e) ok = false;
+        work.push_back(in);
+      }
+    }
+    if (!ok) continue;
+    Instruction chain("hip_conv2d_bn_relu_chain");
+    chain->inputs = first->inputs;  // x, w1, scale1, shift1[, residual]
+    chain->inputs.insert(chain->inputs.end(), second->inputs.begin() + 1, second->inputs.end());
+    chain->outputs = {e, second->outputs[0]};
+    chain->attrs["relu"]       = GetAttr<bool>(first->attrs, "relu", false);
+    chain->attrs["relu_after"] = GetAttr<bool>(second->attrs, "relu", false);
+    std::vector<Instruction> seq;
+    for (size_t h : hoist) {
+      seq.push_back(instrs[h]);
+      dropped[h] = true;
+    }
+    seq.push_back(chain);
+    dropped[i]    = true;
+    dropped[at]   = true;
+    before[where] = seq;
+  }
+  if (before.empty()) return program;
+  std::vector<Instruction> out;
+  for (size_t i = 0; i < instrs.size(); ++i) {
+    auto it = before.find(i);
+    if (it != before.end()) out.insert(out.end(), it->second.begin(), it->second.end());
+    if (!dropped[i]) out.push_back(instrs[i]);
   }
   return Program(std::move(out), program.GetInputs(), program.name());
 }

@@ -34,6 +34,14 @@ Program PretransposeConstMatmulWeights(const Program& program);
 // bias in fp32 as shift - a classifier's bias then costs no kernel of its own.  The sum is rounded once, from the
 // fp32 accumulator plus bias, where the two operators round the product first.
 Program FuseMatmulBias(const Program& program, const std::set<std::string>& fetch_ids);
+// Two folded 1x1, stride 1, unpadded channels-last convolutions of which the second reads the first one's result
+// (the expansion that ends a ResNet bottleneck, with its shortcut and relu, and the reduction that starts the next):
+// one hip_conv2d_bn_relu_chain call with two outputs, when the kernel behind it takes the channel counts
+// (kernels/conv_chain.h).  The call is placed in front of the first result's earliest reader (a projection shortcut
+// may come before the reduction); the instructions that compute the second convolution's scale and shift move there
+// with it.  The first result stays an output - the next shortcut reads it - but is written once and not read back;
+// the results are those of the two calls.
+Program FuseConvChain(const Program& program, const std::set<std::string>& fetch_ids);
 
 }  // namespace frontend
 }  // namespace cinn

@@ -27,6 +27,17 @@ std::string CName(const std::string& id) {
   std::string out;
   for (char c : id) out.push_back((isalnum(static_cast<unsigned char>(c)) || c == '_') ? c : '_');
   if (out.empty() || isdigit(static_cast<unsigned char>(out[0]))) out = "v_" + out;
+  // a tensor may be named like a keyword or a built-in of the kernel language ("short", "float", "threadIdx"): as a
+  // parameter name that would not compile
+  static const std::set<std::string> reserved = {
+      "alignas", "alignof", "and", "asm", "auto", "bool", "break", "case", "catch", "char", "class", "const", "constexpr",
+      "continue", "default", "delete", "do", "double", "else", "enum", "explicit", "export", "extern", "false", "float", "for",
+      "friend", "goto", "if", "inline", "int", "long", "mutable", "namespace", "new", "not", "nullptr", "operator", "or",
+      "private", "protected", "public", "register", "return", "short", "signed", "sizeof", "static", "struct", "switch",
+      "template", "this", "throw", "true", "try", "typedef", "typename", "union", "unsigned", "using", "virtual", "void",
+      "volatile", "while", "xor", "half", "float16", "bfloat16", "threadIdx", "blockIdx", "blockDim", "gridDim", "warpSize",
+      "int8_t", "int16_t", "int32_t", "int64_t", "uint8_t", "uint16_t", "uint32_t", "uint64_t", "size_t", "min", "max"};
+  if (reserved.count(out)) out = "v_" + out;
   return out;
 }
 
@@ -1435,6 +1446,11 @@ ir::LoweredFuncRef OpLowerer::LowerLibraryCall(const Group& group) const {
     } else {
       push_ints({y[0], y[3], y[1], y[2]});
     }
+  } else if (op == "hip_conv2d_bn_relu_chain") {
+    api           = "cinn_call_hip_conv2d_bn_relu_chain";
+    const auto& x = n->inputs[0]->shape;
+    args.push_back(I32((GetAttr<bool>(n->attrs, "relu", false) ? 1 : 0) | (GetAttr<bool>(n->attrs, "relu_after", false) ? 2 : 0)));
+    push_ints({x[0], x[1], x[2], x[3], n->outputs[0]->shape[3], n->outputs[1]->shape[3]});
   } else if (op == "pool2d" || op == "pool2d_grad") {
     // argument list of CustomCallArgsForCudnnPoolForward / ...PoolBackward (custom_call.cc:520-640): the gradient
     // takes x, y and dy and passes the extents of x and y

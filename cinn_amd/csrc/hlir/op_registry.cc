@@ -639,6 +639,25 @@ OpRegistry::OpRegistry() {
     op.infer_dtype = SameTypeAsFirst;
   }
   {
+    // two 1x1 channels-last convolutions in a row, each with hip_conv2d_bn_relu's epilogue, produced by the
+    // FuseConvChain rewrite; inputs x, w1, scale1, shift1, [residual,] w2, scale2, shift2; outputs e (the first
+    // convolution's result) and y
+    auto& op       = r->Register("hip_conv2d_bn_relu_chain");
+    op.pattern     = OpPatternKind::kNonFusible;
+    op.num_inputs  = -1;
+    op.infer_shape = [](const std::vector<ShapeType>& in, const AttributeMap&) {
+      CINN_CHECK(in.size() == 7u || in.size() == 8u) << "hip_conv2d_bn_relu_chain takes 7 or 8 operands";
+      const size_t w2 = in.size() == 8u ? 5 : 4;
+      CINN_CHECK(in[0].size() == 4u && in[1].size() == 4u && in[w2].size() == 4u) << "hip_conv2d_bn_relu_chain: 4-D operands expected";
+      CINN_CHECK(in[1][1] == 1 && in[1][2] == 1 && in[w2][1] == 1 && in[w2][2] == 1 && in[1][3] == in[0][3] && in[w2][3] == in[1][0])
+          << "hip_conv2d_bn_relu_chain: [O][1][1][I] filters whose channel counts follow one another expected";
+      ShapeType e = {in[0][0], in[0][1], in[0][2], in[1][0]};
+      ShapeType y = {in[0][0], in[0][1], in[0][2], in[w2][0]};
+      return std::vector<ShapeType>{e, y};
+    };
+    op.infer_dtype = [](const std::vector<Type>& in, const AttributeMap&) { return std::vector<Type>{in[0], in[0]}; };
+  }
+  {
     // cinn/hlir/op/contrib/sort.cc:307-350: both keep the operand's shape; argsort has two int32 outputs (indices,
     // positions), sort one of the operand's type
     auto check_axis = [](const std::vector<ShapeType>& in, const AttributeMap& a) {

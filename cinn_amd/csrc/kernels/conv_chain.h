@@ -1,0 +1,12 @@
+// What the graph rewrite needs to know about the kernel that runs two 1x1 convolutions in a row (conv_chain_mfma.hip),
+// in plain integers so that host-only translation units can include it.
+#pragma once
+#include <cstdint>
+
+namespace cinn_hip_kernels {
+
+// True when one kernel computes e = act(x w1^T ...) [m][n1] and y = act(e w2^T ...) [m][n2] from x [m][k1] in a 16-bit
+// type: the channel counts it is instantiated for, m a multiple of 16.
+bool ConvChainShape(int64_t m, int k1, int n1, int n2);
+
+}  // namespace cinn_hip_kernels

@@ -427,4 +427,42 @@ void cinn_call_hip_conv2d_bn_relu(void* v_args, int num_args, int format, int re
           groups, output_n, output_c, output_h, output_w, static_cast<hipStream_t>(stream));
 }
 
+void cinn_call_hip_conv2d_bn_relu_chain(void* v_args, int num_args, int relu, int input_n, int input_h, int input_w,
+                                        int input_c, int middle_c, int output_c, void* stream) {
+  CINN_HIP_CLEAR_STALE_ERROR();
+  CINN_RT_CHECK(num_args == 9 || num_args == 10,
+                "cinn_call_hip_conv2d_bn_relu_chain takes x, w1, scale1, shift1, [residual], w2, scale2, shift2, e and y, "
+                "got %d arguments", num_args);
+  const int r = num_args == 10 ? 1 : 0;  // a residual shifts what follows it
+  cinn_buffer_t* x  = BufferArg(v_args, 0);
+  cinn_buffer_t* w1 = BufferArg(v_args, 1);
+  cinn_buffer_t* s1 = BufferArg(v_args, 2);
+  cinn_buffer_t* t1 = BufferArg(v_args, 3);
+  cinn_buffer_t* res = r ? BufferArg(v_args, 4) : nullptr;
+  cinn_buffer_t* w2 = BufferArg(v_args, 4 + r);
+  cinn_buffer_t* s2 = BufferArg(v_args, 5 + r);
+  cinn_buffer_t* t2 = BufferArg(v_args, 6 + r);
+  cinn_buffer_t* e  = BufferArg(v_args, 7 + r);
+  cinn_buffer_t* y  = BufferArg(v_args, 8 + r);
+  for (cinn_buffer_t* f : {s1, t1, s2, t2})
+    CINN_RT_CHECK(f->type.code == cinn_type_float && f->type.bits == 32, "cinn_call_hip_conv2d_bn_relu_chain: scale / shift must be fp32");
+  CINN_RT_CHECK(input_n > 0 && input_h > 0 && input_w > 0 && input_c > 0 && middle_c > 0 && output_c > 0,
+                "cinn_call_hip_conv2d_bn_relu_chain: extents must be positive");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  cinn_hip_kernels::ConvChainArgs a;
+  a.x = x->memory, a.w1 = w1->memory, a.scale1 = reinterpret_cast<const float*>(s1->memory);
+  a.shift1 = reinterpret_cast<const float*>(t1->memory), a.residual = res ? res->memory : nullptr, a.relu1 = (relu & 1) != 0;
+  a.e = e->memory, a.w2 = w2->memory, a.scale2 = reinterpret_cast<const float*>(s2->memory);
+  a.shift2 = reinterpret_cast<const float*>(t2->memory), a.relu2 = (relu & 2) != 0, a.y = y->memory;
+  a.m = (int64_t)input_n * input_h * input_w, a.k1 = input_c, a.n1 = middle_c, a.n2 = output_c, a.type = x->type;
+  const bool same_type = w1->type.code == x->type.code && w1->type.bits == x->type.bits && w2->type.code == x->type.code &&
+                         w2->type.bits == x->type.bits && e->type.bits == x->type.bits && y->type.bits == x->type.bits;
+  if (same_type && cinn_hip_kernels::TryConvChain(a, st)) return;
+  // any other shape or type: the two convolutions one after the other
+  RunConv(x, w1, e, a.scale1, a.shift1, res, a.relu1 ? 2 : 1, 1, 1.0f, 0.0f, input_n, input_c, input_h, input_w, middle_c, input_c,
+          1, 1, 0, 0, 1, 1, 1, 1, 1, input_n, middle_c, input_h, input_w, st);
+  RunConv(e, w2, y, a.scale2, a.shift2, nullptr, a.relu2 ? 2 : 1, 1, 1.0f, 0.0f, input_n, middle_c, input_h, input_w, output_c,
+          middle_c, 1, 1, 0, 0, 1, 1, 1, 1, 1, input_n, output_c, input_h, input_w, st);
+}
+
 }  // extern "C"

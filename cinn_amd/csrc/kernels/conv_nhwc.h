@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 
 #include "cinn_hip_runtime.h"
+#include "kernels/conv_chain.h"
 #include "runtime/scratch.h"
 
 namespace cinn_hip_kernels {
@@ -42,6 +43,28 @@ bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream);
 // rows fit LDS (conv_patch_mfma.hip): the input patch of a band of output rows stays resident in LDS, only the filter
 // streams; same epilogue.  false when the shape does not qualify.
 bool TryConvPatch(const ConvNhwcArgs& a, hipStream_t stream);
+// Two 1x1, stride 1, unpadded convolutions in a row on channels-last 16-bit tensors, seen as matrix products over the
+// m = N * H * W pixels: e = act1(x w1^T * scale1 + shift1 + residual) [m][n1], y = act2(e w2^T * scale2 + shift2)
+// [m][n2], with x [m][k1], w1 [n1][k1], w2 [n2][n1]; both e and y are written (conv_chain_mfma.hip).
+struct ConvChainArgs {
+  const void* x;
+  const void* w1;
+  const float* scale1;
+  const float* shift1;
+  const void* residual;  // may be null
+  bool relu1;
+  void* e;
+  const void* w2;
+  const float* scale2;
+  const float* shift2;
+  bool relu2;
+  void* y;
+  int64_t m;
+  int k1, n1, n2;
+  cinn_type_t type;
+};
+// false when the shape or the types do not qualify (the caller then runs the two convolutions one after the other)
+bool TryConvChain(const ConvChainArgs& a, hipStream_t stream);
 // 256 bytes of zeros in device memory (what masked-out chunks are read from)
 inline const void* ConvZeroPage() { return ZeroPage(); }
 

@@ -174,6 +174,20 @@ void cinn_call_hip_conv2d_bn_relu(void* v_args, int num_args, int format, int re
                                   int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
                                   int groups, int output_n, int output_c, int output_h, int output_w, void* stream);
 
+/* Extension with no counterpart in the reference (there every convolution is one cudnnConvolutionForward,
+ * cinn/runtime/cuda/cuda_util.cc:603-720): two 1x1, stride 1, unpadded channels-last convolutions in a row, each with the
+ * epilogue of cinn_call_hip_conv2d_bn_relu, where the first one's result is wanted as well -
+ *   e = act1(conv(x, w1) * scale1 + shift1 [+ residual])   [n][h][w][middle_c]
+ *   y = act2(conv(e, w2) * scale2 + shift2)                [n][h][w][output_c]
+ * v_args = {x, w1, scale1, shift1, [residual,] w2, scale2, shift2, e, y}; x is [n][h][w][input_c], w1
+ * [middle_c][1][1][input_c], w2 [output_c][1][1][middle_c], scales / shifts fp32.  relu: bit 0 = ReLU in act1, bit 1 = in
+ * act2.  For 16-bit types and the channel counts 64 -> 256 -> 64 | 128 (n h w a multiple of 16) one kernel computes
+ * both and e is never read back; any other shape runs the two convolutions one after the other,
+ * with the same results as two cinn_call_hip_conv2d_bn_relu calls.  The graph rewrite that emits this call
+ * (FuseConvChain) only does so for shapes of the first kind. */
+void cinn_call_hip_conv2d_bn_relu_chain(void* v_args, int num_args, int relu, int input_n, int input_h, int input_w,
+                                        int input_c, int middle_c, int output_c, void* stream);
+
 /* cinn_call_cudnn_conv2d_forward for callers that cannot allocate.  No counterpart in the reference: it exists for
  * code that runs under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  Same arguments and
  * results as the call above for format 1 and 2 with groups == 1 (always on the general channels-last MFMA kernel);
@@ -334,6 +348,10 @@ int cinn_hip_conv_patch_tiles(int tiles);
  * that walks the filter taps in its outer loop and stores at the end.  Both give the same bits.  Returns the previous
  * setting; another value only reads it.  Initial value from FLAGS_cinn_hip_conv_patch_stream.  Atomic like the mode. */
 int cinn_hip_conv_patch_stream(int on);
+/* cinn_call_hip_conv2d_bn_relu_chain: 1 = one kernel where the shape qualifies (default; initial value from
+ * FLAGS_cinn_hip_conv_chain), 0 = always the two convolutions one after the other.  Returns the previous setting;
+ * another value only reads it.  Atomic like the mode. */
+int cinn_hip_conv_chain_mode(int mode);
 /* Device descriptor consumed by schedules.  Replaces common::Target's cudaDeviceGetAttribute
  * queries (cinn/common/target.cc:55-84, 177-221).  Filled from the live device when one is
  * present, otherwise with the MI355X datasheet values (256 CUs, wave64, 160 KiB LDS per CU). */
