@@ -88,15 +88,19 @@ def test_resnet50_fp16_batch2_matches_oracle(gpu):
     assert_logits_close_fp16(got, want)
     fused, comp = gpu_forward(params, x, fuse_conv_bn_relu=True)
     # every batch norm, residual addition and relu now lives in a convolution epilogue, and the max pooling in the
-    # image convolution: 53 convolutions, the global pooling, the classifier with its bias as the shift of its epilogue
-    # (the reshapes around it are views)
-    assert comp.num_instructions() == 53 + 1 + 1, comp.fusion_groups()
+    # image convolution: 53 convolutions - three pairs of them (an expansion 64 -> 256 and the reduction that reads it)
+    # in one call each -, the global pooling, the classifier with its bias as the shift of its epilogue (the reshapes
+    # around it are views)
+    assert comp.num_instructions() == 50 + 1 + 1, comp.fusion_groups()
     assert_logits_close_fp16(fused, want)
+    one_call_per_layer, comp = gpu_forward(params, x, fuse_conv_chain=False)
+    assert comp.num_instructions() == 53 + 1 + 1, comp.fusion_groups()
+    assert_logits_close_fp16(one_call_per_layer, want)
     apart, comp = gpu_forward(params, x, fuse_stem_pool=False)
-    assert comp.num_instructions() == 53 + 2 + 1
+    assert comp.num_instructions() == 50 + 2 + 1
     assert np.array_equal(apart, fused)
     two_ops, comp = gpu_forward(params, x, fuse_matmul_bias=False)
-    assert comp.num_instructions() == 53 + 1 + 2
+    assert comp.num_instructions() == 50 + 1 + 2
     assert_logits_close_fp16(two_ops, want)
 
 
