@@ -465,3 +465,74 @@ def test_bias_after_a_matmul_with_const_weights_is_folded_into_the_product():
         b, y = _classifier(dtype, **kwargs)
         text = compile_only(b, [y], **opts).fusion_groups()
         assert "hip_conv2d_bn_relu" not in text and "matmul" in text, (kwargs, opts, text)
+
+
+def _bottleneck_pair(builder, side_reader):
+    """A projection shortcut 64 -> 256, an expansion 64 -> 256 that takes it, then the reduction 256 -> 64 of the next
+    block (fp16, const parameters): what FuseConvChain turns into one call."""
+    t = Float(16)
+
+    def const(name, shape):
+        v = builder.create_input(t, shape, name)
+        v.set_const()
+        return v
+
+    def bn(y, p, c):
+        return builder.batchnorm(y, const(p + "_g", [c]), const(p + "_b", [c]), const(p + "_m", [c]), const(p + "_v", [c]),
+                                 epsilon=1e-5)[0]
+
+    x = builder.create_input(t, [2, 64, 28, 28], "x")
+    short = bn(builder.conv2d(x, const("w0", [256, 64, 1, 1])), "bn0", 256)
+    e = builder.relu(builder.add(bn(builder.conv2d(x, const("w1", [256, 64, 1, 1])), "bn1", 256), short))
+    side = builder.scale(e, 2.0) if side_reader else None
+    y = builder.relu(bn(builder.conv2d(e, const("w2", [64, 256, 1, 1])), "bn2", 64))
+    out = builder.relu(bn(builder.conv2d(y, const("w3", [64, 64, 3, 3]), paddings=[1, 1]), "bn3", 64))
+    return [out, e] + ([side] if side_reader else [])
+
+
+@pytest.mark.parametrize("side_reader", [False, True])
+def test_two_pointwise_convolutions_in_a_row_become_one_call(side_reader):
+    b = NetBuilder("pair")
+    comp = compile_only(b, _bottleneck_pair(b, side_reader))
+    groups = comp.fusion_groups().strip().splitlines()
+    chains = [i for i, g in enumerate(groups) if "hip_conv2d_bn_relu_chain" in g]
+    assert len(chains) == 1, groups
+    # inputs x, w1, scale1, shift1, shortcut, w2, scale2, shift2; two outputs
+    line = groups[chains[0]]
+    assert len(line.split(" in: ")[1].split(" out: ")[0].split()) == 8 and len(line.split(" out: ")[1].split()) == 2, line
+    if side_reader:
+        # the call produces the first result, so it comes before that result's other reader, and the second layer's
+        # scale / shift computations (const, pre-run) come before the call
+        first_out = line.split(" out: ")[1].split()[0]
+        readers = [i for i, g in enumerate(groups) if i != chains[0] and first_out in g.split(" in: ")[1].split(" out: ")[0].split()]
+        assert readers and min(readers) > chains[0], groups
+    b = NetBuilder("pair")
+    apart = compile_only(b, _bottleneck_pair(b, side_reader), fuse_conv_chain=0)
+    assert "hip_conv2d_bn_relu_chain" not in apart.fusion_groups()
+    assert apart.num_instructions() == comp.num_instructions() + 1
+
+
+def test_pointwise_pairs_the_kernel_does_not_take_stay_two_calls():
+    t = Float(16)
+    b = NetBuilder("pair")
+    x = b.create_input(t, [2, 128, 28, 28], "x")   # 128 -> 512 -> 128: no one-kernel form
+    w1, w2 = b.create_input(t, [512, 128, 1, 1], "w1"), b.create_input(t, [128, 512, 1, 1], "w2")
+    params = []
+    for name, c in (("a", 512), ("b", 128)):
+        params.append([b.create_input(t, [c], "%s_%s" % (name, k)) for k in "gbmv"])
+    for v in [w1, w2] + params[0] + params[1]:
+        v.set_const()
+    e = b.relu(b.batchnorm(b.conv2d(x, w1), *params[0], epsilon=1e-5)[0])
+    y = b.relu(b.batchnorm(b.conv2d(e, w2), *params[1], epsilon=1e-5)[0])
+    comp = compile_only(b, [y, e])
+    assert "chain" not in comp.fusion_groups() and comp.fusion_groups().count("hip_conv2d_bn_relu") == 2
+
+
+def test_tensor_names_that_are_keywords_of_the_kernel_language():
+    b = NetBuilder("kw")
+    a = b.create_input(Float(32), [4, 8], "short")
+    c = b.create_input(Float(32), [4, 8], "float")
+    comp = compile_only(b, [b.relu(b.add(a, c))])   # hiprtc compiles the generated source: "short" must not be a parameter name
+    src = comp.source_code()
+    assert "v_short" in src and "v_float" in src
+    assert comp.get_tensor("short") is not None
