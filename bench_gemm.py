@@ -6,7 +6,10 @@ median of three runs of 200 back-to-back launches after 30 ms of the same load (
 beside it `first_20_us`, the average of the first 20 launches after an idle period, which is what a short timing loop
 reads while the clock governor is still ramping.
     python bench_gemm.py --clock
-prints where the time of a 4096^3 launch goes, from time stamps the kernel writes itself (clock_probe).""" 
+prints where the time of a 4096^3 launch goes, from time stamps the kernel writes itself (clock_probe).
+    python bench_gemm.py --vendor
+times the vendor library (torch.mm -> hipBLASLt) on the same 4096^3 products with the same protocol, as a yardstick for
+what this machine gives a product of that size; the product path never calls it.""" 
 import ctypes
 import json
 import os
@@ -131,6 +134,42 @@ def clock_probe(stream, runtime, dtype="bfloat16", size=4096, launches=200):
                 first_start_to_last_end_us=round(float(wall[:, 3].max() - wall[:, 0].min()), 2), per_xcd=per_xcd)
 
 
+def vendor_yardstick(size=4096, launches=200, runs=3, warm_ms=30.0):
+    """torch.mm on bf16 / fp16 size^3 operands, B stored [K][N] (the benchmark's layout) and [N][K] (passed transposed):
+    30 ms of the same launches, then the median of three runs of 200 back-to-back launches between two events."""
+    import time
+
+    import torch
+    dev = torch.device("cuda:0")
+    out = {}
+    for dtype, tag in ((torch.bfloat16, "bf16"), (torch.float16, "fp16")):
+        a = (torch.randn(size, size, device=dev) * 0.02).to(dtype)
+        b = (torch.randn(size, size, device=dev) * 0.02).to(dtype)
+        c = torch.empty(size, size, device=dev, dtype=dtype)
+        for layout, rhs in (("b_stored_kn", b), ("b_stored_nk", b.t())):
+            torch.mm(a, rhs, out=c)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            while (time.perf_counter() - t0) * 1e3 < warm_ms:
+                for _ in range(20):
+                    torch.mm(a, rhs, out=c)
+                torch.cuda.synchronize()
+            times = []
+            for _ in range(runs):
+                s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                s.record()
+                for _ in range(launches):
+                    torch.mm(a, rhs, out=c)
+                e.record()
+                e.synchronize()
+                times.append(s.elapsed_time(e) / launches)
+            ms = sorted(times)[len(times) // 2]
+            tflops = 2 * size ** 3 / (ms * 1e-3) / 1e12
+            out["vendor_matmul_%s_%d_%s" % (tag, size, layout)] = dict(us=round(ms * 1e3, 2), TFLOPs=round(tflops, 1),
+                                                                      frac_of_mfma_peak=round(tflops / 2500.0, 4))
+    return out
+
+
 def cpu_baselines(budget_s=4.0):
     """The CPU oracle on bounded samples: the fp32 1024^3 product whole, and 256 rows of the 16-bit 4096^3 products
     (fp32 accumulation, one rounding at the end, as the GPU kernels do)."""
@@ -171,7 +210,9 @@ def cpu_baselines(budget_s=4.0):
 
 if __name__ == "__main__":
     from cinn_amd import runtime as rt
-    if "--clock" in sys.argv:
+    if "--vendor" in sys.argv:
+        print(json.dumps(vendor_yardstick()))
+    elif "--clock" in sys.argv:
         # python3 bench_gemm.py --clock : per-phase time stamps of the 4096^3 launches, bf16 and fp16
         st = rt.Stream()
         print(json.dumps([clock_probe(st, rt, dt) for dt in ("bfloat16", "float16")]))
