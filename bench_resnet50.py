@@ -123,7 +123,7 @@ def roofline_of(comp, dtype):
     dense peak of `dtype`, summed over the instructions (they run one after the other).  Multiply-adds are taken from
     the arguments of the instruction: a convolution or product call (x, w, ..., y) does numel(y) * numel(w) / w.shape[0]
     of them (four times that when a 2x2-strided pooling is folded into it: y is then the pooled tensor), a call of two
-    1x1 convolutions in a row those of both."""
+    1x1 convolutions in a row those of both, a 1x1 convolution over two inputs numel(y) times the channels of both."""
     from cinn_amd.common import np_dtype
     peak = MFMA_PEAK_FLOPS[dtype]
     total, rows = 0.0, []
@@ -137,6 +137,10 @@ def roofline_of(comp, dtype):
             x, w1, e, y = (tensors[args[j]].shape() for j in (0, 1, -2, -1))
             pixels = int(np.prod(x[:-1], dtype=np.int64))
             flop = 2 * pixels * (w1[-1] * e[-1] + e[-1] * y[-1])
+        elif "conv2d_pointwise_pair" in fn:
+            # (x, x2, w, shift, y): one 1x1 convolution over the channels of both inputs
+            w, y = tensors[args[2]].shape(), tensors[args[-1]].shape()
+            flop = 2 * int(np.prod(y, dtype=np.int64)) * w[-1]
         elif "conv2d" in fn or "matmul" in fn or "mul" in fn.split("_"):
             x, w, y = tensors[args[0]].shape(), tensors[args[1]].shape(), tensors[args[-1]].shape()
             macs_per_output = int(np.prod(w, dtype=np.int64)) // w[0] if "conv2d" in fn else x[-1]

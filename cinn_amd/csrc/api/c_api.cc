@@ -339,6 +339,8 @@ int cinn_amd_computation_build_and_compile(cinn_amd_builder_t b, const char* con
           opts.fuse_matmul_bias = v != 0;
         } else if (k == "fuse_conv_chain") {
           opts.fuse_conv_chain = v != 0;
+        } else if (k == "fuse_shortcut_projection") {
+          opts.fuse_shortcut_projection = v != 0;
         } else if (k == "reshape_as_view") {
           opts.reshape_as_view = v != 0;
         } else if (k == "merge_independent_kernels") {

@@ -46,6 +46,7 @@ std::shared_ptr<CinnComputation> CinnComputation::Compile(const common::Target& 
   if (options.fuse_conv_bn_relu) lowered = FuseConvBatchNorm(lowered, fetch_ids, options.fuse_stem_pool);
   if (options.fuse_matmul_bias) lowered = FuseMatmulBias(lowered, fetch_ids);
   if (options.fuse_conv_bn_relu && options.fuse_conv_chain) lowered = FuseConvChain(lowered, fetch_ids);
+  if (options.fuse_conv_bn_relu && options.fuse_shortcut_projection) lowered = FuseShortcutProjection(lowered, fetch_ids);
   if (options.use_decomposer) lowered = ApplyDecomposer(lowered);
   if (options.split_reductions) lowered = SplitReductions(lowered, target.get_multi_processor_count());
   comp->graph_    = std::make_shared<Graph>(lowered, fetch_ids, target);

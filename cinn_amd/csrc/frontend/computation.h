@@ -32,6 +32,10 @@ class CinnComputation {
     // two folded 1x1 convolutions in a row whose channel counts the chain kernel takes become one call that writes
     // both results (frontend/layout_pass.h); same results as the two calls
     bool fuse_conv_chain{true};
+    // a folded 1x1 convolution that adds a folded 1x1 projection of another tensor (a bottleneck block's last layer and
+    // its projection shortcut) becomes one call over both inputs, the batch-norm scales multiplied into the filters
+    // (needs fuse_conv_bn_relu)
+    bool fuse_shortcut_projection{true};
     // move conv2d chains written in NCHW to channels-last tensors, the layout the MFMA convolution kernels read
     // with 16-byte accesses (frontend/layout_pass.h); off: every conv2d runs in the layout it was written in
     bool conv_layout_nhwc{true};

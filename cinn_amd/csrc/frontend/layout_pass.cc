@@ -555,5 +555,81 @@ Program FuseConvChain(const Program& program, const std::set<std::string>& fetch
   return Program(std::move(out), program.GetInputs(), program.name());
 }
 
+Program FuseShortcutProjection(const Program& program, const std::set<std::string>& fetch_ids) {
+  const auto& instrs = program.instructions();
+  std::map<std::string, std::vector<size_t>> users;
+  for (size_t i = 0; i < instrs.size(); ++i)
+    for (auto& in : instrs[i]->inputs) users[in->id].push_back(i);
+  std::map<std::string, size_t> defined_at;
+  for (size_t i = 0; i < instrs.size(); ++i)
+    for (auto& o : instrs[i]->outputs) defined_at[o->id] = i;
+  // a folded 1x1 convolution without padding or dilation on channels-last 16-bit tensors, at any stride
+  auto pointwise = [](const Instruction& ins) {
+    if (ins->op_type != "hip_conv2d_bn_relu" || ins->inputs.size() < 4) return false;
+    const auto& a = ins->attrs;
+    if (GetAttr<std::string>(a, "data_format", "NCHW") != "NHWC" || GetAttr<std::string>(a, "input_layout", "NHWC") != "NHWC") return false;
+    if (GetAttr<bool>(a, "max_pool", false) || GetAttr<int>(a, "groups", 1) != 1) return false;
+    if (GetAttr<std::vector<int>>(a, "padding", {0, 0}) != std::vector<int>{0, 0} ||
+        GetAttr<std::vector<int>>(a, "dilation", {1, 1}) != std::vector<int>{1, 1})
+      return false;
+    const auto& x = ins->inputs[0];
+    const auto& w = ins->inputs[1];
+    if (x->shape.size() != 4 || w->shape.size() != 4 || w->shape[1] != 1 || w->shape[2] != 1 || w->shape[3] != x->shape[3]) return false;
+    return x->type.is_floating() && x->type.bits == 16 && w->type == x->type;
+  };
+  std::vector<bool> dropped(instrs.size(), false);
+  std::map<size_t, std::vector<Instruction>> replacement;
+  int serial = 0;
+  for (size_t i = 0; i < instrs.size(); ++i) {
+    const auto& main = instrs[i];
+    if (!pointwise(main) || main->inputs.size() != 5) continue;
+    if (GetAttr<std::vector<int>>(main->attrs, "stride", {1, 1}) != std::vector<int>{1, 1}) continue;
+    const Variable& r = main->inputs[4];
+    auto def = defined_at.find(r->id);
+    if (def == defined_at.end() || def->second >= i || dropped[def->second]) continue;
+    const auto& proj = instrs[def->second];
+    if (!pointwise(proj) || proj->inputs.size() != 4 || GetAttr<bool>(proj->attrs, "relu", false)) continue;
+    // the projection's result feeds this addition and nothing else
+    auto ru = users.find(r->id);
+    if (fetch_ids.count(r->id) || ru == users.end() || ru->second.size() != 1) continue;
+    const Variable &x = main->inputs[0], &x2 = proj->inputs[0], &y = main->outputs[0];
+    if (x == r || !(x2->type == x->type) || r->shape != y->shape) continue;
+    auto stride2 = GetAttr<std::vector<int>>(proj->attrs, "stride", {1, 1});
+    if (stride2.size() != 2 || (x->shape[1] - 1) * stride2[0] >= x2->shape[1] || (x->shape[2] - 1) * stride2[1] >= x2->shape[2]) continue;
+    const int64_t m = static_cast<int64_t>(x->shape[0]) * x->shape[1] * x->shape[2];
+    if (!cinn_hip_kernels::ConvPairShape(m, x->shape[3], x2->shape[3], y->shape[3])) continue;
+
+    // y = act(s1 (w1 x) + t1 + s2 (w2 x2) + t2) = act([s1 w1 | s2 w2] [x; x2] + (t1 + t2)): the scales go into the filters
+    // (multiplied in fp32, rounded once to the storage type), the filters side by side along their channels
+    std::vector<Instruction> seq;
+    Emitter e(&seq, "csp" + std::to_string(serial++) + "_");
+    const std::string store = x->type.is_bfloat16() ? "bfloat16" : "float16";
+    auto scaled = [&](const Variable& w, const Variable& s) {
+      auto w32 = e.Emit1("cast", {w}, {{"dtype", std::string("float32")}});
+      auto sb  = e.Emit1("broadcast_to", {s}, {{"out_shape", w->shape}, {"broadcast_axes", ShapeType{0}}});
+      auto ws  = e.Emit1("elementwise_mul", {w32, sb}, {{"axis", -1}});
+      return e.Emit1("cast", {ws}, {{"dtype", store}});
+    };
+    auto w_both = e.Emit1("concat", {scaled(main->inputs[1], main->inputs[2]), scaled(proj->inputs[1], proj->inputs[2])}, {{"axis", 3}});
+    auto shift  = e.Emit1("elementwise_add", {main->inputs[3], proj->inputs[3]}, {{"axis", -1}});
+    e.EmitInto(y, "hip_conv2d_pointwise_pair", {x, x2, w_both, shift},
+               {{"second_stride", stride2}, {"relu", GetAttr<bool>(main->attrs, "relu", false)}});
+    dropped[def->second] = true;
+    dropped[i]           = true;
+    replacement[i]       = seq;
+  }
+  if (replacement.empty()) return program;
+  std::vector<Instruction> out;
+  for (size_t i = 0; i < instrs.size(); ++i) {
+    auto it = replacement.find(i);
+    if (it != replacement.end()) {
+      out.insert(out.end(), it->second.begin(), it->second.end());
+    } else if (!dropped[i]) {
+      out.push_back(instrs[i]);
+    }
+  }
+  return Program(std::move(out), program.GetInputs(), program.name());
+}
+
 }  // namespace frontend
 }  // namespace cinn

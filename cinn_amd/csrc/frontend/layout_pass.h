@@ -43,5 +43,14 @@ Program FuseMatmulBias(const Program& program, const std::set<std::string>& fetc
 // the results are those of the two calls.
 Program FuseConvChain(const Program& program, const std::set<std::string>& fetch_ids);
 
+// A folded 1x1 convolution whose residual input is the result of a folded 1x1 projection (any stride, no relu, read by
+// nothing else) - the last layer of a bottleneck block and its projection shortcut - becomes one
+// hip_conv2d_pointwise_pair call over both inputs, when the kernel behind it takes the shape (kernels/conv_chain.h,
+// ConvPairShape): y = act(s1 (w1 x) + t1 + s2 (w2 x2) + t2) is computed as act([s1 w1 | s2 w2] [x; x2] + (t1 + t2)).
+// The scaled, concatenated filter and the summed shift are computed by ordinary instructions in front of the call
+// (from parameters alone, so they run once); the scales are multiplied in fp32 and the products rounded once to the
+// 16-bit storage type, which moves a result by at most one rounding of a filter value per term.
+Program FuseShortcutProjection(const Program& program, const std::set<std::string>& fetch_ids);
+
 }  // namespace frontend
 }  // namespace cinn

@@ -86,23 +86,39 @@ Graph::Graph(const frontend::Program& program, const std::set<std::string>& fetc
 // and its outputs are const.  Only fed inputs start const-ness here; a fill_constant joins the pre-run set when
 // a pre-run node consumes it, otherwise it stays with (and is folded into) its consumers.
 void Graph::ConstPropagate() {
-  for (auto& np : nodes_) {
-    Node* n = np.get();
-    if (n->op_type() == "fill_constant") continue;
-    // replicating a const value is left to the consumer, which reads the small tensor in place: materialising the
-    // replicated tensor once would turn a per-channel vector into a full activation-sized read in every execution
-    if (n->op->pattern == OpPatternKind::kBroadcast) continue;
-    bool all_const = !n->inputs.empty();
-    for (auto* in : n->inputs) {
-      bool literal = in->producer && in->producer->op_type() == "fill_constant";
-      all_const    = all_const && (in->is_const || literal);
+  auto known = [](const NodeData* in) {
+    return in->is_const || (in->producer && in->producer->op_type() == "fill_constant");
+  };
+  // Nodes are in program order, so one sweep settles everything but replications, which look at their consumers'
+  // other inputs: sweep until nothing changes.
+  for (bool changed = true; changed;) {
+    changed = false;
+    for (auto& np : nodes_) {
+      Node* n = np.get();
+      if (n->pre_run || n->op_type() == "fill_constant") continue;
+      bool all_const = !n->inputs.empty();
+      for (auto* in : n->inputs) all_const = all_const && known(in);
+      // something fed must take part: a chain of literals alone is folded, not pre-run
+      bool any_fed = false;
+      for (auto* in : n->inputs) any_fed = any_fed || in->is_const;
+      if (!all_const || !any_fed) continue;
+      if (n->op->pattern == OpPatternKind::kBroadcast) {
+        // Replicating a const value is left to the consumer, which reads the small tensor in place: materialising the
+        // replicated tensor once would turn a per-channel vector into a full activation-sized read in every execution.
+        // Unless every consumer is computed from const values alone (a scale multiplied into a filter): then the
+        // replication runs once with them.
+        bool only_const_consumers = !n->outputs.empty();
+        for (auto* o : n->outputs) {
+          only_const_consumers = only_const_consumers && !o->consumers.empty() && !o->is_fetch;
+          for (Node* c : o->consumers)
+            for (auto* in : c->inputs) only_const_consumers = only_const_consumers && (in == o || known(in));
+        }
+        if (!only_const_consumers) continue;
+      }
+      n->pre_run = true;
+      for (auto* o : n->outputs) o->is_const = true;
+      changed = true;
     }
-    // something fed must take part: a chain of literals alone is folded, not pre-run
-    bool any_fed = false;
-    for (auto* in : n->inputs) any_fed = any_fed || in->is_const;
-    if (!all_const || !any_fed) continue;
-    n->pre_run = true;
-    for (auto* o : n->outputs) o->is_const = true;
   }
   for (auto& np : nodes_) {
     Node* n = np.get();

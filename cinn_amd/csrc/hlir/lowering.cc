@@ -1451,6 +1451,13 @@ ir::LoweredFuncRef OpLowerer::LowerLibraryCall(const Group& group) const {
     const auto& x = n->inputs[0]->shape;
     args.push_back(I32((GetAttr<bool>(n->attrs, "relu", false) ? 1 : 0) | (GetAttr<bool>(n->attrs, "relu_after", false) ? 2 : 0)));
     push_ints({x[0], x[1], x[2], x[3], n->outputs[0]->shape[3], n->outputs[1]->shape[3]});
+  } else if (op == "hip_conv2d_pointwise_pair") {
+    api            = "cinn_call_hip_conv2d_pointwise_pair";
+    const auto& x  = n->inputs[0]->shape;
+    const auto& x2 = n->inputs[1]->shape;
+    auto stride2   = GetAttr<std::vector<int>>(n->attrs, "second_stride", {1, 1});
+    args.push_back(I32(GetAttr<bool>(n->attrs, "relu", false) ? 1 : 0));
+    push_ints({x[0], x[1], x[2], x[3], x2[1], x2[2], x2[3], stride2[0], stride2[1], n->outputs[0]->shape[3]});
   } else if (op == "pool2d" || op == "pool2d_grad") {
     // argument list of CustomCallArgsForCudnnPoolForward / ...PoolBackward (custom_call.cc:520-640): the gradient
     // takes x, y and dy and passes the extents of x and y

@@ -658,6 +658,27 @@ OpRegistry::OpRegistry() {
     op.infer_dtype = [](const std::vector<Type>& in, const AttributeMap&) { return std::vector<Type>{in[0], in[0]}; };
   }
   {
+    // a 1x1 channels-last convolution over the channels of two inputs that share the output's pixel grid (the second
+    // one sampled at `second_stride`), produced by the FuseShortcutProjection rewrite; inputs x, x2, w
+    // [O][1][1][C1 + C2], shift [O]
+    auto& op       = r->Register("hip_conv2d_pointwise_pair");
+    op.pattern     = OpPatternKind::kNonFusible;
+    op.num_inputs  = 4;
+    op.infer_shape = [](const std::vector<ShapeType>& in, const AttributeMap& a) {
+      CINN_CHECK_EQ(in.size(), 4u) << "hip_conv2d_pointwise_pair takes x, x2, w and shift";
+      CINN_CHECK(in[0].size() == 4u && in[1].size() == 4u && in[2].size() == 4u && in[3].size() == 1u)
+          << "hip_conv2d_pointwise_pair: 4-D tensors and a 1-D shift expected";
+      auto stride = GetAttr<std::vector<int>>(a, "second_stride", {1, 1});
+      CINN_CHECK(stride.size() == 2u && stride[0] > 0 && stride[1] > 0) << "hip_conv2d_pointwise_pair: second_stride takes two positive values";
+      CINN_CHECK(in[2][1] == 1 && in[2][2] == 1 && in[2][3] == in[0][3] + in[1][3] && in[3][0] == in[2][0] && in[1][0] == in[0][0])
+          << "hip_conv2d_pointwise_pair: a [O][1][1][C1 + C2] filter, an [O] shift and inputs of one batch size expected";
+      CINN_CHECK((in[0][1] - 1) * stride[0] < in[1][1] && (in[0][2] - 1) * stride[1] < in[1][2])
+          << "hip_conv2d_pointwise_pair: the output grid at the second input's stride leaves that input";
+      return std::vector<ShapeType>{{in[0][0], in[0][1], in[0][2], in[2][0]}};
+    };
+    op.infer_dtype = SameTypeAsFirst;
+  }
+  {
     // cinn/hlir/op/contrib/sort.cc:307-350: both keep the operand's shape; argsort has two int32 outputs (indices,
     // positions), sort one of the operand's type
     auto check_axis = [](const std::vector<ShapeType>& in, const AttributeMap& a) {

@@ -9,4 +9,9 @@ namespace cinn_hip_kernels {
 // type: the channel counts it is instantiated for, m a multiple of 16.
 bool ConvChainShape(int64_t m, int k1, int n1, int n2);
 
+// True when the implicit-GEMM kernels (gemm_mfma.hip) compute a 1x1 convolution over two channels-last 16-bit inputs
+// that share the output's pixel grid - y = act([x | x2] w^T + shift) with x [m][c1], x2 read at a stride, w [oc][c1 + c2]
+// - in one launch: both channel counts multiples of the 64-deep K step and enough output tiles to fill the chip.
+bool ConvPairShape(int64_t m, int c1, int c2, int oc);
+
 }  // namespace cinn_hip_kernels

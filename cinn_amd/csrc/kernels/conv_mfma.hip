@@ -465,4 +465,43 @@ void cinn_call_hip_conv2d_bn_relu_chain(void* v_args, int num_args, int relu, in
           middle_c, 1, 1, 0, 0, 1, 1, 1, 1, 1, input_n, output_c, input_h, input_w, st);
 }
 
+void cinn_call_hip_conv2d_pointwise_pair(void* v_args, int num_args, int relu, int input_n, int input_h, int input_w,
+                                         int input_c, int second_h, int second_w, int second_c, int second_stride_h,
+                                         int second_stride_w, int output_c, void* stream) {
+  CINN_HIP_CLEAR_STALE_ERROR();
+  CINN_RT_CHECK(num_args == 5, "cinn_call_hip_conv2d_pointwise_pair takes x, x2, w, shift and y, got %d arguments", num_args);
+  cinn_buffer_t* x     = BufferArg(v_args, 0);
+  cinn_buffer_t* x2    = BufferArg(v_args, 1);
+  cinn_buffer_t* w     = BufferArg(v_args, 2);
+  cinn_buffer_t* shift = BufferArg(v_args, 3);
+  cinn_buffer_t* y     = BufferArg(v_args, 4);
+  CINN_RT_CHECK(shift->type.code == cinn_type_float && shift->type.bits == 32, "cinn_call_hip_conv2d_pointwise_pair: shift must be fp32");
+  const bool is_16 = x->type.bits == 16 && (x->type.code == cinn_type_float || x->type.code == cinn_type_bfloat);
+  for (cinn_buffer_t* b : {x2, w, y})
+    CINN_RT_CHECK(is_16 && b->type.code == x->type.code && b->type.bits == x->type.bits,
+                  "cinn_call_hip_conv2d_pointwise_pair: x, x2, w and y must share one 16-bit floating-point type");
+  CINN_RT_CHECK(input_n > 0 && input_h > 0 && input_w > 0 && input_c > 0 && second_h > 0 && second_w > 0 && second_c > 0 &&
+                    second_stride_h > 0 && second_stride_w > 0 && output_c > 0,
+                "cinn_call_hip_conv2d_pointwise_pair: extents and strides must be positive");
+  CINN_RT_CHECK((input_h - 1) * second_stride_h < second_h && (input_w - 1) * second_stride_w < second_w,
+                "cinn_call_hip_conv2d_pointwise_pair: a %dx%d grid at stride %dx%d does not fit the second input's %dx%d pixels",
+                input_h, input_w, second_stride_h, second_stride_w, second_h, second_w);
+  const int64_t m = (int64_t)input_n * input_h * input_w;
+  CINN_RT_CHECK(cinn_hip_kernels::ConvPairShape(m, input_c, second_c, output_c),
+                "cinn_call_hip_conv2d_pointwise_pair: no kernel for %lld pixels, %d + %d -> %d channels (ConvPairShape)",
+                (long long)m, input_c, second_c, output_c);
+  cinn_hip_kernels::ConvNhwcArgs a;
+  a.x = x->memory, a.w = w->memory, a.y = y->memory;
+  a.scale = nullptr, a.shift = reinterpret_cast<const float*>(shift->memory);
+  a.residual = nullptr, a.alpha = 1.0f, a.residual_scale = 0.0f;
+  a.relu = (relu & 1) != 0, a.nchw_input = false;
+  a.n = input_n, a.h = input_h, a.w_in = input_w, a.c = input_c;
+  a.oc = output_c, a.kh = 1, a.kw = 1, a.oh = input_h, a.ow = input_w;
+  a.pad_h = a.pad_w = 0, a.stride_h = a.stride_w = a.dil_h = a.dil_w = 1;
+  a.type = x->type;
+  a.x2 = x2->memory, a.h2 = second_h, a.w2 = second_w, a.c2 = second_c;
+  a.stride2_h = second_stride_h, a.stride2_w = second_stride_w;
+  cinn_hip_kernels::RunConvNhwc(a, static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

@@ -28,6 +28,12 @@ struct ConvNhwcArgs {
   int oh, ow;
   int pad_h, pad_w, stride_h, stride_w, dil_h, dil_w;
   cinn_type_t type;  // element type of x, w, y and residual
+  // A second channels-last input [N][h2][w2][c2] read through a 1x1 window on the output's pixel grid, or null:
+  //   y[n, oy, ox, :] = act(conv(x, w[:, :kh kw c]) + w[:, kh kw c:] x2[n, oy stride2_h, ox stride2_w, :] + ...)
+  // The filter rows are then [kh][kw][c] followed by c2 more values.  Only the implicit-GEMM kernels take it
+  // (TryPointwiseConvAsGemm; ConvPairShape says for which shapes).
+  const void* x2 = nullptr;
+  int h2 = 0, w2 = 0, c2 = 0, stride2_h = 1, stride2_w = 1;
 };
 
 // true when the channels-last kernels can run this convolution (groups are not supported; the general path needs

@@ -688,6 +688,12 @@ void RunConvNhwc(const ConvNhwcArgs& a, hipStream_t stream) {
   CINN_RT_CHECK(ConvNhwcSupported(a), "conv2d (channels-last): unsupported type or channel count %d", a.c);
   CINN_RT_CHECK((int64_t)a.n * a.h * a.w_in * a.c < INT_MAX && (int64_t)a.n * a.oh * a.ow * a.oc < INT_MAX,
                 "conv2d (channels-last): tensor too large for 32-bit offsets");
+  if (a.x2 != nullptr) {
+    CINN_RT_CHECK(TryPointwiseConvAsGemm(a, stream),
+                  "conv2d (channels-last): no kernel takes a second input for this shape (%d pixels, %d + %d -> %d channels)",
+                  a.n * a.oh * a.ow, a.kh * a.kw * a.c, a.c2, a.oc);
+    return;
+  }
   if (TryConvStem7(a, stream)) return;
   CINN_RT_CHECK(!a.pool_after, "conv2d: only the 7x7 / stride 2 image convolution in a 16-bit type takes a fused max pooling");
   if (ConvStemSupported(a)) {

@@ -343,6 +343,12 @@ struct ConvGeom {
   int kw;               // filter width (dy = tap / kw)
   int stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
   const void* zero_page;  // at least 128 bytes of zeros
+  // A second channels-last input read through a 1x1 window (no padding) on the same output grid, or null: after the
+  // first steps1 K steps (all taps and channels of the first input) the K loop goes on over its c2 channels, pixel
+  // (oy stride2_h, ox stride2_w) for output pixel (oy, ox); the filter rows are [first input's K | c2] accordingly.
+  const void* x2;
+  int h2, w2, c2, stride2_h, stride2_w;
+  int steps1;
 };
 
 // BM x BN block tile on a WAVES_M x WAVES_N grid of wavefronts: 256x256 on 2x4 (8 wavefronts of 128x64) for large
@@ -353,7 +359,9 @@ struct ConvGeom {
 // wavefront per SIMD nobody else is there to issue MFMAs meanwhile: measured on the 128x128 tile (four stages,
 // implicit GEMM, K = 4608) a K step took 1102 clocks for 512 of MFMA with the loads issued by the computing
 // wavefronts and 531 without any loads.
-template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false, int NS = 2, bool FEED = false>
+// PAIR (with CONV): the convolution has a second input (ConvGeom::x2) whose channels continue the K loop.
+template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false, int NS = 2, bool FEED = false,
+          bool PAIR = false>
 __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N * (FEED ? 2 : 1))
 gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B, uint16_t* C, int M, int N, int K,
                   int64_t lda, int64_t ldb, int64_t ldc, DmaEpilogue epi, int64_t stride_a, int64_t stride_b,
@@ -372,8 +380,12 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   constexpr int LPB     = BN / 8 / LW;
   static_assert(LPA >= 1 && LPB >= 1 && LPA <= 8 && LPB <= 8 && TM % 4 == 0 && TN == 4, "unsupported tile shape");
   constexpr int STAGE = A_TILE + B_TILE;
-  static_assert(NS >= 2 && NS * STAGE <= 160 * 1024, "the stages do not fit LDS");
-  __shared__ __attribute__((aligned(1024))) char lds[NS * STAGE];
+  // PAIR: behind the stages, every thread parks its offsets into the second input until the K loop gets there
+  // (registers are what the 256x256 tile has none left of)
+  constexpr int STASH = PAIR ? THREADS * LPA * 8 : 0;
+  static_assert(!PAIR || CONV, "a second input belongs to a convolution");
+  static_assert(NS >= 2 && NS * STAGE + STASH <= 160 * 1024, "the stages do not fit LDS");
+  __shared__ __attribute__((aligned(1024))) char lds[NS * STAGE + STASH];
   const unsigned lds_addr =
       __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) char*)lds);
   // stage s lives in slot s % NS
@@ -428,6 +440,12 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   // CONV: a_off is the byte offset of the lane's chunk at the top-left corner of the pixel's window (it may lie before
   // the image: the tap's offset is added modulo 2^32), a_yx that corner's coordinates, 16 bits each
   int a_yx[LPA];
+  // CONV: the input the loads are reading (the second one of a pair takes over after geom.steps1 steps), and the
+  // lane's offsets and window corners in the second input
+  const char* src = reinterpret_cast<const char*>(A);
+  int src_h = geom.h, src_w = geom.w, src_c = geom.c;
+  int steps_to_switch = PAIR ? geom.steps1 : -1;
+  unsigned* const stash = reinterpret_cast<unsigned*>(lds + NS * STAGE) + tid;  // word i of a thread: stash[i THREADS]
 #pragma unroll
   for (int t = 0; t < LPA; ++t) {
     const int row = 8 * (lwave * LPA + t) + (lane >> 3);
@@ -443,6 +461,12 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
       // a pixel beyond the last one gets a window that starts far above the image: every tap reads zeros
       a_yx[t]         = pixel < M ? (iy0 & 0xffff) | (ix0 << 16) : 0x8000;
       a_off[t]        = ((unsigned)((n * geom.h + iy0) * geom.w + ix0) * (unsigned)geom.c + (((lane & 7) ^ key) << 3)) * 2u;
+      if (PAIR) {
+        const int iy2 = oy * geom.stride2_h;
+        const int ix2 = ox * geom.stride2_w;
+        stash[(2 * t) * THREADS]     = pixel < M ? (iy2 & 0xffff) | (ix2 << 16) : 0x8000;
+        stash[(2 * t + 1) * THREADS] = ((unsigned)((n * geom.h2 + iy2) * geom.w2 + ix2) * (unsigned)geom.c2 + (((lane & 7) ^ key) << 3)) * 2u;
+      }
     } else {
       const int row_c = row < a_last ? row : a_last;
       a_off[t] = (unsigned)(((int64_t)row_c * lda + (((lane & 7) ^ key) << 3)) * 2 + kBias - 1024 * (t & 3));
@@ -460,11 +484,21 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
   }
   auto advance_tap = [&]() {
     tap_c0 += kD64BK;
-    if (tap_c0 == geom.c) {
+    if (tap_c0 == src_c) {
       tap_c0 = 0;
       if (++tap_dx == geom.kw) {
         tap_dx = 0;
         ++tap_dy;
+      }
+    }
+    if (PAIR && --steps_to_switch == 0) {  // the first input is through: the second one's single tap follows
+      src   = static_cast<const char*>(geom.x2);
+      src_h = geom.h2, src_w = geom.w2, src_c = geom.c2;
+      tap_dy = tap_dx = tap_c0 = 0;
+#pragma unroll
+      for (int t = 0; t < LPA; ++t) {
+        a_yx[t]  = (int)stash[(2 * t) * THREADS];
+        a_off[t] = stash[(2 * t + 1) * THREADS];
       }
     }
   };
@@ -491,13 +525,13 @@ gemm16_dma_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B
       if (CONV) {
         const int iy      = (short)(a_yx[t] & 0xffff) + tap_dy * geom.dil_h;
         const int ix      = (a_yx[t] >> 16) + tap_dx * geom.dil_w;
-        const bool inside = (unsigned)iy < (unsigned)geom.h && (unsigned)ix < (unsigned)geom.w;
+        const bool inside = (unsigned)iy < (unsigned)src_h && (unsigned)ix < (unsigned)src_w;
         // the tap's offset is uniform: ((dy dil_h) w + dx dil_w) c + c0 elements
         const unsigned tap_off =
-            ((unsigned)((tap_dy * geom.dil_h) * geom.w + tap_dx * geom.dil_w) * (unsigned)geom.c + tap_c0) * 2u;
-        const char* src = inside ? reinterpret_cast<const char*>(A) + (a_off[t] + tap_off)
-                                 : static_cast<const char*>(geom.zero_page) + ((lane & 7) << 4);
-        AsyncCopy16To(src, lds_addr + (unsigned)(a_tile - lds) + (lwave * LPA + t) * 1024);
+            ((unsigned)((tap_dy * geom.dil_h) * src_w + tap_dx * geom.dil_w) * (unsigned)src_c + tap_c0) * 2u;
+        const char* from = inside ? src + (a_off[t] + tap_off)
+                                  : static_cast<const char*>(geom.zero_page) + ((lane & 7) << 4);
+        AsyncCopy16To(from, lds_addr + (unsigned)(a_tile - lds) + (lwave * LPA + t) * 1024);
       } else {
         SetLdsBase(lds_addr + (unsigned)(a_tile - lds) + (lwave * LPA + (t & ~3)) * 1024);
         AsyncCopy16Slot(a_base + (int64_t)kt * (kD64BK * 2), a_off[t], t & 3);
@@ -1604,7 +1638,8 @@ void XcdRectanglesPadded(int tiles_m, int tiles_n, int* xcd_cols, int* sub_rows,
 // device buffer of the time-stamp hook, or null (cinn_hip_gemm_set_probe)
 std::atomic<unsigned long long*> g_gemm_probe{nullptr};
 
-template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false, int NS = 2, bool FEED = false>
+template <typename T, bool B_KC, int BM, int BN, int WAVES_M, int WAVES_N, bool CONV = false, int NS = 2, bool FEED = false,
+          bool PAIR = false>
 void LaunchDma16(const GemmProblem& p, hipStream_t stream, int splits = 1) {
   int64_t ldb = p.trans_b ? p.k : p.n;
   const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
@@ -1632,7 +1667,7 @@ void LaunchDma16(const GemmProblem& p, hipStream_t stream, int splits = 1) {
   epi.streaming = !p.keep_in_cache && (int64_t)p.batch * p.m * p.n * 2 >= (16 << 20);
   ConvGeom geom{};
   if (CONV) geom = *p.conv;
-  hipLaunchKernelGGL((gemm16_dma_kernel<T, B_KC, BM, BN, WAVES_M, WAVES_N, CONV, NS, FEED>), grid,
+  hipLaunchKernelGGL((gemm16_dma_kernel<T, B_KC, BM, BN, WAVES_M, WAVES_N, CONV, NS, FEED, PAIR>), grid,
                      dim3(64 * WAVES_M * WAVES_N * (FEED ? 2 : 1)), 0,
                      stream, static_cast<const uint16_t*>(p.a), static_cast<const uint16_t*>(p.b),
                      static_cast<uint16_t*>(p.c), p.m, p.n, p.k, (int64_t)p.k, ldb, (int64_t)p.n, epi, p.stride_a,
@@ -1773,7 +1808,7 @@ bool TryDma16(const GemmProblem& p, hipStream_t stream) {
   const int64_t tiles128 = (int64_t)((p.m + 127) / 128) * ((p.n + 127) / 128) * p.batch;
   static const int forced = getenv("FLAGS_cinn_hip_gemm_tile") ? atoi(getenv("FLAGS_cinn_hip_gemm_tile")) : 0;
   // narrow outputs with B stored [N][K] (convolutions to 64 channels): 256x64 tiles on 4x1 wavefronts, two blocks per CU
-  const bool narrow = p.trans_b && p.n % 128 != 0 && p.n % 64 == 0 && forced == 0 &&
+  const bool narrow = p.trans_b && p.n % 128 != 0 && p.n % 64 == 0 && forced == 0 && !(p.conv && p.conv->x2) &&
                       (int64_t)((p.m + 255) / 256) * (p.n / 64) * p.batch >= 256;
   // 128x128 tiles keep two stages of 32 KiB and two blocks per CU, or - when there is at most one block per CU
   // anyway - four stages: three K steps of loads in flight instead of one (2048^3: 27.8 -> 21.9 us; with more
@@ -1802,6 +1837,22 @@ bool TryDma16(const GemmProblem& p, hipStream_t stream) {
   const bool few_tiles_long_k = (tiles128 < 96 && p.k >= 2048) || (tiles128 < 128 && p.k >= 1024);
   if (p.trans_b && !p.conv && ((forced == 0 && FeedWavefronts() && few_tiles_long_k && p.batch == 1) || forced == 64)) {
     LaunchDma16<T, true, 64, 64, 1, 1, false, 4, true>(p, stream);
+    return true;
+  }
+  if (p.conv && p.conv->x2 != nullptr) {
+    // a convolution with a second input: the same tile choices, no split of K (ConvPairShape repeats the conditions)
+    if (!p.trans_b || p.batch != 1) return false;
+    if (tiles256 >= 192 && forced != 128) {
+      LaunchDma16<T, true, 256, 256, 2, 4, true, 2, false, true>(p, stream);
+    } else if (tiles128 >= 192 || (tiles128 >= 128 && p.k >= 4096)) {
+      if (stages == 4) {
+        LaunchDma16<T, true, 128, 128, 2, 2, true, 4, true, true>(p, stream);
+      } else {
+        LaunchDma16<T, true, 128, 128, 2, 2, true, 2, false, true>(p, stream);
+      }
+    } else {
+      return false;
+    }
     return true;
   }
   if (p.conv) {
@@ -2069,12 +2120,22 @@ cinn_buffer_t* BufferArg(void* v_args, int index) {
 
 namespace cinn_hip_kernels {
 
+bool ConvPairShape(int64_t m, int c1, int c2, int oc) {
+  if (m <= 0 || m >= INT_MAX || c1 <= 0 || c2 <= 0 || oc <= 0 || c1 % kD64BK != 0 || c2 % kD64BK != 0 || oc % 8 != 0) return false;
+  // the tile counts from which TryDma16 sends an implicit GEMM to one of its instances without splitting K
+  const int64_t tiles256 = ((m + 255) / 256) * ((oc + 255) / 256);
+  const int64_t tiles128 = ((m + 127) / 128) * ((oc + 127) / 128);
+  return tiles256 >= 192 || tiles128 >= 192 || (tiles128 >= 128 && c1 + c2 >= 4096);
+}
+
 bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream) {
   // FLAGS_cinn_hip_conv_pointwise_gemm: 0 keeps 1x1 layers on the convolution kernel, 2 sends every one the GEMM
   // kernels can take to them, whatever the grid (for measurements)
   static const int mode = getenv("FLAGS_cinn_hip_conv_pointwise_gemm") ? atoi(getenv("FLAGS_cinn_hip_conv_pointwise_gemm")) : 1;
   const bool enabled = mode != 0;
-  if (!enabled || ForceGeneric() || UseRegisterStaging()) return false;
+  // a second input has no other implementation: the measurement flags do not apply to it
+  const bool pair = a.x2 != nullptr;
+  if (!pair && (!enabled || ForceGeneric() || UseRegisterStaging())) return false;
   const bool is_f16  = a.type.code == cinn_type_float && a.type.bits == 16;
   const bool is_bf16 = a.type.code == cinn_type_bfloat && a.type.bits == 16;
   if (!is_f16 && !is_bf16) return false;
@@ -2084,7 +2145,8 @@ bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream) {
   if (reinterpret_cast<uintptr_t>(a.x) % 16 != 0 || reinterpret_cast<uintptr_t>(a.w) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(a.y) % 16 != 0 || reinterpret_cast<uintptr_t>(a.residual) % 16 != 0)
     return false;
-  const bool pointwise = a.kh == 1 && a.kw == 1 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 0 && a.pad_w == 0 &&
+  if (reinterpret_cast<uintptr_t>(a.x2) % 16 != 0) return false;
+  const bool pointwise = !pair && a.kh == 1 && a.kw == 1 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 0 && a.pad_w == 0 &&
                          a.oh == a.h && a.ow == a.w_in;
   GemmProblem p;
   ConvGeom geom{};
@@ -2107,7 +2169,7 @@ bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream) {
   } else {
     // any filter, stride, padding, dilation: implicit GEMM, K = kh * kw * c with 64-channel steps inside a tap
     static const bool conv_enabled = !(getenv("FLAGS_cinn_hip_conv_implicit_gemm") && atoi(getenv("FLAGS_cinn_hip_conv_implicit_gemm")) == 0);
-    if (!conv_enabled || a.c % 64 != 0 || (int64_t)a.n * a.h * a.w_in * a.c >= INT_MAX) return false;
+    if ((!conv_enabled && !pair) || a.c % 64 != 0 || (int64_t)a.n * a.h * a.w_in * a.c >= INT_MAX) return false;
     // window corners are kept as two signed 16-bit coordinates
     if (a.h + a.pad_h >= 32768 || a.w_in + a.pad_w >= 32768) return false;
     geom.h = a.h, geom.w = a.w_in, geom.c = a.c;
@@ -2117,6 +2179,17 @@ bool TryPointwiseConvAsGemm(const ConvNhwcArgs& a, hipStream_t stream) {
     geom.zero_page = ConvZeroPage();
     p.conv = &geom;
     p.k    = a.kh * a.kw * a.c;
+    if (pair) {
+      // the second input's pixel (oy stride2_h, ox stride2_w) must exist for every output pixel
+      if (a.c2 <= 0 || a.c2 % 64 != 0 || a.stride2_h <= 0 || a.stride2_w <= 0 || (a.oh - 1) * a.stride2_h >= a.h2 ||
+          (a.ow - 1) * a.stride2_w >= a.w2 || a.h2 >= 32768 || a.w2 >= 32768 || (int64_t)a.n * a.h2 * a.w2 * a.c2 >= INT_MAX)
+        return false;
+      geom.x2 = a.x2;
+      geom.h2 = a.h2, geom.w2 = a.w2, geom.c2 = a.c2;
+      geom.stride2_h = a.stride2_h, geom.stride2_w = a.stride2_w;
+      geom.steps1    = p.k / kD64BK;
+      p.k += a.c2;
+    }
   }
   p.type    = is_bf16 ? GemmType::kBF16 : GemmType::kF16;
   p.a       = a.x;  // [pixels][c], or the NHWC input of the implicit GEMM

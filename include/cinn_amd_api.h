@@ -47,7 +47,7 @@ int cinn_amd_builder_program_string(cinn_amd_builder_t b, char* out, size_t cap,
 /* ---- CinnComputation (cinn/frontend/computation.h) ---- */
 /* CinnComputation::BuildAndCompile for the AMDGPU target.  outputs: ids to fetch (NULL/0: outputs of the
  * last instruction).  stream: hipStream_t or NULL.  options: "key=value;..." (keys: do_prerun,
- * fuse_conv_bn_relu, fuse_stem_pool, fuse_matmul_bias, fuse_conv_chain, conv_layout_nhwc, split_reductions,
+ * fuse_conv_bn_relu, fuse_stem_pool, fuse_matmul_bias, fuse_conv_chain, fuse_shortcut_projection, conv_layout_nhwc, split_reductions,
  * merge_independent_kernels, memory_arena, reuse_intermediates, and the lowering knobs
  * reduce_cached_elems, reduce_wave_elems, elementwise_block, reduce_rows_per_block).
  * Memory: with memory_arena=1 (default) every tensor the program's instructions touch is a slice of ONE device

@@ -188,6 +188,22 @@ void cinn_call_hip_conv2d_bn_relu(void* v_args, int num_args, int format, int re
 void cinn_call_hip_conv2d_bn_relu_chain(void* v_args, int num_args, int relu, int input_n, int input_h, int input_w,
                                         int input_c, int middle_c, int output_c, void* stream);
 
+/* Extension with no counterpart in the reference (there a projection shortcut is one cudnnConvolutionForward and the
+ * layer that adds it another, cinn/runtime/cuda/cuda_util.cc:603-720): one 1x1 convolution over the channels of two
+ * channels-last inputs that share the output's pixel grid,
+ *   y[n][oy][ox][:] = act(w[:, :input_c] x[n][oy][ox][:] + w[:, input_c:] x2[n][oy second_stride_h][ox second_stride_w][:] + shift)
+ * v_args = {x, x2, w, shift, y}; x is [n][h][w][input_c], x2 [n][second_h][second_w][second_c], w
+ * [output_c][1][1][input_c + second_c] (each row: the weights of x's channels, then those of x2's), shift fp32 [output_c],
+ * y [n][h][w][output_c]; x, x2, w and y share one 16-bit floating-point type.  relu: bit 0 = ReLU.  This is a bottleneck
+ * block's last 1x1 layer and its strided 1x1 projection shortcut in one launch, once their batch-norm scales are
+ * multiplied into the filters (the FuseShortcutProjection rewrite does that); the K loop of the implicit-GEMM kernel
+ * walks x's channels and then x2's.  Shapes the kernel does not take (channel counts that are not multiples of 64, too
+ * few output tiles: ConvPairShape in kernels/conv_chain.h) abort with a message - there is no two-launch form of this
+ * call; the rewrite emits it for qualifying shapes only. */
+void cinn_call_hip_conv2d_pointwise_pair(void* v_args, int num_args, int relu, int input_n, int input_h, int input_w,
+                                         int input_c, int second_h, int second_w, int second_c, int second_stride_h,
+                                         int second_stride_w, int output_c, void* stream);
+
 /* cinn_call_cudnn_conv2d_forward for callers that cannot allocate.  No counterpart in the reference: it exists for
  * code that runs under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  Same arguments and
  * results as the call above for format 1 and 2 with groups == 1 (always on the general channels-last MFMA kernel);

@@ -528,6 +528,53 @@ def test_pointwise_pairs_the_kernel_does_not_take_stay_two_calls():
     assert "chain" not in comp.fusion_groups() and comp.fusion_groups().count("hip_conv2d_bn_relu") == 2
 
 
+def _projection_block(builder, batch, other_reader=False, relu_on_projection=False):
+    """The end of a bottleneck block with a projection shortcut (fp16, const parameters): a strided 1x1 projection of the
+    block's input and the block's last 1x1 layer, added, relu - what FuseShortcutProjection turns into one call."""
+    t = Float(16)
+
+    def const(name, shape):
+        v = builder.create_input(t, shape, name)
+        v.set_const()
+        return v
+
+    def bn(y, p, c):
+        return builder.batchnorm(y, const(p + "_g", [c]), const(p + "_b", [c]), const(p + "_m", [c]), const(p + "_v", [c]),
+                                 epsilon=1e-5)[0]
+
+    block_in = builder.create_input(t, [batch, 256, 56, 56], "block_in")
+    mid = builder.create_input(t, [batch, 128, 28, 28], "mid")
+    short = bn(builder.conv2d(block_in, const("ws", [512, 256, 1, 1]), strides=[2, 2]), "bns", 512)
+    if relu_on_projection:
+        short = builder.relu(short)
+    out = builder.relu(builder.add(bn(builder.conv2d(mid, const("wc", [512, 128, 1, 1])), "bnc", 512), short))
+    return [out] + ([builder.scale(short, 2.0)] if other_reader else [])
+
+
+def test_projection_shortcut_and_the_layer_that_adds_it_become_one_call():
+    b = NetBuilder("proj")
+    comp = compile_only(b, _projection_block(b, 16))
+    groups = comp.fusion_groups().strip().splitlines()
+    pairs = [g for g in groups if "hip_conv2d_pointwise_pair" in g]
+    assert len(pairs) == 1 and "hip_conv2d_bn_relu" not in comp.fusion_groups(), groups
+    # inputs: the block's middle tensor, the block's input, the filters side by side, the summed shift
+    ins = pairs[0].split(" in: ")[1].split(" out: ")[0].split()
+    assert len(ins) == 4, pairs[0]
+    assert comp.get_tensor(ins[2]).shape() == [512, 1, 1, 128 + 256] and comp.get_tensor(ins[3]).shape() == [512]
+    b = NetBuilder("proj")
+    apart = compile_only(b, _projection_block(b, 16), fuse_shortcut_projection=0)
+    text = apart.fusion_groups()
+    assert "pointwise_pair" not in text and text.count("hip_conv2d_bn_relu") == 2
+
+
+@pytest.mark.parametrize("kwargs", [dict(batch=2), dict(batch=16, other_reader=True), dict(batch=16, relu_on_projection=True)])
+def test_projection_shortcuts_that_stay_calls_of_their_own(kwargs):
+    """too few pixels for the kernel's tiles; a projection that something else reads; a projection with a relu of its own"""
+    b = NetBuilder("proj")
+    text = compile_only(b, _projection_block(b, **kwargs)).fusion_groups()
+    assert "pointwise_pair" not in text and text.count("hip_conv2d_bn_relu") == 2, text
+
+
 def test_tensor_names_that_are_keywords_of_the_kernel_language():
     b = NetBuilder("kw")
     a = b.create_input(Float(32), [4, 8], "short")

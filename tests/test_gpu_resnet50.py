@@ -144,6 +144,13 @@ def test_resnet50_batch32(gpu, dtype, tol):
     assert np.abs(got[:2].astype(np.float64) - small.astype(np.float64)).max() <= tol * np.abs(small).max()
     want = torch_forward(params, x)
     assert np.abs(got.astype(np.float64) - want).max() <= tol * np.abs(want).max()
+    if dtype == "float16":
+        # at this batch size the projection shortcuts of stages 2-4 share a call with the layer that adds them (the
+        # first stage's expansion is half of a two-layer call already)
+        assert comp.num_instructions() == 47 + 1 + 1, comp.fusion_groups()
+        apart, comp_apart = gpu_forward(params, x, fuse_shortcut_projection=False)
+        assert comp_apart.num_instructions() == 50 + 1 + 1, comp_apart.fusion_groups()
+        assert np.abs(apart.astype(np.float64) - want).max() <= tol * np.abs(want).max()
     # first and last image of the batch against the oracle (x[31] is x[1]), element by element
     want_ends = oracle_forward(params, x[[0, 31]]).astype(np.float64)
     if dtype == "float32":
