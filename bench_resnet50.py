@@ -137,6 +137,11 @@ def roofline_of(comp, dtype):
             x, w1, e, y = (tensors[args[j]].shape() for j in (0, 1, -2, -1))
             pixels = int(np.prod(x[:-1], dtype=np.int64))
             flop = 2 * pixels * (w1[-1] * e[-1] + e[-1] * y[-1])
+        elif "conv2d_pair_chain" in fn:
+            # (x, x2, w1, shift1, w2, scale2, shift2, e, y): a 1x1 convolution over two inputs, then another one
+            x, w1, e, y = (tensors[args[j]].shape() for j in (0, 2, -2, -1))
+            pixels = int(np.prod(x[:-1], dtype=np.int64))
+            flop = 2 * pixels * (w1[-1] * e[-1] + e[-1] * y[-1])
         elif "conv2d_pointwise_pair" in fn:
             # (x, x2, w, shift, y): one 1x1 convolution over the channels of both inputs
             w, y = tensors[args[2]].shape(), tensors[args[-1]].shape()

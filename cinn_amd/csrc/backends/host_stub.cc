@@ -43,6 +43,9 @@ void InvokeConv2dBnRelu(const std::vector<BakedArg>& a, void* args, int32_t n, v
 void InvokeConv2dBnReluChain(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
   cinn_call_hip_conv2d_bn_relu_chain(args, n, I(a[2]), I(a[3]), I(a[4]), I(a[5]), I(a[6]), I(a[7]), I(a[8]), stream);
 }
+void InvokeConv2dPairChain(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
+  cinn_call_hip_conv2d_pair_chain(args, n, I(a[2]), I(a[3]), I(a[4]), I(a[5]), I(a[6]), I(a[7]), I(a[8]), I(a[9]), stream);
+}
 void InvokeConv2dPointwisePair(const std::vector<BakedArg>& a, void* args, int32_t n, void* stream) {
   cinn_call_hip_conv2d_pointwise_pair(args, n, I(a[2]), I(a[3]), I(a[4]), I(a[5]), I(a[6]), I(a[7]), I(a[8]), I(a[9]), I(a[10]),
                                       I(a[11]), I(a[12]), stream);
@@ -98,6 +101,8 @@ ExternApiRegistry::ExternApiRegistry() {
   Register("cinn_call_hip_conv2d_bn_relu_chain", InvokeConv2dBnReluChain, 10);
   // (kernel_args, kernel_args_num, relu, n, h, w, c, second h, w, c, second stride h, w, output_c, kernel_stream)
   Register("cinn_call_hip_conv2d_pointwise_pair", InvokeConv2dPointwisePair, 14);
+  // (kernel_args, kernel_args_num, relu bits, n, h, w, input_c, second_c, middle_c, output_c, kernel_stream)
+  Register("cinn_call_hip_conv2d_pair_chain", InvokeConv2dPairChain, 11);
   Register("cinn_call_cudnn_pool2d_forward", InvokePool2dForward, 21);
   Register("cinn_call_cudnn_softmax_forward", InvokeSoftmaxForward, 15);
   // (kernel_args, kernel_args_num, outer, size, inner, is_ascend, outputs, kernel_stream)

@@ -580,18 +580,64 @@ Program FuseShortcutProjection(const Program& program, const std::set<std::strin
   std::vector<bool> dropped(instrs.size(), false);
   std::map<size_t, std::vector<Instruction>> replacement;
   int serial = 0;
+  // the filters of two layers side by side along their channels, each times its scale: multiplied in fp32, rounded once
+  // to the storage type
+  auto scaled_side_by_side = [](Emitter& e, const Variable& w1, const Variable& s1, const Variable& w2, const Variable& s2) {
+    const std::string store = w1->type.is_bfloat16() ? "bfloat16" : "float16";
+    auto scaled = [&](const Variable& w, const Variable& s) {
+      auto w32 = e.Emit1("cast", {w}, {{"dtype", std::string("float32")}});
+      auto sb  = e.Emit1("broadcast_to", {s}, {{"out_shape", w->shape}, {"broadcast_axes", ShapeType{0}}});
+      auto ws  = e.Emit1("elementwise_mul", {w32, sb}, {{"axis", -1}});
+      return e.Emit1("cast", {ws}, {{"dtype", store}});
+    };
+    return e.Emit1("concat", {scaled(w1, s1), scaled(w2, s2)}, {{"axis", 3}});
+  };
+  // the projection behind residual r of the instruction at position i, or null: a folded 1x1 projection without relu
+  // that nothing else reads
+  auto projection_of = [&](const Variable& r, size_t i) -> const Instruction* {
+    auto def = defined_at.find(r->id);
+    if (def == defined_at.end() || def->second >= i || dropped[def->second]) return nullptr;
+    const auto& proj = instrs[def->second];
+    if (!pointwise(proj) || proj->inputs.size() != 4 || GetAttr<bool>(proj->attrs, "relu", false)) return nullptr;
+    auto ru = users.find(r->id);
+    if (fetch_ids.count(r->id) || ru == users.end() || ru->second.size() != 1) return nullptr;
+    return &proj;
+  };
   for (size_t i = 0; i < instrs.size(); ++i) {
     const auto& main = instrs[i];
+    if (main->op_type == "hip_conv2d_bn_relu_chain" && main->inputs.size() == 8) {
+      // x, w1, scale1, shift1, residual, w2, scale2, shift2 -> e, y: the residual becomes a second input of the first layer
+      const Variable& r = main->inputs[4];
+      const Instruction* pp = projection_of(r, i);
+      if (!pp) continue;
+      const auto& proj = *pp;
+      const Variable &x = main->inputs[0], &x2 = proj->inputs[0], &e_out = main->outputs[0], &y = main->outputs[1];
+      if (x == r || !(x2->type == x->type) || r->shape != e_out->shape) continue;
+      if (GetAttr<std::vector<int>>(proj->attrs, "stride", {1, 1}) != std::vector<int>{1, 1}) continue;
+      if (x2->shape[0] != x->shape[0] || x2->shape[1] != x->shape[1] || x2->shape[2] != x->shape[2]) continue;
+      const int64_t m = static_cast<int64_t>(x->shape[0]) * x->shape[1] * x->shape[2];
+      if (!cinn_hip_kernels::ConvChainShape2(m, x->shape[3], x2->shape[3], e_out->shape[3], y->shape[3])) continue;
+      std::vector<Instruction> seq;
+      Emitter e(&seq, "csp" + std::to_string(serial++) + "_");
+      auto w_both = scaled_side_by_side(e, main->inputs[1], main->inputs[2], proj->inputs[1], proj->inputs[2]);
+      auto shift  = e.Emit1("elementwise_add", {main->inputs[3], proj->inputs[3]}, {{"axis", -1}});
+      Instruction chain("hip_conv2d_pair_chain");
+      chain->inputs  = {x, x2, w_both, shift, main->inputs[5], main->inputs[6], main->inputs[7]};
+      chain->outputs = main->outputs;
+      chain->attrs["relu"]       = GetAttr<bool>(main->attrs, "relu", false);
+      chain->attrs["relu_after"] = GetAttr<bool>(main->attrs, "relu_after", false);
+      seq.push_back(chain);
+      dropped[defined_at[r->id]] = true;
+      dropped[i]                 = true;
+      replacement[i]             = seq;
+      continue;
+    }
     if (!pointwise(main) || main->inputs.size() != 5) continue;
     if (GetAttr<std::vector<int>>(main->attrs, "stride", {1, 1}) != std::vector<int>{1, 1}) continue;
     const Variable& r = main->inputs[4];
-    auto def = defined_at.find(r->id);
-    if (def == defined_at.end() || def->second >= i || dropped[def->second]) continue;
-    const auto& proj = instrs[def->second];
-    if (!pointwise(proj) || proj->inputs.size() != 4 || GetAttr<bool>(proj->attrs, "relu", false)) continue;
-    // the projection's result feeds this addition and nothing else
-    auto ru = users.find(r->id);
-    if (fetch_ids.count(r->id) || ru == users.end() || ru->second.size() != 1) continue;
+    const Instruction* pp = projection_of(r, i);
+    if (!pp) continue;
+    const auto& proj = *pp;
     const Variable &x = main->inputs[0], &x2 = proj->inputs[0], &y = main->outputs[0];
     if (x == r || !(x2->type == x->type) || r->shape != y->shape) continue;
     auto stride2 = GetAttr<std::vector<int>>(proj->attrs, "stride", {1, 1});
@@ -603,20 +649,13 @@ Program FuseShortcutProjection(const Program& program, const std::set<std::strin
     // (multiplied in fp32, rounded once to the storage type), the filters side by side along their channels
     std::vector<Instruction> seq;
     Emitter e(&seq, "csp" + std::to_string(serial++) + "_");
-    const std::string store = x->type.is_bfloat16() ? "bfloat16" : "float16";
-    auto scaled = [&](const Variable& w, const Variable& s) {
-      auto w32 = e.Emit1("cast", {w}, {{"dtype", std::string("float32")}});
-      auto sb  = e.Emit1("broadcast_to", {s}, {{"out_shape", w->shape}, {"broadcast_axes", ShapeType{0}}});
-      auto ws  = e.Emit1("elementwise_mul", {w32, sb}, {{"axis", -1}});
-      return e.Emit1("cast", {ws}, {{"dtype", store}});
-    };
-    auto w_both = e.Emit1("concat", {scaled(main->inputs[1], main->inputs[2]), scaled(proj->inputs[1], proj->inputs[2])}, {{"axis", 3}});
+    auto w_both = scaled_side_by_side(e, main->inputs[1], main->inputs[2], proj->inputs[1], proj->inputs[2]);
     auto shift  = e.Emit1("elementwise_add", {main->inputs[3], proj->inputs[3]}, {{"axis", -1}});
     e.EmitInto(y, "hip_conv2d_pointwise_pair", {x, x2, w_both, shift},
                {{"second_stride", stride2}, {"relu", GetAttr<bool>(main->attrs, "relu", false)}});
-    dropped[def->second] = true;
-    dropped[i]           = true;
-    replacement[i]       = seq;
+    dropped[defined_at[r->id]] = true;
+    dropped[i]                 = true;
+    replacement[i]             = seq;
   }
   if (replacement.empty()) return program;
   std::vector<Instruction> out;

@@ -1451,6 +1451,11 @@ ir::LoweredFuncRef OpLowerer::LowerLibraryCall(const Group& group) const {
     const auto& x = n->inputs[0]->shape;
     args.push_back(I32((GetAttr<bool>(n->attrs, "relu", false) ? 1 : 0) | (GetAttr<bool>(n->attrs, "relu_after", false) ? 2 : 0)));
     push_ints({x[0], x[1], x[2], x[3], n->outputs[0]->shape[3], n->outputs[1]->shape[3]});
+  } else if (op == "hip_conv2d_pair_chain") {
+    api            = "cinn_call_hip_conv2d_pair_chain";
+    const auto& x  = n->inputs[0]->shape;
+    args.push_back(I32((GetAttr<bool>(n->attrs, "relu", false) ? 1 : 0) | (GetAttr<bool>(n->attrs, "relu_after", false) ? 2 : 0)));
+    push_ints({x[0], x[1], x[2], x[3], n->inputs[1]->shape[3], n->outputs[0]->shape[3], n->outputs[1]->shape[3]});
   } else if (op == "hip_conv2d_pointwise_pair") {
     api            = "cinn_call_hip_conv2d_pointwise_pair";
     const auto& x  = n->inputs[0]->shape;

@@ -679,6 +679,24 @@ OpRegistry::OpRegistry() {
     op.infer_dtype = SameTypeAsFirst;
   }
   {
+    // hip_conv2d_bn_relu_chain whose first layer reads a second input of the same pixel grid instead of adding a
+    // residual (FuseShortcutProjection); inputs x, x2, w1 [M][1][1][C1 + C2], shift1, w2, scale2, shift2; outputs e, y
+    auto& op       = r->Register("hip_conv2d_pair_chain");
+    op.pattern     = OpPatternKind::kNonFusible;
+    op.num_inputs  = 7;
+    op.infer_shape = [](const std::vector<ShapeType>& in, const AttributeMap&) {
+      CINN_CHECK_EQ(in.size(), 7u) << "hip_conv2d_pair_chain takes x, x2, w1, shift1, w2, scale2, shift2";
+      CINN_CHECK(in[0].size() == 4u && in[1].size() == 4u && in[2].size() == 4u && in[4].size() == 4u) << "hip_conv2d_pair_chain: 4-D operands expected";
+      CINN_CHECK(in[1][0] == in[0][0] && in[1][1] == in[0][1] && in[1][2] == in[0][2]) << "hip_conv2d_pair_chain: both inputs cover the same pixels";
+      CINN_CHECK(in[2][1] == 1 && in[2][2] == 1 && in[4][1] == 1 && in[4][2] == 1 && in[2][3] == in[0][3] + in[1][3] && in[4][3] == in[2][0])
+          << "hip_conv2d_pair_chain: [M][1][1][C1 + C2] and [O][1][1][M] filters expected";
+      ShapeType e = {in[0][0], in[0][1], in[0][2], in[2][0]};
+      ShapeType y = {in[0][0], in[0][1], in[0][2], in[4][0]};
+      return std::vector<ShapeType>{e, y};
+    };
+    op.infer_dtype = [](const std::vector<Type>& in, const AttributeMap&) { return std::vector<Type>{in[0], in[0]}; };
+  }
+  {
     // cinn/hlir/op/contrib/sort.cc:307-350: both keep the operand's shape; argsort has two int32 outputs (indices,
     // positions), sort one of the operand's type
     auto check_axis = [](const std::vector<ShapeType>& in, const AttributeMap& a) {

@@ -25,6 +25,9 @@
 //   * Sums are formed in the order of the kernels that run the two layers separately (gemm16_shortk_kernel for the
 //     first - 32-channel blocks in ascending order on unpermuted k chunks -, gemm16_dma_kernel for the second) and the
 //     epilogues are the same arithmetic: the first result is bit-identical to the two-launch form.
+//   * K1B > 0: the first product reads K1B more channels of the same pixels from a second tensor X2 [M][K1B] (W1 is then
+//     [N1][K1 + K1B]): an expansion and a stride-1 projection shortcut of another tensor as one product, instead of a
+//     shortcut tensor of E's size that one kernel writes and this one reads.  No residual in that form.
 // Measured and not kept: the same pair one stage later (128 -> 512 -> 128 on 28 x 28: the filters fill half of a CU's
 // register file, so one block of eight wavefronts per CU, every barrier and LDS latency exposed) took 27.4-28.2 us
 // against 17.5 + 10.5 us for the two launches; a separate wavefront that only loads (rows of X and of the shortcut
@@ -50,6 +53,7 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 struct ChainParams {
   const uint16_t* x;
+  const uint16_t* x2;  // second input of the first product, or null
   const uint16_t* w1;
   const float* scale1;
   const float* shift1;
@@ -63,11 +67,13 @@ struct ChainParams {
   int groups;  // M / 16
 };
 
-template <typename T, int K1, int N1, int N2, int WAVES>
+template <typename T, int K1, int N1, int N2, int WAVES, int K1B = 0>
 __global__ void __launch_bounds__(64 * WAVES) conv1x1_chain_kernel(ChainParams p) {
   typedef typename Mfma16<T>::vec8 vec8;
   constexpr int THREADS = 64 * WAVES;
-  constexpr int KB1     = K1 / 32;             // 32-channel blocks of the first product
+  constexpr int KT      = K1 + K1B;            // channels of the first product: X's, then X2's
+  constexpr int KB1     = KT / 32;             // 32-channel blocks of the first product
+  static_assert(K1 % 32 == 0 && K1B % 32 == 0, "whole 32-channel blocks from either input");
   constexpr int KB2     = N1 / 32;             // ... of the second
   constexpr int J1      = N1 / (16 * WAVES);   // 16-column tiles of E per wavefront
   constexpr int J2      = N2 / (16 * WAVES);   // 16-column tiles of Y per wavefront
@@ -106,7 +112,7 @@ __global__ void __launch_bounds__(64 * WAVES) conv1x1_chain_kernel(ChainParams p
   for (int j = 0; j < J1; ++j)
 #pragma unroll
     for (int kb = 0; kb < KB1; ++kb)
-      wf1[j][kb] = *reinterpret_cast<const vec8*>(p.w1 + (int64_t)(c1 + 16 * j + frow) * K1 + 32 * kb + fk1);
+      wf1[j][kb] = *reinterpret_cast<const vec8*>(p.w1 + (int64_t)(c1 + 16 * j + frow) * KT + 32 * kb + fk1);
 #pragma unroll
   for (int j = 0; j < J2; ++j)
 #pragma unroll
@@ -127,7 +133,7 @@ __global__ void __launch_bounds__(64 * WAVES) conv1x1_chain_kernel(ChainParams p
 
   int g = blockIdx.x;
   if (g >= p.groups) return;
-  const T* const R = reinterpret_cast<const T*>(p.residual);
+  const T* const R = K1B == 0 ? reinterpret_cast<const T*>(p.residual) : nullptr;
   T* const E       = reinterpret_cast<T*>(p.e);
   T* const Y       = reinterpret_cast<T*>(p.y);
   // a thread's chunk of pass i: row i (THREADS / CPR) + tid / CPR of the group, columns 8 (tid % CPR) ..
@@ -135,7 +141,12 @@ __global__ void __launch_bounds__(64 * WAVES) conv1x1_chain_kernel(ChainParams p
   auto request = [&](int grp, vec8* xa, vec8* rr) {
     const uint16_t* const x_g = p.x + (int64_t)grp * 16 * K1;
 #pragma unroll
-    for (int kb = 0; kb < KB1; ++kb) xa[kb] = *reinterpret_cast<const vec8*>(x_g + frow * K1 + 32 * kb + fk1);
+    for (int kb = 0; kb < K1 / 32; ++kb) xa[kb] = *reinterpret_cast<const vec8*>(x_g + frow * K1 + 32 * kb + fk1);
+    if (K1B > 0) {
+      const uint16_t* const x2_g = p.x2 + (int64_t)grp * 16 * K1B;
+#pragma unroll
+      for (int kb = 0; kb < K1B / 32; ++kb) xa[K1 / 32 + kb] = *reinterpret_cast<const vec8*>(x2_g + frow * K1B + 32 * kb + fk1);
+    }
     if (R) {
       const T* const r_g = R + (int64_t)grp * 16 * N1;
 #pragma unroll
@@ -230,11 +241,11 @@ __global__ void __launch_bounds__(64 * WAVES) conv1x1_chain_kernel(ChainParams p
   }
 }
 
-template <typename T, int K1, int N1, int N2, int WAVES, int BLOCKS_PER_CU>
+template <typename T, int K1, int N1, int N2, int WAVES, int BLOCKS_PER_CU, int K1B = 0>
 void LaunchChain(const ChainParams& p, hipStream_t stream) {
   const int resident = 256 * BLOCKS_PER_CU;
   dim3 grid(p.groups < resident ? p.groups : resident);
-  hipLaunchKernelGGL((conv1x1_chain_kernel<T, K1, N1, N2, WAVES>), grid, dim3(64 * WAVES), 0, stream, p);
+  hipLaunchKernelGGL((conv1x1_chain_kernel<T, K1, N1, N2, WAVES, K1B>), grid, dim3(64 * WAVES), 0, stream, p);
 }
 
 // 1: where the shape qualifies (default), 0: never; -1: not read yet
@@ -257,16 +268,26 @@ bool ConvChainShape(int64_t m, int k1, int n1, int n2) {
   return k1 == 64 && n1 == 256 && (n2 == 64 || n2 == 128);
 }
 
+bool ConvChainShape2(int64_t m, int k1, int k1b, int n1, int n2) {
+  if (m <= 0 || m % 16 != 0 || m * n1 >= INT_MAX) return false;
+  return k1 == 64 && k1b == 64 && n1 == 256 && n2 == 64;
+}
+
 bool TryConvChain(const ConvChainArgs& a, hipStream_t stream) {
   if (!ChainMode()) return false;
   const bool is_f16  = a.type.code == cinn_type_float && a.type.bits == 16;
   const bool is_bf16 = a.type.code == cinn_type_bfloat && a.type.bits == 16;
-  if ((!is_f16 && !is_bf16) || !ConvChainShape(a.m, a.k1, a.n1, a.n2)) return false;
-  const void* ptrs[] = {a.x, a.w1, a.residual, a.e, a.w2, a.y};
+  if (!is_f16 && !is_bf16) return false;
+  if (a.x2 != nullptr) {
+    if (a.residual != nullptr || !ConvChainShape2(a.m, a.k1, a.k1b, a.n1, a.n2)) return false;
+  } else if (!ConvChainShape(a.m, a.k1, a.n1, a.n2)) {
+    return false;
+  }
+  const void* ptrs[] = {a.x, a.x2, a.w1, a.residual, a.e, a.w2, a.y};
   for (const void* ptr : ptrs)
     if (reinterpret_cast<uintptr_t>(ptr) % 16 != 0) return false;
   ChainParams p;
-  p.x = static_cast<const uint16_t*>(a.x), p.w1 = static_cast<const uint16_t*>(a.w1);
+  p.x = static_cast<const uint16_t*>(a.x), p.x2 = static_cast<const uint16_t*>(a.x2), p.w1 = static_cast<const uint16_t*>(a.w1);
   p.scale1 = a.scale1, p.shift1 = a.shift1, p.residual = static_cast<const uint16_t*>(a.residual);
   p.e = static_cast<uint16_t*>(a.e), p.w2 = static_cast<const uint16_t*>(a.w2);
   p.scale2 = a.scale2, p.shift2 = a.shift2, p.y = static_cast<uint16_t*>(a.y);
@@ -280,7 +301,13 @@ bool TryConvChain(const ConvChainArgs& a, hipStream_t stream) {
       LaunchChain<_Float16, K1, N1, N2, WAVES, BPC>(p, stream); \
     }                                                           \
   } while (0)
-  if (a.n2 == 64) {
+  if (a.x2 != nullptr) {
+    if (is_bf16) {
+      LaunchChain<__bf16, 64, 256, 64, 4, 2, 64>(p, stream);  // twice the filter registers of the first product: two blocks per CU
+    } else {
+      LaunchChain<_Float16, 64, 256, 64, 4, 2, 64>(p, stream);
+    }
+  } else if (a.n2 == 64) {
     CINN_CHAIN(64, 256, 64, 4, 3);   // 163 registers: three blocks per CU
   } else {
     CINN_CHAIN(64, 256, 128, 4, 2);  // 200 registers: two

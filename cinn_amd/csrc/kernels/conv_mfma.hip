@@ -465,6 +465,50 @@ void cinn_call_hip_conv2d_bn_relu_chain(void* v_args, int num_args, int relu, in
           middle_c, 1, 1, 0, 0, 1, 1, 1, 1, 1, input_n, output_c, input_h, input_w, st);
 }
 
+void cinn_call_hip_conv2d_pair_chain(void* v_args, int num_args, int relu, int input_n, int input_h, int input_w, int input_c,
+                                     int second_c, int middle_c, int output_c, void* stream) {
+  CINN_HIP_CLEAR_STALE_ERROR();
+  CINN_RT_CHECK(num_args == 9, "cinn_call_hip_conv2d_pair_chain takes x, x2, w1, shift1, w2, scale2, shift2, e and y, got %d arguments",
+                num_args);
+  cinn_buffer_t* x  = BufferArg(v_args, 0);
+  cinn_buffer_t* x2 = BufferArg(v_args, 1);
+  cinn_buffer_t* w1 = BufferArg(v_args, 2);
+  cinn_buffer_t* t1 = BufferArg(v_args, 3);
+  cinn_buffer_t* w2 = BufferArg(v_args, 4);
+  cinn_buffer_t* s2 = BufferArg(v_args, 5);
+  cinn_buffer_t* t2 = BufferArg(v_args, 6);
+  cinn_buffer_t* e  = BufferArg(v_args, 7);
+  cinn_buffer_t* y  = BufferArg(v_args, 8);
+  for (cinn_buffer_t* f : {t1, s2, t2})
+    CINN_RT_CHECK(f->type.code == cinn_type_float && f->type.bits == 32, "cinn_call_hip_conv2d_pair_chain: scale / shift must be fp32");
+  const bool is_16 = x->type.bits == 16 && (x->type.code == cinn_type_float || x->type.code == cinn_type_bfloat);
+  for (cinn_buffer_t* b : {x2, w1, w2, e, y})
+    CINN_RT_CHECK(is_16 && b->type.code == x->type.code && b->type.bits == x->type.bits,
+                  "cinn_call_hip_conv2d_pair_chain: x, x2, w1, w2, e and y must share one 16-bit floating-point type");
+  CINN_RT_CHECK(input_n > 0 && input_h > 0 && input_w > 0 && input_c > 0 && second_c > 0 && middle_c > 0 && output_c > 0,
+                "cinn_call_hip_conv2d_pair_chain: extents must be positive");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  cinn_hip_kernels::ConvChainArgs a;
+  a.x = x->memory, a.w1 = w1->memory, a.scale1 = nullptr;
+  a.shift1 = reinterpret_cast<const float*>(t1->memory), a.residual = nullptr, a.relu1 = (relu & 1) != 0;
+  a.e = e->memory, a.w2 = w2->memory, a.scale2 = reinterpret_cast<const float*>(s2->memory);
+  a.shift2 = reinterpret_cast<const float*>(t2->memory), a.relu2 = (relu & 2) != 0, a.y = y->memory;
+  a.m = (int64_t)input_n * input_h * input_w, a.k1 = input_c, a.n1 = middle_c, a.n2 = output_c, a.type = x->type;
+  a.x2 = x2->memory, a.k1b = second_c;
+  if (cinn_hip_kernels::TryConvChain(a, st)) return;
+  // any other shape: the first layer over both inputs (which has shape limits of its own), then the second layer
+  cinn_pod_value_t first[5];
+  cinn_buffer_t* first_bufs[5] = {x, x2, w1, t1, e};
+  for (int i = 0; i < 5; ++i) {
+    first[i].type_code_      = CINN_POD_BUFFER_P;
+    first[i].value_.v_handle = first_bufs[i];
+  }
+  cinn_call_hip_conv2d_pointwise_pair(first, 5, relu & 1, input_n, input_h, input_w, input_c, input_h, input_w, second_c, 1, 1, middle_c,
+                                      stream);
+  RunConv(e, w2, y, a.scale2, a.shift2, nullptr, a.relu2 ? 2 : 1, 1, 1.0f, 0.0f, input_n, middle_c, input_h, input_w, output_c,
+          middle_c, 1, 1, 0, 0, 1, 1, 1, 1, 1, input_n, output_c, input_h, input_w, st);
+}
+
 void cinn_call_hip_conv2d_pointwise_pair(void* v_args, int num_args, int relu, int input_n, int input_h, int input_w,
                                          int input_c, int second_h, int second_w, int second_c, int second_stride_h,
                                          int second_stride_w, int output_c, void* stream) {

@@ -68,6 +68,10 @@ struct ConvChainArgs {
   int64_t m;
   int k1, n1, n2;
   cinn_type_t type;
+  // a second input of the first product, [m][k1b], or null: e = act1([x | x2] w1^T * scale1 + shift1) with w1
+  // [n1][k1 + k1b]; no residual then
+  const void* x2 = nullptr;
+  int k1b = 0;
 };
 // false when the shape or the types do not qualify (the caller then runs the two convolutions one after the other)
 bool TryConvChain(const ConvChainArgs& a, hipStream_t stream);

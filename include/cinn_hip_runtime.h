@@ -204,6 +204,19 @@ void cinn_call_hip_conv2d_pointwise_pair(void* v_args, int num_args, int relu, i
                                          int input_c, int second_h, int second_w, int second_c, int second_stride_h,
                                          int second_stride_w, int output_c, void* stream);
 
+/* Extension with no counterpart in the reference: cinn_call_hip_conv2d_bn_relu_chain whose first layer reads a second
+ * input of the same pixel grid instead of adding a residual -
+ *   e = act1([w1[:, :input_c] x + w1[:, input_c:] x2] + shift1)   [n][h][w][middle_c]
+ *   y = act2(conv(e, w2) * scale2 + shift2)                       [n][h][w][output_c]
+ * v_args = {x, x2, w1, shift1, w2, scale2, shift2, e, y}; x is [n][h][w][input_c], x2 [n][h][w][second_c], w1
+ * [middle_c][1][1][input_c + second_c], w2 [output_c][1][1][middle_c], shifts and scale fp32; 16-bit types.  relu: bit 0
+ * = ReLU in act1, bit 1 = in act2.  This is the first bottleneck block of a stage whose projection shortcut has
+ * stride 1: expansion and projection as one product (their batch-norm scales multiplied into w1's halves by the
+ * FuseShortcutProjection rewrite), then the next block's reduction.  For 64 + 64 -> 256 -> 64 channels (n h w a multiple of
+ * 16) one kernel computes both; other shapes run cinn_call_hip_conv2d_pointwise_pair and then the second layer. */
+void cinn_call_hip_conv2d_pair_chain(void* v_args, int num_args, int relu, int input_n, int input_h, int input_w, int input_c,
+                                     int second_c, int middle_c, int output_c, void* stream);
+
 /* cinn_call_cudnn_conv2d_forward for callers that cannot allocate.  No counterpart in the reference: it exists for
  * code that runs under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  Same arguments and
  * results as the call above for format 1 and 2 with groups == 1 (always on the general channels-last MFMA kernel);

@@ -493,7 +493,7 @@ def _bottleneck_pair(builder, side_reader):
 @pytest.mark.parametrize("side_reader", [False, True])
 def test_two_pointwise_convolutions_in_a_row_become_one_call(side_reader):
     b = NetBuilder("pair")
-    comp = compile_only(b, _bottleneck_pair(b, side_reader))
+    comp = compile_only(b, _bottleneck_pair(b, side_reader), fuse_shortcut_projection=0)
     groups = comp.fusion_groups().strip().splitlines()
     chains = [i for i, g in enumerate(groups) if "hip_conv2d_bn_relu_chain" in g]
     assert len(chains) == 1, groups
@@ -510,6 +510,16 @@ def test_two_pointwise_convolutions_in_a_row_become_one_call(side_reader):
     apart = compile_only(b, _bottleneck_pair(b, side_reader), fuse_conv_chain=0)
     assert "hip_conv2d_bn_relu_chain" not in apart.fusion_groups()
     assert apart.num_instructions() == comp.num_instructions() + 1
+    # by default the stride-1 projection shortcut becomes a second input of the call's first layer: x, x2, the two
+    # filters side by side, the summed shift, then the second layer's filter, scale and shift
+    b = NetBuilder("pair")
+    both = compile_only(b, _bottleneck_pair(b, side_reader))
+    lines = [g for g in both.fusion_groups().strip().splitlines() if "hip_conv2d_pair_chain" in g]
+    assert len(lines) == 1 and both.fusion_groups().count("hip_conv2d_bn_relu") == 1, both.fusion_groups()   # the 3x3 layer
+    ins = lines[0].split(" in: ")[1].split(" out: ")[0].split()
+    assert len(ins) == 7 and len(lines[0].split(" out: ")[1].split()) == 2, lines[0]
+    assert both.get_tensor(ins[2]).shape() == [256, 1, 1, 128]
+    assert both.num_instructions() == comp.num_instructions() - 1
 
 
 def test_pointwise_pairs_the_kernel_does_not_take_stay_two_calls():

@@ -153,10 +153,11 @@ def _two_bottlenecks(builder, x, params, side_reader=False):
 
 
 @pytest.mark.parametrize("side_reader", [False, True])
-@pytest.mark.parametrize("fuse", [1, 0])
+@pytest.mark.parametrize("fuse", [1, 0, 2])
 def test_program_with_two_bottlenecks(gpu, fuse, side_reader):
     """The rewrite turns the expansion + reduction pair into one instruction; the program's result stays within the
     fp16 bound of the oracle's evaluation of the operators as written, and of the program compiled without the rewrite.
+    fuse = 2: the projection shortcut becomes a second input of that instruction's first layer as well (the default).
     A const input named like a keyword of the kernel language ("short") must not reach the generated source as is."""
     from cinn_amd.common import DefaultAMDGPUTarget
     from cinn_amd.frontend import Computation
@@ -178,7 +179,7 @@ def test_program_with_two_bottlenecks(gpu, fuse, side_reader):
         b = NetBuilder("two_bottlenecks")
         xin, out, side = _two_bottlenecks(b, x, params, side_reader)
         comp = Computation.build_and_compile(DefaultAMDGPUTarget(), b, outputs=[out] + ([side] if side_reader else []),
-                                             fuse_conv_chain=fuse_chain)
+                                             fuse_conv_chain=fuse_chain != 0, fuse_shortcut_projection=fuse_chain == 2)
         comp.get_tensor("x").from_numpy(x)
         for name, arr in params.items():
             comp.get_tensor(name).from_numpy(arr)
@@ -190,7 +191,8 @@ def test_program_with_two_bottlenecks(gpu, fuse, side_reader):
     got, names, side_got = compiled(fuse)
     chains = [nm for nm in names if "chain" in nm]
     assert len(chains) == (1 if fuse else 0), names
-    other, other_names, side_other = compiled(1 - fuse)
+    assert ("pair_chain" in chains[0]) == (fuse == 2) if fuse else True
+    other, other_names, side_other = compiled(1 if fuse == 2 else 1 - fuse)
     assert len(names) == len(other_names) + (-1 if fuse else 1)
 
     # oracle: the operators as written, float64 sums, storage rounding after every folded layer
@@ -212,8 +214,10 @@ def test_program_with_two_bottlenecks(gpu, fuse, side_reader):
     assert np.all(np.abs(got - want) <= bound)
     assert np.all(np.abs(got - other) <= bound)
     if side_reader:
-        # 2 e, NCHW; the first result is the same bits with and without the rewrite
-        assert np.array_equal(side_got, side_other)
+        # 2 e, NCHW; the first result is the same bits with and without the two-layer rewrite (with the projection as
+        # a second input its scales are applied to the filter values: the same bound as against the oracle)
+        if fuse != 2:
+            assert np.array_equal(side_got, side_other)
         assert np.all(np.abs(side_got - 2 * e) <= 1e-2 * np.maximum(np.abs(2 * e), 0.05 * np.abs(e).max()))
 
 

@@ -173,3 +173,54 @@ def test_projection_shortcut_program_against_the_oracle(gpu, dtype_name, tol):
     assert np.abs(got - want).max() <= tol * scale, np.abs(got - want).max() / scale
     assert np.abs(apart - want).max() <= tol * scale
     assert np.abs(got - apart).max() <= tol * scale
+
+
+def _pair_chain_call(x, x2, w1, shift1, w2, scale2, shift2, relu_bits, dtype):
+    lib = _lib.load()
+    n, h, w_, c1 = x.shape
+    c2, n1, n2 = x2.shape[3], w1.shape[0], w2.shape[0]
+    bufs = [_dev(x, dtype), _dev(x2, dtype), _dev(w1.reshape(n1, 1, 1, c1 + c2), dtype),
+            runtime.DeviceBuffer.from_numpy(shift1.astype(np.float32), "float32"), _dev(w2.reshape(n2, 1, 1, n1), dtype),
+            runtime.DeviceBuffer.from_numpy(scale2.astype(np.float32), "float32"),
+            runtime.DeviceBuffer.from_numpy(shift2.astype(np.float32), "float32"),
+            runtime.DeviceBuffer((n, h, w_, n1), dtype), runtime.DeviceBuffer((n, h, w_, n2), dtype)]
+    args = runtime.pod_args(bufs)
+    lib.cinn_call_hip_conv2d_pair_chain.argtypes = [ctypes.c_void_p] + [ctypes.c_int] * 9 + [ctypes.c_void_p]
+    lib.cinn_call_hip_conv2d_pair_chain.restype = None
+    lib.cinn_call_hip_conv2d_pair_chain(args, 9, relu_bits, n, h, w_, c1, c2, n1, n2, None)
+    runtime.synchronize()
+    return _host(bufs[7], dtype), _host(bufs[8], dtype)
+
+
+@pytest.mark.parametrize("dtype,tol", [("float16", 2.0 ** -10), ("bfloat16", 2.0 ** -7)])
+@pytest.mark.parametrize("case", [
+    # (n, h, w, c1, c2, n1, n2, one kernel)
+    (32, 56, 56, 64, 64, 256, 64, True),     # ResNet-50's first block at batch 32: more groups than resident blocks
+    (1, 7, 16, 64, 64, 256, 64, True),       # seven groups of 16 pixels
+    (16, 28, 28, 128, 64, 256, 128, False),  # no one-kernel form: the first layer over both inputs, then the second layer
+])
+@pytest.mark.parametrize("relu_bits", [3, 0])
+def test_pair_chain_against_the_oracle(gpu, case, dtype, tol, relu_bits):
+    n, h, w_, c1, c2, n1, n2, one_kernel = case
+    rng = np.random.default_rng(900 + n + c1 + n2 + relu_bits)
+    x = _round(rng.standard_normal((n, h, w_, c1)), dtype)
+    x2 = _round(rng.standard_normal((n, h, w_, c2)), dtype)
+    w1 = _round(rng.standard_normal((n1, c1 + c2)) * np.sqrt(2.0 / (c1 + c2)), dtype)
+    w2 = _round(rng.standard_normal((n2, n1)) * np.sqrt(2.0 / n1), dtype)
+    t1 = rng.standard_normal(n1).astype(np.float32) * 0.1
+    s2, t2 = rng.uniform(0.5, 1.5, n2).astype(np.float32), rng.standard_normal(n2).astype(np.float32) * 0.1
+    e, y = _pair_chain_call(x, x2, w1, t1, w2, s2, t2, relu_bits, dtype)
+    want_e, mag_e = _oracle_pair(x, x2, w1, t1, relu_bits & 1, (1, 1))
+    assert np.all(np.abs(e - want_e) <= tol * np.maximum(np.abs(want_e), 1e-2 * mag_e) + 1e-6)
+    # the second layer from the first result as the device stored it
+    want_y = _mm(e.reshape(-1, n1), w2) * s2 + t2
+    mag_y = _mm(np.abs(e.reshape(-1, n1)), np.abs(w2)) * s2 + np.abs(t2)
+    if relu_bits & 2:
+        want_y = np.maximum(want_y, 0)
+    got_y = y.reshape(-1, n2)
+    assert np.all(np.abs(got_y - want_y) <= tol * np.maximum(np.abs(want_y), 1e-2 * mag_y) + 1e-6)
+    if one_kernel:
+        # the first layer alone through the call that takes two inputs gives the same sums in another order
+        if n * h * w_ >= 24576:
+            alone = _pair_call(x, x2, w1, t1, relu_bits & 1, (1, 1), dtype)
+            assert np.all(np.abs(e - alone) <= tol * np.maximum(np.abs(want_e), 1e-2 * mag_e) + 1e-6)

@@ -89,18 +89,21 @@ def test_resnet50_fp16_batch2_matches_oracle(gpu):
     fused, comp = gpu_forward(params, x, fuse_conv_bn_relu=True)
     # every batch norm, residual addition and relu now lives in a convolution epilogue, and the max pooling in the
     # image convolution: 53 convolutions - three pairs of them (an expansion 64 -> 256 and the reduction that reads it)
-    # in one call each -, the global pooling, the classifier with its bias as the shift of its epilogue (the reshapes
-    # around it are views)
-    assert comp.num_instructions() == 50 + 1 + 1, comp.fusion_groups()
+    # in one call each, the first of them with the first stage's projection shortcut as a second input -, the global
+    # pooling, the classifier with its bias as the shift of its epilogue (the reshapes around it are views)
+    assert comp.num_instructions() == 49 + 1 + 1, comp.fusion_groups()
     assert_logits_close_fp16(fused, want)
     one_call_per_layer, comp = gpu_forward(params, x, fuse_conv_chain=False)
     assert comp.num_instructions() == 53 + 1 + 1, comp.fusion_groups()
     assert_logits_close_fp16(one_call_per_layer, want)
     apart, comp = gpu_forward(params, x, fuse_stem_pool=False)
-    assert comp.num_instructions() == 50 + 2 + 1
+    assert comp.num_instructions() == 49 + 2 + 1
     assert np.array_equal(apart, fused)
     two_ops, comp = gpu_forward(params, x, fuse_matmul_bias=False)
-    assert comp.num_instructions() == 50 + 1 + 2
+    assert comp.num_instructions() == 49 + 1 + 2
+    own_projections, comp = gpu_forward(params, x, fuse_shortcut_projection=False)
+    assert comp.num_instructions() == 50 + 1 + 1
+    assert_logits_close_fp16(own_projections, want)
     assert_logits_close_fp16(two_ops, want)
 
 
@@ -145,9 +148,9 @@ def test_resnet50_batch32(gpu, dtype, tol):
     want = torch_forward(params, x)
     assert np.abs(got.astype(np.float64) - want).max() <= tol * np.abs(want).max()
     if dtype == "float16":
-        # at this batch size the projection shortcuts of stages 2-4 share a call with the layer that adds them (the
-        # first stage's expansion is half of a two-layer call already)
-        assert comp.num_instructions() == 47 + 1 + 1, comp.fusion_groups()
+        # at this batch size the projection shortcuts of stages 2-4 share a call with the layer that adds them as well
+        # (the first stage's is a second input of a two-layer call at any batch size)
+        assert comp.num_instructions() == 46 + 1 + 1, comp.fusion_groups()
         apart, comp_apart = gpu_forward(params, x, fuse_shortcut_projection=False)
         assert comp_apart.num_instructions() == 50 + 1 + 1, comp_apart.fusion_groups()
         assert np.abs(apart.astype(np.float64) - want).max() <= tol * np.abs(want).max()
@@ -182,8 +185,9 @@ def test_resnet50_hip_graph_replay_matches_eager(gpu, monkeypatch):
     _, comp = gpu_forward(params, x, stream=stream)
     lanes = comp.graph_lanes()
     assert len(lanes) == comp.num_instructions()
-    # four blocks have a projection shortcut: in each, either it or the main branch leaves the first lane
-    assert lanes[0] == 0 and sum(1 for a, b in zip(lanes, lanes[1:]) if a == 0 and b == 1) >= 4, lanes
+    # three blocks have a projection shortcut that is an instruction of its own at this batch size (the first stage's is
+    # a second input of a two-layer call): in each, either it or the main branch leaves the first lane
+    assert lanes[0] == 0 and sum(1 for a, b in zip(lanes, lanes[1:]) if a == 0 and b == 1) >= 3, lanes
     out = comp.output_names()[0]
     for data, want in ((x, eager), (x, eager), (x2, eager2), (x, eager)):
         comp.get_tensor("image").from_numpy(data)
