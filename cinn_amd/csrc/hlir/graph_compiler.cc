@@ -457,6 +457,23 @@ ir::Module GraphCompiler::LowerGraph(const CompileOptions& options) {
   KernelMergeOptions merge;
   const char* flag = getenv("FLAGS_cinn_hip_merge_kernels");
   merge.enabled    = options.merge_independent_kernels && !(flag && flag[0] == '0');
+  if (merge.enabled && options.lowering.merged_rows_per_wave > 1) {
+    // Which groups will share a launch is known once every kernel exists; row-reduce members are then lowered again
+    // with that knowledge (a member's schedule may differ from the one it has alone, its block shape does not).
+    std::vector<ir::LoweredFuncRef> trial;
+    for (auto& unit : MergeIndependentKernels(graph_->groups, funcs, barrier, merge, &trial)) {
+      if (unit.members.size() < 2) continue;
+      for (const Group* member : unit.members) {
+        if (member->kind != GroupKind::kRowReduce) continue;
+        for (size_t i = 0; i < graph_->groups.size(); ++i) {
+          if (graph_->groups[i].get() != member) continue;
+          auto func = lowerer.Lower(*member, /*merged_member=*/true);
+          if (func->is_device) optim::OptimizeFuncGPU(func.get());
+          funcs[i] = func;
+        }
+      }
+    }
+  }
   units_           = MergeIndependentKernels(graph_->groups, funcs, barrier, merge, &module.functions);
   return module;
 }

@@ -38,6 +38,26 @@ std::string CName(const std::string& id) {
       "volatile", "while", "xor", "half", "float16", "bfloat16", "threadIdx", "blockIdx", "blockDim", "gridDim", "warpSize",
       "int8_t", "int16_t", "int32_t", "int64_t", "uint8_t", "uint16_t", "uint32_t", "uint64_t", "size_t", "min", "max"};
   if (reserved.count(out)) out = "v_" + out;
+  // ... or like a name the generated code uses for its own variables: the loop and index variables, the numbered
+  // temporaries (<hint>_<n>) and the members of a merged kernel (m<k>_...)
+  auto all_digits = [](const std::string& t) {
+    return !t.empty() && std::all_of(t.begin(), t.end(), [](char c) { return isdigit(static_cast<unsigned char>(c)); });
+  };
+  static const std::set<std::string> loop_vars = {"i",  "j",  "k",  "r",  "u",   "io",  "ki",  "kc", "kl", "ks", "rr",
+                                                  "tx", "ty", "bx", "bid", "row", "col", "kernel_args", "kernel_args_num",
+                                                  "kernel_stream"};
+  bool local = loop_vars.count(out) > 0;
+  const size_t us = out.rfind('_');
+  if (!local && us != std::string::npos && all_digits(out.substr(us + 1))) {
+    static const std::set<std::string> hints = {"acc", "acc_idx", "t",  "o",  "base", "red", "rcp",  "r",  "q0",
+                                                "n0",  "last",    "kv", "cv", "b",    "a",   "x",    "tile", "res"};
+    local = hints.count(out.substr(0, us)) > 0;
+  }
+  if (!local && out.size() >= 3 && out[0] == 'm') {
+    const size_t first_us = out.find('_');
+    local = first_us != std::string::npos && all_digits(out.substr(1, first_us - 1));
+  }
+  if (local) out = "v_" + out;
   return out;
 }
 
@@ -247,6 +267,7 @@ LoweringOptions LoweringOptions::FromEnv() {
   o.nontemporal_store_bytes     = static_cast<int64_t>(EnvInt("FLAGS_cinn_hip_nontemporal_store_mb", 8)) << 20;
   o.nontemporal_load_bytes      = static_cast<int64_t>(EnvInt("FLAGS_cinn_hip_nontemporal_load_mb", 0)) << 20;
   o.rows_per_wave               = EnvInt("FLAGS_cinn_hip_reduce_rows_per_wave", o.rows_per_wave);
+  o.merged_rows_per_wave        = EnvInt("FLAGS_cinn_hip_merged_rows_per_wave", o.merged_rows_per_wave);
   o.elementwise_block           = EnvInt("FLAGS_cinn_hip_elementwise_block", o.elementwise_block);
   o.rows_per_block              = EnvInt("FLAGS_cinn_hip_reduce_rows_per_block", o.rows_per_block);
   o.column_reduce               = EnvInt("FLAGS_cinn_hip_column_reduce", 1) != 0;
@@ -265,10 +286,10 @@ std::vector<NodeData*> OpLowerer::ArgumentsOf(const Group& group) {
   return args;
 }
 
-ir::LoweredFuncRef OpLowerer::Lower(const Group& group) const {
+ir::LoweredFuncRef OpLowerer::Lower(const Group& group, bool merged_member) const {
   switch (group.kind) {
     case GroupKind::kElementwise: return LowerElementwise(group);
-    case GroupKind::kRowReduce: return LowerRowReduce(group);
+    case GroupKind::kRowReduce: return LowerRowReduce(group, merged_member);
     case GroupKind::kGeneralReduce: return LowerGeneralReduce(group);
     case GroupKind::kLibraryCall: return LowerLibraryCall(group);
   }
@@ -991,7 +1012,7 @@ class RowReduceEmitter {
 
 }  // namespace
 
-ir::LoweredFuncRef OpLowerer::LowerRowReduce(const Group& group) const {
+ir::LoweredFuncRef OpLowerer::LowerRowReduce(const Group& group, bool merged_member) const {
   GroupContext ctx(group);
   MarkStreamingOutputs(&ctx, options_.nontemporal_store_bytes);
   MarkStreamingInputs(&ctx, options_.nontemporal_load_bytes);
@@ -1049,6 +1070,17 @@ ir::LoweredFuncRef OpLowerer::LowerRowReduce(const Group& group) const {
   int rows_per_wave = 1;
   if (plan.team == wave) {
     rows_per_wave = std::max(1, options_.rows_per_wave);
+    if (merged_member && rows_per_wave == 1 && options_.merged_rows_per_wave > 1) {
+      // A member of a merged launch runs at the occupancy the heaviest member's registers allow.  Wavefronts that
+      // request at most 32 bytes per lane for a row and leave then have too few bytes in flight per CU: such rows are
+      // taken several per wavefront.
+      int64_t row_bytes = 0;  // what a lane requests per row
+      for (auto& kv : kinds)
+        if (!ctx.produced.count(kv.first) && kv.second == RowKind::kElem) row_bytes += per_lane * kv.first->dtype.bytes();
+      while (rows_per_wave * 2 <= options_.merged_rows_per_wave && row_bytes * rows_per_wave * 2 <= 64 &&
+             plan.rows % (static_cast<int64_t>(plan.rows_per_block) * rows_per_wave * 2) == 0)
+        rows_per_wave *= 2;
+    }
   }
   Expr bx = ir::MakeVar("bx", common::Int(32));
   Expr ty = ir::MakeVar("ty", common::Int(32));

@@ -41,6 +41,11 @@ struct LoweringOptions {
   // rows one wavefront works through (unrolled, so their loads overlap).  Measured on MI355X this does
   // not pay for the BASELINE shapes (1 is the best setting for every one of them), so it stays a knob.
   int rows_per_wave{1};
+  // the same for a row-reduce group that becomes a member of a merged launch (hlir/kernel_merge.h) and requests at
+  // most 32 bytes per lane and row: there the heaviest member's registers set the occupancy of all, and such rows need
+  // two per wavefront to keep as many bytes in flight as their own kernel has (configs[1] step: 64.5 -> 62.5 us;
+  // four rows, or two rows of 64 bytes per lane, measured slower).  1 switches it off.
+  int merged_rows_per_wave{2};
   // reductions over one non-trailing run of axes use the column-reduce kernel (off: one thread per output element)
   bool column_reduce{true};
   // element-wise groups around a transpose that moves the innermost axis stage the input through LDS tiles
@@ -55,13 +60,14 @@ class OpLowerer {
   OpLowerer(const common::Target& target, const LoweringOptions& options = LoweringOptions::FromEnv());
   // One function per group.  Device functions come back scheduled, with loops still carrying their
   // GPU bindings (optim::OptimizeFuncGPU turns them into a kernel body and launch dimensions).
-  ir::LoweredFuncRef Lower(const Group& group) const;
+  // merged_member: the group's kernel will share a launch with others (see merged_rows_per_wave)
+  ir::LoweredFuncRef Lower(const Group& group, bool merged_member = false) const;
   // argument order of the function generated for `group`: inputs, then outputs
   static std::vector<NodeData*> ArgumentsOf(const Group& group);
 
  private:
   ir::LoweredFuncRef LowerElementwise(const Group& group) const;
-  ir::LoweredFuncRef LowerRowReduce(const Group& group) const;
+  ir::LoweredFuncRef LowerRowReduce(const Group& group, bool merged_member) const;
   ir::LoweredFuncRef LowerGeneralReduce(const Group& group) const;
   ir::LoweredFuncRef LowerLibraryCall(const Group& group) const;
   common::Target target_;

@@ -593,3 +593,15 @@ def test_tensor_names_that_are_keywords_of_the_kernel_language():
     src = comp.source_code()
     assert "v_short" in src and "v_float" in src
     assert comp.get_tensor("short") is not None
+    # ... nor may a tensor take the name of a variable the generated code declares itself: loop and index variables
+    # (i, j, row, col, ...), numbered temporaries (t_3, acc_0), the prefix of a merged kernel's members (m1_...)
+    b = NetBuilder("locals")
+    names = ["i", "j", "k", "row", "col", "t_3", "acc_0", "m1_x"]
+    ins = [b.create_input(Float(32), [64, 512], n) for n in names]
+    total = ins[0]
+    for v in ins[1:]:
+        total = b.add(total, v)
+    comp = compile_only(b, [b.reduce_sum(total, [1]), b.softmax(ins[1], axes=[-1])])
+    src = comp.source_code()
+    for n in names:
+        assert "__restrict__ v_%s" % n in src and comp.get_tensor(n) is not None, n

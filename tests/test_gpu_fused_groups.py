@@ -303,3 +303,39 @@ def test_sibling_elementwise_groups_share_their_input_and_dependent_ones_stay_ap
     assert comp.num_instructions() >= 2, comp.fusion_groups()
     np.testing.assert_allclose(y, a - a.sum(1, keepdims=True, dtype=np.float32), rtol=1e-5, atol=1e-5)
     np.testing.assert_allclose(cols, a.sum(0), rtol=1e-5, atol=1e-5)
+
+
+def test_light_members_of_a_merged_launch_take_two_rows_per_wavefront(gpu):
+    """Independent kernels of one program share a launch; there a row reduction that requests at most 32 bytes per lane
+    and row works through two rows per wavefront (its own kernel takes one).  Results: bit-exact for the integer
+    members, the oracle's bar for softmax; the same values as the program compiled with one launch per group."""
+    import oracle
+    from cinn_amd.common import Int
+    rng = np.random.default_rng(41)
+    xs = rng.standard_normal((64, 4096)).astype(np.float32)
+    xi = rng.integers(-1000, 1001, (1030, 512)).astype(np.int32)       # 1030 rows: not a multiple of 2 x 4 rows
+    xj = rng.integers(-1000, 1001, (2048, 512)).astype(np.int32)
+    xj[5] = 7                                                           # a constant row: the first index wins
+
+    def program(**options):
+        b = NetBuilder("merged_rows")
+        S = b.create_input(Float(32), xs.shape, "s")
+        I = b.create_input(Int(32), xi.shape, "i")
+        J = b.create_input(Int(32), xj.shape, "j")
+        outs = [b.softmax(S, axes=[-1]), b.reduce_sum(I, [1]), b.reduce_sum(J, [1]), b.argmax(J, axis=1)]
+        got, comp = run(b, {S: xs, I: xi, J: xj}, outs, **options)
+        return got, comp
+
+    got, comp = program()
+    assert comp.num_instructions() == 1, comp.fusion_groups()
+    src = comp.source_code()
+    # the sum and the argmax over [2048, 512] (siblings: one group) take two rows per wavefront; 1030 rows do not divide
+    # by 2 x 4 and keep one, and so does the softmax with its 256 bytes per lane
+    assert src.count("rr < 2") == 1, src.count("rr < 2")
+    apart, comp1 = program(merge_independent_kernels=False)
+    assert comp1.num_instructions() == 3 and "rr < 2" not in comp1.source_code()
+    np.testing.assert_allclose(got[0], oracle.softmax(xs), rtol=1e-5, atol=0)
+    assert np.array_equal(got[1], xi.sum(1, dtype=np.int32)) and np.array_equal(got[2], xj.sum(1, dtype=np.int32))
+    assert np.array_equal(got[3], np.argmax(xj, 1).astype(np.int32)) and got[3][5] == 0
+    for a, c in zip(got, apart):
+        assert np.array_equal(a, c)
