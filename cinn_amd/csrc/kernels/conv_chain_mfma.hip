@@ -67,8 +67,9 @@ struct ChainParams {
   int groups;  // M / 16
 };
 
-template <typename T, int K1, int N1, int N2, int WAVES, int K1B = 0>
+template <typename T, int K1, int N1, int N2, int WAVES, int K1B = 0, bool RES = false>
 __global__ void __launch_bounds__(64 * WAVES) conv1x1_chain_kernel(ChainParams p) {
+  static_assert(!(RES && K1B > 0), "a second input takes the place of the residual");
   typedef typename Mfma16<T>::vec8 vec8;
   constexpr int THREADS = 64 * WAVES;
   constexpr int KT      = K1 + K1B;            // channels of the first product: X's, then X2's
@@ -133,7 +134,9 @@ __global__ void __launch_bounds__(64 * WAVES) conv1x1_chain_kernel(ChainParams p
 
   int g = blockIdx.x;
   if (g >= p.groups) return;
-  const T* const R = K1B == 0 ? reinterpret_cast<const T*>(p.residual) : nullptr;
+  // whether there is a residual is a template parameter: with a run-time condition around its loads the compiler
+  // cannot count the loads in flight (see the request below)
+  const T* const R = RES ? reinterpret_cast<const T*>(p.residual) : nullptr;
   T* const E       = reinterpret_cast<T*>(p.e);
   T* const Y       = reinterpret_cast<T*>(p.y);
   // a thread's chunk of pass i: row i (THREADS / CPR) + tid / CPR of the group, columns 8 (tid % CPR) ..
@@ -162,7 +165,10 @@ __global__ void __launch_bounds__(64 * WAVES) conv1x1_chain_kernel(ChainParams p
     for (int u = 0; u < 2; ++u) {
       const int gn        = g + (int)gridDim.x;
       const bool has_next = gn < p.groups;
-      if (has_next) request(gn, xa[u ^ 1], rr[u ^ 1]);
+      // Requested whether or not there is a next group (then the last group's rows once more, unused): with a request
+      // that depends on a condition the compiler cannot count the loads in flight at the first use of this group's
+      // rows and waits for all of them - the ones requested a moment ago included, i.e. no group is ever fetched ahead
+      request(has_next ? gn : p.groups - 1, xa[u ^ 1], rr[u ^ 1]);
       // ---- first product: this wavefront's J1 tiles of the group's 16 pixels
       f32x4 acc1[J1];
 #pragma unroll
@@ -245,7 +251,11 @@ template <typename T, int K1, int N1, int N2, int WAVES, int BLOCKS_PER_CU, int 
 void LaunchChain(const ChainParams& p, hipStream_t stream) {
   const int resident = 256 * BLOCKS_PER_CU;
   dim3 grid(p.groups < resident ? p.groups : resident);
-  hipLaunchKernelGGL((conv1x1_chain_kernel<T, K1, N1, N2, WAVES, K1B>), grid, dim3(64 * WAVES), 0, stream, p);
+  if (K1B == 0 && p.residual != nullptr) {
+    hipLaunchKernelGGL((conv1x1_chain_kernel<T, K1, N1, N2, WAVES, 0, true>), grid, dim3(64 * WAVES), 0, stream, p);
+  } else {
+    hipLaunchKernelGGL((conv1x1_chain_kernel<T, K1, N1, N2, WAVES, K1B, false>), grid, dim3(64 * WAVES), 0, stream, p);
+  }
 }
 
 // 1: where the shape qualifies (default), 0: never; -1: not read yet
