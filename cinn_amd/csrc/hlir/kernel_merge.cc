@@ -32,6 +32,26 @@ bool SameBlock(const ir::LoweredFunc& a, const ir::LoweredFunc& b) {
   return true;
 }
 
+// A block of bx x by threads whose body can run in a flat block of bx * by threads, with threadIdx.x and threadIdx.y
+// recovered from the flat index: bx a power of two, no third axis, no use of the block's extents (the device library's
+// wave and block reductions work on the linear thread index; the column reduction walks blockDim.y and is excluded
+// by the group kinds that get here).
+bool Flattenable(const Group& g, const ir::LoweredFunc& f) {
+  if (g.kind != GroupKind::kElementwise && g.kind != GroupKind::kRowReduce) return false;
+  const int bx = f.axis_info.block[0];
+  if (f.axis_info.block[2] != 1 || bx <= 0 || (bx & (bx - 1)) != 0) return false;
+  for (const char* v : {"blockDim.x", "blockDim.y", "blockDim.z", "threadIdx.z"})
+    if (ir::UsesVar(f.body, v)) return false;
+  return true;
+}
+
+// same block shape, or both runnable as a flat block of the same number of threads
+bool CompatibleBlock(const Group& ga, const ir::LoweredFunc& a, const Group& gb, const ir::LoweredFunc& b) {
+  if (SameBlock(a, b)) return true;
+  return Flattenable(ga, a) && Flattenable(gb, b) &&
+         a.axis_info.block[0] * a.axis_info.block[1] == b.axis_info.block[0] * b.axis_info.block[1];
+}
+
 LaunchUnit UnitOf(const Group& g) {
   LaunchUnit u;
   u.func_name = g.func_name;
@@ -65,7 +85,7 @@ std::vector<LaunchUnit> MergeIndependentKernels(const std::vector<std::unique_pt
     size_t end     = i + 1;
     while (end < groups.size() && static_cast<int>(end - i) < options.max_members) {
       const Group& g = *groups[end];
-      if (barrier[end] || !Mergeable(*funcs[end]) || !SameBlock(*funcs[i], *funcs[end]) || g.pre_run != first.pre_run) break;
+      if (barrier[end] || !Mergeable(*funcs[end]) || !CompatibleBlock(first, *funcs[i], g, *funcs[end]) || g.pre_run != first.pre_run) break;
       bool depends = false;
       for (auto* in : g.inputs) depends |= written.count(in) > 0;
       if (depends) break;
@@ -87,6 +107,13 @@ std::vector<LaunchUnit> MergeIndependentKernels(const std::vector<std::unique_pt
     merged->is_device = true;
     merged->axis_info = funcs[i]->axis_info;
     merged->axis_info.grid[0] = static_cast<int>(blocks);
+    // members of different block shapes: the launch is a flat block and every member recovers its own threadIdx.x / y
+    bool flat = false;
+    for (size_t k = i + 1; k < end; ++k) flat = flat || !SameBlock(*funcs[i], *funcs[k]);
+    if (flat) {
+      merged->axis_info.block[0] = funcs[i]->axis_info.block[0] * funcs[i]->axis_info.block[1];
+      merged->axis_info.block[1] = 1;
+    }
     merged->name = first.func_name + "_and_" + std::to_string(end - i - 1) + "_more";
     std::map<std::string, ir::Argument> arg_of;  // by buffer name: the first member's buffer object is declared
     for (size_t k = i; k < end; ++k) {
@@ -139,6 +166,16 @@ std::vector<LaunchUnit> MergeIndependentKernels(const std::vector<std::unique_pt
         merged->temp_bufs.push_back(buf);
       }
       Expr body = start == 0 ? funcs[k]->body : ir::Substitute(funcs[k]->body, "blockIdx.x", block_x - Expr(static_cast<int>(start)));
+      if (flat && funcs[k]->axis_info.block[1] > 1) {
+        const int bx = funcs[k]->axis_info.block[0];
+        int shift    = 0;
+        while ((1 << shift) < bx) ++shift;
+        const std::string tag = "m" + std::to_string(k - i);
+        Expr tx = ir::MakeVar(tag + "_tx", common::Int(32)), ty = ir::MakeVar(tag + "_ty", common::Int(32));
+        Expr tid = ir::MakeVar("threadIdx.x", common::Int(32));
+        body = ir::Substitute(ir::Substitute(body, "threadIdx.x", tx), "threadIdx.y", ty);
+        body = ir::MakeBlock({ir::MakeLet(tx, tid % Expr(bx)), ir::MakeLet(ty, tid / Expr(bx)), body});
+      }
       if (!chain.defined()) {
         chain = ir::MakeBlock({body});  // the last member takes every remaining block
       } else {

@@ -339,3 +339,36 @@ def test_light_members_of_a_merged_launch_take_two_rows_per_wavefront(gpu):
     assert np.array_equal(got[3], np.argmax(xj, 1).astype(np.int32)) and got[3][5] == 0
     for a, c in zip(got, apart):
         assert np.array_equal(a, c)
+
+
+def test_kernels_of_different_block_shapes_share_a_flat_launch(gpu):
+    """An element-wise kernel (256 x 1 threads), a wavefront-per-row reduction (64 x 4), a block-per-row softmax
+    (256 x 1) and a team-per-row reduction (16 x 16) that do not depend on each other run as one launch of flat
+    256-thread blocks; every member recovers its own thread coordinates.  Same values as one launch per group."""
+    import oracle
+    from cinn_amd.common import Int
+    rng = np.random.default_rng(43)
+    a = rng.uniform(-1, 1, (300, 1000)).astype(np.float32)
+    s = rng.standard_normal((50, 4096)).astype(np.float32)      # with reduce_wave_elems=32: a block of 256 threads per row
+    xi = rng.integers(-1000, 1001, (1031, 512)).astype(np.int32)
+    xt = rng.integers(-1000, 1001, (777, 60)).astype(np.int32)  # short rows: teams of 16 lanes
+
+    def program(**options):
+        b = NetBuilder("flat")
+        A = b.create_input(Float(32), a.shape, "a")
+        S = b.create_input(Float(32), s.shape, "s")
+        I = b.create_input(Int(32), xi.shape, "xi")
+        Tn = b.create_input(Int(32), xt.shape, "xt")
+        outs = [b.relu(A), b.softmax(S, axes=[-1]), b.reduce_sum(I, [1]), b.reduce_max(Tn, [1])]
+        return run(b, {A: a, S: s, I: xi, Tn: xt}, outs, reduce_wave_elems=32, **options)
+
+    got, comp = program()
+    assert comp.num_instructions() == 1, comp.fusion_groups()
+    assert "cinn_block_reduce" in comp.source_code()
+    apart, comp1 = program(merge_independent_kernels=False)
+    assert comp1.num_instructions() == 4
+    assert np.array_equal(got[0], np.maximum(a, 0))
+    np.testing.assert_allclose(got[1], oracle.softmax(s), rtol=1e-5, atol=0)
+    assert np.array_equal(got[2], xi.sum(1, dtype=np.int32)) and np.array_equal(got[3], xt.max(1))
+    for x, y in zip(got, apart):
+        assert np.array_equal(x, y)
