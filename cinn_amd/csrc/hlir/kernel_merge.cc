@@ -45,12 +45,7 @@ bool Flattenable(const Group& g, const ir::LoweredFunc& f) {
   return true;
 }
 
-// same block shape, or both runnable as a flat block of the same number of threads
-bool CompatibleBlock(const Group& ga, const ir::LoweredFunc& a, const Group& gb, const ir::LoweredFunc& b) {
-  if (SameBlock(a, b)) return true;
-  return Flattenable(ga, a) && Flattenable(gb, b) &&
-         a.axis_info.block[0] * a.axis_info.block[1] == b.axis_info.block[0] * b.axis_info.block[1];
-}
+int Threads(const ir::LoweredFunc& f) { return f.axis_info.block[0] * f.axis_info.block[1] * f.axis_info.block[2]; }
 
 LaunchUnit UnitOf(const Group& g) {
   LaunchUnit u;
@@ -83,15 +78,27 @@ std::vector<LaunchUnit> MergeIndependentKernels(const std::vector<std::unique_pt
     std::set<const NodeData*> written(first.outputs.begin(), first.outputs.end());
     int64_t blocks = funcs[i]->axis_info.grid[0];
     size_t end     = i + 1;
+    // A run keeps one block shape, or - once a member of another shape joins - every member must be able to run in a
+    // flat block of the same number of threads (a member that cannot, e.g. a column reduction, shares launches only
+    // with kernels of its own shape).
+    bool run_flat        = false;
+    bool all_flattenable = Flattenable(first, *funcs[i]);
     while (end < groups.size() && static_cast<int>(end - i) < options.max_members) {
       const Group& g = *groups[end];
-      if (barrier[end] || !Mergeable(*funcs[end]) || !CompatibleBlock(first, *funcs[i], g, *funcs[end]) || g.pre_run != first.pre_run) break;
+      if (barrier[end] || !Mergeable(*funcs[end]) || g.pre_run != first.pre_run) break;
+      const bool same   = SameBlock(*funcs[i], *funcs[end]);
+      const bool g_flat = Flattenable(g, *funcs[end]);
+      if (run_flat || !same) {
+        if (!all_flattenable || !g_flat || Threads(*funcs[i]) != Threads(*funcs[end])) break;
+      }
       bool depends = false;
       for (auto* in : g.inputs) depends |= written.count(in) > 0;
       if (depends) break;
       if (blocks + funcs[end]->axis_info.grid[0] > 0x7fffffff) break;
       blocks += funcs[end]->axis_info.grid[0];
       written.insert(g.outputs.begin(), g.outputs.end());
+      run_flat        = run_flat || !same;
+      all_flattenable = all_flattenable && g_flat;
       ++end;
     }
     if (end - i < 2) {

@@ -372,3 +372,23 @@ def test_kernels_of_different_block_shapes_share_a_flat_launch(gpu):
     assert np.array_equal(got[2], xi.sum(1, dtype=np.int32)) and np.array_equal(got[3], xt.max(1))
     for x, y in zip(got, apart):
         assert np.array_equal(x, y)
+
+
+def test_a_column_reduction_shares_launches_only_with_kernels_of_its_own_block_shape(gpu):
+    """The reduction over a non-trailing axis walks blockDim.y in the device library, so it cannot run in a flat block:
+    next to a team-per-row kernel of the same 16 x 16 shape it shares a launch as it is, and an element-wise kernel
+    (256 x 1) that follows stays a launch of its own instead of flattening the run."""
+    import oracle
+    rng = np.random.default_rng(47)
+    x = rng.uniform(-2, 2, (13, 15)).astype(np.float32)
+    y = rng.uniform(-2, 2, (13, 15)).astype(np.float32)
+    b = NetBuilder("colred")
+    X = b.create_input(Float(32), x.shape, "x")
+    Y = b.create_input(Float(32), y.shape, "y")
+    outs = [b.softmax(X, axes=[-1]), b.reduce_max(X, [0], keep_dim=True), b.min(Y, X)]
+    got, comp = run(b, {X: x, Y: y}, outs)
+    names = [comp.instruction_info(i)[0] for i in range(comp.num_instructions())]
+    assert len(names) == 2 and "and_1_more" in names[0], names
+    assert "_tx = " not in comp.source_code()            # nobody was flattened
+    np.testing.assert_allclose(got[0], oracle.softmax(x), rtol=1e-5, atol=0)
+    assert np.array_equal(got[1], x.max(0, keepdims=True)) and np.array_equal(got[2], np.minimum(y, x))
