@@ -137,7 +137,13 @@ struct WaveMma {
 };
 
 // ---- the kernel -----------------------------------------------------------------------------------------------
-template <typename T, int BM, int BN, int WM, int WN, bool NCHW_IN, int PF>
+// FAST (channels-last loader, C a multiple of one K step, both operands below 2 GiB): a K step lies inside one filter
+// tap, so the tap and its channel offset are block-uniform and advance on the scalar unit; chunks are fetched with raw
+// buffer loads whose range check returns zeros for a chunk outside the image (its offset is replaced by one beyond the
+// tensor) - no page of zeros, no 64-bit address arithmetic, no select per address half.  The fp32 MFMAs run on the same
+// lanes as the other vector instructions (64 more of those per K step cost the fp32 kernel 17-22 %), so every vector
+// instruction the loader does not execute is matrix time: 63 -> 14 per K step.
+template <typename T, int BM, int BN, int WM, int WN, bool NCHW_IN, int PF, bool FAST>
 __global__ void __launch_bounds__(64 * WM * WN)
 conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, const float* __restrict__ scale,
                       const float* __restrict__ shift, const T* residual, float* __restrict__ workspace,
@@ -221,7 +227,15 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   const int step0       = blockIdx.y * p.steps_per_split;
   const int step1       = step0 + p.steps_per_split < total_steps ? step0 + p.steps_per_split : total_steps;
   int ck = 0, dy = 0, dx = 0;
-  if (!NCHW_IN) {
+  static_assert(!(FAST && NCHW_IN), "the uniform-tap loader reads channels-last images");
+  if (FAST) {
+    // block-uniform: ck is the channel offset of the step's first chunk
+    int kc  = step0 * BK;
+    int tap = FastDiv(kc, p.magic_c, p.shift_c);
+    ck      = kc - tap * p.c;
+    dy      = FastDiv(tap, p.magic_kw, p.shift_kw);
+    dx      = tap - dy * p.kw;
+  } else if (!NCHW_IN) {
     int kc  = step0 * BK + cc * E;
     int tap = FastDiv(kc, p.magic_c, p.shift_c);
     ck      = kc - tap * p.c;
@@ -236,6 +250,20 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
     wrow[i] = oc < p.oc ? oc * p.k_total : -1;  // checked on the host: oc * k_total < 2^31
   }
 
+  // uniform-tap loader: byte offsets of this thread's chunk of each row at tap (0, 0), channel 0 (a window origin may
+  // lie before the tensor: the 32-bit sum with the tap's offset is what has to be in range), and the two buffers
+  unsigned a_off[RA], b_off[RB];
+  __amdgpu_buffer_rsrc_t x_rsrc, w_rsrc;
+  if constexpr (FAST) {
+#pragma unroll
+    for (int i = 0; i < RA; ++i) a_off[i] = (unsigned)(base[i] + cc * E) * (unsigned)sizeof(T);
+#pragma unroll
+    for (int i = 0; i < RB; ++i)  // a filter row beyond OC stays out of range whatever is added (operands < 2 GiB)
+      b_off[i] = wrow[i] >= 0 ? (unsigned)(wrow[i] + cc * E) * (unsigned)sizeof(T) : 0x80000000u;
+    x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(x), 0, p.n * p.h * p.w * p.c * (int)sizeof(T), 0x00020000);
+    w_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(w), 0, p.oc * p.k_total * (int)sizeof(T), 0x00020000);
+  }
+
   // Register slots for the K steps in flight: the loads of step s + PF are issued while step s is computed, so a
   // block keeps PF steps of global-memory latency covered by itself (slot of step t: t % PF).
   u32x4 ra_slots[PF][RA], rb_slots[PF][RB];
@@ -245,7 +273,27 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   const T* zeros = static_cast<const T*>(zero_page);
   auto load_step = [&](int step, u32x4 (&ra)[RA], u32x4 (&rb)[RB]) {
     const bool live = step < step1;
-    if (!NCHW_IN) {
+    if constexpr (FAST) {
+      // steps beyond this block's range fetch something in range or zeros; nothing multiplies what they bring
+      const int dyo = dy * p.dil_h, dxo = dx * p.dil_w;
+      const unsigned tap_bytes = (unsigned)((dyo * p.w + dxo) * p.c + ck) * (unsigned)sizeof(T);
+#pragma unroll
+      for (int i = 0; i < RA; ++i) {
+        const bool ok = (unsigned)(ih0[i] + dyo) < (unsigned)p.h && (unsigned)(iw0[i] + dxo) < (unsigned)p.w;
+        ra[i] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, ok ? a_off[i] + tap_bytes : 0x80000000u, 0, 0);
+      }
+      const unsigned kb_bytes = (unsigned)(step * BK) * (unsigned)sizeof(T);
+#pragma unroll
+      for (int i = 0; i < RB; ++i) rb[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, b_off[i] + kb_bytes, 0, 0);
+      ck += BK;
+      if (ck == p.c) {
+        ck = 0;
+        if (++dx == p.kw) {
+          dx = 0;
+          ++dy;
+        }
+      }
+    } else if (!NCHW_IN) {
       const bool tap_ok = live && dy < p.kh;
       const int dyo = dy * p.dil_h, dxo = dx * p.dil_w;
       const int tap_offset = (dyo * p.w + dxo) * p.c + ck;  // the same for every row of this thread
@@ -541,12 +589,12 @@ void PlanSplits(Params* p, int bm, int bn, int elem_bytes) {
 // Raises the dynamic LDS limit of one kernel instantiation, once per instantiation and process (a failed attempt is
 // tried again by the next call).  The runtime does not allow the call while a stream is being captured, which is why
 // cinn_hip_conv2d_forward_noalloc_init walks every instantiation ahead of time.
-template <typename T, int BM, int BN, int WM, int WN, bool NCHW_IN, int PF = 2>
+template <typename T, int BM, int BN, int WM, int WN, bool NCHW_IN, int PF = 2, bool FAST = false>
 hipError_t Configure() {
   static std::atomic<bool> done{false};
   if (done.load(std::memory_order_acquire)) return hipSuccess;
   const hipError_t status = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(conv_nhwc_mfma_kernel<T, BM, BN, WM, WN, NCHW_IN, PF>),
+      reinterpret_cast<const void*>(conv_nhwc_mfma_kernel<T, BM, BN, WM, WN, NCHW_IN, PF, FAST>),
       hipFuncAttributeMaxDynamicSharedMemorySize, LdsBytes(BM, BN, WM));
   if (status == hipSuccess) done.store(true, std::memory_order_release);
   return status;
@@ -560,12 +608,12 @@ int LaunchFailed(const ScratchSource& src, hipError_t err, const char* what) {
   return 1;
 }
 
-template <typename T, int BM, int BN, int WM, int WN, bool NCHW_IN, int PF = 2>
+template <typename T, int BM, int BN, int WM, int WN, bool NCHW_IN, int PF = 2, bool FAST = false>
 int Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream, const ScratchSource& src) {
   // PF: K steps in flight per block
-  auto kernel      = conv_nhwc_mfma_kernel<T, BM, BN, WM, WN, NCHW_IN, PF>;
+  auto kernel      = conv_nhwc_mfma_kernel<T, BM, BN, WM, WN, NCHW_IN, PF, FAST>;
   const int bytes  = LdsBytes(BM, BN, WM);
-  if (hipError_t err = Configure<T, BM, BN, WM, WN, NCHW_IN, PF>(); err != hipSuccess)
+  if (hipError_t err = Configure<T, BM, BN, WM, WN, NCHW_IN, PF, FAST>(); err != hipSuccess)
     return LaunchFailed(src, err, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
   Params p = p_in;
   PlanSplits(&p, BM, BN, sizeof(T));
@@ -613,12 +661,33 @@ TileShape TileFor(const ConvNhwcArgs& a, const Params& p) {
   return {64, 64, 2, 2};
 }
 
+// The uniform-tap loader takes channels-last layers whose channel count is a multiple of one K step (128 bytes) and
+// whose operands stay below 2 GiB (32-bit byte offsets; an offset with the top bit set is its "out of range").
+// FLAGS_cinn_hip_conv_uniform_tap=0 keeps every layer on the per-lane loader.
+template <typename T>
+bool UniformTap(const ConvNhwcArgs& a, const Params& p) {
+  static const bool enabled = [] {
+    const char* e = getenv("FLAGS_cinn_hip_conv_uniform_tap");
+    return !(e && e[0] == '0');
+  }();
+  constexpr int64_t kLimit = ((int64_t)1 << 31) - 4096;  // the steps requested beyond the last stay below 2^32
+  const int bk = kRowBytes / (int)sizeof(T);
+  return enabled && !a.nchw_input && a.c % bk == 0 && (int64_t)a.n * a.h * a.w_in * a.c * (int64_t)sizeof(T) < kLimit &&
+         (int64_t)a.oc * p.k_total * (int64_t)sizeof(T) < kLimit;
+}
+
 template <typename T>
 int Dispatch(const ConvNhwcArgs& a, const Params& p, hipStream_t stream, const ScratchSource& src = ScratchSource()) {
   const TileShape t = TileFor(a, p);
   if (a.nchw_input) {
     if (t.bm == 128) return Launch<T, 128, 64, 2, 2, true>(a, p, stream, src);
     return Launch<T, 64, 64, 2, 2, true>(a, p, stream, src);
+  }
+  if (UniformTap<T>(a, p)) {
+    if (t.bm == 128 && t.bn == 128 && t.wn == 4) return Launch<T, 128, 128, 2, 4, false, 2, true>(a, p, stream, src);
+    if (t.bm == 128 && t.bn == 128) return Launch<T, 128, 128, 2, 2, false, 2, true>(a, p, stream, src);
+    if (t.bm == 128) return Launch<T, 128, 64, 2, 2, false, 2, true>(a, p, stream, src);
+    return Launch<T, 64, 64, 2, 2, false, 2, true>(a, p, stream, src);
   }
   if (t.bm == 128 && t.bn == 128 && t.wn == 4) return Launch<T, 128, 128, 2, 4, false>(a, p, stream, src);
   if (t.bm == 128 && t.bn == 128) return Launch<T, 128, 128, 2, 2, false>(a, p, stream, src);
@@ -629,9 +698,16 @@ int Dispatch(const ConvNhwcArgs& a, const Params& p, hipStream_t stream, const S
 // every instantiation Dispatch<T> can reach
 template <typename T>
 hipError_t ConfigureAll() {
-  const hipError_t all[6] = {Configure<T, 128, 64, 2, 2, true>(),   Configure<T, 64, 64, 2, 2, true>(),
-                             Configure<T, 128, 128, 2, 4, false>(), Configure<T, 128, 128, 2, 2, false>(),
-                             Configure<T, 128, 64, 2, 2, false>(),  Configure<T, 64, 64, 2, 2, false>()};
+  const hipError_t all[10] = {Configure<T, 128, 64, 2, 2, true>(),
+                              Configure<T, 64, 64, 2, 2, true>(),
+                              Configure<T, 128, 128, 2, 4, false>(),
+                              Configure<T, 128, 128, 2, 2, false>(),
+                              Configure<T, 128, 64, 2, 2, false>(),
+                              Configure<T, 64, 64, 2, 2, false>(),
+                              Configure<T, 128, 128, 2, 4, false, 2, true>(),
+                              Configure<T, 128, 128, 2, 2, false, 2, true>(),
+                              Configure<T, 128, 64, 2, 2, false, 2, true>(),
+                              Configure<T, 64, 64, 2, 2, false, 2, true>()};
   for (hipError_t e : all)
     if (e != hipSuccess) return e;
   return hipSuccess;
