@@ -21,6 +21,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <type_traits>
 #include <climits>
 #include <cstdint>
 #include <cstdio>
@@ -58,6 +59,10 @@ struct Params {
   int steps_per_split;  // K steps each blockIdx.y handles; with more than one split the kernel writes raw fp32 partial
                         // sums to the workspace and SplitReduceKernel applies the epilogue
   int splits;
+  // Tail split (splits == 1): the first full_tiles tiles (a multiple of the CU count) are one block each; every tile
+  // after them is tail_splits blocks of tail_steps K steps, which write fp32 partial sums [tile - full_tiles][part]
+  // [BM][BN] to the workspace for TailReduceKernel.  tail_splits == 1: no tile is split.
+  int full_tiles, tail_splits, tail_steps;
 };
 
 __device__ __forceinline__ int FastDiv(int n, unsigned magic, unsigned shift) {
@@ -173,10 +178,17 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   const int tiles_n = (p.oc + BN - 1) / BN;
   const int tiles   = ((p.pixels + BM - 1) / BM) * tiles_n;
   int bid           = blockIdx.x;
-  {
-    const int q = tiles >> 3, r = tiles & 7, xcd = bid & 7;
+  int tail_part     = -1;  // >= 0: this block computes part tail_part of a split tile
+  if (p.tail_splits > 1 && bid >= p.full_tiles) {
+    const int c = bid - p.full_tiles;
+    bid         = p.full_tiles + c / p.tail_splits;
+    tail_part   = c - (bid - p.full_tiles) * p.tail_splits;
+  } else {
+    const int whole = p.tail_splits > 1 ? p.full_tiles : tiles;
+    const int q = whole >> 3, r = whole & 7, xcd = bid & 7;
     bid = xcd * q + (xcd < r ? xcd : r) + (bid >> 3);
   }
+  const int tile_id = bid;
   const int m0 = (bid / tiles_n) * BM;
   const int n0 = (bid % tiles_n) * BN;
 
@@ -191,7 +203,8 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   constexpr int EPI_RPT  = BM / EPI_ROWS;  // output rows per thread
   struct alignas(16) Res8 { T v[8]; };
   Res8 res_pre[EPI_RPT];
-  const bool prefetch_res = residual != nullptr && p.splits == 1 && (p.oc & 7) == 0 && n0 + (tid % EPI_CPR) * 8 < p.oc;
+  const bool prefetch_res =
+      residual != nullptr && p.splits == 1 && tail_part < 0 && (p.oc & 7) == 0 && n0 + (tid % EPI_CPR) * 8 < p.oc;
   if (prefetch_res) {
 #pragma unroll
     for (int i = 0; i < EPI_RPT; ++i) {
@@ -224,8 +237,9 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   }
   // position of this thread's chunk in the reduction: channel offset and filter tap (channels-last loader)
   const int total_steps = (p.k_total + BK - 1) / BK;
-  const int step0       = blockIdx.y * p.steps_per_split;
-  const int step1       = step0 + p.steps_per_split < total_steps ? step0 + p.steps_per_split : total_steps;
+  const int my_steps    = tail_part >= 0 ? p.tail_steps : p.steps_per_split;
+  const int step0       = (tail_part >= 0 ? tail_part : (int)blockIdx.y) * my_steps;
+  const int step1       = step0 + my_steps < total_steps ? step0 + my_steps : total_steps;
   int ck = 0, dy = 0, dx = 0;
   static_assert(!(FAST && NCHW_IN), "the uniform-tap loader reads channels-last images");
   if (FAST) {
@@ -416,7 +430,7 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   const bool active       = oc0 < p.oc;
   const bool full         = (p.oc & 7) == 0;  // then every group is whole and 16-byte aligned
   float sc[8], sh[8];
-  if (active && p.splits == 1) {
+  if (active && p.splits == 1 && tail_part < 0) {
     if (full && scale && shift) {
       __builtin_memcpy(sc, scale + oc0, 32);
       __builtin_memcpy(sh, shift + oc0, 32);
@@ -430,6 +444,8 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
     }
   }
   float* ws = workspace + (int64_t)blockIdx.y * p.pixels * p.oc;  // split-K: fp32 partial sums [split][pixel][oc]
+  // tail split: this block's [BM][BN] slice
+  float* tail_ws = workspace + ((int64_t)(tile_id - p.full_tiles) * p.tail_splits + tail_part) * (BM * BN);
 #pragma unroll
   for (int pass = 0; pass < PASSES; ++pass) {
     if (pass > 0) __syncthreads();  // the previous pass has been read
@@ -457,6 +473,12 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
       float v[8];
       *reinterpret_cast<f32x4*>(&v[0]) = *reinterpret_cast<const f32x4*>(&st[row * SLD + cg * 8]);
       *reinterpret_cast<f32x4*>(&v[4]) = *reinterpret_cast<const f32x4*>(&st[row * SLD + cg * 8 + 4]);
+      if (tail_part >= 0) {
+        float* dst = tail_ws + (pass * PROWS + row) * BN + cg * 8;
+        *reinterpret_cast<f32x4*>(dst)     = *reinterpret_cast<const f32x4*>(&v[0]);
+        *reinterpret_cast<f32x4*>(dst + 4) = *reinterpret_cast<const f32x4*>(&v[4]);
+        continue;
+      }
       const int64_t off = (int64_t)m * p.oc + oc0;
       if (p.splits > 1) {
         if (full) {
@@ -519,6 +541,36 @@ SplitReduceKernel(const float* __restrict__ workspace, T* y, const float* __rest
     out[e] = (T)(p.relu ? fmaxf(t, 0.0f) : t);
   }
   __builtin_memcpy(y + off, out, V * sizeof(T));
+}
+
+// Sums the parts of the split tiles behind the first full_tiles tiles and applies the epilogue: one thread per 4
+// channels of one pixel of one split tile.
+template <typename T, int BM, int BN>
+__global__ void __launch_bounds__(256)
+TailReduceKernel(const float* __restrict__ workspace, T* y, const float* __restrict__ scale, const float* __restrict__ shift,
+                 const T* residual, Params p) {
+  constexpr int PER_TILE = BM * BN / 4;
+  const int idx     = blockIdx.x * 256 + threadIdx.x;
+  const int tile    = idx / PER_TILE;  // among the split tiles
+  const int e       = idx - tile * PER_TILE;
+  const int row     = e / (BN / 4);
+  const int col     = (e - row * (BN / 4)) * 4;
+  const int tiles_n = (p.oc + BN - 1) / BN;
+  const int t       = p.full_tiles + tile;
+  const int m       = (t / tiles_n) * BM + row;
+  const int oc0     = (t % tiles_n) * BN + col;
+  if (m >= p.pixels || oc0 >= p.oc) return;
+  f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+  const float* src = workspace + (int64_t)tile * p.tail_splits * (BM * BN) + row * BN + col;
+  for (int part = 0; part < p.tail_splits; ++part) v += *reinterpret_cast<const f32x4*>(src + (int64_t)part * (BM * BN));
+  const int64_t off = (int64_t)m * p.oc + oc0;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    if (oc0 + k >= p.oc) break;
+    float r = __builtin_fmaf(v[k], scale ? scale[oc0 + k] : p.alpha, shift ? shift[oc0 + k] : 0.0f);
+    if (residual) r = __builtin_fmaf(p.residual_scale, (float)residual[off + k], r);
+    y[off + k] = (T)(p.relu ? fmaxf(r, 0.0f) : r);
+  }
 }
 
 // ---- host side ------------------------------------------------------------------------------------------------
@@ -584,6 +636,47 @@ void PlanSplits(Params* p, int bm, int bn, int elem_bytes) {
   p->splits          = ChooseSplits(tiles, steps);
   p->steps_per_split = (steps + p->splits - 1) / p->splits;
   p->splits          = (steps + p->steps_per_split - 1) / p->steps_per_split;
+  p->full_tiles      = tiles;
+  p->tail_splits     = 1;
+  p->tail_steps      = steps;
+}
+
+// Tail split of an fp32 launch.  Its blocks are bound by the matrix pipe, a CU holds four of them and runs them at a
+// quarter of the speed each, so a launch takes as long as the CU with the most tiles: 784 tiles on 256 CUs take the
+// time of 4 per CU although the average is 3.06.  The tiles beyond the last multiple of the CU count are therefore
+// cut along K into parts small enough to spread evenly, and their partial sums go through the workspace (a fraction
+// of what a split of the whole grid moves).  Returns the bytes of workspace needed, 0 when no tile is split.
+// FLAGS_cinn_hip_conv_tail_split=0 switches it off.
+size_t PlanTailSplit(Params* p, int bm, int bn, int elem_bytes) {
+  static const bool enabled = [] {
+    const char* e = getenv("FLAGS_cinn_hip_conv_tail_split");
+    return !(e && e[0] == '0');
+  }();
+  constexpr int kCus = 256;
+  const int bk    = 128 / elem_bytes;
+  const int tiles = ((p->pixels + bm - 1) / bm) * ((p->oc + bn - 1) / bn);
+  const int steps = (p->k_total + bk - 1) / bk;
+  if (!enabled || p->splits != 1 || tiles < kCus) return 0;
+  const int full = tiles / kCus * kCus, rest = tiles - full;
+  if (rest == 0) return 0;
+  // time of the remainder in units of one tile on a CU of its own: ceil(rest * parts / CUs) / parts
+  double best = 1.0;
+  int best_parts = 1;
+  for (int parts = 2; parts <= 16; parts *= 2) {
+    const int part_steps = (steps + parts - 1) / parts;
+    if (part_steps < 2) break;
+    const int real_parts = (steps + part_steps - 1) / part_steps;
+    if ((size_t)rest * real_parts * bm * bn * sizeof(float) > ((size_t)24 << 20)) break;
+    const double t = (double)((rest * real_parts + kCus - 1) / kCus) / real_parts;
+    if (t < best - 1e-9) best = t, best_parts = real_parts;
+  }
+  // Worth a second launch (4-6 us) only when it saves more than that: a tile on a CU of its own takes about half a
+  // microsecond per K step (16 MFMAs of 64 clocks), so the remainder gets (1 - best) * steps / 2 us shorter.
+  if (best_parts == 1 || (1.0 - best) * steps < 20.0) return 0;
+  p->full_tiles  = full;
+  p->tail_steps  = (steps + best_parts - 1) / best_parts;
+  p->tail_splits = (steps + p->tail_steps - 1) / p->tail_steps;
+  return (size_t)rest * p->tail_splits * bm * bn * sizeof(float);
 }
 
 // Raises the dynamic LDS limit of one kernel instantiation, once per instantiation and process (a failed attempt is
@@ -619,6 +712,17 @@ int Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream, const 
   PlanSplits(&p, BM, BN, sizeof(T));
   const int tiles  = ((p.pixels + BM - 1) / BM) * ((p.oc + BN - 1) / BN);
   float* workspace = nullptr;
+  int blocks       = tiles;
+  if constexpr (std::is_same<T, float>::value && BM == 64 && BN == 64 && !NCHW_IN) {
+    if (const size_t need = PlanTailSplit(&p, BM, BN, sizeof(T)); need > 0) {
+      if (src.fixed_partials && need > src.fixed_partials_bytes) {
+        p.full_tiles = tiles, p.tail_splits = 1;  // the fixed scratch is too small: every tile stays whole
+      } else {
+        workspace = src.fixed_partials ? src.fixed_partials : static_cast<float*>(Scratch(ScratchKind::kSplitK, need, stream));
+        blocks    = p.full_tiles + (tiles - p.full_tiles) * p.tail_splits;
+      }
+    }
+  }
   // fp32 partial sums [split][pixel][oc]
   if (p.splits > 1) {
     const size_t need = (size_t)p.splits * p.pixels * p.oc * sizeof(float);
@@ -629,10 +733,16 @@ int Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream, const 
       workspace = static_cast<float*>(Scratch(ScratchKind::kSplitK, need, stream));
     }
   }
-  hipLaunchKernelGGL(kernel, dim3(tiles, p.splits), dim3(64 * WM * WN), bytes, stream, static_cast<const T*>(a.x),
+  hipLaunchKernelGGL(kernel, dim3(blocks, p.splits), dim3(64 * WM * WN), bytes, stream, static_cast<const T*>(a.x),
                      static_cast<const T*>(a.w), static_cast<T*>(a.y), a.scale, a.shift, static_cast<const T*>(a.residual),
                      workspace, src.zero_page ? src.zero_page : ZeroPage(), p);
   if (hipError_t err = hipGetLastError(); err != hipSuccess) return LaunchFailed(src, err, "kernel launch");
+  if (p.tail_splits > 1) {
+    const int threads = (tiles - p.full_tiles) * (BM * BN / 4);
+    hipLaunchKernelGGL((TailReduceKernel<T, BM, BN>), dim3((unsigned)(threads / 256)), dim3(256), 0, stream, workspace,
+                       static_cast<T*>(a.y), a.scale, a.shift, static_cast<const T*>(a.residual), p);
+    if (hipError_t err = hipGetLastError(); err != hipSuccess) return LaunchFailed(src, err, "launch of the tail reduction");
+  }
   if (p.splits > 1) {
     if (p.oc % 4 == 0) {
       const int64_t total = (int64_t)p.pixels * p.oc / 4;

@@ -510,6 +510,22 @@ def test_implicit_gemm_convolution_with_dilation(gpu, dtype, tol):
     assert np.all(np.abs(got - want) <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
 
 
+def test_fp32_convolution_whose_last_tiles_are_split_along_k(gpu):
+    """784 tiles of 64x64 on 256 CUs: the 16 tiles beyond 768 are cut into parts along K and summed by a second
+    kernel, which also applies alpha / beta; the last pixel tile and the last channel tile are ragged."""
+    n, ic, h, w_, oc = 5, 128, 28, 179, 72
+    rng = np.random.default_rng(784)
+    x = rng.standard_normal((n, ic, h, w_)).astype(np.float32)
+    w = (rng.standard_normal((oc, ic, 3, 3)) * np.sqrt(2.0 / (ic * 9))).astype(np.float32)
+    y0 = rng.standard_normal((n, oc, h, w_)).astype(np.float32)
+    got = call_conv_nhwc(x, w, 1, 1, 1, "float32", alpha=0.5, beta=2.0, y_init=y0).astype(np.float64)
+    want = 0.5 * oracle.conv2d_nchw(x, w, (1, 1), (1, 1)).astype(np.float64) + 2.0 * y0
+    scale = 0.5 * oracle.conv2d_nchw(np.abs(x), np.abs(w), (1, 1), (1, 1)) + 2.0 * np.abs(y0)
+    assert np.all(np.abs(got - want) <= 1e-5 * scale)
+    plain = call_conv_nhwc(x, w, 1, 1, 1, "float32").astype(np.float64)
+    assert np.all(np.abs(plain - (want - 2.0 * y0) * 2.0) <= 1e-5 * (scale - 2.0 * np.abs(y0)) * 2.0 + 1e-30)
+
+
 def test_implicit_gemm_convolution_with_residual_epilogue(gpu):
     """alpha / beta through the fp32-staged epilogue of the GEMM kernel, on a padded 3x3 convolution."""
     n, ic, h, w_, oc = 8, 64, 32, 32, 512
