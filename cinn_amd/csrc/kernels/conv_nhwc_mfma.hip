@@ -606,12 +606,29 @@ TileChoice ChooseTile(int pixels, int oc) {
 
 // K splits: layers whose tile grid cannot fill the 256 CUs spend their time waiting for one block's serial chain of
 // loads; splitting the reduction puts several blocks of the same tile on different CUs
-int ChooseSplits(int tiles, int steps) {
+int ChooseSplits(int tiles, int steps, bool fp32, size_t bytes_per_split, size_t cap) {
   static const int forced = [] {
     const char* e = getenv("FLAGS_cinn_hip_conv_splits");
     return e ? atoi(e) : 0;
   }();
   if (forced > 0) return forced < steps ? forced : steps;
+  static const bool balance = [] {  // FLAGS_cinn_hip_conv_split_balance=0: the powers of two below for fp32 as well
+    const char* e = getenv("FLAGS_cinn_hip_conv_split_balance");
+    return !(e && e[0] == '0');
+  }();
+  if (fp32 && balance && tiles < 256) {
+    // fp32 blocks are bound by the matrix pipe, which the blocks of a CU share: the launch takes as long as the CU
+    // with the most parts, ceil(tiles * s / 256) / s of a whole tile - 200 tiles: four ways 1.0, five ways 0.8.  Every
+    // part keeps at least 8 K steps; 0.02 per part stands for the partial sums it writes and the reduction reads.
+    int best = 1;
+    double best_cost = 1.0;
+    for (int s = 2; s <= 8 && steps / s >= 8; ++s) {
+      if (cap != 0 && (size_t)s * bytes_per_split > cap) break;
+      const double cost = (double)((tiles * s + 255) / 256) / s + 0.02 * s;
+      if (cost < best_cost - 1e-9) best_cost = cost, best = s;
+    }
+    return best;
+  }
   // only grids that leave CUs without a single block are split, and every part keeps at least 8 K steps
   int splits = 1;
   if (tiles >= 256) return 1;
@@ -629,11 +646,12 @@ struct ScratchSource {
 };
 
 // split count and K steps per split of one launch
-void PlanSplits(Params* p, int bm, int bn, int elem_bytes) {
+// cap: bytes the partial sums may take (0: no limit; the entry point that allocates nothing has a fixed region)
+void PlanSplits(Params* p, int bm, int bn, int elem_bytes, size_t cap = 0) {
   const int bk    = 128 / elem_bytes;
   const int tiles = ((p->pixels + bm - 1) / bm) * ((p->oc + bn - 1) / bn);
   const int steps = (p->k_total + bk - 1) / bk;
-  p->splits          = ChooseSplits(tiles, steps);
+  p->splits          = ChooseSplits(tiles, steps, elem_bytes == 4, (size_t)p->pixels * p->oc * sizeof(float), cap);
   p->steps_per_split = (steps + p->splits - 1) / p->splits;
   p->splits          = (steps + p->steps_per_split - 1) / p->steps_per_split;
   p->full_tiles      = tiles;
@@ -709,7 +727,7 @@ int Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream, const 
   if (hipError_t err = Configure<T, BM, BN, WM, WN, NCHW_IN, PF, FAST>(); err != hipSuccess)
     return LaunchFailed(src, err, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
   Params p = p_in;
-  PlanSplits(&p, BM, BN, sizeof(T));
+  PlanSplits(&p, BM, BN, sizeof(T), src.fixed_partials ? src.fixed_partials_bytes : 0);
   const int tiles  = ((p.pixels + BM - 1) / BM) * ((p.oc + BN - 1) / BN);
   float* workspace = nullptr;
   int blocks       = tiles;
@@ -1014,7 +1032,7 @@ int cinn_call_hip_conv2d_forward_noalloc(void* v_args, int num_args, int format,
   // the size check comes before any launch: the partial sums of the split this shape gets must fit
   Params p          = MakeParams(a);
   const TileShape t = TileFor(a, p);
-  PlanSplits(&p, t.bm, t.bn, a.type.bits / CHAR_BIT);
+  PlanSplits(&p, t.bm, t.bn, a.type.bits / CHAR_BIT, kNoAllocPartialsBytes);
   const size_t need = p.splits > 1 ? (size_t)p.splits * p.pixels * p.oc * sizeof(float) : 0;
   if (need > kNoAllocPartialsBytes)
     CINN_NOALLOC_REJECT(2, "this shape splits its reduction %d ways and needs %zu bytes of partial sums; the static scratch holds %zu",

@@ -118,12 +118,12 @@ def test_noalloc_rejects_what_it_cannot_run_without_launching(gpu):
     lib = _lib.load()
     lib.cinn_call_hip_conv2d_forward_noalloc.argtypes = CONV_ARGTYPES
     lib.cinn_call_hip_conv2d_forward_noalloc.restype = ctypes.c_int
-    # 150 tiles of 64x64 with 144 K steps split eight ways: 19.7 MB of partial sums > 16 MiB
-    n, c, hw, oc = 48, 512, 14, 64   # 9408 pixels
-    X = runtime.DeviceBuffer((n, hw, hw, c), "float32")
-    W = runtime.DeviceBuffer((oc, 3, 3, c), "float32")
-    Y = runtime.DeviceBuffer((n, hw, hw, oc), "float32")
-    sentinel = np.full((n, hw, hw, oc), 3.0, np.float32)
+    # fp16: 147 tiles of 64x64 with 144 K steps split eight ways: 19.3 MB of partial sums > 16 MiB
+    n, c, hw, oc = 48, 1024, 14, 64   # 9408 pixels
+    X = runtime.DeviceBuffer((n, hw, hw, c), "float16")
+    W = runtime.DeviceBuffer((oc, 3, 3, c), "float16")
+    Y = runtime.DeviceBuffer((n, hw, hw, oc), "float16")
+    sentinel = np.full((n, hw, hw, oc), 3.0, np.float16)
     Y.copy_from(sentinel)
     args = runtime.pod_args([X, W, Y])
     rc = lib.cinn_call_hip_conv2d_forward_noalloc(args, 3, 1, 1.0, 0.0, n, c, hw, hw, oc, c, 3, 3, 1, 1, 1, 1, 1, 1, 1, n, oc, hw, hw, None)
@@ -135,6 +135,19 @@ def test_noalloc_rejects_what_it_cannot_run_without_launching(gpu):
     assert lib.cinn_call_hip_conv2d_forward_noalloc(args, 2, 1, 1.0, 0.0, n, c, hw, hw, oc, c, 3, 3, 1, 1, 1, 1, 1, 1, 1, n, oc, hw, hw, None) == 1
     runtime.synchronize()
     assert np.array_equal(Y.numpy(), sentinel)
+
+
+def test_noalloc_fp32_split_is_chosen_to_fit_the_static_scratch(gpu):
+    """fp32 layers pick their split count by balance over the CUs among the counts whose partial sums fit: 147 tiles
+    with 144 K steps take five parts (12 MB) under both entry points, where eight (19.3 MB) would be refused."""
+    rng = np.random.default_rng(147)
+    x, w = case(rng, np.float32, 48, 512, 14, 64, 3)
+    got, ref, rc = both_entry_points(x, w, 1, 1)
+    assert rc == 0 and np.array_equal(got, ref)
+    sample = [0, 23, 47]
+    want = oracle.conv2d_nchw(x[sample], w, (1, 1), (1, 1)).astype(np.float64)
+    scale = oracle.conv2d_nchw(np.abs(x[sample]), np.abs(w), (1, 1), (1, 1))
+    assert np.all(np.abs(got[sample] - want) <= 1e-5 * scale)
 
 
 def test_noalloc_allocates_nothing_and_runs_under_stream_capture(gpu):
