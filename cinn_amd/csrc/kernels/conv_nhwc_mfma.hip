@@ -149,7 +149,8 @@ struct WaveMma {
 // lanes as the other vector instructions (64 more of those per K step cost the fp32 kernel 17-22 %), so every vector
 // instruction the loader does not execute is matrix time: 63 -> 14 per K step.
 template <typename T, int BM, int BN, int WM, int WN, bool NCHW_IN, int PF, bool FAST>
-__global__ void __launch_bounds__(64 * WM * WN)
+__global__ void
+__launch_bounds__(64 * WM * WN, (sizeof(T) == 4 && BM == 64 && BN == 64 && !NCHW_IN) ? 4 : 1)  // fp32 64x64: four blocks per CU
 conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, const float* __restrict__ scale,
                       const float* __restrict__ shift, const T* residual, float* __restrict__ workspace,
                       const void* __restrict__ zero_page, Params p) {
@@ -202,8 +203,11 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
   constexpr int EPI_ROWS = THREADS / EPI_CPR;
   constexpr int EPI_RPT  = BM / EPI_ROWS;  // output rows per thread
   struct alignas(16) Res8 { T v[8]; };
-  Res8 res_pre[EPI_RPT];
-  const bool prefetch_res =
+  // (not in the fp32 64x64 instance: its blocks are bound by the matrix pipe with four wavefronts per SIMD to cover a
+  // late read, and its register budget goes to the grouped sums below)
+  constexpr bool EARLY_RES = !(sizeof(T) == 4 && BM == 64 && BN == 64 && !NCHW_IN);
+  Res8 res_pre[EARLY_RES ? EPI_RPT : 1];
+  const bool prefetch_res = EARLY_RES &&
       residual != nullptr && p.splits == 1 && tail_part < 0 && (p.oc & 7) == 0 && n0 + (tid % EPI_CPR) * 8 < p.oc;
   if (prefetch_res) {
 #pragma unroll
@@ -383,6 +387,38 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+  // A launch with a tail split: a whole tile adds its products up in the same groups of tail_steps K steps as the
+  // parts of a split tile, group sums added in ascending order like TailReduceKernel adds the parts, so that a pixel's
+  // result does not depend on which kind of tile it fell into (equal images at two batch positions give equal bits).
+  constexpr bool GROUPED = std::is_same<T, float>::value && BM == 64 && BN == 64 && !NCHW_IN;
+  f32x16 total[GROUPED ? TM : 1][GROUPED ? TN : 1];
+  int until_group_end = INT_MAX;
+  if constexpr (GROUPED) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) total[i][j][r] = 0.0f;
+    if (p.tail_splits > 1 && tail_part < 0) until_group_end = p.tail_steps;
+  }
+  auto end_of_step = [&]() {
+    if constexpr (GROUPED) {
+      if (--until_group_end == 0) {
+        // a real branch, taken once per group: as selects the compiler reads every accumulator after every K step
+        asm volatile("; end of a group of K steps");
+        until_group_end = p.tail_steps;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            total[i][j] += acc[i][j];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+          }
+      }
+    }
+  };
 
   static_assert(PF % 2 == 0, "the LDS stage of a step must be a compile-time function of its slot");
   const int steps = step1 - step0;
@@ -403,6 +439,7 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
       WaveMma<T, TM, TN>::Step(cur, cur + A_TILE, a_row, b_row, lane, acc);
       store_step(lds + ((i + 1) & 1) * STAGE, ra_slots[(i + 1) % PF], rb_slots[(i + 1) % PF]);
       load_step(step0 + s + i + 1 + PF, ra_slots[(i + 1) % PF], rb_slots[(i + 1) % PF]);
+      end_of_step();
       __syncthreads();
     }
   }
@@ -413,7 +450,16 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
       char* cur = lds + (i & 1) * STAGE;
       WaveMma<T, TM, TN>::Step(cur, cur + A_TILE, a_row, b_row, lane, acc);
       store_step(lds + ((i + 1) & 1) * STAGE, ra_slots[(i + 1) % PF], rb_slots[(i + 1) % PF]);
+      end_of_step();
       __syncthreads();
+    }
+  }
+  if constexpr (GROUPED) {
+    if (p.tail_splits > 1 && tail_part < 0) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = total[i][j] + acc[i][j];  // the last group, like the last part
     }
   }
 
@@ -494,7 +540,8 @@ conv_nhwc_mfma_kernel(const T* __restrict__ x, const T* __restrict__ w, T* y, co
       if (full) {
         T out[8];
         if (residual) {
-          const Res8& rv = res_pre[pass * (PROWS / ROWS) + it];  // requested at the start of the kernel
+          // requested at the start of the kernel, or read here
+          const Res8 rv = EARLY_RES ? res_pre[EARLY_RES ? pass * (PROWS / ROWS) + it : 0] : *reinterpret_cast<const Res8*>(residual + off);
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[e] = __builtin_fmaf(p.residual_scale, (float)rv.v[e], v[e]);
         }
