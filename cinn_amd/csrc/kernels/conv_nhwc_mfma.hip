@@ -800,7 +800,7 @@ int Launch(const ConvNhwcArgs& a, const Params& p_in, hipStream_t stream, const 
   }
   hipLaunchKernelGGL(kernel, dim3(blocks, p.splits), dim3(64 * WM * WN), bytes, stream, static_cast<const T*>(a.x),
                      static_cast<const T*>(a.w), static_cast<T*>(a.y), a.scale, a.shift, static_cast<const T*>(a.residual),
-                     workspace, src.zero_page ? src.zero_page : ZeroPage(), p);
+                     workspace, FAST ? nullptr : (src.zero_page ? src.zero_page : ZeroPage()), p);  // FAST reads no page of zeros
   if (hipError_t err = hipGetLastError(); err != hipSuccess) return LaunchFailed(src, err, "kernel launch");
   if (p.tail_splits > 1) {
     const int threads = (tiles - p.full_tiles) * (BM * BN / 4);

@@ -90,6 +90,7 @@ extern "C" {
 
 int cinn_hip_scratch_reserve(void* stream, size_t split_k_bytes, size_t transpose_bytes) {
   using namespace cinn_hip_kernels;
+  ZeroPage();  // allocated and cleared on first use, which must not fall into a capture either
   Arena& arena = TheArena();
   std::lock_guard<std::mutex> lock(arena.mu);
   if (split_k_bytes) Ensure(arena, ScratchKind::kSplitK, split_k_bytes, static_cast<hipStream_t>(stream));

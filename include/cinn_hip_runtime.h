@@ -349,6 +349,7 @@ const char* cinn_hip_error_string(int status);
  * and purpose, grown on demand by the cinn_call_* that needs it; an outgrown buffer is retired, not freed, because a
  * captured graph may still hold its address, and no call waits for the device.  While a stream is being captured
  * nothing can be allocated: reserve first (one eager run of the same calls does it, or this call; 0 = leave as is).
+ * The call also creates the device's 256-byte page of zeros that convolution kernels read masked-out chunks from.
  * cinn_hip_scratch_release_retired frees the retired buffers; only a caller that knows that no instantiated graph
  * refers to them may call it. */
 int cinn_hip_scratch_reserve(void* stream, size_t split_k_bytes, size_t transpose_bytes);

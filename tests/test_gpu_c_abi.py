@@ -245,6 +245,59 @@ def test_nchw_convolution_of_a_new_shape_is_captured_without_an_eager_run(gpu):
     hip.hipGraphDestroy(graph)
 
 
+def test_fp32_convolution_with_a_tail_split_is_captured_after_reserving_its_scratch(gpu):
+    """A channels-last fp32 convolution of 400 tiles: 256 whole tiles, 144 cut along K, and the kernel that sums the
+    parts - two launches and 18.9 MB of partial sums, recorded into a graph without an eager run of the shape (kernel
+    attributes set by cinn_hip_conv2d_forward_noalloc_init, scratch by cinn_hip_scratch_reserve), replayed with eager
+    work in between; the replays, an eager call and the oracle agree."""
+    import oracle
+    lib = _lib.load()
+    hip = ctypes.CDLL("libamdhip64.so")
+    conv_argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_float] + [ctypes.c_int] * 19 + [ctypes.c_void_p]
+    lib.cinn_call_cudnn_conv2d_forward.argtypes = conv_argtypes
+    lib.cinn_call_cudnn_conv2d_forward.restype = None
+    assert lib.cinn_hip_conv2d_forward_noalloc_init() == 0
+    rng = np.random.default_rng(400)
+    stream = runtime.Stream()
+    assert lib.cinn_hip_scratch_reserve(stream.handle, ctypes.c_size_t(24 << 20), ctypes.c_size_t(0)) == 0
+    n, c, h, w, f = 4, 256, 56, 57, 128
+    x = rng.standard_normal((n, c, h, w)).astype(np.float32)
+    wt = (rng.standard_normal((f, c, 3, 3)) * np.sqrt(2.0 / (c * 9))).astype(np.float32)
+    X = runtime.DeviceBuffer.from_numpy(np.ascontiguousarray(x.transpose(0, 2, 3, 1)), "float32")
+    W = runtime.DeviceBuffer.from_numpy(np.ascontiguousarray(wt.transpose(0, 2, 3, 1)), "float32")
+    Y = runtime.DeviceBuffer((n, h, w, f), "float32")
+    zeros = np.zeros((n, h, w, f), np.float32)
+    Y.copy_from(zeros)
+    args = runtime.pod_args([X, W, Y])
+
+    def call():
+        lib.cinn_call_cudnn_conv2d_forward(args, 3, 1, 1.0, 0.0, n, c, h, w, f, c, 3, 3, 1, 1, 1, 1, 1, 1, 1, n, f, h, w, stream.handle)
+
+    graph, graph_exec = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipStreamBeginCapture(stream.handle, 1) == 0  # hipStreamCaptureModeThreadLocal
+    call()
+    assert hip.hipStreamEndCapture(stream.handle, ctypes.byref(graph)) == 0
+    assert hip.hipGraphInstantiate(ctypes.byref(graph_exec), graph, None, None, ctypes.c_size_t(0)) == 0
+    got = None
+    for replay in range(3):
+        Y.copy_from(zeros)  # eager work between the replays
+        assert hip.hipGraphLaunch(graph_exec, stream.handle) == 0
+        stream.synchronize()
+        out = Y.numpy()
+        assert got is None or np.array_equal(out, got), "replay %d" % replay
+        got = out
+    Y.copy_from(zeros)
+    call()
+    stream.synchronize()
+    assert np.array_equal(Y.numpy(), got)
+    sample = [0, 3]  # the last image lies in the tiles that are cut
+    want = oracle.conv2d_nchw(x[sample], wt, (1, 1), (1, 1))
+    scale = oracle.conv2d_nchw(np.abs(x[sample]), np.abs(wt), (1, 1), (1, 1))
+    assert np.all(np.abs(got[sample].transpose(0, 3, 1, 2) - want) <= 1e-5 * scale)
+    hip.hipGraphExecDestroy(graph_exec)
+    hip.hipGraphDestroy(graph)
+
+
 RESIZE_KERNELS = r'''
 #include "cinn_hip_runtime_source.h"
 // out[n][c][y][x] = resize(in)[n][c][y][x], one thread per output element, through the reference-named entry points
