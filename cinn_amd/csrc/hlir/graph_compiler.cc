@@ -387,7 +387,7 @@ void Program::ExecuteGraph(void* stream) {
   auto s = static_cast<hipStream_t>(stream);
   if (!prerun_done_) RunPreRunInstructions(stream);
   if (!graph_exec_) {
-    // Library-call kernels build per-shape tables and set function attributes on their first launch, which a
+    // Library-call kernels allocate what they need on first use (the page of zeros, per-stream scratch), which a
     // capturing stream does not allow: run the program once before recording it, on the streams it will be recorded
     // on.
     RunLanes(stream);

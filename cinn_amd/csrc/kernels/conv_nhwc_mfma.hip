@@ -745,8 +745,9 @@ size_t PlanTailSplit(Params* p, int bm, int bn, int elem_bytes) {
 }
 
 // Raises the dynamic LDS limit of one kernel instantiation, once per instantiation and process (a failed attempt is
-// tried again by the next call).  The runtime does not allow the call while a stream is being captured, which is why
-// cinn_hip_conv2d_forward_noalloc_init walks every instantiation ahead of time.
+// tried again by the next call).  cinn_hip_conv2d_forward_noalloc_init walks every instantiation ahead of time, so
+// that a first call under capture does nothing but launch (this runtime accepts the attribute call during a capture;
+// what it refuses there is allocating or clearing memory).
 template <typename T, int BM, int BN, int WM, int WN, bool NCHW_IN, int PF = 2, bool FAST = false>
 hipError_t Configure() {
   static std::atomic<bool> done{false};
@@ -1013,7 +1014,7 @@ int cinn_hip_conv2d_forward_noalloc_init(void) {
   using namespace cinn_hip_kernels;
   unsigned char* base = nullptr;
   if (NoAllocScratch(&base) != 0) return 1;
-  // the LDS limit of every kernel the entry point can launch: a capturing stream does not allow this set-up call
+  // the LDS limit of every kernel the entry point can launch, so that a call under capture only launches
   for (hipError_t e : {ConfigureAll<float>(), ConfigureAll<_Float16>(), ConfigureAll<__bf16>()}) {
     if (e != hipSuccess) {
       fprintf(stderr, "cinn_hip_conv2d_forward_noalloc_init: hipFuncSetAttribute failed: %s\n", hipGetErrorString(e));

@@ -4,7 +4,7 @@ first call's partial sums), with and without a split reduction, plus the error r
 kernel under both entry points and must agree bit for bit; the fp16 case may be routed to another MFMA kernel by the
 allocating entry point (different summation order) and is held to the 1e-2 bar; every result is also compared with
 the CPU oracle.  A last test makes the call while its stream is being captured (after
-cinn_hip_conv2d_forward_noalloc_init, which does the per-kernel set-up a capture does not allow), replays the graph and
+cinn_hip_conv2d_forward_noalloc_init, which does the per-kernel set-up ahead of the capture), replays the graph and
 checks that neither the library's arena nor the device's free memory moved across the calls."""
 import ctypes
 
