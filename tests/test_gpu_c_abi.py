@@ -245,28 +245,30 @@ def test_nchw_convolution_of_a_new_shape_is_captured_without_an_eager_run(gpu):
     hip.hipGraphDestroy(graph)
 
 
-def test_fp32_convolution_with_a_tail_split_is_captured_after_reserving_its_scratch(gpu):
-    """A channels-last fp32 convolution of 400 tiles: 256 whole tiles, 144 cut along K, and the kernel that sums the
-    parts - two launches and 18.9 MB of partial sums, recorded into a graph without an eager run of the shape (kernel
-    attributes set by cinn_hip_conv2d_forward_noalloc_init, scratch by cinn_hip_scratch_reserve), replayed with eager
-    work in between; the replays, an eager call and the oracle agree."""
+@pytest.mark.parametrize("dtype,shape,tol", [("float32", (4, 256, 56, 57, 128), 1e-5), ("float16", (8, 64, 33, 32, 512), 1e-2),
+                                             ("float16", (3, 128, 28, 28, 128), 1e-2)])
+def test_channels_last_convolution_is_captured_after_reserving_its_scratch(gpu, dtype, shape, tol):
+    """Channels-last 3x3 convolutions recorded into a graph without an eager run of the shape, after
+    cinn_hip_scratch_reserve only (it sizes the scratch and creates the page of zeros), replayed with eager work in
+    between; the replays, an eager call and the oracle agree.  fp32: 400 tiles, 256 whole and 144 cut along K, plus the
+    kernel that sums the parts (two launches, 18.9 MB of partial sums); fp16: the direct-to-LDS implicit GEMM and the
+    kernel that keeps the input patch in LDS by channel chunks."""
     import oracle
     lib = _lib.load()
     hip = ctypes.CDLL("libamdhip64.so")
     conv_argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_float] + [ctypes.c_int] * 19 + [ctypes.c_void_p]
     lib.cinn_call_cudnn_conv2d_forward.argtypes = conv_argtypes
     lib.cinn_call_cudnn_conv2d_forward.restype = None
-    assert lib.cinn_hip_conv2d_forward_noalloc_init() == 0
     rng = np.random.default_rng(400)
     stream = runtime.Stream()
     assert lib.cinn_hip_scratch_reserve(stream.handle, ctypes.c_size_t(24 << 20), ctypes.c_size_t(0)) == 0
-    n, c, h, w, f = 4, 256, 56, 57, 128
-    x = rng.standard_normal((n, c, h, w)).astype(np.float32)
-    wt = (rng.standard_normal((f, c, 3, 3)) * np.sqrt(2.0 / (c * 9))).astype(np.float32)
-    X = runtime.DeviceBuffer.from_numpy(np.ascontiguousarray(x.transpose(0, 2, 3, 1)), "float32")
-    W = runtime.DeviceBuffer.from_numpy(np.ascontiguousarray(wt.transpose(0, 2, 3, 1)), "float32")
-    Y = runtime.DeviceBuffer((n, h, w, f), "float32")
-    zeros = np.zeros((n, h, w, f), np.float32)
+    n, c, h, w, f = shape
+    x = rng.standard_normal((n, c, h, w)).astype(dtype)
+    wt = (rng.standard_normal((f, c, 3, 3)) * np.sqrt(2.0 / (c * 9))).astype(dtype)
+    X = runtime.DeviceBuffer.from_numpy(np.ascontiguousarray(x.transpose(0, 2, 3, 1)), dtype)
+    W = runtime.DeviceBuffer.from_numpy(np.ascontiguousarray(wt.transpose(0, 2, 3, 1)), dtype)
+    Y = runtime.DeviceBuffer((n, h, w, f), dtype)
+    zeros = np.zeros((n, h, w, f), dtype)
     Y.copy_from(zeros)
     args = runtime.pod_args([X, W, Y])
 
@@ -290,10 +292,14 @@ def test_fp32_convolution_with_a_tail_split_is_captured_after_reserving_its_scra
     call()
     stream.synchronize()
     assert np.array_equal(Y.numpy(), got)
-    sample = [0, 3]  # the last image lies in the tiles that are cut
-    want = oracle.conv2d_nchw(x[sample], wt, (1, 1), (1, 1))
-    scale = oracle.conv2d_nchw(np.abs(x[sample]), np.abs(wt), (1, 1), (1, 1))
-    assert np.all(np.abs(got[sample].transpose(0, 3, 1, 2) - want) <= 1e-5 * scale)
+    sample = [0, n - 1]  # fp32: the last image lies in the tiles that are cut
+    want = oracle.conv2d_nchw(x[sample], wt, (1, 1), (1, 1)).astype(np.float64)
+    scale = oracle.conv2d_nchw(np.abs(x[sample]).astype(np.float32), np.abs(wt).astype(np.float32), (1, 1), (1, 1))
+    err = np.abs(got[sample].transpose(0, 3, 1, 2).astype(np.float64) - want)
+    if dtype == "float32":
+        assert np.all(err <= tol * scale)
+    else:
+        assert np.all(err <= tol * np.maximum(np.abs(want), 1e-2 * scale) + 1e-6)
     hip.hipGraphExecDestroy(graph_exec)
     hip.hipGraphDestroy(graph)
 
